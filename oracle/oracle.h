@@ -1,0 +1,104 @@
+/*
+ * CPU oracle for the convolution / depthwise / pooling path.
+ *
+ * TEST INFRASTRUCTURE ONLY: this library is the checker the HIP kernels are
+ * compared against and the CPU baseline that is timed beside them.  Nothing in
+ * the shipped library links, loads or calls it.
+ *
+ * Every function restates, in plain C, what the corresponding portDNN kernel
+ * computes (reference file:line cited per function in oracle.c).  Layouts:
+ * tensors NHWC row-major, dense filter HWCF [R][S][C][K], depthwise filter
+ * [R][S][C][multiplier] with output channel c*multiplier+j.
+ *
+ * How each function is pinned (nothing here is "parity unpinned"):
+ *   conv2d fwd/inbk/filbk, depthwise fwd/inbk/filbk, max/avg pool fwd+grad:
+ *     the reference's generated golden vectors (tests/golden/ *.npz, exact
+ *     integers) -- tests/test_oracle_golden.py.
+ *   max-pool NaN rules: the hand-written cases of
+ *     test/pooling/max_pooling_with_nan.cc -- tests/test_oracle_golden.py.
+ *   padding helper: known answers of test/helpers/padding.cc.
+ *   tiled forward: must equal the direct forward bit-for-bit on integer data
+ *     and is checked against the same goldens.
+ *   matmul: textbook definition, checked against numpy float64 matmul for all
+ *     transpose/beta combinations.
+ *   Winograd transforms: algebraic identity against the direct convolution.
+ */
+#ifndef PORTDNN_AMD_ORACLE_H_
+#define PORTDNN_AMD_ORACLE_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* One record serves conv2d, depthwise (features = channel multiplier) and
+ * pooling (features ignored). */
+typedef struct oracle_params {
+  int channels;
+  int features;
+  int batch;
+  int in_rows, in_cols;
+  int window_rows, window_cols;
+  int stride_rows, stride_cols;
+  int out_rows, out_cols;
+  int pad_rows, pad_cols;
+} oracle_params;
+
+/* include/portdnn/helpers/padding.h:51-69.  same != 0 selects SAME. */
+void oracle_calculate_padding(int input, int window, int stride, int same,
+                              int* padding, int* output);
+
+/* acc64 != 0 accumulates in double and rounds once at the end (the
+ * "mathematically exact" answer used for tolerance checks); acc64 == 0
+ * accumulates in float in the reference's loop order. */
+void oracle_conv2d_forward(const float* in, const float* fil, float* out,
+                           const oracle_params* p, int acc64);
+void oracle_conv2d_input_backprop(const float* dy, const float* fil, float* dx,
+                                  const oracle_params* p, int acc64);
+void oracle_conv2d_filter_backprop(const float* in, const float* dy, float* dw,
+                                   const oracle_params* p, int acc64);
+
+/* portDNN's Tiled forward with the generic tile list entry
+ * (window, stride, 2 rows, 2 cols, channel vector 1, feature vector 4):
+ * one "work-item" per 2x2x4 output tile, float mad, channel-outermost
+ * accumulation.  Requires window 1 or 3 (square), stride 1 or 2 and
+ * features % 4 == 0; returns non-zero otherwise.  threads <= 0 uses every
+ * host core. */
+int oracle_conv2d_tiled_forward(const float* in, const float* fil, float* out,
+                                const oracle_params* p, int threads);
+
+void oracle_depthwise_forward(const float* in, const float* fil, float* out,
+                              const oracle_params* p, int acc64);
+void oracle_depthwise_input_backprop(const float* dy, const float* fil,
+                                     float* dx, const oracle_params* p,
+                                     int acc64);
+void oracle_depthwise_filter_backprop(const float* in, const float* dy,
+                                      float* dw, const oracle_params* p,
+                                      int acc64);
+
+/* nan_mode 0: pooling::Max (scalar form: NaN inputs never win);
+ * nan_mode 1: pooling::MaxWithNan (a NaN in the window wins). */
+void oracle_pool_max_forward(const float* in, float* out,
+                             const oracle_params* p, int nan_mode);
+void oracle_pool_avg_forward(const float* in, float* out,
+                             const oracle_params* p, int acc64);
+/* in: forward input, out: forward output, dy: gradient w.r.t. out,
+ * dx: gradient w.r.t. in (written). */
+void oracle_pool_max_grad(const float* in, const float* out, const float* dy,
+                          float* dx, const oracle_params* p, int nan_mode);
+void oracle_pool_avg_grad(const float* dy, float* dx, const oracle_params* p,
+                          int acc64);
+
+/* Batched row-major GEMM  C[b] = op(A[b]) * op(B[b]) + beta * C[b]
+ * with op(A) m x k, op(B) k x n. */
+void oracle_matmul(const float* a, const float* b, float* c, int batches, int m,
+                   int k, int n, int trans_a, int trans_b, float beta,
+                   int acc64);
+
+/* Thread count used by the OpenMP loops (<= 0: all cores). Returns the count
+ * now in force. */
+int oracle_set_threads(int threads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PORTDNN_AMD_ORACLE_H_ */

@@ -1,0 +1,137 @@
+#!/usr/bin/env python3
+"""Turn the reference's generated golden tests into compact data fixtures.
+
+The reference keeps its expected outputs as literal arrays inside generated
+gtest sources (test/conv2d/forward_window3_stride1.cc:57-67,
+test/depthwise_conv2d/forward_window3_stride1.cc, test/pooling/*_forward.cc,
+test/pooling/*_grad.cc).  Those sources are parsed here AS TEXT -- nothing is
+compiled or executed -- and only the data (case shape, padding mode,
+max_input_val and the expected output values) is written to
+tests/golden/<group>.npz.  The operands are never stored: every case
+regenerates them as 1,2,...,max_val,1,2,... exactly as
+test/gen/iota_initialised_data.h:74-79 does.
+
+Run inside the build container only (needs /root/reference):
+    python tests/golden/extract_fixtures.py
+"""
+import os
+import re
+import sys
+
+import numpy as np
+
+REF = os.environ.get("PORTDNN_REFERENCE", "/root/reference")
+OUT = os.path.dirname(os.path.abspath(__file__))
+
+CASE_RE = re.compile(r"TYPED_TEST\((\w+), (\w+)\) \{(.*?)\n\}", re.S)
+EXP_RE = re.compile(r"exp_out = \{(.*?)\};", re.S)
+SHAPE_RE = re.compile(r"in_shape = \{\{(.*?)\}\}", re.S)
+FEAT_RE = re.compile(r"(features|multiplier) = (\d+)")
+PAD_RE = re.compile(r"PaddingMode::(\w+)")
+MAXV_RE = re.compile(r"max_input_val = ([\d.]+)")
+
+# (window, stride) pairs extracted per family.
+CONV_FWD = [(1, 1), (1, 2), (3, 1), (3, 2), (5, 1), (5, 2), (7, 1), (7, 4)]
+CONV_BK = [(1, 1), (3, 1), (3, 2), (5, 1), (7, 4)]
+DW = [(1, 1), (3, 1), (3, 2), (5, 1), (7, 4)]
+POOL_FWD = [(1, 1), (3, 1), (3, 2), (5, 1), (5, 2), (7, 1), (7, 4), (11, 1),
+            (11, 4)]
+POOL_GRAD = [(3, 1), (3, 2), (5, 2), (7, 1)]
+
+
+def parse_file(path, window, stride):
+    """Returns (meta[int64 n_cases x 10], values[float64]) for one file.
+
+    meta columns: window, stride, N, H, W, C, K_or_multiplier (0 for pooling),
+    is_same, max_input_val, n_values.
+    """
+    with open(path) as f:
+        text = f.read()
+    metas, vals = [], []
+    for _suite, _name, body in CASE_RE.findall(text):
+        exp = EXP_RE.search(body).group(1)
+        values = np.array(
+            [float(tok) for tok in exp.replace("\n", " ").split(",")
+             if tok.strip()], dtype=np.float64)
+        shape = [int(t) for t in SHAPE_RE.search(body).group(1).split(",")]
+        feat = FEAT_RE.search(body)
+        k = int(feat.group(2)) if feat else 0
+        same = 1 if PAD_RE.search(body).group(1) == "SAME" else 0
+        maxv = int(float(MAXV_RE.search(body).group(1)))
+        metas.append([window, stride] + shape + [k, same, maxv, values.size])
+        vals.append(values)
+    if not metas:
+        raise RuntimeError("no cases parsed from " + path)
+    return np.array(metas, dtype=np.int64), np.concatenate(vals)
+
+
+def write_group(name, rel_dir, pattern, pairs, integral):
+    metas, vals = [], []
+    for w, s in pairs:
+        path = os.path.join(REF, "test", rel_dir, pattern.format(w=w, s=s))
+        m, v = parse_file(path, w, s)
+        metas.append(m)
+        vals.append(v)
+    meta = np.concatenate(metas)
+    values = np.concatenate(vals)
+    if integral:
+        assert np.all(values == np.round(values)), name
+        assert np.abs(values).max() <= 2 ** 24, name
+        values = values.astype(np.int32)
+    out = os.path.join(OUT, name + ".npz")
+    np.savez_compressed(out, meta=meta, values=values)
+    print("%-28s %5d cases %9d values %8d bytes" %
+          (name, len(meta), values.size, os.path.getsize(out)))
+
+
+def write_padding_kat():
+    """Known answers of test/helpers/padding.cc:54-..., one row per input:
+    is_same, window, stride, input, expected padding, expected output."""
+    with open(os.path.join(REF, "test", "helpers", "padding.cc")) as f:
+        text = f.read()
+    rows = []
+    pat = re.compile(
+        r"TYPED_TEST\(PaddingTest, (Valid|Same)Window(\d+)Stride(\d+)\) \{"
+        r"(.*?)\n\}", re.S)
+    for mode, window, stride, body in pat.findall(text):
+        vecs = {}
+        for name in ("inputs", "exp_pad", "exp_out"):
+            m = re.search(name + r" = \{(.*?)\};", body, re.S)
+            vecs[name] = [int(t) for t in m.group(1).split(",")]
+        for i, pad, out in zip(vecs["inputs"], vecs["exp_pad"],
+                               vecs["exp_out"]):
+            rows.append([mode == "Same", int(window), int(stride), i, pad, out])
+    rows = np.array(rows, dtype=np.int64)
+    assert len(rows) >= 64
+    np.savez_compressed(os.path.join(OUT, "padding_kat.npz"), rows=rows)
+    print("%-28s %5d rows" % ("padding_kat", len(rows)))
+
+
+def main():
+    if not os.path.isdir(REF):
+        sys.exit("reference tree not found at " + REF)
+    write_padding_kat()
+    write_group("conv2d_forward", "conv2d",
+                "forward_window{w}_stride{s}.cc", CONV_FWD, True)
+    write_group("conv2d_input_backprop", "conv2d",
+                "input_backprop_window{w}_stride{s}.cc", CONV_BK, True)
+    write_group("conv2d_filter_backprop", "conv2d",
+                "filter_backprop_window{w}_stride{s}.cc", CONV_BK, True)
+    write_group("depthwise_forward", "depthwise_conv2d",
+                "forward_window{w}_stride{s}.cc", DW, True)
+    write_group("depthwise_input_backprop", "depthwise_conv2d",
+                "input_backprop_window{w}_stride{s}.cc", DW, True)
+    write_group("depthwise_filter_backprop", "depthwise_conv2d",
+                "filter_backprop_window{w}_stride{s}.cc", DW, True)
+    write_group("pool_max_forward", "pooling",
+                "max_window{w}_stride{s}_forward.cc", POOL_FWD, True)
+    write_group("pool_avg_forward", "pooling",
+                "avg_window{w}_stride{s}_forward.cc", POOL_FWD, False)
+    write_group("pool_max_grad", "pooling",
+                "max_window{w}_stride{s}_grad.cc", POOL_GRAD, True)
+    write_group("pool_avg_grad", "pooling",
+                "avg_window{w}_stride{s}_grad.cc", POOL_GRAD, False)
+
+
+if __name__ == "__main__":
+    main()
