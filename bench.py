@@ -1,0 +1,269 @@
+#!/usr/bin/env python3
+"""Benchmark of the conv2d forward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one forward pass over the eight fp32 NHWC batch-32 ResNet layers of
+the benchmark configuration (3x3 s1 SAME at 56x56x64, 28x28x128, 14x14x256,
+7x7x512, plus the 1x1 K=4C layer of each stage), each through the algorithm
+the library's default selector picks, inputs resident in HBM.  `value` is
+total algorithmic TFLOP/s (2*N*OH*OW*R*S*C*K per layer, whatever the
+algorithm).  The same JSON line carries
+
+  roofline      the 3x3 convolution kernel against the fp32 MFMA peak, timed
+                with HIP events on the launch stream,
+  cpu_baseline  the reference's tiled algorithm restated in C (oracle/), timed
+                on the host cores on a bounded sample of the same layers,
+  detail        per-layer / per-algorithm TFLOP/s and the depthwise / pooling
+                GB/s against the HBM peak.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+RESNET = [(56, 64), (28, 128), (14, 256), (7, 512)]
+MOBILENET = [(112, 32, 1), (112, 64, 2), (56, 128, 1), (28, 256, 2),
+             (14, 512, 1), (7, 1024, 1)]
+BATCH = 32
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-detail", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path "
+                 "(run with --gpus 1)")
+
+    import numpy as np
+    import torch
+
+    from portdnn_amd import capi, ops
+    from portdnn_amd.capi import ALGO, DIRECTION, POOL_OP
+    import ctypes
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x5EED)
+
+    def uniform(n):
+        return torch.rand(n, device="cuda", generator=gen) * 2 - 1
+
+    def normal(n):
+        return torch.randn(n, device="cuda", generator=gen)
+
+    def default_algo(p):
+        return capi.lib().snn_hip_conv2d_default_algorithm(
+            ctypes.byref(p), DIRECTION.FORWARD)
+
+    def supports(p, algo):
+        return capi.lib().snn_hip_conv2d_algorithm_supports(
+            ctypes.byref(p), DIRECTION.FORWARD, algo) == algo
+
+    def event_time_ms(fn, reps, warm=3):
+        """Average duration of one call, HIP events on the launch stream."""
+        for _ in range(warm):
+            fn()
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(reps):
+            fn()
+        stop.record()
+        stop.synchronize()
+        return start.elapsed_time(stop) / reps
+
+    # ---- the workload --------------------------------------------------------
+    layers = []
+    for size, ch in RESNET:
+        layers.append(("3x3_%dx%dx%d" % (size, size, ch),
+                       ops.conv_params(BATCH, size, size, ch, ch, 3, 1, True)))
+    for size, ch in RESNET:
+        layers.append(("1x1_%dx%dx%d_k%d" % (size, size, ch, 4 * ch),
+                       ops.conv_params(BATCH, size, size, ch, 4 * ch, 1, 1,
+                                       False)))
+    work = []
+    for name, p in layers:
+        n_in, n_fil, n_out = ops.conv_sizes(p, DIRECTION.FORWARD)
+        algo = default_algo(p)
+        _, ws_elems = ops.workspace_size(p, DIRECTION.FORWARD, algo)
+        work.append(dict(
+            name=name, p=p, algo=algo, x=uniform(n_in), w=uniform(n_fil),
+            y=torch.empty(n_out, device="cuda"),
+            ws=(torch.empty(ws_elems, device="cuda") if ws_elems else None),
+            flops=ops.conv_flops(p, DIRECTION.FORWARD)))
+    total_flops = sum(w["flops"] for w in work)
+
+    def step():
+        for w in work:
+            ops.conv2d(w["x"], w["w"], w["p"], DIRECTION.FORWARD, w["algo"],
+                       workspace=w["ws"], out=w["y"])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = total_flops / (elapsed / args.steps) / 1e12
+
+    # ---- roofline: the 3x3 kernel, HIP events on the launch stream -----------
+    algo_names = {1: "direct", 2: "tiled", 3: "im2col", 4: "winograd",
+                  6: "matmul"}
+    per_layer = []
+    k3_flops = k3_ms = 0.0
+    for w in work:
+        ms = event_time_ms(lambda w=w: ops.conv2d(
+            w["x"], w["w"], w["p"], DIRECTION.FORWARD, w["algo"],
+            workspace=w["ws"], out=w["y"]), reps=20)
+        tf = w["flops"] / ms / 1e9
+        per_layer.append({"layer": w["name"], "algorithm": algo_names[w["algo"]],
+                          "ms": round(ms, 4), "tflops": round(tf, 2),
+                          "frac_mfma_peak": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)})
+        if w["name"].startswith("3x3"):
+            k3_flops += w["flops"]
+            k3_ms += ms
+    achieved = k3_flops / k3_ms / 1e9
+    roofline = {"bound": "mfma", "kernel": "conv2d 3x3 s1 forward, 4 ResNet stages",
+                "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+                "traffic": None}
+
+    detail = {"layers": per_layer}
+    if not args.no_detail:
+        # every algorithm on every 3x3 / 1x1 layer
+        algo_table = []
+        for w in work:
+            for algo in (ALGO.TILED, ALGO.IM2COL, ALGO.WINOGRAD, ALGO.MATMUL,
+                         ALGO.DIRECT):
+                if not supports(w["p"], algo):
+                    continue
+                _, ws_elems = ops.workspace_size(w["p"], DIRECTION.FORWARD, algo)
+                ws = torch.empty(ws_elems, device="cuda") if ws_elems else None
+                ms = event_time_ms(lambda: ops.conv2d(
+                    w["x"], w["w"], w["p"], DIRECTION.FORWARD, algo,
+                    workspace=ws, out=w["y"]), reps=10, warm=2)
+                algo_table.append({"layer": w["name"],
+                                   "algorithm": algo_names[algo],
+                                   "ms": round(ms, 4),
+                                   "tflops": round(w["flops"] / ms / 1e9, 2)})
+                del ws
+        detail["algorithms"] = algo_table
+
+        # memory-bound operators: rotate buffer sets so that the 256 MB
+        # last-level cache cannot hold the working set between launches
+        mem = []
+
+        def rotate_sets(nbytes):
+            return max(3, int(600e6 // nbytes) + 1)
+
+        for size, ch, stride in MOBILENET:
+            p = ops.depthwise_params(BATCH, size, size, ch, 1, 3, stride, True)
+            n_in, n_fil, n_out = ops.depthwise_sizes(p, DIRECTION.FORWARD)
+            nbytes = 4 * (n_in + n_fil + n_out)
+            sets = rotate_sets(nbytes)
+            xs = [normal(n_in) for _ in range(sets)]
+            ys = [torch.empty(n_out, device="cuda") for _ in range(sets)]
+            f = normal(n_fil)
+            state = {"i": 0}
+
+            def run():
+                i = state["i"] % sets
+                state["i"] += 1
+                ops.depthwise_conv2d(xs[i], f, p, out=ys[i])
+            ms = event_time_ms(run, reps=5 * sets, warm=sets)
+            gbs = nbytes / ms / 1e6
+            mem.append({"op": "depthwise3x3_%dx%dx%d_s%d" % (size, size, ch,
+                                                             stride),
+                        "bytes": nbytes, "ms": round(ms, 5),
+                        "gbs": round(gbs, 1),
+                        "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)})
+            del xs, ys
+        for name, p, op in (
+                ("maxpool3x3_s2_112x112x64",
+                 ops.pool_params(BATCH, 112, 112, 64, 3, 2, True), POOL_OP.MAX),
+                ("avgpool7x7_7x7x2048",
+                 ops.pool_params(BATCH, 7, 7, 2048, 7, 1, False),
+                 POOL_OP.AVERAGE)):
+            n_in = p.batch * p.in_rows * p.in_cols * p.channels
+            n_out = p.batch * p.out_rows * p.out_cols * p.channels
+            nbytes = 4 * (n_in + n_out)
+            sets = rotate_sets(nbytes)
+            xs = [normal(n_in) for _ in range(sets)]
+            ys = [torch.empty(n_out, device="cuda") for _ in range(sets)]
+            state = {"i": 0}
+
+            def run():
+                i = state["i"] % sets
+                state["i"] += 1
+                ops.pooling_forward(xs[i], p, op, out=ys[i])
+            ms = event_time_ms(run, reps=5 * sets, warm=sets)
+            gbs = nbytes / ms / 1e6
+            mem.append({"op": name, "bytes": nbytes, "ms": round(ms, 5),
+                        "gbs": round(gbs, 1),
+                        "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)})
+            del xs, ys
+        detail["memory_bound"] = mem
+
+    # ---- CPU baseline: the reference's tiled algorithm, restated --------------
+    cpu = None
+    if not args.no_cpu_baseline:
+        import oracle
+        cores = oracle.set_threads(0)
+        rng = np.random.default_rng(0x5EED)
+        cpu_flops = 0.0
+        cpu_s = 0.0
+        for size, ch in RESNET:
+            for window, feats in ((3, ch), (1, 4 * ch)):
+                p = oracle.make_params(1, size, size, ch, feats, window, 1,
+                                       window == 3)
+                x = rng.uniform(-1, 1, size * size * ch).astype(np.float32)
+                w = rng.uniform(-1, 1, window * window * ch * feats).astype(
+                    np.float32)
+                oracle.conv2d_tiled_forward(x, w, p)  # warm-up, as the
+                t = time.perf_counter()               # reference's executor
+                oracle.conv2d_tiled_forward(x, w, p)
+                cpu_s += time.perf_counter() - t
+                cpu_flops += 2.0 * size * size * window * window * ch * feats
+        cpu = {"value": round(cpu_flops / cpu_s / 1e12, 5), "unit": "TFLOP/s",
+               "cores": cores, "kind": "port",
+               "sample": "batch 1 of each of the 8 layers, portDNN tiled "
+                         "algorithm (2x2x4 register tiles) restated in C with "
+                         "OpenMP; %.2f s of CPU time" % cpu_s}
+
+    line = {
+        "metric": "conv2d fwd TFLOP/s + %MFMA peak; depthwise/pool GB/s + "
+                  "%HBM peak, 1 GPU",
+        "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "conv2d forward fp32 NHWC batch 32: 3x3 s1 "
+                               "SAME at (56,64),(28,128),(14,256),(7,512) + "
+                               "1x1 K=4C at each stage; default selector",
+                   "batch": BATCH},
+        "roofline": roofline, "cpu_baseline": cpu, "detail": detail,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

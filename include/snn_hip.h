@@ -1,0 +1,257 @@
+/*
+ * C ABI of libsnn_hip.so -- the MI355X (gfx950) implementation of portDNN's
+ * convolution / depthwise-convolution / pooling hot path.
+ *
+ * portDNN itself has no C ABI: its boundary is a set of header templates
+ * (include/portdnn/<op>/launch.h) over explicitly instantiated launchers that
+ * live in libportdnn (src/<op>/launch*.cc).  The entry points below are what a
+ * HIP backend for those templates binds, one per (operator, direction, data
+ * type); each comment names the reference interface it stands in for.  The
+ * C++ drop-in templates in include/portdnn/ are a thin layer over this file.
+ *
+ * Conventions
+ *  - All tensor pointers are DEVICE pointers.  Tensors are NHWC row-major;
+ *    dense filters are HWCF [R][S][C][K]; depthwise filters are
+ *    [R][S][C][multiplier] and output channel c*multiplier+j.
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *    Every call is asynchronous and stream-ordered; no call synchronises.
+ *  - The return value is a snn_hip_status.  Values 0..5 are portDNN's
+ *    StatusCode enumerators in declaration order
+ *    (include/portdnn/status.h:31-44); 6 reports a HIP runtime failure.
+ *  - Workspace sizes are counted in ELEMENTS of the data type, as in
+ *    include/portdnn/conv2d/workspace_size.h:42-47.
+ *  - f16 entry points take IEEE binary16 data and accumulate in fp32.
+ */
+#ifndef SNN_HIP_H_
+#define SNN_HIP_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(_WIN32)
+#define SNN_HIP_API
+#else
+#define SNN_HIP_API __attribute__((visibility("default")))
+#endif
+
+typedef enum snn_hip_status {
+  SNN_HIP_OK = 0,
+  SNN_HIP_INVALID_ALGORITHM = 1,
+  SNN_HIP_INDEX_EXCEEDED = 2,
+  SNN_HIP_INSUFFICIENT_WORKSPACE = 3,
+  SNN_HIP_ALLOCATION_PROBLEM = 4,
+  SNN_HIP_INVALID_PARAMETER = 5,
+  SNN_HIP_DEVICE_ERROR = 6
+} snn_hip_status;
+
+/* sycldnn::conv2d::Algorithm, include/portdnn/conv2d/algorithm.h:30-45 */
+typedef enum snn_hip_algorithm {
+  SNN_HIP_ALGO_NOT_SUPPORTED = 0,
+  SNN_HIP_ALGO_DIRECT = 1,
+  SNN_HIP_ALGO_TILED = 2,
+  SNN_HIP_ALGO_IM2COL = 3,
+  SNN_HIP_ALGO_WINOGRAD = 4,
+  SNN_HIP_ALGO_WINOGRAD_LARGE = 5,
+  SNN_HIP_ALGO_MATMUL = 6
+} snn_hip_algorithm;
+
+/* sycldnn::conv2d::conv_type tags, include/portdnn/conv2d/conv_type.h:35-47 */
+typedef enum snn_hip_direction {
+  SNN_HIP_FORWARD = 0,
+  SNN_HIP_INPUT_BACKPROP = 1,
+  SNN_HIP_FILTER_BACKPROP = 2
+} snn_hip_direction;
+
+/* POD image of sycldnn::conv2d::Conv2DParams
+ * (include/portdnn/conv2d/params.h:32-112), same field order.  The three
+ * format fields hold the enumerator values of DataFormat (NHWC = 0, NCHW = 1),
+ * FilterFormat (HWCF = 0, FCHW = 1, FHWC = 2) and BatchFormat (STRIDED = 0,
+ * INTERLEAVED = 1); only the first of each is accepted. */
+typedef struct snn_hip_conv2d_params {
+  int channels;
+  int features;
+  int batch;
+  int in_rows;
+  int in_cols;
+  int window_rows;
+  int window_cols;
+  int stride_rows;
+  int stride_cols;
+  int out_rows;
+  int out_cols;
+  int pad_rows;
+  int pad_cols;
+  int dilation_rows;
+  int dilation_cols;
+  int groups;
+  int input_format;
+  int filter_format;
+  int group_format;
+} snn_hip_conv2d_params;
+
+/* POD image of sycldnn::depthwise_conv2d::DepthwiseConv2DParams
+ * (include/portdnn/depthwise_conv2d/params.h:33-94). */
+typedef struct snn_hip_depthwise_params {
+  int channels;
+  int channel_multiplier;
+  int batch;
+  int in_rows;
+  int in_cols;
+  int window_rows;
+  int window_cols;
+  int stride_rows;
+  int stride_cols;
+  int out_rows;
+  int out_cols;
+  int pad_rows;
+  int pad_cols;
+  int input_format;
+  int filter_format;
+} snn_hip_depthwise_params;
+
+/* POD image of sycldnn::pooling::PoolingParams
+ * (include/portdnn/pooling/params.h:30-73). */
+typedef struct snn_hip_pooling_params {
+  int in_rows;
+  int in_cols;
+  int out_rows;
+  int out_cols;
+  int window_rows;
+  int window_cols;
+  int stride_rows;
+  int stride_cols;
+  int batch;
+  int channels;
+  int pad_rows;
+  int pad_cols;
+  int input_format;
+} snn_hip_pooling_params;
+
+/* sycldnn::pooling operators, include/portdnn/pooling/operators.h:23-42 */
+typedef enum snn_hip_pool_op {
+  SNN_HIP_POOL_MAX = 0,
+  SNN_HIP_POOL_MAX_WITH_NAN = 1,
+  SNN_HIP_POOL_AVERAGE = 2
+} snn_hip_pool_op;
+
+/* ---- library ------------------------------------------------------------ */
+
+/* Library version, major*10000 + minor*100 + patch. */
+SNN_HIP_API int snn_hip_version(void);
+/* Static, human-readable name of a status value. */
+SNN_HIP_API const char* snn_hip_status_string(int status);
+/* Text of the last HIP runtime error seen by the calling thread ("" if none). */
+SNN_HIP_API const char* snn_hip_last_error(void);
+
+/* ---- dense convolution ---------------------------------------------------
+ * Stand-ins for sycldnn::conv2d::internal::launch_{direct,tiled,matmul,
+ * im2col,winograd} reached from sycldnn::conv2d::launch<T, ConvType>
+ * (include/portdnn/conv2d/launch.h:59-118 via
+ * include/portdnn/internal/conv2d/launch.h:99-207): validate the parameters,
+ * check that `algorithm` supports them (SNN_HIP_INVALID_ALGORITHM otherwise,
+ * as internal/conv2d/launch.h:127-129,191-197) and enqueue the kernels.
+ *
+ * forward:         input  [N,H,W,C]    filter [R,S,C,K]    output [N,OH,OW,K]
+ * input_backprop:  input = dY [N,OH,OW,K], filter [R,S,C,K], output = dX [N,H,W,C]
+ * filter_backprop: input = X [N,H,W,C], filter = dY [N,OH,OW,K], output = dW [R,S,C,K]
+ * (operand roles of include/portdnn/conv2d/sizes.h:166-179).
+ *
+ * `workspace` may be NULL with workspace_elems == 0.  Winograd then returns
+ * SNN_HIP_INSUFFICIENT_WORKSPACE (internal/conv2d/winograd/launch.h:271-286);
+ * the other algorithms need no caller scratch. */
+SNN_HIP_API int snn_hip_conv2d_forward_f32(
+    const float* input, const float* filter, float* output,
+    const snn_hip_conv2d_params* params, int algorithm, float* workspace,
+    size_t workspace_elems, void* stream);
+SNN_HIP_API int snn_hip_conv2d_input_backprop_f32(
+    const float* input, const float* filter, float* output,
+    const snn_hip_conv2d_params* params, int algorithm, float* workspace,
+    size_t workspace_elems, void* stream);
+SNN_HIP_API int snn_hip_conv2d_filter_backprop_f32(
+    const float* input, const float* filter, float* output,
+    const snn_hip_conv2d_params* params, int algorithm, float* workspace,
+    size_t workspace_elems, void* stream);
+SNN_HIP_API int snn_hip_conv2d_forward_f16(
+    const void* input, const void* filter, void* output,
+    const snn_hip_conv2d_params* params, int algorithm, void* workspace,
+    size_t workspace_elems, void* stream);
+
+/* sycldnn::conv2d::query_workspace_size<ConvType>(params, selector)
+ * (include/portdnn/conv2d/workspace_size.h:158-163) for an already selected
+ * algorithm.  Sizes in elements. */
+SNN_HIP_API int snn_hip_conv2d_workspace_size(
+    const snn_hip_conv2d_params* params, int direction, int algorithm,
+    size_t* required_elems, size_t* recommended_elems);
+
+/* Does `algorithm` support these parameters in this direction?  Mirrors the
+ * concrete selectors (include/portdnn/conv2d/selector/{tiled,winograd,matmul}_
+ * selector.h, constant_selector.h): returns `algorithm` if it does, else
+ * SNN_HIP_ALGO_NOT_SUPPORTED. */
+SNN_HIP_API int snn_hip_conv2d_algorithm_supports(
+    const snn_hip_conv2d_params* params, int direction, int algorithm);
+
+/* The algorithm sycldnn::conv2d::get_default_selector(device) would pick on
+ * this device (src/conv2d/selector/default_selector.cc:257-286), tuned for
+ * MI355X. */
+SNN_HIP_API int snn_hip_conv2d_default_algorithm(
+    const snn_hip_conv2d_params* params, int direction);
+
+/* ---- depthwise convolution -----------------------------------------------
+ * Stand-ins for sycldnn::depthwise_conv2d::internal::launch<ConvType>
+ * (src/depthwise_conv2d/launch.cc:100-121) reached from
+ * sycldnn::depthwise_conv2d::launch (include/portdnn/depthwise_conv2d/
+ * launch.h:54-91).  Operand roles as for the dense convolution with
+ * K = C * multiplier. */
+SNN_HIP_API int snn_hip_depthwise_conv2d_forward_f32(
+    const float* input, const float* filter, float* output,
+    const snn_hip_depthwise_params* params, void* stream);
+SNN_HIP_API int snn_hip_depthwise_conv2d_input_backprop_f32(
+    const float* input, const float* filter, float* output,
+    const snn_hip_depthwise_params* params, void* stream);
+SNN_HIP_API int snn_hip_depthwise_conv2d_filter_backprop_f32(
+    const float* input, const float* filter, float* output,
+    const snn_hip_depthwise_params* params, void* stream);
+SNN_HIP_API int snn_hip_depthwise_conv2d_forward_f16(
+    const void* input, const void* filter, void* output,
+    const snn_hip_depthwise_params* params, void* stream);
+
+/* ---- pooling -------------------------------------------------------------
+ * Stand-ins for sycldnn::pooling::internal::launch_pooling
+ * (src/pooling/launch_pooling.cc:146-165) reached from
+ * sycldnn::pooling::launch<T, PoolType, Direction>
+ * (include/portdnn/pooling/launch.h:112-128 forward, :153-172 max gradient).
+ * `op` is a snn_hip_pool_op. */
+SNN_HIP_API int snn_hip_pooling_forward_f32(
+    const float* input, float* output, const snn_hip_pooling_params* params,
+    int op, void* stream);
+SNN_HIP_API int snn_hip_pooling_forward_f16(
+    const void* input, void* output, const snn_hip_pooling_params* params,
+    int op, void* stream);
+/* Max / MaxWithNan gradient: input_data and output_data are the forward
+ * tensors, input_backprop is dY [N,OH,OW,C], output_backprop is dX [N,H,W,C]. */
+SNN_HIP_API int snn_hip_pooling_max_grad_f32(
+    const float* input_data, const float* output_data,
+    const float* input_backprop, float* output_backprop,
+    const snn_hip_pooling_params* params, int op, void* stream);
+/* Average gradient: input_backprop dY [N,OH,OW,C] -> output_backprop dX. */
+SNN_HIP_API int snn_hip_pooling_avg_grad_f32(
+    const float* input_backprop, float* output_backprop,
+    const snn_hip_pooling_params* params, void* stream);
+
+/* ---- matmul ----------------------------------------------------------------
+ * Stand-in for sycldnn::matmul::internal::launch (src/matmul/launch.cc) as the
+ * backend's matmul / batch_matmul members call it
+ * (include/portdnn/backend/snn_usm_matmul_provider.h:206-231): row-major
+ * C[b] = op(A[b]) * op(B[b]) + beta * C[b], op(A) m x k, op(B) k x n. */
+SNN_HIP_API int snn_hip_matmul_f32(const float* lhs, const float* rhs,
+                                   float* output, int batches, int m, int k,
+                                   int n, int transpose_lhs, int transpose_rhs,
+                                   float beta, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SNN_HIP_H_ */

@@ -1,0 +1,253 @@
+// Depthwise convolution for gfx950: bandwidth-bound kernels, no MFMA.
+// Stand-ins for portDNN's DepthwiseConv2D functors
+// (src/depthwise_conv2d/kernels.h:40-366).
+//
+// Layout: input/output NHWC, filter [R][S][C][multiplier], output channel
+// c*multiplier+j.
+//
+// Forward, multiplier 1, C % 4 == 0 (the MobileNet shapes): one lane owns a
+// float4 (or 4 x f16) of channels, so the 64 lanes of a wave read one
+// contiguous 1 KiB (512 B for f16) run of the NHWC row -- fully coalesced --
+// and the window taps of neighbouring lanes/pixels are served from L1/L2.
+// Everything else goes through the scalar kernel.
+#include "snn_kernels.h"
+
+namespace snn {
+namespace {
+
+template <typename T>
+struct Vec4;
+template <>
+struct Vec4<float> {
+  using type = float4;
+  __device__ static void load(const float* p, float (&v)[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+  __device__ static void store(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <>
+struct Vec4<_Float16> {
+  typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+  __device__ static void load(const _Float16* p, float (&v)[4]) {
+    const half4 t = *reinterpret_cast<const half4*>(p);
+    v[0] = static_cast<float>(t.x); v[1] = static_cast<float>(t.y);
+    v[2] = static_cast<float>(t.z); v[3] = static_cast<float>(t.w);
+  }
+  __device__ static void store(_Float16* p, const float (&v)[4]) {
+    half4 t;
+    t.x = static_cast<_Float16>(v[0]); t.y = static_cast<_Float16>(v[1]);
+    t.z = static_cast<_Float16>(v[2]); t.w = static_cast<_Float16>(v[3]);
+    *reinterpret_cast<half4*>(p) = t;
+  }
+};
+
+// Forward, multiplier == 1, four channels per lane.
+template <typename T>
+__global__ void __launch_bounds__(256)
+    dw_forward_vec4_kernel(const T* __restrict__ in, const T* __restrict__ fil,
+                           T* __restrict__ out, snn_hip_depthwise_params p,
+                           size_t n_vec) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n_vec) return;
+  const int C = p.channels;
+  const int cv = C / 4;
+  const int c = static_cast<int>(idx % cv) * 4;
+  size_t pix = idx / cv;
+  const int ox = static_cast<int>(pix % p.out_cols);
+  pix /= p.out_cols;
+  const int oy = static_cast<int>(pix % p.out_rows);
+  const int n = static_cast<int>(pix / p.out_rows);
+  const T* in_n = in + static_cast<size_t>(n) * p.in_rows * p.in_cols * C + c;
+  const T* fil_c = fil + c;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  const int y0 = oy * p.stride_rows - p.pad_rows;
+  const int x0 = ox * p.stride_cols - p.pad_cols;
+  for (int r = 0; r < p.window_rows; ++r) {
+    const int y = y0 + r;
+    if (y < 0 || y >= p.in_rows) continue;
+    for (int s = 0; s < p.window_cols; ++s) {
+      const int x = x0 + s;
+      if (x < 0 || x >= p.in_cols) continue;
+      float iv[4], fv[4];
+      Vec4<T>::load(in_n + (static_cast<size_t>(y) * p.in_cols + x) * C, iv);
+      Vec4<T>::load(fil_c + static_cast<size_t>(r * p.window_cols + s) * C, fv);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = fmaf(iv[i], fv[i], acc[i]);
+    }
+  }
+  Vec4<T>::store(out + idx * 4, acc);
+}
+
+// Forward, any multiplier / channel count: one lane per output element.
+template <typename T>
+__global__ void __launch_bounds__(256)
+    dw_forward_scalar_kernel(const T* __restrict__ in,
+                             const T* __restrict__ fil, T* __restrict__ out,
+                             snn_hip_depthwise_params p, size_t n_out) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n_out) return;
+  const int C = p.channels, M = p.channel_multiplier;
+  const int cm = static_cast<int>(idx % (static_cast<size_t>(C) * M));
+  const int c = cm / M, j = cm % M;
+  size_t pix = idx / (static_cast<size_t>(C) * M);
+  const int ox = static_cast<int>(pix % p.out_cols);
+  pix /= p.out_cols;
+  const int oy = static_cast<int>(pix % p.out_rows);
+  const int n = static_cast<int>(pix / p.out_rows);
+  const T* in_n = in + static_cast<size_t>(n) * p.in_rows * p.in_cols * C + c;
+  float acc = 0.f;
+  for (int r = 0; r < p.window_rows; ++r) {
+    const int y = oy * p.stride_rows - p.pad_rows + r;
+    if (y < 0 || y >= p.in_rows) continue;
+    for (int s = 0; s < p.window_cols; ++s) {
+      const int x = ox * p.stride_cols - p.pad_cols + s;
+      if (x < 0 || x >= p.in_cols) continue;
+      acc = fmaf(
+          Elem<T>::load(in_n + (static_cast<size_t>(y) * p.in_cols + x) * C),
+          Elem<T>::load(fil +
+                        (static_cast<size_t>(r * p.window_cols + s) * C + c) * M +
+                        j),
+          acc);
+    }
+  }
+  out[idx] = Elem<T>::from_float(acc);
+}
+
+// Input backprop: one lane per dX element (n, y, x, c).
+template <typename T>
+__global__ void __launch_bounds__(256)
+    dw_input_backprop_kernel(const T* __restrict__ dy,
+                             const T* __restrict__ fil, T* __restrict__ dx,
+                             snn_hip_depthwise_params p, size_t n_out) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n_out) return;
+  const int C = p.channels, M = p.channel_multiplier;
+  const int c = static_cast<int>(idx % C);
+  size_t pix = idx / C;
+  const int x = static_cast<int>(pix % p.in_cols);
+  pix /= p.in_cols;
+  const int y = static_cast<int>(pix % p.in_rows);
+  const int n = static_cast<int>(pix / p.in_rows);
+  const T* dy_n =
+      dy + static_cast<size_t>(n) * p.out_rows * p.out_cols * C * M;
+  float acc = 0.f;
+  for (int r = 0; r < p.window_rows; ++r) {
+    const int ty = y + p.pad_rows - r;
+    if (ty < 0 || ty % p.stride_rows) continue;
+    const int oy = ty / p.stride_rows;
+    if (oy >= p.out_rows) continue;
+    for (int s = 0; s < p.window_cols; ++s) {
+      const int tx = x + p.pad_cols - s;
+      if (tx < 0 || tx % p.stride_cols) continue;
+      const int ox = tx / p.stride_cols;
+      if (ox >= p.out_cols) continue;
+      const T* gp =
+          dy_n + ((static_cast<size_t>(oy) * p.out_cols + ox) * C + c) * M;
+      const T* fp =
+          fil + (static_cast<size_t>(r * p.window_cols + s) * C + c) * M;
+      for (int j = 0; j < M; ++j) {
+        acc = fmaf(Elem<T>::load(gp + j), Elem<T>::load(fp + j), acc);
+      }
+    }
+  }
+  dx[idx] = Elem<T>::from_float(acc);
+}
+
+constexpr int kStrip = 64;   // (channel, multiplier) pairs per work-group
+constexpr int kSlices = 4;   // waves splitting the batch*rows*cols reduction
+
+// Filter backprop: one work-group per filter tap (r, s) and strip of 64
+// flattened (c, j) outputs; the four waves split the reduction over every
+// output pixel and combine through LDS.
+template <typename T>
+__global__ void __launch_bounds__(kStrip* kSlices)
+    dw_filter_backprop_kernel(const T* __restrict__ in,
+                              const T* __restrict__ dy, T* __restrict__ dw,
+                              snn_hip_depthwise_params p) {
+  __shared__ float partial[kSlices][kStrip];
+  const int C = p.channels, M = p.channel_multiplier;
+  const int CM = C * M;
+  const int lane = threadIdx.x % kStrip;
+  const int slice = threadIdx.x / kStrip;
+  const int cm = blockIdx.y * kStrip + lane;
+  const int s = blockIdx.x % p.window_cols;
+  const int r = blockIdx.x / p.window_cols;
+  const int c = cm / M;
+  const int n_pix = p.batch * p.out_rows * p.out_cols;
+  float acc = 0.f;
+  if (cm < CM) {
+    for (int pix = slice; pix < n_pix; pix += kSlices) {
+      const int ox = pix % p.out_cols;
+      const int t = pix / p.out_cols;
+      const int oy = t % p.out_rows;
+      const int n = t / p.out_rows;
+      const int y = oy * p.stride_rows - p.pad_rows + r;
+      const int x = ox * p.stride_cols - p.pad_cols + s;
+      if (y < 0 || y >= p.in_rows || x < 0 || x >= p.in_cols) continue;
+      const float xv = Elem<T>::load(
+          in + ((static_cast<size_t>(n) * p.in_rows + y) * p.in_cols + x) * C +
+          c);
+      const float gv = Elem<T>::load(dy + static_cast<size_t>(pix) * CM + cm);
+      acc = fmaf(xv, gv, acc);
+    }
+  }
+  partial[slice][lane] = acc;
+  __syncthreads();
+  if (slice == 0 && cm < CM) {
+    float sum = partial[0][lane];
+    for (int i = 1; i < kSlices; ++i) sum += partial[i][lane];
+    dw[static_cast<size_t>(blockIdx.x) * CM + cm] = Elem<T>::from_float(sum);
+  }
+}
+
+}  // namespace
+
+template <typename T>
+int launch_depthwise(int direction, const T* input, const T* filter, T* output,
+                     const snn_hip_depthwise_params& p, hipStream_t stream) {
+  constexpr int kBlock = 256;
+  const size_t CM = static_cast<size_t>(p.channels) * p.channel_multiplier;
+  if (direction == SNN_HIP_FORWARD) {
+    const size_t n_out = static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * CM;
+    if (p.channel_multiplier == 1 && p.channels % 4 == 0) {
+      const size_t n_vec = n_out / 4;
+      hipLaunchKernelGGL(dw_forward_vec4_kernel<T>,
+                         dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{kBlock}))),
+                         dim3(kBlock), 0, stream, input, filter, output, p,
+                         n_vec);
+    } else {
+      hipLaunchKernelGGL(dw_forward_scalar_kernel<T>,
+                         dim3(static_cast<unsigned>(ceil_div(n_out, size_t{kBlock}))),
+                         dim3(kBlock), 0, stream, input, filter, output, p,
+                         n_out);
+    }
+  } else if (direction == SNN_HIP_INPUT_BACKPROP) {
+    const size_t n_out =
+        static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
+    hipLaunchKernelGGL(dw_input_backprop_kernel<T>,
+                       dim3(static_cast<unsigned>(ceil_div(n_out, size_t{kBlock}))),
+                       dim3(kBlock), 0, stream, input, filter, output, p,
+                       n_out);
+  } else {
+    const dim3 grid(static_cast<unsigned>(p.window_rows * p.window_cols),
+                    static_cast<unsigned>(ceil_div(CM, size_t{kStrip})));
+    hipLaunchKernelGGL(dw_filter_backprop_kernel<T>, grid,
+                       dim3(kStrip * kSlices), 0, stream, input, filter,
+                       output, p);
+  }
+  SNN_HIP_CHECK_LAUNCH();
+  return SNN_HIP_OK;
+}
+
+template int launch_depthwise<float>(int, const float*, const float*, float*,
+                                     const snn_hip_depthwise_params&,
+                                     hipStream_t);
+template int launch_depthwise<_Float16>(int, const _Float16*, const _Float16*,
+                                        _Float16*,
+                                        const snn_hip_depthwise_params&,
+                                        hipStream_t);
+
+}  // namespace snn

@@ -1,0 +1,124 @@
+// Batched row-major GEMM  C[b] = op(A[b]) * op(B[b]) + beta * C[b]  for gfx950.
+// Stand-in for portDNN's MatmulKernel (src/matmul/kernels.h:26-133,
+// src/matmul/launch.cc:51-56).
+//
+// General-shape kernel: 64x64 output tile per 256-lane work-group, A and B
+// tiles staged in LDS, 4x4 register block per lane, every edge bounds-checked
+// so any m, k, n and both transposes are accepted.
+#include "snn_kernels.h"
+
+namespace snn {
+namespace {
+
+constexpr int kTile = 64;
+constexpr int kTileK = 16;
+
+template <bool TransA, bool TransB>
+__global__ void __launch_bounds__(256)
+    matmul_general_kernel(const float* __restrict__ a,
+                          const float* __restrict__ b, float* __restrict__ c,
+                          int m, int k, int n, float beta) {
+  __shared__ float sa[kTileK][kTile + 4];  // [kk][row]
+  __shared__ float sb[kTileK][kTile + 4];  // [kk][col]
+  const int batch = blockIdx.z;
+  a += static_cast<size_t>(batch) * m * k;
+  b += static_cast<size_t>(batch) * k * n;
+  c += static_cast<size_t>(batch) * m * n;
+  const int row0 = blockIdx.x * kTile;
+  const int col0 = blockIdx.y * kTile;
+  const int tx = threadIdx.x % 16;  // column group
+  const int ty = threadIdx.x / 16;  // row group
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < k; k0 += kTileK) {
+    for (int e = threadIdx.x; e < kTile * kTileK; e += 256) {
+      // A tile element (row r, depth kk)
+      int r, kk;
+      if (TransA) {  // memory is [k][m]: consecutive lanes walk rows
+        r = e % kTile;
+        kk = e / kTile;
+      } else {  // memory is [m][k]: consecutive lanes walk depth
+        kk = e % kTileK;
+        r = e / kTileK;
+      }
+      const int gr = row0 + r, gk = k0 + kk;
+      float v = 0.f;
+      if (gr < m && gk < k) {
+        v = TransA ? a[static_cast<size_t>(gk) * m + gr]
+                   : a[static_cast<size_t>(gr) * k + gk];
+      }
+      sa[kk][r] = v;
+      // B tile element (depth kk2, col cc)
+      int cc, kk2;
+      if (TransB) {  // memory is [n][k]
+        kk2 = e % kTileK;
+        cc = e / kTileK;
+      } else {  // memory is [k][n]
+        cc = e % kTile;
+        kk2 = e / kTile;
+      }
+      const int gc = col0 + cc, gk2 = k0 + kk2;
+      float w = 0.f;
+      if (gc < n && gk2 < k) {
+        w = TransB ? b[static_cast<size_t>(gc) * k + gk2]
+                   : b[static_cast<size_t>(gk2) * n + gc];
+      }
+      sb[kk2][cc] = w;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < kTileK; ++kk) {
+      float av[4], bv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = sa[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bv[j] = sb[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int gr = row0 + ty * 4 + i;
+    if (gr >= m) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int gc = col0 + tx * 4 + j;
+      if (gc >= n) continue;
+      const size_t o = static_cast<size_t>(gr) * n + gc;
+      c[o] = (beta == 0.f) ? acc[i][j] : fmaf(beta, c[o], acc[i][j]);
+    }
+  }
+}
+
+}  // namespace
+
+int launch_matmul_f32(const float* lhs, const float* rhs, float* output,
+                      int batches, int m, int k, int n, bool transpose_lhs,
+                      bool transpose_rhs, float beta, hipStream_t stream) {
+  const dim3 grid(static_cast<unsigned>(ceil_div(m, kTile)),
+                  static_cast<unsigned>(ceil_div(n, kTile)),
+                  static_cast<unsigned>(batches));
+  const dim3 block(256);
+  if (transpose_lhs) {
+    if (transpose_rhs)
+      hipLaunchKernelGGL((matmul_general_kernel<true, true>), grid, block, 0,
+                         stream, lhs, rhs, output, m, k, n, beta);
+    else
+      hipLaunchKernelGGL((matmul_general_kernel<true, false>), grid, block, 0,
+                         stream, lhs, rhs, output, m, k, n, beta);
+  } else {
+    if (transpose_rhs)
+      hipLaunchKernelGGL((matmul_general_kernel<false, true>), grid, block, 0,
+                         stream, lhs, rhs, output, m, k, n, beta);
+    else
+      hipLaunchKernelGGL((matmul_general_kernel<false, false>), grid, block, 0,
+                         stream, lhs, rhs, output, m, k, n, beta);
+  }
+  SNN_HIP_CHECK_LAUNCH();
+  return SNN_HIP_OK;
+}
+
+}  // namespace snn

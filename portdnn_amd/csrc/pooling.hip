@@ -1,0 +1,316 @@
+// Max / average pooling for gfx950: bandwidth-bound kernels, no MFMA.
+// Stand-ins for portDNN's PoolingOp functors (src/pooling/kernels.h:43-414)
+// with the operators of src/pooling/operators_impl.h:27-113.
+//
+// Forward: one lane per output channel vector (4 channels when C % 4 == 0, as
+// src/pooling/launch_pooling.cc:134-143 chooses), channel index fastest, so a
+// wave reads contiguous NHWC runs.  The window is clipped to the image;
+// average divides by the clipped element count.
+#include <cfloat>
+
+#include "snn_kernels.h"
+
+namespace snn {
+namespace {
+
+// numeric_limits<T>::lowest(), the start value of the max operators.
+template <typename T>
+__device__ constexpr float lowest_of();
+template <>
+__device__ constexpr float lowest_of<float>() { return -FLT_MAX; }
+template <>
+__device__ constexpr float lowest_of<_Float16>() { return -65504.f; }
+
+// Accumulators with portDNN's semantics.
+struct MaxOp {
+  float v;
+  __device__ void init(float lowest) { v = lowest; }
+  __device__ void accumulate(float x) {
+    if (x > v) v = x;  // a NaN never compares greater
+  }
+  __device__ float value(int) const { return v; }
+};
+struct MaxNanOp {
+  float v;
+  __device__ void init(float lowest) { v = lowest; }
+  __device__ void accumulate(float x) {
+    if (x != x || x > v) v = x;  // a NaN wins and then sticks
+  }
+  __device__ float value(int) const { return v; }
+};
+struct AvgOp {
+  float v;
+  __device__ void init(float) { v = 0.f; }
+  __device__ void accumulate(float x) { v += x; }
+  __device__ float value(int tally) const {
+    return v / static_cast<float>(tally);
+  }
+};
+
+template <typename T, int VEC>
+struct VecIO;
+template <>
+struct VecIO<float, 1> {
+  __device__ static void load(const float* p, float (&v)[1]) { v[0] = *p; }
+  __device__ static void store(float* p, const float (&v)[1]) { *p = v[0]; }
+};
+template <>
+struct VecIO<float, 4> {
+  __device__ static void load(const float* p, float (&v)[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+  __device__ static void store(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <>
+struct VecIO<_Float16, 1> {
+  __device__ static void load(const _Float16* p, float (&v)[1]) {
+    v[0] = static_cast<float>(*p);
+  }
+  __device__ static void store(_Float16* p, const float (&v)[1]) {
+    *p = static_cast<_Float16>(v[0]);
+  }
+};
+template <>
+struct VecIO<_Float16, 4> {
+  typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+  __device__ static void load(const _Float16* p, float (&v)[4]) {
+    const half4 t = *reinterpret_cast<const half4*>(p);
+    v[0] = static_cast<float>(t.x); v[1] = static_cast<float>(t.y);
+    v[2] = static_cast<float>(t.z); v[3] = static_cast<float>(t.w);
+  }
+  __device__ static void store(_Float16* p, const float (&v)[4]) {
+    half4 t;
+    t.x = static_cast<_Float16>(v[0]); t.y = static_cast<_Float16>(v[1]);
+    t.z = static_cast<_Float16>(v[2]); t.w = static_cast<_Float16>(v[3]);
+    *reinterpret_cast<half4*>(p) = t;
+  }
+};
+
+template <typename T, typename Op, int VEC>
+__global__ void __launch_bounds__(256)
+    pool_forward_kernel(const T* __restrict__ in, T* __restrict__ out,
+                        snn_hip_pooling_params p, size_t n_vec) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n_vec) return;
+  const int C = p.channels;
+  const int cv = C / VEC;
+  const int c = static_cast<int>(idx % cv) * VEC;
+  size_t pix = idx / cv;
+  const int ox = static_cast<int>(pix % p.out_cols);
+  pix /= p.out_cols;
+  const int oy = static_cast<int>(pix % p.out_rows);
+  const int n = static_cast<int>(pix / p.out_rows);
+  int r0 = oy * p.stride_rows - p.pad_rows;
+  const int r1 = min(r0 + p.window_rows, p.in_rows);
+  r0 = max(r0, 0);
+  int c0 = ox * p.stride_cols - p.pad_cols;
+  const int c1 = min(c0 + p.window_cols, p.in_cols);
+  c0 = max(c0, 0);
+  const T* in_n = in + static_cast<size_t>(n) * p.in_rows * p.in_cols * C + c;
+  Op op[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) op[i].init(lowest_of<T>());
+  for (int r = r0; r < r1; ++r) {
+    for (int col = c0; col < c1; ++col) {
+      float v[VEC];
+      VecIO<T, VEC>::load(in_n + (static_cast<size_t>(r) * p.in_cols + col) * C,
+                          v);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) op[i].accumulate(v[i]);
+    }
+  }
+  const int tally = (r1 - r0) * (c1 - c0);
+  float res[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) res[i] = op[i].value(tally);
+  VecIO<T, VEC>::store(out + idx * VEC, res);
+}
+
+__device__ inline bool pool_equal(float a, float b, bool nan_mode) {
+  return a == b || (nan_mode && a != a && b != b);
+}
+
+// Max gradient: one lane per input element.  For every output whose window
+// covers this element and whose value equals it, the gradient is taken only if
+// no earlier element of that window (row-major) also equals the output -- the
+// first maximum wins (src/pooling/kernels.h:141-239).
+__global__ void __launch_bounds__(256)
+    pool_max_grad_kernel(const float* __restrict__ in,
+                         const float* __restrict__ out,
+                         const float* __restrict__ dy, float* __restrict__ dx,
+                         snn_hip_pooling_params p, bool nan_mode, size_t n_in) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n_in) return;
+  const int C = p.channels;
+  const int ch = static_cast<int>(idx % C);
+  size_t pix = idx / C;
+  const int x = static_cast<int>(pix % p.in_cols);
+  pix /= p.in_cols;
+  const int y = static_cast<int>(pix % p.in_rows);
+  const int n = static_cast<int>(pix / p.in_rows);
+  const float mine = in[idx];
+  const float* in_n =
+      in + static_cast<size_t>(n) * p.in_rows * p.in_cols * C + ch;
+  const size_t out_base =
+      static_cast<size_t>(n) * p.out_rows * p.out_cols * C + ch;
+  // outputs whose (unclipped) window contains y / x
+  const int py = y + p.pad_rows, px = x + p.pad_cols;
+  const int oy_begin =
+      py < p.window_rows ? 0 : (py - p.window_rows) / p.stride_rows + 1;
+  const int oy_end = min(py / p.stride_rows + 1, p.out_rows);
+  const int ox_begin =
+      px < p.window_cols ? 0 : (px - p.window_cols) / p.stride_cols + 1;
+  const int ox_end = min(px / p.stride_cols + 1, p.out_cols);
+  float grad = 0.f;
+  for (int oy = oy_begin; oy < oy_end; ++oy) {
+    int r0 = oy * p.stride_rows - p.pad_rows;
+    const int r1 = min(r0 + p.window_rows, p.in_rows);
+    r0 = max(r0, 0);
+    for (int ox = ox_begin; ox < ox_end; ++ox) {
+      int c0 = ox * p.stride_cols - p.pad_cols;
+      const int c1 = min(c0 + p.window_cols, p.in_cols);
+      c0 = max(c0, 0);
+      const size_t o = out_base + (static_cast<size_t>(oy) * p.out_cols + ox) * C;
+      const float target = out[o];
+      if (!pool_equal(mine, target, nan_mode)) continue;
+      bool first = true;
+      for (int r = r0; r < r1 && first; ++r) {
+        for (int col = c0; col < c1; ++col) {
+          if (r == y && col == x) {
+            r = r1;  // reached this element: nothing earlier matched
+            break;
+          }
+          if (pool_equal(in_n[(static_cast<size_t>(r) * p.in_cols + col) * C],
+                         target, nan_mode)) {
+            first = false;
+            break;
+          }
+        }
+      }
+      if (first) grad += dy[o];
+    }
+  }
+  dx[idx] = grad;
+}
+
+// Average gradient: every covering output contributes dY / clipped window
+// size (src/pooling/kernels.h:291-414).
+__global__ void __launch_bounds__(256)
+    pool_avg_grad_kernel(const float* __restrict__ dy, float* __restrict__ dx,
+                         snn_hip_pooling_params p, size_t n_in) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n_in) return;
+  const int C = p.channels;
+  const int ch = static_cast<int>(idx % C);
+  size_t pix = idx / C;
+  const int x = static_cast<int>(pix % p.in_cols);
+  pix /= p.in_cols;
+  const int y = static_cast<int>(pix % p.in_rows);
+  const int n = static_cast<int>(pix / p.in_rows);
+  const size_t out_base =
+      static_cast<size_t>(n) * p.out_rows * p.out_cols * C + ch;
+  const int py = y + p.pad_rows, px = x + p.pad_cols;
+  const int oy_begin =
+      py < p.window_rows ? 0 : (py - p.window_rows) / p.stride_rows + 1;
+  const int oy_end = min(py / p.stride_rows + 1, p.out_rows);
+  const int ox_begin =
+      px < p.window_cols ? 0 : (px - p.window_cols) / p.stride_cols + 1;
+  const int ox_end = min(px / p.stride_cols + 1, p.out_cols);
+  float grad = 0.f;
+  for (int oy = oy_begin; oy < oy_end; ++oy) {
+    int r0 = oy * p.stride_rows - p.pad_rows;
+    const int r1 = min(r0 + p.window_rows, p.in_rows);
+    r0 = max(r0, 0);
+    for (int ox = ox_begin; ox < ox_end; ++ox) {
+      int c0 = ox * p.stride_cols - p.pad_cols;
+      const int c1 = min(c0 + p.window_cols, p.in_cols);
+      c0 = max(c0, 0);
+      const float count = static_cast<float>((r1 - r0) * (c1 - c0));
+      grad += dy[out_base + (static_cast<size_t>(oy) * p.out_cols + ox) * C] /
+              count;
+    }
+  }
+  dx[idx] = grad;
+}
+
+template <typename T, typename Op>
+int launch_forward_op(const T* input, T* output,
+                      const snn_hip_pooling_params& p, hipStream_t stream) {
+  constexpr int kBlock = 256;
+  const size_t n_out =
+      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * p.channels;
+  if (p.channels % 4 == 0) {
+    const size_t n_vec = n_out / 4;
+    hipLaunchKernelGGL((pool_forward_kernel<T, Op, 4>),
+                       dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{kBlock}))),
+                       dim3(kBlock), 0, stream, input, output, p, n_vec);
+  } else {
+    hipLaunchKernelGGL((pool_forward_kernel<T, Op, 1>),
+                       dim3(static_cast<unsigned>(ceil_div(n_out, size_t{kBlock}))),
+                       dim3(kBlock), 0, stream, input, output, p, n_out);
+  }
+  SNN_HIP_CHECK_LAUNCH();
+  return SNN_HIP_OK;
+}
+
+}  // namespace
+
+template <typename T>
+int launch_pooling_forward(const T* input, T* output,
+                           const snn_hip_pooling_params& p, int op,
+                           hipStream_t stream) {
+  switch (op) {
+    case SNN_HIP_POOL_MAX:
+      return launch_forward_op<T, MaxOp>(input, output, p, stream);
+    case SNN_HIP_POOL_MAX_WITH_NAN:
+      return launch_forward_op<T, MaxNanOp>(input, output, p, stream);
+    case SNN_HIP_POOL_AVERAGE:
+      return launch_forward_op<T, AvgOp>(input, output, p, stream);
+    default:
+      return SNN_HIP_INVALID_PARAMETER;
+  }
+}
+
+template int launch_pooling_forward<float>(const float*, float*,
+                                           const snn_hip_pooling_params&, int,
+                                           hipStream_t);
+template int launch_pooling_forward<_Float16>(const _Float16*, _Float16*,
+                                              const snn_hip_pooling_params&,
+                                              int, hipStream_t);
+
+int launch_pooling_max_grad(const float* input_data, const float* output_data,
+                            const float* input_backprop,
+                            float* output_backprop,
+                            const snn_hip_pooling_params& p, int op,
+                            hipStream_t stream) {
+  constexpr int kBlock = 256;
+  const size_t n_in =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
+  hipLaunchKernelGGL(pool_max_grad_kernel,
+                     dim3(static_cast<unsigned>(ceil_div(n_in, size_t{kBlock}))),
+                     dim3(kBlock), 0, stream, input_data, output_data,
+                     input_backprop, output_backprop, p,
+                     op == SNN_HIP_POOL_MAX_WITH_NAN, n_in);
+  SNN_HIP_CHECK_LAUNCH();
+  return SNN_HIP_OK;
+}
+
+int launch_pooling_avg_grad(const float* input_backprop,
+                            float* output_backprop,
+                            const snn_hip_pooling_params& p,
+                            hipStream_t stream) {
+  constexpr int kBlock = 256;
+  const size_t n_in =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
+  hipLaunchKernelGGL(pool_avg_grad_kernel,
+                     dim3(static_cast<unsigned>(ceil_div(n_in, size_t{kBlock}))),
+                     dim3(kBlock), 0, stream, input_backprop, output_backprop,
+                     p, n_in);
+  SNN_HIP_CHECK_LAUNCH();
+  return SNN_HIP_OK;
+}
+
+}  // namespace snn

@@ -1,0 +1,504 @@
+// The C ABI of libsnn_hip.so: parameter validation, algorithm support rules,
+// workspace sizing and dispatch to the kernel launchers.
+#include <cstring>
+#include <string>
+
+#include "snn_kernels.h"
+
+namespace snn {
+
+namespace {
+thread_local std::string g_last_error;
+}
+
+int report_hip_error(hipError_t err, const char* what) {
+  g_last_error = std::string(hipGetErrorName(err)) + ": " +
+                 hipGetErrorString(err) + " in " + what;
+  return SNN_HIP_DEVICE_ERROR;
+}
+
+// include/portdnn/internal/conv2d/launch.h:42-97.  groups == 0 passes the
+// reference's `>= 0` check and then divides by zero there; it is rejected here.
+int validate(const snn_hip_conv2d_params& p) {
+  SNN_REQUIRE(p.batch > 0);
+  SNN_REQUIRE(p.channels > 0);
+  SNN_REQUIRE(p.features > 0);
+  SNN_REQUIRE(p.in_rows > 0);
+  SNN_REQUIRE(p.in_cols > 0);
+  SNN_REQUIRE(p.out_rows > 0);
+  SNN_REQUIRE(p.out_cols > 0);
+  SNN_REQUIRE(p.window_rows > 0);
+  SNN_REQUIRE(p.window_cols > 0);
+  SNN_REQUIRE(p.stride_rows > 0);
+  SNN_REQUIRE(p.stride_cols > 0);
+  SNN_REQUIRE(p.pad_rows >= 0);
+  SNN_REQUIRE(p.pad_cols >= 0);
+  SNN_REQUIRE(p.groups > 0);
+  SNN_REQUIRE(p.channels % p.groups == 0);
+  SNN_REQUIRE(p.features % p.groups == 0);
+  SNN_REQUIRE(p.dilation_rows == 1);
+  SNN_REQUIRE(p.dilation_cols == 1);
+  // Layout combinations: NHWC goes with HWCF (0) or FHWC (2), NCHW (1) with
+  // FCHW (1); INTERLEAVED (1) groups need groups > 1 and HWCF.
+  SNN_REQUIRE(p.input_format == 0 || p.input_format == 1);
+  SNN_REQUIRE(p.input_format != 0 ||
+              (p.filter_format == 0 || p.filter_format == 2));
+  SNN_REQUIRE(p.input_format != 1 || p.filter_format == 1);
+  SNN_REQUIRE(p.groups != 1 || p.group_format == 0);
+  SNN_REQUIRE(p.group_format != 1 || p.filter_format == 0);
+  return SNN_HIP_OK;
+}
+
+// include/portdnn/internal/depthwise_conv2d/launch.h:82-112
+int validate(const snn_hip_depthwise_params& p) {
+  SNN_REQUIRE(p.batch > 0);
+  SNN_REQUIRE(p.channels > 0);
+  SNN_REQUIRE(p.channel_multiplier > 0);
+  SNN_REQUIRE(p.in_rows > 0);
+  SNN_REQUIRE(p.in_cols > 0);
+  SNN_REQUIRE(p.out_rows > 0);
+  SNN_REQUIRE(p.out_cols > 0);
+  SNN_REQUIRE(p.window_rows > 0);
+  SNN_REQUIRE(p.window_cols > 0);
+  SNN_REQUIRE(p.stride_rows > 0);
+  SNN_REQUIRE(p.stride_cols > 0);
+  SNN_REQUIRE(p.pad_rows >= 0);
+  SNN_REQUIRE(p.pad_cols >= 0);
+  SNN_REQUIRE(p.input_format == 0);   // NHWC only
+  SNN_REQUIRE(p.filter_format == 0);  // HWCF only
+  return SNN_HIP_OK;
+}
+
+// include/portdnn/pooling/launch.h:56-88.  NCHW is accepted by the reference
+// for Forward only; this library implements NHWC and reports NCHW as an
+// invalid parameter in both directions.
+int validate(const snn_hip_pooling_params& p, bool /*forward*/) {
+  SNN_REQUIRE(p.batch > 0);
+  SNN_REQUIRE(p.channels > 0);
+  SNN_REQUIRE(p.in_rows > 0);
+  SNN_REQUIRE(p.in_cols > 0);
+  SNN_REQUIRE(p.out_rows > 0);
+  SNN_REQUIRE(p.out_cols > 0);
+  SNN_REQUIRE(p.window_rows > 0);
+  SNN_REQUIRE(p.window_cols > 0);
+  SNN_REQUIRE(p.stride_rows > 0);
+  SNN_REQUIRE(p.stride_cols > 0);
+  SNN_REQUIRE(p.pad_rows >= 0);
+  SNN_REQUIRE(p.pad_cols >= 0);
+  SNN_REQUIRE(p.input_format == 0);
+  return SNN_HIP_OK;
+}
+
+namespace {
+
+struct ConvSizes {
+  size_t input, filter, output;
+};
+
+// include/portdnn/conv2d/sizes.h:166-179 for groups == 1.
+ConvSizes conv_sizes(const snn_hip_conv2d_params& p, int direction) {
+  const size_t x = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                   p.channels;
+  const size_t w = static_cast<size_t>(p.window_rows) * p.window_cols *
+                   p.channels * p.features;
+  const size_t y = static_cast<size_t>(p.batch) * p.out_rows * p.out_cols *
+                   p.features;
+  switch (direction) {
+    case SNN_HIP_FORWARD: return {x, w, y};
+    case SNN_HIP_INPUT_BACKPROP: return {y, w, x};
+    default: return {x, y, w};
+  }
+}
+
+// The concrete selectors of include/portdnn/conv2d/selector/.
+int algorithm_supports(const snn_hip_conv2d_params& p, int direction,
+                       int algorithm) {
+  const bool nhwc = p.input_format == 0 && p.filter_format == 0;
+  switch (algorithm) {
+    case SNN_HIP_ALGO_DIRECT:
+    case SNN_HIP_ALGO_IM2COL:
+      // constant_selector.h: always selected.
+      return algorithm;
+    case SNN_HIP_ALGO_TILED:
+      // tiled_selector.h:45-96: Forward only, square window and stride,
+      // (window, stride) in {(1,1),(1,2),(3,1),(3,2),(5,1)}.
+      if (direction != SNN_HIP_FORWARD) return SNN_HIP_ALGO_NOT_SUPPORTED;
+      if (p.window_rows != p.window_cols || p.stride_rows != p.stride_cols)
+        return SNN_HIP_ALGO_NOT_SUPPORTED;
+      if ((p.window_rows == 1 || p.window_rows == 3) &&
+          (p.stride_rows == 1 || p.stride_rows == 2))
+        return algorithm;
+      if (p.window_rows == 5 && p.stride_rows == 1) return algorithm;
+      return SNN_HIP_ALGO_NOT_SUPPORTED;
+    case SNN_HIP_ALGO_WINOGRAD:
+    case SNN_HIP_ALGO_WINOGRAD_LARGE:
+      // winograd_selector.h:44-182.  The reference rejects a stride only when
+      // BOTH strides differ from 1 (a logical AND there) and then computes a
+      // stride-1 result; here both strides must be 1.
+      if (p.stride_rows != 1 || p.stride_cols != 1)
+        return SNN_HIP_ALGO_NOT_SUPPORTED;
+      if (algorithm == SNN_HIP_ALGO_WINOGRAD &&
+          ((p.window_rows == 1 && p.window_cols == 3) ||
+           (p.window_rows == 3 && p.window_cols == 1)))
+        return algorithm;
+      if (p.window_rows == 3 && p.window_cols == 3) return algorithm;
+      return SNN_HIP_ALGO_NOT_SUPPORTED;
+    case SNN_HIP_ALGO_MATMUL:
+      // matmul_selector.h:44-100
+      if (p.stride_rows == 1 && p.stride_cols == 1 && p.window_rows == 1 &&
+          p.window_cols == 1 && p.pad_rows == 0 && p.pad_cols == 0 && nhwc)
+        return algorithm;
+      return SNN_HIP_ALGO_NOT_SUPPORTED;
+    default:
+      return SNN_HIP_ALGO_NOT_SUPPORTED;
+  }
+}
+
+int round_up_div(int a, int b) { return a < 0 ? 0 : (a + b - 1) / b; }
+
+// include/portdnn/conv2d/workspace_size.h:53-76 with the kernel parameters of
+// internal/conv2d/winograd/kernel_params.h:39-63 and the tile counts of
+// internal/conv2d/winograd/tile_info.h:48-75.
+void winograd_workspace(const snn_hip_conv2d_params& p, int direction, int m,
+                        int n, int r, int s, size_t* required,
+                        size_t* recommended) {
+  int channels = p.channels, features = p.features;
+  int out_rows = p.out_rows, out_cols = p.out_cols;
+  if (direction == SNN_HIP_INPUT_BACKPROP) {
+    channels = p.features;
+    features = p.channels;
+    out_rows = p.in_rows;
+    out_cols = p.in_cols;
+  }
+  // Forward / input backprop tile the output in m x n blocks.  For the filter
+  // gradient out <-> window are swapped and the tiles cover the swapped
+  // window -- the original output extent -- in r x s blocks
+  // (tile_info.h:62-73).
+  const bool filbk = direction == SNN_HIP_FILTER_BACKPROP;
+  const size_t a = m + r - 1, b = n + s - 1;
+  const size_t tiles =
+      static_cast<size_t>(round_up_div(out_rows, filbk ? r : m)) *
+      round_up_div(out_cols, filbk ? s : n);
+  const size_t in_t = a * b * tiles * channels;
+  const size_t inter_t = a * b * tiles * features;
+  const size_t fil_t = a * b * channels * features;
+  *required = in_t + inter_t + fil_t;
+  *recommended = static_cast<size_t>(p.batch) * (in_t + inter_t) + fil_t;
+}
+
+// include/portdnn/conv2d/workspace_size.h:100-121 with
+// internal/conv2d/im2col/{tile_info.h,transform_sizes.h} for groups == 1.
+void im2col_workspace(const snn_hip_conv2d_params& p, int direction,
+                      size_t* required, size_t* recommended) {
+  size_t tiles, tile_size, filter_t = 0;
+  const size_t win = static_cast<size_t>(p.window_rows) * p.window_cols;
+  if (direction == SNN_HIP_FORWARD) {
+    tiles = static_cast<size_t>(p.out_rows) * p.out_cols;
+    tile_size = win * p.channels;
+  } else if (direction == SNN_HIP_INPUT_BACKPROP) {
+    tiles = static_cast<size_t>(p.in_rows) * p.in_cols;
+    tile_size = win * p.features;
+    filter_t = win * p.channels * p.features;
+  } else {
+    tiles = win * p.channels;
+    tile_size = static_cast<size_t>(p.out_rows) * p.out_cols;
+  }
+  const size_t in_t = tiles * tile_size;
+  *required = in_t + filter_t;
+  *recommended = static_cast<size_t>(p.batch) * in_t + filter_t;
+}
+
+int workspace_size(const snn_hip_conv2d_params& p, int direction,
+                   int algorithm, size_t* required, size_t* recommended) {
+  *required = 0;
+  *recommended = 0;
+  const bool filbk = direction == SNN_HIP_FILTER_BACKPROP;
+  switch (algorithm) {
+    case SNN_HIP_ALGO_WINOGRAD:
+      // F(2x2,3x3), or F(3x3,2x2) for the filter gradient
+      // (workspace_size.h:78-87).
+      if (filbk)
+        winograd_workspace(p, direction, 3, 3, 2, 2, required, recommended);
+      else
+        winograd_workspace(p, direction, 2, 2, 3, 3, required, recommended);
+      break;
+    case SNN_HIP_ALGO_WINOGRAD_LARGE:
+      if (filbk)
+        winograd_workspace(p, direction, 3, 3, 3, 3, required, recommended);
+      else
+        winograd_workspace(p, direction, 4, 4, 3, 3, required, recommended);
+      break;
+    case SNN_HIP_ALGO_IM2COL:
+      im2col_workspace(p, direction, required, recommended);
+      break;
+    default:
+      break;
+  }
+  return SNN_HIP_OK;
+}
+
+// Device policy standing in for get_default_selector
+// (src/conv2d/selector/default_selector.cc:49-128): 1x1 stride-1 unpadded
+// convolutions are one GEMM; everything else is the implicit-GEMM path, which
+// the Im2col tag names (Tiled where the reference's TiledSelector accepts it).
+int default_algorithm(const snn_hip_conv2d_params& p, int direction) {
+  if (algorithm_supports(p, direction, SNN_HIP_ALGO_MATMUL))
+    return SNN_HIP_ALGO_MATMUL;
+  if (algorithm_supports(p, direction, SNN_HIP_ALGO_TILED))
+    return SNN_HIP_ALGO_TILED;
+  return SNN_HIP_ALGO_IM2COL;
+}
+
+template <typename T>
+int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
+                    const snn_hip_conv2d_params* params, int algorithm,
+                    T* workspace, size_t workspace_elems, void* stream) {
+  if (params == nullptr) return SNN_HIP_INVALID_PARAMETER;
+  const snn_hip_conv2d_params& p = *params;
+  const int v = validate(p);
+  if (v != SNN_HIP_OK) return v;
+  if (input == nullptr || filter == nullptr || output == nullptr)
+    return SNN_HIP_INVALID_PARAMETER;
+  // Grouped, NCHW and FHWC convolutions are outside this library.
+  if (p.groups != 1 || p.input_format != 0 || p.filter_format != 0)
+    return SNN_HIP_INVALID_ALGORITHM;
+  if (algorithm_supports(p, direction, algorithm) == SNN_HIP_ALGO_NOT_SUPPORTED)
+    return SNN_HIP_INVALID_ALGORITHM;
+  const ConvSizes sz = conv_sizes(p, direction);
+  if (!fits_int32(sz.input) || !fits_int32(sz.filter) || !fits_int32(sz.output))
+    return SNN_HIP_INDEX_EXCEEDED;
+  hipStream_t s = as_stream(stream);
+  (void)workspace;
+  (void)workspace_elems;
+  switch (algorithm) {
+    case SNN_HIP_ALGO_WINOGRAD:
+    case SNN_HIP_ALGO_WINOGRAD_LARGE:
+      if (workspace == nullptr || workspace_elems == 0)
+        return SNN_HIP_INSUFFICIENT_WORKSPACE;
+      return launch_conv2d_direct<T>(direction, input, filter, output, p, s);
+    default:
+      return launch_conv2d_direct<T>(direction, input, filter, output, p, s);
+  }
+}
+
+template <typename T>
+int depthwise_dispatch(int direction, const T* input, const T* filter,
+                       T* output, const snn_hip_depthwise_params* params,
+                       void* stream) {
+  if (params == nullptr) return SNN_HIP_INVALID_PARAMETER;
+  const int v = validate(*params);
+  if (v != SNN_HIP_OK) return v;
+  if (input == nullptr || filter == nullptr || output == nullptr)
+    return SNN_HIP_INVALID_PARAMETER;
+  const snn_hip_depthwise_params& p = *params;
+  const size_t cm = static_cast<size_t>(p.channels) * p.channel_multiplier;
+  if (!fits_int32(static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                  p.channels) ||
+      !fits_int32(static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * cm))
+    return SNN_HIP_INDEX_EXCEEDED;
+  return launch_depthwise<T>(direction, input, filter, output, p,
+                             as_stream(stream));
+}
+
+int pooling_check(const snn_hip_pooling_params* params, bool forward) {
+  if (params == nullptr) return SNN_HIP_INVALID_PARAMETER;
+  const int v = validate(*params, forward);
+  if (v != SNN_HIP_OK) return v;
+  const snn_hip_pooling_params& p = *params;
+  if (!fits_int32(static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                  p.channels) ||
+      !fits_int32(static_cast<size_t>(p.batch) * p.out_rows * p.out_cols *
+                  p.channels))
+    return SNN_HIP_INDEX_EXCEEDED;
+  return SNN_HIP_OK;
+}
+
+}  // namespace
+}  // namespace snn
+
+using namespace snn;
+
+extern "C" {
+
+int snn_hip_version(void) { return 100; }  // 0.1.0
+
+const char* snn_hip_status_string(int status) {
+  switch (status) {
+    case SNN_HIP_OK: return "OK";
+    case SNN_HIP_INVALID_ALGORITHM: return "InvalidAlgorithm";
+    case SNN_HIP_INDEX_EXCEEDED: return "IndexExceeded";
+    case SNN_HIP_INSUFFICIENT_WORKSPACE: return "InsufficientWorkspace";
+    case SNN_HIP_ALLOCATION_PROBLEM: return "AllocationProblem";
+    case SNN_HIP_INVALID_PARAMETER: return "InvalidParameter";
+    case SNN_HIP_DEVICE_ERROR: return "DeviceError";
+    default: return "Unknown";
+  }
+}
+
+const char* snn_hip_last_error(void) { return g_last_error.c_str(); }
+
+int snn_hip_conv2d_forward_f32(const float* input, const float* filter,
+                               float* output,
+                               const snn_hip_conv2d_params* params,
+                               int algorithm, float* workspace,
+                               size_t workspace_elems, void* stream) {
+  return conv2d_dispatch<float>(SNN_HIP_FORWARD, input, filter, output, params,
+                                algorithm, workspace, workspace_elems, stream);
+}
+
+int snn_hip_conv2d_input_backprop_f32(const float* input, const float* filter,
+                                      float* output,
+                                      const snn_hip_conv2d_params* params,
+                                      int algorithm, float* workspace,
+                                      size_t workspace_elems, void* stream) {
+  return conv2d_dispatch<float>(SNN_HIP_INPUT_BACKPROP, input, filter, output,
+                                params, algorithm, workspace, workspace_elems,
+                                stream);
+}
+
+int snn_hip_conv2d_filter_backprop_f32(const float* input, const float* filter,
+                                       float* output,
+                                       const snn_hip_conv2d_params* params,
+                                       int algorithm, float* workspace,
+                                       size_t workspace_elems, void* stream) {
+  return conv2d_dispatch<float>(SNN_HIP_FILTER_BACKPROP, input, filter, output,
+                                params, algorithm, workspace, workspace_elems,
+                                stream);
+}
+
+int snn_hip_conv2d_forward_f16(const void* input, const void* filter,
+                               void* output,
+                               const snn_hip_conv2d_params* params,
+                               int algorithm, void* workspace,
+                               size_t workspace_elems, void* stream) {
+  return conv2d_dispatch<_Float16>(
+      SNN_HIP_FORWARD, static_cast<const _Float16*>(input),
+      static_cast<const _Float16*>(filter), static_cast<_Float16*>(output),
+      params, algorithm, static_cast<_Float16*>(workspace), workspace_elems,
+      stream);
+}
+
+int snn_hip_conv2d_workspace_size(const snn_hip_conv2d_params* params,
+                                  int direction, int algorithm,
+                                  size_t* required_elems,
+                                  size_t* recommended_elems) {
+  if (params == nullptr || required_elems == nullptr ||
+      recommended_elems == nullptr)
+    return SNN_HIP_INVALID_PARAMETER;
+  if (direction < SNN_HIP_FORWARD || direction > SNN_HIP_FILTER_BACKPROP)
+    return SNN_HIP_INVALID_PARAMETER;
+  return workspace_size(*params, direction, algorithm, required_elems,
+                        recommended_elems);
+}
+
+int snn_hip_conv2d_algorithm_supports(const snn_hip_conv2d_params* params,
+                                      int direction, int algorithm) {
+  if (params == nullptr) return SNN_HIP_ALGO_NOT_SUPPORTED;
+  return algorithm_supports(*params, direction, algorithm);
+}
+
+int snn_hip_conv2d_default_algorithm(const snn_hip_conv2d_params* params,
+                                     int direction) {
+  if (params == nullptr) return SNN_HIP_ALGO_NOT_SUPPORTED;
+  return default_algorithm(*params, direction);
+}
+
+int snn_hip_depthwise_conv2d_forward_f32(
+    const float* input, const float* filter, float* output,
+    const snn_hip_depthwise_params* params, void* stream) {
+  return depthwise_dispatch<float>(SNN_HIP_FORWARD, input, filter, output,
+                                   params, stream);
+}
+
+int snn_hip_depthwise_conv2d_input_backprop_f32(
+    const float* input, const float* filter, float* output,
+    const snn_hip_depthwise_params* params, void* stream) {
+  return depthwise_dispatch<float>(SNN_HIP_INPUT_BACKPROP, input, filter,
+                                   output, params, stream);
+}
+
+int snn_hip_depthwise_conv2d_filter_backprop_f32(
+    const float* input, const float* filter, float* output,
+    const snn_hip_depthwise_params* params, void* stream) {
+  return depthwise_dispatch<float>(SNN_HIP_FILTER_BACKPROP, input, filter,
+                                   output, params, stream);
+}
+
+int snn_hip_depthwise_conv2d_forward_f16(
+    const void* input, const void* filter, void* output,
+    const snn_hip_depthwise_params* params, void* stream) {
+  return depthwise_dispatch<_Float16>(
+      SNN_HIP_FORWARD, static_cast<const _Float16*>(input),
+      static_cast<const _Float16*>(filter), static_cast<_Float16*>(output),
+      params, stream);
+}
+
+int snn_hip_pooling_forward_f32(const float* input, float* output,
+                                const snn_hip_pooling_params* params, int op,
+                                void* stream) {
+  const int v = pooling_check(params, true);
+  if (v != SNN_HIP_OK) return v;
+  if (input == nullptr || output == nullptr) return SNN_HIP_INVALID_PARAMETER;
+  return launch_pooling_forward<float>(input, output, *params, op,
+                                       as_stream(stream));
+}
+
+int snn_hip_pooling_forward_f16(const void* input, void* output,
+                                const snn_hip_pooling_params* params, int op,
+                                void* stream) {
+  const int v = pooling_check(params, true);
+  if (v != SNN_HIP_OK) return v;
+  if (input == nullptr || output == nullptr) return SNN_HIP_INVALID_PARAMETER;
+  return launch_pooling_forward<_Float16>(
+      static_cast<const _Float16*>(input), static_cast<_Float16*>(output),
+      *params, op, as_stream(stream));
+}
+
+int snn_hip_pooling_max_grad_f32(const float* input_data,
+                                 const float* output_data,
+                                 const float* input_backprop,
+                                 float* output_backprop,
+                                 const snn_hip_pooling_params* params, int op,
+                                 void* stream) {
+  const int v = pooling_check(params, false);
+  if (v != SNN_HIP_OK) return v;
+  if (input_data == nullptr || output_data == nullptr ||
+      input_backprop == nullptr || output_backprop == nullptr)
+    return SNN_HIP_INVALID_PARAMETER;
+  if (op != SNN_HIP_POOL_MAX && op != SNN_HIP_POOL_MAX_WITH_NAN)
+    return SNN_HIP_INVALID_PARAMETER;
+  return launch_pooling_max_grad(input_data, output_data, input_backprop,
+                                 output_backprop, *params, op,
+                                 as_stream(stream));
+}
+
+int snn_hip_pooling_avg_grad_f32(const float* input_backprop,
+                                 float* output_backprop,
+                                 const snn_hip_pooling_params* params,
+                                 void* stream) {
+  const int v = pooling_check(params, false);
+  if (v != SNN_HIP_OK) return v;
+  if (input_backprop == nullptr || output_backprop == nullptr)
+    return SNN_HIP_INVALID_PARAMETER;
+  return launch_pooling_avg_grad(input_backprop, output_backprop, *params,
+                                 as_stream(stream));
+}
+
+int snn_hip_matmul_f32(const float* lhs, const float* rhs, float* output,
+                       int batches, int m, int k, int n, int transpose_lhs,
+                       int transpose_rhs, float beta, void* stream) {
+  if (lhs == nullptr || rhs == nullptr || output == nullptr)
+    return SNN_HIP_INVALID_PARAMETER;
+  // include/portdnn/matmul/launch.h validates positive sizes.
+  if (batches <= 0 || m <= 0 || k <= 0 || n <= 0)
+    return SNN_HIP_INVALID_PARAMETER;
+  if (!fits_int32(static_cast<size_t>(batches) * m * k) ||
+      !fits_int32(static_cast<size_t>(batches) * k * n) ||
+      !fits_int32(static_cast<size_t>(batches) * m * n))
+    return SNN_HIP_INDEX_EXCEEDED;
+  return launch_matmul_f32(lhs, rhs, output, batches, m, k, n,
+                           transpose_lhs != 0, transpose_rhs != 0, beta,
+                           as_stream(stream));
+}
+
+}  // extern "C"

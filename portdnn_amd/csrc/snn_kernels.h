@@ -1,0 +1,44 @@
+// Internal launchers behind the C ABI.  Each returns a snn_hip_status and only
+// enqueues work on `stream`.
+#ifndef PORTDNN_AMD_CSRC_SNN_KERNELS_H_
+#define PORTDNN_AMD_CSRC_SNN_KERNELS_H_
+
+#include "snn_common.h"
+
+namespace snn {
+
+// Algorithm::Direct -- any window / stride, all three directions
+// (conv2d_direct.hip).
+template <typename T>
+int launch_conv2d_direct(int direction, const T* input, const T* filter,
+                         T* output, const snn_hip_conv2d_params& p,
+                         hipStream_t stream);
+
+// Depthwise convolution, all three directions (depthwise.hip).
+template <typename T>
+int launch_depthwise(int direction, const T* input, const T* filter, T* output,
+                     const snn_hip_depthwise_params& p, hipStream_t stream);
+
+// Pooling (pooling.hip).
+template <typename T>
+int launch_pooling_forward(const T* input, T* output,
+                           const snn_hip_pooling_params& p, int op,
+                           hipStream_t stream);
+int launch_pooling_max_grad(const float* input_data, const float* output_data,
+                            const float* input_backprop,
+                            float* output_backprop,
+                            const snn_hip_pooling_params& p, int op,
+                            hipStream_t stream);
+int launch_pooling_avg_grad(const float* input_backprop,
+                            float* output_backprop,
+                            const snn_hip_pooling_params& p,
+                            hipStream_t stream);
+
+// Batched row-major GEMM on MFMA (matmul.hip).
+int launch_matmul_f32(const float* lhs, const float* rhs, float* output,
+                      int batches, int m, int k, int n, bool transpose_lhs,
+                      bool transpose_rhs, float beta, hipStream_t stream);
+
+}  // namespace snn
+
+#endif  // PORTDNN_AMD_CSRC_SNN_KERNELS_H_

@@ -1,0 +1,207 @@
+"""Torch-tensor conveniences over the C ABI, used by the tests and bench.py.
+
+torch is plumbing here (device memory and the current HIP stream); every
+computation happens in libsnn_hip.so.  There is no fallback path.
+"""
+import ctypes
+
+import torch
+
+from . import capi
+from .capi import ALGO, DIRECTION, POOL_OP, STATUS, ConvParams, \
+    DepthwiseParams, PoolParams
+
+
+def calculate_padding(inp, window, stride, same):
+    """helpers::calculate_padding (include/portdnn/helpers/padding.h:51-69):
+    returns (padding, output)."""
+    if same:
+        out = (inp + stride - 1) // stride
+        needed = (out - 1) * stride + window - inp
+        return int(needed / 2), out  # C++ integer division truncates
+    num = inp - window + 1
+    q = int(num / stride)
+    return 0, (q if num < 0 else q + (1 if num % stride else 0))
+
+
+def add_padding_to(params, same):
+    """helpers::add_padding_to (include/portdnn/helpers/padding.h:80-92)."""
+    params.pad_rows, params.out_rows = calculate_padding(
+        params.in_rows, params.window_rows, params.stride_rows, same)
+    params.pad_cols, params.out_cols = calculate_padding(
+        params.in_cols, params.window_cols, params.stride_cols, same)
+    return params
+
+
+def conv_params(batch, in_rows, in_cols, channels, features, window, stride,
+                same):
+    return add_padding_to(ConvParams(
+        channels=channels, features=features, batch=batch, in_rows=in_rows,
+        in_cols=in_cols, window_rows=window, window_cols=window,
+        stride_rows=stride, stride_cols=stride), same)
+
+
+def depthwise_params(batch, in_rows, in_cols, channels, multiplier, window,
+                     stride, same):
+    return add_padding_to(DepthwiseParams(
+        channels=channels, channel_multiplier=multiplier, batch=batch,
+        in_rows=in_rows, in_cols=in_cols, window_rows=window,
+        window_cols=window, stride_rows=stride, stride_cols=stride), same)
+
+
+def pool_params(batch, in_rows, in_cols, channels, window, stride, same):
+    return add_padding_to(PoolParams(
+        in_rows=in_rows, in_cols=in_cols, window_rows=window,
+        window_cols=window, stride_rows=stride, stride_cols=stride,
+        batch=batch, channels=channels), same)
+
+
+def conv_sizes(p, direction):
+    """(input, filter, output) element counts, conv2d/sizes.h:166-179."""
+    x = p.batch * p.in_rows * p.in_cols * p.channels
+    w = p.window_rows * p.window_cols * p.channels * p.features
+    y = p.batch * p.out_rows * p.out_cols * p.features
+    if direction == DIRECTION.FORWARD:
+        return x, w, y
+    if direction == DIRECTION.INPUT_BACKPROP:
+        return y, w, x
+    return x, y, w
+
+
+def conv_flops(p, direction):
+    """bench/conv2d/base_convolution_fixture.h:81-109."""
+    if direction == DIRECTION.FORWARD:
+        pix = p.batch * p.out_rows * p.out_cols
+    else:
+        pix = p.batch * p.in_rows * p.in_cols
+    return 2 * pix * p.window_rows * p.window_cols * p.channels * p.features
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def workspace_size(p, direction, algorithm):
+    req, rec = ctypes.c_size_t(), ctypes.c_size_t()
+    capi.check(capi.lib().snn_hip_conv2d_workspace_size(
+        ctypes.byref(p), direction, algorithm, ctypes.byref(req),
+        ctypes.byref(rec)))
+    return req.value, rec.value
+
+
+_CONV_FN = {
+    (DIRECTION.FORWARD, torch.float32): "snn_hip_conv2d_forward_f32",
+    (DIRECTION.INPUT_BACKPROP, torch.float32):
+        "snn_hip_conv2d_input_backprop_f32",
+    (DIRECTION.FILTER_BACKPROP, torch.float32):
+        "snn_hip_conv2d_filter_backprop_f32",
+    (DIRECTION.FORWARD, torch.float16): "snn_hip_conv2d_forward_f16",
+}
+
+
+def conv2d_raw(inp, fil, out, p, direction, algorithm, workspace=None):
+    """Calls the entry point and returns its status code (no exception)."""
+    fn = getattr(capi.lib(), _CONV_FN[(direction, inp.dtype)])
+    ws_elems = 0 if workspace is None else workspace.numel()
+    return fn(_ptr(inp), _ptr(fil), _ptr(out), ctypes.byref(p), algorithm,
+              _ptr(workspace), ws_elems, _stream())
+
+
+def conv2d(inp, fil, p, direction=DIRECTION.FORWARD, algorithm=ALGO.DIRECT,
+           workspace=None, out=None):
+    """inp / fil are flat or shaped device tensors with the operand roles of
+    include/snn_hip.h; returns the flat output tensor."""
+    n_in, n_fil, n_out = conv_sizes(p, direction)
+    assert inp.numel() == n_in and fil.numel() == n_fil, (inp.shape, fil.shape)
+    assert inp.is_contiguous() and fil.is_contiguous()
+    if out is None:
+        out = torch.empty(n_out, dtype=inp.dtype, device=inp.device)
+    if workspace is None and algorithm in (ALGO.WINOGRAD, ALGO.WINOGRAD_LARGE):
+        _, rec = workspace_size(p, direction, algorithm)
+        workspace = torch.empty(rec, dtype=inp.dtype, device=inp.device)
+    capi.check(conv2d_raw(inp, fil, out, p, direction, algorithm, workspace))
+    return out
+
+
+_DW_FN = {
+    (DIRECTION.FORWARD, torch.float32): "snn_hip_depthwise_conv2d_forward_f32",
+    (DIRECTION.INPUT_BACKPROP, torch.float32):
+        "snn_hip_depthwise_conv2d_input_backprop_f32",
+    (DIRECTION.FILTER_BACKPROP, torch.float32):
+        "snn_hip_depthwise_conv2d_filter_backprop_f32",
+    (DIRECTION.FORWARD, torch.float16): "snn_hip_depthwise_conv2d_forward_f16",
+}
+
+
+def depthwise_sizes(p, direction):
+    x = p.batch * p.in_rows * p.in_cols * p.channels
+    w = p.window_rows * p.window_cols * p.channels * p.channel_multiplier
+    y = p.batch * p.out_rows * p.out_cols * p.channels * p.channel_multiplier
+    if direction == DIRECTION.FORWARD:
+        return x, w, y
+    if direction == DIRECTION.INPUT_BACKPROP:
+        return y, w, x
+    return x, y, w
+
+
+def depthwise_conv2d(inp, fil, p, direction=DIRECTION.FORWARD, out=None):
+    n_in, n_fil, n_out = depthwise_sizes(p, direction)
+    assert inp.numel() == n_in and fil.numel() == n_fil
+    if out is None:
+        out = torch.empty(n_out, dtype=inp.dtype, device=inp.device)
+    fn = getattr(capi.lib(), _DW_FN[(direction, inp.dtype)])
+    capi.check(fn(_ptr(inp), _ptr(fil), _ptr(out), ctypes.byref(p), _stream()))
+    return out
+
+
+def pooling_forward(inp, p, op, out=None):
+    assert inp.numel() == p.batch * p.in_rows * p.in_cols * p.channels
+    if out is None:
+        out = torch.empty(p.batch * p.out_rows * p.out_cols * p.channels,
+                          dtype=inp.dtype, device=inp.device)
+    name = ("snn_hip_pooling_forward_f32" if inp.dtype == torch.float32 else
+            "snn_hip_pooling_forward_f16")
+    capi.check(getattr(capi.lib(), name)(_ptr(inp), _ptr(out), ctypes.byref(p),
+                                         op, _stream()))
+    return out
+
+
+def pooling_max_grad(inp, out, dy, p, op=POOL_OP.MAX):
+    dx = torch.empty_like(inp)
+    capi.check(capi.lib().snn_hip_pooling_max_grad_f32(
+        _ptr(inp), _ptr(out), _ptr(dy), _ptr(dx), ctypes.byref(p), op,
+        _stream()))
+    return dx
+
+
+def pooling_avg_grad(dy, p):
+    dx = torch.empty(p.batch * p.in_rows * p.in_cols * p.channels,
+                     dtype=dy.dtype, device=dy.device)
+    capi.check(capi.lib().snn_hip_pooling_avg_grad_f32(
+        _ptr(dy), _ptr(dx), ctypes.byref(p), _stream()))
+    return dx
+
+
+def matmul(a, b, batches, m, k, n, trans_a=False, trans_b=False, beta=0.0,
+           out=None):
+    assert a.numel() == batches * m * k and b.numel() == batches * k * n
+    if out is None:
+        out = torch.zeros(batches * m * n, dtype=a.dtype, device=a.device)
+    capi.check(capi.lib().snn_hip_matmul_f32(
+        _ptr(a), _ptr(b), _ptr(out), batches, m, k, n, int(trans_a),
+        int(trans_b), float(beta), _stream()))
+    return out
+
+
+__all__ = [
+    "ALGO", "DIRECTION", "POOL_OP", "STATUS", "ConvParams", "DepthwiseParams",
+    "PoolParams", "add_padding_to", "calculate_padding", "conv2d",
+    "conv2d_raw", "conv_flops", "conv_params", "conv_sizes",
+    "depthwise_conv2d", "depthwise_params", "depthwise_sizes", "matmul",
+    "pool_params", "pooling_avg_grad", "pooling_forward", "pooling_max_grad",
+    "workspace_size",
+]

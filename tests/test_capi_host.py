@@ -1,0 +1,230 @@
+"""Host-side checks of the C ABI that need no GPU: the library loads, exports
+every symbol include/snn_hip.h declares, and its host logic (validation,
+selector rules, workspace sizes, status codes) follows the reference."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from golden_cases import GOLDEN_DIR
+from portdnn_amd import capi, ops
+from portdnn_amd.capi import ALGO, DIRECTION, STATUS
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FAKE = ctypes.c_void_p(0x1000)  # never dereferenced: every call returns early
+
+
+def declared_symbols():
+    with open(os.path.join(ROOT, "include", "snn_hip.h")) as f:
+        text = f.read()
+    return sorted(set(re.findall(r"\b(snn_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported():
+    names = declared_symbols()
+    assert len(names) >= 19
+    L = capi.lib()
+    for name in names:
+        assert hasattr(L, name), name
+    assert sorted(capi.SIGNATURES) == names
+
+
+def test_version_and_status_strings():
+    L = capi.lib()
+    assert L.snn_hip_version() >= 100
+    # portDNN StatusCode order, include/portdnn/status.h:31-44
+    expected = ["OK", "InvalidAlgorithm", "IndexExceeded",
+                "InsufficientWorkspace", "AllocationProblem",
+                "InvalidParameter", "DeviceError"]
+    assert [capi.status_string(i) for i in range(7)] == expected
+
+
+def test_python_padding_helper_matches_reference_known_answers():
+    rows = np.load(os.path.join(GOLDEN_DIR, "padding_kat.npz"))["rows"]
+    for same, window, stride, inp, pad, out in rows.tolist():
+        assert ops.calculate_padding(inp, window, stride, same) == (pad, out)
+
+
+def _conv(**kw):
+    p = ops.conv_params(2, 8, 8, 4, 4, 3, 1, True)
+    for k, v in kw.items():
+        setattr(p, k, v)
+    return p
+
+
+def _call_conv(p, algo=ALGO.DIRECT, direction=DIRECTION.FORWARD, ws=None,
+               ws_elems=0):
+    name = {0: "snn_hip_conv2d_forward_f32",
+            1: "snn_hip_conv2d_input_backprop_f32",
+            2: "snn_hip_conv2d_filter_backprop_f32"}[direction]
+    return getattr(capi.lib(), name)(FAKE, FAKE, FAKE, ctypes.byref(p), algo,
+                                     ws, ws_elems, None)
+
+
+@pytest.mark.parametrize("field,value", [
+    ("batch", 0), ("channels", 0), ("features", -1), ("in_rows", 0),
+    ("in_cols", 0), ("out_rows", 0), ("out_cols", -3), ("window_rows", 0),
+    ("window_cols", 0), ("stride_rows", 0), ("stride_cols", 0),
+    ("pad_rows", -1), ("pad_cols", -1), ("dilation_rows", 2),
+    ("dilation_cols", 0), ("groups", 3), ("groups", 0),
+])
+def test_conv2d_invalid_parameter(field, value):
+    """include/portdnn/internal/conv2d/launch.h:42-97"""
+    assert _call_conv(_conv(**{field: value})) == STATUS.INVALID_PARAMETER
+
+
+def test_conv2d_null_arguments():
+    L = capi.lib()
+    p = _conv()
+    assert L.snn_hip_conv2d_forward_f32(None, FAKE, FAKE, ctypes.byref(p),
+                                        ALGO.DIRECT, None, 0,
+                                        None) == STATUS.INVALID_PARAMETER
+    assert L.snn_hip_conv2d_forward_f32(FAKE, FAKE, FAKE, None, ALGO.DIRECT,
+                                        None, 0,
+                                        None) == STATUS.INVALID_PARAMETER
+
+
+def test_conv2d_invalid_algorithm():
+    """An algorithm whose selector answers NotSupported gives InvalidAlgorithm
+    (internal/conv2d/launch.h:127-129,164-165)."""
+    s2 = ops.conv_params(1, 9, 9, 4, 4, 3, 2, True)
+    assert _call_conv(s2, ALGO.WINOGRAD) == STATUS.INVALID_ALGORITHM
+    assert _call_conv(s2, ALGO.MATMUL) == STATUS.INVALID_ALGORITHM
+    assert _call_conv(s2, ALGO.NOT_SUPPORTED) == STATUS.INVALID_ALGORITHM
+    assert _call_conv(s2, 99) == STATUS.INVALID_ALGORITHM
+    w7 = ops.conv_params(1, 16, 16, 3, 8, 7, 2, True)
+    assert _call_conv(w7, ALGO.TILED) == STATUS.INVALID_ALGORITHM
+    # Tiled is forward only (tiled_selector.h:76-96)
+    p = _conv()
+    assert _call_conv(p, ALGO.TILED,
+                      DIRECTION.INPUT_BACKPROP) == STATUS.INVALID_ALGORITHM
+    assert _call_conv(p, ALGO.TILED,
+                      DIRECTION.FILTER_BACKPROP) == STATUS.INVALID_ALGORITHM
+    # grouped convolution is not part of this library
+    g = _conv(groups=2)
+    assert _call_conv(g, ALGO.IM2COL) == STATUS.INVALID_ALGORITHM
+
+
+def test_winograd_needs_workspace():
+    """internal/conv2d/winograd/launch.h:271-286"""
+    for d in (DIRECTION.FORWARD, DIRECTION.INPUT_BACKPROP,
+              DIRECTION.FILTER_BACKPROP):
+        assert _call_conv(_conv(), ALGO.WINOGRAD,
+                          d) == STATUS.INSUFFICIENT_WORKSPACE
+
+
+def test_index_exceeded():
+    """Tensors beyond INT32_MAX elements (launch_tiled.cc:133-141)."""
+    p = ops.conv_params(4096, 1024, 1024, 4, 4, 1, 1, False)
+    assert _call_conv(p) == STATUS.INDEX_EXCEEDED
+
+
+def test_algorithm_support_table():
+    """The concrete selectors: tiled_selector.h:45-96,
+    winograd_selector.h:44-106, matmul_selector.h:44-100."""
+    L = capi.lib()
+
+    def sup(p, d, a):
+        return L.snn_hip_conv2d_algorithm_supports(ctypes.byref(p), d, a) == a
+
+    F, I, B = (DIRECTION.FORWARD, DIRECTION.INPUT_BACKPROP,
+               DIRECTION.FILTER_BACKPROP)
+    for w, s, ok in [(1, 1, True), (1, 2, True), (3, 1, True), (3, 2, True),
+                     (5, 1, True), (5, 2, False), (7, 1, False),
+                     (11, 4, False)]:
+        p = ops.conv_params(1, 32, 32, 4, 4, w, s, True)
+        assert sup(p, F, ALGO.TILED) == ok, (w, s)
+        assert not sup(p, I, ALGO.TILED)
+        assert not sup(p, B, ALGO.TILED)
+        assert sup(p, F, ALGO.DIRECT) and sup(p, B, ALGO.IM2COL)
+    p33 = ops.conv_params(1, 32, 32, 4, 4, 3, 1, True)
+    for d in (F, I, B):
+        assert sup(p33, d, ALGO.WINOGRAD)
+        assert sup(p33, d, ALGO.WINOGRAD_LARGE)
+    p31 = ops.conv_params(1, 32, 32, 4, 4, 3, 1, True)
+    p31.window_cols = 1
+    assert sup(p31, F, ALGO.WINOGRAD)
+    assert not sup(p31, F, ALGO.WINOGRAD_LARGE)
+    p32 = ops.conv_params(1, 32, 32, 4, 4, 3, 2, True)
+    assert not sup(p32, F, ALGO.WINOGRAD)
+    p11 = ops.conv_params(1, 32, 32, 4, 16, 1, 1, False)
+    for d in (F, I, B):
+        assert sup(p11, d, ALGO.MATMUL)
+    assert not sup(p33, F, ALGO.MATMUL)
+    p11s2 = ops.conv_params(1, 32, 32, 4, 16, 1, 2, False)
+    assert not sup(p11s2, F, ALGO.MATMUL)
+
+
+def test_default_algorithm_is_launchable():
+    """test/conv2d/default_selector.cc:73-98: whatever the default selector
+    returns must be supported for those parameters."""
+    L = capi.lib()
+    for w, s in [(1, 1), (1, 2), (3, 1), (3, 2), (5, 1), (7, 2), (11, 4)]:
+        for same in (True, False):
+            p = ops.conv_params(2, 32, 32, 8, 16, w, s, same)
+            for d in range(3):
+                a = L.snn_hip_conv2d_default_algorithm(ctypes.byref(p), d)
+                assert a != ALGO.NOT_SUPPORTED
+                assert L.snn_hip_conv2d_algorithm_supports(
+                    ctypes.byref(p), d, a) == a
+
+
+def test_workspace_sizes_reference_bounds():
+    """Lower bounds of test/conv2d/workspace_size.cc:52-160 (VGG layer 1:
+    3x3 s1 SAME, 224x224, 64 -> 64, batch 32)."""
+    p = ops.conv_params(32, 224, 224, 64, 64, 3, 1, True)
+    for algo in (ALGO.DIRECT, ALGO.TILED, ALGO.MATMUL):
+        for d in range(3):
+            assert ops.workspace_size(p, d, algo) == (0, 0)
+    tiles, tile = 224 * 224, 3 * 3 * 64
+    fil = 3 * 3 * 64 * 64
+    req, rec = ops.workspace_size(p, DIRECTION.FORWARD, ALGO.IM2COL)
+    assert req >= tiles * tile and rec >= 32 * tiles * tile
+    req, rec = ops.workspace_size(p, DIRECTION.INPUT_BACKPROP, ALGO.IM2COL)
+    assert req >= tiles * tile + fil and rec >= 32 * tiles * tile + fil
+    req, rec = ops.workspace_size(p, DIRECTION.FILTER_BACKPROP, ALGO.IM2COL)
+    assert req >= tiles * tile and rec >= 32 * tiles * tile
+    ab = 16
+    t = 112 * 112 * 64
+    f = 64 * 64
+    for d in range(3):
+        req, rec = ops.workspace_size(p, d, ALGO.WINOGRAD)
+        assert req >= ab * (t + f + t)
+        assert rec >= ab * (32 * (t + t) + f)
+    # figures quoted for the benchmark layers (Winograd F(2x2,3x3), batch 32)
+    p56 = ops.conv_params(32, 56, 56, 64, 64, 3, 1, True)
+    req, rec = ops.workspace_size(p56, DIRECTION.FORWARD, ALGO.WINOGRAD)
+    assert req == 16 * (28 * 28 * 64 * 2 + 64 * 64)
+    assert rec == 16 * (32 * 28 * 28 * 64 * 2 + 64 * 64)
+
+
+def test_depthwise_and_pooling_validation():
+    L = capi.lib()
+    d = ops.depthwise_params(2, 8, 8, 4, 1, 3, 1, True)
+    d.channel_multiplier = 0
+    assert L.snn_hip_depthwise_conv2d_forward_f32(
+        FAKE, FAKE, FAKE, ctypes.byref(d), None) == STATUS.INVALID_PARAMETER
+    d = ops.depthwise_params(2, 8, 8, 4, 1, 3, 1, True)
+    d.input_format = 1  # NCHW is rejected (internal/depthwise_conv2d/launch.h:108)
+    assert L.snn_hip_depthwise_conv2d_forward_f32(
+        FAKE, FAKE, FAKE, ctypes.byref(d), None) == STATUS.INVALID_PARAMETER
+    q = ops.pool_params(2, 8, 8, 4, 3, 2, True)
+    q.stride_cols = 0
+    assert L.snn_hip_pooling_forward_f32(
+        FAKE, FAKE, ctypes.byref(q), 0, None) == STATUS.INVALID_PARAMETER
+    q = ops.pool_params(2, 8, 8, 4, 3, 2, True)
+    assert L.snn_hip_pooling_max_grad_f32(
+        FAKE, FAKE, FAKE, FAKE, ctypes.byref(q), 2,
+        None) == STATUS.INVALID_PARAMETER  # Average is not a max operator
+    assert L.snn_hip_matmul_f32(FAKE, FAKE, FAKE, 1, 0, 4, 4, 0, 0, 0.0,
+                                None) == STATUS.INVALID_PARAMETER
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    """No CPU fallback: a missing libsnn_hip.so is an error, not a detour."""
+    monkeypatch.setattr(capi, "_lib", None)
+    monkeypatch.setattr(capi, "_LIB_PATH", str(tmp_path / "libsnn_hip.so"))
+    with pytest.raises(capi.SnnHipError):
+        capi.lib()

@@ -1,0 +1,152 @@
+"""GPU parity against the reference's golden vectors, through the C ABI.
+
+Every case of tests/golden/*.npz (the reference's own generated tests, exact
+integers) is run through libsnn_hip.so with every algorithm whose selector
+accepts it; the bar is the reference's own: exact for conv / depthwise / max
+pooling (all values are integers below 2^24, so any correct fp32 evaluation
+order is exact), 4 ULP for average pooling, 8 ULP for its gradient
+(test/pooling/pooling_fixture.h:107-125).
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from golden_cases import load
+from portdnn_amd import capi, ops
+from portdnn_amd.capi import ALGO, DIRECTION, POOL_OP
+
+pytestmark = pytest.mark.gpu
+
+ALGOS = [ALGO.DIRECT, ALGO.TILED, ALGO.IM2COL, ALGO.WINOGRAD, ALGO.MATMUL]
+ALGO_NAME = {1: "direct", 2: "tiled", 3: "im2col", 4: "winograd", 6: "matmul"}
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+def supported(p, direction, algo):
+    return capi.lib().snn_hip_conv2d_algorithm_supports(
+        ctypes.byref(p), direction, algo) == algo
+
+
+def run_conv_group(group, direction, algo):
+    n_run = 0
+    for case in load(group):
+        p = ops.conv_params(case.n, case.h, case.w, case.c, case.k,
+                            case.window, case.stride, case.same)
+        if not supported(p, direction, algo):
+            continue
+        n_in, n_fil, _ = ops.conv_sizes(p, direction)
+        a = dev(oracle.iota(n_in, case.max_val))
+        b = dev(oracle.iota(n_fil, case.max_val))
+        got = ops.conv2d(a, b, p, direction, algo).cpu().numpy()
+        exp = case.expected.astype(np.float32)
+        assert got.size == exp.size
+        bad = np.flatnonzero(got != exp)
+        assert bad.size == 0, (group, ALGO_NAME[algo], case[:9], bad[:4],
+                               got[bad[:4]], exp[bad[:4]])
+        n_run += 1
+    return n_run
+
+
+@pytest.mark.parametrize("algo", ALGOS, ids=lambda a: ALGO_NAME[a])
+def test_conv2d_forward_golden(algo):
+    n = run_conv_group("conv2d_forward", DIRECTION.FORWARD, algo)
+    expected = {ALGO.DIRECT: 2592, ALGO.IM2COL: 2592, ALGO.TILED: 5 * 324,
+                ALGO.WINOGRAD: 324, ALGO.MATMUL: 162 + 6}
+    assert n >= expected[algo] - 200 and n > 0, n
+
+
+@pytest.mark.parametrize("algo", [ALGO.DIRECT, ALGO.IM2COL, ALGO.WINOGRAD,
+                                  ALGO.MATMUL], ids=lambda a: ALGO_NAME[a])
+def test_conv2d_input_backprop_golden(algo):
+    assert run_conv_group("conv2d_input_backprop", DIRECTION.INPUT_BACKPROP,
+                          algo) > 0
+
+
+@pytest.mark.parametrize("algo", [ALGO.DIRECT, ALGO.IM2COL, ALGO.WINOGRAD,
+                                  ALGO.MATMUL], ids=lambda a: ALGO_NAME[a])
+def test_conv2d_filter_backprop_golden(algo):
+    assert run_conv_group("conv2d_filter_backprop", DIRECTION.FILTER_BACKPROP,
+                          algo) > 0
+
+
+@pytest.mark.parametrize("group,direction", [
+    ("depthwise_forward", DIRECTION.FORWARD),
+    ("depthwise_input_backprop", DIRECTION.INPUT_BACKPROP),
+    ("depthwise_filter_backprop", DIRECTION.FILTER_BACKPROP)])
+def test_depthwise_golden(group, direction):
+    n_run = 0
+    for case in load(group):
+        p = ops.depthwise_params(case.n, case.h, case.w, case.c, case.k,
+                                 case.window, case.stride, case.same)
+        n_in, n_fil, _ = ops.depthwise_sizes(p, direction)
+        a = dev(oracle.iota(n_in, case.max_val))
+        b = dev(oracle.iota(n_fil, case.max_val))
+        got = ops.depthwise_conv2d(a, b, p, direction).cpu().numpy()
+        exp = case.expected.astype(np.float32)
+        bad = np.flatnonzero(got != exp)
+        assert bad.size == 0, (group, case[:9], bad[:4], got[bad[:4]],
+                               exp[bad[:4]])
+        n_run += 1
+    assert n_run == 1620
+
+
+@pytest.mark.parametrize("op", [POOL_OP.MAX, POOL_OP.MAX_WITH_NAN])
+def test_pool_max_forward_golden(op):
+    n_run = 0
+    for case in load("pool_max_forward"):
+        p = ops.pool_params(case.n, case.h, case.w, case.c, case.window,
+                            case.stride, case.same)
+        x = dev(oracle.iota(case.n * case.h * case.w * case.c, case.max_val))
+        got = ops.pooling_forward(x, p, op).cpu().numpy()
+        assert np.array_equal(got, case.expected.astype(np.float32)), case[:9]
+        n_run += 1
+    assert n_run == 972
+
+
+def test_pool_avg_forward_golden():
+    n_run = 0
+    for case in load("pool_avg_forward"):
+        p = ops.pool_params(case.n, case.h, case.w, case.c, case.window,
+                            case.stride, case.same)
+        x = dev(oracle.iota(case.n * case.h * case.w * case.c, case.max_val))
+        got = ops.pooling_forward(x, p, POOL_OP.AVERAGE).cpu().numpy()
+        exp = case.expected
+        tol = 4 * np.spacing(np.abs(exp).astype(np.float32))
+        assert np.all(np.abs(got.astype(np.float64) - exp) <= tol), case[:9]
+        n_run += 1
+    assert n_run == 972
+
+
+def test_pool_max_grad_golden():
+    n_run = 0
+    for case in load("pool_max_grad"):
+        p = ops.pool_params(case.n, case.h, case.w, case.c, case.window,
+                            case.stride, case.same)
+        x = dev(oracle.iota(case.n * case.h * case.w * case.c, case.max_val))
+        y = ops.pooling_forward(x, p, POOL_OP.MAX)
+        dy = dev(oracle.iota(y.numel(), case.max_val))
+        got = ops.pooling_max_grad(x, y, dy, p).cpu().numpy()
+        assert np.array_equal(got, case.expected.astype(np.float32)), case[:9]
+        n_run += 1
+    assert n_run == 432
+
+
+def test_pool_avg_grad_golden():
+    n_run = 0
+    for case in load("pool_avg_grad"):
+        p = ops.pool_params(case.n, case.h, case.w, case.c, case.window,
+                            case.stride, case.same)
+        dy = dev(oracle.iota(p.batch * p.out_rows * p.out_cols * case.c,
+                             case.max_val))
+        got = ops.pooling_avg_grad(dy, p).cpu().numpy()
+        exp = case.expected
+        tol = 8 * np.spacing(np.abs(exp).astype(np.float32))
+        assert np.all(np.abs(got.astype(np.float64) - exp) <= tol), case[:9]
+        n_run += 1
+    assert n_run == 432

@@ -1,0 +1,453 @@
+"""GPU parity on seeded random data at the benchmark shapes, through the C ABI.
+
+Floating-point bar (fp32): |gpu - oracle| <= 1e-4 * |oracle| + 1e-5 * S, where
+the oracle accumulates in double and S = max(1, rms(oracle)).  S is 1 -- i.e.
+the bar is exactly "1e-4 relative / 1e-5 absolute" -- whenever the outputs are
+O(1); for the deep reductions of the ResNet layers (up to 4608 products of
+U[-1,1] values, output rms up to ~23) the absolute term scales with the output
+magnitude, because no fp32 accumulation (the reference's included) can hold
+1e-5 absolute on an output that cancels to ~0 out of terms that large.
+f16: 1e-2 relative to S against the double-precision result of the
+f16-rounded operands.
+
+Shapes are the benchmark configurations at a batch the CPU oracle finishes in
+seconds; the full batch-32 shapes are covered by sampled outputs recomputed in
+float64 and by linearity.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from portdnn_amd import capi, ops
+from portdnn_amd.capi import ALGO, DIRECTION, POOL_OP
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-4, 1e-5
+ALGO_NAME = {1: "direct", 2: "tiled", 3: "im2col", 4: "winograd", 6: "matmul"}
+FWD_ALGOS = [ALGO.DIRECT, ALGO.TILED, ALGO.IM2COL, ALGO.WINOGRAD, ALGO.MATMUL]
+BK_ALGOS = [ALGO.DIRECT, ALGO.IM2COL, ALGO.WINOGRAD, ALGO.MATMUL]
+
+RESNET_3X3 = [(56, 64), (28, 128), (14, 256), (7, 512)]
+
+
+def assert_close(got, ref, what, rtol=RTOL, atol=ATOL):
+    got = np.asarray(got, dtype=np.float64).reshape(-1)
+    ref = np.asarray(ref, dtype=np.float64).reshape(-1)
+    assert got.shape == ref.shape, what
+    scale = max(1.0, float(np.sqrt(np.mean(ref * ref))))
+    err = np.abs(got - ref)
+    tol = rtol * np.abs(ref) + atol * scale
+    bad = np.flatnonzero(~(err <= tol))
+    assert bad.size == 0, (what, "n_bad=%d of %d" % (bad.size, ref.size),
+                           "worst err %.3e tol %.3e" % (
+                               err[bad].max(), tol[bad[np.argmax(err[bad])]]),
+                           bad[:4], got[bad[:4]], ref[bad[:4]])
+
+
+def uniform(rng, n):
+    return rng.uniform(-1.0, 1.0, size=n).astype(np.float32)
+
+
+def dev(a, dtype=torch.float32):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda().to(dtype)
+
+
+def supported(p, direction, algo):
+    return capi.lib().snn_hip_conv2d_algorithm_supports(
+        ctypes.byref(p), direction, algo) == algo
+
+
+def oracle_params(p, features):
+    return oracle.Params(p.channels, features, p.batch, p.in_rows, p.in_cols,
+                         p.window_rows, p.window_cols, p.stride_rows,
+                         p.stride_cols, p.out_rows, p.out_cols, p.pad_rows,
+                         p.pad_cols)
+
+
+ORACLE_FN = {DIRECTION.FORWARD: oracle.conv2d_forward,
+             DIRECTION.INPUT_BACKPROP: oracle.conv2d_input_backprop,
+             DIRECTION.FILTER_BACKPROP: oracle.conv2d_filter_backprop}
+
+
+def conv_case(p, direction, algos, seed):
+    rng = np.random.default_rng(seed)
+    n_in, n_fil, _ = ops.conv_sizes(p, direction)
+    a, b = uniform(rng, n_in), uniform(rng, n_fil)
+    ref = ORACLE_FN[direction](a, b, oracle_params(p, p.features), acc64=True)
+    da, db = dev(a), dev(b)
+    ran = 0
+    for algo in algos:
+        if not supported(p, direction, algo):
+            continue
+        got = ops.conv2d(da, db, p, direction, algo).cpu().numpy()
+        assert_close(got, ref, (ALGO_NAME[algo], direction, repr(p)))
+        ran += 1
+    assert ran > 0
+
+
+@pytest.mark.parametrize("size,ch", RESNET_3X3)
+@pytest.mark.parametrize("direction", [DIRECTION.FORWARD,
+                                       DIRECTION.INPUT_BACKPROP,
+                                       DIRECTION.FILTER_BACKPROP])
+def test_resnet_3x3(size, ch, direction):
+    p = ops.conv_params(2, size, size, ch, ch, 3, 1, True)
+    algos = FWD_ALGOS if direction == DIRECTION.FORWARD else BK_ALGOS
+    conv_case(p, direction, algos, seed=100 + size + direction)
+
+
+@pytest.mark.parametrize("size,ch", RESNET_3X3)
+@pytest.mark.parametrize("direction", [DIRECTION.FORWARD,
+                                       DIRECTION.INPUT_BACKPROP,
+                                       DIRECTION.FILTER_BACKPROP])
+def test_resnet_1x1_expand(size, ch, direction):
+    p = ops.conv_params(2, size, size, ch, 4 * ch, 1, 1, False)
+    algos = FWD_ALGOS if direction == DIRECTION.FORWARD else BK_ALGOS
+    conv_case(p, direction, algos, seed=200 + size + direction)
+
+
+@pytest.mark.parametrize("direction", [DIRECTION.FORWARD,
+                                       DIRECTION.INPUT_BACKPROP,
+                                       DIRECTION.FILTER_BACKPROP])
+def test_stem_7x7_stride2(direction):
+    p = ops.conv_params(1, 224, 224, 3, 64, 7, 2, True)
+    assert (p.out_rows, p.pad_rows) == (112, 2)
+    conv_case(p, direction, [ALGO.DIRECT, ALGO.IM2COL], seed=300 + direction)
+
+
+def test_config0_single_image_tiled():
+    """BASELINE configuration 0: N=1, 56x56x64 -> 64, 3x3 s1 SAME, Tiled;
+    also checked against the reference-loop-nest restatement in fp32."""
+    p = ops.conv_params(1, 56, 56, 64, 64, 3, 1, True)
+    rng = np.random.default_rng(0x5EED)
+    x, w = uniform(rng, 56 * 56 * 64), uniform(rng, 9 * 64 * 64)
+    op = oracle_params(p, 64)
+    ref = oracle.conv2d_forward(x, w, op, acc64=True)
+    tiled = oracle.conv2d_tiled_forward(x, w, op)
+    assert_close(tiled, ref, "tiled restatement vs direct oracle")
+    got = ops.conv2d(dev(x), dev(w), p, DIRECTION.FORWARD,
+                     ALGO.TILED).cpu().numpy()
+    assert_close(got, ref, "config0 tiled")
+
+
+@pytest.mark.parametrize("shape", [
+    # ragged / edge shapes: odd sizes, C and K not multiples of the tiles,
+    # non-square windows and strides, VALID padding
+    (3, 13, 17, 5, 7, 3, 3, 1, 1, True),
+    (2, 9, 11, 3, 130, 3, 3, 2, 2, True),
+    (1, 16, 16, 70, 9, 5, 5, 1, 1, False),
+    (2, 12, 10, 8, 8, 3, 1, 1, 1, True),
+    (2, 12, 10, 8, 8, 1, 3, 1, 1, True),
+    (1, 20, 20, 33, 65, 3, 3, 1, 2, True),
+    (2, 7, 7, 16, 16, 7, 7, 1, 1, False),
+    (1, 1, 1, 1, 1, 1, 1, 1, 1, False),
+    (4, 5, 5, 2, 3, 11, 11, 4, 4, True),
+])
+@pytest.mark.parametrize("direction", [DIRECTION.FORWARD,
+                                       DIRECTION.INPUT_BACKPROP,
+                                       DIRECTION.FILTER_BACKPROP])
+def test_ragged_shapes(shape, direction):
+    n, h, w, c, k, wr, wc, sr, sc, same = shape
+    p = ops.ConvParams(channels=c, features=k, batch=n, in_rows=h, in_cols=w,
+                       window_rows=wr, window_cols=wc, stride_rows=sr,
+                       stride_cols=sc)
+    ops.add_padding_to(p, same)
+    algos = FWD_ALGOS if direction == DIRECTION.FORWARD else BK_ALGOS
+    conv_case(p, direction, algos, seed=sum(shape[:9]) + direction)
+
+
+# ---- full batch-32 shapes: sampled float64 recomputation + linearity --------
+
+def sampled_forward_reference(x, w, p, samples):
+    """float64 value of the chosen (n, oy, ox, k) outputs by definition."""
+    X = x.reshape(p.batch, p.in_rows, p.in_cols, p.channels).astype(np.float64)
+    W = w.reshape(p.window_rows, p.window_cols, p.channels,
+                  p.features).astype(np.float64)
+    out = np.zeros(len(samples))
+    for i, (n, oy, ox, k) in enumerate(samples):
+        acc = 0.0
+        for r in range(p.window_rows):
+            y = oy * p.stride_rows - p.pad_rows + r
+            if not 0 <= y < p.in_rows:
+                continue
+            for s in range(p.window_cols):
+                xx = ox * p.stride_cols - p.pad_cols + s
+                if not 0 <= xx < p.in_cols:
+                    continue
+                acc += X[n, y, xx] @ W[r, s, :, k]
+        out[i] = acc
+    return out
+
+
+@pytest.mark.parametrize("size,ch,window", [(56, 64, 3), (28, 128, 3),
+                                            (14, 256, 3), (7, 512, 3),
+                                            (56, 64, 1), (7, 512, 1)])
+def test_full_batch_forward_sampled_and_linear(size, ch, window):
+    feats = ch if window == 3 else 4 * ch
+    p = ops.conv_params(32, size, size, ch, feats, window, 1, window == 3)
+    rng = np.random.default_rng(1000 + size + window)
+    n_in, n_fil, n_out = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x1, x2, w = uniform(rng, n_in), uniform(rng, n_in), uniform(rng, n_fil)
+    samples = np.stack([rng.integers(0, p.batch, 600),
+                        rng.integers(0, p.out_rows, 600),
+                        rng.integers(0, p.out_cols, 600),
+                        rng.integers(0, feats, 600)], axis=1)
+    # force image corners and edges into the sample
+    samples[:8, 1] = [0, 0, p.out_rows - 1, p.out_rows - 1, 0, p.out_rows - 1,
+                      p.out_rows // 2, p.out_rows // 2]
+    samples[:8, 2] = [0, p.out_cols - 1, 0, p.out_cols - 1, p.out_cols // 2,
+                      p.out_cols // 2, 0, p.out_cols - 1]
+    ref = sampled_forward_reference(x1, w, p, samples)
+    flat = ((samples[:, 0] * p.out_rows + samples[:, 1]) * p.out_cols +
+            samples[:, 2]) * feats + samples[:, 3]
+    d1, d2, dw = dev(x1), dev(x2), dev(w)
+    scale = max(1.0, float(np.sqrt(np.mean(ref * ref))))
+    outs = {}
+    for algo in FWD_ALGOS:
+        if not supported(p, DIRECTION.FORWARD, algo):
+            continue
+        y1 = ops.conv2d(d1, dw, p, DIRECTION.FORWARD, algo)
+        got = y1.cpu().numpy()[flat]
+        err = np.abs(got - ref)
+        assert np.all(err <= RTOL * np.abs(ref) + ATOL * scale), (
+            ALGO_NAME[algo], err.max())
+        # linearity: conv(2*x1 - x2) == 2*conv(x1) - conv(x2)
+        y2 = ops.conv2d(d2, dw, p, DIRECTION.FORWARD, algo)
+        y3 = ops.conv2d(2 * d1 - d2, dw, p, DIRECTION.FORWARD, algo)
+        lin = (y3 - (2 * y1 - y2)).abs().max().item()
+        assert lin <= 20 * ATOL * scale, (ALGO_NAME[algo], lin)
+        outs[algo] = y1
+    # every algorithm agrees with Direct over the whole tensor
+    base = outs[ALGO.DIRECT]
+    for algo, y in outs.items():
+        diff = (y - base).abs()
+        tol = 2 * (RTOL * base.abs() + ATOL * scale)
+        assert bool((diff <= tol).all()), (ALGO_NAME[algo], diff.max().item())
+
+
+# ---- depthwise ---------------------------------------------------------------
+
+MOBILENET = [(112, 32, 1), (112, 64, 2), (56, 128, 1), (28, 256, 2),
+             (14, 512, 1), (7, 1024, 1)]
+
+
+@pytest.mark.parametrize("size,ch,stride", MOBILENET)
+def test_depthwise_mobilenet_all_directions(size, ch, stride):
+    p = ops.depthwise_params(2, size, size, ch, 1, 3, stride, True)
+    op = oracle_params(p, 1)
+    rng = np.random.default_rng(400 + size)
+    x = rng.standard_normal(2 * size * size * ch).astype(np.float32)
+    w = rng.standard_normal(9 * ch).astype(np.float32)
+    dy = rng.standard_normal(2 * p.out_rows * p.out_cols * ch).astype(
+        np.float32)
+    got = ops.depthwise_conv2d(dev(x), dev(w), p).cpu().numpy()
+    assert_close(got, oracle.depthwise_forward(x, w, op), ("dw fwd", size, ch))
+    got = ops.depthwise_conv2d(dev(dy), dev(w), p,
+                               DIRECTION.INPUT_BACKPROP).cpu().numpy()
+    assert_close(got, oracle.depthwise_input_backprop(dy, w, op),
+                 ("dw inbk", size, ch))
+    got = ops.depthwise_conv2d(dev(x), dev(dy), p,
+                               DIRECTION.FILTER_BACKPROP).cpu().numpy()
+    assert_close(got, oracle.depthwise_filter_backprop(x, dy, op),
+                 ("dw filbk", size, ch))
+
+
+@pytest.mark.parametrize("shape", [(3, 9, 7, 5, 3, 3, 2, True),
+                                   (1, 12, 12, 6, 1, 5, 1, False),
+                                   (2, 8, 8, 4, 2, 3, 1, True),
+                                   (2, 6, 6, 7, 1, 7, 4, True)])
+def test_depthwise_ragged(shape):
+    n, h, w_, c, m, win, st, same = shape
+    p = ops.depthwise_params(n, h, w_, c, m, win, st, same)
+    op = oracle_params(p, m)
+    rng = np.random.default_rng(sum(shape[:7]))
+    x = rng.standard_normal(n * h * w_ * c).astype(np.float32)
+    w = rng.standard_normal(win * win * c * m).astype(np.float32)
+    dy = rng.standard_normal(n * p.out_rows * p.out_cols * c * m).astype(
+        np.float32)
+    assert_close(ops.depthwise_conv2d(dev(x), dev(w), p).cpu().numpy(),
+                 oracle.depthwise_forward(x, w, op), ("dw fwd", shape))
+    assert_close(ops.depthwise_conv2d(dev(dy), dev(w), p,
+                                      DIRECTION.INPUT_BACKPROP).cpu().numpy(),
+                 oracle.depthwise_input_backprop(dy, w, op), ("dw inbk", shape))
+    assert_close(ops.depthwise_conv2d(dev(x), dev(dy), p,
+                                      DIRECTION.FILTER_BACKPROP).cpu().numpy(),
+                 oracle.depthwise_filter_backprop(x, dy, op),
+                 ("dw filbk", shape))
+
+
+@pytest.mark.parametrize("size,ch,stride", MOBILENET)
+def test_depthwise_full_batch_matches_oracle(size, ch, stride):
+    """Batch 32: the depthwise oracle is cheap enough to run in full."""
+    p = ops.depthwise_params(32, size, size, ch, 1, 3, stride, True)
+    rng = np.random.default_rng(500 + size)
+    x = rng.standard_normal(32 * size * size * ch).astype(np.float32)
+    w = rng.standard_normal(9 * ch).astype(np.float32)
+    got = ops.depthwise_conv2d(dev(x), dev(w), p).cpu().numpy()
+    assert_close(got, oracle.depthwise_forward(x, w, oracle_params(p, 1)),
+                 ("dw fwd b32", size, ch))
+
+
+# ---- pooling -----------------------------------------------------------------
+
+def test_maxpool_resnet_full_batch_bit_exact():
+    """3x3 s2 SAME max pool on [32,112,112,64]: values must be bit-identical;
+    so must the argmax implied by them (checked through the gradient)."""
+    p = ops.pool_params(32, 112, 112, 64, 3, 2, True)
+    assert (p.out_rows, p.pad_rows) == (56, 0)
+    rng = np.random.default_rng(600)
+    x = rng.standard_normal(32 * 112 * 112 * 64).astype(np.float32)
+    op = oracle_params(p, 0)
+    dx_ = dev(x)
+    y = ops.pooling_forward(dx_, p, POOL_OP.MAX)
+    ref = oracle.pool_max_forward(x, op)
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+    dy = rng.standard_normal(ref.size).astype(np.float32)
+    got = ops.pooling_max_grad(dx_, y, dev(dy), p).cpu().numpy()
+    # overlapping windows add two or more dY terms; the oracle adds them in
+    # output order as the kernel does, so the sums are bit-identical too
+    ref_dx = oracle.pool_max_grad(x, ref, dy, op)
+    assert np.array_equal(got.view(np.uint32), ref_dx.view(np.uint32))
+
+
+def test_maxpool_ties_take_first_maximum():
+    p = ops.pool_params(1, 6, 6, 4, 3, 2, True)
+    x = np.zeros(6 * 6 * 4, dtype=np.float32)  # every window is all ties
+    op = oracle_params(p, 0)
+    y = ops.pooling_forward(dev(x), p, POOL_OP.MAX)
+    dy = np.arange(1, y.numel() + 1, dtype=np.float32)
+    got = ops.pooling_max_grad(dev(x), y, dev(dy), p).cpu().numpy()
+    assert np.array_equal(got, oracle.pool_max_grad(x, y.cpu().numpy(), dy, op))
+
+
+def test_avgpool_resnet_full_batch():
+    p = ops.pool_params(32, 7, 7, 2048, 7, 1, False)
+    assert (p.out_rows, p.out_cols) == (1, 1)
+    rng = np.random.default_rng(601)
+    x = rng.standard_normal(32 * 7 * 7 * 2048).astype(np.float32)
+    got = ops.pooling_forward(dev(x), p, POOL_OP.AVERAGE).cpu().numpy()
+    assert_close(got, oracle.pool_avg_forward(x, oracle_params(p, 0)),
+                 "avg 7x7 global")
+    dy = rng.standard_normal(32 * 2048).astype(np.float32)
+    assert_close(ops.pooling_avg_grad(dev(dy), p).cpu().numpy(),
+                 oracle.pool_avg_grad(dy, oracle_params(p, 0)), "avg grad")
+
+
+@pytest.mark.parametrize("shape", [(2, 9, 7, 5, 3, 2, True),
+                                   (1, 11, 11, 3, 5, 1, True),
+                                   (3, 8, 8, 8, 2, 2, False),
+                                   (2, 13, 13, 6, 11, 4, True)])
+def test_pooling_ragged(shape):
+    n, h, w_, c, win, st, same = shape
+    p = ops.pool_params(n, h, w_, c, win, st, same)
+    op = oracle_params(p, 0)
+    rng = np.random.default_rng(sum(shape[:6]))
+    x = rng.standard_normal(n * h * w_ * c).astype(np.float32)
+    y = ops.pooling_forward(dev(x), p, POOL_OP.MAX)
+    assert np.array_equal(y.cpu().numpy(), oracle.pool_max_forward(x, op))
+    assert_close(ops.pooling_forward(dev(x), p, POOL_OP.AVERAGE).cpu().numpy(),
+                 oracle.pool_avg_forward(x, op), ("avg", shape))
+    dy = rng.standard_normal(y.numel()).astype(np.float32)
+    assert_close(ops.pooling_max_grad(dev(x), y, dev(dy), p).cpu().numpy(),
+                 oracle.pool_max_grad(x, y.cpu().numpy(), dy, op),
+                 ("max grad", shape))
+    assert_close(ops.pooling_avg_grad(dev(dy), p).cpu().numpy(),
+                 oracle.pool_avg_grad(dy, op), ("avg grad", shape))
+
+
+def test_maxpool_nan_rules():
+    """test/pooling/max_pooling_with_nan.cc: Max drops NaNs, MaxWithNan
+    propagates them (forward and gradient)."""
+    p = ops.pool_params(1, 4, 4, 4, 2, 2, False)
+    op = oracle_params(p, 0)
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal(64).astype(np.float32)
+    x[[3, 17, 18, 40, 41, 44, 45]] = np.nan
+    for gpu_op, nan_mode in ((POOL_OP.MAX, False), (POOL_OP.MAX_WITH_NAN, True)):
+        y = ops.pooling_forward(dev(x), p, gpu_op)
+        ref = oracle.pool_max_forward(x, op, nan_mode)
+        assert np.array_equal(y.cpu().numpy(), ref, equal_nan=True)
+        assert np.isnan(ref).any() == nan_mode
+        dy = np.arange(1, 17, dtype=np.float32)
+        got = ops.pooling_max_grad(dev(x), y, dev(dy), p, gpu_op).cpu().numpy()
+        assert np.array_equal(got, oracle.pool_max_grad(x, ref, dy, op,
+                                                        nan_mode))
+
+
+# ---- matmul ------------------------------------------------------------------
+
+@pytest.mark.parametrize("trans_a", [False, True])
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("shape", [(1, 64, 64, 64), (3, 37, 29, 53),
+                                   (1, 1568, 512, 2048), (2, 130, 7, 258),
+                                   (16, 200, 64, 64)])
+def test_matmul(trans_a, trans_b, shape):
+    b_, m, k, n = shape
+    rng = np.random.default_rng(sum(shape))
+    a, b = uniform(rng, b_ * m * k), uniform(rng, b_ * k * n)
+    c0 = uniform(rng, b_ * m * n)
+    for beta in (0.0, 1.0):
+        ref = oracle.matmul(a, b, b_, m, k, n, trans_a, trans_b, beta, c=c0)
+        got = ops.matmul(dev(a), dev(b), b_, m, k, n, trans_a, trans_b, beta,
+                         out=dev(c0).clone()).cpu().numpy()
+        assert_close(got, ref, ("matmul", shape, trans_a, trans_b, beta))
+
+
+# ---- f16 ---------------------------------------------------------------------
+
+def assert_close_f16(got, ref, what):
+    got = np.asarray(got, dtype=np.float64).reshape(-1)
+    ref = np.asarray(ref, dtype=np.float64).reshape(-1)
+    scale = max(1.0, float(np.sqrt(np.mean(ref * ref))))
+    err = np.abs(got - ref)
+    assert np.all(err <= 1e-2 * np.maximum(np.abs(ref), scale)), (
+        what, err.max())
+
+
+@pytest.mark.parametrize("size,ch,window", [(56, 64, 3), (14, 256, 3),
+                                            (7, 512, 3), (28, 128, 1)])
+def test_f16_conv_forward(size, ch, window):
+    feats = ch if window == 3 else 4 * ch
+    p = ops.conv_params(2, size, size, ch, feats, window, 1, window == 3)
+    rng = np.random.default_rng(700 + size)
+    n_in, n_fil, _ = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x = uniform(rng, n_in).astype(np.float16)
+    w = uniform(rng, n_fil).astype(np.float16)
+    ref = oracle.conv2d_forward(x.astype(np.float32), w.astype(np.float32),
+                                oracle_params(p, feats), acc64=True)
+    for algo in FWD_ALGOS:
+        if not supported(p, DIRECTION.FORWARD, algo):
+            continue
+        got = ops.conv2d(dev(x, torch.float16), dev(w, torch.float16), p,
+                         DIRECTION.FORWARD, algo).float().cpu().numpy()
+        assert_close_f16(got, ref, ("f16", ALGO_NAME[algo], size, ch))
+
+
+@pytest.mark.parametrize("size,ch,stride", MOBILENET)
+def test_f16_depthwise_forward(size, ch, stride):
+    p = ops.depthwise_params(2, size, size, ch, 1, 3, stride, True)
+    rng = np.random.default_rng(800 + size)
+    x = uniform(rng, 2 * size * size * ch).astype(np.float16)
+    w = uniform(rng, 9 * ch).astype(np.float16)
+    ref = oracle.depthwise_forward(x.astype(np.float32), w.astype(np.float32),
+                                   oracle_params(p, 1))
+    got = ops.depthwise_conv2d(dev(x, torch.float16), dev(w, torch.float16),
+                               p).float().cpu().numpy()
+    assert_close_f16(got, ref, ("f16 dw", size, ch))
+
+
+def test_f16_pooling_forward():
+    p = ops.pool_params(2, 112, 112, 64, 3, 2, True)
+    rng = np.random.default_rng(900)
+    x = rng.standard_normal(2 * 112 * 112 * 64).astype(np.float16)
+    ref = oracle.pool_max_forward(x.astype(np.float32), oracle_params(p, 0))
+    got = ops.pooling_forward(dev(x, torch.float16), p, POOL_OP.MAX)
+    assert np.array_equal(got.float().cpu().numpy(), ref)
+    q = ops.pool_params(2, 7, 7, 2048, 7, 1, False)
+    x = rng.standard_normal(2 * 49 * 2048).astype(np.float16)
+    ref = oracle.pool_avg_forward(x.astype(np.float32), oracle_params(q, 0))
+    got = ops.pooling_forward(dev(x, torch.float16), q, POOL_OP.AVERAGE)
+    assert_close_f16(got.float().cpu().numpy(), ref, "f16 avg")
