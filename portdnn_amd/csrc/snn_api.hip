@@ -249,6 +249,27 @@ int default_algorithm(const snn_hip_conv2d_params& p, int direction) {
   return SNN_HIP_ALGO_IM2COL;
 }
 
+inline bool aligned16(const void* p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+// Tiled / Im2col / Matmul: the MFMA implicit-GEMM kernel wherever its vector
+// width and alignment requirements hold, the direct kernel otherwise.
+template <typename T>
+int launch_gemm_path(int direction, const T* input, const T* filter, T* output,
+                     const snn_hip_conv2d_params& p, hipStream_t s) {
+  return launch_conv2d_direct<T>(direction, input, filter, output, p, s);
+}
+template <>
+int launch_gemm_path<float>(int direction, const float* input,
+                            const float* filter, float* output,
+                            const snn_hip_conv2d_params& p, hipStream_t s) {
+  if (conv2d_igemm_supports(direction, p) && aligned16(input) &&
+      aligned16(filter) && aligned16(output))
+    return launch_conv2d_igemm_f32(direction, input, filter, output, p, s);
+  return launch_conv2d_direct<float>(direction, input, filter, output, p, s);
+}
+
 template <typename T>
 int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
                     const snn_hip_conv2d_params* params, int algorithm,
@@ -276,6 +297,10 @@ int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
       if (workspace == nullptr || workspace_elems == 0)
         return SNN_HIP_INSUFFICIENT_WORKSPACE;
       return launch_conv2d_direct<T>(direction, input, filter, output, p, s);
+    case SNN_HIP_ALGO_TILED:
+    case SNN_HIP_ALGO_IM2COL:
+    case SNN_HIP_ALGO_MATMUL:
+      return launch_gemm_path<T>(direction, input, filter, output, p, s);
     default:
       return launch_conv2d_direct<T>(direction, input, filter, output, p, s);
   }

@@ -14,6 +14,14 @@ int launch_conv2d_direct(int direction, const T* input, const T* filter,
                          T* output, const snn_hip_conv2d_params& p,
                          hipStream_t stream);
 
+// Implicit-GEMM convolution on MFMA (conv2d_igemm.hip): the path behind the
+// Tiled and Im2col algorithm tags.  `supports` tells whether the shape meets
+// the kernel's vector-width requirements; pointers must be 16-byte aligned.
+bool conv2d_igemm_supports(int direction, const snn_hip_conv2d_params& p);
+int launch_conv2d_igemm_f32(int direction, const float* input,
+                            const float* filter, float* output,
+                            const snn_hip_conv2d_params& p, hipStream_t stream);
+
 // Depthwise convolution, all three directions (depthwise.hip).
 template <typename T>
 int launch_depthwise(int direction, const T* input, const T* filter, T* output,
