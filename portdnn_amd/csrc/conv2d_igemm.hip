@@ -17,6 +17,9 @@
 //   filter backprop  dW[q][k] = sum_m A[m][q] * dY[m][k]
 //                    reduction over every output pixel; the reduction is split
 //                    across work-groups and combined with float atomics.
+#include <cstdio>
+#include <cstdlib>
+
 #include "gemm_tile.h"
 #include "snn_kernels.h"
 
@@ -43,11 +46,32 @@ struct Gather {
   int n_total;               // GEMM columns
 };
 
-template <int BM, int BN, int WM, int WN, bool B_K_INNER, bool STRIDED>
+// Buffer addressing: loads go through raw buffer descriptors so that an
+// out-of-range byte offset returns zeros.  Padding taps, rows past the last
+// pixel and the ragged end of the reduction all become "offset = kOob" with
+// no branch and no select on the loaded data.
+typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+constexpr unsigned kOob = 0x7FFFFFF0u;       // beyond any accepted tensor
+constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
+
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const float* p,
+                                                   unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p), 0, bytes,
+                                           0x00020000);
+}
+__device__ inline float4 buffer_load4(__amdgpu_buffer_rsrc_t r, unsigned off) {
+  const uint4v v = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+  return __builtin_bit_cast(float4, v);
+}
+
+template <int BM, int BN, int WM, int WN, bool B_K_INNER, bool STRIDED,
+          bool ATOMIC>
 __global__ void __launch_bounds__(kThreads)
     conv_igemm_kernel(const float* __restrict__ src,
                       const float* __restrict__ wgt, float* __restrict__ dst,
-                      Gather g, unsigned n_tiles_n, unsigned n_blocks) {
+                      Gather g, unsigned src_bytes, unsigned wgt_bytes,
+                      unsigned n_tiles_n, unsigned n_tiles,
+                      int chunks_per_split) {
   static_assert(WM * WN == 4, "four waves per work-group");
   constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
   constexpr int TM = WTM / 32, TN = WTN / 32;  // MFMA blocks per wave
@@ -63,16 +87,24 @@ __global__ void __launch_bounds__(kThreads)
   const int wave = tid >> 6;
   const int wave_m = wave / WN, wave_n = wave % WN;
 
-  const unsigned tile = xcd_remap(blockIdx.x, n_blocks);
+  const unsigned tile = xcd_remap(blockIdx.x, n_tiles);
   const int m0 = static_cast<int>(tile / n_tiles_n) * BM;
   const int n0 = static_cast<int>(tile % n_tiles_n) * BN;
+  // reduction range of this work-group (blockIdx.y = split index)
+  const int n_chunks_total = (g.k_total + kBK - 1) / kBK;
+  const int chunk_begin = blockIdx.y * chunks_per_split;
+  const int n_chunks = min(chunks_per_split, n_chunks_total - chunk_begin);
+  const int q_begin = chunk_begin * kBK;
+
+  const __amdgpu_buffer_rsrc_t src_rsrc = make_rsrc(src, src_bytes);
+  const __amdgpu_buffer_rsrc_t wgt_rsrc = make_rsrc(wgt, wgt_bytes);
 
   // ---- A gather bookkeeping: this lane copies chunk column `a_cc` (4 floats
-  // at k offset 4 * a_cc) of rows a_r0 + 32 * i.
+  // at reduction offset 4 * a_cc) of tile rows a_r0 + 32 * i.
   constexpr int A_ROWS_PER_THREAD = BM / 32;
   const int a_cc = tid & 7;
   const int a_r0 = tid >> 3;
-  int a_base[A_ROWS_PER_THREAD];  // element offset of (n, iy0, ix0, 0)
+  int a_off[A_ROWS_PER_THREAD];  // element offset of (n, iy0, ix0, channel 0)
   int a_iy0[A_ROWS_PER_THREAD], a_ix0[A_ROWS_PER_THREAD];
 #pragma unroll
   for (int i = 0; i < A_ROWS_PER_THREAD; ++i) {
@@ -84,25 +116,30 @@ __global__ void __launch_bounds__(kThreads)
       const int n = t / g.p_rows;
       a_iy0[i] = py * g.step_rows + g.off_rows;
       a_ix0[i] = px * g.step_cols + g.off_cols;
-      a_base[i] = n * g.src_rows * g.src_cols * g.src_ch;
+      a_off[i] = n * g.src_rows * g.src_cols * g.src_ch;
+      if (!STRIDED) {
+        a_off[i] += (a_iy0[i] * g.src_cols + a_ix0[i]) * g.src_ch;
+      }
     } else {
       a_iy0[i] = -(1 << 28);  // never in range
       a_ix0[i] = 0;
-      a_base[i] = 0;
+      a_off[i] = 0;
     }
   }
-  // (tap row, tap col, channel) of this lane's chunk; advanced by BK each step
-  int a_c = 4 * a_cc, a_s = 0, a_r = 0;
-  while (a_c >= g.src_ch) {
-    a_c -= g.src_ch;
-    if (++a_s == g.win_cols) { a_s = 0; ++a_r; }
+  // (tap row, tap col, channel) of this lane's chunk; advanced by BK per step
+  int a_c, a_s, a_r;
+  {
+    const int q = q_begin + 4 * a_cc;
+    const int tap = q / g.src_ch;
+    a_c = q - tap * g.src_ch;
+    a_r = tap / g.win_cols;
+    a_s = tap - a_r * g.win_cols;
   }
 
   // ---- B copy bookkeeping
   constexpr int B_VEC_PER_ROW = B_K_INNER ? kBK / 4 : BN / 4;
   constexpr int B_ROWS_PER_PASS = kThreads / B_VEC_PER_ROW;
-  constexpr int B_PASSES =
-      (B_K_INNER ? BN : kBK) / B_ROWS_PER_PASS;
+  constexpr int B_PASSES = (B_K_INNER ? BN : kBK) / B_ROWS_PER_PASS;
   const int b_vec = tid % B_VEC_PER_ROW;
   const int b_row0 = tid / B_VEC_PER_ROW;
 
@@ -111,24 +148,30 @@ __global__ void __launch_bounds__(kThreads)
 
   auto load_a = [&]() {
     const bool tap_ok = a_r < g.win_rows;
+    // offset of this lane's tap relative to (iy0, ix0)
+    const int tap_off =
+        g.tap_sign * (a_r * g.src_cols + a_s) * g.src_ch + a_c;
 #pragma unroll
     for (int i = 0; i < A_ROWS_PER_THREAD; ++i) {
       int iy = a_iy0[i] + g.tap_sign * a_r;
       int ix = a_ix0[i] + g.tap_sign * a_s;
       bool ok = tap_ok;
+      int off;
       if (STRIDED) {
-        ok = ok && iy >= 0 && ix >= 0 && (iy % g.div_rows == 0) &&
+        ok = ok & (iy >= 0) & (ix >= 0) & (iy % g.div_rows == 0) &
              (ix % g.div_cols == 0);
         iy /= g.div_rows;
         ix /= g.div_cols;
+        off = a_off[i] + (iy * g.src_cols + ix) * g.src_ch + a_c;
+      } else {
+        off = a_off[i] + tap_off;
       }
-      ok = ok && iy >= 0 && iy < g.src_rows && ix >= 0 && ix < g.src_cols;
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (ok) {
-        v = *reinterpret_cast<const float4*>(
-            src + a_base[i] + (iy * g.src_cols + ix) * g.src_ch + a_c);
-      }
-      a_reg[i] = v;
+      // bitwise, not short-circuit: no branches in the gather
+      ok = ok &
+           (static_cast<unsigned>(iy) < static_cast<unsigned>(g.src_rows)) &
+           (static_cast<unsigned>(ix) < static_cast<unsigned>(g.src_cols));
+      a_reg[i] = buffer_load4(src_rsrc,
+                              ok ? static_cast<unsigned>(off) * 4u : kOob);
     }
   };
   auto advance_a = [&]() {
@@ -141,7 +184,7 @@ __global__ void __launch_bounds__(kThreads)
   auto load_b = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < B_PASSES; ++i) {
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      unsigned off = kOob;
       if (B_K_INNER) {
         // Wt[q][col]: element (col, q) lives at wgt[(tap * n_total + col) *
         // src_ch + kk] with q = tap * src_ch + kk; rows of the LDS tile are
@@ -151,20 +194,18 @@ __global__ void __launch_bounds__(kThreads)
         if (col < g.n_total && q < g.k_total) {
           const int tap = q / g.src_ch;
           const int kk = q - tap * g.src_ch;
-          v = *reinterpret_cast<const float4*>(
-              wgt + (static_cast<size_t>(tap) * g.n_total + col) * g.src_ch +
-              kk);
+          off = static_cast<unsigned>((tap * g.n_total + col) * g.src_ch + kk) *
+                4u;
         }
       } else {
-        // W[q][col], col contiguous.
+        // W[q][col], col contiguous; q >= k_total is past the end of the
+        // buffer and reads zeros by itself.
         const int q = k0 + b_row0 + B_ROWS_PER_PASS * i;
         const int col = n0 + 4 * b_vec;
-        if (q < g.k_total && col < g.n_total) {
-          v = *reinterpret_cast<const float4*>(
-              wgt + static_cast<size_t>(q) * g.n_total + col);
-        }
+        if (col < g.n_total)
+          off = static_cast<unsigned>(q * g.n_total + col) * 4u;
       }
-      b_reg[i] = v;
+      b_reg[i] = buffer_load4(wgt_rsrc, off);
     }
   };
   auto store_tiles = [&](int stage) {
@@ -192,9 +233,8 @@ __global__ void __launch_bounds__(kThreads)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  const int n_chunks = (g.k_total + kBK - 1) / kBK;
   load_a();
-  load_b(0);
+  load_b(q_begin);
   advance_a();
   store_tiles(0);
   __syncthreads();
@@ -203,7 +243,7 @@ __global__ void __launch_bounds__(kThreads)
     const bool more = it + 1 < n_chunks;
     if (more) {
       load_a();
-      load_b((it + 1) * kBK);
+      load_b(q_begin + (it + 1) * kBK);
       advance_a();
     }
     mma_chunk<TM, TN, true, B_K_INNER, BM, BN>(
@@ -227,36 +267,415 @@ __global__ void __launch_bounds__(kThreads)
       for (int v = 0; v < 16; ++v) {
         const int m = m0 + wave_m * WTM + 32 * i + 8 * (v >> 2) + row_l + (v & 3);
         if (m < g.m_total) {
-          dst[static_cast<size_t>(m) * g.n_total + col] = acc[i][j][v];
+          float* o = dst + static_cast<size_t>(m) * g.n_total + col;
+          if (ATOMIC)
+            unsafeAtomicAdd(o, acc[i][j][v]);
+          else
+            *o = acc[i][j][v];
         }
       }
     }
   }
 }
 
+// ---------------------------------------------------------------------------
+// Fast path.  Measured on MI355X: VALU instructions issued between MFMAs are
+// not hidden behind them -- every vector ALU cycle in the main loop is a cycle
+// the matrix pipe idles -- so this kernel keeps per-chunk vector work to three
+// instructions per gathered row and nothing else:
+//   * src_ch % 32 == 0, so a 32-wide reduction chunk lies inside one filter
+//     tap and the tap / channel bookkeeping is wave-uniform (scalar ALU);
+//   * per-row validity of every tap is a precomputed 32-bit mask; an invalid
+//     tap sets bit 31 of the buffer offset, which the descriptor's range
+//     check turns into a zero fill;
+//   * weight and output accesses use a per-lane constant offset plus a scalar
+//     offset operand, LDS addresses are constants plus immediates (the chunk
+//     loop is unrolled by the two LDS stages).
+template <int BM, int BN, int WM, int WN, bool B_K_INNER, bool ATOMIC>
+__global__ void __launch_bounds__(kThreads)
+    conv_igemm_fast_kernel(const float* __restrict__ src,
+                           const float* __restrict__ wgt,
+                           float* __restrict__ dst, Gather g,
+                           unsigned src_bytes, unsigned wgt_bytes,
+                           unsigned dst_bytes, unsigned n_tiles_n,
+                           unsigned n_tiles, int chunks_per_split) {
+  static_assert(WM * WN == 4, "four waves per work-group");
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int A_FLOATS = k_inner_floats(BM);
+  constexpr int B_FLOATS =
+      B_K_INNER ? k_inner_floats(BN) : row_inner_floats(BN);
+  constexpr int STAGE_FLOATS = A_FLOATS + B_FLOATS;
+  extern __shared__ __align__(16) float lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_m = wave / WN, wave_n = wave % WN;
+
+  const unsigned tile = xcd_remap(blockIdx.x, n_tiles);
+  const int m0 = static_cast<int>(tile / n_tiles_n) * BM;
+  const int n0 = static_cast<int>(tile % n_tiles_n) * BN;
+  const int chunks_per_tap = g.src_ch / kBK;
+  const int n_chunks_total = g.win_rows * g.win_cols * chunks_per_tap;
+  const int chunk_begin = blockIdx.y * chunks_per_split;
+  const int n_chunks = min(chunks_per_split, n_chunks_total - chunk_begin);
+
+  const __amdgpu_buffer_rsrc_t src_rsrc = make_rsrc(src, src_bytes);
+  const __amdgpu_buffer_rsrc_t wgt_rsrc = make_rsrc(wgt, wgt_bytes);
+
+  // ---- A gather: lane copies 16 bytes at chunk column a_cc of tile rows
+  // a_r0 + 32 * i.  a_voff = byte offset of (n, iy0, ix0, 4 * a_cc) in two's
+  // complement (it may lie before the tensor for border pixels; adding a
+  // valid tap's offset brings it back in range).
+  constexpr int A_PASSES = BM / 32;
+  const int a_cc = tid & 7;
+  const int a_r0 = tid >> 3;
+  unsigned a_voff[A_PASSES];
+  unsigned a_inval[A_PASSES];  // bit t set: filter tap t is padding
+  const int n_taps = g.win_rows * g.win_cols;
+#pragma unroll
+  for (int i = 0; i < A_PASSES; ++i) {
+    const int m = m0 + a_r0 + 32 * i;
+    unsigned inval = 0xFFFFFFFFu;
+    int off = 0;
+    if (m < g.m_total) {
+      const int px = m % g.p_cols;
+      const int t = m / g.p_cols;
+      const int py = t % g.p_rows;
+      const int n = t / g.p_rows;
+      const int iy0 = py * g.step_rows + g.off_rows;
+      const int ix0 = px * g.step_cols + g.off_cols;
+      off = ((n * g.src_rows + iy0) * g.src_cols + ix0) * g.src_ch + 4 * a_cc;
+      inval = 0;
+      for (int tp = 0; tp < n_taps; ++tp) {
+        const int r = tp / g.win_cols, c = tp - r * g.win_cols;
+        const int iy = iy0 + g.tap_sign * r, ix = ix0 + g.tap_sign * c;
+        const bool ok =
+            static_cast<unsigned>(iy) < static_cast<unsigned>(g.src_rows) &&
+            static_cast<unsigned>(ix) < static_cast<unsigned>(g.src_cols);
+        inval |= ok ? 0u : (1u << tp);
+      }
+    }
+    a_voff[i] = static_cast<unsigned>(off) * 4u;
+    a_inval[i] = inval;
+  }
+
+  // ---- B copy: per-lane constant offsets, scalar chunk offsets
+  constexpr int B_VEC_PER_ROW = B_K_INNER ? kBK / 4 : BN / 4;
+  constexpr int B_ROWS_PER_PASS = kThreads / B_VEC_PER_ROW;
+  constexpr int B_PASSES = (B_K_INNER ? BN : kBK) / B_ROWS_PER_PASS;
+  const int b_vec = tid % B_VEC_PER_ROW;
+  const int b_row0 = tid / B_VEC_PER_ROW;
+  unsigned b_voff[B_K_INNER ? B_PASSES : 1];
+  if (B_K_INNER) {
+#pragma unroll
+    for (int i = 0; i < B_PASSES; ++i) {
+      const int col = n0 + b_row0 + B_ROWS_PER_PASS * i;
+      b_voff[i] = col < g.n_total
+                      ? static_cast<unsigned>(col * g.src_ch + 4 * b_vec) * 4u
+                      : kOob;
+    }
+  } else {
+    const int col = n0 + 4 * b_vec;
+    b_voff[0] = col < g.n_total
+                    ? static_cast<unsigned>(b_row0 * g.n_total + col) * 4u
+                    : kOob;
+  }
+  // scalar byte strides
+  const unsigned b_pass_stride =
+      static_cast<unsigned>(B_ROWS_PER_PASS * g.n_total) * 4u;  // NN only
+  const unsigned b_tap_stride =
+      static_cast<unsigned>(g.n_total * g.src_ch) * 4u;  // K-inner only
+
+  // wave-uniform reduction position: tap index, its (row, col), channel base
+  int tap = chunk_begin / chunks_per_tap;
+  int c0 = (chunk_begin - tap * chunks_per_tap) * kBK;
+  int tap_r = tap / g.win_cols;
+  int tap_c = tap - tap_r * g.win_cols;
+  int chunk = chunk_begin;
+
+  float4 a_reg[A_PASSES];
+  float4 b_reg[B_PASSES];
+
+  auto load_global = [&]() {
+    const unsigned a_soff = static_cast<unsigned>(
+        (g.tap_sign * (tap_r * g.src_cols + tap_c) * g.src_ch + c0) * 4);
+#pragma unroll
+    for (int i = 0; i < A_PASSES; ++i) {
+      const unsigned bad = __builtin_amdgcn_ubfe(a_inval[i], tap, 1);
+      const unsigned voff = (bad << 31) | (a_voff[i] + a_soff);
+      a_reg[i] = __builtin_bit_cast(
+          float4, __builtin_amdgcn_raw_buffer_load_b128(src_rsrc, voff, 0, 0));
+    }
+    if (B_K_INNER) {
+      const unsigned soff =
+          static_cast<unsigned>(tap) * b_tap_stride + static_cast<unsigned>(c0) * 4u;
+#pragma unroll
+      for (int i = 0; i < B_PASSES; ++i) {
+        b_reg[i] = __builtin_bit_cast(
+            float4,
+            __builtin_amdgcn_raw_buffer_load_b128(wgt_rsrc, b_voff[i], soff, 0));
+      }
+    } else {
+      const unsigned soff =
+          static_cast<unsigned>(chunk * kBK * g.n_total) * 4u;
+#pragma unroll
+      for (int i = 0; i < B_PASSES; ++i) {
+        b_reg[i] = __builtin_bit_cast(
+            float4, __builtin_amdgcn_raw_buffer_load_b128(
+                        wgt_rsrc, b_voff[0], soff + i * b_pass_stride, 0));
+      }
+    }
+    // advance the scalar position by one chunk
+    ++chunk;
+    c0 += kBK;
+    if (c0 == g.src_ch) {
+      c0 = 0;
+      ++tap;
+      if (++tap_c == g.win_cols) { tap_c = 0; ++tap_r; }
+    }
+  };
+
+  float* const a_store = lds + a_r0 * (kBK + kPad) + 4 * a_cc;
+  float* const b_store =
+      lds + A_FLOATS +
+      (B_K_INNER ? b_row0 * (kBK + kPad) + 4 * b_vec
+                 : b_row0 * (BN + kPad) + 4 * b_vec);
+  auto store_tiles = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < A_PASSES; ++i) {
+      *reinterpret_cast<float4*>(a_store + stage * STAGE_FLOATS +
+                                 32 * i * (kBK + kPad)) = a_reg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < B_PASSES; ++i) {
+      constexpr int ROW_WORDS = B_K_INNER ? kBK + kPad : BN + kPad;
+      *reinterpret_cast<float4*>(b_store + stage * STAGE_FLOATS +
+                                 B_ROWS_PER_PASS * i * ROW_WORDS) = b_reg[i];
+    }
+  };
+
+  float16v acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  auto compute = [&](int stage) {
+    mma_chunk<TM, TN, true, B_K_INNER, BM, BN>(
+        lds + stage * STAGE_FLOATS, lds + stage * STAGE_FLOATS + A_FLOATS,
+        wave_m * WTM, wave_n * WTN, lane, acc);
+  };
+
+  load_global();
+  store_tiles(0);
+  __syncthreads();
+  // Chunk loop unrolled by the two LDS stages so that every LDS address is a
+  // per-lane constant plus an immediate.
+  int it = 0;
+  for (; it + 2 <= n_chunks - 1; it += 2) {
+    load_global();
+    compute(0);
+    store_tiles(1);
+    __syncthreads();
+    load_global();
+    compute(1);
+    store_tiles(0);
+    __syncthreads();
+  }
+  // 1 or 2 chunks remain in flight: chunk `it` sits in stage 0
+  if (it + 1 < n_chunks) {
+    load_global();
+    compute(0);
+    store_tiles(1);
+    __syncthreads();
+    compute(1);
+  } else {
+    compute(0);
+  }
+
+  // ---- epilogue through a buffer descriptor: rows past the end fall outside
+  // it and are dropped; per-lane constant offset + scalar row offsets.
+  const __amdgpu_buffer_rsrc_t dst_rsrc = make_rsrc(dst, dst_bytes);
+  const int col_l = lane & 31;
+  const int row_l = 4 * (lane >> 5);
+  const unsigned row_bytes = static_cast<unsigned>(g.n_total) * 4u;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wave_n * WTN + 32 * j + col_l;
+      const int m_base = m0 + wave_m * WTM + 32 * i + row_l;
+      const unsigned voff =
+          (col < g.n_total && m_base < g.m_total)
+              ? static_cast<unsigned>(m_base) * row_bytes +
+                    static_cast<unsigned>(col) * 4u
+              : kOob;
+      // The row offset goes into the vector offset, not the scalar offset
+      // operand: hipcc (ROCm 7.2) treats buffer stores that differ only in
+      // their scalar offset as stores to one address and forwards the first
+      // value to all of them.
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const unsigned off =
+            voff + static_cast<unsigned>(8 * (v >> 2) + (v & 3)) * row_bytes;
+        const float val = acc[i][j][v];
+        if (ATOMIC) {
+          __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(val, dst_rsrc, off, 0,
+                                                          0);
+        } else {
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), dst_rsrc,
+                                                off, 0, 0);
+        }
+      }
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256)
+    zero_fill_kernel(float4* __restrict__ p, size_t n_vec) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i < n_vec) p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
 template <int BM, int BN, int WM, int WN, bool B_K_INNER, bool STRIDED>
 void launch_tile(const float* src, const float* wgt, float* dst,
-                 const Gather& g, hipStream_t stream) {
+                 const Gather& g, size_t src_elems, size_t wgt_elems,
+                 int splits, hipStream_t stream) {
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(g.m_total, BM));
   const unsigned tiles_n = static_cast<unsigned>(ceil_div(g.n_total, BN));
-  const unsigned n_blocks = tiles_m * tiles_n;
+  const unsigned n_tiles = tiles_m * tiles_n;
+  const int n_chunks = ceil_div(g.k_total, kBK);
+  const int per_split = ceil_div(n_chunks, splits);
+  splits = ceil_div(n_chunks, per_split);
   constexpr size_t kLdsBytes =
       2 * sizeof(float) *
       (k_inner_floats(BM) +
        (B_K_INNER ? k_inner_floats(BN) : row_inner_floats(BN)));
-  auto kernel = conv_igemm_kernel<BM, BN, WM, WN, B_K_INNER, STRIDED>;
-  // More than the 64 KiB default needs an explicit opt-in (160 KiB per CU).
-  static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(kernel),
-      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  (void)attr;
-  hipLaunchKernelGGL(kernel, dim3(n_blocks), dim3(kThreads), kLdsBytes, stream,
-                     src, wgt, dst, g, tiles_n, n_blocks);
+  const unsigned src_bytes = static_cast<unsigned>(src_elems * sizeof(float));
+  const unsigned wgt_bytes = static_cast<unsigned>(wgt_elems * sizeof(float));
+  const bool fast = !STRIDED && g.src_ch % kBK == 0 &&
+                    g.win_rows * g.win_cols <= 32;
+  const unsigned dst_bytes = static_cast<unsigned>(
+      static_cast<size_t>(g.m_total) * g.n_total * sizeof(float));
+  if (splits > 1) {
+    // Partial sums meet in the output through float atomics: start from zero.
+    const size_t n_vec =
+        static_cast<size_t>(g.m_total) * g.n_total / 4;  // n_total % 4 == 0
+    hipLaunchKernelGGL(zero_fill_kernel,
+                       dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
+                       dim3(256), 0, stream, reinterpret_cast<float4*>(dst),
+                       n_vec);
+    if (fast) {
+      auto kernel = conv_igemm_fast_kernel<BM, BN, WM, WN, B_K_INNER, true>;
+      static const hipError_t attr = hipFuncSetAttribute(
+          reinterpret_cast<const void*>(kernel),
+          hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+      (void)attr;
+      hipLaunchKernelGGL(kernel, dim3(n_tiles, splits), dim3(kThreads),
+                         kLdsBytes, stream, src, wgt, dst, g, src_bytes,
+                         wgt_bytes, dst_bytes, tiles_n, n_tiles, per_split);
+      return;
+    }
+    auto kernel = conv_igemm_kernel<BM, BN, WM, WN, B_K_INNER, STRIDED, true>;
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel),
+        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    (void)attr;
+    hipLaunchKernelGGL(kernel, dim3(n_tiles, splits), dim3(kThreads),
+                       kLdsBytes, stream, src, wgt, dst, g, src_bytes,
+                       wgt_bytes, tiles_n, n_tiles, per_split);
+  } else {
+    if (fast) {
+      auto kernel = conv_igemm_fast_kernel<BM, BN, WM, WN, B_K_INNER, false>;
+      static const hipError_t attr = hipFuncSetAttribute(
+          reinterpret_cast<const void*>(kernel),
+          hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+      (void)attr;
+      hipLaunchKernelGGL(kernel, dim3(n_tiles, 1), dim3(kThreads), kLdsBytes,
+                         stream, src, wgt, dst, g, src_bytes, wgt_bytes,
+                         dst_bytes, tiles_n, n_tiles, per_split);
+      return;
+    }
+    auto kernel = conv_igemm_kernel<BM, BN, WM, WN, B_K_INNER, STRIDED, false>;
+    // More than the 64 KiB default needs an explicit opt-in (160 KiB per CU).
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel),
+        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    (void)attr;
+    hipLaunchKernelGGL(kernel, dim3(n_tiles, 1), dim3(kThreads), kLdsBytes,
+                       stream, src, wgt, dst, g, src_bytes, wgt_bytes, tiles_n,
+                       n_tiles, per_split);
+  }
+}
+
+// Tile shape and reduction split.  The chip has 256 CUs; a launch is balanced
+// when it has several work units per CU, so the largest tile that still
+// yields kTargetUnits tiles is taken, and when even 64x64 tiles are too few
+// the reduction is split across work-groups.
+constexpr int kTargetUnits = 1024;
+
+template <bool B_K_INNER, bool STRIDED>
+void launch_auto(const float* src, const float* wgt, float* dst,
+                 const Gather& g, size_t src_elems, size_t wgt_elems,
+                 hipStream_t stream) {
+  auto tiles = [&](int bm, int bn) {
+    return static_cast<long>(ceil_div(g.m_total, bm)) * ceil_div(g.n_total, bn);
+  };
+  const int n_chunks = ceil_div(g.k_total, kBK);
+  // Developer override for tuning runs: SNN_HIP_IGEMM="<tile>,<splits>" with
+  // tile 0 = 128x128, 1 = 128x64, 2 = 64x64.
+  static const char* tune = getenv("SNN_HIP_IGEMM");
+  if (tune != nullptr) {
+    int tile = 2, splits = 1;
+    sscanf(tune, "%d,%d", &tile, &splits);
+    splits = max(1, min(splits, n_chunks));
+    if (g.n_total % 4 != 0) splits = 1;
+    if (tile == 0)
+      launch_tile<128, 128, 2, 2, B_K_INNER, STRIDED>(
+          src, wgt, dst, g, src_elems, wgt_elems, splits, stream);
+    else if (tile == 1)
+      launch_tile<128, 64, 4, 1, B_K_INNER, STRIDED>(
+          src, wgt, dst, g, src_elems, wgt_elems, splits, stream);
+    else
+      launch_tile<64, 64, 2, 2, B_K_INNER, STRIDED>(
+          src, wgt, dst, g, src_elems, wgt_elems, splits, stream);
+    return;
+  }
+  if (g.n_total > 64 && tiles(128, 128) >= kTargetUnits) {
+    launch_tile<128, 128, 2, 2, B_K_INNER, STRIDED>(src, wgt, dst, g, src_elems,
+                                                    wgt_elems, 1, stream);
+  } else if (tiles(128, 64) >= kTargetUnits) {
+    launch_tile<128, 64, 4, 1, B_K_INNER, STRIDED>(src, wgt, dst, g, src_elems,
+                                                   wgt_elems, 1, stream);
+  } else {
+    const long t = tiles(64, 64);
+    int splits = 1;
+    // n_total % 4 == 0 is needed by the zero fill of the split path
+    if (t < kTargetUnits && g.n_total % 4 == 0) {
+      splits = static_cast<int>((kTargetUnits + t - 1) / t);
+      // keep at least 8 chunks (256 reduction elements) per split
+      splits = max(1, min(splits, n_chunks / 8));
+    }
+    launch_tile<64, 64, 2, 2, B_K_INNER, STRIDED>(src, wgt, dst, g, src_elems,
+                                                  wgt_elems, splits, stream);
+  }
 }
 
 }  // namespace
 
 bool conv2d_igemm_supports(int direction, const snn_hip_conv2d_params& p) {
+  // buffer descriptors address at most kMaxBufferBytes
+  const size_t x = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                   p.channels;
+  const size_t y = static_cast<size_t>(p.batch) * p.out_rows * p.out_cols *
+                   p.features;
+  const size_t w = static_cast<size_t>(p.window_rows) * p.window_cols *
+                   p.channels * p.features;
+  if (max(max(x, y), w) * sizeof(float) > kMaxBufferBytes) return false;
   if (direction == SNN_HIP_FORWARD)
     return p.channels % 4 == 0 && p.features % 4 == 0;
   if (direction == SNN_HIP_INPUT_BACKPROP)
@@ -294,20 +713,19 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
   g.m_total = g.batch * g.p_rows * g.p_cols;
   g.k_total = g.win_rows * g.win_cols * g.src_ch;
 
+  const size_t src_elems = static_cast<size_t>(g.batch) * g.src_rows *
+                           g.src_cols * g.src_ch;
+  const size_t wgt_elems = static_cast<size_t>(p.window_rows) * p.window_cols *
+                           p.channels * p.features;
   if (direction == SNN_HIP_FORWARD) {
-    if (g.n_total > 64)
-      launch_tile<128, 128, 2, 2, false, false>(input, filter, output, g, stream);
-    else
-      launch_tile<128, 64, 4, 1, false, false>(input, filter, output, g, stream);
+    launch_auto<false, false>(input, filter, output, g, src_elems, wgt_elems,
+                              stream);
+  } else if (g.div_rows != 1 || g.div_cols != 1) {
+    launch_auto<true, true>(input, filter, output, g, src_elems, wgt_elems,
+                            stream);
   } else {
-    const bool strided = g.div_rows != 1 || g.div_cols != 1;
-    if (strided) {
-      launch_tile<128, 64, 4, 1, true, true>(input, filter, output, g, stream);
-    } else if (g.n_total > 64) {
-      launch_tile<128, 128, 2, 2, true, false>(input, filter, output, g, stream);
-    } else {
-      launch_tile<128, 64, 4, 1, true, false>(input, filter, output, g, stream);
-    }
+    launch_auto<true, false>(input, filter, output, g, src_elems, wgt_elems,
+                             stream);
   }
   SNN_HIP_CHECK_LAUNCH();
   return SNN_HIP_OK;

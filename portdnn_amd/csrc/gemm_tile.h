@@ -68,30 +68,40 @@ __device__ inline float comp(const float4& v, int t) {
 
 // One BK chunk of MFMA work for a wave tile of TM x TN 32x32 blocks.
 // a_tile / b_tile point at the current LDS stage; a_row0 / b_row0 are the
-// first tile rows (m resp. n) of this wave.
+// first tile rows (m resp. n) of this wave.  Every operand of the chunk is
+// fetched from LDS up front (the fetches of the second half overlap the MFMAs
+// of the first), so the matrix pipe is not gated by one LDS round trip per
+// instruction pair.
 template <int TM, int TN, bool A_K_INNER, bool B_K_INNER, int A_ROWS,
           int B_ROWS>
 __device__ inline void mma_chunk(const float* a_tile, const float* b_tile,
                                  int a_row0, int b_row0, int lane,
                                  float16v (&acc)[TM][TN]) {
+  constexpr int S = kBK / 8;  // sub-steps of 8 reduction indices
   const int l32 = lane & 31;
+  float4 a[S][TM], b[S][TN];
 #pragma unroll
-  for (int s = 0; s < kBK / 8; ++s) {
-    float4 a[TM], b[TN];
+  for (int s = 0; s < S; ++s) {
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      a[i] = A_K_INNER
-                 ? fetch_k_inner(a_tile, a_row0 + 32 * i + l32, s, lane)
-                 : fetch_row_inner<A_ROWS>(a_tile, a_row0 + 32 * i + l32, s,
-                                           lane);
+      a[s][i] = A_K_INNER
+                    ? fetch_k_inner(a_tile, a_row0 + 32 * i + l32, s, lane)
+                    : fetch_row_inner<A_ROWS>(a_tile, a_row0 + 32 * i + l32, s,
+                                              lane);
     }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      b[j] = B_K_INNER
-                 ? fetch_k_inner(b_tile, b_row0 + 32 * j + l32, s, lane)
-                 : fetch_row_inner<B_ROWS>(b_tile, b_row0 + 32 * j + l32, s,
-                                           lane);
+      b[s][j] = B_K_INNER
+                    ? fetch_k_inner(b_tile, b_row0 + 32 * j + l32, s, lane)
+                    : fetch_row_inner<B_ROWS>(b_tile, b_row0 + 32 * j + l32, s,
+                                              lane);
     }
+  }
+  // Keep the compiler's scheduler from sinking the fetches back down between
+  // the MFMAs (it would, to save registers).
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int s = 0; s < S; ++s) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
 #pragma unroll
@@ -99,7 +109,7 @@ __device__ inline void mma_chunk(const float* a_tile, const float* b_tile,
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-              comp(a[i], t), comp(b[j], t), acc[i][j], 0, 0, 0);
+              comp(a[s][i], t), comp(b[s][j], t), acc[i][j], 0, 0, 0);
         }
       }
     }
