@@ -333,7 +333,6 @@ __global__ void __launch_bounds__(kThreads)
   const int a_r0 = tid >> 3;
   unsigned a_voff[A_PASSES];
   unsigned a_inval[A_PASSES];  // bit t set: filter tap t is padding
-  const int n_taps = g.win_rows * g.win_cols;
 #pragma unroll
   for (int i = 0; i < A_PASSES; ++i) {
     const int m = m0 + a_r0 + 32 * i;
@@ -347,14 +346,20 @@ __global__ void __launch_bounds__(kThreads)
       const int iy0 = py * g.step_rows + g.off_rows;
       const int ix0 = px * g.step_cols + g.off_cols;
       off = ((n * g.src_rows + iy0) * g.src_cols + ix0) * g.src_ch + 4 * a_cc;
+      // bit c of col_bad: tap column c falls outside the source row
+      unsigned col_bad = 0;
+      for (int c = 0; c < g.win_cols; ++c) {
+        const unsigned ix = static_cast<unsigned>(ix0 + g.tap_sign * c);
+        col_bad |= (ix < static_cast<unsigned>(g.src_cols) ? 0u : 1u) << c;
+      }
+      const unsigned all_cols = (1u << g.win_cols) - 1u;  // win_cols <= 31
       inval = 0;
-      for (int tp = 0; tp < n_taps; ++tp) {
-        const int r = tp / g.win_cols, c = tp - r * g.win_cols;
-        const int iy = iy0 + g.tap_sign * r, ix = ix0 + g.tap_sign * c;
-        const bool ok =
-            static_cast<unsigned>(iy) < static_cast<unsigned>(g.src_rows) &&
-            static_cast<unsigned>(ix) < static_cast<unsigned>(g.src_cols);
-        inval |= ok ? 0u : (1u << tp);
+      int shift = 0;
+      for (int r = 0; r < g.win_rows; ++r, shift += g.win_cols) {
+        const unsigned iy = static_cast<unsigned>(iy0 + g.tap_sign * r);
+        const unsigned row =
+            iy < static_cast<unsigned>(g.src_rows) ? col_bad : all_cols;
+        inval |= row << shift;
       }
     }
     a_voff[i] = static_cast<unsigned>(off) * 4u;
@@ -395,17 +400,22 @@ __global__ void __launch_bounds__(kThreads)
   int tap_c = tap - tap_r * g.win_cols;
   int chunk = chunk_begin;
 
-  float4 a_reg[A_PASSES];
-  float4 b_reg[B_PASSES];
+  // Two register sets: the global loads of a chunk are issued two chunks
+  // before its data is written to LDS, so their latency is covered by two
+  // chunks of MFMA work (a wave of a 64x64 tile has only 16 MFMAs per chunk).
+  float4 a_reg[2][A_PASSES];
+  float4 b_reg[2][B_PASSES];
+  const int chunk_end = chunk_begin + n_chunks;
 
-  auto load_global = [&]() {
+  auto load_global = [&](int set) {
+    if (chunk >= chunk_end) return;  // wave-uniform
     const unsigned a_soff = static_cast<unsigned>(
         (g.tap_sign * (tap_r * g.src_cols + tap_c) * g.src_ch + c0) * 4);
 #pragma unroll
     for (int i = 0; i < A_PASSES; ++i) {
       const unsigned bad = __builtin_amdgcn_ubfe(a_inval[i], tap, 1);
       const unsigned voff = (bad << 31) | (a_voff[i] + a_soff);
-      a_reg[i] = __builtin_bit_cast(
+      a_reg[set][i] = __builtin_bit_cast(
           float4, __builtin_amdgcn_raw_buffer_load_b128(src_rsrc, voff, 0, 0));
     }
     if (B_K_INNER) {
@@ -413,7 +423,7 @@ __global__ void __launch_bounds__(kThreads)
           static_cast<unsigned>(tap) * b_tap_stride + static_cast<unsigned>(c0) * 4u;
 #pragma unroll
       for (int i = 0; i < B_PASSES; ++i) {
-        b_reg[i] = __builtin_bit_cast(
+        b_reg[set][i] = __builtin_bit_cast(
             float4,
             __builtin_amdgcn_raw_buffer_load_b128(wgt_rsrc, b_voff[i], soff, 0));
       }
@@ -422,7 +432,7 @@ __global__ void __launch_bounds__(kThreads)
           static_cast<unsigned>(chunk * kBK * g.n_total) * 4u;
 #pragma unroll
       for (int i = 0; i < B_PASSES; ++i) {
-        b_reg[i] = __builtin_bit_cast(
+        b_reg[set][i] = __builtin_bit_cast(
             float4, __builtin_amdgcn_raw_buffer_load_b128(
                         wgt_rsrc, b_voff[0], soff + i * b_pass_stride, 0));
       }
@@ -442,17 +452,18 @@ __global__ void __launch_bounds__(kThreads)
       lds + A_FLOATS +
       (B_K_INNER ? b_row0 * (kBK + kPad) + 4 * b_vec
                  : b_row0 * (BN + kPad) + 4 * b_vec);
-  auto store_tiles = [&](int stage) {
+  auto store_tiles = [&](int stage, int set) {
 #pragma unroll
     for (int i = 0; i < A_PASSES; ++i) {
       *reinterpret_cast<float4*>(a_store + stage * STAGE_FLOATS +
-                                 32 * i * (kBK + kPad)) = a_reg[i];
+                                 32 * i * (kBK + kPad)) = a_reg[set][i];
     }
 #pragma unroll
     for (int i = 0; i < B_PASSES; ++i) {
       constexpr int ROW_WORDS = B_K_INNER ? kBK + kPad : BN + kPad;
       *reinterpret_cast<float4*>(b_store + stage * STAGE_FLOATS +
-                                 B_ROWS_PER_PASS * i * ROW_WORDS) = b_reg[i];
+                                 B_ROWS_PER_PASS * i * ROW_WORDS) =
+          b_reg[set][i];
     }
   };
 
@@ -470,31 +481,24 @@ __global__ void __launch_bounds__(kThreads)
         wave_m * WTM, wave_n * WTN, lane, acc);
   };
 
-  load_global();
-  store_tiles(0);
+  // Chunk j is loaded into register set j % 2 and staged in LDS stage j % 2.
+  // The loop is unrolled by two so that stage and set are literals (every LDS
+  // address is then a per-lane constant plus an immediate).
+  load_global(0);  // chunk 0
+  store_tiles(0, 0);
   __syncthreads();
-  // Chunk loop unrolled by the two LDS stages so that every LDS address is a
-  // per-lane constant plus an immediate.
-  int it = 0;
-  for (; it + 2 <= n_chunks - 1; it += 2) {
-    load_global();
-    compute(0);
-    store_tiles(1);
+  load_global(1);  // chunk 1
+  for (int done = 0;; done += 2) {
+    load_global(0);  // chunk done + 2
+    compute(0);      // chunk done
+    if (done + 1 >= n_chunks) break;
+    store_tiles(1, 1);  // chunk done + 1
     __syncthreads();
-    load_global();
-    compute(1);
-    store_tiles(0);
+    load_global(1);  // chunk done + 3
+    compute(1);      // chunk done + 1
+    if (done + 2 >= n_chunks) break;
+    store_tiles(0, 0);  // chunk done + 2
     __syncthreads();
-  }
-  // 1 or 2 chunks remain in flight: chunk `it` sits in stage 0
-  if (it + 1 < n_chunks) {
-    load_global();
-    compute(0);
-    store_tiles(1);
-    __syncthreads();
-    compute(1);
-  } else {
-    compute(0);
   }
 
   // ---- epilogue through a buffer descriptor: rows past the end fall outside
@@ -612,11 +616,18 @@ void launch_tile(const float* src, const float* wgt, float* dst,
   }
 }
 
-// Tile shape and reduction split.  The chip has 256 CUs; a launch is balanced
-// when it has several work units per CU, so the largest tile that still
-// yields kTargetUnits tiles is taken, and when even 64x64 tiles are too few
-// the reduction is split across work-groups.
-constexpr int kTargetUnits = 1024;
+// Tile shape and reduction split.  Measured on MI355X with the ResNet layers:
+// 64x64 tiles (four work-groups resident per CU) beat the larger tiles unless
+// the problem is several times bigger than the chip, because a launch only
+// lasts a few dozen chunk times and balance across the 256 CUs matters more
+// than per-tile reuse.  When 64x64 tiles number fewer than one per resident
+// slot, the reduction is split across work-groups so that there are about
+// kSplitUnits work units; their partial sums meet in the output through float
+// atomics (the order of those additions is not fixed, so the last bits of
+// such outputs can differ from run to run).
+constexpr int kResidentSlots = 1024;  // 256 CUs x 4 work-groups of 64x64
+constexpr int kSplitUnits = 2048;
+constexpr int kMinChunksPerSplit = 8;
 
 template <bool B_K_INNER, bool STRIDED>
 void launch_auto(const float* src, const float* wgt, float* dst,
@@ -645,24 +656,20 @@ void launch_auto(const float* src, const float* wgt, float* dst,
           src, wgt, dst, g, src_elems, wgt_elems, splits, stream);
     return;
   }
-  if (g.n_total > 64 && tiles(128, 128) >= kTargetUnits) {
+  if (g.n_total > 64 && tiles(128, 128) >= 4 * kResidentSlots) {
     launch_tile<128, 128, 2, 2, B_K_INNER, STRIDED>(src, wgt, dst, g, src_elems,
                                                     wgt_elems, 1, stream);
-  } else if (tiles(128, 64) >= kTargetUnits) {
-    launch_tile<128, 64, 4, 1, B_K_INNER, STRIDED>(src, wgt, dst, g, src_elems,
-                                                   wgt_elems, 1, stream);
-  } else {
-    const long t = tiles(64, 64);
-    int splits = 1;
-    // n_total % 4 == 0 is needed by the zero fill of the split path
-    if (t < kTargetUnits && g.n_total % 4 == 0) {
-      splits = static_cast<int>((kTargetUnits + t - 1) / t);
-      // keep at least 8 chunks (256 reduction elements) per split
-      splits = max(1, min(splits, n_chunks / 8));
-    }
-    launch_tile<64, 64, 2, 2, B_K_INNER, STRIDED>(src, wgt, dst, g, src_elems,
-                                                  wgt_elems, splits, stream);
+    return;
   }
+  const long t = tiles(64, 64);
+  int splits = 1;
+  // n_total % 4 == 0 is needed by the zero fill of the split path
+  if (t < kResidentSlots && g.n_total % 4 == 0) {
+    splits = static_cast<int>((kSplitUnits + t - 1) / t);
+    splits = max(1, min(splits, n_chunks / kMinChunksPerSplit));
+  }
+  launch_tile<64, 64, 2, 2, B_K_INNER, STRIDED>(src, wgt, dst, g, src_elems,
+                                                wgt_elems, splits, stream);
 }
 
 }  // namespace
