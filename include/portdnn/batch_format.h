@@ -1,0 +1,5 @@
+// portDNN include path kept for source compatibility.
+#ifndef SNN_FWD_BATCH_FORMAT_H
+#define SNN_FWD_BATCH_FORMAT_H
+#include "portdnn/hip/core.h"
+#endif

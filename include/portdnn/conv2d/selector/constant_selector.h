@@ -1,0 +1,5 @@
+// portDNN include path kept for source compatibility.
+#ifndef SNN_FWD_CONV2D_SELECTOR_CONSTANT_SELECTOR_H
+#define SNN_FWD_CONV2D_SELECTOR_CONSTANT_SELECTOR_H
+#include "portdnn/hip/conv2d.h"
+#endif

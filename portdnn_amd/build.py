@@ -70,11 +70,14 @@ def build_cpp_tests():
     for src in sources:
         exe = os.path.join(out_dir,
                            os.path.splitext(os.path.basename(src))[0])
-        cmd = [HIPCC, "-O2", "-std=c++17", "-x", "hip",
-               "--offload-arch=" + ARCH, "-Wall", "-Wextra",
+        oracle_dir = os.path.join(ROOT, "oracle")
+        # Host programs: the drop-in headers only need the HIP runtime API.
+        cmd = ["g++", "-O2", "-std=c++17", "-Wall", "-Wextra",
                "-Wno-unused-parameter", "-I" + os.path.join(ROOT, "include"),
-               src, "-o", exe, "-L" + HERE, "-lsnn_hip",
-               "-Wl,-rpath," + HERE]
+               "-I/opt/rocm/include", src, "-o", exe, "-L" + HERE,
+               "-lsnn_hip", "-L" + oracle_dir, "-loracle",
+               "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath," + HERE,
+               "-Wl,-rpath," + oracle_dir, "-Wl,-rpath,/opt/rocm/lib"]
         proc = subprocess.run(cmd, stdout=subprocess.PIPE,
                               stderr=subprocess.STDOUT, text=True)
         if proc.returncode != 0:

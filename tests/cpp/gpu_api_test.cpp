@@ -1,0 +1,286 @@
+// GPU test of the sycldnn:: drop-in API through backend::HIPBackend, written
+// in the shape of the reference's fixtures (test/conv2d/convolution_fixture.h:
+// 45-154, test/depthwise_conv2d/depthwise_conv2d_fixture.h:43-89,
+// test/pooling/pooling_fixture.h:53-216): operands 1,2,3,...,max_val repeated,
+// launch through the public template, wait on the returned event, compare
+// with the CPU oracle (which the golden tests pin to the reference's vectors).
+#include <portdnn/backend/hip_backend.h>
+#include <portdnn/conv2d/launch.h>
+#include <portdnn/conv2d/selector/default_selector.h>
+#include <portdnn/conv2d/selector/direct_selector.h>
+#include <portdnn/conv2d/selector/im2col_selector.h>
+#include <portdnn/conv2d/selector/matmul_selector.h>
+#include <portdnn/conv2d/selector/tiled_selector.h>
+#include <portdnn/conv2d/selector/winograd_selector.h>
+#include <portdnn/conv2d/workspace_size.h>
+#include <portdnn/depthwise_conv2d/launch.h>
+#include <portdnn/helpers/padding.h>
+#include <portdnn/pooling/launch.h>
+
+#include <cmath>
+#include <random>
+#include <vector>
+
+#include "../../oracle/oracle.h"
+#include "check.h"
+
+using namespace sycldnn;
+using conv2d::Conv2DParams;
+namespace ct = conv2d::conv_type;
+
+static std::vector<float> iota_data(size_t n, int max_val) {
+  std::vector<float> v(n);
+  for (size_t i = 0; i < n; ++i) v[i] = static_cast<float>(i % max_val + 1);
+  return v;
+}
+static std::vector<float> uniform_data(size_t n, unsigned seed) {
+  std::mt19937 gen(seed);
+  std::uniform_real_distribution<float> d(-1.f, 1.f);
+  std::vector<float> v(n);
+  for (auto& x : v) x = d(gen);
+  return v;
+}
+
+struct DeviceBuffer {
+  float* ptr = nullptr;
+  size_t n = 0;
+  backend::HIPBackend* b;
+  DeviceBuffer(backend::HIPBackend& be, std::vector<float> const& host)
+      : n(host.size()), b(&be) {
+    ptr = be.allocate<float>(n > 0 ? n : 1);
+    (void)hipMemcpy(ptr, host.data(), n * sizeof(float), hipMemcpyHostToDevice);
+  }
+  DeviceBuffer(backend::HIPBackend& be, size_t count) : n(count), b(&be) {
+    ptr = be.allocate<float>(n > 0 ? n : 1);
+    (void)hipMemset(ptr, 0xff, n * sizeof(float));  // NaN pattern
+  }
+  ~DeviceBuffer() { b->deallocate(ptr); }
+  std::vector<float> host() const {
+    std::vector<float> h(n);
+    (void)hipMemcpy(h.data(), ptr, n * sizeof(float), hipMemcpyDeviceToHost);
+    return h;
+  }
+};
+
+static bool close(std::vector<float> const& got, std::vector<float> const& ref,
+                  bool exact) {
+  if (got.size() != ref.size()) return false;
+  double sq = 0;
+  for (float r : ref) sq += static_cast<double>(r) * r;
+  const double scale = std::max(1.0, std::sqrt(sq / std::max<size_t>(1, ref.size())));
+  for (size_t i = 0; i < ref.size(); ++i) {
+    const double err = std::fabs(static_cast<double>(got[i]) - ref[i]);
+    const double tol = exact ? 0.0 : 1e-4 * std::fabs(ref[i]) + 1e-5 * scale;
+    if (!(err <= tol)) {
+      std::printf("  mismatch at %zu: got %g expected %g\n", i, got[i], ref[i]);
+      return false;
+    }
+  }
+  return true;
+}
+
+static oracle_params to_oracle(Conv2DParams const& p) {
+  return {p.channels, p.features,    p.batch,       p.in_rows,  p.in_cols,
+          p.window_rows, p.window_cols, p.stride_rows, p.stride_cols,
+          p.out_rows, p.out_cols,    p.pad_rows,    p.pad_cols};
+}
+
+template <typename ConvType>
+static void test_conv(Conv2DParams const& params, conv2d::Selector& selector,
+                      backend::HIPBackend& backend, bool iota) {
+  if (selector.select<ConvType>(params) == conv2d::Algorithm::NotSupported)
+    return;  // as GTEST_SKIP in the reference fixture
+  const auto sizes = conv2d::get_sizes<ConvType>(params);
+  const auto in = iota ? iota_data(sizes.input_size, 64)
+                       : uniform_data(sizes.input_size, 11);
+  const auto fil = iota ? iota_data(sizes.filter_size, 64)
+                        : uniform_data(sizes.filter_size, 12);
+  DeviceBuffer d_in(backend, in), d_fil(backend, fil);
+  DeviceBuffer d_out(backend, sizes.output_size);
+  const auto ws = conv2d::query_workspace_size<ConvType>(params, selector);
+  DeviceBuffer d_ws(backend, ws.recommended_size);
+  auto status = conv2d::launch<float, ConvType>(
+      d_in.ptr, d_fil.ptr, d_out.ptr, params, selector, backend, d_ws.ptr,
+      ws.recommended_size);
+  CHECK(status.status == StatusCode::OK);
+  status.event.wait_and_throw();
+  std::vector<float> ref(sizes.output_size);
+  const oracle_params op = to_oracle(params);
+  if (std::is_same<ConvType, ct::Forward>::value)
+    oracle_conv2d_forward(in.data(), fil.data(), ref.data(), &op, 1);
+  else if (std::is_same<ConvType, ct::InputBackprop>::value)
+    oracle_conv2d_input_backprop(in.data(), fil.data(), ref.data(), &op, 1);
+  else
+    oracle_conv2d_filter_backprop(in.data(), fil.data(), ref.data(), &op, 1);
+  const bool ok = close(d_out.host(), ref, iota);
+  if (!ok)
+    std::printf("  selector %s window %d stride %d C %d K %d\n",
+                selector.name(), params.window_rows, params.stride_rows,
+                params.channels, params.features);
+  CHECK(ok);
+}
+
+static Conv2DParams conv_params(int n, int h, int w, int c, int k, int window,
+                                int stride, PaddingMode mode) {
+  Conv2DParams p{};
+  p.channels = c; p.features = k; p.batch = n; p.in_rows = h; p.in_cols = w;
+  p.window_rows = p.window_cols = window;
+  p.stride_rows = p.stride_cols = stride;
+  p.dilation_rows = p.dilation_cols = 1;
+  return helpers::add_padding_to(p, mode);
+}
+
+static void test_all_conv(backend::HIPBackend& backend) {
+  conv2d::DirectSelector direct;
+  conv2d::TiledSelector tiled;
+  conv2d::Im2colSelector im2col;
+  conv2d::WinogradSelector wino;
+  conv2d::MatmulSelector mm;
+  auto def = conv2d::get_default_selector(backend);
+  conv2d::Selector* selectors[] = {&direct, &tiled, &im2col, &wino, &mm,
+                                   def.get()};
+  const Conv2DParams shapes[] = {
+      conv_params(1, 4, 4, 1, 1, 3, 1, PaddingMode::SAME),
+      conv_params(3, 5, 6, 2, 4, 3, 2, PaddingMode::VALID),
+      conv_params(2, 9, 9, 4, 4, 5, 1, PaddingMode::SAME),
+      conv_params(2, 12, 12, 32, 64, 3, 1, PaddingMode::SAME),
+      conv_params(2, 8, 8, 64, 256, 1, 1, PaddingMode::VALID),
+      conv_params(1, 20, 20, 3, 8, 7, 2, PaddingMode::SAME),
+  };
+  for (auto* sel : selectors) {
+    for (auto const& p : shapes) {
+      for (bool iota : {true, false}) {
+        test_conv<ct::Forward>(p, *sel, backend, iota);
+        test_conv<ct::InputBackprop>(p, *sel, backend, iota);
+        test_conv<ct::FilterBackprop>(p, *sel, backend, iota);
+      }
+    }
+  }
+}
+
+static void test_depthwise(backend::HIPBackend& backend) {
+  depthwise_conv2d::DepthwiseConv2DParams p{};
+  p.channels = 32; p.channel_multiplier = 1; p.batch = 2;
+  p.in_rows = p.in_cols = 14; p.window_rows = p.window_cols = 3;
+  p.stride_rows = p.stride_cols = 2;
+  p = helpers::add_padding_to(p, PaddingMode::SAME);
+  const auto sizes = depthwise_conv2d::get_sizes<ct::Forward>(p);
+  const auto in = uniform_data(sizes.input_size, 3);
+  const auto fil = uniform_data(sizes.filter_size, 4);
+  DeviceBuffer d_in(backend, in), d_fil(backend, fil);
+  DeviceBuffer d_out(backend, sizes.output_size);
+  auto st = depthwise_conv2d::launch<float, ct::Forward>(
+      d_in.ptr, d_fil.ptr, d_out.ptr, p, backend);
+  CHECK(st.status == StatusCode::OK);
+  st.event.wait_and_throw();
+  const oracle_params op = {p.channels, p.channel_multiplier, p.batch,
+                            p.in_rows, p.in_cols, p.window_rows, p.window_cols,
+                            p.stride_rows, p.stride_cols, p.out_rows,
+                            p.out_cols, p.pad_rows, p.pad_cols};
+  std::vector<float> ref(sizes.output_size);
+  oracle_depthwise_forward(in.data(), fil.data(), ref.data(), &op, 1);
+  CHECK(close(d_out.host(), ref, false));
+  // gradient w.r.t. the input: dY has the forward output's size
+  const auto dy = uniform_data(sizes.output_size, 5);
+  DeviceBuffer d_dy(backend, dy), d_dx(backend, sizes.input_size);
+  st = depthwise_conv2d::launch<float, ct::InputBackprop>(
+      d_dy.ptr, d_fil.ptr, d_dx.ptr, p, backend);
+  CHECK(st.status == StatusCode::OK);
+  st.event.wait_and_throw();
+  std::vector<float> ref_dx(sizes.input_size);
+  oracle_depthwise_input_backprop(dy.data(), fil.data(), ref_dx.data(), &op, 1);
+  CHECK(close(d_dx.host(), ref_dx, false));
+}
+
+static void test_pooling(backend::HIPBackend& backend) {
+  pooling::PoolingParams p{};
+  p.in_rows = p.in_cols = 15; p.window_rows = p.window_cols = 3;
+  p.stride_rows = p.stride_cols = 2; p.batch = 2; p.channels = 16;
+  p = helpers::add_padding_to(p, PaddingMode::SAME);
+  const auto sizes = pooling::get_sizes<pooling::Forward>(p);
+  const auto in = uniform_data(sizes.input_size, 7);
+  DeviceBuffer d_in(backend, in), d_out(backend, sizes.output_size);
+  const oracle_params op = {p.channels, 0, p.batch, p.in_rows, p.in_cols,
+                            p.window_rows, p.window_cols, p.stride_rows,
+                            p.stride_cols, p.out_rows, p.out_cols, p.pad_rows,
+                            p.pad_cols};
+  auto st = pooling::launch<float, pooling::Max, pooling::Forward>(
+      d_in.ptr, d_out.ptr, p, backend);
+  CHECK(st.status == StatusCode::OK);
+  st.event.wait_and_throw();
+  std::vector<float> ref(sizes.output_size);
+  oracle_pool_max_forward(in.data(), ref.data(), &op, 0);
+  const auto y = d_out.host();
+  CHECK(close(y, ref, true));
+  // max gradient through the four-pointer overload
+  const auto dy = iota_data(sizes.output_size, 97);
+  DeviceBuffer d_dy(backend, dy), d_dx(backend, sizes.input_size);
+  st = pooling::launch<float, pooling::Max, pooling::Backpropagate>(
+      d_in.ptr, d_out.ptr, d_dy.ptr, d_dx.ptr, p, backend);
+  CHECK(st.status == StatusCode::OK);
+  st.event.wait_and_throw();
+  std::vector<float> ref_dx(sizes.input_size);
+  oracle_pool_max_grad(in.data(), ref.data(), dy.data(), ref_dx.data(), &op, 0);
+  CHECK(close(d_dx.host(), ref_dx, true));
+  // average forward and gradient
+  st = pooling::launch<float, pooling::Average, pooling::Forward>(
+      d_in.ptr, d_out.ptr, p, backend);
+  CHECK(st.status == StatusCode::OK);
+  st.event.wait_and_throw();
+  oracle_pool_avg_forward(in.data(), ref.data(), &op, 1);
+  CHECK(close(d_out.host(), ref, false));
+  st = pooling::launch<float, pooling::Average, pooling::Backpropagate>(
+      d_dy.ptr, d_dx.ptr, p, backend);
+  CHECK(st.status == StatusCode::OK);
+  st.event.wait_and_throw();
+  oracle_pool_avg_grad(dy.data(), ref_dx.data(), &op, 1);
+  CHECK(close(d_dx.host(), ref_dx, false));
+}
+
+static void test_event_dependencies(backend::HIPBackend& backend) {
+  // test/conv2d/conv2d_event_dependencies.cc: a launch given an event must
+  // run after it.  Here: conv B consumes conv A's output on another stream.
+  hipStream_t other;
+  if (hipStreamCreate(&other) != hipSuccess) { CHECK(false); return; }
+  backend::HIPBackend backend2(other);
+  conv2d::Im2colSelector sel;
+  auto p = conv_params(4, 28, 28, 32, 32, 3, 1, PaddingMode::SAME);
+  const auto sizes = conv2d::get_sizes<ct::Forward>(p);
+  const auto in = uniform_data(sizes.input_size, 21);
+  const auto fil = uniform_data(sizes.filter_size, 22);
+  DeviceBuffer d_in(backend, in), d_fil(backend, fil);
+  DeviceBuffer d_mid(backend, sizes.output_size), d_out(backend, sizes.output_size);
+  auto a = conv2d::launch<float, ct::Forward>(d_in.ptr, d_fil.ptr, d_mid.ptr, p,
+                                              sel, backend, nullptr, 0);
+  CHECK(a.status == StatusCode::OK);
+  auto b = conv2d::launch<float, ct::Forward>(d_mid.ptr, d_fil.ptr, d_out.ptr,
+                                              p, sel, backend2, nullptr, 0,
+                                              {a.event});
+  CHECK(b.status == StatusCode::OK);
+  b.event.wait_and_throw();
+  const oracle_params op = to_oracle(p);
+  std::vector<float> mid(sizes.output_size), ref(sizes.output_size);
+  oracle_conv2d_forward(in.data(), fil.data(), mid.data(), &op, 1);
+  oracle_conv2d_forward(mid.data(), fil.data(), ref.data(), &op, 1);
+  CHECK(close(d_out.host(), ref, false));
+  (void)hipStreamDestroy(other);
+}
+
+int main() {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
+    std::printf("gpu_api_test: no GPU\n");
+    return 2;
+  }
+  hipStream_t stream;
+  if (hipStreamCreate(&stream) != hipSuccess) return 2;
+  {
+    backend::HIPBackend backend(stream);
+    test_all_conv(backend);
+    test_depthwise(backend);
+    test_pooling(backend);
+    test_event_dependencies(backend);
+  }
+  (void)hipStreamDestroy(stream);
+  return report("gpu_api_test");
+}
