@@ -539,6 +539,165 @@ __global__ void __launch_bounds__(kThreads)
   }
 }
 
+// ---------------------------------------------------------------------------
+// Filter backprop: dW[q][k] = sum_m A[m][q] * dY[m][k], q = (r, s, c),
+// m = (n, oy, ox).  The reduction runs over every output pixel, so both
+// operands are read with the reduction index as the slow dimension and both
+// LDS tiles are row-inner ([32 pixels][64 + 4]); a 64-wide q tile lies inside
+// one filter tap (C % 64 == 0).  The pixel range is split across work-groups
+// (blockIdx.y) and the partial tiles are added into dW with float atomics.
+struct FilterBackpropGeom {
+  int batch, in_rows, in_cols, channels;
+  int out_rows, out_cols, features;
+  int win_rows, win_cols;
+  int stride_rows, stride_cols, pad_rows, pad_cols;
+  int m_total;  // batch * out_rows * out_cols
+};
+
+__global__ void __launch_bounds__(kThreads)
+    conv_filter_backprop_kernel(const float* __restrict__ x,
+                                const float* __restrict__ dy,
+                                float* __restrict__ dw, FilterBackpropGeom g,
+                                unsigned x_bytes, unsigned dy_bytes,
+                                unsigned dw_bytes, int chunks_per_split) {
+  constexpr int BM = 64, BN = 64;
+  constexpr int A_FLOATS = row_inner_floats(BM);
+  constexpr int STAGE_FLOATS = A_FLOATS + row_inner_floats(BN);
+  __shared__ __align__(16) float lds[2 * STAGE_FLOATS];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_m = wave >> 1, wave_n = wave & 1;
+
+  // tile: 64 consecutive q inside one tap x 64 features
+  const int tiles_n = (g.features + BN - 1) / BN;
+  const int tile_q = blockIdx.x / tiles_n;
+  const int n0 = (blockIdx.x - tile_q * tiles_n) * BN;
+  const int q0 = tile_q * BM;
+  const int tap = q0 / g.channels;
+  const int c0 = q0 - tap * g.channels;
+  const int tap_r = tap / g.win_cols;
+  const int tap_c = tap - tap_r * g.win_cols;
+
+  const int n_chunks_total = (g.m_total + kBK - 1) / kBK;
+  const int chunk_begin = blockIdx.y * chunks_per_split;
+  const int n_chunks = min(chunks_per_split, n_chunks_total - chunk_begin);
+
+  const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, x_bytes);
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, dy_bytes);
+
+  // This lane copies float4 `vec` of pixel rows row0 and row0 + 16 of every
+  // 32-pixel chunk, for both operands.
+  const int vec = tid & 15;
+  const int row0 = tid >> 4;
+  int ox[2], iy[2];      // output column; input row of this tap
+  int x_off[2];          // element offset of (n, iy, ox*stride - pad + tap_c, c0 + 4*vec)
+  unsigned dy_off[2];    // byte offset of (m, n0 + 4*vec)
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m = chunk_begin * kBK + row0 + 16 * i;
+    const int o = m % g.out_cols;
+    const int t = m / g.out_cols;
+    const int oy = t % g.out_rows;
+    const int n = t / g.out_rows;
+    ox[i] = o;
+    iy[i] = oy * g.stride_rows - g.pad_rows + tap_r;
+    x_off[i] = ((n * g.in_rows + iy[i]) * g.in_cols + o * g.stride_cols -
+                g.pad_cols + tap_c) * g.channels + c0 + 4 * vec;
+    dy_off[i] = (n0 + 4 * vec < g.features)
+                    ? static_cast<unsigned>(m * g.features + n0 + 4 * vec) * 4u
+                    : kOob;
+  }
+  // element-offset deltas of the pixel walk
+  const int step_px = g.stride_cols * g.channels;  // ox += 1
+  const int step_row =
+      (g.stride_rows * g.in_cols - g.out_cols * g.stride_cols) * g.channels;
+  const int step_img =
+      (g.in_rows - g.out_rows * g.stride_rows) * g.in_cols * g.channels;
+  const int iy_first = -g.pad_rows + tap_r;
+  const int iy_end = iy_first + g.out_rows * g.stride_rows;
+
+  float4 a_reg[2], b_reg[2];
+  auto load_global = [&]() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int ix = ox[i] * g.stride_cols - g.pad_cols + tap_c;
+      const bool ok =
+          (static_cast<unsigned>(iy[i]) < static_cast<unsigned>(g.in_rows)) &
+          (static_cast<unsigned>(ix) < static_cast<unsigned>(g.in_cols));
+      a_reg[i] = buffer_load4(
+          x_rsrc, ok ? static_cast<unsigned>(x_off[i]) * 4u : kOob);
+      b_reg[i] = buffer_load4(dy_rsrc, dy_off[i]);
+      // advance this row by one chunk (32 pixels)
+      ox[i] += kBK;
+      x_off[i] += kBK * step_px;
+      while (ox[i] >= g.out_cols) {
+        ox[i] -= g.out_cols;
+        x_off[i] += step_row;
+        iy[i] += g.stride_rows;
+        if (iy[i] == iy_end) {
+          iy[i] = iy_first;
+          x_off[i] += step_img;
+        }
+      }
+      if (dy_off[i] != kOob) dy_off[i] += kBK * g.features * 4u;
+    }
+  };
+  float* const a_store = lds + row0 * (BM + kPad) + 4 * vec;
+  float* const b_store = lds + A_FLOATS + row0 * (BN + kPad) + 4 * vec;
+  auto store_tiles = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      *reinterpret_cast<float4*>(a_store + stage * STAGE_FLOATS +
+                                 16 * i * (BM + kPad)) = a_reg[i];
+      *reinterpret_cast<float4*>(b_store + stage * STAGE_FLOATS +
+                                 16 * i * (BN + kPad)) = b_reg[i];
+    }
+  };
+
+  float16v acc[1][1];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[0][0][v] = 0.f;
+  auto compute = [&](int stage) {
+    mma_chunk<1, 1, false, false, BM, BN>(
+        lds + stage * STAGE_FLOATS, lds + stage * STAGE_FLOATS + A_FLOATS,
+        wave_m * 32, wave_n * 32, lane, acc);
+  };
+
+  load_global();
+  store_tiles(0);
+  __syncthreads();
+  for (int done = 0;; done += 2) {
+    if (done + 1 < n_chunks) load_global();
+    compute(0);
+    if (done + 1 >= n_chunks) break;
+    store_tiles(1);
+    __syncthreads();
+    if (done + 2 < n_chunks) load_global();
+    compute(1);
+    if (done + 2 >= n_chunks) break;
+    store_tiles(0);
+    __syncthreads();
+  }
+
+  const __amdgpu_buffer_rsrc_t dw_rsrc = make_rsrc(dw, dw_bytes);
+  const int col = n0 + wave_n * 32 + (lane & 31);
+  const int q_base = q0 + wave_m * 32 + 4 * (lane >> 5);
+  const unsigned row_bytes = static_cast<unsigned>(g.features) * 4u;
+  const unsigned voff = col < g.features
+                            ? static_cast<unsigned>(q_base) * row_bytes +
+                                  static_cast<unsigned>(col) * 4u
+                            : kOob;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const unsigned off =
+        voff + static_cast<unsigned>(8 * (v >> 2) + (v & 3)) * row_bytes;
+    const float val = acc[0][0][v];
+    __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(val, dw_rsrc, off, 0, 0);
+  }
+}
+
 __global__ void __launch_bounds__(256)
     zero_fill_kernel(float4* __restrict__ p, size_t n_vec) {
   const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
@@ -674,6 +833,40 @@ void launch_auto(const float* src, const float* wgt, float* dst,
 
 }  // namespace
 
+static int launch_filter_backprop(const float* x, const float* dy, float* dw,
+                           const snn_hip_conv2d_params& p, hipStream_t stream) {
+  FilterBackpropGeom g;
+  g.batch = p.batch; g.in_rows = p.in_rows; g.in_cols = p.in_cols;
+  g.channels = p.channels; g.out_rows = p.out_rows; g.out_cols = p.out_cols;
+  g.features = p.features; g.win_rows = p.window_rows;
+  g.win_cols = p.window_cols; g.stride_rows = p.stride_rows;
+  g.stride_cols = p.stride_cols; g.pad_rows = p.pad_rows;
+  g.pad_cols = p.pad_cols;
+  g.m_total = p.batch * p.out_rows * p.out_cols;
+  const size_t x_elems =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
+  const size_t dy_elems = static_cast<size_t>(g.m_total) * p.features;
+  const size_t dw_elems = static_cast<size_t>(p.window_rows) * p.window_cols *
+                          p.channels * p.features;
+  const int tiles = (p.window_rows * p.window_cols * p.channels / 64) *
+                    ceil_div(p.features, 64);
+  const int n_chunks = ceil_div(g.m_total, kBK);
+  int splits = max(1, min(ceil_div(kSplitUnits, tiles),
+                          n_chunks / kMinChunksPerSplit));
+  const int per_split = ceil_div(n_chunks, splits);
+  splits = ceil_div(n_chunks, per_split);
+  const size_t n_vec = dw_elems / 4;
+  hipLaunchKernelGGL(zero_fill_kernel,
+                     dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
+                     dim3(256), 0, stream, reinterpret_cast<float4*>(dw), n_vec);
+  hipLaunchKernelGGL(conv_filter_backprop_kernel, dim3(tiles, splits),
+                     dim3(kThreads), 0, stream, x, dy, dw, g,
+                     static_cast<unsigned>(x_elems * 4),
+                     static_cast<unsigned>(dy_elems * 4),
+                     static_cast<unsigned>(dw_elems * 4), per_split);
+  return SNN_HIP_OK;
+}
+
 bool conv2d_igemm_supports(int direction, const snn_hip_conv2d_params& p) {
   // buffer descriptors address at most kMaxBufferBytes
   const size_t x = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
@@ -687,13 +880,19 @@ bool conv2d_igemm_supports(int direction, const snn_hip_conv2d_params& p) {
     return p.channels % 4 == 0 && p.features % 4 == 0;
   if (direction == SNN_HIP_INPUT_BACKPROP)
     return p.features % 4 == 0;
-  return false;
+  // filter backprop: a 64-wide tile of (tap, channel) must lie inside one tap
+  return p.channels % 64 == 0 && p.features % 4 == 0;
 }
 
 int launch_conv2d_igemm_f32(int direction, const float* input,
                             const float* filter, float* output,
                             const snn_hip_conv2d_params& p,
                             hipStream_t stream) {
+  if (direction == SNN_HIP_FILTER_BACKPROP) {
+    const int rc = launch_filter_backprop(input, filter, output, p, stream);
+    SNN_HIP_CHECK_LAUNCH();
+    return rc;
+  }
   Gather g;
   g.batch = p.batch;
   g.win_rows = p.window_rows;
