@@ -44,6 +44,9 @@ struct Gather {
   int m_total;               // batch * p_rows * p_cols
   int k_total;               // win_rows * win_cols * src_ch
   int n_total;               // GEMM columns
+  // Independent problems of the same shape (blockIdx.z): element strides
+  // between their operands.  All zero for a convolution.
+  int z_src, z_wgt, z_dst;
 };
 
 // Buffer addressing: loads go through raw buffer descriptors so that an
@@ -321,6 +324,9 @@ __global__ void __launch_bounds__(kThreads)
   const int chunk_begin = blockIdx.y * chunks_per_split;
   const int n_chunks = min(chunks_per_split, n_chunks_total - chunk_begin);
 
+  src += static_cast<size_t>(blockIdx.z) * g.z_src;
+  wgt += static_cast<size_t>(blockIdx.z) * g.z_wgt;
+  dst += static_cast<size_t>(blockIdx.z) * g.z_dst;
   const __amdgpu_buffer_rsrc_t src_rsrc = make_rsrc(src, src_bytes);
   const __amdgpu_buffer_rsrc_t wgt_rsrc = make_rsrc(wgt, wgt_bytes);
 
@@ -707,7 +713,7 @@ __global__ void __launch_bounds__(256)
 template <int BM, int BN, int WM, int WN, bool B_K_INNER, bool STRIDED>
 void launch_tile(const float* src, const float* wgt, float* dst,
                  const Gather& g, size_t src_elems, size_t wgt_elems,
-                 int splits, hipStream_t stream) {
+                 int splits, hipStream_t stream, int batches = 1) {
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(g.m_total, BM));
   const unsigned tiles_n = static_cast<unsigned>(ceil_div(g.n_total, BN));
   const unsigned n_tiles = tiles_m * tiles_n;
@@ -726,8 +732,9 @@ void launch_tile(const float* src, const float* wgt, float* dst,
       static_cast<size_t>(g.m_total) * g.n_total * sizeof(float));
   if (splits > 1) {
     // Partial sums meet in the output through float atomics: start from zero.
-    const size_t n_vec =
-        static_cast<size_t>(g.m_total) * g.n_total / 4;  // n_total % 4 == 0
+    // (a batched launch keeps its problems contiguous: z_dst == m * n)
+    const size_t n_vec = static_cast<size_t>(batches) * g.m_total *
+                         g.n_total / 4;  // n_total % 4 == 0
     hipLaunchKernelGGL(zero_fill_kernel,
                        dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
                        dim3(256), 0, stream, reinterpret_cast<float4*>(dst),
@@ -738,9 +745,10 @@ void launch_tile(const float* src, const float* wgt, float* dst,
           reinterpret_cast<const void*>(kernel),
           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
       (void)attr;
-      hipLaunchKernelGGL(kernel, dim3(n_tiles, splits), dim3(kThreads),
-                         kLdsBytes, stream, src, wgt, dst, g, src_bytes,
-                         wgt_bytes, dst_bytes, tiles_n, n_tiles, per_split);
+      hipLaunchKernelGGL(kernel, dim3(n_tiles, splits, batches),
+                         dim3(kThreads), kLdsBytes, stream, src, wgt, dst, g,
+                         src_bytes, wgt_bytes, dst_bytes, tiles_n, n_tiles,
+                         per_split);
       return;
     }
     auto kernel = conv_igemm_kernel<BM, BN, WM, WN, B_K_INNER, STRIDED, true>;
@@ -758,9 +766,9 @@ void launch_tile(const float* src, const float* wgt, float* dst,
           reinterpret_cast<const void*>(kernel),
           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
       (void)attr;
-      hipLaunchKernelGGL(kernel, dim3(n_tiles, 1), dim3(kThreads), kLdsBytes,
-                         stream, src, wgt, dst, g, src_bytes, wgt_bytes,
-                         dst_bytes, tiles_n, n_tiles, per_split);
+      hipLaunchKernelGGL(kernel, dim3(n_tiles, 1, batches), dim3(kThreads),
+                         kLdsBytes, stream, src, wgt, dst, g, src_bytes,
+                         wgt_bytes, dst_bytes, tiles_n, n_tiles, per_split);
       return;
     }
     auto kernel = conv_igemm_kernel<BM, BN, WM, WN, B_K_INNER, STRIDED, false>;
@@ -884,6 +892,52 @@ bool conv2d_igemm_supports(int direction, const snn_hip_conv2d_params& p) {
   return p.channels % 64 == 0 && p.features % 4 == 0;
 }
 
+bool batched_gemm_mfma_supports(int m, int k, int n, const void* a,
+                                const void* b, const void* c) {
+  auto aligned = [](const void* p) {
+    return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+  };
+  return k % kBK == 0 && n % 4 == 0 && aligned(a) && aligned(b) &&
+         aligned(c) &&
+         static_cast<size_t>(m) * max(k, n) * sizeof(float) <= kMaxBufferBytes &&
+         static_cast<size_t>(k) * n * sizeof(float) <= kMaxBufferBytes;
+}
+
+int launch_batched_gemm_mfma_f32(const float* a, const float* b, float* c,
+                                 int batches, int m, int k, int n,
+                                 hipStream_t stream) {
+  // C[z] = A[z] (m x k) * B[z] (k x n): a 1x1 "convolution" over m pixels.
+  Gather g;
+  g.batch = 1;
+  g.p_rows = 1; g.p_cols = m;
+  g.src_rows = 1; g.src_cols = m;
+  g.src_ch = k;
+  g.win_rows = g.win_cols = 1;
+  g.step_rows = g.step_cols = 1;
+  g.off_rows = g.off_cols = 0;
+  g.tap_sign = 1;
+  g.div_rows = g.div_cols = 1;
+  g.m_total = m;
+  g.k_total = k;
+  g.n_total = n;
+  g.z_src = m * k;
+  g.z_wgt = k * n;
+  g.z_dst = m * n;
+  const long tiles = static_cast<long>(ceil_div(m, 64)) * ceil_div(n, 64) * batches;
+  const int n_chunks = k / kBK;
+  int splits = 1;
+  if (tiles < kResidentSlots) {
+    splits = static_cast<int>((kSplitUnits + tiles - 1) / tiles);
+    splits = max(1, min(splits, n_chunks / kMinChunksPerSplit));
+  }
+  launch_tile<64, 64, 2, 2, false, false>(a, b, c, g,
+                                          static_cast<size_t>(m) * k,
+                                          static_cast<size_t>(k) * n, splits,
+                                          stream, batches);
+  SNN_HIP_CHECK_LAUNCH();
+  return SNN_HIP_OK;
+}
+
 int launch_conv2d_igemm_f32(int direction, const float* input,
                             const float* filter, float* output,
                             const snn_hip_conv2d_params& p,
@@ -918,6 +972,7 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
   }
   g.m_total = g.batch * g.p_rows * g.p_cols;
   g.k_total = g.win_rows * g.win_cols * g.src_ch;
+  g.z_src = g.z_wgt = g.z_dst = 0;
 
   const size_t src_elems = static_cast<size_t>(g.batch) * g.src_rows *
                            g.src_cols * g.src_ch;

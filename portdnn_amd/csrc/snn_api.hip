@@ -270,6 +270,29 @@ int launch_gemm_path<float>(int direction, const float* input,
   return launch_conv2d_direct<float>(direction, input, filter, output, p, s);
 }
 
+// Winograd / WinogradLarge: F(2x2,3x3) for forward and input backprop of 3x3
+// stride-1 convolutions.  The filter gradient and the 1x3 / 3x1 windows the
+// selector also accepts are computed by the implicit-GEMM kernels (the result
+// is the same convolution; no Winograd tiling exists for them here), and so
+// is WinogradLarge's F(4x4,3x3), whose larger constants cost accuracy.
+template <typename T>
+int launch_winograd_path(int direction, const T* input, const T* filter,
+                         T* output, const snn_hip_conv2d_params& p,
+                         T* workspace, size_t workspace_elems, hipStream_t s) {
+  return launch_gemm_path<T>(direction, input, filter, output, p, s);
+}
+template <>
+int launch_winograd_path<float>(int direction, const float* input,
+                                const float* filter, float* output,
+                                const snn_hip_conv2d_params& p,
+                                float* workspace, size_t workspace_elems,
+                                hipStream_t s) {
+  if (conv2d_winograd_supports(direction, p))
+    return launch_conv2d_winograd_f32(direction, input, filter, output, p,
+                                      workspace, workspace_elems, s);
+  return launch_gemm_path<float>(direction, input, filter, output, p, s);
+}
+
 template <typename T>
 int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
                     const snn_hip_conv2d_params* params, int algorithm,
@@ -289,14 +312,13 @@ int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
   if (!fits_int32(sz.input) || !fits_int32(sz.filter) || !fits_int32(sz.output))
     return SNN_HIP_INDEX_EXCEEDED;
   hipStream_t s = as_stream(stream);
-  (void)workspace;
-  (void)workspace_elems;
   switch (algorithm) {
     case SNN_HIP_ALGO_WINOGRAD:
     case SNN_HIP_ALGO_WINOGRAD_LARGE:
       if (workspace == nullptr || workspace_elems == 0)
         return SNN_HIP_INSUFFICIENT_WORKSPACE;
-      return launch_conv2d_direct<T>(direction, input, filter, output, p, s);
+      return launch_winograd_path<T>(direction, input, filter, output, p,
+                                     workspace, workspace_elems, s);
     case SNN_HIP_ALGO_TILED:
     case SNN_HIP_ALGO_IM2COL:
     case SNN_HIP_ALGO_MATMUL:

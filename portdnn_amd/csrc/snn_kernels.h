@@ -22,6 +22,24 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
                             const float* filter, float* output,
                             const snn_hip_conv2d_params& p, hipStream_t stream);
 
+// Batched row-major GEMM C[z] = A[z] (m x k) * B[z] (k x n) on the same MFMA
+// kernel; operands of consecutive problems are contiguous.  `supports` checks
+// k % 32 == 0, n % 4 == 0 and 16-byte alignment.
+bool batched_gemm_mfma_supports(int m, int k, int n, const void* a,
+                                const void* b, const void* c);
+int launch_batched_gemm_mfma_f32(const float* a, const float* b, float* c,
+                                 int batches, int m, int k, int n,
+                                 hipStream_t stream);
+
+// Winograd F(2x2,3x3) convolution, forward and input backprop
+// (conv2d_winograd.hip).  `workspace` holds the three transform buffers.
+bool conv2d_winograd_supports(int direction, const snn_hip_conv2d_params& p);
+int launch_conv2d_winograd_f32(int direction, const float* input,
+                               const float* filter, float* output,
+                               const snn_hip_conv2d_params& p,
+                               float* workspace, size_t workspace_elems,
+                               hipStream_t stream);
+
 // Depthwise convolution, all three directions (depthwise.hip).
 template <typename T>
 int launch_depthwise(int direction, const T* input, const T* filter, T* output,
