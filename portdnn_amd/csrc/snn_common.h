@@ -40,6 +40,7 @@ inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 constexpr int kWave = 64;
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+inline unsigned ceil_div(unsigned a, unsigned b) { return (a + b - 1) / b; }
 inline size_t ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
 
 // True when a tensor of `elems` elements can be addressed with 32-bit signed
