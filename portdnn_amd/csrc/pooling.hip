@@ -28,6 +28,7 @@ struct MaxOp {
   __device__ void accumulate(float x) {
     if (x > v) v = x;  // a NaN never compares greater
   }
+  __device__ void merge(float partial) { accumulate(partial); }
   __device__ float value(int) const { return v; }
 };
 struct MaxNanOp {
@@ -36,12 +37,14 @@ struct MaxNanOp {
   __device__ void accumulate(float x) {
     if (x != x || x > v) v = x;  // a NaN wins and then sticks
   }
+  __device__ void merge(float partial) { accumulate(partial); }
   __device__ float value(int) const { return v; }
 };
 struct AvgOp {
   float v;
   __device__ void init(float) { v = 0.f; }
   __device__ void accumulate(float x) { v += x; }
+  __device__ void merge(float partial) { v += partial; }
   __device__ float value(int tally) const {
     return v / static_cast<float>(tally);
   }
@@ -127,6 +130,216 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
   for (int i = 0; i < VEC; ++i) res[i] = op[i].value(tally);
   VecIO<T, VEC>::store(out + idx * VEC, res);
+}
+
+// ---- 3x3 forward, four channels per lane, TH consecutive output rows -------
+// Each input row of the strip is loaded once (three column taps) and folded
+// into every output row it belongs to, so vertically adjacent windows share
+// their rows in registers.  Taps outside the image are redirected to the
+// nearest in-image tap of the same window for the max operators (a duplicate
+// does not change a maximum, nor whether a NaN is present) and read as zero
+// for the average, whose divisor is the analytic in-bounds count.
+typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
+constexpr unsigned kOobOffset = 0x7FFFFFF0u;
+
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* p, size_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0,
+                                           static_cast<unsigned>(bytes),
+                                           0x00020000);
+}
+template <typename T>
+struct BufVec4;
+template <>
+struct BufVec4<float> {
+  __device__ static void load(__amdgpu_buffer_rsrc_t r, unsigned off,
+                              float (&v)[4]) {
+    const float4 t = __builtin_bit_cast(
+        float4, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0));
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+  __device__ static void store(__amdgpu_buffer_rsrc_t r, unsigned off,
+                               const float (&v)[4]) {
+    __builtin_amdgcn_raw_buffer_store_b128(
+        __builtin_bit_cast(uint4v, make_float4(v[0], v[1], v[2], v[3])), r, off,
+        0, 2);  // streaming store
+  }
+};
+template <>
+struct BufVec4<_Float16> {
+  typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+  __device__ static void load(__amdgpu_buffer_rsrc_t r, unsigned off,
+                              float (&v)[4]) {
+    const half4 t = __builtin_bit_cast(
+        half4, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0));
+    v[0] = static_cast<float>(t.x); v[1] = static_cast<float>(t.y);
+    v[2] = static_cast<float>(t.z); v[3] = static_cast<float>(t.w);
+  }
+  __device__ static void store(__amdgpu_buffer_rsrc_t r, unsigned off,
+                               const float (&v)[4]) {
+    half4 t;
+    t.x = static_cast<_Float16>(v[0]); t.y = static_cast<_Float16>(v[1]);
+    t.z = static_cast<_Float16>(v[2]); t.w = static_cast<_Float16>(v[3]);
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2v, t), r, off,
+                                          0, 2);
+  }
+};
+
+template <typename Op>
+struct IsAverage {
+  static constexpr bool value = false;
+};
+template <>
+struct IsAverage<AvgOp> {
+  static constexpr bool value = true;
+};
+
+template <typename T, typename Op, int STRIDE, int TH>
+__global__ void __launch_bounds__(256)
+    pool_forward_3x3_strip_kernel(const T* __restrict__ in, T* __restrict__ out,
+                                  snn_hip_pooling_params p, int n_strips,
+                                  unsigned n_items) {
+  const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+  if (idx >= n_items) return;
+  const int C = p.channels;
+  const unsigned cv = static_cast<unsigned>(C) / 4u;
+  const int c = static_cast<int>(idx % cv) * 4;
+  unsigned rest = idx / cv;
+  const int ox = static_cast<int>(rest % static_cast<unsigned>(p.out_cols));
+  rest /= static_cast<unsigned>(p.out_cols);
+  const int strip = static_cast<int>(rest % static_cast<unsigned>(n_strips));
+  const int n = static_cast<int>(rest / static_cast<unsigned>(n_strips));
+  const int oy0 = strip * TH;
+  constexpr unsigned kEsz = sizeof(T);
+  constexpr bool kAvg = IsAverage<Op>::value;
+  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(
+      in, static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * C * kEsz);
+  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(
+      out, static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * C * kEsz);
+  Op acc[TH][4];
+#pragma unroll
+  for (int t = 0; t < TH; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[t][i].init(lowest_of<T>());
+  const int x0 = ox * STRIDE - p.pad_cols;
+  const int y0 = oy0 * STRIDE - p.pad_rows;
+  const int img = n * p.in_rows * p.in_cols;
+  // column taps: clamp into the image (max) or mark as zero fill (average)
+  int col[3];
+  bool col_ok[3];
+#pragma unroll
+  for (int sx = 0; sx < 3; ++sx) {
+    col_ok[sx] = static_cast<unsigned>(x0 + sx) < static_cast<unsigned>(p.in_cols);
+    col[sx] = min(max(x0 + sx, 0), p.in_cols - 1);
+  }
+  constexpr int NR = (TH - 1) * STRIDE + 3;
+#pragma unroll
+  for (int j = 0; j < NR; ++j) {
+    const int y = y0 + j;
+    const bool row_ok = static_cast<unsigned>(y) < static_cast<unsigned>(p.in_rows);
+    // For the max operators a row below / above the image is replaced by the
+    // nearest image row of the same window; rows that belong to no window of
+    // this strip are never folded in.
+    const int yc = min(max(y, 0), p.in_rows - 1);
+    float row[3][4];
+#pragma unroll
+    for (int sx = 0; sx < 3; ++sx) {
+      unsigned off;
+      if (kAvg) {
+        off = (row_ok & col_ok[sx])
+                  ? static_cast<unsigned>((img + y * p.in_cols + x0 + sx) * C + c) * kEsz
+                  : kOobOffset;
+      } else {
+        off = static_cast<unsigned>((img + yc * p.in_cols + col[sx]) * C + c) * kEsz;
+      }
+      BufVec4<T>::load(in_rsrc, off, row[sx]);
+    }
+#pragma unroll
+    for (int t = 0; t < TH; ++t) {
+      const int r = j - t * STRIDE;
+      if (r < 0 || r > 2) continue;
+#pragma unroll
+      for (int sx = 0; sx < 3; ++sx)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[t][i].accumulate(row[sx][i]);
+    }
+  }
+  const int c_lo = max(x0, 0), c_hi = min(x0 + 3, p.in_cols);
+  const int out_base = ((n * p.out_rows + oy0) * p.out_cols + ox) * C + c;
+#pragma unroll
+  for (int t = 0; t < TH; ++t) {
+    const int ry = y0 + t * STRIDE;
+    const int tally = (min(ry + 3, p.in_rows) - max(ry, 0)) * (c_hi - c_lo);
+    float res[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) res[i] = acc[t][i].value(tally);
+    BufVec4<T>::store(out_rsrc,
+                      oy0 + t < p.out_rows
+                          ? static_cast<unsigned>(out_base + t * p.out_cols * C) * kEsz
+                          : kOobOffset,
+                      res);
+  }
+}
+
+// ---- windows covering most of a small image (global pooling) ---------------
+// One work-group per (image, 64-channel-vector group, output pixel); the
+// window rows are spread over the 4 waves and combined through LDS, so the 49
+// taps of a 7x7 global average are 13 loads deep instead of 49.
+template <typename T, typename Op>
+__global__ void __launch_bounds__(256)
+    pool_forward_rowsplit_kernel(const T* __restrict__ in, T* __restrict__ out,
+                                 snn_hip_pooling_params p, int n_groups) {
+  __shared__ float part[4][64][4];
+  const int C = p.channels;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  unsigned b = blockIdx.x;
+  const int grp = static_cast<int>(b % static_cast<unsigned>(n_groups));
+  b /= static_cast<unsigned>(n_groups);
+  const int ox = static_cast<int>(b % static_cast<unsigned>(p.out_cols));
+  b /= static_cast<unsigned>(p.out_cols);
+  const int oy = static_cast<int>(b % static_cast<unsigned>(p.out_rows));
+  const int n = static_cast<int>(b / static_cast<unsigned>(p.out_rows));
+  const int c = (grp * 64 + lane) * 4;
+  const bool active = c < C;
+  int r0 = oy * p.stride_rows - p.pad_rows;
+  const int r1 = min(r0 + p.window_rows, p.in_rows);
+  r0 = max(r0, 0);
+  int c0 = ox * p.stride_cols - p.pad_cols;
+  const int c1 = min(c0 + p.window_cols, p.in_cols);
+  c0 = max(c0, 0);
+  Op acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc[i].init(lowest_of<T>());
+  if (active) {
+    const T* base =
+        in + static_cast<size_t>(n) * p.in_rows * p.in_cols * C + c;
+    for (int r = r0 + wave; r < r1; r += 4) {
+      for (int col = c0; col < c1; ++col) {
+        float v[4];
+        VecIO<T, 4>::load(base + (static_cast<size_t>(r) * p.in_cols + col) * C,
+                          v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i].accumulate(v[i]);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) part[wave][lane][i] = acc[i].v;
+  __syncthreads();
+  if (wave == 0 && active) {
+    float res[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      Op total = acc[i];
+      for (int w = 1; w < 4; ++w) total.merge(part[w][lane][i]);
+      res[i] = total.value((r1 - r0) * (c1 - c0));
+    }
+    VecIO<T, 4>::store(
+        out + ((static_cast<size_t>(n) * p.out_rows + oy) * p.out_cols + ox) * C +
+            c,
+        res);
+  }
 }
 
 __device__ inline bool pool_equal(float a, float b, bool nan_mode) {
@@ -242,7 +455,51 @@ int launch_forward_op(const T* input, T* output,
   constexpr int kBlock = 256;
   const size_t n_out =
       static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * p.channels;
-  if (p.channels % 4 == 0) {
+  const size_t in_bytes = static_cast<size_t>(p.batch) * p.in_rows *
+                          p.in_cols * p.channels * sizeof(T);
+  const bool is3x3 = p.window_rows == 3 && p.window_cols == 3 &&
+                     p.stride_rows == p.stride_cols &&
+                     (p.stride_rows == 1 || p.stride_rows == 2);
+  // every window must overlap the image (the strip kernel redirects outside
+  // taps to the nearest inside tap of the same window)
+  const bool overlaps =
+      p.pad_rows < 3 && p.pad_cols < 3 &&
+      (p.out_rows - 1) * p.stride_rows - p.pad_rows < p.in_rows &&
+      (p.out_cols - 1) * p.stride_cols - p.pad_cols < p.in_cols;
+  if (p.channels % 4 == 0 && is3x3 && overlaps && in_bytes < 0x7FFFFFF0u &&
+      n_out * sizeof(T) < 0x7FFFFFF0u) {
+    const size_t per_row =
+        static_cast<size_t>(p.batch) * p.out_cols * (p.channels / 4);
+    int th = 4;
+    while (th > 1 && per_row * ceil_div(p.out_rows, th) < 150000) th /= 2;
+    const int n_strips = ceil_div(p.out_rows, th);
+    const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
+    const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
+#define SNN_POOL_STRIP(STRIDE, TH)                                             \
+  hipLaunchKernelGGL((pool_forward_3x3_strip_kernel<T, Op, STRIDE, TH>), grid, \
+                     dim3(kBlock), 0, stream, input, output, p, n_strips,      \
+                     n_items)
+    if (p.stride_rows == 1) {
+      if (th == 4) SNN_POOL_STRIP(1, 4);
+      else if (th == 2) SNN_POOL_STRIP(1, 2);
+      else SNN_POOL_STRIP(1, 1);
+    } else {
+      if (th == 4) SNN_POOL_STRIP(2, 4);
+      else if (th == 2) SNN_POOL_STRIP(2, 2);
+      else SNN_POOL_STRIP(2, 1);
+    }
+#undef SNN_POOL_STRIP
+  } else if (p.channels % 4 == 0 && p.window_rows >= 4 &&
+             static_cast<size_t>(p.batch) * p.out_rows * p.out_cols *
+                     ceil_div(p.channels, 256) >= 256 &&
+             n_out / 4 < 200000) {
+    // few, large windows: split the window rows over the waves
+    const int n_groups = ceil_div(p.channels, 256);
+    const unsigned blocks = static_cast<unsigned>(
+        static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * n_groups);
+    hipLaunchKernelGGL((pool_forward_rowsplit_kernel<T, Op>), dim3(blocks),
+                       dim3(kBlock), 0, stream, input, output, p, n_groups);
+  } else if (p.channels % 4 == 0) {
     const size_t n_vec = n_out / 4;
     hipLaunchKernelGGL((pool_forward_kernel<T, Op, 4>),
                        dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{kBlock}))),
