@@ -257,13 +257,24 @@ inline bool aligned16(const void* p) {
 // width and alignment requirements hold, the direct kernel otherwise.
 template <typename T>
 int launch_gemm_path(int direction, const T* input, const T* filter, T* output,
-                     const snn_hip_conv2d_params& p, hipStream_t s) {
-  return launch_conv2d_direct<T>(direction, input, filter, output, p, s);
+                     const snn_hip_conv2d_params& p, hipStream_t s,
+                     T* workspace = nullptr, size_t workspace_elems = 0);
+template <>
+int launch_gemm_path<_Float16>(int direction, const _Float16* input,
+                               const _Float16* filter, _Float16* output,
+                               const snn_hip_conv2d_params& p, hipStream_t s,
+                               _Float16* workspace, size_t workspace_elems) {
+  if (direction == SNN_HIP_FORWARD && conv2d_igemm_f16_supports(p) &&
+      aligned16(input) && aligned16(filter) && aligned16(output))
+    return launch_conv2d_igemm_f16(input, filter, output, p, workspace,
+                                   workspace_elems, s);
+  return launch_conv2d_direct<_Float16>(direction, input, filter, output, p, s);
 }
 template <>
 int launch_gemm_path<float>(int direction, const float* input,
                             const float* filter, float* output,
-                            const snn_hip_conv2d_params& p, hipStream_t s) {
+                            const snn_hip_conv2d_params& p, hipStream_t s,
+                            float*, size_t) {
   if (conv2d_igemm_supports(direction, p) && aligned16(input) &&
       aligned16(filter) && aligned16(output))
     return launch_conv2d_igemm_f32(direction, input, filter, output, p, s);
@@ -322,7 +333,8 @@ int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
     case SNN_HIP_ALGO_TILED:
     case SNN_HIP_ALGO_IM2COL:
     case SNN_HIP_ALGO_MATMUL:
-      return launch_gemm_path<T>(direction, input, filter, output, p, s);
+      return launch_gemm_path<T>(direction, input, filter, output, p, s,
+                                 workspace, workspace_elems);
     default:
       return launch_conv2d_direct<T>(direction, input, filter, output, p, s);
   }

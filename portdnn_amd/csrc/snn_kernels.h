@@ -40,6 +40,14 @@ int launch_conv2d_winograd_f32(int direction, const float* input,
                                float* workspace, size_t workspace_elems,
                                hipStream_t stream);
 
+// Half-precision forward convolution on MFMA (conv2d_igemm_f16.hip).  The
+// workspace, when large enough, receives the re-laid-out filter.
+bool conv2d_igemm_f16_supports(const snn_hip_conv2d_params& p);
+int launch_conv2d_igemm_f16(const _Float16* input, const _Float16* filter,
+                            _Float16* output, const snn_hip_conv2d_params& p,
+                            _Float16* workspace, size_t workspace_elems,
+                            hipStream_t stream);
+
 // Depthwise convolution, all three directions (depthwise.hip).
 template <typename T>
 int launch_depthwise(int direction, const T* input, const T* filter, T* output,

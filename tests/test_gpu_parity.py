@@ -426,6 +426,51 @@ def test_f16_conv_forward(size, ch, window):
         assert_close_f16(got, ref, ("f16", ALGO_NAME[algo], size, ch))
 
 
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, window, stride, same
+    (3, 13, 11, 64, 40, 3, 1, True),     # ragged rows, features not x32
+    (2, 17, 9, 128, 72, 3, 2, True),     # stride 2
+    (1, 9, 9, 64, 200, 5, 1, False),     # VALID, 25 taps
+    (5, 7, 7, 192, 8, 1, 1, False),      # 1x1, three chunks per tap
+    (2, 33, 31, 64, 130, 3, 2, False),   # features just past two tiles
+])
+def test_f16_conv_forward_ragged(shape):
+    batch, rows, cols, ch, feats, window, stride, same = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, window, stride, same)
+    rng = np.random.default_rng(750 + rows)
+    n_in, n_fil, _ = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x = uniform(rng, n_in).astype(np.float16)
+    w = uniform(rng, n_fil).astype(np.float16)
+    ref = oracle.conv2d_forward(x.astype(np.float32), w.astype(np.float32),
+                                oracle_params(p, feats), acc64=True)
+    for algo in (ALGO.IM2COL, ALGO.DIRECT):
+        got = ops.conv2d(dev(x, torch.float16), dev(w, torch.float16), p,
+                         DIRECTION.FORWARD, algo).float().cpu().numpy()
+        assert_close_f16(got, ref, ("f16 ragged", ALGO_NAME[algo], shape))
+
+
+def test_f16_conv_forward_full_batch_sampled():
+    # Batch 128 takes the 128x128 work-group tile of the f16 kernel.
+    p = ops.conv_params(128, 28, 28, 128, 128, 3, 1, True)
+    rng = np.random.default_rng(760)
+    n_in, n_fil, _ = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x = uniform(rng, n_in).astype(np.float16)
+    w = uniform(rng, n_fil).astype(np.float16)
+    got = ops.conv2d(dev(x, torch.float16), dev(w, torch.float16), p,
+                     DIRECTION.FORWARD, ALGO.IM2COL).float().cpu().numpy()
+    samples = np.stack([rng.integers(0, p.batch, 800),
+                        rng.integers(0, p.out_rows, 800),
+                        rng.integers(0, p.out_cols, 800),
+                        rng.integers(0, p.features, 800)], axis=1)
+    samples[:4, 1] = [0, 0, p.out_rows - 1, p.out_rows - 1]
+    samples[:4, 2] = [0, p.out_cols - 1, 0, p.out_cols - 1]
+    samples[:4, 0] = [0, p.batch - 1, p.batch - 1, 0]
+    ref = sampled_forward_reference(x, w, p, samples)
+    flat = ((samples[:, 0] * p.out_rows + samples[:, 1]) * p.out_cols +
+            samples[:, 2]) * p.features + samples[:, 3]
+    assert_close_f16(got[flat], ref, "f16 batch 128 sampled")
+
+
 @pytest.mark.parametrize("size,ch,stride", MOBILENET)
 def test_f16_depthwise_forward(size, ch, stride):
     p = ops.depthwise_params(2, size, size, ch, 1, 3, stride, True)
