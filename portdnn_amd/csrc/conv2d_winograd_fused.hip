@@ -1,0 +1,727 @@
+// Winograd F(2x2,3x3) convolution in one pass over the data (gfx950), forward
+// and input backprop, fp32.
+//
+// Same mathematics as the three-stage chain in conv2d_winograd.hip, which
+// follows portDNN's (include/portdnn/internal/conv2d/winograd/launch.h:63-264,
+// src/conv2d/winograd/kernels/tiles_impl.h:70-240), but the transformed input
+// V and the products M never reach HBM:
+//
+//   * a small kernel transforms the filter once per launch into U, stored in
+//     the exact order the matrix instruction wants its B operand, so that the
+//     main kernel fetches it with one contiguous 1 KiB wave load per
+//     (xi, 32 features, 8 channels) straight into registers;
+//   * a work-group owns 32 tiles (2x2 output pixels each) x 32 features and
+//     walks the channels 16 at a time: every lane gathers one tile's 4x4
+//     patch for a channel pair (zero-filling buffer loads for the padding),
+//     applies Bt d B in registers and writes the 16 transformed values to
+//     LDS as V[xi][tile][channel];
+//   * wave w multiplies the four xi = 4w .. 4w+3 planes,
+//     M[xi] (32 tiles x 32 features) += V[xi] (32 x 16) * U[xi] (16 x 32),
+//     on v_mfma_f32_32x32x2_f32 (4 x 16 accumulator registers);
+//   * at the end At m A is applied: along xi's column index inside each lane,
+//     along its row index across the four waves through LDS, and the 2x2
+//     output pixels are written with 16-byte stores (or float atomics when
+//     the channel range is split across work-groups to fill the GPU).
+//
+// The multiplications done on the matrix cores are 16/36 of the direct
+// algorithm's.
+#include <cstdlib>
+#ifndef WF_EXP
+#define WF_EXP 0
+#endif
+
+#include "gemm_tile.h"
+#include "snn_kernels.h"
+
+namespace snn {
+namespace {
+
+using gemm::comp;
+using gemm::float16v;
+using gemm::xcd_remap;
+
+constexpr int kTiles = 32;              // Winograd tiles per work-group
+constexpr int kFeat = 32;               // features per work-group
+constexpr int kChunk = 16;              // channels per LDS stage
+constexpr int kRow = kChunk + 4;        // floats per LDS row (bank spread)
+constexpr int kPlane = kTiles * kRow;   // floats per xi plane
+constexpr int kLdsFloats = 16 * kPlane;
+constexpr unsigned kOob = 0x7FFFFFF0u;
+constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
+
+typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+
+struct FusedGeom {
+  int in_rows, in_cols, in_ch;
+  int out_rows, out_cols, out_ch;
+  int pad_rows, pad_cols;
+  int tile_rows, tile_cols;
+  int n_tiles;
+};
+
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* p,
+                                                   unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes,
+                                           0x00020000);
+}
+
+__device__ inline float2 operator+(float2 a, float2 b) {
+  return make_float2(a.x + b.x, a.y + b.y);
+}
+__device__ inline float2 operator-(float2 a, float2 b) {
+  return make_float2(a.x - b.x, a.y - b.y);
+}
+__device__ inline float4 operator+(float4 a, float4 b) {
+  return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
+}
+__device__ inline float4 operator-(float4 a, float4 b) {
+  return make_float4(a.x - b.x, a.y - b.y, a.z - b.z, a.w - b.w);
+}
+
+// U = G g Gt for four consecutive input channels of one output channel,
+// written in B-operand order:
+//   u[xi][co / 32][ci / 8][lane = co % 32 + 32 * ((ci % 8) / 4)][ci % 4].
+// For the input gradient g[r][s] = W[2-r][2-s][co][ci] (mirrored taps, channel
+// and feature roles swapped).
+__global__ void __launch_bounds__(256)
+    wino_filter_pack_kernel(const float* __restrict__ w, float* __restrict__ u,
+                            int channels, int features, bool backprop) {
+  const int cin = backprop ? features : channels;
+  const int cout = backprop ? channels : features;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (cin / 4) * cout) return;
+  const int co = idx % cout, cq = idx / cout;
+  float uu[16][4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int ci = 4 * cq + t;
+    float g[3][3];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+      for (int s = 0; s < 3; ++s) {
+        g[r][s] =
+            backprop
+                ? w[((static_cast<size_t>(2 - r) * 3 + (2 - s)) * channels +
+                     co) * features + ci]
+                : w[((static_cast<size_t>(r) * 3 + s) * channels + ci) *
+                        features + co];
+      }
+    float h[4][3];  // G g
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+      h[0][s] = g[0][s];
+      h[1][s] = 0.5f * (g[0][s] + g[1][s] + g[2][s]);
+      h[2][s] = 0.5f * (g[0][s] - g[1][s] + g[2][s]);
+      h[3][s] = g[2][s];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uu[i * 4 + 0][t] = h[i][0];
+      uu[i * 4 + 1][t] = 0.5f * (h[i][0] + h[i][1] + h[i][2]);
+      uu[i * 4 + 2][t] = 0.5f * (h[i][0] - h[i][1] + h[i][2]);
+      uu[i * 4 + 3][t] = h[i][2];
+    }
+  }
+  const int fblocks = cout / kFeat;
+  const int cgroups = cin / 8;
+  const int lane = co % kFeat + 32 * (cq & 1);
+  const size_t base =
+      ((static_cast<size_t>(co / kFeat) * cgroups + cq / 2) * 64 + lane) * 4;
+  const size_t xi_stride = static_cast<size_t>(fblocks) * cgroups * 256;
+#pragma unroll
+  for (int xi = 0; xi < 16; ++xi) {
+    *reinterpret_cast<float4*>(u + xi * xi_stride + base) =
+        make_float4(uu[xi][0], uu[xi][1], uu[xi][2], uu[xi][3]);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+    wino_zero_fill_kernel(float4* __restrict__ p, size_t n_vec) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i < n_vec) p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+template <bool ATOMIC>
+__global__ void __launch_bounds__(256)
+    wino_fused_kernel(const float* __restrict__ in, const float* __restrict__ u,
+                      float* __restrict__ out, FusedGeom g, unsigned in_bytes,
+                      unsigned u_bytes, unsigned out_bytes, unsigned n_fblocks,
+                      unsigned n_units, int chunks_per_split) {
+  __shared__ __align__(16) float lds_v[kLdsFloats];
+  __shared__ int lds_tile_off[kTiles];
+  __shared__ int lds_tile_flags[kTiles];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const unsigned unit = xcd_remap(blockIdx.x, n_units);
+  const unsigned fb = unit % n_fblocks;
+  const int mb = static_cast<int>(unit / n_fblocks);
+  const int n_chunks = g.in_ch / kChunk;
+  const int chunk_begin = static_cast<int>(blockIdx.y) * chunks_per_split;
+  const int chunk_end = min(n_chunks, chunk_begin + chunks_per_split);
+
+  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_bytes);
+  const __amdgpu_buffer_rsrc_t u_rsrc = make_rsrc(u, u_bytes);
+
+  // Gather role: this lane owns tile `tile_l` of the work-group and the
+  // channel pair `pair` of every chunk.
+  const int tile_l = tid >> 3, pair = tid & 7;
+  unsigned p_off[16];
+  {
+    const int tile = mb * kTiles + tile_l;
+    const bool live = tile < g.n_tiles;
+    const int tx = tile % g.tile_cols;
+    const int t2 = tile / g.tile_cols;
+    const int ty = t2 % g.tile_rows;
+    const int n = t2 / g.tile_rows;
+    const int y0 = 2 * ty - g.pad_rows, x0 = 2 * tx - g.pad_cols;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int y = y0 + i, x = x0 + j;
+        const bool ok = live && static_cast<unsigned>(y) <
+                                    static_cast<unsigned>(g.in_rows) &&
+                        static_cast<unsigned>(x) <
+                            static_cast<unsigned>(g.in_cols);
+        p_off[i * 4 + j] =
+            ok ? static_cast<unsigned>(
+                     (((n * g.in_rows + y) * g.in_cols + x) * g.in_ch +
+                      2 * pair) * 4)
+               : kOob;
+      }
+    if (pair == 0) {
+      lds_tile_off[tile_l] =
+          live ? ((n * g.out_rows + 2 * ty) * g.out_cols + 2 * tx) *
+                     g.out_ch * 4
+               : -1;
+      lds_tile_flags[tile_l] = (2 * ty + 1 < g.out_rows ? 1 : 0) |
+                               (2 * tx + 1 < g.out_cols ? 2 : 0);
+    }
+  }
+
+  // B operand addresses: wave-uniform plane bases, lane * 16 bytes inside a
+  // 1 KiB (xi, feature block, channel group) record.
+  const unsigned u_lane = static_cast<unsigned>(lane) * 16u;
+  const unsigned cgroups = static_cast<unsigned>(g.in_ch) / 8u;
+  unsigned u_base[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    u_base[j] = ((static_cast<unsigned>(4 * wave + j) * n_fblocks + fb) *
+                 cgroups) * 1024u;
+
+  auto load_patch = [&](int chunk, float2 (&d)[16]) {
+    const unsigned soff = static_cast<unsigned>(chunk * kChunk * 4);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      d[q] = __builtin_bit_cast(
+          float2,
+          __builtin_amdgcn_raw_buffer_load_b64(in_rsrc, p_off[q], soff, 0));
+    }
+  };
+  auto load_b = [&](int chunk, float4 (&b)[2][4]) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        b[s][j] = __builtin_bit_cast(
+            float4, __builtin_amdgcn_raw_buffer_load_b128(
+                        u_rsrc, u_lane,
+                        u_base[j] + static_cast<unsigned>(2 * chunk + s) * 1024u,
+                        0));
+      }
+  };
+  float* const v_store = lds_v + tile_l * kRow + 2 * pair;
+  auto transform_store = [&](const float2 (&d)[16]) {
+    float2 t[4][4];  // Bt d
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      t[0][j] = d[0 * 4 + j] - d[2 * 4 + j];
+      t[1][j] = d[1 * 4 + j] + d[2 * 4 + j];
+      t[2][j] = d[2 * 4 + j] - d[1 * 4 + j];
+      t[3][j] = d[1 * 4 + j] - d[3 * 4 + j];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *reinterpret_cast<float2*>(v_store + (i * 4 + 0) * kPlane) =
+          t[i][0] - t[i][2];
+      *reinterpret_cast<float2*>(v_store + (i * 4 + 1) * kPlane) =
+          t[i][1] + t[i][2];
+      *reinterpret_cast<float2*>(v_store + (i * 4 + 2) * kPlane) =
+          t[i][2] - t[i][1];
+      *reinterpret_cast<float2*>(v_store + (i * 4 + 3) * kPlane) =
+          t[i][1] - t[i][3];
+    }
+  };
+
+  float16v acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+
+  const float* const a_base =
+      lds_v + (4 * wave * kTiles + (lane & 31)) * kRow + 4 * (lane >> 5);
+  auto compute = [&](const float4 (&b)[2][4]) {
+    float4 a[2][4];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        a[s][j] = *reinterpret_cast<const float4*>(a_base + j * kPlane + 8 * s);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+              comp(a[s][j], t), comp(b[s][j], t), acc[j], 0, 0, 0);
+  };
+
+  // Loads for the next chunk are issued unconditionally (the last iteration
+  // re-reads its own chunk) so that the wait counters the compiler places
+  // before the matrix instructions stay exact instead of being merged over a
+  // branch.
+  float4 b[2][4], b_next[2][4];
+  float2 d[16];
+  load_patch(chunk_begin, d);
+  load_b(chunk_begin, b);
+  transform_store(d);
+  __syncthreads();
+  for (int c = chunk_begin; c < chunk_end; ++c) {
+    const int next = min(c + 1, chunk_end - 1);
+#if !(WF_EXP & 1)
+    load_patch(next, d);
+#endif
+#if !(WF_EXP & 2)
+    load_b(next, b_next);
+#endif
+#if !(WF_EXP & 8)
+    compute(b);
+#endif
+    __syncthreads();  // every wave has read this chunk's V
+#if !(WF_EXP & 4)
+    if (c + 1 < chunk_end) transform_store(d);
+#endif
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[s][j] = b_next[s][j];
+  }
+
+  // At m A.  Along xi's column index (inside the lane): s[b] for b = 0, 1;
+  // S[i = wave][b][v][lane] goes to LDS (32 KiB, the V buffer is free now).
+  {
+    float* const s_base = lds_v + (wave * 2 * 16) * 64 + lane;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      s_base[v * 64] = acc[0][v] + acc[1][v] + acc[2][v];
+      s_base[(16 + v) * 64] = acc[1][v] - acc[2][v] - acc[3][v];
+    }
+  }
+  __syncthreads();
+  // Along xi's row index (across waves), four consecutive features per lane.
+  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_bytes);
+  const unsigned out_row_bytes =
+      static_cast<unsigned>(g.out_cols) * g.out_ch * 4u;
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const int q = tid & 15;   // lanes 4q .. 4q+3 of the accumulator layout
+    const int v = tid >> 4;   // accumulator register
+    float4 s[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      s[i] = *reinterpret_cast<const float4*>(
+          lds_v + ((i * 2 + b) * 16 + v) * 64 + 4 * q);
+    const float4 y0 = s[0] + s[1] + s[2];
+    const float4 y1 = s[1] - s[2] - s[3];
+    const int m = 8 * (v >> 2) + 4 * (q >> 3) + (v & 3);  // tile in the group
+    const int f = static_cast<int>(fb) * kFeat + 4 * (q & 7);
+    const int tile_off = lds_tile_off[m];
+    const int flags = lds_tile_flags[m];
+    const bool col_ok = tile_off >= 0 && (b == 0 || (flags & 2) != 0);
+    const unsigned off0 =
+        col_ok ? static_cast<unsigned>(tile_off) +
+                     static_cast<unsigned>(b * g.out_ch + f) * 4u
+               : kOob;
+    const unsigned off1 =
+        (col_ok && (flags & 1) != 0) ? off0 + out_row_bytes : kOob;
+    if (ATOMIC) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(
+            comp(y0, e), out_rsrc, off0 + 4u * e, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(
+            comp(y1, e), out_rsrc, off1 + 4u * e, 0, 0);
+      }
+    } else {
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y0),
+                                             out_rsrc, off0, 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y1),
+                                             out_rsrc, off1, 0, 0);
+    }
+  }
+}
+
+// Wave-specialised variant: a work-group of 8 waves in which waves 0-3 only
+// multiply (wave w owns xi = 4w .. 4w+3, B operand straight from L2) and
+// waves 4-7 only gather and transform the input.  V is double buffered in
+// LDS, so the transform of chunk c+1 runs while chunk c is being multiplied
+// and one barrier per chunk is enough.  V rows hold 16 floats without padding;
+// the 16-byte group index is xor-ed with (tile / 2) % 4, which makes both the
+// ds_read_b128 of the multiplying waves and the ds_write_b64 of the
+// transforming waves conflict free.
+constexpr int kVBuf = 16 * kTiles * kChunk;  // floats per V buffer (32 KiB)
+
+template <bool ATOMIC>
+__global__ void __launch_bounds__(512)
+    __attribute__((amdgpu_waves_per_eu(4, 4)))
+    wino_fused_ws_kernel(const float* __restrict__ in,
+                         const float* __restrict__ u, float* __restrict__ out,
+                         FusedGeom g, unsigned in_bytes, unsigned u_bytes,
+                         unsigned out_bytes, unsigned n_fblocks,
+                         unsigned n_units, int chunks_per_split) {
+  __shared__ __align__(16) float lds_v[2 * kVBuf];
+  __shared__ int lds_tile_off[kTiles];
+  __shared__ int lds_tile_flags[kTiles];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const unsigned unit = xcd_remap(blockIdx.x, n_units);
+  const unsigned fb = unit % n_fblocks;
+  const int mb = static_cast<int>(unit / n_fblocks);
+  const int n_chunks = g.in_ch / kChunk;
+  const int chunk_begin = static_cast<int>(blockIdx.y) * chunks_per_split;
+  const int chunk_end = min(n_chunks, chunk_begin + chunks_per_split);
+
+  float16v acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+
+  if (wave >= 4) {
+    // ---- gather + transform waves --------------------------------------
+    const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_bytes);
+    const int ptid = tid - 256;
+    const int tile_l = ptid >> 3, pair = ptid & 7;
+    unsigned p_off[16];
+    {
+      const int tile = mb * kTiles + tile_l;
+      const bool live = tile < g.n_tiles;
+      const int tx = tile % g.tile_cols;
+      const int t2 = tile / g.tile_cols;
+      const int ty = t2 % g.tile_rows;
+      const int n = t2 / g.tile_rows;
+      const int y0 = 2 * ty - g.pad_rows, x0 = 2 * tx - g.pad_cols;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int y = y0 + i, x = x0 + j;
+          const bool ok = live && static_cast<unsigned>(y) <
+                                      static_cast<unsigned>(g.in_rows) &&
+                          static_cast<unsigned>(x) <
+                              static_cast<unsigned>(g.in_cols);
+          p_off[i * 4 + j] =
+              ok ? static_cast<unsigned>(
+                       (((n * g.in_rows + y) * g.in_cols + x) * g.in_ch +
+                        2 * pair) * 4)
+                 : kOob;
+        }
+      if (pair == 0) {
+        lds_tile_off[tile_l] =
+            live ? ((n * g.out_rows + 2 * ty) * g.out_cols + 2 * tx) *
+                       g.out_ch * 4
+                 : -1;
+        lds_tile_flags[tile_l] = (2 * ty + 1 < g.out_rows ? 1 : 0) |
+                                 (2 * tx + 1 < g.out_cols ? 2 : 0);
+      }
+    }
+    float* const v_store =
+        lds_v + tile_l * kChunk +
+        4 * ((pair >> 1) ^ ((tile_l >> 1) & 3)) + 2 * (pair & 1);
+    auto load_patch = [&](int chunk, float2 (&d)[16]) {
+      const unsigned soff =
+          static_cast<unsigned>(min(chunk, chunk_end - 1) * kChunk * 4);
+#pragma unroll
+      for (int q = 0; q < 16; ++q)
+        d[q] = __builtin_bit_cast(
+            float2,
+            __builtin_amdgcn_raw_buffer_load_b64(in_rsrc, p_off[q], soff, 0));
+    };
+    auto transform_store = [&](const float2 (&d)[16], int buf) {
+      float* const dst = v_store + buf * kVBuf;
+      float2 t[4][4];  // Bt d
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        t[0][j] = d[0 * 4 + j] - d[2 * 4 + j];
+        t[1][j] = d[1 * 4 + j] + d[2 * 4 + j];
+        t[2][j] = d[2 * 4 + j] - d[1 * 4 + j];
+        t[3][j] = d[1 * 4 + j] - d[3 * 4 + j];
+      }
+      constexpr int kXi = kTiles * kChunk;  // floats per xi plane
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        *reinterpret_cast<float2*>(dst + (i * 4 + 0) * kXi) = t[i][0] - t[i][2];
+        *reinterpret_cast<float2*>(dst + (i * 4 + 1) * kXi) = t[i][1] + t[i][2];
+        *reinterpret_cast<float2*>(dst + (i * 4 + 2) * kXi) = t[i][2] - t[i][1];
+        *reinterpret_cast<float2*>(dst + (i * 4 + 3) * kXi) = t[i][1] - t[i][3];
+      }
+    };
+    // Two patch register sets: the loads run two chunks ahead of the
+    // transform that consumes them (chunk indices past the end re-read the
+    // last chunk and are never stored).
+    float2 d_even[16], d_odd[16];
+    load_patch(chunk_begin, d_even);
+    load_patch(chunk_begin + 1, d_odd);
+    transform_store(d_even, 0);
+    load_patch(chunk_begin + 2, d_even);
+    __syncthreads();
+    for (int c = chunk_begin; c < chunk_end; c += 2) {
+      // chunk c is being multiplied from buffer 0
+#if !(WF_EXP & 4)
+      if (c + 1 < chunk_end) transform_store(d_odd, 1);
+#endif
+#if !(WF_EXP & 1)
+      load_patch(c + 3, d_odd);
+#endif
+      __syncthreads();
+      if (c + 1 >= chunk_end) break;
+      // chunk c + 1 is being multiplied from buffer 1
+#if !(WF_EXP & 4)
+      if (c + 2 < chunk_end) transform_store(d_even, 0);
+#endif
+#if !(WF_EXP & 1)
+      load_patch(c + 4, d_even);
+#endif
+      __syncthreads();
+    }
+  } else {
+    // ---- multiplying waves ---------------------------------------------
+    const __amdgpu_buffer_rsrc_t u_rsrc = make_rsrc(u, u_bytes);
+    const unsigned u_lane = static_cast<unsigned>(lane) * 16u;
+    const unsigned cgroups = static_cast<unsigned>(g.in_ch) / 8u;
+    unsigned u_base[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      u_base[j] = ((static_cast<unsigned>(4 * wave + j) * n_fblocks + fb) *
+                   cgroups) * 1024u;
+    auto load_b = [&](int cgroup, float4 (&b)[4]) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        b[j] = __builtin_bit_cast(
+            float4, __builtin_amdgcn_raw_buffer_load_b128(
+                        u_rsrc, u_lane,
+                        u_base[j] + static_cast<unsigned>(cgroup) * 1024u, 0));
+    };
+    const int tile_r = lane & 31;
+    const int swz = (tile_r >> 1) & 3;
+    constexpr int kXi = kTiles * kChunk;
+    const float* const a_base = lds_v + (4 * wave * kTiles + tile_r) * kChunk;
+    const int a_grp0 = 4 * ((0 + (lane >> 5)) ^ swz);
+    const int a_grp1 = 4 * ((2 + (lane >> 5)) ^ swz);
+    auto mma_group = [&](const float* a_ptr, const float4 (&b)[4]) {
+      float4 a[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        a[j] = *reinterpret_cast<const float4*>(a_ptr + j * kXi);
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+              comp(a[j], t), comp(b[j], t), acc[j], 0, 0, 0);
+    };
+    float4 b_lo[4], b_hi[4];
+    load_b(2 * chunk_begin, b_lo);
+    load_b(2 * chunk_begin + 1, b_hi);
+    __syncthreads();
+    for (int c = chunk_begin; c < chunk_end; ++c) {
+      const float* const a_buf = a_base + ((c - chunk_begin) & 1) * kVBuf;
+      const int next = min(c + 1, chunk_end - 1);
+#if !(WF_EXP & 8)
+      mma_group(a_buf + a_grp0, b_lo);
+#endif
+#if !(WF_EXP & 2)
+      load_b(2 * next, b_lo);
+#endif
+#if !(WF_EXP & 8)
+      mma_group(a_buf + a_grp1, b_hi);
+#endif
+#if !(WF_EXP & 2)
+      load_b(2 * next + 1, b_hi);
+#endif
+      __syncthreads();
+    }
+    // At m A along xi's column index, inside the lane.
+    float* const s_base = lds_v + (wave * 2 * 16) * 64 + lane;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      s_base[v * 64] = acc[0][v] + acc[1][v] + acc[2][v];
+      s_base[(16 + v) * 64] = acc[1][v] - acc[2][v] - acc[3][v];
+    }
+  }
+  __syncthreads();
+  // Along xi's row index (across the multiplying waves); all 512 lanes write.
+  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_bytes);
+  const unsigned out_row_bytes =
+      static_cast<unsigned>(g.out_cols) * g.out_ch * 4u;
+  {
+    const int b = tid >> 8;
+    const int q = tid & 15;
+    const int v = (tid >> 4) & 15;
+    float4 s[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      s[i] = *reinterpret_cast<const float4*>(
+          lds_v + ((i * 2 + b) * 16 + v) * 64 + 4 * q);
+    const float4 y0 = s[0] + s[1] + s[2];
+    const float4 y1 = s[1] - s[2] - s[3];
+    const int m = 8 * (v >> 2) + 4 * (q >> 3) + (v & 3);
+    const int f = static_cast<int>(fb) * kFeat + 4 * (q & 7);
+    const int tile_off = lds_tile_off[m];
+    const int flags = lds_tile_flags[m];
+    const bool col_ok = tile_off >= 0 && (b == 0 || (flags & 2) != 0);
+    const unsigned off0 =
+        col_ok ? static_cast<unsigned>(tile_off) +
+                     static_cast<unsigned>(b * g.out_ch + f) * 4u
+               : kOob;
+    const unsigned off1 =
+        (col_ok && (flags & 1) != 0) ? off0 + out_row_bytes : kOob;
+    if (ATOMIC) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(
+            comp(y0, e), out_rsrc, off0 + 4u * e, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(
+            comp(y1, e), out_rsrc, off1 + 4u * e, 0, 0);
+      }
+    } else {
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y0),
+                                             out_rsrc, off0, 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y1),
+                                             out_rsrc, off1, 0, 0);
+    }
+  }
+}
+
+inline bool aligned16(const void* p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+}  // namespace
+
+bool conv2d_winograd_fused_supports(int direction,
+                                    const snn_hip_conv2d_params& p) {
+  if (!conv2d_winograd_supports(direction, p)) return false;
+  const bool backprop = direction == SNN_HIP_INPUT_BACKPROP;
+  const int in_ch = backprop ? p.features : p.channels;
+  const int out_ch = backprop ? p.channels : p.features;
+  const size_t x = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                   p.channels;
+  const size_t y = static_cast<size_t>(p.batch) * p.out_rows * p.out_cols *
+                   p.features;
+  const size_t u = static_cast<size_t>(16) * p.channels * p.features;
+  const size_t biggest = x > y ? (x > u ? x : u) : (y > u ? y : u);
+  return in_ch % kChunk == 0 && out_ch % kFeat == 0 &&
+         biggest * sizeof(float) <= kMaxBufferBytes;
+}
+
+int launch_conv2d_winograd_fused_f32(int direction, const float* input,
+                                     const float* filter, float* output,
+                                     const snn_hip_conv2d_params& p,
+                                     float* workspace, size_t workspace_elems,
+                                     hipStream_t stream) {
+  const bool backprop = direction == SNN_HIP_INPUT_BACKPROP;
+  FusedGeom g;
+  g.in_rows = backprop ? p.out_rows : p.in_rows;
+  g.in_cols = backprop ? p.out_cols : p.in_cols;
+  g.in_ch = backprop ? p.features : p.channels;
+  g.out_rows = backprop ? p.in_rows : p.out_rows;
+  g.out_cols = backprop ? p.in_cols : p.out_cols;
+  g.out_ch = backprop ? p.channels : p.features;
+  g.pad_rows = backprop ? 2 - p.pad_rows : p.pad_rows;
+  g.pad_cols = backprop ? 2 - p.pad_cols : p.pad_cols;
+  g.tile_rows = ceil_div(g.out_rows, 2);
+  g.tile_cols = ceil_div(g.out_cols, 2);
+  g.n_tiles = p.batch * g.tile_rows * g.tile_cols;
+  const size_t u_elems = static_cast<size_t>(16) * g.in_ch * g.out_ch;
+  // Only U is stored, but the size contract stays the reference's minimum
+  // (transformed filter plus one image of V and M, winograd/launch.h:237-261).
+  const size_t per_image = static_cast<size_t>(16) * g.tile_rows *
+                           g.tile_cols * (g.in_ch + g.out_ch);
+  if (workspace == nullptr || workspace_elems < u_elems + per_image)
+    return SNN_HIP_INSUFFICIENT_WORKSPACE;
+  if (!aligned16(workspace) || !aligned16(input) || !aligned16(output))
+    return SNN_HIP_INVALID_PARAMETER;
+  const size_t in_elems = static_cast<size_t>(p.batch) * g.in_rows *
+                          g.in_cols * g.in_ch;
+  const size_t out_elems = static_cast<size_t>(p.batch) * g.out_rows *
+                           g.out_cols * g.out_ch;
+
+  hipLaunchKernelGGL(wino_filter_pack_kernel,
+                     dim3(ceil_div((g.in_ch / 4) * g.out_ch, 256)), dim3(256),
+                     0, stream, filter, workspace, p.channels, p.features,
+                     backprop);
+
+  const unsigned n_fblocks = static_cast<unsigned>(g.out_ch / kFeat);
+  const unsigned n_units =
+      static_cast<unsigned>(ceil_div(g.n_tiles, kTiles)) * n_fblocks;
+  const int n_chunks = g.in_ch / kChunk;
+  // Fill the GPU: when there are few (tile block, feature block) units the
+  // channel range is split across work-groups, at least kMinChunks each.
+  constexpr unsigned kTargetGroups = 1536;
+  constexpr int kMinChunks = 4;
+  int splits = 1;
+  if (n_units < kTargetGroups / 2)
+    splits = static_cast<int>(ceil_div(kTargetGroups, n_units));
+  splits = max(1, min(splits, n_chunks / kMinChunks));
+  if (const char* tune = std::getenv("SNN_HIP_WINO")) {
+    if (tune[0] != 0) splits = max(1, min(std::atoi(tune), n_chunks));
+  }
+  const bool ws = std::getenv("SNN_HIP_WINO_V1") == nullptr;
+  const int per_split = ceil_div(n_chunks, splits);
+  splits = ceil_div(n_chunks, per_split);
+
+  const unsigned in_bytes = static_cast<unsigned>(in_elems * 4);
+  const unsigned u_bytes = static_cast<unsigned>(u_elems * 4);
+  const unsigned out_bytes = static_cast<unsigned>(out_elems * 4);
+  if (splits > 1) {
+    const size_t n_vec = out_elems / 4;  // out_ch % 32 == 0
+    hipLaunchKernelGGL(wino_zero_fill_kernel,
+                       dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
+                       dim3(256), 0, stream, reinterpret_cast<float4*>(output),
+                       n_vec);
+    if (ws)
+      hipLaunchKernelGGL(wino_fused_ws_kernel<true>, dim3(n_units, splits),
+                         dim3(512), 0, stream, input, workspace, output, g,
+                         in_bytes, u_bytes, out_bytes, n_fblocks, n_units,
+                         per_split);
+    else
+      hipLaunchKernelGGL(wino_fused_kernel<true>, dim3(n_units, splits),
+                         dim3(256), 0, stream, input, workspace, output, g,
+                         in_bytes, u_bytes, out_bytes, n_fblocks, n_units,
+                         per_split);
+  } else {
+    if (ws)
+      hipLaunchKernelGGL(wino_fused_ws_kernel<false>, dim3(n_units, 1),
+                         dim3(512), 0, stream, input, workspace, output, g,
+                         in_bytes, u_bytes, out_bytes, n_fblocks, n_units,
+                         per_split);
+    else
+      hipLaunchKernelGGL(wino_fused_kernel<false>, dim3(n_units, 1), dim3(256),
+                         0, stream, input, workspace, output, g, in_bytes,
+                         u_bytes, out_bytes, n_fblocks, n_units, per_split);
+  }
+  SNN_HIP_CHECK_LAUNCH();
+  return SNN_HIP_OK;
+}
+
+}  // namespace snn

@@ -1,5 +1,6 @@
 // The C ABI of libsnn_hip.so: parameter validation, algorithm support rules,
 // workspace sizing and dispatch to the kernel launchers.
+#include <cstdlib>
 #include <cstring>
 #include <string>
 
@@ -298,6 +299,13 @@ int launch_winograd_path<float>(int direction, const float* input,
                                 const snn_hip_conv2d_params& p,
                                 float* workspace, size_t workspace_elems,
                                 hipStream_t s) {
+  // SNN_HIP_WINO_UNFUSED is a development switch that forces the three-stage
+  // chain on shapes the fused kernel would take.
+  if (conv2d_winograd_fused_supports(direction, p) && aligned16(input) &&
+      aligned16(output) && aligned16(workspace) &&
+      std::getenv("SNN_HIP_WINO_UNFUSED") == nullptr)
+    return launch_conv2d_winograd_fused_f32(direction, input, filter, output,
+                                            p, workspace, workspace_elems, s);
   if (conv2d_winograd_supports(direction, p))
     return launch_conv2d_winograd_f32(direction, input, filter, output, p,
                                       workspace, workspace_elems, s);

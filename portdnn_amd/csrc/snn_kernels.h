@@ -40,6 +40,17 @@ int launch_conv2d_winograd_f32(int direction, const float* input,
                                float* workspace, size_t workspace_elems,
                                hipStream_t stream);
 
+// The same convolution in one fused kernel (conv2d_winograd_fused.hip): needs
+// channel counts that are multiples of 16 (reduced) and 32 (produced), 16-byte
+// aligned pointers and only the transformed-filter part of the workspace.
+bool conv2d_winograd_fused_supports(int direction,
+                                    const snn_hip_conv2d_params& p);
+int launch_conv2d_winograd_fused_f32(int direction, const float* input,
+                                     const float* filter, float* output,
+                                     const snn_hip_conv2d_params& p,
+                                     float* workspace, size_t workspace_elems,
+                                     hipStream_t stream);
+
 // Half-precision forward convolution on MFMA (conv2d_igemm_f16.hip).  The
 // workspace, when large enough, receives the re-laid-out filter.
 bool conv2d_igemm_f16_supports(const snn_hip_conv2d_params& p);

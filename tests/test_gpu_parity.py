@@ -159,6 +159,22 @@ def test_ragged_shapes(shape, direction):
     conv_case(p, direction, algos, seed=sum(shape[:9]) + direction)
 
 
+@pytest.mark.parametrize("direction", [DIRECTION.FORWARD,
+                                       DIRECTION.INPUT_BACKPROP])
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, same
+    (3, 13, 11, 32, 64, True),    # odd sizes: clipped tiles on both edges
+    (2, 9, 10, 16, 32, False),    # VALID, single chunk
+    (1, 7, 7, 512, 512, True),    # channel range split across work-groups
+    (5, 6, 5, 48, 96, True),      # three chunks, three feature blocks
+    (2, 30, 4, 64, 32, False),    # narrow image
+])
+def test_winograd_fused_shapes(shape, direction):
+    batch, rows, cols, ch, feats, same = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, 3, 1, same)
+    conv_case(p, direction, [ALGO.WINOGRAD], seed=1300 + rows + ch)
+
+
 # ---- full batch-32 shapes: sampled float64 recomputation + linearity --------
 
 def sampled_forward_reference(x, w, p, samples):
