@@ -26,9 +26,6 @@
 // The multiplications done on the matrix cores are 16/36 of the direct
 // algorithm's.
 #include <cstdlib>
-#ifndef WF_EXP
-#define WF_EXP 0
-#endif
 
 #include "gemm_tile.h"
 #include "snn_kernels.h"
@@ -43,9 +40,6 @@ using gemm::xcd_remap;
 constexpr int kTiles = 32;              // Winograd tiles per work-group
 constexpr int kFeat = 32;               // features per work-group
 constexpr int kChunk = 16;              // channels per LDS stage
-constexpr int kRow = kChunk + 4;        // floats per LDS row (bank spread)
-constexpr int kPlane = kTiles * kRow;   // floats per xi plane
-constexpr int kLdsFloats = 16 * kPlane;
 constexpr unsigned kOob = 0x7FFFFFF0u;
 constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
 
@@ -142,235 +136,9 @@ __global__ void __launch_bounds__(256)
   if (i < n_vec) p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
-template <bool ATOMIC>
-__global__ void __launch_bounds__(256)
-    wino_fused_kernel(const float* __restrict__ in, const float* __restrict__ u,
-                      float* __restrict__ out, FusedGeom g, unsigned in_bytes,
-                      unsigned u_bytes, unsigned out_bytes, unsigned n_fblocks,
-                      unsigned n_units, int chunks_per_split) {
-  __shared__ __align__(16) float lds_v[kLdsFloats];
-  __shared__ int lds_tile_off[kTiles];
-  __shared__ int lds_tile_flags[kTiles];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const unsigned unit = xcd_remap(blockIdx.x, n_units);
-  const unsigned fb = unit % n_fblocks;
-  const int mb = static_cast<int>(unit / n_fblocks);
-  const int n_chunks = g.in_ch / kChunk;
-  const int chunk_begin = static_cast<int>(blockIdx.y) * chunks_per_split;
-  const int chunk_end = min(n_chunks, chunk_begin + chunks_per_split);
-
-  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_bytes);
-  const __amdgpu_buffer_rsrc_t u_rsrc = make_rsrc(u, u_bytes);
-
-  // Gather role: this lane owns tile `tile_l` of the work-group and the
-  // channel pair `pair` of every chunk.
-  const int tile_l = tid >> 3, pair = tid & 7;
-  unsigned p_off[16];
-  {
-    const int tile = mb * kTiles + tile_l;
-    const bool live = tile < g.n_tiles;
-    const int tx = tile % g.tile_cols;
-    const int t2 = tile / g.tile_cols;
-    const int ty = t2 % g.tile_rows;
-    const int n = t2 / g.tile_rows;
-    const int y0 = 2 * ty - g.pad_rows, x0 = 2 * tx - g.pad_cols;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int y = y0 + i, x = x0 + j;
-        const bool ok = live && static_cast<unsigned>(y) <
-                                    static_cast<unsigned>(g.in_rows) &&
-                        static_cast<unsigned>(x) <
-                            static_cast<unsigned>(g.in_cols);
-        p_off[i * 4 + j] =
-            ok ? static_cast<unsigned>(
-                     (((n * g.in_rows + y) * g.in_cols + x) * g.in_ch +
-                      2 * pair) * 4)
-               : kOob;
-      }
-    if (pair == 0) {
-      lds_tile_off[tile_l] =
-          live ? ((n * g.out_rows + 2 * ty) * g.out_cols + 2 * tx) *
-                     g.out_ch * 4
-               : -1;
-      lds_tile_flags[tile_l] = (2 * ty + 1 < g.out_rows ? 1 : 0) |
-                               (2 * tx + 1 < g.out_cols ? 2 : 0);
-    }
-  }
-
-  // B operand addresses: wave-uniform plane bases, lane * 16 bytes inside a
-  // 1 KiB (xi, feature block, channel group) record.
-  const unsigned u_lane = static_cast<unsigned>(lane) * 16u;
-  const unsigned cgroups = static_cast<unsigned>(g.in_ch) / 8u;
-  unsigned u_base[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-    u_base[j] = ((static_cast<unsigned>(4 * wave + j) * n_fblocks + fb) *
-                 cgroups) * 1024u;
-
-  auto load_patch = [&](int chunk, float2 (&d)[16]) {
-    const unsigned soff = static_cast<unsigned>(chunk * kChunk * 4);
-#pragma unroll
-    for (int q = 0; q < 16; ++q) {
-      d[q] = __builtin_bit_cast(
-          float2,
-          __builtin_amdgcn_raw_buffer_load_b64(in_rsrc, p_off[q], soff, 0));
-    }
-  };
-  auto load_b = [&](int chunk, float4 (&b)[2][4]) {
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        b[s][j] = __builtin_bit_cast(
-            float4, __builtin_amdgcn_raw_buffer_load_b128(
-                        u_rsrc, u_lane,
-                        u_base[j] + static_cast<unsigned>(2 * chunk + s) * 1024u,
-                        0));
-      }
-  };
-  float* const v_store = lds_v + tile_l * kRow + 2 * pair;
-  auto transform_store = [&](const float2 (&d)[16]) {
-    float2 t[4][4];  // Bt d
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      t[0][j] = d[0 * 4 + j] - d[2 * 4 + j];
-      t[1][j] = d[1 * 4 + j] + d[2 * 4 + j];
-      t[2][j] = d[2 * 4 + j] - d[1 * 4 + j];
-      t[3][j] = d[1 * 4 + j] - d[3 * 4 + j];
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      *reinterpret_cast<float2*>(v_store + (i * 4 + 0) * kPlane) =
-          t[i][0] - t[i][2];
-      *reinterpret_cast<float2*>(v_store + (i * 4 + 1) * kPlane) =
-          t[i][1] + t[i][2];
-      *reinterpret_cast<float2*>(v_store + (i * 4 + 2) * kPlane) =
-          t[i][2] - t[i][1];
-      *reinterpret_cast<float2*>(v_store + (i * 4 + 3) * kPlane) =
-          t[i][1] - t[i][3];
-    }
-  };
-
-  float16v acc[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
-
-  const float* const a_base =
-      lds_v + (4 * wave * kTiles + (lane & 31)) * kRow + 4 * (lane >> 5);
-  auto compute = [&](const float4 (&b)[2][4]) {
-    float4 a[2][4];
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        a[s][j] = *reinterpret_cast<const float4*>(a_base + j * kPlane + 8 * s);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-              comp(a[s][j], t), comp(b[s][j], t), acc[j], 0, 0, 0);
-  };
-
-  // Loads for the next chunk are issued unconditionally (the last iteration
-  // re-reads its own chunk) so that the wait counters the compiler places
-  // before the matrix instructions stay exact instead of being merged over a
-  // branch.
-  float4 b[2][4], b_next[2][4];
-  float2 d[16];
-  load_patch(chunk_begin, d);
-  load_b(chunk_begin, b);
-  transform_store(d);
-  __syncthreads();
-  for (int c = chunk_begin; c < chunk_end; ++c) {
-    const int next = min(c + 1, chunk_end - 1);
-#if !(WF_EXP & 1)
-    load_patch(next, d);
-#endif
-#if !(WF_EXP & 2)
-    load_b(next, b_next);
-#endif
-#if !(WF_EXP & 8)
-    compute(b);
-#endif
-    __syncthreads();  // every wave has read this chunk's V
-#if !(WF_EXP & 4)
-    if (c + 1 < chunk_end) transform_store(d);
-#endif
-    __syncthreads();
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) b[s][j] = b_next[s][j];
-  }
-
-  // At m A.  Along xi's column index (inside the lane): s[b] for b = 0, 1;
-  // S[i = wave][b][v][lane] goes to LDS (32 KiB, the V buffer is free now).
-  {
-    float* const s_base = lds_v + (wave * 2 * 16) * 64 + lane;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      s_base[v * 64] = acc[0][v] + acc[1][v] + acc[2][v];
-      s_base[(16 + v) * 64] = acc[1][v] - acc[2][v] - acc[3][v];
-    }
-  }
-  __syncthreads();
-  // Along xi's row index (across waves), four consecutive features per lane.
-  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_bytes);
-  const unsigned out_row_bytes =
-      static_cast<unsigned>(g.out_cols) * g.out_ch * 4u;
-#pragma unroll
-  for (int b = 0; b < 2; ++b) {
-    const int q = tid & 15;   // lanes 4q .. 4q+3 of the accumulator layout
-    const int v = tid >> 4;   // accumulator register
-    float4 s[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      s[i] = *reinterpret_cast<const float4*>(
-          lds_v + ((i * 2 + b) * 16 + v) * 64 + 4 * q);
-    const float4 y0 = s[0] + s[1] + s[2];
-    const float4 y1 = s[1] - s[2] - s[3];
-    const int m = 8 * (v >> 2) + 4 * (q >> 3) + (v & 3);  // tile in the group
-    const int f = static_cast<int>(fb) * kFeat + 4 * (q & 7);
-    const int tile_off = lds_tile_off[m];
-    const int flags = lds_tile_flags[m];
-    const bool col_ok = tile_off >= 0 && (b == 0 || (flags & 2) != 0);
-    const unsigned off0 =
-        col_ok ? static_cast<unsigned>(tile_off) +
-                     static_cast<unsigned>(b * g.out_ch + f) * 4u
-               : kOob;
-    const unsigned off1 =
-        (col_ok && (flags & 1) != 0) ? off0 + out_row_bytes : kOob;
-    if (ATOMIC) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(
-            comp(y0, e), out_rsrc, off0 + 4u * e, 0, 0);
-        __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(
-            comp(y1, e), out_rsrc, off1 + 4u * e, 0, 0);
-      }
-    } else {
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y0),
-                                             out_rsrc, off0, 0, 0);
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y1),
-                                             out_rsrc, off1, 0, 0);
-    }
-  }
-}
-
-// Wave-specialised variant: a work-group of 8 waves in which waves 0-3 only
-// multiply (wave w owns xi = 4w .. 4w+3, B operand straight from L2) and
-// waves 4-7 only gather and transform the input.  V is double buffered in
+// The main kernel: a work-group of 8 waves per (32 tiles, 32 features) unit in
+// which waves 0-3 only multiply (wave w owns xi = 4w .. 4w+3, B operand
+// straight from L2) and waves 4-7 only gather and transform the input.  V is double buffered in
 // LDS, so the transform of chunk c+1 runs while chunk c is being multiplied
 // and one barrier per chunk is enough.  V rows hold 16 floats without padding;
 // the 16-byte group index is xor-ed with (tile / 2) % 4, which makes both the
@@ -381,7 +149,7 @@ constexpr int kVBuf = 16 * kTiles * kChunk;  // floats per V buffer (32 KiB)
 template <bool ATOMIC>
 __global__ void __launch_bounds__(512)
     __attribute__((amdgpu_waves_per_eu(4, 4)))
-    wino_fused_ws_kernel(const float* __restrict__ in,
+    wino_fused_kernel(const float* __restrict__ in,
                          const float* __restrict__ u, float* __restrict__ out,
                          FusedGeom g, unsigned in_bytes, unsigned u_bytes,
                          unsigned out_bytes, unsigned n_fblocks,
@@ -486,21 +254,13 @@ __global__ void __launch_bounds__(512)
     __syncthreads();
     for (int c = chunk_begin; c < chunk_end; c += 2) {
       // chunk c is being multiplied from buffer 0
-#if !(WF_EXP & 4)
       if (c + 1 < chunk_end) transform_store(d_odd, 1);
-#endif
-#if !(WF_EXP & 1)
       load_patch(c + 3, d_odd);
-#endif
       __syncthreads();
       if (c + 1 >= chunk_end) break;
       // chunk c + 1 is being multiplied from buffer 1
-#if !(WF_EXP & 4)
       if (c + 2 < chunk_end) transform_store(d_even, 0);
-#endif
-#if !(WF_EXP & 1)
       load_patch(c + 4, d_even);
-#endif
       __syncthreads();
     }
   } else {
@@ -546,18 +306,10 @@ __global__ void __launch_bounds__(512)
     for (int c = chunk_begin; c < chunk_end; ++c) {
       const float* const a_buf = a_base + ((c - chunk_begin) & 1) * kVBuf;
       const int next = min(c + 1, chunk_end - 1);
-#if !(WF_EXP & 8)
       mma_group(a_buf + a_grp0, b_lo);
-#endif
-#if !(WF_EXP & 2)
       load_b(2 * next, b_lo);
-#endif
-#if !(WF_EXP & 8)
       mma_group(a_buf + a_grp1, b_hi);
-#endif
-#if !(WF_EXP & 2)
       load_b(2 * next + 1, b_hi);
-#endif
       __syncthreads();
     }
     // At m A along xi's column index, inside the lane.
@@ -675,18 +427,20 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
   const unsigned n_units =
       static_cast<unsigned>(ceil_div(g.n_tiles, kTiles)) * n_fblocks;
   const int n_chunks = g.in_ch / kChunk;
-  // Fill the GPU: when there are few (tile block, feature block) units the
-  // channel range is split across work-groups, at least kMinChunks each.
-  constexpr unsigned kTargetGroups = 1536;
+  // Splitting the channel range across work-groups costs a zero fill and
+  // float atomics on every output (measured: slower than leaving CUs idle as
+  // soon as there are a few hundred units), so it is kept for launches that
+  // would otherwise occupy only a fraction of the GPU.
+  constexpr unsigned kFewUnits = 128;
+  constexpr unsigned kTargetGroups = 512;
   constexpr int kMinChunks = 4;
   int splits = 1;
-  if (n_units < kTargetGroups / 2)
+  if (n_units < kFewUnits)
     splits = static_cast<int>(ceil_div(kTargetGroups, n_units));
   splits = max(1, min(splits, n_chunks / kMinChunks));
   if (const char* tune = std::getenv("SNN_HIP_WINO")) {
     if (tune[0] != 0) splits = max(1, min(std::atoi(tune), n_chunks));
   }
-  const bool ws = std::getenv("SNN_HIP_WINO_V1") == nullptr;
   const int per_split = ceil_div(n_chunks, splits);
   splits = ceil_div(n_chunks, per_split);
 
@@ -699,26 +453,14 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
                        dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
                        dim3(256), 0, stream, reinterpret_cast<float4*>(output),
                        n_vec);
-    if (ws)
-      hipLaunchKernelGGL(wino_fused_ws_kernel<true>, dim3(n_units, splits),
-                         dim3(512), 0, stream, input, workspace, output, g,
-                         in_bytes, u_bytes, out_bytes, n_fblocks, n_units,
-                         per_split);
-    else
-      hipLaunchKernelGGL(wino_fused_kernel<true>, dim3(n_units, splits),
-                         dim3(256), 0, stream, input, workspace, output, g,
-                         in_bytes, u_bytes, out_bytes, n_fblocks, n_units,
-                         per_split);
+    hipLaunchKernelGGL(wino_fused_kernel<true>, dim3(n_units, splits),
+                       dim3(512), 0, stream, input, workspace, output, g,
+                       in_bytes, u_bytes, out_bytes, n_fblocks, n_units,
+                       per_split);
   } else {
-    if (ws)
-      hipLaunchKernelGGL(wino_fused_ws_kernel<false>, dim3(n_units, 1),
-                         dim3(512), 0, stream, input, workspace, output, g,
-                         in_bytes, u_bytes, out_bytes, n_fblocks, n_units,
-                         per_split);
-    else
-      hipLaunchKernelGGL(wino_fused_kernel<false>, dim3(n_units, 1), dim3(256),
-                         0, stream, input, workspace, output, g, in_bytes,
-                         u_bytes, out_bytes, n_fblocks, n_units, per_split);
+    hipLaunchKernelGGL(wino_fused_kernel<false>, dim3(n_units, 1), dim3(512),
+                       0, stream, input, workspace, output, g, in_bytes,
+                       u_bytes, out_bytes, n_fblocks, n_units, per_split);
   }
   SNN_HIP_CHECK_LAUNCH();
   return SNN_HIP_OK;
