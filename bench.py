@@ -10,8 +10,9 @@ the library's default selector picks, inputs resident in HBM.  `value` is
 total algorithmic TFLOP/s (2*N*OH*OW*R*S*C*K per layer, whatever the
 algorithm).  The same JSON line carries
 
-  roofline      the 3x3 convolution kernel against the fp32 MFMA peak, timed
-                with HIP events on the launch stream,
+  roofline      the main kernel of the 3x3 convolutions against the fp32 MFMA
+                peak: algorithmic flops per launch over its average duration,
+                timed with HIP events on the launch stream,
   cpu_baseline  the reference's tiled algorithm restated in C (oracle/), timed
                 on the host cores on a bounded sample of the same layers,
   detail        per-layer / per-algorithm TFLOP/s and the depthwise / pooling
@@ -28,6 +29,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the fused Winograd kernel, mean over the four 3x3
+# layers, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (FETCH_SIZE scaled
+# by the factor a plain copy kernel of known size shows, 2.0; WRITE_SIZE 1.0).
+WINOGRAD_TRAFFIC_BYTES = None
 
 RESNET = [(56, 64), (28, 128), (14, 256), (7, 512)]
 MOBILENET = [(112, 32, 1), (112, 64, 2), (56, 128, 1), (28, 256, 2),
@@ -124,27 +129,46 @@ def main():
     ms_per_step = elapsed * 1e3 / args.steps
     value = total_flops / (elapsed / args.steps) / 1e12
 
-    # ---- roofline: the 3x3 kernel, HIP events on the launch stream -----------
+    # ---- roofline: the dominant kernel, HIP events on the launch stream -------
+    # The library brackets the main kernel of each convolution launch (not the
+    # filter preparation in front of it) with events on the stream it launches
+    # on; these per-kernel times are what `rocprofv3 --kernel-trace --stats`
+    # reports for the same kernel.
     algo_names = {1: "direct", 2: "tiled", 3: "im2col", 4: "winograd",
                   6: "matmul"}
     per_layer = []
-    k3_flops = k3_ms = 0.0
+    k3_flops = k3_kernel_ms = 0.0
+    k3_kernels = 0
     for w in work:
-        ms = event_time_ms(lambda w=w: ops.conv2d(
-            w["x"], w["w"], w["p"], DIRECTION.FORWARD, w["algo"],
-            workspace=w["ws"], out=w["y"]), reps=20)
+        def call(w=w):
+            ops.conv2d(w["x"], w["w"], w["p"], DIRECTION.FORWARD, w["algo"],
+                       workspace=w["ws"], out=w["y"])
+        ms = event_time_ms(call, reps=20)
+        with ops.kernel_timing() as kt:
+            for _ in range(20):
+                call()
+        kernel_ms = kt.total_ms / max(1, kt.kernels)
         tf = w["flops"] / ms / 1e9
         per_layer.append({"layer": w["name"], "algorithm": algo_names[w["algo"]],
-                          "ms": round(ms, 4), "tflops": round(tf, 2),
+                          "ms": round(ms, 4), "kernel_ms": round(kernel_ms, 4),
+                          "tflops": round(tf, 2),
                           "frac_mfma_peak": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)})
         if w["name"].startswith("3x3"):
-            k3_flops += w["flops"]
-            k3_ms += ms
-    achieved = k3_flops / k3_ms / 1e9
-    roofline = {"bound": "mfma", "kernel": "conv2d 3x3 s1 forward, 4 ResNet stages",
-                "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                "traffic": None}
+            k3_flops += w["flops"] * kt.kernels
+            k3_kernel_ms += kt.total_ms
+            k3_kernels += kt.kernels
+    achieved = k3_flops / k3_kernel_ms / 1e9
+    k3_algos = sorted({algo_names[w["algo"]] for w in work
+                       if w["name"].startswith("3x3")})
+    roofline = {
+        "bound": "mfma",
+        "kernel": "main kernel of the 3x3 s1 forward convolution (%s), the four "
+                  "ResNet stages, one launch each per step" % "/".join(k3_algos),
+        "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
+        "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+        "avg_kernel_ms": round(k3_kernel_ms / k3_kernels, 5),
+        "algorithmic_gflop_per_launch": round(k3_flops / k3_kernels / 1e9, 4),
+        "traffic": WINOGRAD_TRAFFIC_BYTES if k3_algos == ["winograd"] else None}
 
     detail = {"layers": per_layer}
     if not args.no_detail:
@@ -230,23 +254,34 @@ def main():
         rng = np.random.default_rng(0x5EED)
         cpu_flops = 0.0
         cpu_s = 0.0
+        cpu_batch = 8
+        cases = []
         for size, ch in RESNET:
             for window, feats in ((3, ch), (1, 4 * ch)):
-                p = oracle.make_params(1, size, size, ch, feats, window, 1,
-                                       window == 3)
-                x = rng.uniform(-1, 1, size * size * ch).astype(np.float32)
+                p = oracle.make_params(cpu_batch, size, size, ch, feats, window,
+                                       1, window == 3)
+                x = rng.uniform(-1, 1, cpu_batch * size * size * ch).astype(
+                    np.float32)
                 w = rng.uniform(-1, 1, window * window * ch * feats).astype(
                     np.float32)
-                oracle.conv2d_tiled_forward(x, w, p)  # warm-up, as the
-                t = time.perf_counter()               # reference's executor
+                cases.append((p, x, w, 2.0 * cpu_batch * size * size * window *
+                              window * ch * feats))
+        for p, x, w, _ in cases:               # warm-up pass, as the
+            oracle.conv2d_tiled_forward(x, w, p)   # reference's executor does
+        passes = 0
+        while cpu_s < 10.0 and passes < 40:
+            for p, x, w, fl in cases:
+                t = time.perf_counter()
                 oracle.conv2d_tiled_forward(x, w, p)
                 cpu_s += time.perf_counter() - t
-                cpu_flops += 2.0 * size * size * window * window * ch * feats
+                cpu_flops += fl
+            passes += 1
         cpu = {"value": round(cpu_flops / cpu_s / 1e12, 5), "unit": "TFLOP/s",
                "cores": cores, "kind": "port",
-               "sample": "batch 1 of each of the 8 layers, portDNN tiled "
-                         "algorithm (2x2x4 register tiles) restated in C with "
-                         "OpenMP; %.2f s of CPU time" % cpu_s}
+               "sample": "%d passes over batch %d of each of the 8 layers, "
+                         "portDNN tiled algorithm (2x2x4 register tiles) "
+                         "restated in C with OpenMP; %.1f s of CPU time"
+                         % (passes, cpu_batch, cpu_s)}
 
     line = {
         "metric": "conv2d fwd TFLOP/s + %MFMA peak; depthwise/pool GB/s + "

@@ -146,6 +146,17 @@ SNN_HIP_API const char* snn_hip_status_string(int status);
 /* Text of the last HIP runtime error seen by the calling thread ("" if none). */
 SNN_HIP_API const char* snn_hip_last_error(void);
 
+/* Kernel timing for benchmarks (no counterpart in the reference, whose
+ * launches return a cl::sycl::event that carries profiling information).
+ * While enabled, every convolution launch brackets its dominant kernel -- the
+ * implicit-GEMM or fused Winograd kernel, not the filter preparation or zero
+ * fill around it -- with HIP events recorded on the launch stream.
+ * snn_hip_kernel_timing_read waits for the recorded events, returns the summed
+ * kernel time in milliseconds and the number of kernels, and clears the
+ * record.  Not thread safe; meant for a single benchmarking thread. */
+SNN_HIP_API int snn_hip_kernel_timing_enable(int enable);
+SNN_HIP_API int snn_hip_kernel_timing_read(double* total_ms, int* kernels);
+
 /* ---- dense convolution ---------------------------------------------------
  * Stand-ins for sycldnn::conv2d::internal::launch_{direct,tiled,matmul,
  * im2col,winograd} reached from sycldnn::conv2d::launch<T, ConvType>

@@ -93,6 +93,9 @@ SIGNATURES = {
     "snn_hip_version": [],
     "snn_hip_status_string": [_I],
     "snn_hip_last_error": [],
+    "snn_hip_kernel_timing_enable": [_I],
+    "snn_hip_kernel_timing_read": [ctypes.POINTER(ctypes.c_double),
+                                   ctypes.POINTER(ctypes.c_int)],
     "snn_hip_conv2d_forward_f32": [_P, _P, _P, _P, _I, _P, _SZ, _P],
     "snn_hip_conv2d_input_backprop_f32": [_P, _P, _P, _P, _I, _P, _SZ, _P],
     "snn_hip_conv2d_filter_backprop_f32": [_P, _P, _P, _P, _I, _P, _SZ, _P],

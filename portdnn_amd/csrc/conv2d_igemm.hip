@@ -739,6 +739,7 @@ void launch_tile(const float* src, const float* wgt, float* dst,
                        dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
                        dim3(256), 0, stream, reinterpret_cast<float4*>(dst),
                        n_vec);
+    KernelTimer timer(stream);
     if (fast) {
       auto kernel = conv_igemm_fast_kernel<BM, BN, WM, WN, B_K_INNER, true>;
       static const hipError_t attr = hipFuncSetAttribute(
@@ -760,6 +761,7 @@ void launch_tile(const float* src, const float* wgt, float* dst,
                        kLdsBytes, stream, src, wgt, dst, g, src_bytes,
                        wgt_bytes, tiles_n, n_tiles, per_split);
   } else {
+    KernelTimer timer(stream);
     if (fast) {
       auto kernel = conv_igemm_fast_kernel<BM, BN, WM, WN, B_K_INNER, false>;
       static const hipError_t attr = hipFuncSetAttribute(
@@ -867,6 +869,7 @@ static int launch_filter_backprop(const float* x, const float* dy, float* dw,
   hipLaunchKernelGGL(zero_fill_kernel,
                      dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
                      dim3(256), 0, stream, reinterpret_cast<float4*>(dw), n_vec);
+  KernelTimer timer(stream);
   hipLaunchKernelGGL(conv_filter_backprop_kernel, dim3(tiles, splits),
                      dim3(kThreads), 0, stream, x, dy, dw, g,
                      static_cast<unsigned>(x_elems * 4),

@@ -269,6 +269,7 @@ void launch_f16_tile(const _Float16* src, const _Float16* wgt_t, _Float16* dst,
       reinterpret_cast<const void*>(kernel),
       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
   (void)attr;
+  KernelTimer timer(stream);
   hipLaunchKernelGGL(
       kernel, dim3(n_tiles), dim3(kThreads), kLdsBytes, stream, src, wgt_t, dst,
       g, static_cast<unsigned>(src_elems * 2),

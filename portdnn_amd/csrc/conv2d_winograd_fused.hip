@@ -453,11 +453,13 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
                        dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
                        dim3(256), 0, stream, reinterpret_cast<float4*>(output),
                        n_vec);
+    KernelTimer timer(stream);
     hipLaunchKernelGGL(wino_fused_kernel<true>, dim3(n_units, splits),
                        dim3(512), 0, stream, input, workspace, output, g,
                        in_bytes, u_bytes, out_bytes, n_fblocks, n_units,
                        per_split);
   } else {
+    KernelTimer timer(stream);
     hipLaunchKernelGGL(wino_fused_kernel<false>, dim3(n_units, 1), dim3(512),
                        0, stream, input, workspace, output, g, in_bytes,
                        u_bytes, out_bytes, n_fblocks, n_units, per_split);

@@ -37,6 +37,21 @@ int report_hip_error(hipError_t err, const char* what);
 
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 
+// Brackets the kernels launched during its lifetime with HIP events on
+// `stream` when kernel timing is enabled (snn_hip_kernel_timing_enable);
+// otherwise does nothing.
+class KernelTimer {
+ public:
+  explicit KernelTimer(hipStream_t stream);
+  ~KernelTimer();
+  KernelTimer(const KernelTimer&) = delete;
+  KernelTimer& operator=(const KernelTimer&) = delete;
+
+ private:
+  hipStream_t stream_;
+  hipEvent_t stop_;
+};
+
 constexpr int kWave = 64;
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }

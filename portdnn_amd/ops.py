@@ -205,3 +205,26 @@ __all__ = [
     "pool_params", "pooling_avg_grad", "pooling_forward", "pooling_max_grad",
     "workspace_size",
 ]
+
+
+class kernel_timing:
+    """Context manager around snn_hip_kernel_timing_*: times the dominant
+    kernel of every convolution launched inside it with HIP events on the
+    launch stream.  After exit `.total_ms` and `.kernels` hold the result."""
+
+    def __enter__(self):
+        capi.check(capi.lib().snn_hip_kernel_timing_enable(1))
+        self.total_ms = 0.0
+        self.kernels = 0
+        return self
+
+    def __exit__(self, *exc):
+        lib = capi.lib()
+        capi.check(lib.snn_hip_kernel_timing_enable(0))
+        ms = ctypes.c_double(0.0)
+        n = ctypes.c_int(0)
+        capi.check(lib.snn_hip_kernel_timing_read(ctypes.byref(ms),
+                                                  ctypes.byref(n)))
+        self.total_ms = ms.value
+        self.kernels = n.value
+        return False
