@@ -35,7 +35,6 @@ namespace {
 
 using gemm::comp;
 using gemm::float16v;
-using gemm::xcd_remap;
 
 constexpr int kTiles = 32;              // Winograd tiles per work-group
 constexpr int kFeat = 32;               // features per work-group
@@ -44,6 +43,13 @@ constexpr unsigned kOob = 0x7FFFFFF0u;
 constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
 
 typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+
+// The (tile block, feature block) units of a launch and how they are dealt
+// to the 8 XCDs: xcd_m x xcd_f = 8.
+struct UnitGrid {
+  int n_mblocks, n_fblocks;
+  int xcd_m, xcd_f;
+};
 
 struct FusedGeom {
   int in_rows, in_cols, in_ch;
@@ -152,8 +158,8 @@ __global__ void __launch_bounds__(512)
     wino_fused_kernel(const float* __restrict__ in,
                          const float* __restrict__ u, float* __restrict__ out,
                          FusedGeom g, unsigned in_bytes, unsigned u_bytes,
-                         unsigned out_bytes, unsigned n_fblocks,
-                         unsigned n_units, int chunks_per_split) {
+                         unsigned out_bytes, UnitGrid ug,
+                         int chunks_per_split) {
   __shared__ __align__(16) float lds_v[2 * kVBuf];
   __shared__ int lds_tile_off[kTiles];
   __shared__ int lds_tile_flags[kTiles];
@@ -161,9 +167,21 @@ __global__ void __launch_bounds__(512)
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const unsigned unit = xcd_remap(blockIdx.x, n_units);
-  const unsigned fb = unit % n_fblocks;
-  const int mb = static_cast<int>(unit / n_fblocks);
+  // Work-group b runs on XCD b % 8 (round-robin dispatch); XCD (a, c) of the
+  // xcd_m x xcd_f arrangement owns one range of tile blocks and one range of
+  // feature blocks, so its L2 holds only that slice of the input and of U.
+  const int xcd = static_cast<int>(blockIdx.x & 7u);
+  const int local = static_cast<int>(blockIdx.x >> 3);
+  const int xa = xcd / ug.xcd_f, xc = xcd % ug.xcd_f;
+  const int m_lo = xa * ug.n_mblocks / ug.xcd_m;
+  const int m_hi = (xa + 1) * ug.n_mblocks / ug.xcd_m;
+  const int f_lo = xc * ug.n_fblocks / ug.xcd_f;
+  const int f_hi = (xc + 1) * ug.n_fblocks / ug.xcd_f;
+  const int f_cnt = f_hi - f_lo;
+  if (local >= (m_hi - m_lo) * f_cnt) return;  // whole group, before any barrier
+  const unsigned n_fblocks = static_cast<unsigned>(ug.n_fblocks);
+  const unsigned fb = static_cast<unsigned>(f_lo + local % f_cnt);
+  const int mb = m_lo + local / f_cnt;
   const int n_chunks = g.in_ch / kChunk;
   const int chunk_begin = static_cast<int>(blockIdx.y) * chunks_per_split;
   const int chunk_end = min(n_chunks, chunk_begin + chunks_per_split);
@@ -423,9 +441,40 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
                      0, stream, filter, workspace, p.channels, p.features,
                      backprop);
 
-  const unsigned n_fblocks = static_cast<unsigned>(g.out_ch / kFeat);
-  const unsigned n_units =
-      static_cast<unsigned>(ceil_div(g.n_tiles, kTiles)) * n_fblocks;
+  UnitGrid ug;
+  ug.n_mblocks = ceil_div(g.n_tiles, kTiles);
+  ug.n_fblocks = g.out_ch / kFeat;
+  const unsigned n_units = static_cast<unsigned>(ug.n_mblocks) * ug.n_fblocks;
+  // Each XCD has its own L2: with the XCDs arranged xcd_m x xcd_f over (tile
+  // blocks, feature blocks), U is fetched from memory xcd_m times and the
+  // input xcd_f times.  Take the arrangement with the least traffic that
+  // still gives every XCD work.
+  ug.xcd_m = 8;
+  ug.xcd_f = 1;
+  {
+    double best = -1.0;
+    for (int xf = 1; xf <= 8; xf *= 2) {
+      const int xm = 8 / xf;
+      if (xf > ug.n_fblocks || (xm > ug.n_mblocks && xm > 1)) continue;
+      const double traffic = static_cast<double>(u_elems) * xm +
+                             static_cast<double>(in_elems) * xf;
+      if (best < 0.0 || traffic < best) {
+        best = traffic;
+        ug.xcd_m = xm;
+        ug.xcd_f = xf;
+      }
+    }
+  }
+  if (const char* tune = std::getenv("SNN_HIP_WINO_XCDF")) {
+    const int xf = std::atoi(tune);
+    if (xf == 1 || xf == 2 || xf == 4 || xf == 8) {
+      ug.xcd_f = xf;
+      ug.xcd_m = 8 / xf;
+    }
+  }
+  const unsigned grid_x =
+      8u * static_cast<unsigned>(ceil_div(ug.n_mblocks, ug.xcd_m)) *
+      static_cast<unsigned>(ceil_div(ug.n_fblocks, ug.xcd_f));
   const int n_chunks = g.in_ch / kChunk;
   // Splitting the channel range across work-groups costs a zero fill and
   // float atomics on every output (measured: slower than leaving CUs idle as
@@ -454,15 +503,14 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
                        dim3(256), 0, stream, reinterpret_cast<float4*>(output),
                        n_vec);
     KernelTimer timer(stream);
-    hipLaunchKernelGGL(wino_fused_kernel<true>, dim3(n_units, splits),
+    hipLaunchKernelGGL(wino_fused_kernel<true>, dim3(grid_x, splits),
                        dim3(512), 0, stream, input, workspace, output, g,
-                       in_bytes, u_bytes, out_bytes, n_fblocks, n_units,
-                       per_split);
+                       in_bytes, u_bytes, out_bytes, ug, per_split);
   } else {
     KernelTimer timer(stream);
-    hipLaunchKernelGGL(wino_fused_kernel<false>, dim3(n_units, 1), dim3(512),
+    hipLaunchKernelGGL(wino_fused_kernel<false>, dim3(grid_x, 1), dim3(512),
                        0, stream, input, workspace, output, g, in_bytes,
-                       u_bytes, out_bytes, n_fblocks, n_units, per_split);
+                       u_bytes, out_bytes, ug, per_split);
   }
   SNN_HIP_CHECK_LAUNCH();
   return SNN_HIP_OK;
