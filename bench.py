@@ -32,7 +32,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the fused Winograd kernel, mean over the four 3x3
 # layers, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (FETCH_SIZE scaled
 # by the factor a plain copy kernel of known size shows, 2.0; WRITE_SIZE 1.0).
-WINOGRAD_TRAFFIC_BYTES = None
+WINOGRAD_TRAFFIC_BYTES = 42.5e6
 
 RESNET = [(56, 64), (28, 128), (14, 256), (7, 512)]
 MOBILENET = [(112, 32, 1), (112, 64, 2), (56, 128, 1), (28, 256, 2),
