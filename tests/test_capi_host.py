@@ -171,6 +171,35 @@ def test_default_algorithm_is_launchable():
                     ctypes.byref(p), d, a) == a
 
 
+def test_default_algorithm_policy_on_benchmark_layers():
+    """1x1 stride-1 layers are one GEMM; 3x3 stride-1 layers whose channel
+    counts fit the fused Winograd kernel take it for forward and input
+    backprop; everything else is the implicit GEMM (Tiled / Im2col tags)."""
+    L = capi.lib()
+
+    def default(p, d):
+        return L.snn_hip_conv2d_default_algorithm(ctypes.byref(p), d)
+
+    for size, ch in [(56, 64), (28, 128), (14, 256), (7, 512)]:
+        p3 = ops.conv_params(32, size, size, ch, ch, 3, 1, True)
+        assert default(p3, DIRECTION.FORWARD) == ALGO.WINOGRAD
+        assert default(p3, DIRECTION.INPUT_BACKPROP) == ALGO.WINOGRAD
+        assert default(p3, DIRECTION.FILTER_BACKPROP) in (ALGO.TILED,
+                                                          ALGO.IM2COL)
+        p1 = ops.conv_params(32, size, size, ch, 4 * ch, 1, 1, False)
+        assert default(p1, DIRECTION.FORWARD) == ALGO.MATMUL
+    stem = ops.conv_params(32, 224, 224, 3, 64, 7, 2, True)
+    assert default(stem, DIRECTION.FORWARD) in (ALGO.TILED, ALGO.IM2COL)
+    odd = ops.conv_params(32, 28, 28, 24, 40, 3, 1, True)
+    assert default(odd, DIRECTION.FORWARD) in (ALGO.TILED, ALGO.IM2COL)
+
+
+def test_kernel_timing_argument_checks():
+    L = capi.lib()
+    assert L.snn_hip_kernel_timing_read(None, None) == STATUS.INVALID_PARAMETER
+    assert L.snn_hip_kernel_timing_enable(0) == STATUS.OK
+
+
 def test_workspace_sizes_reference_bounds():
     """Lower bounds of test/conv2d/workspace_size.cc:52-160 (VGG layer 1:
     3x3 s1 SAME, 224x224, 64 -> 64, batch 32)."""

@@ -512,3 +512,22 @@ def test_f16_pooling_forward():
     ref = oracle.pool_avg_forward(x.astype(np.float32), oracle_params(q, 0))
     got = ops.pooling_forward(dev(x, torch.float16), q, POOL_OP.AVERAGE)
     assert_close_f16(got.float().cpu().numpy(), ref, "f16 avg")
+
+
+def test_kernel_timing_brackets_the_main_kernel():
+    p = ops.conv_params(8, 28, 28, 128, 128, 3, 1, True)
+    rng = np.random.default_rng(1500)
+    n_in, n_fil, _ = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x, w = dev(uniform(rng, n_in)), dev(uniform(rng, n_fil))
+    for algo in (ALGO.WINOGRAD, ALGO.IM2COL):
+        ops.conv2d(x, w, p, DIRECTION.FORWARD, algo)
+        with ops.kernel_timing() as kt:
+            for _ in range(3):
+                ops.conv2d(x, w, p, DIRECTION.FORWARD, algo)
+        assert kt.kernels == 3
+        assert 0.001 < kt.total_ms / 3 < 5.0
+    # disabled again: nothing is recorded
+    ops.conv2d(x, w, p, DIRECTION.FORWARD, ALGO.IM2COL)
+    with ops.kernel_timing() as kt:
+        pass
+    assert kt.kernels == 0
