@@ -131,6 +131,13 @@ def lib():
             raise SnnHipError(
                 "libsnn_hip.so is missing: build it with "
                 "`python -m portdnn_amd.build` (there is no CPU fallback)")
+        # torch bundles its own libamdhip64; load it first so that this
+        # library binds to the same HIP runtime the tensors live in (two
+        # runtimes in one process do not see each other's devices).
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = ctypes.CDLL(_LIB_PATH)
         for name, argtypes in SIGNATURES.items():
             fn = getattr(L, name)
