@@ -67,8 +67,11 @@ __device__ inline float4 buffer_load4(__amdgpu_buffer_rsrc_t r, unsigned off) {
   return __builtin_bit_cast(float4, v);
 }
 
+// SCALAR_A: the gathered tensor's channel count is not a multiple of 4 (e.g.
+// the 3-channel stem), so four consecutive reduction indices are not four
+// consecutive floats of one tap; each is located and loaded on its own.
 template <int BM, int BN, int WM, int WN, bool B_K_INNER, bool STRIDED,
-          bool ATOMIC>
+          bool ATOMIC, bool SCALAR_A = false>
 __global__ void __launch_bounds__(kThreads)
     conv_igemm_kernel(const float* __restrict__ src,
                       const float* __restrict__ wgt, float* __restrict__ dst,
@@ -79,6 +82,7 @@ __global__ void __launch_bounds__(kThreads)
   constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
   constexpr int TM = WTM / 32, TN = WTN / 32;  // MFMA blocks per wave
   static_assert(TM >= 1 && TN >= 1, "wave tile must hold a 32x32 block");
+  static_assert(!(SCALAR_A && STRIDED), "scalar gather is forward-style only");
   constexpr int A_FLOATS = k_inner_floats(BM);
   constexpr int B_FLOATS =
       B_K_INNER ? k_inner_floats(BN) : row_inner_floats(BN);
@@ -149,7 +153,49 @@ __global__ void __launch_bounds__(kThreads)
   float4 a_reg[A_ROWS_PER_THREAD];
   float4 b_reg[B_PASSES];
 
+  int a_q = q_begin + 4 * a_cc;  // SCALAR_A: first reduction index of the lane
+  auto load_a_scalar = [&]() {
+    // (tap row, tap col, channel) of the four indices, by carry from the first
+    int r = a_r, sc = a_s, c = a_c;
+    int tap_off[4], tr[4], ts[4];
+    bool q_ok[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      q_ok[e] = a_q + e < g.k_total;
+      tr[e] = r;
+      ts[e] = sc;
+      tap_off[e] = (r * g.src_cols + sc) * g.src_ch + c;
+      if (++c == g.src_ch) {
+        c = 0;
+        if (++sc == g.win_cols) { sc = 0; ++r; }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < A_ROWS_PER_THREAD; ++i) {
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int iy = a_iy0[i] + tr[e];
+        const int ix = a_ix0[i] + ts[e];
+        const bool ok =
+            q_ok[e] &
+            (static_cast<unsigned>(iy) < static_cast<unsigned>(g.src_rows)) &
+            (static_cast<unsigned>(ix) < static_cast<unsigned>(g.src_cols));
+        v[e] = __builtin_bit_cast(
+            float, __builtin_amdgcn_raw_buffer_load_b32(
+                       src_rsrc,
+                       ok ? static_cast<unsigned>(a_off[i] + tap_off[e]) * 4u
+                          : kOob,
+                       0, 0));
+      }
+      a_reg[i] = make_float4(v[0], v[1], v[2], v[3]);
+    }
+  };
   auto load_a = [&]() {
+    if (SCALAR_A) {
+      load_a_scalar();
+      return;
+    }
     const bool tap_ok = a_r < g.win_rows;
     // offset of this lane's tap relative to (iy0, ix0)
     const int tap_off =
@@ -178,6 +224,14 @@ __global__ void __launch_bounds__(kThreads)
     }
   };
   auto advance_a = [&]() {
+    if (SCALAR_A) {
+      a_q += kBK;
+      const int tap = a_q / g.src_ch;
+      a_c = a_q - tap * g.src_ch;
+      a_r = tap / g.win_cols;
+      a_s = tap - a_r * g.win_cols;
+      return;
+    }
     a_c += kBK;
     while (a_c >= g.src_ch) {
       a_c -= g.src_ch;
@@ -841,6 +895,33 @@ void launch_auto(const float* src, const float* wgt, float* dst,
                                                 wgt_elems, splits, stream);
 }
 
+// Forward convolution whose channel count is not a multiple of 4: 64x64
+// tiles, scalar gather, no reduction split (such layers have few channels
+// and many pixels).
+void launch_scalar_gather_forward(const float* src, const float* wgt,
+                                  float* dst, const Gather& g,
+                                  size_t src_elems, size_t wgt_elems,
+                                  hipStream_t stream) {
+  constexpr int BM = 64, BN = 64;
+  const unsigned tiles_m = static_cast<unsigned>(ceil_div(g.m_total, BM));
+  const unsigned tiles_n = static_cast<unsigned>(ceil_div(g.n_total, BN));
+  const unsigned n_tiles = tiles_m * tiles_n;
+  const int n_chunks = ceil_div(g.k_total, kBK);
+  constexpr size_t kLdsBytes =
+      2 * sizeof(float) * (k_inner_floats(BM) + row_inner_floats(BN));
+  auto kernel = conv_igemm_kernel<BM, BN, 2, 2, false, false, false, true>;
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(kernel),
+      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  (void)attr;
+  KernelTimer timer(stream);
+  hipLaunchKernelGGL(kernel, dim3(n_tiles, 1), dim3(kThreads), kLdsBytes,
+                     stream, src, wgt, dst, g,
+                     static_cast<unsigned>(src_elems * sizeof(float)),
+                     static_cast<unsigned>(wgt_elems * sizeof(float)), tiles_n,
+                     n_tiles, n_chunks);
+}
+
 }  // namespace
 
 static int launch_filter_backprop(const float* x, const float* dy, float* dw,
@@ -887,8 +968,7 @@ bool conv2d_igemm_supports(int direction, const snn_hip_conv2d_params& p) {
   const size_t w = static_cast<size_t>(p.window_rows) * p.window_cols *
                    p.channels * p.features;
   if (max(max(x, y), w) * sizeof(float) > kMaxBufferBytes) return false;
-  if (direction == SNN_HIP_FORWARD)
-    return p.channels % 4 == 0 && p.features % 4 == 0;
+  if (direction == SNN_HIP_FORWARD) return p.features % 4 == 0;
   if (direction == SNN_HIP_INPUT_BACKPROP)
     return p.features % 4 == 0;
   // filter backprop: a 64-wide tile of (tap, channel) must lie inside one tap
@@ -981,7 +1061,10 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
                            g.src_cols * g.src_ch;
   const size_t wgt_elems = static_cast<size_t>(p.window_rows) * p.window_cols *
                            p.channels * p.features;
-  if (direction == SNN_HIP_FORWARD) {
+  if (direction == SNN_HIP_FORWARD && g.src_ch % 4 != 0) {
+    launch_scalar_gather_forward(input, filter, output, g, src_elems,
+                                 wgt_elems, stream);
+  } else if (direction == SNN_HIP_FORWARD) {
     launch_auto<false, false>(input, filter, output, g, src_elems, wgt_elems,
                               stream);
   } else if (g.div_rows != 1 || g.div_cols != 1) {
