@@ -758,6 +758,205 @@ __global__ void __launch_bounds__(kThreads)
   }
 }
 
+// Filter backprop for layers with few input channels (the 7x7x3 stem): the
+// whole (tap, channel) range q = 0 .. R*S*C - 1 (at most 192) fits one
+// work-group, which therefore owns all of dW for 64 features and walks a
+// range of output pixels, 32 per chunk.  A tile: [32 pixels][q], gathered
+// element by element (consecutive q are not aligned runs of the input);
+// rows are 193 floats apart so that lanes that differ in the pixel hit
+// different banks.  The up to 6 x 2 accumulator blocks are dealt to the four
+// waves round-robin.  Partial sums meet in dW through float atomics.
+constexpr int kSmallQMax = 192;
+constexpr int kSmallQStride = kSmallQMax + 1;
+
+__global__ void __launch_bounds__(kThreads)
+    conv_filter_backprop_smallq_kernel(const float* __restrict__ x,
+                                       const float* __restrict__ dy,
+                                       float* __restrict__ dw,
+                                       FilterBackpropGeom g, unsigned x_bytes,
+                                       unsigned dy_bytes, unsigned dw_bytes,
+                                       int chunks_per_split) {
+  constexpr int BN = 64;
+  constexpr int A_FLOATS = kBK * kSmallQStride;
+  constexpr int STAGE_FLOATS = A_FLOATS + row_inner_floats(BN);
+  extern __shared__ __align__(16) float lds[];  // 2 * STAGE_FLOATS (65.25 KiB)
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n0 = blockIdx.x * BN;
+  const int q_total = g.win_rows * g.win_cols * g.channels;
+  const int n_mblocks = (q_total + 31) / 32;
+  const int n_blocks = 2 * n_mblocks;
+
+  const int n_chunks_total = (g.m_total + kBK - 1) / kBK;
+  const int chunk_begin = blockIdx.y * chunks_per_split;
+  const int n_chunks = min(chunks_per_split, n_chunks_total - chunk_begin);
+
+  const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, x_bytes);
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, dy_bytes);
+
+  // A gather: this lane owns pixel `a_px` of every chunk and the 24
+  // consecutive q starting at a_q0.
+  constexpr int A_PER_LANE = kSmallQMax * kBK / kThreads;  // 24
+  const int a_px = tid & 31;
+  const int a_q0 = (tid >> 5) * A_PER_LANE;
+  int a_ox, a_iy0, a_base;  // output column, first input row, element offset
+  {
+    const int m = chunk_begin * kBK + a_px;
+    a_ox = m % g.out_cols;
+    const int t = m / g.out_cols;
+    const int oy = t % g.out_rows;
+    const int n = t / g.out_rows;
+    a_iy0 = oy * g.stride_rows - g.pad_rows;
+    a_base = ((n * g.in_rows + a_iy0) * g.in_cols + a_ox * g.stride_cols -
+              g.pad_cols) * g.channels;
+  }
+  const int step_px = g.stride_cols * g.channels;
+  const int step_row =
+      (g.stride_rows * g.in_cols - g.out_cols * g.stride_cols) * g.channels;
+  const int step_img =
+      (g.in_rows - g.out_rows * g.stride_rows) * g.in_cols * g.channels;
+  const int iy_end = -g.pad_rows + g.out_rows * g.stride_rows;
+  // (tap row, tap col, channel) of a_q0
+  int q_r, q_s, q_c;
+  {
+    const int tap = a_q0 / g.channels;
+    q_c = a_q0 - tap * g.channels;
+    q_r = tap / g.win_cols;
+    q_s = tap - q_r * g.win_cols;
+  }
+  // B copy: float4 `b_vec` of pixel rows b_row0 and b_row0 + 16
+  const int b_vec = tid & 15;
+  const int b_row0 = tid >> 4;
+  unsigned dy_off[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m = chunk_begin * kBK + b_row0 + 16 * i;
+    dy_off[i] = (n0 + 4 * b_vec < g.features)
+                    ? static_cast<unsigned>(m * g.features + n0 + 4 * b_vec) * 4u
+                    : kOob;
+  }
+
+  float a_reg[A_PER_LANE];
+  float4 b_reg[2];
+  auto load_global = [&]() {
+    const int ix0 = a_ox * g.stride_cols - g.pad_cols;
+    int r = q_r, sc = q_s, c = q_c;
+#pragma unroll
+    for (int j = 0; j < A_PER_LANE; ++j) {
+      const int iy = a_iy0 + r;
+      const int ix = ix0 + sc;
+      const bool ok =
+          (a_q0 + j < q_total) &
+          (static_cast<unsigned>(iy) < static_cast<unsigned>(g.in_rows)) &
+          (static_cast<unsigned>(ix) < static_cast<unsigned>(g.in_cols));
+      const int off = a_base + (r * g.in_cols + sc) * g.channels + c;
+      a_reg[j] = __builtin_bit_cast(
+          float, __builtin_amdgcn_raw_buffer_load_b32(
+                     x_rsrc, ok ? static_cast<unsigned>(off) * 4u : kOob, 0,
+                     0));
+      if (++c == g.channels) {
+        c = 0;
+        if (++sc == g.win_cols) { sc = 0; ++r; }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      b_reg[i] = buffer_load4(dy_rsrc, dy_off[i]);
+      if (dy_off[i] != kOob) dy_off[i] += kBK * g.features * 4u;
+    }
+    // advance the pixel by one chunk
+    a_ox += kBK;
+    a_base += kBK * step_px;
+    while (a_ox >= g.out_cols) {
+      a_ox -= g.out_cols;
+      a_base += step_row;
+      a_iy0 += g.stride_rows;
+      if (a_iy0 == iy_end) {
+        a_iy0 = -g.pad_rows;
+        a_base += step_img;
+      }
+    }
+  };
+  float* const a_store = lds + a_px * kSmallQStride + a_q0;
+  float* const b_store = lds + A_FLOATS + b_row0 * (BN + kPad) + 4 * b_vec;
+  auto store_tiles = [&](int stage) {
+#pragma unroll
+    for (int j = 0; j < A_PER_LANE; ++j)
+      a_store[stage * STAGE_FLOATS + j] = a_reg[j];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      *reinterpret_cast<float4*>(b_store + stage * STAGE_FLOATS +
+                                 16 * i * (BN + kPad)) = b_reg[i];
+  };
+
+  constexpr int BLOCKS_PER_WAVE = 3;  // 12 blocks over 4 waves
+  float16v acc[BLOCKS_PER_WAVE];
+#pragma unroll
+  for (int i = 0; i < BLOCKS_PER_WAVE; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+  const int l32 = lane & 31;
+  auto compute = [&](int stage) {
+    const float* a_tile = lds + stage * STAGE_FLOATS;
+    const float* b_tile = a_tile + A_FLOATS;
+#pragma unroll
+    for (int i = 0; i < BLOCKS_PER_WAVE; ++i) {
+      const int blk = wave + 4 * i;
+      if (blk >= n_blocks) break;
+      const int mb = blk >> 1, nb = blk & 1;
+      float4 a[kBK / 8], b[kBK / 8];
+#pragma unroll
+      for (int s4 = 0; s4 < kBK / 8; ++s4) {
+        a[s4] = fetch_row_inner<kSmallQStride - kPad>(a_tile, mb * 32 + l32,
+                                                      s4, lane);
+        b[s4] = fetch_row_inner<BN>(b_tile, nb * 32 + l32, s4, lane);
+      }
+#pragma unroll
+      for (int s4 = 0; s4 < kBK / 8; ++s4)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+              comp(a[s4], t), comp(b[s4], t), acc[i], 0, 0, 0);
+    }
+  };
+
+  load_global();
+  store_tiles(0);
+  __syncthreads();
+  for (int done = 0; done < n_chunks; ++done) {
+    const int stage = done & 1;
+    const bool more = done + 1 < n_chunks;
+    if (more) load_global();
+    compute(stage);
+    if (more) store_tiles(stage ^ 1);
+    __syncthreads();
+  }
+
+  const __amdgpu_buffer_rsrc_t dw_rsrc = make_rsrc(dw, dw_bytes);
+  const unsigned row_bytes = static_cast<unsigned>(g.features) * 4u;
+#pragma unroll
+  for (int i = 0; i < BLOCKS_PER_WAVE; ++i) {
+    const int blk = wave + 4 * i;
+    if (blk >= n_blocks) break;
+    const int mb = blk >> 1, nb = blk & 1;
+    const int col = n0 + nb * 32 + l32;
+    const int q_base = mb * 32 + 4 * (lane >> 5);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int q = q_base + 8 * (v >> 2) + (v & 3);
+      const unsigned off =
+          (col < g.features && q < q_total)
+              ? static_cast<unsigned>(q) * row_bytes +
+                    static_cast<unsigned>(col) * 4u
+              : kOob;
+      __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(acc[i][v], dw_rsrc, off,
+                                                      0, 0);
+    }
+  }
+}
+
 __global__ void __launch_bounds__(256)
     zero_fill_kernel(float4* __restrict__ p, size_t n_vec) {
   const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
@@ -939,6 +1138,34 @@ static int launch_filter_backprop(const float* x, const float* dy, float* dw,
   const size_t dy_elems = static_cast<size_t>(g.m_total) * p.features;
   const size_t dw_elems = static_cast<size_t>(p.window_rows) * p.window_cols *
                           p.channels * p.features;
+  if (p.channels % 64 != 0) {
+    // few (tap, channel) pairs: one work-group column per 64 features, the
+    // pixel range split over about two work-groups per CU
+    const int n_chunks = ceil_div(g.m_total, kBK);
+    const int col_groups = ceil_div(p.features, 64);
+    int splits = max(1, min(ceil_div(512, col_groups), n_chunks / 4));
+    const int per_split = ceil_div(n_chunks, splits);
+    splits = ceil_div(n_chunks, per_split);
+    const size_t n_vec = dw_elems / 4;  // features % 4 == 0
+    hipLaunchKernelGGL(zero_fill_kernel,
+                       dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
+                       dim3(256), 0, stream, reinterpret_cast<float4*>(dw),
+                       n_vec);
+    constexpr size_t kLdsBytes =
+        2 * sizeof(float) * (kBK * kSmallQStride + row_inner_floats(64));
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(conv_filter_backprop_smallq_kernel),
+        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    (void)attr;
+    KernelTimer timer(stream);
+    hipLaunchKernelGGL(conv_filter_backprop_smallq_kernel,
+                       dim3(col_groups, splits), dim3(kThreads), kLdsBytes,
+                       stream, x,
+                       dy, dw, g, static_cast<unsigned>(x_elems * 4),
+                       static_cast<unsigned>(dy_elems * 4),
+                       static_cast<unsigned>(dw_elems * 4), per_split);
+    return SNN_HIP_OK;
+  }
   const int tiles = (p.window_rows * p.window_cols * p.channels / 64) *
                     ceil_div(p.features, 64);
   const int n_chunks = ceil_div(g.m_total, kBK);
@@ -971,8 +1198,11 @@ bool conv2d_igemm_supports(int direction, const snn_hip_conv2d_params& p) {
   if (direction == SNN_HIP_FORWARD) return p.features % 4 == 0;
   if (direction == SNN_HIP_INPUT_BACKPROP)
     return p.features % 4 == 0;
-  // filter backprop: a 64-wide tile of (tap, channel) must lie inside one tap
-  return p.channels % 64 == 0 && p.features % 4 == 0;
+  // filter backprop: a 64-wide tile of (tap, channel) must lie inside one
+  // tap, or the whole (tap, channel) range must fit one work-group
+  return p.features % 4 == 0 &&
+         (p.channels % 64 == 0 ||
+          p.window_rows * p.window_cols * p.channels <= kSmallQMax);
 }
 
 bool batched_gemm_mfma_supports(int m, int k, int n, const void* a,

@@ -175,6 +175,25 @@ def test_winograd_fused_shapes(shape, direction):
     conv_case(p, direction, [ALGO.WINOGRAD], seed=1300 + rows + ch)
 
 
+@pytest.mark.parametrize("direction", [DIRECTION.FORWARD,
+                                       DIRECTION.FILTER_BACKPROP])
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, window, stride, same
+    (3, 17, 13, 3, 64, 7, 2, True),     # stem-like, ragged image
+    (2, 9, 9, 5, 36, 3, 1, True),       # 45 (tap, channel) pairs
+    (2, 12, 10, 20, 40, 3, 1, False),   # 180 pairs, features not x64
+    (4, 8, 8, 6, 128, 5, 2, True),      # 150 pairs, two feature groups
+    (1, 6, 7, 1, 4, 3, 1, True),        # a single channel
+    (2, 30, 30, 3, 32, 7, 4, False),    # stride 4
+])
+def test_small_channel_counts_on_mfma(shape, direction):
+    """Channel counts that are not multiples of 4 (forward: scalar gather)
+    and (tap, channel) ranges that fit one work-group (filter backprop)."""
+    batch, rows, cols, ch, feats, window, stride, same = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, window, stride, same)
+    conv_case(p, direction, [ALGO.IM2COL], seed=1400 + rows + ch)
+
+
 # ---- full batch-32 shapes: sampled float64 recomputation + linearity --------
 
 def sampled_forward_reference(x, w, p, samples):
