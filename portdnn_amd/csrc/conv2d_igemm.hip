@@ -336,10 +336,10 @@ __global__ void __launch_bounds__(kThreads)
 }
 
 // ---------------------------------------------------------------------------
-// Fast path.  Measured on MI355X: VALU instructions issued between MFMAs are
-// not hidden behind them -- every vector ALU cycle in the main loop is a cycle
-// the matrix pipe idles -- so this kernel keeps per-chunk vector work to three
-// instructions per gathered row and nothing else:
+// Fast path.  The gather of the generic kernel spends dozens of integer
+// vector instructions (multiplies, divisions by the channel count) per chunk
+// and lane; this kernel keeps per-chunk vector work to three instructions per
+// gathered row and nothing else:
 //   * src_ch % 32 == 0, so a 32-wide reduction chunk lies inside one filter
 //     tap and the tap / channel bookkeeping is wave-uniform (scalar ALU);
 //   * per-row validity of every tap is a precomputed 32-bit mask; an invalid
@@ -957,6 +957,46 @@ __global__ void __launch_bounds__(kThreads)
   }
 }
 
+// Second half of the input gradient for layers with very few input channels
+// (the stem): Z[m][(r, s, c)] = sum_k dY[m][k] * W[r][s][c][k] has been
+// computed as one GEMM over the output pixels m; every input element then
+// sums the Z entries of the taps that reach it,
+//   dX[n][y][x][c] = sum_{r,s} Z[(n, (y+pad-r)/stride, (x+pad-s)/stride)][r][s][c]
+// over the taps for which the divisions are exact and in range.  One lane per
+// dX element, channel fastest.
+__global__ void __launch_bounds__(256)
+    col2im_gather_kernel(const float* __restrict__ z, float* __restrict__ dx,
+                         FilterBackpropGeom g, int images) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  const size_t total =
+      static_cast<size_t>(images) * g.in_rows * g.in_cols * g.channels;
+  if (idx >= total) return;
+  const int c = static_cast<int>(idx % g.channels);
+  size_t t = idx / g.channels;
+  const int xx = static_cast<int>(t % g.in_cols);
+  t /= g.in_cols;
+  const int yy = static_cast<int>(t % g.in_rows);
+  const int n = static_cast<int>(t / g.in_rows);
+  const int q_total = g.win_rows * g.win_cols * g.channels;
+  float acc = 0.f;
+  for (int r = 0; r < g.win_rows; ++r) {
+    const int ty = yy + g.pad_rows - r;
+    if (ty < 0 || ty % g.stride_rows != 0) continue;
+    const int oy = ty / g.stride_rows;
+    if (oy >= g.out_rows) continue;
+    for (int sc = 0; sc < g.win_cols; ++sc) {
+      const int tx = xx + g.pad_cols - sc;
+      if (tx < 0 || tx % g.stride_cols != 0) continue;
+      const int ox = tx / g.stride_cols;
+      if (ox >= g.out_cols) continue;
+      acc += z[(static_cast<size_t>(n * g.out_rows + oy) * g.out_cols + ox) *
+                   q_total +
+               (r * g.win_cols + sc) * g.channels + c];
+    }
+  }
+  dx[idx] = acc;
+}
+
 __global__ void __launch_bounds__(256)
     zero_fill_kernel(float4* __restrict__ p, size_t n_vec) {
   const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
@@ -1123,6 +1163,86 @@ void launch_scalar_gather_forward(const float* src, const float* wgt,
 
 }  // namespace
 
+// Input gradient with very few input channels: as a GEMM over (r, s, k) the
+// 3 output columns would waste 29/32 of every matrix instruction, so the
+// product is taken per output pixel against all (r, s, c) at once (a 1x1
+// "convolution" of dY with R*S*C features, the HWCF filter being exactly the
+// K-contiguous operand that needs) and col2im_gather_kernel folds the taps.
+// Z takes out_rows * out_cols * R*S*C floats per image: the caller's
+// workspace when it is big enough for at least one image, else a
+// stream-ordered temporary of up to 64 MiB; images go through in minibatches.
+static int launch_input_backprop_col2im(const float* dy, const float* filter,
+                                        float* dx,
+                                        const snn_hip_conv2d_params& p,
+                                        float* workspace,
+                                        size_t workspace_elems,
+                                        hipStream_t stream) {
+  const int q_total = p.window_rows * p.window_cols * p.channels;
+  const size_t z_per_image =
+      static_cast<size_t>(p.out_rows) * p.out_cols * q_total;
+  float* z = workspace;
+  size_t z_elems = workspace_elems;
+  bool temporary = false;
+  if (z == nullptr || z_elems < z_per_image ||
+      (reinterpret_cast<uintptr_t>(z) & 15u) != 0) {
+    const size_t cap = max(z_per_image, (size_t{64} << 20) / sizeof(float));
+    z_elems = min(cap, z_per_image * p.batch);
+    void* ptr = nullptr;
+    if (hipMallocAsync(&ptr, z_elems * sizeof(float), stream) != hipSuccess)
+      return SNN_HIP_ALLOCATION_PROBLEM;
+    z = static_cast<float*>(ptr);
+    temporary = true;
+  }
+  // at most kMaxBufferBytes of Z per GEMM launch
+  const size_t max_images = min(z_elems, kMaxBufferBytes / sizeof(float)) /
+                            z_per_image;
+  const int minibatch = static_cast<int>(
+      max(size_t{1}, min(static_cast<size_t>(p.batch), max_images)));
+
+  FilterBackpropGeom fg;
+  fg.batch = p.batch; fg.in_rows = p.in_rows; fg.in_cols = p.in_cols;
+  fg.channels = p.channels; fg.out_rows = p.out_rows; fg.out_cols = p.out_cols;
+  fg.features = p.features; fg.win_rows = p.window_rows;
+  fg.win_cols = p.window_cols; fg.stride_rows = p.stride_rows;
+  fg.stride_cols = p.stride_cols; fg.pad_rows = p.pad_rows;
+  fg.pad_cols = p.pad_cols; fg.m_total = 0;
+
+  const size_t wgt_elems = static_cast<size_t>(q_total) * p.features;
+  for (int first = 0; first < p.batch; first += minibatch) {
+    const int images = min(minibatch, p.batch - first);
+    Gather g;
+    g.batch = images;
+    g.p_rows = p.out_rows; g.p_cols = p.out_cols;
+    g.src_rows = p.out_rows; g.src_cols = p.out_cols;
+    g.src_ch = p.features;
+    g.win_rows = g.win_cols = 1;
+    g.step_rows = g.step_cols = 1;
+    g.off_rows = g.off_cols = 0;
+    g.tap_sign = 1;
+    g.div_rows = g.div_cols = 1;
+    g.m_total = images * p.out_rows * p.out_cols;
+    g.k_total = p.features;
+    g.n_total = q_total;
+    g.z_src = g.z_wgt = g.z_dst = 0;
+    const size_t dy_elems = static_cast<size_t>(g.m_total) * p.features;
+    const float* dy_mb = dy + static_cast<size_t>(first) * p.out_rows *
+                                  p.out_cols * p.features;
+    launch_tile<64, 64, 2, 2, true, false>(dy_mb, filter, z, g, dy_elems,
+                                           wgt_elems, 1, stream);
+    const size_t dx_elems = static_cast<size_t>(images) * p.in_rows *
+                            p.in_cols * p.channels;
+    float* dx_mb = dx + static_cast<size_t>(first) * p.in_rows * p.in_cols *
+                            p.channels;
+    hipLaunchKernelGGL(col2im_gather_kernel,
+                       dim3(static_cast<unsigned>(ceil_div(dx_elems, size_t{256}))),
+                       dim3(256), 0, stream, z, dx_mb, fg, images);
+  }
+  const hipError_t err = hipGetLastError();
+  if (temporary) (void)hipFreeAsync(z, stream);
+  if (err != hipSuccess) return report_hip_error(err, "input backprop col2im");
+  return SNN_HIP_OK;
+}
+
 static int launch_filter_backprop(const float* x, const float* dy, float* dw,
                            const snn_hip_conv2d_params& p, hipStream_t stream) {
   FilterBackpropGeom g;
@@ -1254,7 +1374,14 @@ int launch_batched_gemm_mfma_f32(const float* a, const float* b, float* c,
 int launch_conv2d_igemm_f32(int direction, const float* input,
                             const float* filter, float* output,
                             const snn_hip_conv2d_params& p,
-                            hipStream_t stream) {
+                            hipStream_t stream, float* workspace,
+                            size_t workspace_elems) {
+  if (direction == SNN_HIP_INPUT_BACKPROP && p.channels < 16 &&
+      p.features % kBK == 0 &&
+      static_cast<size_t>(p.out_rows) * p.out_cols * p.window_rows *
+              p.window_cols * p.channels * sizeof(float) <= kMaxBufferBytes)
+    return launch_input_backprop_col2im(input, filter, output, p, workspace,
+                                        workspace_elems, stream);
   if (direction == SNN_HIP_FILTER_BACKPROP) {
     const int rc = launch_filter_backprop(input, filter, output, p, stream);
     SNN_HIP_CHECK_LAUNCH();

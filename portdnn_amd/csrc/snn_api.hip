@@ -307,10 +307,11 @@ template <>
 int launch_gemm_path<float>(int direction, const float* input,
                             const float* filter, float* output,
                             const snn_hip_conv2d_params& p, hipStream_t s,
-                            float*, size_t) {
+                            float* workspace, size_t workspace_elems) {
   if (conv2d_igemm_supports(direction, p) && aligned16(input) &&
       aligned16(filter) && aligned16(output))
-    return launch_conv2d_igemm_f32(direction, input, filter, output, p, s);
+    return launch_conv2d_igemm_f32(direction, input, filter, output, p, s,
+                                   workspace, workspace_elems);
   return launch_conv2d_direct<float>(direction, input, filter, output, p, s);
 }
 

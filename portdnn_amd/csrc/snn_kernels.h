@@ -20,7 +20,9 @@ int launch_conv2d_direct(int direction, const T* input, const T* filter,
 bool conv2d_igemm_supports(int direction, const snn_hip_conv2d_params& p);
 int launch_conv2d_igemm_f32(int direction, const float* input,
                             const float* filter, float* output,
-                            const snn_hip_conv2d_params& p, hipStream_t stream);
+                            const snn_hip_conv2d_params& p, hipStream_t stream,
+                            float* workspace = nullptr,
+                            size_t workspace_elems = 0);
 
 // Batched row-major GEMM C[z] = A[z] (m x k) * B[z] (k x n) on the same MFMA
 // kernel; operands of consecutive problems are contiguous.  `supports` checks

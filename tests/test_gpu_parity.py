@@ -176,6 +176,7 @@ def test_winograd_fused_shapes(shape, direction):
 
 
 @pytest.mark.parametrize("direction", [DIRECTION.FORWARD,
+                                       DIRECTION.INPUT_BACKPROP,
                                        DIRECTION.FILTER_BACKPROP])
 @pytest.mark.parametrize("shape", [
     # batch, rows, cols, channels, features, window, stride, same
@@ -187,8 +188,10 @@ def test_winograd_fused_shapes(shape, direction):
     (2, 30, 30, 3, 32, 7, 4, False),    # stride 4
 ])
 def test_small_channel_counts_on_mfma(shape, direction):
-    """Channel counts that are not multiples of 4 (forward: scalar gather)
-    and (tap, channel) ranges that fit one work-group (filter backprop)."""
+    """Channel counts that are not multiples of 4 (forward: scalar gather),
+    (tap, channel) ranges that fit one work-group (filter backprop) and
+    fewer than 16 channels (input backprop: GEMM per output pixel + tap
+    gather when the feature count is a multiple of 32)."""
     batch, rows, cols, ch, feats, window, stride, same = shape
     p = ops.conv_params(batch, rows, cols, ch, feats, window, stride, same)
     conv_case(p, direction, [ALGO.IM2COL], seed=1400 + rows + ch)
