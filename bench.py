@@ -78,19 +78,24 @@ def main():
         return capi.lib().snn_hip_conv2d_algorithm_supports(
             ctypes.byref(p), DIRECTION.FORWARD, algo) == algo
 
-    def event_time_ms(fn, reps, warm=3):
-        """Average duration of one call, HIP events on the launch stream."""
+    def event_time_ms(fn, reps, warm=3, repeats=5):
+        """Duration of one call: `reps` back-to-back calls between two HIP
+        events on the launch stream, median over `repeats` such runs."""
         for _ in range(warm):
             fn()
-        start = torch.cuda.Event(enable_timing=True)
-        stop = torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        start.record()
-        for _ in range(reps):
-            fn()
-        stop.record()
-        stop.synchronize()
-        return start.elapsed_time(stop) / reps
+        times = []
+        for _ in range(repeats):
+            start = torch.cuda.Event(enable_timing=True)
+            stop = torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            start.record()
+            for _ in range(reps):
+                fn()
+            stop.record()
+            stop.synchronize()
+            times.append(start.elapsed_time(stop) / reps)
+        times.sort()
+        return times[len(times) // 2]
 
     # ---- the workload --------------------------------------------------------
     layers = []
@@ -168,6 +173,13 @@ def main():
         "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
         "avg_kernel_ms": round(k3_kernel_ms / k3_kernels, 5),
         "algorithmic_gflop_per_launch": round(k3_flops / k3_kernels / 1e9, 4),
+        # Winograd F(2x2,3x3) executes 16/36 of the algorithmic flops on the
+        # matrix cores; this is the MFMA pipe's own utilisation
+        "mfma_executed_tflops": round(
+            achieved * (4.0 / 9.0 if k3_algos == ["winograd"] else 1.0), 2),
+        "mfma_executed_frac": round(
+            achieved * (4.0 / 9.0 if k3_algos == ["winograd"] else 1.0) /
+            PEAK_FP32_MFMA_TFLOPS, 4),
         "traffic": WINOGRAD_TRAFFIC_BYTES if k3_algos == ["winograd"] else None}
 
     detail = {"layers": per_layer}
@@ -212,7 +224,7 @@ def main():
                 i = state["i"] % sets
                 state["i"] += 1
                 ops.depthwise_conv2d(xs[i], f, p, out=ys[i])
-            ms = event_time_ms(run, reps=5 * sets, warm=sets)
+            ms = event_time_ms(run, reps=5 * sets, warm=sets, repeats=3)
             gbs = nbytes / ms / 1e6
             mem.append({"op": "depthwise3x3_%dx%dx%d_s%d" % (size, size, ch,
                                                              stride),
@@ -238,7 +250,7 @@ def main():
                 i = state["i"] % sets
                 state["i"] += 1
                 ops.pooling_forward(xs[i], p, op, out=ys[i])
-            ms = event_time_ms(run, reps=5 * sets, warm=sets)
+            ms = event_time_ms(run, reps=5 * sets, warm=sets, repeats=3)
             gbs = nbytes / ms / 1e6
             mem.append({"op": name, "bytes": nbytes, "ms": round(ms, 5),
                         "gbs": round(gbs, 1),
