@@ -119,7 +119,7 @@ def test_stem_7x7_stride2(direction):
 
 
 def test_config0_single_image_tiled():
-    """BASELINE configuration 0: N=1, 56x56x64 -> 64, 3x3 s1 SAME, Tiled;
+    """Benchmark configuration 0: N=1, 56x56x64 -> 64, 3x3 s1 SAME, Tiled;
     also checked against the reference-loop-nest restatement in fp32."""
     p = ops.conv_params(1, 56, 56, 64, 64, 3, 1, True)
     rng = np.random.default_rng(0x5EED)
