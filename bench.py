@@ -258,6 +258,24 @@ def main():
             del xs, ys
         detail["memory_bound"] = mem
 
+        # the public matmul op (sycldnn::matmul::launch) on the same MFMA kernel
+        mm = []
+        for batches, m, k, n, tb in ((1, 4096, 1024, 1024, False),
+                                    (1, 4096, 1024, 1024, True),
+                                    (16, 1568, 256, 256, False)):
+            a = uniform(batches * m * k)
+            b = uniform(batches * k * n)
+            c = torch.empty(batches * m * n, device="cuda")
+            ms = event_time_ms(lambda: ops.matmul(a, b, batches, m, k, n, False,
+                                                  tb, 0.0, out=c), reps=10,
+                               warm=2, repeats=3)
+            tf = 2.0 * batches * m * k * n / ms / 1e9
+            mm.append({"op": "matmul b%d %dx%dx%d%s" % (
+                batches, m, k, n, " rhs^T" if tb else ""), "ms": round(ms, 4),
+                "tflops": round(tf, 2),
+                "frac_mfma_peak": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)})
+        detail["matmul"] = mm
+
     # ---- CPU baseline: the reference's tiled algorithm, restated --------------
     cpu = None
     if not args.no_cpu_baseline:

@@ -1,0 +1,5 @@
+// portDNN include path kept for source compatibility.
+#ifndef SNN_FWD_MATMUL_PARAMS_H
+#define SNN_FWD_MATMUL_PARAMS_H
+#include "portdnn/hip/matmul.h"
+#endif

@@ -1006,7 +1006,10 @@ __global__ void __launch_bounds__(256)
 template <int BM, int BN, int WM, int WN, bool B_K_INNER, bool STRIDED>
 void launch_tile(const float* src, const float* wgt, float* dst,
                  const Gather& g, size_t src_elems, size_t wgt_elems,
-                 int splits, hipStream_t stream, int batches = 1) {
+                 int splits, hipStream_t stream, int batches = 1,
+                 bool accumulate = false) {
+  // accumulate: add the product to what dst holds (atomic kernel, no zero
+  // fill) instead of overwriting it.
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(g.m_total, BM));
   const unsigned tiles_n = static_cast<unsigned>(ceil_div(g.n_total, BN));
   const unsigned n_tiles = tiles_m * tiles_n;
@@ -1023,15 +1026,16 @@ void launch_tile(const float* src, const float* wgt, float* dst,
                     g.win_rows * g.win_cols <= 32;
   const unsigned dst_bytes = static_cast<unsigned>(
       static_cast<size_t>(g.m_total) * g.n_total * sizeof(float));
-  if (splits > 1) {
+  if (splits > 1 || accumulate) {
     // Partial sums meet in the output through float atomics: start from zero.
     // (a batched launch keeps its problems contiguous: z_dst == m * n)
     const size_t n_vec = static_cast<size_t>(batches) * g.m_total *
-                         g.n_total / 4;  // n_total % 4 == 0
-    hipLaunchKernelGGL(zero_fill_kernel,
-                       dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
-                       dim3(256), 0, stream, reinterpret_cast<float4*>(dst),
-                       n_vec);
+                         g.n_total / 4;  // a multiple of 4 elements
+    if (!accumulate)
+      hipLaunchKernelGGL(
+          zero_fill_kernel,
+          dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))), dim3(256),
+          0, stream, reinterpret_cast<float4*>(dst), n_vec);
     KernelTimer timer(stream);
     if (fast) {
       auto kernel = conv_igemm_fast_kernel<BM, BN, WM, WN, B_K_INNER, true>;
@@ -1326,20 +1330,24 @@ bool conv2d_igemm_supports(int direction, const snn_hip_conv2d_params& p) {
 }
 
 bool batched_gemm_mfma_supports(int m, int k, int n, const void* a,
-                                const void* b, const void* c) {
+                                const void* b, const void* c,
+                                bool transpose_b) {
   auto aligned = [](const void* p) {
     return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
   };
-  return k % kBK == 0 && n % 4 == 0 && aligned(a) && aligned(b) &&
-         aligned(c) &&
+  return k % kBK == 0 && (transpose_b || n % 4 == 0) && aligned(a) &&
+         aligned(b) && aligned(c) &&
          static_cast<size_t>(m) * max(k, n) * sizeof(float) <= kMaxBufferBytes &&
          static_cast<size_t>(k) * n * sizeof(float) <= kMaxBufferBytes;
 }
 
 int launch_batched_gemm_mfma_f32(const float* a, const float* b, float* c,
                                  int batches, int m, int k, int n,
-                                 hipStream_t stream) {
-  // C[z] = A[z] (m x k) * B[z] (k x n): a 1x1 "convolution" over m pixels.
+                                 hipStream_t stream, bool transpose_b,
+                                 bool accumulate) {
+  // C[z] (+)= A[z] (m x k) * op(B[z]): a 1x1 "convolution" over m pixels.  B
+  // as k x n is the forward filter layout, B as n x k (transpose_b) the
+  // K-contiguous layout of the input-gradient kernel.
   Gather g;
   g.batch = 1;
   g.p_rows = 1; g.p_cols = m;
@@ -1359,14 +1367,23 @@ int launch_batched_gemm_mfma_f32(const float* a, const float* b, float* c,
   const long tiles = static_cast<long>(ceil_div(m, 64)) * ceil_div(n, 64) * batches;
   const int n_chunks = k / kBK;
   int splits = 1;
-  if (tiles < kResidentSlots) {
+  // the zero fill of a split launch writes float4s
+  const bool can_split =
+      accumulate || (static_cast<size_t>(batches) * m * n) % 4 == 0;
+  if (tiles < kResidentSlots && can_split) {
     splits = static_cast<int>((kSplitUnits + tiles - 1) / tiles);
     splits = max(1, min(splits, n_chunks / kMinChunksPerSplit));
   }
-  launch_tile<64, 64, 2, 2, false, false>(a, b, c, g,
-                                          static_cast<size_t>(m) * k,
-                                          static_cast<size_t>(k) * n, splits,
-                                          stream, batches);
+  if (transpose_b)
+    launch_tile<64, 64, 2, 2, true, false>(a, b, c, g,
+                                           static_cast<size_t>(m) * k,
+                                           static_cast<size_t>(k) * n, splits,
+                                           stream, batches, accumulate);
+  else
+    launch_tile<64, 64, 2, 2, false, false>(a, b, c, g,
+                                            static_cast<size_t>(m) * k,
+                                            static_cast<size_t>(k) * n, splits,
+                                            stream, batches, accumulate);
   SNN_HIP_CHECK_LAUNCH();
   return SNN_HIP_OK;
 }

@@ -2,9 +2,10 @@
 // Stand-in for portDNN's MatmulKernel (src/matmul/kernels.h:26-133,
 // src/matmul/launch.cc:51-56).
 //
-// General-shape kernel: 64x64 output tile per 256-lane work-group, A and B
-// tiles staged in LDS, 4x4 register block per lane, every edge bounds-checked
-// so any m, k, n and both transposes are accepted.
+// Shapes the matrix-core kernel takes (see launch_matmul_f32) go to it; this
+// file holds the general-shape kernel: 64x64 output tile per 256-lane
+// work-group, A and B tiles staged in LDS, 4x4 register block per lane, every
+// edge bounds-checked so any m, k, n and both transposes are accepted.
 #include "snn_kernels.h"
 
 namespace snn {
@@ -93,11 +94,34 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+__global__ void __launch_bounds__(256)
+    scale_kernel(float* __restrict__ c, size_t n, float beta) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i < n) c[i] *= beta;
+}
+
 }  // namespace
 
 int launch_matmul_f32(const float* lhs, const float* rhs, float* output,
                       int batches, int m, int k, int n, bool transpose_lhs,
                       bool transpose_rhs, float beta, hipStream_t stream) {
+  // Matrix-core path: A not transposed, k a multiple of 32, operands aligned
+  // (the implicit-GEMM kernel of the 1x1 convolution; B^T is its K-contiguous
+  // filter layout).  beta == 0 overwrites, beta != 0 first scales C in place
+  // (unless beta == 1) and then accumulates with float atomics.
+  if (!transpose_lhs && m >= 32 &&
+      batched_gemm_mfma_supports(m, k, n, lhs, rhs, output, transpose_rhs) &&
+      (batches == 1 || (static_cast<size_t>(m) * n) % 4 == 0)) {
+    const bool accumulate = beta != 0.f;
+    if (accumulate && beta != 1.f) {
+      const size_t total = static_cast<size_t>(batches) * m * n;
+      hipLaunchKernelGGL(scale_kernel,
+                         dim3(static_cast<unsigned>(ceil_div(total, size_t{256}))),
+                         dim3(256), 0, stream, output, total, beta);
+    }
+    return launch_batched_gemm_mfma_f32(lhs, rhs, output, batches, m, k, n,
+                                        stream, transpose_rhs, accumulate);
+  }
   const dim3 grid(static_cast<unsigned>(ceil_div(m, kTile)),
                   static_cast<unsigned>(ceil_div(n, kTile)),
                   static_cast<unsigned>(batches));

@@ -24,14 +24,18 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
                             float* workspace = nullptr,
                             size_t workspace_elems = 0);
 
-// Batched row-major GEMM C[z] = A[z] (m x k) * B[z] (k x n) on the same MFMA
-// kernel; operands of consecutive problems are contiguous.  `supports` checks
-// k % 32 == 0, n % 4 == 0 and 16-byte alignment.
+// Batched row-major GEMM C[z] = A[z] (m x k) * op(B[z]) on the same MFMA
+// kernel, op(B) = B (k x n) or B^T with B stored n x k; operands of
+// consecutive problems are contiguous.  `accumulate` adds the product to C
+// (float atomics) instead of overwriting it.  `supports` checks k % 32 == 0,
+// n % 4 == 0 unless B is transposed, and 16-byte alignment.
 bool batched_gemm_mfma_supports(int m, int k, int n, const void* a,
-                                const void* b, const void* c);
+                                const void* b, const void* c,
+                                bool transpose_b = false);
 int launch_batched_gemm_mfma_f32(const float* a, const float* b, float* c,
                                  int batches, int m, int k, int n,
-                                 hipStream_t stream);
+                                 hipStream_t stream, bool transpose_b = false,
+                                 bool accumulate = false);
 
 // Winograd F(2x2,3x3) convolution, forward and input backprop
 // (conv2d_winograd.hip).  `workspace` holds the three transform buffers.

@@ -15,6 +15,7 @@
 #include <portdnn/conv2d/workspace_size.h>
 #include <portdnn/depthwise_conv2d/launch.h>
 #include <portdnn/helpers/padding.h>
+#include <portdnn/matmul/launch.h>
 #include <portdnn/pooling/launch.h>
 
 #include <cmath>
@@ -266,6 +267,82 @@ static void test_event_dependencies(backend::HIPBackend& backend) {
   (void)hipStreamDestroy(other);
 }
 
+// test/matmul/fixture.h:37-76: iota operands and initial output, offset
+// pointers, every transpose / beta combination; here also sizes that take the
+// matrix-core path (k a multiple of 32) and ones that do not.
+template <bool TL, bool TR>
+static void test_matmul_case(backend::HIPBackend& backend, int batches, int m,
+                             int k, int n, float beta, int offset) {
+  const size_t lhs_n = static_cast<size_t>(batches) * m * k + offset;
+  const size_t rhs_n = static_cast<size_t>(batches) * k * n + offset;
+  const size_t out_n = static_cast<size_t>(batches) * m * n + offset;
+  const auto lhs = iota_data(lhs_n, 16), rhs = iota_data(rhs_n, 16);
+  const auto out0 = iota_data(out_n, 16);
+  DeviceBuffer d_lhs(backend, lhs), d_rhs(backend, rhs), d_out(backend, out0);
+  auto status = matmul::launch<float, TL, TR>(
+      d_lhs.ptr + offset, d_rhs.ptr + offset, d_out.ptr + offset,
+      matmul::MatmulParams{batches, m, k, n, beta}, backend);
+  CHECK(status.status == StatusCode::OK);
+  status.event.wait_and_throw();
+  std::vector<float> ref = out0;
+  oracle_matmul(lhs.data() + offset, rhs.data() + offset, ref.data() + offset,
+                batches, m, k, n, TL, TR, beta, 1);
+  const bool ok = close(d_out.host(), ref, true);
+  if (!ok)
+    std::printf("  matmul TL %d TR %d batches %d m %d k %d n %d beta %g\n", TL,
+                TR, batches, m, k, n, beta);
+  CHECK(ok);
+}
+
+static void test_matmul(backend::HIPBackend& backend) {
+  const int shapes[][4] = {{1, 14, 15, 16}, {3, 16, 14, 15}, {2, 70, 64, 36},
+                           {1, 130, 96, 64}, {3, 33, 32, 8}};
+  for (auto const& s : shapes) {
+    for (float beta : {0.f, 1.f, 2.f}) {
+      for (int offset : {0, 8}) {
+        test_matmul_case<false, false>(backend, s[0], s[1], s[2], s[3], beta,
+                                       offset);
+        test_matmul_case<false, true>(backend, s[0], s[1], s[2], s[3], beta,
+                                      offset);
+        test_matmul_case<true, false>(backend, s[0], s[1], s[2], s[3], beta,
+                                      offset);
+        test_matmul_case<true, true>(backend, s[0], s[1], s[2], s[3], beta,
+                                     offset);
+      }
+    }
+  }
+  // internal/matmul/launch.h:66-70: non-positive sizes are invalid parameters
+  DeviceBuffer a(backend, 16), b(backend, 16), c(backend, 16);
+  CHECK((matmul::launch<float, false, false>(
+             a.ptr, b.ptr, c.ptr, matmul::MatmulParams{0, 4, 4, 4, 0.f},
+             backend).status == StatusCode::InvalidParameter));
+  CHECK((matmul::launch<float, false, false>(
+             a.ptr, b.ptr, c.ptr, matmul::MatmulParams{1, 4, -1, 4, 0.f},
+             backend).status == StatusCode::InvalidParameter));
+  // test/matmul/matmul_event_dependency.cc: the launch waits for its events
+  hipStream_t other;
+  CHECK(hipStreamCreate(&other) == hipSuccess);
+  {
+    backend::HIPBackend producer(other);
+    const auto x = iota_data(64 * 64, 8);
+    DeviceBuffer d_x(backend, x), d_y(backend, 64 * 64), d_z(backend, 64 * 64);
+    auto first = matmul::launch<float, false, false>(
+        d_x.ptr, d_x.ptr, d_y.ptr, matmul::MatmulParams{1, 64, 64, 64, 0.f},
+        producer);
+    CHECK(first.status == StatusCode::OK);
+    auto second = matmul::launch<float, false, false>(
+        d_y.ptr, d_x.ptr, d_z.ptr, matmul::MatmulParams{1, 64, 64, 64, 0.f},
+        backend, {first.event});
+    CHECK(second.status == StatusCode::OK);
+    second.event.wait_and_throw();
+    std::vector<float> y(64 * 64, 0.f), z(64 * 64, 0.f);
+    oracle_matmul(x.data(), x.data(), y.data(), 1, 64, 64, 64, 0, 0, 0.f, 1);
+    oracle_matmul(y.data(), x.data(), z.data(), 1, 64, 64, 64, 0, 0, 0.f, 1);
+    CHECK(close(d_z.host(), z, true));
+  }
+  (void)hipStreamDestroy(other);
+}
+
 int main() {
   int n = 0;
   if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
@@ -280,6 +357,7 @@ int main() {
     test_depthwise(backend);
     test_pooling(backend);
     test_event_dependencies(backend);
+    test_matmul(backend);
   }
   (void)hipStreamDestroy(stream);
   return report("gpu_api_test");

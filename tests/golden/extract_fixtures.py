@@ -4,7 +4,7 @@
 The reference keeps its expected outputs as literal arrays inside generated
 gtest sources (test/conv2d/forward_window3_stride1.cc:57-67,
 test/depthwise_conv2d/forward_window3_stride1.cc, test/pooling/*_forward.cc,
-test/pooling/*_grad.cc).  Those sources are parsed here AS TEXT -- nothing is
+test/pooling/*_grad.cc, test/matmul/matmul_*.cc).  Those sources are parsed here AS TEXT -- nothing is
 compiled or executed -- and only the data (case shape, padding mode,
 max_input_val and the expected output values) is written to
 tests/golden/<group>.npz.  The operands are never stored: every case
@@ -107,6 +107,53 @@ def write_padding_kat():
     print("%-28s %5d rows" % ("padding_kat", len(rows)))
 
 
+def write_matmul():
+    """test/matmul/matmul_batch{1,3}_beta{0,1}_{lhsT}_{rhsT}.cc (27 cases per
+    file) and matmul_offset.cc.  meta columns: batches, m, k, n, beta,
+    transpose_lhs, transpose_rhs, lhs_offset, rhs_offset, out_offset,
+    max_input_val (0 = no wrap), n_values.  Operands and the initial output
+    are 1,2,...,max_val,1,... (test/matmul/fixture.h:44-46)."""
+    def grab(body, name):
+        m = re.search(r"const (?:int|auto|DataType) " + name +
+                      r" =\s*(?:static_cast<DataType>\()?([\d.]+)", body)
+        return float(m.group(1)) if m else None
+
+    metas, vals = [], []
+    files = []
+    for b in (1, 3):
+        for beta in (0, 1):
+            for tl in ("false", "true"):
+                for tr in ("false", "true"):
+                    files.append(("matmul_batch%d_beta%d_%s_%s.cc" %
+                                  (b, beta, tl, tr), tl == "true",
+                                  tr == "true"))
+    files.append(("matmul_offset.cc", False, False))
+    for fname, tl, tr in files:
+        with open(os.path.join(REF, "test", "matmul", fname)) as f:
+            text = f.read()
+        cases = CASE_RE.findall(text)
+        assert cases, fname
+        for _suite, _name, body in cases:
+            exp = re.search(r"exp(?:_out)? = \{(.*?)\};", body, re.S).group(1)
+            values = np.array(
+                [float(tok) for tok in exp.replace("\n", " ").split(",")
+                 if tok.strip()], dtype=np.float64)
+            row = [grab(body, n) for n in ("batches", "m", "k", "n", "beta")]
+            offs = [grab(body, n) or 0 for n in ("lhs_offset", "rhs_offset",
+                                                 "out_offset")]
+            maxv = grab(body, "max_input_val") or 0
+            metas.append([int(v) for v in row] + [int(tl), int(tr)] +
+                         [int(v) for v in offs] + [int(maxv), values.size])
+            vals.append(values)
+    meta = np.array(metas, dtype=np.int64)
+    values = np.concatenate(vals)
+    assert np.all(values == np.round(values))
+    out = os.path.join(OUT, "matmul.npz")
+    np.savez_compressed(out, meta=meta, values=values)
+    print("%-28s %5d cases %9d values %8d bytes" %
+          ("matmul", len(meta), values.size, os.path.getsize(out)))
+
+
 def main():
     if not os.path.isdir(REF):
         sys.exit("reference tree not found at " + REF)
@@ -131,6 +178,7 @@ def main():
                 "max_window{w}_stride{s}_grad.cc", POOL_GRAD, True)
     write_group("pool_avg_grad", "pooling",
                 "avg_window{w}_stride{s}_grad.cc", POOL_GRAD, False)
+    write_matmul()
 
 
 if __name__ == "__main__":

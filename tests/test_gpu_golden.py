@@ -14,7 +14,7 @@ import pytest
 import torch
 
 import oracle
-from golden_cases import load
+from golden_cases import load, load_matmul
 from portdnn_amd import capi, ops
 from portdnn_amd.capi import ALGO, DIRECTION, POOL_OP
 
@@ -150,3 +150,17 @@ def test_pool_avg_grad_golden():
         assert np.all(np.abs(got.astype(np.float64) - exp) <= tol), case[:9]
         n_run += 1
     assert n_run == 432
+
+
+def test_matmul_golden():
+    """The reference's matmul cases through snn_hip_matmul_f32, offsets into
+    the buffers included (test/matmul/fixture.h:37-76); exact."""
+    for c in load_matmul():
+        lhs = dev(oracle.iota(c.batches * c.m * c.k + c.lhs_offset, c.max_val))
+        rhs = dev(oracle.iota(c.batches * c.k * c.n + c.rhs_offset, c.max_val))
+        out = dev(oracle.iota(c.batches * c.m * c.n + c.out_offset, c.max_val))
+        ops.matmul(lhs[c.lhs_offset:], rhs[c.rhs_offset:], c.batches, c.m, c.k,
+                   c.n, c.trans_lhs, c.trans_rhs, c.beta,
+                   out=out[c.out_offset:])
+        assert np.array_equal(out.cpu().numpy(),
+                              c.expected.astype(np.float32)), c[:11]

@@ -421,13 +421,14 @@ def test_maxpool_nan_rules():
 @pytest.mark.parametrize("trans_b", [False, True])
 @pytest.mark.parametrize("shape", [(1, 64, 64, 64), (3, 37, 29, 53),
                                    (1, 1568, 512, 2048), (2, 130, 7, 258),
-                                   (16, 200, 64, 64)])
+                                   (16, 200, 64, 64), (3, 100, 96, 50),
+                                   (1, 4096, 1024, 1024), (2, 33, 32, 3)])
 def test_matmul(trans_a, trans_b, shape):
     b_, m, k, n = shape
     rng = np.random.default_rng(sum(shape))
     a, b = uniform(rng, b_ * m * k), uniform(rng, b_ * k * n)
     c0 = uniform(rng, b_ * m * n)
-    for beta in (0.0, 1.0):
+    for beta in (0.0, 1.0, -0.5):
         ref = oracle.matmul(a, b, b_, m, k, n, trans_a, trans_b, beta, c=c0)
         got = ops.matmul(dev(a), dev(b), b_, m, k, n, trans_a, trans_b, beta,
                          out=dev(c0).clone()).cpu().numpy()
