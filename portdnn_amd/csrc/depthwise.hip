@@ -11,6 +11,7 @@
 // and the window taps of neighbouring lanes/pixels are served from L1/L2.
 // Everything else goes through the scalar kernel.
 #include <cstdlib>
+#include <type_traits>
 
 #include "gemm_tile.h"
 #include "snn_kernels.h"
@@ -147,7 +148,9 @@ struct BufVec4<_Float16> {
 // it belongs to, so the reuse between adjacent windows happens in registers.
 // Per output the taps are still accumulated in filter-row, filter-column
 // order.
-template <typename T, int STRIDE, int TH, int TW>
+// FLIP reads the filter taps in reverse order: with the output gradient as
+// "input" and padding 2 - pad this is the stride-1 input gradient.
+template <typename T, int STRIDE, int TH, int TW, bool FLIP = false>
 __global__ void __launch_bounds__(256)
     dw_forward_3x3_strip_kernel(const T* __restrict__ in,
                                 const T* __restrict__ fil, T* __restrict__ out,
@@ -180,7 +183,9 @@ __global__ void __launch_bounds__(256)
   float f[9][4];
 #pragma unroll
   for (int t = 0; t < 9; ++t)
-    BufVec4<T>::load(fil_rsrc, static_cast<unsigned>(t * C + c) * sizeof(T),
+    BufVec4<T>::load(fil_rsrc,
+                     static_cast<unsigned>((FLIP ? 8 - t : t) * C + c) *
+                         sizeof(T),
                      f[t]);
   float acc[TH][TW][4];
 #pragma unroll
@@ -320,6 +325,148 @@ __global__ void __launch_bounds__(256)
   dx[idx] = Elem<T>::from_float(acc);
 }
 
+// Input backprop, multiplier == 1, C % 4 == 0, any window / stride: one lane
+// per four channels of a dX pixel; for stride 2 at most two taps per axis
+// reach a pixel.
+template <typename T>
+__global__ void __launch_bounds__(256)
+    dw_input_backprop_vec4_kernel(const T* __restrict__ dy,
+                                  const T* __restrict__ fil,
+                                  T* __restrict__ dx,
+                                  snn_hip_depthwise_params p, unsigned n_vec) {
+  const unsigned idx = gemm::xcd_remap(blockIdx.x, gridDim.x) * 256u +
+                       threadIdx.x;
+  if (idx >= n_vec) return;
+  const int C = p.channels;
+  const unsigned cv = static_cast<unsigned>(C) / 4u;
+  const int c = static_cast<int>(idx % cv) * 4;
+  unsigned pix = idx / cv;
+  const int x = static_cast<int>(pix % static_cast<unsigned>(p.in_cols));
+  pix /= static_cast<unsigned>(p.in_cols);
+  const int y = static_cast<int>(pix % static_cast<unsigned>(p.in_rows));
+  const int n = static_cast<int>(pix / static_cast<unsigned>(p.in_rows));
+  const size_t dy_elems =
+      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * C;
+  const size_t dx_elems =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * C;
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, dy_elems * sizeof(T));
+  const __amdgpu_buffer_rsrc_t fil_rsrc = make_rsrc(
+      fil, static_cast<size_t>(p.window_rows) * p.window_cols * C * sizeof(T));
+  const __amdgpu_buffer_rsrc_t dx_rsrc = make_rsrc(dx, dx_elems * sizeof(T));
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  // first tap row / column whose offset from (y + pad) is a multiple of the
+  // stride
+  const int ty0 = y + p.pad_rows, tx0 = x + p.pad_cols;
+  for (int r = ty0 % p.stride_rows; r < p.window_rows; r += p.stride_rows) {
+    const int oy = (ty0 - r) / p.stride_rows;
+    if (ty0 - r < 0 || oy >= p.out_rows) continue;
+    for (int sc = tx0 % p.stride_cols; sc < p.window_cols;
+         sc += p.stride_cols) {
+      const int ox = (tx0 - sc) / p.stride_cols;
+      if (tx0 - sc < 0 || ox >= p.out_cols) continue;
+      float g[4], f[4];
+      BufVec4<T>::load(
+          dy_rsrc,
+          static_cast<unsigned>(((n * p.out_rows + oy) * p.out_cols + ox) * C +
+                                c) * sizeof(T),
+          g);
+      BufVec4<T>::load(
+          fil_rsrc,
+          static_cast<unsigned>((r * p.window_cols + sc) * C + c) * sizeof(T),
+          f);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = fmaf(g[i], f[i], acc[i]);
+    }
+  }
+  BufVec4<T>::store(dx_rsrc, idx * 4u * static_cast<unsigned>(sizeof(T)), acc);
+}
+
+// Filter backprop, 3x3, multiplier == 1, C % 4 == 0.  A work-group covers
+// `cvw` channel vectors x (256 / cvw) pixels at a time and walks a range of
+// output pixels; each lane keeps the 9 x 4 partial sums of its channels, the
+// pixel lanes are then added up through LDS and the result goes to the
+// zero-filled dF with float atomics.  fp32 only (float atomics).
+constexpr int kDwFilbkThreads = 256;
+
+__global__ void __launch_bounds__(kDwFilbkThreads)
+    dw_filter_backprop_3x3_kernel(const float* __restrict__ in,
+                                  const float* __restrict__ dy,
+                                  float* __restrict__ dw,
+                                  snn_hip_depthwise_params p, int cvw,
+                                  int pixels_per_group) {
+  __shared__ float partial[kDwFilbkThreads][37];
+  const int C = p.channels;
+  const int tid = threadIdx.x;
+  const int cl = tid % cvw;          // channel vector inside the group
+  const int pl = tid / cvw;          // pixel lane
+  const int n_pl = kDwFilbkThreads / cvw;
+  const int c = (blockIdx.y * cvw + cl) * 4;
+  const int n_pix = p.batch * p.out_rows * p.out_cols;
+  const int pix_begin = blockIdx.x * pixels_per_group;
+  const int pix_end = min(n_pix, pix_begin + pixels_per_group);
+  const size_t in_elems =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * C;
+  const size_t dy_elems = static_cast<size_t>(n_pix) * C;
+  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_elems * 4);
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, dy_elems * 4);
+  float acc[9][4];
+#pragma unroll
+  for (int t = 0; t < 9; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[t][i] = 0.f;
+  if (c < C) {
+    for (int pix = pix_begin + pl; pix < pix_end; pix += n_pl) {
+      const int ox = pix % p.out_cols;
+      const int t2 = pix / p.out_cols;
+      const int oy = t2 % p.out_rows;
+      const int n = t2 / p.out_rows;
+      const int y0 = oy * p.stride_rows - p.pad_rows;
+      const int x0 = ox * p.stride_cols - p.pad_cols;
+      float g[4];
+      BufVec4<float>::load(dy_rsrc, static_cast<unsigned>(pix * C + c) * 4u, g);
+      const int base = ((n * p.in_rows + y0) * p.in_cols + x0) * C + c;
+#pragma unroll
+      for (int r = 0; r < 3; ++r) {
+        const bool row_ok =
+            static_cast<unsigned>(y0 + r) < static_cast<unsigned>(p.in_rows);
+#pragma unroll
+        for (int sc = 0; sc < 3; ++sc) {
+          const bool ok = row_ok & (static_cast<unsigned>(x0 + sc) <
+                                    static_cast<unsigned>(p.in_cols));
+          float xv[4];
+          BufVec4<float>::load(
+              in_rsrc,
+              ok ? static_cast<unsigned>(base + (r * p.in_cols + sc) * C) * 4u
+                 : kOobOffset,
+              xv);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            acc[r * 3 + sc][i] = fmaf(xv[i], g[i], acc[r * 3 + sc][i]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < 9; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) partial[tid][t * 4 + i] = acc[t][i];
+  __syncthreads();
+  // lane e of the first cvw * 36 adds up one (channel vector, tap, component)
+  for (int e = tid; e < cvw * 36; e += kDwFilbkThreads) {
+    const int ecl = e % cvw, comp = e / cvw;  // comp = tap * 4 + i
+    float sum = 0.f;
+    for (int q = 0; q < n_pl; ++q) sum += partial[q * cvw + ecl][comp];
+    const int ch = (blockIdx.y * cvw + ecl) * 4 + (comp & 3);
+    if (ch < C) atomicAdd(dw + (comp >> 2) * C + ch, sum);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+    dw_zero_kernel(float* __restrict__ p, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0.f;
+}
+
 constexpr int kStrip = 64;   // (channel, multiplier) pairs per work-group
 constexpr int kSlices = 4;   // waves splitting the batch*rows*cols reduction
 
@@ -429,16 +576,87 @@ int launch_depthwise(int direction, const T* input, const T* filter, T* output,
   } else if (direction == SNN_HIP_INPUT_BACKPROP) {
     const size_t n_out =
         static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
+    const bool vec_ok =
+        p.channel_multiplier == 1 && p.channels % 4 == 0 &&
+        n_out * sizeof(T) < 0x7FFFFFF0u &&
+        static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * p.channels *
+                sizeof(T) < 0x7FFFFFF0u;
+    if (vec_ok && p.window_rows == 3 && p.window_cols == 3 &&
+        p.stride_rows == 1 && p.stride_cols == 1 && p.pad_rows <= 2 &&
+        p.pad_cols <= 2) {
+      // stride 1: the forward strip kernel on dY with the taps reversed
+      snn_hip_depthwise_params q = p;
+      q.in_rows = p.out_rows;  q.in_cols = p.out_cols;
+      q.out_rows = p.in_rows;  q.out_cols = p.in_cols;
+      q.pad_rows = 2 - p.pad_rows;
+      q.pad_cols = 2 - p.pad_cols;
+      constexpr int kTw = 1;
+      const size_t per_row = static_cast<size_t>(q.batch) * q.out_cols *
+                             (q.channels / 4);
+      int th = 8;
+      while (th > 1 && per_row * ceil_div(q.out_rows, th) < 150000) th /= 2;
+      const int n_strips = ceil_div(q.out_rows, th);
+      const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
+      const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
+#define SNN_DW_STRIP_BK(TH)                                                   \
+  hipLaunchKernelGGL((dw_forward_3x3_strip_kernel<T, 1, TH, kTw, true>), grid, \
+                     dim3(kBlock), 0, stream, input, filter, output, q,       \
+                     n_strips, q.out_cols, n_items)
+      if (th == 8) SNN_DW_STRIP_BK(8);
+      else if (th == 4) SNN_DW_STRIP_BK(4);
+      else if (th == 2) SNN_DW_STRIP_BK(2);
+      else SNN_DW_STRIP_BK(1);
+#undef SNN_DW_STRIP_BK
+    } else if (vec_ok) {
+      const unsigned n_vec = static_cast<unsigned>(n_out / 4);
+      hipLaunchKernelGGL(dw_input_backprop_vec4_kernel<T>,
+                         dim3(ceil_div(n_vec, static_cast<unsigned>(kBlock))),
+                         dim3(kBlock), 0, stream, input, filter, output, p,
+                         n_vec);
+    } else
     hipLaunchKernelGGL(dw_input_backprop_kernel<T>,
                        dim3(static_cast<unsigned>(ceil_div(n_out, size_t{kBlock}))),
                        dim3(kBlock), 0, stream, input, filter, output, p,
                        n_out);
   } else {
-    const dim3 grid(static_cast<unsigned>(p.window_rows * p.window_cols),
-                    static_cast<unsigned>(ceil_div(CM, size_t{kStrip})));
-    hipLaunchKernelGGL(dw_filter_backprop_kernel<T>, grid,
-                       dim3(kStrip * kSlices), 0, stream, input, filter,
-                       output, p);
+    const size_t n_pix_sz =
+        static_cast<size_t>(p.batch) * p.out_rows * p.out_cols;
+    bool done = false;
+    if constexpr (std::is_same<T, float>::value) {
+      if (p.channel_multiplier == 1 && p.channels % 4 == 0 &&
+          p.window_rows == 3 && p.window_cols == 3 &&
+          n_pix_sz * p.channels * sizeof(T) < 0x7FFFFFF0u &&
+          static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels *
+                  sizeof(T) < 0x7FFFFFF0u) {
+        const int cv = p.channels / 4;
+        int cvw = 1;
+        while (cvw * 2 <= cv && cvw < 32) cvw *= 2;  // >= 8 pixel lanes
+        const int n_pl = kDwFilbkThreads / cvw;
+        const int grid_y = ceil_div(cv, cvw);
+        const int n_pix = static_cast<int>(n_pix_sz);
+        // about 1024 work-groups (every one ends with cvw * 36 atomics), each
+        // at least 8 passes over its pixel lanes
+        int ppg = max(n_pl * 8, ceil_div(n_pix, max(1, 1024 / grid_y)));
+        ppg = ceil_div(ppg, n_pl) * n_pl;
+        const int grid_x = ceil_div(n_pix, ppg);
+        const int dw_elems = 9 * p.channels;
+        hipLaunchKernelGGL(dw_zero_kernel, dim3(ceil_div(dw_elems, 256)),
+                           dim3(256), 0, stream, output, dw_elems);
+        hipLaunchKernelGGL(dw_filter_backprop_3x3_kernel,
+                           dim3(static_cast<unsigned>(grid_x),
+                                static_cast<unsigned>(grid_y)),
+                           dim3(kDwFilbkThreads), 0, stream, input, filter,
+                           output, p, cvw, ppg);
+        done = true;
+      }
+    }
+    if (!done) {
+      const dim3 grid(static_cast<unsigned>(p.window_rows * p.window_cols),
+                      static_cast<unsigned>(ceil_div(CM, size_t{kStrip})));
+      hipLaunchKernelGGL(dw_filter_backprop_kernel<T>, grid,
+                         dim3(kStrip * kSlices), 0, stream, input, filter,
+                         output, p);
+    }
   }
   SNN_HIP_CHECK_LAUNCH();
   return SNN_HIP_OK;
