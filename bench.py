@@ -258,6 +258,69 @@ def main():
             del xs, ys
         detail["memory_bound"] = mem
 
+        # gradients of the memory-bound operators (same byte accounting:
+        # every operand read or written once)
+        grads = []
+        for size, ch, stride in MOBILENET[:4]:
+            p = ops.depthwise_params(BATCH, size, size, ch, 1, 3, stride, True)
+            for direction, tag in ((DIRECTION.INPUT_BACKPROP, "input_backprop"),
+                                   (DIRECTION.FILTER_BACKPROP,
+                                    "filter_backprop")):
+                n_a, n_b, n_o = ops.depthwise_sizes(p, direction)
+                nbytes = 4 * (n_a + n_b + n_o)
+                sets = rotate_sets(nbytes)
+                a_s = [normal(n_a) for _ in range(sets)]
+                b_s = ([normal(n_b) for _ in range(sets)]
+                       if direction == DIRECTION.FILTER_BACKPROP
+                       else [normal(n_b)] * sets)
+                o_s = [torch.empty(n_o, device="cuda") for _ in range(sets)]
+                state = {"i": 0}
+
+                def run():
+                    i = state["i"] % sets
+                    state["i"] += 1
+                    ops.depthwise_conv2d(a_s[i], b_s[i], p, direction,
+                                         out=o_s[i])
+                ms = event_time_ms(run, reps=5 * sets, warm=sets, repeats=3)
+                gbs = nbytes / ms / 1e6
+                grads.append({"op": "depthwise3x3_%dx%dx%d_s%d_%s" % (
+                    size, size, ch, stride, tag), "bytes": nbytes,
+                    "ms": round(ms, 5), "gbs": round(gbs, 1),
+                    "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)})
+                del a_s, b_s, o_s
+        p = ops.pool_params(BATCH, 112, 112, 64, 3, 2, True)
+        n_in = p.batch * p.in_rows * p.in_cols * p.channels
+        n_out = p.batch * p.out_rows * p.out_cols * p.channels
+        sets = rotate_sets(4 * (2 * n_in + 2 * n_out))
+        xs = [normal(n_in) for _ in range(sets)]
+        ys = [ops.pooling_forward(x, p, POOL_OP.MAX) for x in xs]
+        dys = [normal(n_out) for _ in range(sets)]
+        state = {"i": 0}
+
+        def run_max_grad():
+            i = state["i"] % sets
+            state["i"] += 1
+            ops.pooling_max_grad(xs[i], ys[i], dys[i], p)
+        ms = event_time_ms(run_max_grad, reps=3 * sets, warm=sets, repeats=3)
+        nbytes = 4 * (2 * n_in + 2 * n_out)
+        grads.append({"op": "maxpool3x3_s2_112x112x64_grad", "bytes": nbytes,
+                      "ms": round(ms, 5), "gbs": round(nbytes / ms / 1e6, 1),
+                      "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS,
+                                             4)})
+
+        def run_avg_grad():
+            i = state["i"] % sets
+            state["i"] += 1
+            ops.pooling_avg_grad(dys[i], p)
+        ms = event_time_ms(run_avg_grad, reps=3 * sets, warm=sets, repeats=3)
+        nbytes = 4 * (n_in + n_out)
+        grads.append({"op": "avgpool3x3_s2_112x112x64_grad", "bytes": nbytes,
+                      "ms": round(ms, 5), "gbs": round(nbytes / ms / 1e6, 1),
+                      "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS,
+                                             4)})
+        del xs, ys, dys
+        detail["memory_bound_gradients"] = grads
+
         # the public matmul op (sycldnn::matmul::launch) on the same MFMA kernel
         mm = []
         for batches, m, k, n, tb in ((1, 4096, 1024, 1024, False),

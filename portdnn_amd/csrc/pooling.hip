@@ -350,21 +350,44 @@ __device__ inline bool pool_equal(float a, float b, bool nan_mode) {
 // covers this element and whose value equals it, the gradient is taken only if
 // no earlier element of that window (row-major) also equals the output -- the
 // first maximum wins (src/pooling/kernels.h:141-239).
+template <int VEC>
+struct GradVec;
+template <>
+struct GradVec<1> {
+  __device__ static void load(const float* p, float (&v)[1]) { v[0] = *p; }
+  __device__ static void store(float* p, const float (&v)[1]) { *p = v[0]; }
+};
+template <>
+struct GradVec<4> {
+  __device__ static void load(const float* p, float (&v)[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+  __device__ static void store(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+
+// VEC channels per lane (4 when the channel count and the pointers allow
+// 16-byte accesses).
+template <int VEC>
 __global__ void __launch_bounds__(256)
     pool_max_grad_kernel(const float* __restrict__ in,
                          const float* __restrict__ out,
                          const float* __restrict__ dy, float* __restrict__ dx,
-                         snn_hip_pooling_params p, bool nan_mode, size_t n_in) {
+                         snn_hip_pooling_params p, bool nan_mode, size_t n_vec) {
   const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (idx >= n_in) return;
+  if (idx >= n_vec) return;
   const int C = p.channels;
-  const int ch = static_cast<int>(idx % C);
-  size_t pix = idx / C;
+  const int cv = C / VEC;
+  const int ch = static_cast<int>(idx % cv) * VEC;
+  size_t pix = idx / cv;
   const int x = static_cast<int>(pix % p.in_cols);
   pix /= p.in_cols;
   const int y = static_cast<int>(pix % p.in_rows);
   const int n = static_cast<int>(pix / p.in_rows);
-  const float mine = in[idx];
+  float mine[VEC];
+  GradVec<VEC>::load(in + idx * VEC, mine);
   const float* in_n =
       in + static_cast<size_t>(n) * p.in_rows * p.in_cols * C + ch;
   const size_t out_base =
@@ -377,7 +400,9 @@ __global__ void __launch_bounds__(256)
   const int ox_begin =
       px < p.window_cols ? 0 : (px - p.window_cols) / p.stride_cols + 1;
   const int ox_end = min(px / p.stride_cols + 1, p.out_cols);
-  float grad = 0.f;
+  float grad[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) grad[i] = 0.f;
   for (int oy = oy_begin; oy < oy_end; ++oy) {
     int r0 = oy * p.stride_rows - p.pad_rows;
     const int r1 = min(r0 + p.window_rows, p.in_rows);
@@ -387,38 +412,60 @@ __global__ void __launch_bounds__(256)
       const int c1 = min(c0 + p.window_cols, p.in_cols);
       c0 = max(c0, 0);
       const size_t o = out_base + (static_cast<size_t>(oy) * p.out_cols + ox) * C;
-      const float target = out[o];
-      if (!pool_equal(mine, target, nan_mode)) continue;
-      bool first = true;
-      for (int r = r0; r < r1 && first; ++r) {
+      float target[VEC];
+      GradVec<VEC>::load(out + o, target);
+      // components of this lane that equal the window's maximum and have not
+      // yet been ruled out by an earlier equal element
+      bool live[VEC];
+      bool any = false;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        live[i] = pool_equal(mine[i], target[i], nan_mode);
+        any |= live[i];
+      }
+      if (!any) continue;
+      bool reached = false;
+      for (int r = r0; r < r1 && any && !reached; ++r) {
         for (int col = c0; col < c1; ++col) {
           if (r == y && col == x) {
-            r = r1;  // reached this element: nothing earlier matched
+            reached = true;  // nothing earlier matched for the live components
             break;
           }
-          if (pool_equal(in_n[(static_cast<size_t>(r) * p.in_cols + col) * C],
-                         target, nan_mode)) {
-            first = false;
-            break;
+          float v[VEC];
+          GradVec<VEC>::load(
+              in_n + (static_cast<size_t>(r) * p.in_cols + col) * C, v);
+          any = false;
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) {
+            live[i] = live[i] && !pool_equal(v[i], target[i], nan_mode);
+            any |= live[i];
           }
+          if (!any) break;
         }
       }
-      if (first) grad += dy[o];
+      if (!any) continue;
+      float g[VEC];
+      GradVec<VEC>::load(dy + o, g);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i)
+        if (live[i]) grad[i] += g[i];
     }
   }
-  dx[idx] = grad;
+  GradVec<VEC>::store(dx + idx * VEC, grad);
 }
 
 // Average gradient: every covering output contributes dY / clipped window
 // size (src/pooling/kernels.h:291-414).
+template <int VEC>
 __global__ void __launch_bounds__(256)
     pool_avg_grad_kernel(const float* __restrict__ dy, float* __restrict__ dx,
-                         snn_hip_pooling_params p, size_t n_in) {
+                         snn_hip_pooling_params p, size_t n_vec) {
   const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (idx >= n_in) return;
+  if (idx >= n_vec) return;
   const int C = p.channels;
-  const int ch = static_cast<int>(idx % C);
-  size_t pix = idx / C;
+  const int cv = C / VEC;
+  const int ch = static_cast<int>(idx % cv) * VEC;
+  size_t pix = idx / cv;
   const int x = static_cast<int>(pix % p.in_cols);
   pix /= p.in_cols;
   const int y = static_cast<int>(pix % p.in_rows);
@@ -432,7 +479,9 @@ __global__ void __launch_bounds__(256)
   const int ox_begin =
       px < p.window_cols ? 0 : (px - p.window_cols) / p.stride_cols + 1;
   const int ox_end = min(px / p.stride_cols + 1, p.out_cols);
-  float grad = 0.f;
+  float grad[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) grad[i] = 0.f;
   for (int oy = oy_begin; oy < oy_end; ++oy) {
     int r0 = oy * p.stride_rows - p.pad_rows;
     const int r1 = min(r0 + p.window_rows, p.in_rows);
@@ -442,11 +491,14 @@ __global__ void __launch_bounds__(256)
       const int c1 = min(c0 + p.window_cols, p.in_cols);
       c0 = max(c0, 0);
       const float count = static_cast<float>((r1 - r0) * (c1 - c0));
-      grad += dy[out_base + (static_cast<size_t>(oy) * p.out_cols + ox) * C] /
-              count;
+      float g[VEC];
+      GradVec<VEC>::load(
+          dy + out_base + (static_cast<size_t>(oy) * p.out_cols + ox) * C, g);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) grad[i] += g[i] / count;
     }
   }
-  dx[idx] = grad;
+  GradVec<VEC>::store(dx + idx * VEC, grad);
 }
 
 template <typename T, typename Op>
@@ -538,6 +590,10 @@ template int launch_pooling_forward<_Float16>(const _Float16*, _Float16*,
                                               const snn_hip_pooling_params&,
                                               int, hipStream_t);
 
+static inline bool grad_aligned16(const void* ptr) {
+  return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0;
+}
+
 int launch_pooling_max_grad(const float* input_data, const float* output_data,
                             const float* input_backprop,
                             float* output_backprop,
@@ -546,11 +602,21 @@ int launch_pooling_max_grad(const float* input_data, const float* output_data,
   constexpr int kBlock = 256;
   const size_t n_in =
       static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
-  hipLaunchKernelGGL(pool_max_grad_kernel,
-                     dim3(static_cast<unsigned>(ceil_div(n_in, size_t{kBlock}))),
-                     dim3(kBlock), 0, stream, input_data, output_data,
-                     input_backprop, output_backprop, p,
-                     op == SNN_HIP_POOL_MAX_WITH_NAN, n_in);
+  const bool nan_mode = op == SNN_HIP_POOL_MAX_WITH_NAN;
+  if (p.channels % 4 == 0 && grad_aligned16(input_data) &&
+      grad_aligned16(output_data) && grad_aligned16(input_backprop) &&
+      grad_aligned16(output_backprop)) {
+    const size_t n_vec = n_in / 4;
+    hipLaunchKernelGGL(pool_max_grad_kernel<4>,
+                       dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{kBlock}))),
+                       dim3(kBlock), 0, stream, input_data, output_data,
+                       input_backprop, output_backprop, p, nan_mode, n_vec);
+  } else {
+    hipLaunchKernelGGL(pool_max_grad_kernel<1>,
+                       dim3(static_cast<unsigned>(ceil_div(n_in, size_t{kBlock}))),
+                       dim3(kBlock), 0, stream, input_data, output_data,
+                       input_backprop, output_backprop, p, nan_mode, n_in);
+  }
   SNN_HIP_CHECK_LAUNCH();
   return SNN_HIP_OK;
 }
@@ -562,10 +628,19 @@ int launch_pooling_avg_grad(const float* input_backprop,
   constexpr int kBlock = 256;
   const size_t n_in =
       static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
-  hipLaunchKernelGGL(pool_avg_grad_kernel,
-                     dim3(static_cast<unsigned>(ceil_div(n_in, size_t{kBlock}))),
-                     dim3(kBlock), 0, stream, input_backprop, output_backprop,
-                     p, n_in);
+  if (p.channels % 4 == 0 && grad_aligned16(input_backprop) &&
+      grad_aligned16(output_backprop)) {
+    const size_t n_vec = n_in / 4;
+    hipLaunchKernelGGL(pool_avg_grad_kernel<4>,
+                       dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{kBlock}))),
+                       dim3(kBlock), 0, stream, input_backprop,
+                       output_backprop, p, n_vec);
+  } else {
+    hipLaunchKernelGGL(pool_avg_grad_kernel<1>,
+                       dim3(static_cast<unsigned>(ceil_div(n_in, size_t{kBlock}))),
+                       dim3(kBlock), 0, stream, input_backprop,
+                       output_backprop, p, n_in);
+  }
   SNN_HIP_CHECK_LAUNCH();
   return SNN_HIP_OK;
 }
