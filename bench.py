@@ -203,6 +203,81 @@ def main():
                 del ws
         detail["algorithms"] = algo_table
 
+        # backprops of the 3x3 layers and the 7x7 s2 stem in all directions
+        # (flops as the reference's benchmarks count them: by input pixels
+        # for the two gradients)
+        bk = []
+        stem = ops.conv_params(BATCH, 224, 224, 3, 64, 7, 2, True)
+        cases = [("stem7x7_s2_224x224x3_k64", stem, d) for d in (
+            DIRECTION.FORWARD, DIRECTION.INPUT_BACKPROP,
+            DIRECTION.FILTER_BACKPROP)]
+        for w in work[:4]:
+            cases += [(w["name"], w["p"], DIRECTION.INPUT_BACKPROP),
+                      (w["name"], w["p"], DIRECTION.FILTER_BACKPROP)]
+        dir_names = {DIRECTION.FORWARD: "forward",
+                     DIRECTION.INPUT_BACKPROP: "input_backprop",
+                     DIRECTION.FILTER_BACKPROP: "filter_backprop"}
+        for name, p, direction in cases:
+            algo = capi.lib().snn_hip_conv2d_default_algorithm(
+                ctypes.byref(p), direction)
+            n_a, n_b, n_o = ops.conv_sizes(p, direction)
+            _, ws_elems = ops.workspace_size(p, direction, algo)
+            a, b = uniform(n_a), uniform(n_b)
+            o = torch.empty(n_o, device="cuda")
+            ws = torch.empty(ws_elems, device="cuda") if ws_elems else None
+            ms = event_time_ms(lambda: ops.conv2d(
+                a, b, p, direction, algo, workspace=ws, out=o), reps=10,
+                warm=2, repeats=3)
+            fl = ops.conv_flops(p, direction)
+            bk.append({"layer": name, "direction": dir_names[direction],
+                       "algorithm": algo_names[algo], "ms": round(ms, 4),
+                       "tflops": round(fl / ms / 1e9, 2)})
+            del a, b, o, ws
+        detail["backprop_and_stem"] = bk
+
+        # half precision (fp32 accumulation), batch 128
+        h = []
+        for size, ch in RESNET:
+            for window, feats in ((3, ch), (1, 4 * ch)):
+                p = ops.conv_params(128, size, size, ch, feats, window, 1,
+                                    window == 3)
+                n_a, n_b, n_o = ops.conv_sizes(p, DIRECTION.FORWARD)
+                a, b = uniform(n_a).half(), uniform(n_b).half()
+                o = torch.empty(n_o, device="cuda", dtype=torch.float16)
+                ws = torch.empty(n_b, device="cuda", dtype=torch.float16)
+                ms = event_time_ms(lambda: ops.conv2d(
+                    a, b, p, DIRECTION.FORWARD, ALGO.IM2COL, workspace=ws,
+                    out=o), reps=10, warm=2, repeats=3)
+                fl = ops.conv_flops(p, DIRECTION.FORWARD)
+                h.append({"op": "conv%dx%d_%dx%dx%d_k%d_b128_f16" % (
+                    window, window, size, size, ch, feats), "ms": round(ms, 4),
+                    "tflops": round(fl / ms / 1e9, 1),
+                    "frac_f16_mfma_peak": round(fl / ms / 1e9 / 2500.0, 4)})
+                del a, b, o, ws
+        for size, ch, stride in MOBILENET:
+            p = ops.depthwise_params(128, size, size, ch, 1, 3, stride, True)
+            n_a, n_b, n_o = ops.depthwise_sizes(p, DIRECTION.FORWARD)
+            nbytes = 2 * (n_a + n_b + n_o)
+            sets = max(3, int(600e6 // nbytes) + 1)
+            xs = [normal(n_a).half() for _ in range(sets)]
+            ys = [torch.empty(n_o, device="cuda", dtype=torch.float16)
+                  for _ in range(sets)]
+            f = normal(n_b).half()
+            state = {"i": 0}
+
+            def run_h():
+                i = state["i"] % sets
+                state["i"] += 1
+                ops.depthwise_conv2d(xs[i], f, p, out=ys[i])
+            ms = event_time_ms(run_h, reps=5 * sets, warm=sets, repeats=3)
+            gbs = nbytes / ms / 1e6
+            h.append({"op": "depthwise3x3_%dx%dx%d_s%d_b128_f16" % (
+                size, size, ch, stride), "bytes": nbytes, "ms": round(ms, 5),
+                "gbs": round(gbs, 1),
+                "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)})
+            del xs, ys
+        detail["f16_batch128"] = h
+
         # memory-bound operators: rotate buffer sets so that the 256 MB
         # last-level cache cannot hold the working set between launches
         mem = []
