@@ -142,6 +142,30 @@ struct BufVec4<_Float16> {
   }
 };
 
+// V channels per lane: 4 (16 bytes of fp32, 8 bytes of f16) or, for f16, 8
+// (16 bytes).
+template <typename T, int V>
+struct BufVecN : BufVec4<T> {};
+template <>
+struct BufVecN<_Float16, 8> {
+  typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+  __device__ static void load(__amdgpu_buffer_rsrc_t r, unsigned off,
+                              float (&v)[8]) {
+    const half8 t = __builtin_bit_cast(
+        half8, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0));
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = static_cast<float>(t[i]);
+  }
+  __device__ static void store(__amdgpu_buffer_rsrc_t r, unsigned off,
+                               const float (&v)[8]) {
+    half8 t;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t[i] = static_cast<_Float16>(v[i]);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, t), r,
+                                           off, 0, kStoreAux);
+  }
+};
+
 // Forward 3x3, multiplier == 1, four channels per lane, a TH x TW block of
 // outputs per lane.  Every input row of the block is loaded once
 // ((TW - 1) * STRIDE + 3 column taps) and added into each output row / column
@@ -150,7 +174,7 @@ struct BufVec4<_Float16> {
 // order.
 // FLIP reads the filter taps in reverse order: with the output gradient as
 // "input" and padding 2 - pad this is the stride-1 input gradient.
-template <typename T, int STRIDE, int TH, int TW, bool FLIP = false>
+template <typename T, int STRIDE, int TH, int TW, bool FLIP = false, int V = 4>
 __global__ void __launch_bounds__(256)
     dw_forward_3x3_strip_kernel(const T* __restrict__ in,
                                 const T* __restrict__ fil, T* __restrict__ out,
@@ -163,8 +187,8 @@ __global__ void __launch_bounds__(256)
       gemm::xcd_remap(blockIdx.x, gridDim.x) * 256u + threadIdx.x;
   if (idx >= n_items) return;
   const int C = p.channels;
-  const unsigned cv = static_cast<unsigned>(C) / 4u;
-  const int c = static_cast<int>(idx % cv) * 4;
+  const unsigned cv = static_cast<unsigned>(C) / V;
+  const int c = static_cast<int>(idx % cv) * V;
   unsigned rest = idx / cv;
   const int ox0 =
       static_cast<int>(rest % static_cast<unsigned>(n_col_blocks)) * TW;
@@ -180,20 +204,20 @@ __global__ void __launch_bounds__(256)
   const __amdgpu_buffer_rsrc_t fil_rsrc =
       make_rsrc(fil, static_cast<size_t>(9) * C * sizeof(T));
   const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_elems * sizeof(T));
-  float f[9][4];
+  float f[9][V];
 #pragma unroll
   for (int t = 0; t < 9; ++t)
-    BufVec4<T>::load(fil_rsrc,
+    BufVecN<T, V>::load(fil_rsrc,
                      static_cast<unsigned>((FLIP ? 8 - t : t) * C + c) *
                          sizeof(T),
                      f[t]);
-  float acc[TH][TW][4];
+  float acc[TH][TW][V];
 #pragma unroll
   for (int t = 0; t < TH; ++t)
 #pragma unroll
     for (int u = 0; u < TW; ++u)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc[t][u][i] = 0.f;
+      for (int i = 0; i < V; ++i) acc[t][u][i] = 0.f;
   const int x0 = ox0 * STRIDE - p.pad_cols;
   const int y0 = oy0 * STRIDE - p.pad_rows;
   // Element offset of (n, y0, x0, c); it may lie before the tensor on the
@@ -213,14 +237,14 @@ __global__ void __launch_bounds__(256)
   for (int j = 0; j < NR; ++j) {
     const bool row_ok =
         static_cast<unsigned>(y0 + j) < static_cast<unsigned>(p.in_rows);
-    float row[NC][4];
+    float row[NC][V];
 #pragma unroll
     for (int sx = 0; sx < NC; ++sx) {
       const unsigned off =
           (row_ok & col_ok[sx])
               ? static_cast<unsigned>(base + (j * p.in_cols + sx) * C) * kEsz
               : kOobOffset;
-      BufVec4<T>::load(in_rsrc, off, row[sx]);
+      BufVecN<T, V>::load(in_rsrc, off, row[sx]);
     }
 #pragma unroll
     for (int t = 0; t < TH; ++t) {
@@ -231,7 +255,7 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
         for (int sx = 0; sx < 3; ++sx)
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
+          for (int i = 0; i < V; ++i)
             acc[t][u][i] = fmaf(row[u * STRIDE + sx][i], f[r * 3 + sx][i],
                                 acc[t][u][i]);
     }
@@ -245,7 +269,7 @@ __global__ void __launch_bounds__(256)
           (oy0 + t < p.out_rows && ox0 + u < p.out_cols)
               ? static_cast<unsigned>(out_base + (t * p.out_cols + u) * C) * kEsz
               : kOobOffset;
-      BufVec4<T>::store(out_rsrc, off, acc[t][u]);
+      BufVecN<T, V>::store(out_rsrc, off, acc[t][u]);
     }
   }
 }
@@ -514,6 +538,44 @@ __global__ void __launch_bounds__(kStrip* kSlices)
   }
 }
 
+// Launches the 3x3 strip kernel with V channels per lane.  Output rows per
+// lane: as many as still leave every CU a few thousand lanes (measured best:
+// 8 rows x 1 column for the large layers).
+template <typename T, int V, bool FLIP>
+void launch_dw_strip(const T* input, const T* filter, T* output,
+                     const snn_hip_depthwise_params& p, hipStream_t stream) {
+  constexpr int kBlock = 256;
+  constexpr int kTw = 1;
+  const int n_col_blocks = ceil_div(p.out_cols, kTw);
+  const size_t per_row = static_cast<size_t>(p.batch) * n_col_blocks *
+                         (p.channels / V);
+  int th = V == 8 ? 4 : 8;  // 8 rows x 8 channels would need ~250 registers
+  while (th > 1 && per_row * ceil_div(p.out_rows, th) < 150000) th /= 2;
+  // Developer override for tuning runs: SNN_HIP_DW_TH=<1|2|4|8>.
+  static const char* tune = getenv("SNN_HIP_DW_TH");
+  if (tune != nullptr && tune[0] != 0) th = max(1, min(8, atoi(tune)));
+  if (th != 1 && th != 2 && th != 4) th = th >= 8 ? 8 : 4;
+  const int n_strips = ceil_div(p.out_rows, th);
+  const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
+  const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
+#define SNN_DW_STRIP(STRIDE, TH)                                               \
+  hipLaunchKernelGGL((dw_forward_3x3_strip_kernel<T, STRIDE, TH, kTw, FLIP, V>), \
+                     grid, dim3(kBlock), 0, stream, input, filter, output, p,  \
+                     n_strips, n_col_blocks, n_items)
+  if (p.stride_rows == 1) {
+    if (th == 8) SNN_DW_STRIP(1, 8);
+    else if (th == 4) SNN_DW_STRIP(1, 4);
+    else if (th == 2) SNN_DW_STRIP(1, 2);
+    else SNN_DW_STRIP(1, 1);
+  } else {
+    if (th == 8) SNN_DW_STRIP(2, 8);
+    else if (th == 4) SNN_DW_STRIP(2, 4);
+    else if (th == 2) SNN_DW_STRIP(2, 2);
+    else SNN_DW_STRIP(2, 1);
+  }
+#undef SNN_DW_STRIP
+}
+
 }  // namespace
 
 template <typename T>
@@ -530,37 +592,14 @@ int launch_depthwise(int direction, const T* input, const T* filter, T* output,
                        static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
                                p.channels * sizeof(T) < 0x7FFFFFF0u;
     if (p.channel_multiplier == 1 && p.channels % 4 == 0 && is3x3 && small) {
-      // Output rows per lane: as many as still leave every CU a few thousand
-      // lanes (measured best: 8 rows x 1 column for the large layers).
-      constexpr int kTw = 1;
-      const int n_col_blocks = ceil_div(p.out_cols, kTw);
-      const size_t per_row = static_cast<size_t>(p.batch) * n_col_blocks *
-                             (p.channels / 4);
-      int th = 8;
-      while (th > 1 && per_row * ceil_div(p.out_rows, th) < 150000) th /= 2;
-      // Developer override for tuning runs: SNN_HIP_DW_TH=<1|2|4|8>.
-      static const char* tune = getenv("SNN_HIP_DW_TH");
-      if (tune != nullptr && tune[0] != 0) th = max(1, min(8, atoi(tune)));
-      if (th != 1 && th != 2 && th != 4) th = th >= 8 ? 8 : 4;
-      const int n_strips = ceil_div(p.out_rows, th);
-      const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
-      const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
-#define SNN_DW_STRIP(STRIDE, TH)                                              \
-  hipLaunchKernelGGL((dw_forward_3x3_strip_kernel<T, STRIDE, TH, kTw>), grid, \
-                     dim3(kBlock), 0, stream, input, filter, output, p,       \
-                     n_strips, n_col_blocks, n_items)
-      if (p.stride_rows == 1) {
-        if (th == 8) SNN_DW_STRIP(1, 8);
-        else if (th == 4) SNN_DW_STRIP(1, 4);
-        else if (th == 2) SNN_DW_STRIP(1, 2);
-        else SNN_DW_STRIP(1, 1);
-      } else {
-        if (th == 8) SNN_DW_STRIP(2, 8);
-        else if (th == 4) SNN_DW_STRIP(2, 4);
-        else if (th == 2) SNN_DW_STRIP(2, 2);
-        else SNN_DW_STRIP(2, 1);
+      bool wide = false;
+      if constexpr (std::is_same<T, _Float16>::value) {
+        if (p.channels % 8 == 0) {
+          launch_dw_strip<T, 8, false>(input, filter, output, p, stream);
+          wide = true;
+        }
       }
-#undef SNN_DW_STRIP
+      if (!wide) launch_dw_strip<T, 4, false>(input, filter, output, p, stream);
     } else if (p.channel_multiplier == 1 && p.channels % 4 == 0) {
       const size_t n_vec = n_out / 4;
       hipLaunchKernelGGL(dw_forward_vec4_kernel<T>,
@@ -590,23 +629,14 @@ int launch_depthwise(int direction, const T* input, const T* filter, T* output,
       q.out_rows = p.in_rows;  q.out_cols = p.in_cols;
       q.pad_rows = 2 - p.pad_rows;
       q.pad_cols = 2 - p.pad_cols;
-      constexpr int kTw = 1;
-      const size_t per_row = static_cast<size_t>(q.batch) * q.out_cols *
-                             (q.channels / 4);
-      int th = 8;
-      while (th > 1 && per_row * ceil_div(q.out_rows, th) < 150000) th /= 2;
-      const int n_strips = ceil_div(q.out_rows, th);
-      const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
-      const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
-#define SNN_DW_STRIP_BK(TH)                                                   \
-  hipLaunchKernelGGL((dw_forward_3x3_strip_kernel<T, 1, TH, kTw, true>), grid, \
-                     dim3(kBlock), 0, stream, input, filter, output, q,       \
-                     n_strips, q.out_cols, n_items)
-      if (th == 8) SNN_DW_STRIP_BK(8);
-      else if (th == 4) SNN_DW_STRIP_BK(4);
-      else if (th == 2) SNN_DW_STRIP_BK(2);
-      else SNN_DW_STRIP_BK(1);
-#undef SNN_DW_STRIP_BK
+      bool wide = false;
+      if constexpr (std::is_same<T, _Float16>::value) {
+        if (q.channels % 8 == 0) {
+          launch_dw_strip<T, 8, true>(input, filter, output, q, stream);
+          wide = true;
+        }
+      }
+      if (!wide) launch_dw_strip<T, 4, true>(input, filter, output, q, stream);
     } else if (vec_ok) {
       const unsigned n_vec = static_cast<unsigned>(n_out / 4);
       hipLaunchKernelGGL(dw_input_backprop_vec4_kernel<T>,
