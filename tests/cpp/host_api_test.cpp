@@ -15,6 +15,8 @@
 #include <portdnn/depthwise_conv2d/launch.h>
 #include <portdnn/depthwise_conv2d/sizes.h>
 #include <portdnn/helpers/padding.h>
+#include <portdnn/matmul/launch.h>
+#include <portdnn/matmul/params.h>
 #include <portdnn/pooling/launch.h>
 #include <portdnn/pooling/sizes.h>
 
@@ -208,6 +210,16 @@ static void test_status_codes() {
   st = pooling::launch<float, pooling::Max, pooling::Backpropagate>(
       fake, fake, fake, fake, q, backend);
   CHECK(st.status == StatusCode::InvalidParameter);
+
+  // internal/matmul/launch.h:66-70; defaults of matmul/params.h:52
+  matmul::MatmulParams mp{1, 4, 0, 4, 0.f};
+  CHECK(mp.batch_type == sycldnn::BatchFormat::STRIDED);
+  st = matmul::launch<float, false, true>(fake, fake, fake, mp, backend);
+  CHECK(st.status == StatusCode::InvalidParameter);
+  mp.k = 4;
+  mp.batch_type = sycldnn::BatchFormat::INTERLEAVED;
+  st = matmul::launch<float, false, false>(fake, fake, fake, mp, backend);
+  CHECK(st.status == StatusCode::InvalidAlgorithm);
 }
 
 int main() {
