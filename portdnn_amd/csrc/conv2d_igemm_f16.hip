@@ -16,6 +16,8 @@
 // portDNN's half build accumulates in half (e.g. `DataType out_val{0}` with
 // T = cl::sycl::half in src/conv2d/direct/kernels_nhwc.h:92); accumulating in
 // fp32 is more accurate and stays inside the 1e-2 relative bar against it.
+#include <cstdlib>
+
 #include "gemm_tile.h"
 #include "snn_kernels.h"
 
@@ -305,6 +307,13 @@ int launch_conv2d_igemm_f16(const _Float16* input, const _Float16* filter,
       return SNN_HIP_ALLOCATION_PROBLEM;
     wgt_t = static_cast<_Float16*>(ptr);
     temporary = true;
+  }
+  static const bool no_rowtile = getenv("SNN_HIP_F16_IGEMM") != nullptr;
+  if (!no_rowtile && conv2d_rowtile_f16_supports(p)) {
+    const int status =
+        launch_conv2d_rowtile_f16(input, filter, output, p, wgt_t, stream);
+    if (temporary) (void)hipFreeAsync(wgt_t, stream);
+    return status;
   }
   hipLaunchKernelGGL(repack_filter_kernel,
                      dim3(static_cast<unsigned>(ceil_div(wgt_elems, size_t{256}))),

@@ -65,6 +65,15 @@ int launch_conv2d_igemm_f16(const _Float16* input, const _Float16* filter,
                             _Float16* workspace, size_t workspace_elems,
                             hipStream_t stream);
 
+// Half-precision stride-1 forward convolution with the input tile resident
+// in LDS (conv2d_rowtile_f16.hip).  `packed` receives the filter in MFMA
+// operand order: window_rows * window_cols * channels * features halves,
+// 16-byte aligned.
+bool conv2d_rowtile_f16_supports(const snn_hip_conv2d_params& p);
+int launch_conv2d_rowtile_f16(const _Float16* input, const _Float16* filter,
+                              _Float16* output, const snn_hip_conv2d_params& p,
+                              _Float16* packed, hipStream_t stream);
+
 // Depthwise convolution, all three directions (depthwise.hip).
 template <typename T>
 int launch_depthwise(int direction, const T* input, const T* filter, T* output,

@@ -488,10 +488,44 @@ def test_f16_conv_forward_ragged(shape):
         assert_close_f16(got, ref, ("f16 ragged", ALGO_NAME[algo], shape))
 
 
-def test_f16_conv_forward_full_batch_sampled():
-    # Batch 128 takes the 128x128 work-group tile of the f16 kernel.
-    p = ops.conv_params(128, 28, 28, 128, 128, 3, 1, True)
-    rng = np.random.default_rng(760)
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, win_rows, win_cols, same
+    (5, 7, 7, 128, 64, 3, 3, True),      # tiles run over image boundaries
+    (3, 14, 14, 64, 128, 3, 3, True),    # one channel block, two wave rows
+    (2, 28, 28, 192, 192, 3, 3, True),   # three channel blocks, 64-wide slice
+    (3, 12, 10, 128, 128, 5, 5, True),   # 25 taps, pad 2
+    (2, 11, 13, 64, 64, 3, 3, False),    # VALID
+    (2, 9, 20, 128, 256, 1, 3, True),    # 1 x 3 window
+    (2, 20, 9, 128, 64, 3, 1, True),     # 3 x 1 window
+    (7, 5, 5, 256, 320, 1, 1, False),    # 1x1, four channel blocks
+    (1, 6, 200, 64, 64, 3, 3, True),     # rows wider than half a tile
+    (130, 3, 3, 128, 128, 3, 3, True),   # many images per tile
+])
+def test_f16_conv_forward_lds_tile_kernel(shape):
+    batch, rows, cols, ch, feats, wr, wc, same = shape
+    p = ops.add_padding_to(ops.ConvParams(
+        channels=ch, features=feats, batch=batch, in_rows=rows, in_cols=cols,
+        window_rows=wr, window_cols=wc, stride_rows=1, stride_cols=1), same)
+    rng = np.random.default_rng(770 + rows * cols)
+    n_in, n_fil, _ = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x = uniform(rng, n_in).astype(np.float16)
+    w = uniform(rng, n_fil).astype(np.float16)
+    ref = oracle.conv2d_forward(x.astype(np.float32), w.astype(np.float32),
+                                oracle_params(p, feats), acc64=True)
+    got = ops.conv2d(dev(x, torch.float16), dev(w, torch.float16), p,
+                     DIRECTION.FORWARD, ALGO.IM2COL).float().cpu().numpy()
+    assert_close_f16(got, ref, ("f16 lds tile", shape))
+
+
+@pytest.mark.parametrize("size,ch,feats,window", [
+    (28, 128, 128, 3),   # LDS-tile kernel, four channel blocks
+    (56, 64, 64, 3),     # LDS-tile kernel, one channel block
+    (7, 512, 512, 3),    # LDS-tile kernel, 64 x 64 wave tiles
+    (28, 128, 512, 1),   # implicit-GEMM kernel, 128 x 128 work-group tile
+])
+def test_f16_conv_forward_full_batch_sampled(size, ch, feats, window):
+    p = ops.conv_params(128, size, size, ch, feats, window, 1, window == 3)
+    rng = np.random.default_rng(760 + size)
     n_in, n_fil, _ = ops.conv_sizes(p, DIRECTION.FORWARD)
     x = uniform(rng, n_in).astype(np.float16)
     w = uniform(rng, n_fil).astype(np.float16)
@@ -507,7 +541,7 @@ def test_f16_conv_forward_full_batch_sampled():
     ref = sampled_forward_reference(x, w, p, samples)
     flat = ((samples[:, 0] * p.out_rows + samples[:, 1]) * p.out_cols +
             samples[:, 2]) * p.features + samples[:, 3]
-    assert_close_f16(got[flat], ref, "f16 batch 128 sampled")
+    assert_close_f16(got[flat], ref, ("f16 batch 128 sampled", size, window))
 
 
 @pytest.mark.parametrize("size,ch,stride", MOBILENET)
