@@ -112,7 +112,9 @@ constexpr int kWaitVm8 = 0x0F78;
 
 // WF x WP waves: WF feature groups of 64, WP pixel groups of PB * 32.  KC =
 // channels per LDS tile.  MULTI: more than one channel block (two LDS tiles,
-// the next one loading while the current one is multiplied).
+// the next one loading while the current one is multiplied).  WIN3: 3x3
+// window, whose reduction loop is unrolled over a filter row with all tap
+// bookkeeping resolved at compile time.
 //
 // LDS tile: [pixel slot][KC halves], no padding; the 16-byte pieces of a slot
 // are stored at piece position (piece ^ swizzle(slot)), which keeps the
@@ -120,7 +122,7 @@ constexpr int kWaitVm8 = 0x0F78;
 // filled by buffer loads that write LDS directly (64 lanes x 16 bytes = 1 KB
 // of consecutive LDS per instruction), so a whole tile is in flight without
 // holding registers; out-of-range offsets (padding pixels) store zeros.
-template <int WF, int WP, int PB, int KC, bool MULTI>
+template <int WF, int WP, int PB, int KC, bool MULTI, bool WIN3>
 __global__ void __launch_bounds__(64 * WF * WP)
     __attribute__((amdgpu_waves_per_eu(2, 2)))
     conv_rowtile_f16_kernel(const _Float16* __restrict__ src,
@@ -232,12 +234,15 @@ __global__ void __launch_bounds__(64 * WF * WP)
   const unsigned a_voff = static_cast<unsigned>(fb0 * 64 + lane) * 16u;
   const unsigned a_step_bytes = static_cast<unsigned>(n_fb) * 1024u;
   // The reduction runs in units of two MFMA steps (32 channels of one tap).
-  // Filter fragments: three buffers of one unit each in rotation.  Unit u
-  // multiplies out of buffer u % 3 while the buffer unit u - 1 used is
-  // refilled with the fragments of unit u + 2, so a load has two units of
-  // MFMAs to arrive and no register copies wait on it.  Reads past the end of
-  // the packed filter return zeros.
-  half8 a_buf0[2][kFA], a_buf1[2][kFA], a_buf2[2][kFA];
+  // Filter fragments: DEPTH buffers of one unit each in rotation.  Unit u
+  // multiplies out of buffer u % DEPTH while the buffer unit u - 1 used is
+  // refilled with the fragments of unit u + DEPTH - 1, so a load has
+  // DEPTH - 1 units of MFMAs to arrive and no register copies wait on it.
+  // The smaller wave tile has half the MFMAs per unit and registers to
+  // spare: it prefetches twice as far.  Reads past the end of the packed
+  // filter return zeros.
+  constexpr int DEPTH = (PB == 2 && !WIN3) ? 5 : 3;
+  half8 a_buf[DEPTH][2][kFA];
   auto load_a = [&](half8 (&frag)[2][kFA], unsigned first_step) {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks)
@@ -251,8 +256,9 @@ __global__ void __launch_bounds__(64 * WF * WP)
                                a_step_bytes,
                        0, 0));
   };
-  load_a(a_buf0, 0);
-  load_a(a_buf1, 2);
+#pragma unroll
+  for (int d = 0; d + 1 < DEPTH; ++d)
+    load_a(a_buf[d], static_cast<unsigned>(2 * d));
 
   float16v acc[kFA][PB];
 #pragma unroll
@@ -270,21 +276,8 @@ __global__ void __launch_bounds__(64 * WF * WP)
   const int n_chunks = g.channels / KC;
   const int units_per_chunk = taps * UPT;
   const int total_units = n_chunks * units_per_chunk;
-  const unsigned char* cur = bufs;
-  unsigned char* nxt = bufs + buf_bytes;
-  int chunk = 0, tap = 0, tap_r = 0, tap_c = 0, sub = 0;
-  int tap_slots = 0;  // slot offset of the current tap: r * Wh + s
   unsigned step = 0;  // first reduction step of the unit
   half8 b_even[PB], b_odd[PB];  // pixel fragments of even / odd steps
-  // Pixel fragments of reduction step `ks` (0 .. KS-1) of a tap.
-  auto load_b = [&](half8 (&b)[PB], int slots, int ks) {
-#pragma unroll
-    for (int j = 0; j < PB; ++j) {
-      const int slot = b_slot[j] + slots;
-      const int pos = (2 * ks + khalf) ^ swizzle(slot);
-      b[j] = *reinterpret_cast<const half8*>(cur + slot * ROWB + pos * 16);
-    }
-  };
   auto mfma_step = [&](const half8 (&a)[kFA], const half8 (&b)[PB]) {
 #pragma unroll
     for (int i = 0; i < kFA; ++i)
@@ -293,81 +286,178 @@ __global__ void __launch_bounds__(64 * WF * WP)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j],
                                                            acc[i][j], 0, 0, 0);
   };
-  load_b(b_even, 0, 0);
-
-  // One unit.  Pixel fragments of a reduction step are read from LDS while
-  // the MFMAs of the step before run; the loads of the next channel block's
-  // tile start in the first unit of a block.  The scheduling barriers keep
-  // the compiler from sinking these prefetches below the MFMAs that hide
-  // their latency.
-  auto do_unit = [&](half8 (&a_use)[2][kFA], half8 (&a_fill)[2][kFA]) {
-    const int slots = tap_slots;
-    const int ks0 = 2 * sub;
-    const bool tap_ends = sub + 1 == UPT;
-    const bool last = tap_ends && tap + 1 == taps;
-    int next_ks = ks0 + 2;
-    if (tap_ends) {
-      if (++tap_c == g.win_cols) { tap_c = 0; ++tap_r; }
-      // After the last tap the tiles swap and the fragment is read again;
-      // any slot inside the tile will do here.
-      tap_slots = last ? 0 : tap_r * g.halo_cols + tap_c;
-      next_ks = 0;
-    }
-    load_a(a_fill, step + 4);
-    if constexpr (MULTI) {
-      if (tap == 0 && sub == 0 && chunk + 1 < n_chunks) {
-        __builtin_amdgcn_sched_barrier(0);
-        start_tile(nxt, static_cast<unsigned>((chunk + 1) * KC * 2));
+  if constexpr (WIN3) {
+    // Scalar and branch instructions between MFMAs leave the matrix pipe
+    // idle, so this path has none per unit: the loop runs over filter rows
+    // with the three taps of a row (UPT units each) unrolled, which also
+    // keeps the rotation of the three filter buffers static.
+    int cur_off = 0, nxt_off = buf_bytes;
+    // LDS byte offset of this lane's fragment of step 0 of a tap; step ks is
+    // at the same offset with ks * 32 XOR-ed in (the swizzle only permutes
+    // 16-byte pieces inside a slot).
+    auto tap_base = [&](int (&base)[PB], int buf_off, int slots) {
+#pragma unroll
+      for (int j = 0; j < PB; ++j) {
+        const int slot = b_slot[j] + slots;
+        base[j] = buf_off + slot * ROWB + ((khalf ^ swizzle(slot)) << 4);
       }
-    }
-    load_b(b_odd, slots, ks0 + 1);
-    __builtin_amdgcn_sched_barrier(0);
-    mfma_step(a_use[0], b_even);
-    __builtin_amdgcn_sched_barrier(0);
-    load_b(b_even, tap_slots, next_ks);
-    __builtin_amdgcn_sched_barrier(0);
-    mfma_step(a_use[1], b_odd);
-    __builtin_amdgcn_sched_barrier(0);
-    step += 2;
-    if (last) {
+    };
+    auto read_b = [&](half8 (&b)[PB], const int (&base)[PB], int ks) {
+#pragma unroll
+      for (int j = 0; j < PB; ++j)
+        b[j] = *reinterpret_cast<const half8*>(bufs + (base[j] ^ (ks * 32)));
+    };
+    int base[PB];
+    tap_base(base, cur_off, 0);
+    read_b(b_even, base, 0);
+#pragma unroll 1
+    for (int c = 0; c < n_chunks; ++c) {
+#pragma unroll 1
+      for (int r = 0; r < 3; ++r) {
+#pragma unroll
+        for (int sc = 0; sc < 3; ++sc) {
+          // first step of the next tap (after the last tap the tiles swap
+          // and the fragment is read again; slot 0 will do here)
+          const int next_slots =
+              sc < 2 ? r * g.halo_cols + sc + 1
+                     : (r < 2 ? (r + 1) * g.halo_cols : 0);
+#pragma unroll
+          for (int u = 0; u < UPT; ++u) {
+            constexpr int kRot = 3;
+            const int v = sc * UPT + u;  // unit within the filter row
+            half8 (&a_use)[2][kFA] = a_buf[v % kRot];
+            half8 (&a_fill)[2][kFA] = a_buf[(v + 2) % kRot];
+            if constexpr (MULTI) {
+              if (sc == 0 && u == 0) {
+                if (r == 0 && c + 1 < n_chunks)
+                  start_tile(bufs + nxt_off,
+                             static_cast<unsigned>((c + 1) * KC * 2));
+              }
+            }
+            read_b(b_odd, base, 2 * u + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            // Address arithmetic shares a scheduling region with MFMAs so
+            // that it issues in their shadow: the filter prefetch and, in
+            // the last unit of a tap, the next tap's LDS offsets (the
+            // current ones are dead once the odd step's reads are issued).
+            load_a(a_fill, step + 4);
+            step += 2;
+            mfma_step(a_use[0], b_even);
+            if (u + 1 == UPT) tap_base(base, cur_off, next_slots);
+            __builtin_amdgcn_sched_barrier(0);
+            read_b(b_even, base, u + 1 < UPT ? 2 * u + 2 : 0);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_step(a_use[1], b_odd);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+      }
       if constexpr (MULTI) {
-        // End of the channel block.  Vector-memory loads complete in order:
-        // the next tile was issued before the filter loads of all units but
-        // the first, so it has landed once only the last two units' filter
-        // loads (four each) can still be outstanding.
-        if (units_per_chunk >= 3)
-          __builtin_amdgcn_s_waitcnt(kWaitVm8);
-        else if (units_per_chunk == 2)
-          __builtin_amdgcn_s_waitcnt(kWaitVm4);
-        else
-          __builtin_amdgcn_s_waitcnt(kWaitVm0);
+        // End of the channel block; the compiler waits for the LDS-direct
+        // loads of the next tile before the barrier.
         __syncthreads();
-        unsigned char* const t = const_cast<unsigned char*>(cur);
-        cur = nxt;
-        nxt = t;
-        ++chunk;
-        load_b(b_even, 0, 0);
+        const int t = cur_off;
+        cur_off = nxt_off;
+        nxt_off = t;
+        tap_base(base, cur_off, 0);
+        read_b(b_even, base, 0);
       }
-      tap = 0;
-      tap_r = 0;
-      tap_c = 0;
-      sub = 0;
-    } else if (tap_ends) {
-      ++tap;
-      sub = 0;
-    } else {
-      ++sub;
     }
-  };
+  } else {
+    const unsigned char* cur = bufs;
+    unsigned char* nxt = bufs + buf_bytes;
+    int chunk = 0, tap = 0, tap_r = 0, tap_c = 0, sub = 0;
+    int tap_slots = 0;  // slot offset of the current tap: r * Wh + s
+    // Pixel fragments of reduction step `ks` (0 .. KS-1) of a tap.
+    auto load_b = [&](half8 (&b)[PB], int slots, int ks) {
+#pragma unroll
+      for (int j = 0; j < PB; ++j) {
+        const int slot = b_slot[j] + slots;
+        const int pos = (2 * ks + khalf) ^ swizzle(slot);
+        b[j] = *reinterpret_cast<const half8*>(cur + slot * ROWB + pos * 16);
+      }
+    };
+    load_b(b_even, 0, 0);
 
-  int done = 0;
-  for (; done + 3 <= total_units; done += 3) {
-    do_unit(a_buf0, a_buf2);
-    do_unit(a_buf1, a_buf0);
-    do_unit(a_buf2, a_buf1);
+    // One unit.  Pixel fragments of a reduction step are read from LDS while
+    // the MFMAs of the step before run; the loads of the next channel block's
+    // tile start in the first unit of a block.  The scheduling barriers keep
+    // the compiler from sinking these prefetches below the MFMAs that hide
+    // their latency.
+    auto do_unit = [&](half8 (&a_use)[2][kFA], half8 (&a_fill)[2][kFA]) {
+      const int slots = tap_slots;
+      const int ks0 = 2 * sub;
+      const bool tap_ends = sub + 1 == UPT;
+      const bool last = tap_ends && tap + 1 == taps;
+      int next_ks = ks0 + 2;
+      if (tap_ends) {
+        if (++tap_c == g.win_cols) { tap_c = 0; ++tap_r; }
+        // After the last tap the tiles swap and the fragment is read again;
+        // any slot inside the tile will do here.
+        tap_slots = last ? 0 : tap_r * g.halo_cols + tap_c;
+        next_ks = 0;
+      }
+      load_a(a_fill, step + 2 * (DEPTH - 1));
+      if constexpr (MULTI) {
+        if (tap == 0 && sub == 0 && chunk + 1 < n_chunks) {
+          __builtin_amdgcn_sched_barrier(0);
+          start_tile(nxt, static_cast<unsigned>((chunk + 1) * KC * 2));
+        }
+      }
+      load_b(b_odd, slots, ks0 + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_step(a_use[0], b_even);
+      __builtin_amdgcn_sched_barrier(0);
+      load_b(b_even, tap_slots, next_ks);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_step(a_use[1], b_odd);
+      __builtin_amdgcn_sched_barrier(0);
+      step += 2;
+      if (last) {
+        if constexpr (MULTI) {
+          // End of the channel block.  Vector-memory loads complete in order:
+          // the next tile was issued before the filter loads of all units but
+          // the first, so it has landed once only the last two units' filter
+          // loads (four each) can still be outstanding.  (The compiler adds
+          // its own, stricter wait before a barrier that follows LDS-direct
+          // loads.)
+          if (units_per_chunk >= 3)
+            __builtin_amdgcn_s_waitcnt(kWaitVm8);
+          else if (units_per_chunk == 2)
+            __builtin_amdgcn_s_waitcnt(kWaitVm4);
+          else
+            __builtin_amdgcn_s_waitcnt(kWaitVm0);
+          __syncthreads();
+          unsigned char* const t = const_cast<unsigned char*>(cur);
+          cur = nxt;
+          nxt = t;
+          ++chunk;
+          load_b(b_even, 0, 0);
+        }
+        tap = 0;
+        tap_r = 0;
+        tap_c = 0;
+        sub = 0;
+      } else if (tap_ends) {
+        ++tap;
+        sub = 0;
+      } else {
+        ++sub;
+      }
+    };
+
+    int done = 0;
+    for (; done + DEPTH <= total_units; done += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d)
+        do_unit(a_buf[d], a_buf[(d + DEPTH - 1) % DEPTH]);
+    }
+#pragma unroll
+    for (int d = 0; d + 1 < DEPTH; ++d)
+      if (done + d < total_units)
+        do_unit(a_buf[d], a_buf[(d + DEPTH - 1) % DEPTH]);
+
   }
-  if (done < total_units) do_unit(a_buf0, a_buf2);
-  if (done + 1 < total_units) do_unit(a_buf1, a_buf0);
 
   const __amdgpu_buffer_rsrc_t dst_rsrc = make_rsrc(dst, dst_bytes);
   const unsigned row_bytes = static_cast<unsigned>(g.features) * 2u;
@@ -496,7 +586,6 @@ RowTilePlan make_plan(const snn_hip_conv2d_params& p) {
 }
 
 RowTilePlan compute_plan(const snn_hip_conv2d_params& p) {
-  const int taps = p.window_rows * p.window_cols;
   const int kc = p.channels == 64 ? 64 : 32;
   const int wf = p.features % 128 == 0 ? 2 : 1;
   const long pixels = static_cast<long>(p.batch) * p.out_rows * p.out_cols;
@@ -508,11 +597,11 @@ RowTilePlan compute_plan(const snn_hip_conv2d_params& p) {
   return small.lds_bytes != 0 ? small : big;
 }
 
-template <int WF, int WP, int PB, int KC, bool MULTI>
+template <int WF, int WP, int PB, int KC, bool MULTI, bool WIN3>
 void launch_plan(const _Float16* input, const _Float16* wpk, _Float16* output,
                  const snn_hip_conv2d_params& p, const RowTilePlan& plan,
                  size_t wgt_elems, hipStream_t stream) {
-  auto kernel = conv_rowtile_f16_kernel<WF, WP, PB, KC, MULTI>;
+  auto kernel = conv_rowtile_f16_kernel<WF, WP, PB, KC, MULTI, WIN3>;
   static const hipError_t attr = hipFuncSetAttribute(
       reinterpret_cast<const void*>(kernel),
       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
@@ -536,14 +625,17 @@ bool launch_shape(const _Float16* input, const _Float16* wpk,
                   hipStream_t stream) {
   if (plan.wf != WF || plan.wp != WP || plan.pb != PB) return false;
   const bool multi = p.channels > plan.kc;
-#define SNN_ROWTILE_CASE(KC, MULTI)                                           \
-  if (plan.kc == KC && multi == MULTI) {                                      \
-    launch_plan<WF, WP, PB, KC, MULTI>(input, wpk, output, p, plan,           \
-                                       wgt_elems, stream);                    \
+  const bool win3 = p.window_rows == 3 && p.window_cols == 3;
+#define SNN_ROWTILE_CASE(KC, MULTI, WIN3)                                     \
+  if (plan.kc == KC && multi == MULTI && win3 == WIN3) {                      \
+    launch_plan<WF, WP, PB, KC, MULTI, WIN3>(input, wpk, output, p, plan,     \
+                                             wgt_elems, stream);              \
     return true;                                                              \
   }
-  SNN_ROWTILE_CASE(64, false)
-  SNN_ROWTILE_CASE(32, true)
+  SNN_ROWTILE_CASE(64, false, true)
+  SNN_ROWTILE_CASE(32, true, true)
+  SNN_ROWTILE_CASE(64, false, false)
+  SNN_ROWTILE_CASE(32, true, false)
 #undef SNN_ROWTILE_CASE
   return false;
 }
