@@ -333,6 +333,38 @@ def main():
             del xs, ys
         detail["memory_bound"] = mem
 
+        # element-wise operators on the 56x56x256 activation of the first
+        # ResNet stage: ReLU (read + write) and bias add (read + write + bias)
+        from portdnn_amd.capi import BINARY_OP, POINTWISE_OP
+        elem = []
+        dims = [BATCH, 56, 56, 256]
+        n_act = BATCH * 56 * 56 * 256
+        sets = rotate_sets(8 * n_act)
+        xs = [normal(n_act) for _ in range(sets)]
+        ys = [torch.empty(n_act, device="cuda") for _ in range(sets)]
+        bias = normal(256)
+        state = {"i": 0}
+
+        def run_relu():
+            i = state["i"] % sets
+            state["i"] += 1
+            ops.pointwise_forward(xs[i], POINTWISE_OP.RELU, out=ys[i])
+
+        def run_bias():
+            i = state["i"] % sets
+            state["i"] += 1
+            ops.binaryop(xs[i], bias, dims, [256], BINARY_OP.ADD, out=ys[i])
+        for name, fn, nbytes in (("relu_56x56x256", run_relu, 8 * n_act),
+                                 ("bias_add_56x56x256", run_bias,
+                                  8 * n_act + 1024)):
+            ms = event_time_ms(fn, reps=5 * sets, warm=sets, repeats=3)
+            gbs = nbytes / ms / 1e6
+            elem.append({"op": name, "bytes": nbytes, "ms": round(ms, 5),
+                         "gbs": round(gbs, 1),
+                         "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)})
+        del xs, ys
+        detail["elementwise"] = elem
+
         # gradients of the memory-bound operators (same byte accounting:
         # every operand read or written once)
         grads = []

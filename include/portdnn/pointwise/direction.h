@@ -1,0 +1,5 @@
+// portDNN include path kept for source compatibility.
+#ifndef SNN_FWD_POINTWISE_DIRECTION_H
+#define SNN_FWD_POINTWISE_DIRECTION_H
+#include "portdnn/hip/pointwise.h"
+#endif

@@ -262,6 +262,67 @@ SNN_HIP_API int snn_hip_matmul_f32(const float* lhs, const float* rhs,
                                    int n, int transpose_lhs, int transpose_rhs,
                                    float beta, void* stream);
 
+/* ---- pointwise -------------------------------------------------------------
+ * Stand-ins for sycldnn::pointwise::internal::launch_pointwise
+ * (src/pointwise/launch_pointwise_forward.cc, launch_pointwise_grad.cc)
+ * reached from sycldnn::pointwise::launch<T, Op, Direction>
+ * (include/portdnn/pointwise/launch.h:73-100 forward, :120-150 gradient).
+ * `op` is a snn_hip_pointwise_op; n_items must be positive
+ * (include/portdnn/internal/pointwise/launch_internal.h:69). */
+typedef enum snn_hip_pointwise_op {
+  SNN_HIP_POINTWISE_RELU = 0,
+  SNN_HIP_POINTWISE_TANH = 1,
+  SNN_HIP_POINTWISE_EXP = 2,
+  SNN_HIP_POINTWISE_LOG = 3,
+  SNN_HIP_POINTWISE_FLOOR = 4,
+  SNN_HIP_POINTWISE_SQRT = 5
+} snn_hip_pointwise_op;
+SNN_HIP_API int snn_hip_pointwise_forward_f32(const float* input, float* output,
+                                              size_t n_items, int op,
+                                              void* stream);
+SNN_HIP_API int snn_hip_pointwise_forward_f16(const void* input, void* output,
+                                              size_t n_items, int op,
+                                              void* stream);
+/* Gradient: input_forward is what the reference's operators call `val` (the
+ * forward OUTPUT for relu, tanh, exp and sqrt, the forward INPUT for log;
+ * src/pointwise/kernels.h:53-57, :75-77, :100-102, :122-124, :158-160),
+ * input_backprop the incoming error.  Floor has no gradient. */
+SNN_HIP_API int snn_hip_pointwise_grad_f32(const float* input_forward,
+                                           const float* input_backprop,
+                                           float* output_backprop,
+                                           size_t n_items, int op,
+                                           void* stream);
+SNN_HIP_API int snn_hip_pointwise_grad_f16(const void* input_forward,
+                                           const void* input_backprop,
+                                           void* output_backprop,
+                                           size_t n_items, int op,
+                                           void* stream);
+
+/* ---- binaryop --------------------------------------------------------------
+ * Stand-ins for sycldnn::binaryop::internal::launch_binaryop
+ * (src/binaryop/launch_binaryop.cc) reached from
+ * sycldnn::binaryop::launch<T, Op>
+ * (include/portdnn/binaryop/launch.h:61-85).  The dimension lists are
+ * BinaryParams::lhs_dims / rhs_dims (include/portdnn/binaryop/params.h:37-46):
+ * at most four each (none = scalar), right-aligned, a dimension of 1
+ * broadcasts; shapes that do not broadcast return
+ * SNN_HIP_INVALID_PARAMETER
+ * (include/portdnn/internal/binaryop/launch.h:40-62). */
+typedef enum snn_hip_binary_op {
+  SNN_HIP_BINARY_ADD = 0,
+  SNN_HIP_BINARY_SUB = 1,
+  SNN_HIP_BINARY_MUL = 2,
+  SNN_HIP_BINARY_DIV = 3
+} snn_hip_binary_op;
+SNN_HIP_API int snn_hip_binaryop_f32(const float* lhs, const float* rhs,
+                                     float* output, const int* lhs_dims,
+                                     int n_lhs_dims, const int* rhs_dims,
+                                     int n_rhs_dims, int op, void* stream);
+SNN_HIP_API int snn_hip_binaryop_f16(const void* lhs, const void* rhs,
+                                     void* output, const int* lhs_dims,
+                                     int n_lhs_dims, const int* rhs_dims,
+                                     int n_rhs_dims, int op, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

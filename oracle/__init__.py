@@ -57,6 +57,13 @@ def lib():
         L.oracle_pool_avg_grad.argtypes = [_FP, _FP, _PP, ctypes.c_int]
         L.oracle_matmul.argtypes = [_FP, _FP, _FP] + [ctypes.c_int] * 6 + [
             ctypes.c_float, ctypes.c_int]
+        L.oracle_pointwise_forward.argtypes = [ctypes.c_int, _FP, _FP,
+                                               ctypes.c_long]
+        L.oracle_pointwise_grad.argtypes = [ctypes.c_int, _FP, _FP, _FP,
+                                            ctypes.c_long]
+        _IP = ctypes.POINTER(ctypes.c_int)
+        L.oracle_binaryop.argtypes = [ctypes.c_int, _FP, _FP, _FP, _IP,
+                                      ctypes.c_int, _IP, ctypes.c_int]
         L.oracle_set_threads.argtypes = [ctypes.c_int]
         L.oracle_set_threads.restype = ctypes.c_int
     return _lib
@@ -197,3 +204,64 @@ def iota(size, max_val):
     if max_val >= 1:
         idx = idx % int(max_val)
     return (idx + 1).astype(np.float32)
+
+
+POINTWISE_OPS = {"relu": 0, "tanh": 1, "exp": 2, "log": 3, "floor": 4,
+                 "sqrt": 5}
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+
+
+def pointwise_forward(op, x):
+    x, xp = _f(x)
+    out = np.empty_like(x)
+    rc = lib().oracle_pointwise_forward(POINTWISE_OPS[op], xp,
+                                        out.ctypes.data_as(_FP), x.size)
+    assert rc == 0, op
+    return out
+
+
+def pointwise_grad(op, val, err):
+    """`val` is the forward output (the forward input for log)."""
+    val, vp = _f(val)
+    err, ep = _f(err)
+    out = np.empty_like(val)
+    rc = lib().oracle_pointwise_grad(POINTWISE_OPS[op], vp, ep,
+                                     out.ctypes.data_as(_FP), val.size)
+    assert rc == 0, op
+    return out
+
+
+def binaryop_out_dims(lhs_dims, rhs_dims):
+    """include/portdnn/internal/binaryop/launch.h:40-62; None when the shapes
+    do not broadcast."""
+    n = max(len(lhs_dims), len(rhs_dims), 1)
+    l = [1] * (n - len(lhs_dims)) + list(lhs_dims)
+    r = [1] * (n - len(rhs_dims)) + list(rhs_dims)
+    out = []
+    for a, b in zip(l, r):
+        if a != b and a != 1 and b != 1:
+            return None
+        out.append(max(a, b))
+    return out
+
+
+def binaryop(op, lhs, rhs, lhs_dims, rhs_dims):
+    lhs, lp = _f(lhs)
+    rhs, rp = _f(rhs)
+    out_dims = binaryop_out_dims(lhs_dims, rhs_dims)
+    assert out_dims is not None
+    out = np.empty(int(np.prod(out_dims)), dtype=np.float32)
+    ld = (ctypes.c_int * max(len(lhs_dims), 1))(*lhs_dims)
+    rd = (ctypes.c_int * max(len(rhs_dims), 1))(*rhs_dims)
+    rc = lib().oracle_binaryop(BINARY_OPS[op], lp, rp,
+                               out.ctypes.data_as(_FP), ld, len(lhs_dims), rd,
+                               len(rhs_dims))
+    assert rc == 0, (op, lhs_dims, rhs_dims)
+    return out
+
+
+def iota_signed(size):
+    """-ceil(size / 2), ..., size - 1 - ceil(size / 2)
+    (test/gen/iota_initialised_data.h:89-97)."""
+    half = (size + 1) // 2
+    return (np.arange(size, dtype=np.int64) - half).astype(np.float32)

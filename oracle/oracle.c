@@ -289,3 +289,77 @@ int oracle_conv2d_tiled_forward(const float* in, const float* fil, float* out,
   }
   return 0;
 }
+
+/* src/pointwise/kernels.h: Relu<Forward> :47-49 max(val, 0); Tanh :69-71;
+ * Exp :91-93; Log :116-118; Floor :137-139; Sqrt :152-154. */
+int oracle_pointwise_forward(int op, const float* in, float* out, long n) {
+  for (long i = 0; i < n; ++i) {
+    const float v = in[i];
+    switch (op) {
+      case ORACLE_RELU: out[i] = fmaxf(v, 0.0f); break;
+      case ORACLE_TANH: out[i] = tanhf(v); break;
+      case ORACLE_EXP: out[i] = expf(v); break;
+      case ORACLE_LOG: out[i] = logf(v); break;
+      case ORACLE_FLOOR: out[i] = floorf(v); break;
+      case ORACLE_SQRT: out[i] = sqrtf(v); break;
+      default: return 1;
+    }
+  }
+  return 0;
+}
+
+/* src/pointwise/kernels.h: Relu<Gradient> :53-57 select(0, err, val > 0);
+ * Tanh :75-77 (1 - val*val) * err; Exp :100-102 exp(val) + err (as written
+ * there); Log :122-124 (1 / val) * err; Sqrt :158-160 (0.5 / val) * err. */
+int oracle_pointwise_grad(int op, const float* val, const float* err,
+                          float* out, long n) {
+  for (long i = 0; i < n; ++i) {
+    const float v = val[i], e = err[i];
+    switch (op) {
+      case ORACLE_RELU: out[i] = v > 0.0f ? e : 0.0f; break;
+      case ORACLE_TANH: out[i] = (1.0f - v * v) * e; break;
+      case ORACLE_EXP: out[i] = expf(v) + e; break;
+      case ORACLE_LOG: out[i] = (1.0f / v) * e; break;
+      case ORACLE_SQRT: out[i] = (0.5f / v) * e; break;
+      default: return 1;
+    }
+  }
+  return 0;
+}
+
+/* include/portdnn/internal/binaryop/launch.h:40-62 (output shape) and
+ * src/binaryop/kernels.h:86-124 (index arithmetic of the general kernel). */
+int oracle_binaryop(int op, const float* lhs, const float* rhs, float* out,
+                    const int* lhs_dims, int n_lhs, const int* rhs_dims,
+                    int n_rhs) {
+  int l[4] = {1, 1, 1, 1}, r[4] = {1, 1, 1, 1}, o[4];
+  if (n_lhs > 4 || n_rhs > 4 || n_lhs < 0 || n_rhs < 0) return 1;
+  for (int i = 0; i < n_lhs; ++i) l[4 - n_lhs + i] = lhs_dims[i];
+  for (int i = 0; i < n_rhs; ++i) r[4 - n_rhs + i] = rhs_dims[i];
+  for (int i = 0; i < 4; ++i) {
+    if (l[i] < 1 || r[i] < 1) return 1;
+    if (l[i] != r[i] && l[i] != 1 && r[i] != 1) return 1;
+    o[i] = l[i] > r[i] ? l[i] : r[i];
+  }
+  const long total = (long)o[0] * o[1] * o[2] * o[3];
+  for (long idx = 0; idx < total; ++idx) {
+    long rem = idx, li = 0, ri = 0, ls = 1, rs = 1;
+    for (int d = 3; d >= 0; --d) {
+      const long c = d > 0 ? rem % o[d] : rem;
+      if (c < l[d]) li += c * ls;
+      if (c < r[d]) ri += c * rs;
+      ls *= l[d];
+      rs *= r[d];
+      if (d > 0) rem /= o[d];
+    }
+    const float a = lhs[li], b = rhs[ri];
+    switch (op) {
+      case ORACLE_ADD: out[idx] = a + b; break;
+      case ORACLE_SUB: out[idx] = a - b; break;
+      case ORACLE_MUL: out[idx] = a * b; break;
+      case ORACLE_DIV: out[idx] = a / b; break;
+      default: return 1;
+    }
+  }
+  return 0;
+}

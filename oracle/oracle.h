@@ -22,6 +22,12 @@
  *   matmul: textbook definition, checked against numpy float64 matmul for all
  *     transpose/beta combinations.
  *   Winograd transforms: algebraic identity against the direct convolution.
+ *   pointwise (relu, tanh, log, floor, sqrt; forward and gradient) and
+ *     binaryop (add, sub, mul, div with broadcasting): the reference's golden
+ *     vectors of test/pointwise/ *.cc and test/binaryop/ *.cc
+ *     (tests/golden/pointwise.npz, binaryop.npz).  The reference holds no
+ *     vectors for exp: it is pinned against libm's exp (forward) and the
+ *     identity exp(val) + err the reference kernel computes (gradient).
  */
 #ifndef PORTDNN_AMD_ORACLE_H_
 #define PORTDNN_AMD_ORACLE_H_
@@ -93,6 +99,28 @@ void oracle_pool_avg_grad(const float* dy, float* dx, const oracle_params* p,
 void oracle_matmul(const float* a, const float* b, float* c, int batches, int m,
                    int k, int n, int trans_a, int trans_b, float beta,
                    int acc64);
+
+/* Element-wise operators of src/pointwise/kernels.h:36-153. */
+enum {
+  ORACLE_RELU = 0, ORACLE_TANH = 1, ORACLE_EXP = 2, ORACLE_LOG = 3,
+  ORACLE_FLOOR = 4, ORACLE_SQRT = 5
+};
+/* out[i] = op(in[i]).  Returns non-zero for an unknown operator. */
+int oracle_pointwise_forward(int op, const float* in, float* out, long n);
+/* out[i] = op'(val[i], err[i]) with the reference's meaning of `val`: the
+ * forward OUTPUT for relu / tanh / exp / sqrt, the forward INPUT for log
+ * (test/pointwise/pointwise_fixture.h:115-124).  Floor has no gradient. */
+int oracle_pointwise_grad(int op, const float* val, const float* err,
+                          float* out, long n);
+
+/* Broadcasting binary operators of src/binaryop/kernels.h:33-124:
+ * dimensions are right-aligned, missing leading ones are 1, a dimension of 1
+ * broadcasts.  n_lhs, n_rhs <= 4 (0 = scalar).  Returns non-zero when the
+ * shapes do not broadcast. */
+enum { ORACLE_ADD = 0, ORACLE_SUB = 1, ORACLE_MUL = 2, ORACLE_DIV = 3 };
+int oracle_binaryop(int op, const float* lhs, const float* rhs, float* out,
+                    const int* lhs_dims, int n_lhs, const int* rhs_dims,
+                    int n_rhs);
 
 /* Thread count used by the OpenMP loops (<= 0: all cores). Returns the count
  * now in force. */

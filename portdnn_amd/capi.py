@@ -46,6 +46,22 @@ class POOL_OP:
     AVERAGE = 2
 
 
+class POINTWISE_OP:
+    RELU = 0
+    TANH = 1
+    EXP = 2
+    LOG = 3
+    FLOOR = 4
+    SQRT = 5
+
+
+class BINARY_OP:
+    ADD = 0
+    SUB = 1
+    MUL = 2
+    DIV = 3
+
+
 def _struct(name, fields, defaults):
     class S(ctypes.Structure):
         _fields_ = [(f, ctypes.c_int) for f in fields]
@@ -114,6 +130,14 @@ SIGNATURES = {
     "snn_hip_pooling_avg_grad_f32": [_P, _P, _P, _P],
     "snn_hip_matmul_f32": [_P, _P, _P, _I, _I, _I, _I, _I, _I,
                            ctypes.c_float, _P],
+    "snn_hip_pointwise_forward_f32": [_P, _P, _SZ, _I, _P],
+    "snn_hip_pointwise_forward_f16": [_P, _P, _SZ, _I, _P],
+    "snn_hip_pointwise_grad_f32": [_P, _P, _P, _SZ, _I, _P],
+    "snn_hip_pointwise_grad_f16": [_P, _P, _P, _SZ, _I, _P],
+    "snn_hip_binaryop_f32": [_P, _P, _P, ctypes.POINTER(_I), _I,
+                             ctypes.POINTER(_I), _I, _I, _P],
+    "snn_hip_binaryop_f16": [_P, _P, _P, ctypes.POINTER(_I), _I,
+                             ctypes.POINTER(_I), _I, _I, _P],
 }
 
 _lib = None

@@ -632,4 +632,72 @@ int snn_hip_matmul_f32(const float* lhs, const float* rhs, float* output,
                            as_stream(stream));
 }
 
+int snn_hip_pointwise_forward_f32(const float* input, float* output,
+                                  size_t n_items, int op, void* stream) {
+  if (input == nullptr || output == nullptr || n_items == 0)
+    return SNN_HIP_INVALID_PARAMETER;
+  return launch_pointwise_forward_f32(op, input, output, n_items,
+                                      as_stream(stream));
+}
+
+int snn_hip_pointwise_forward_f16(const void* input, void* output,
+                                  size_t n_items, int op, void* stream) {
+  if (input == nullptr || output == nullptr || n_items == 0)
+    return SNN_HIP_INVALID_PARAMETER;
+  return launch_pointwise_forward_f16(
+      op, static_cast<const _Float16*>(input), static_cast<_Float16*>(output),
+      n_items, as_stream(stream));
+}
+
+int snn_hip_pointwise_grad_f32(const float* input_forward,
+                               const float* input_backprop,
+                               float* output_backprop, size_t n_items, int op,
+                               void* stream) {
+  if (input_forward == nullptr || input_backprop == nullptr ||
+      output_backprop == nullptr || n_items == 0)
+    return SNN_HIP_INVALID_PARAMETER;
+  return launch_pointwise_grad_f32(op, input_forward, input_backprop,
+                                   output_backprop, n_items, as_stream(stream));
+}
+
+int snn_hip_pointwise_grad_f16(const void* input_forward,
+                               const void* input_backprop,
+                               void* output_backprop, size_t n_items, int op,
+                               void* stream) {
+  if (input_forward == nullptr || input_backprop == nullptr ||
+      output_backprop == nullptr || n_items == 0)
+    return SNN_HIP_INVALID_PARAMETER;
+  return launch_pointwise_grad_f16(
+      op, static_cast<const _Float16*>(input_forward),
+      static_cast<const _Float16*>(input_backprop),
+      static_cast<_Float16*>(output_backprop), n_items, as_stream(stream));
+}
+
+int snn_hip_binaryop_f32(const float* lhs, const float* rhs, float* output,
+                         const int* lhs_dims, int n_lhs_dims,
+                         const int* rhs_dims, int n_rhs_dims, int op,
+                         void* stream) {
+  if (lhs == nullptr || rhs == nullptr || output == nullptr ||
+      (n_lhs_dims > 0 && lhs_dims == nullptr) ||
+      (n_rhs_dims > 0 && rhs_dims == nullptr))
+    return SNN_HIP_INVALID_PARAMETER;
+  return launch_binaryop_f32(op, lhs, rhs, output, lhs_dims, n_lhs_dims,
+                             rhs_dims, n_rhs_dims, as_stream(stream));
+}
+
+int snn_hip_binaryop_f16(const void* lhs, const void* rhs, void* output,
+                         const int* lhs_dims, int n_lhs_dims,
+                         const int* rhs_dims, int n_rhs_dims, int op,
+                         void* stream) {
+  if (lhs == nullptr || rhs == nullptr || output == nullptr ||
+      (n_lhs_dims > 0 && lhs_dims == nullptr) ||
+      (n_rhs_dims > 0 && rhs_dims == nullptr))
+    return SNN_HIP_INVALID_PARAMETER;
+  return launch_binaryop_f16(op, static_cast<const _Float16*>(lhs),
+                             static_cast<const _Float16*>(rhs),
+                             static_cast<_Float16*>(output), lhs_dims,
+                             n_lhs_dims, rhs_dims, n_rhs_dims,
+                             as_stream(stream));
+}
+
 }  // extern "C"

@@ -99,6 +99,23 @@ int launch_matmul_f32(const float* lhs, const float* rhs, float* output,
                       int batches, int m, int k, int n, bool transpose_lhs,
                       bool transpose_rhs, float beta, hipStream_t stream);
 
+// Element-wise operators (elementwise.hip).  `op` is a snn_hip_pointwise_op
+// or snn_hip_binary_op; operands may alias the output element for element.
+int launch_pointwise_forward_f32(int op, const float* in, float* out, size_t n,
+                                 hipStream_t stream);
+int launch_pointwise_forward_f16(int op, const _Float16* in, _Float16* out,
+                                 size_t n, hipStream_t stream);
+int launch_pointwise_grad_f32(int op, const float* val, const float* err,
+                              float* out, size_t n, hipStream_t stream);
+int launch_pointwise_grad_f16(int op, const _Float16* val, const _Float16* err,
+                              _Float16* out, size_t n, hipStream_t stream);
+int launch_binaryop_f32(int op, const float* lhs, const float* rhs, float* out,
+                        const int* lhs_dims, int n_lhs, const int* rhs_dims,
+                        int n_rhs, hipStream_t stream);
+int launch_binaryop_f16(int op, const _Float16* lhs, const _Float16* rhs,
+                        _Float16* out, const int* lhs_dims, int n_lhs,
+                        const int* rhs_dims, int n_rhs, hipStream_t stream);
+
 }  // namespace snn
 
 #endif  // PORTDNN_AMD_CSRC_SNN_KERNELS_H_

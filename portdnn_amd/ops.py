@@ -8,8 +8,8 @@ import ctypes
 import torch
 
 from . import capi
-from .capi import ALGO, DIRECTION, POOL_OP, STATUS, ConvParams, \
-    DepthwiseParams, PoolParams
+from .capi import ALGO, BINARY_OP, DIRECTION, POINTWISE_OP, POOL_OP, STATUS, \
+    ConvParams, DepthwiseParams, PoolParams
 
 
 def calculate_padding(inp, window, stride, same):
@@ -197,12 +197,61 @@ def matmul(a, b, batches, m, k, n, trans_a=False, trans_b=False, beta=0.0,
     return out
 
 
+def _suffix(t):
+    return "_f32" if t.dtype == torch.float32 else "_f16"
+
+
+def pointwise_forward(x, op, out=None):
+    """sycldnn::pointwise::launch<T, Op, Forward>; `out` may be `x`."""
+    if out is None:
+        out = torch.empty_like(x)
+    fn = getattr(capi.lib(), "snn_hip_pointwise_forward" + _suffix(x))
+    capi.check(fn(_ptr(x), _ptr(out), x.numel(), op, _stream()))
+    return out
+
+
+def pointwise_grad(val, err, op, out=None):
+    """sycldnn::pointwise::launch<T, Op, Gradient>: `val` is the forward
+    output (the forward input for LOG), `err` the incoming gradient."""
+    if out is None:
+        out = torch.empty_like(val)
+    fn = getattr(capi.lib(), "snn_hip_pointwise_grad" + _suffix(val))
+    capi.check(fn(_ptr(val), _ptr(err), _ptr(out), val.numel(), op, _stream()))
+    return out
+
+
+def binaryop_raw(lhs, rhs, out, lhs_dims, rhs_dims, op):
+    """Calls the entry point and returns its status code (no exception)."""
+    ld = (ctypes.c_int * max(len(lhs_dims), 1))(*lhs_dims)
+    rd = (ctypes.c_int * max(len(rhs_dims), 1))(*rhs_dims)
+    fn = getattr(capi.lib(), "snn_hip_binaryop" + _suffix(lhs))
+    return fn(_ptr(lhs), _ptr(rhs), _ptr(out), ld, len(lhs_dims), rd,
+              len(rhs_dims), op, _stream())
+
+
+def binaryop(lhs, rhs, lhs_dims, rhs_dims, op, out=None):
+    """sycldnn::binaryop::launch<T, Op> with BinaryParams{lhs_dims, rhs_dims};
+    `out` may be either operand when that operand has the output's shape."""
+    n = max(len(lhs_dims), len(rhs_dims), 1)
+    l = [1] * (n - len(lhs_dims)) + list(lhs_dims)
+    r = [1] * (n - len(rhs_dims)) + list(rhs_dims)
+    size = 1
+    for a, b in zip(l, r):
+        size *= max(a, b)
+    if out is None:
+        out = torch.empty(size, dtype=lhs.dtype, device=lhs.device)
+    capi.check(binaryop_raw(lhs, rhs, out, lhs_dims, rhs_dims, op))
+    return out
+
+
 __all__ = [
-    "ALGO", "DIRECTION", "POOL_OP", "STATUS", "ConvParams", "DepthwiseParams",
-    "PoolParams", "add_padding_to", "calculate_padding", "conv2d",
+    "ALGO", "BINARY_OP", "DIRECTION", "POINTWISE_OP", "POOL_OP", "STATUS",
+    "ConvParams", "DepthwiseParams", "PoolParams", "add_padding_to",
+    "binaryop", "binaryop_raw", "calculate_padding", "conv2d",
     "conv2d_raw", "conv_flops", "conv_params", "conv_sizes",
     "depthwise_conv2d", "depthwise_params", "depthwise_sizes", "matmul",
-    "pool_params", "pooling_avg_grad", "pooling_forward", "pooling_max_grad",
+    "pointwise_forward", "pointwise_grad", "pool_params", "pooling_avg_grad",
+    "pooling_forward", "pooling_max_grad",
     "workspace_size",
 ]
 

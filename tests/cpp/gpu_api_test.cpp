@@ -5,6 +5,7 @@
 // launch through the public template, wait on the returned event, compare
 // with the CPU oracle (which the golden tests pin to the reference's vectors).
 #include <portdnn/backend/hip_backend.h>
+#include <portdnn/binaryop/launch.h>
 #include <portdnn/conv2d/launch.h>
 #include <portdnn/conv2d/selector/default_selector.h>
 #include <portdnn/conv2d/selector/direct_selector.h>
@@ -16,6 +17,7 @@
 #include <portdnn/depthwise_conv2d/launch.h>
 #include <portdnn/helpers/padding.h>
 #include <portdnn/matmul/launch.h>
+#include <portdnn/pointwise/launch.h>
 #include <portdnn/pooling/launch.h>
 
 #include <cmath>
@@ -343,6 +345,62 @@ static void test_matmul(backend::HIPBackend& backend) {
   (void)hipStreamDestroy(other);
 }
 
+// test/pointwise/pointwise_fixture.h:37-70 (forward) and :72-137 (gradient),
+// test/binaryop/fixture.h:37-76.
+static void test_elementwise(backend::HIPBackend& backend) {
+  const size_t n = 4099;
+  std::vector<float> x(n);
+  for (size_t i = 0; i < n; ++i)
+    x[i] = static_cast<float>(static_cast<long>(i % 17) - 8);
+  DeviceBuffer d_x(backend, x), d_y(backend, n), d_g(backend, n);
+  auto st = pointwise::launch<float, pointwise::Relu, pointwise::Forward>(
+      d_x.ptr, d_y.ptr, n, backend);
+  CHECK(st.status == StatusCode::OK);
+  auto gr = pointwise::launch<float, pointwise::Relu, pointwise::Gradient>(
+      d_y.ptr, d_x.ptr, d_g.ptr, n, backend, {st.event});
+  CHECK(gr.status == StatusCode::OK);
+  gr.event.wait_and_throw();
+  std::vector<float> y(n), g(n);
+  CHECK(oracle_pointwise_forward(ORACLE_RELU, x.data(), y.data(), n) == 0);
+  CHECK(oracle_pointwise_grad(ORACLE_RELU, y.data(), x.data(), g.data(), n) ==
+        0);
+  CHECK(close(d_y.host(), y, true));
+  CHECK(close(d_g.host(), g, true));
+  CHECK((pointwise::launch<float, pointwise::Tanh, pointwise::Forward>(
+             d_x.ptr, d_y.ptr, 0, backend).status ==
+         StatusCode::InvalidParameter));
+
+  // bias add over an NHWC tensor, then a general broadcast
+  const std::vector<int> t_dims = {2, 5, 7, 12}, b_dims = {12};
+  const auto t = iota_data(2 * 5 * 7 * 12, 9), b = iota_data(12, 5);
+  DeviceBuffer d_t(backend, t), d_b(backend, b), d_o(backend, t.size());
+  binaryop::BinaryParams params{t_dims, b_dims};
+  auto add = binaryop::launch<float, binaryop::Add>(d_t.ptr, d_b.ptr, d_o.ptr,
+                                                    params, backend);
+  CHECK(add.status == StatusCode::OK);
+  add.event.wait_and_throw();
+  std::vector<float> ref(t.size());
+  CHECK(oracle_binaryop(ORACLE_ADD, t.data(), b.data(), ref.data(),
+                        t_dims.data(), 4, b_dims.data(), 1) == 0);
+  CHECK(close(d_o.host(), ref, true));
+  const std::vector<int> l_dims = {3, 1, 4}, r_dims = {2, 1, 5, 1};
+  const auto l = iota_data(12, 7), r = iota_data(10, 3);
+  DeviceBuffer d_l(backend, l), d_r(backend, r), d_q(backend, 2 * 3 * 5 * 4);
+  auto mul = binaryop::launch<float, binaryop::Mul>(
+      d_l.ptr, d_r.ptr, d_q.ptr, binaryop::BinaryParams{l_dims, r_dims},
+      backend);
+  CHECK(mul.status == StatusCode::OK);
+  mul.event.wait_and_throw();
+  std::vector<float> ref2(2 * 3 * 5 * 4);
+  CHECK(oracle_binaryop(ORACLE_MUL, l.data(), r.data(), ref2.data(),
+                        l_dims.data(), 3, r_dims.data(), 4) == 0);
+  CHECK(close(d_q.host(), ref2, true));
+  // internal/binaryop/launch.h:52-56: shapes that do not broadcast
+  CHECK((binaryop::launch<float, binaryop::Sub>(
+             d_l.ptr, d_r.ptr, d_q.ptr, binaryop::BinaryParams{{3, 4}, {5, 4}},
+             backend).status == StatusCode::InvalidParameter));
+}
+
 int main() {
   int n = 0;
   if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
@@ -358,6 +416,7 @@ int main() {
     test_pooling(backend);
     test_event_dependencies(backend);
     test_matmul(backend);
+    test_elementwise(backend);
   }
   (void)hipStreamDestroy(stream);
   return report("gpu_api_test");

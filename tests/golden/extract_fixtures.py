@@ -4,7 +4,8 @@
 The reference keeps its expected outputs as literal arrays inside generated
 gtest sources (test/conv2d/forward_window3_stride1.cc:57-67,
 test/depthwise_conv2d/forward_window3_stride1.cc, test/pooling/*_forward.cc,
-test/pooling/*_grad.cc, test/matmul/matmul_*.cc).  Those sources are parsed here AS TEXT -- nothing is
+test/pooling/*_grad.cc, test/matmul/matmul_*.cc, test/pointwise/*.cc,
+test/binaryop/binaryop_*.cc).  Those sources are parsed here AS TEXT -- nothing is
 compiled or executed -- and only the data (case shape, padding mode,
 max_input_val and the expected output values) is written to
 tests/golden/<group>.npz.  The operands are never stored: every case
@@ -154,6 +155,87 @@ def write_matmul():
           ("matmul", len(meta), values.size, os.path.getsize(out)))
 
 
+def _floats(text):
+    return np.array([float(tok) for tok in text.replace("\n", " ").split(",")
+                     if tok.strip()], dtype=np.float64)
+
+
+POINTWISE_FILES = [  # (file, operator id, is_gradient)
+    ("relu_forward.cc", 0, 0), ("relu_grad.cc", 0, 1),
+    ("tanh_forward.cc", 1, 0), ("tanh_grad.cc", 1, 1),
+    ("log_forward.cc", 3, 0), ("log_grad.cc", 3, 1),
+    ("floor_forward.cc", 4, 0),
+    ("sqrt_forward.cc", 5, 0), ("sqrt_grad.cc", 5, 1),
+]
+
+
+def write_pointwise():
+    """test/pointwise/<op>_{forward,grad}.cc.  meta columns: operator
+    (0 relu, 1 tanh, 3 log, 4 floor, 5 sqrt), is_gradient, input is signed,
+    size, max_val (unsigned generator only), n_values.  Inputs regenerate
+    from iota_initialised_signed_data(size) or iota_initialised_data(size,
+    max_val) (test/gen/iota_initialised_data.h:74-97); a gradient case feeds
+    the same data as forward input and as incoming error
+    (test/pointwise/pointwise_fixture.h:80-124)."""
+    gen = re.compile(r"input =\s*iota_initialised_(signed_)?data<DataType>\("
+                     r"(\d+)(?:,\s*(\d+))?\)")
+    metas, vals = [], []
+    for fname, op, grad in POINTWISE_FILES:
+        with open(os.path.join(REF, "test", "pointwise", fname)) as f:
+            text = f.read()
+        cases = CASE_RE.findall(text)
+        assert cases, fname
+        for _suite, _name, body in cases:
+            values = _floats(EXP_RE.search(body).group(1))
+            m = gen.search(body)
+            assert m, (fname, _name)
+            signed, size, maxv = m.group(1) is not None, int(m.group(2)), \
+                int(m.group(3) or 0)
+            assert size == values.size, (fname, _name)
+            metas.append([op, grad, int(signed), size, maxv, values.size])
+            vals.append(values)
+    meta = np.array(metas, dtype=np.int64)
+    values = np.concatenate(vals)
+    out = os.path.join(OUT, "pointwise.npz")
+    np.savez_compressed(out, meta=meta, values=values)
+    print("%-28s %5d cases %9d values %8d bytes" %
+          ("pointwise", len(meta), values.size, os.path.getsize(out)))
+
+
+def write_binaryop():
+    """test/binaryop/binaryop_{add,sub,mul,div}.cc.  meta columns: operator
+    (0 add, 1 sub, 2 mul, 3 div), n_lhs, lhs dims x4, n_rhs, rhs dims x4,
+    max_input_val, n_values (unused dims are 0).  Both operands are
+    1,2,...,max_val,1,... (test/binaryop/fixture.h:41-45)."""
+    metas, vals = [], []
+    for op, name in enumerate(("add", "sub", "mul", "div")):
+        with open(os.path.join(REF, "test", "binaryop",
+                               "binaryop_%s.cc" % name)) as f:
+            text = f.read()
+        cases = CASE_RE.findall(text)
+        assert cases, name
+        for _suite, _name, body in cases:
+            values = _floats(EXP_RE.search(body).group(1))
+            dims = []
+            for side in ("lhs_dims", "rhs_dims"):
+                m = re.search(side + r" = \{(.*?)\};", body, re.S)
+                d = [int(t) for t in m.group(1).split(",") if t.strip()]
+                assert len(d) <= 4
+                dims.append(d)
+            maxv = int(float(MAXV_RE.search(body).group(1)))
+            row = [op]
+            for d in dims:
+                row += [len(d)] + d + [0] * (4 - len(d))
+            metas.append(row + [maxv, values.size])
+            vals.append(values)
+    meta = np.array(metas, dtype=np.int64)
+    values = np.concatenate(vals)
+    out = os.path.join(OUT, "binaryop.npz")
+    np.savez_compressed(out, meta=meta, values=values)
+    print("%-28s %5d cases %9d values %8d bytes" %
+          ("binaryop", len(meta), values.size, os.path.getsize(out)))
+
+
 def main():
     if not os.path.isdir(REF):
         sys.exit("reference tree not found at " + REF)
@@ -179,6 +261,8 @@ def main():
     write_group("pool_avg_grad", "pooling",
                 "avg_window{w}_stride{s}_grad.cc", POOL_GRAD, False)
     write_matmul()
+    write_pointwise()
+    write_binaryop()
 
 
 if __name__ == "__main__":

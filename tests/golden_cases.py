@@ -48,3 +48,42 @@ def load_matmul():
                          ro, oo, max_val, data["values"][off:off + count])
         off += count
     assert off == data["values"].size
+
+
+POINTWISE_NAMES = {0: "relu", 1: "tanh", 2: "exp", 3: "log", 4: "floor",
+                   5: "sqrt"}
+PointwiseCase = namedtuple("PointwiseCase",
+                           "op is_grad signed size max_val expected")
+
+
+def load_pointwise():
+    """Yields every PointwiseCase of tests/golden/pointwise.npz (the
+    reference's test/pointwise/<op>_{forward,grad}.cc)."""
+    data = np.load(os.path.join(GOLDEN_DIR, "pointwise.npz"))
+    off = 0
+    for row in data["meta"]:
+        op, grad, signed, size, max_val, count = (int(v) for v in row)
+        yield PointwiseCase(POINTWISE_NAMES[op], bool(grad), bool(signed),
+                            size, max_val, data["values"][off:off + count])
+        off += count
+    assert off == data["values"].size
+
+
+BINARY_NAMES = ("add", "sub", "mul", "div")
+BinaryCase = namedtuple("BinaryCase", "op lhs_dims rhs_dims max_val expected")
+
+
+def load_binaryop():
+    """Yields every BinaryCase of tests/golden/binaryop.npz (the reference's
+    test/binaryop/binaryop_{add,sub,mul,div}.cc)."""
+    data = np.load(os.path.join(GOLDEN_DIR, "binaryop.npz"))
+    off = 0
+    for row in data["meta"]:
+        row = [int(v) for v in row]
+        op, n_l, n_r = row[0], row[1], row[6]
+        lhs_dims, rhs_dims = row[2:2 + n_l], row[7:7 + n_r]
+        max_val, count = row[11], row[12]
+        yield BinaryCase(BINARY_NAMES[op], lhs_dims, rhs_dims, max_val,
+                         data["values"][off:off + count])
+        off += count
+    assert off == data["values"].size

@@ -200,6 +200,27 @@ def test_kernel_timing_argument_checks():
     assert L.snn_hip_kernel_timing_enable(0) == STATUS.OK
 
 
+def test_elementwise_argument_checks():
+    """No device work: null pointers, zero items
+    (include/portdnn/internal/pointwise/launch_internal.h:69) and missing
+    dimension lists are rejected before any launch."""
+    L = capi.lib()
+    for name in ("snn_hip_pointwise_forward_f32",
+                 "snn_hip_pointwise_forward_f16"):
+        assert getattr(L, name)(None, None, 4, 0, None) == \
+            STATUS.INVALID_PARAMETER
+    buf = ctypes.create_string_buffer(64)
+    ptr = ctypes.cast(buf, ctypes.c_void_p)
+    assert L.snn_hip_pointwise_forward_f32(ptr, ptr, 0, 0, None) == \
+        STATUS.INVALID_PARAMETER
+    assert L.snn_hip_pointwise_grad_f32(ptr, None, ptr, 4, 0, None) == \
+        STATUS.INVALID_PARAMETER
+    assert L.snn_hip_binaryop_f32(ptr, ptr, ptr, None, 2, None, 0, 0, None) == \
+        STATUS.INVALID_PARAMETER
+    assert L.snn_hip_binaryop_f16(None, ptr, ptr, None, 0, None, 0, 0, None) == \
+        STATUS.INVALID_PARAMETER
+
+
 def test_workspace_sizes_reference_bounds():
     """Lower bounds of test/conv2d/workspace_size.cc:52-160 (VGG layer 1:
     3x3 s1 SAME, 224x224, 64 -> 64, batch 32)."""

@@ -14,9 +14,9 @@ import pytest
 import torch
 
 import oracle
-from golden_cases import load, load_matmul
+from golden_cases import load, load_binaryop, load_matmul, load_pointwise
 from portdnn_amd import capi, ops
-from portdnn_amd.capi import ALGO, DIRECTION, POOL_OP
+from portdnn_amd.capi import ALGO, BINARY_OP, DIRECTION, POINTWISE_OP, POOL_OP
 
 pytestmark = pytest.mark.gpu
 
@@ -164,3 +164,46 @@ def test_matmul_golden():
                    out=out[c.out_offset:])
         assert np.array_equal(out.cpu().numpy(),
                               c.expected.astype(np.float32)), c[:11]
+
+
+def ulp_close(got, exp, ulps=10):
+    """SNN_ALMOST_EQUAL(exp, got, 10u) of test/helpers/float_comparison.h."""
+    got = np.asarray(got, dtype=np.float32)
+    exp = np.asarray(exp, dtype=np.float32)
+    tol = ulps * np.spacing(np.maximum(np.abs(exp), np.abs(got)))
+    return np.all(np.abs(got.astype(np.float64) - exp.astype(np.float64))
+                  <= tol.astype(np.float64))
+
+
+def test_pointwise_golden():
+    """test/pointwise/<op>_{forward,grad}.cc through snn_hip_pointwise_*,
+    driven as test/pointwise/pointwise_fixture.h drives the reference."""
+    n_cases = 0
+    for c in load_pointwise():
+        op = getattr(POINTWISE_OP, c.op.upper())
+        x = dev(oracle.iota_signed(c.size) if c.signed
+                else oracle.iota(c.size, c.max_val))
+        if not c.is_grad:
+            got = ops.pointwise_forward(x, op).cpu().numpy()
+            assert ulp_close(got, c.expected), (c.op, c.size)
+        else:
+            val = x if c.op == "log" else ops.pointwise_forward(x, op)
+            got = ops.pointwise_grad(val, x, op).cpu().numpy()
+            assert np.allclose(got, c.expected, rtol=0, atol=1e-5), \
+                (c.op, c.size)
+        n_cases += 1
+    assert n_cases == 36
+
+
+def test_binaryop_golden():
+    """test/binaryop/binaryop_{add,sub,mul,div}.cc through snn_hip_binaryop_f32
+    (test/binaryop/fixture.h:37-76, 10 ULP)."""
+    n_cases = 0
+    for c in load_binaryop():
+        lhs = dev(oracle.iota(int(np.prod(c.lhs_dims)), c.max_val))
+        rhs = dev(oracle.iota(int(np.prod(c.rhs_dims)), c.max_val))
+        got = ops.binaryop(lhs, rhs, c.lhs_dims, c.rhs_dims,
+                           getattr(BINARY_OP, c.op.upper())).cpu().numpy()
+        assert ulp_close(got, c.expected), (c.op, c.lhs_dims, c.rhs_dims)
+        n_cases += 1
+    assert n_cases == 52

@@ -22,7 +22,8 @@ import torch
 
 import oracle
 from portdnn_amd import capi, ops
-from portdnn_amd.capi import ALGO, DIRECTION, POOL_OP
+from portdnn_amd.capi import ALGO, BINARY_OP, DIRECTION, POINTWISE_OP, POOL_OP, \
+    STATUS
 
 pytestmark = pytest.mark.gpu
 
@@ -588,3 +589,125 @@ def test_kernel_timing_brackets_the_main_kernel():
     with ops.kernel_timing() as kt:
         pass
     assert kt.kernels == 0
+
+
+# ---- pointwise / binaryop ---------------------------------------------------
+
+POINTWISE = ["relu", "tanh", "exp", "log", "floor", "sqrt"]
+
+
+def pointwise_data(rng, op, n):
+    x = rng.standard_normal(n).astype(np.float32) * 2
+    if op in ("log", "sqrt"):
+        x = np.abs(x) + 0.1
+    return x
+
+
+def assert_ulp(got, ref, ulps, what):
+    got = np.asarray(got, dtype=np.float32)
+    ref = np.asarray(ref, dtype=np.float32)
+    tol = ulps * np.spacing(np.maximum(np.abs(ref), np.abs(got)))
+    err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
+    assert np.all(err <= tol), (what, float(err.max()))
+
+
+@pytest.mark.parametrize("op", POINTWISE)
+@pytest.mark.parametrize("n", [1, 7, 1024, 4099, 1 << 20])
+def test_pointwise_forward_and_grad(op, n):
+    """Against the oracle; device libm may differ from the host's by a few
+    ULP on tanh / exp / log (the reference's own tests allow 10)."""
+    rng = np.random.default_rng(900 + n)
+    x = pointwise_data(rng, op, n)
+    code = getattr(POINTWISE_OP, op.upper())
+    ref = oracle.pointwise_forward(op, x)
+    got = ops.pointwise_forward(dev(x), code).cpu().numpy()
+    assert_ulp(got, ref, 10, (op, n, "forward"))
+    if op == "floor":
+        return
+    err = rng.standard_normal(n).astype(np.float32)
+    val = x if op == "log" else ref
+    got = ops.pointwise_grad(dev(val), dev(err), code).cpu().numpy()
+    # (1 - val * val) cancels near |val| = 1, where a fused multiply-add on
+    # the device and the oracle's separate rounding differ by more than ULPs
+    # of the result: absolute bar, tighter than the 1e-5 the reference's
+    # gradient tests use (test/pointwise/pointwise_fixture.h:66-70).
+    assert np.allclose(got, oracle.pointwise_grad(op, val, err), rtol=1e-5,
+                       atol=1e-6), (op, n, "grad")
+
+
+def test_pointwise_in_place_unaligned_and_f16():
+    rng = np.random.default_rng(950)
+    x = rng.standard_normal(5000).astype(np.float32)
+    # in place
+    d = dev(x)
+    ops.pointwise_forward(d, POINTWISE_OP.RELU, out=d)
+    assert np.array_equal(d.cpu().numpy(), np.maximum(x, 0))
+    # operands 4 bytes off a 16-byte boundary: the one-element-per-lane kernel
+    d = dev(np.concatenate([[0.0], x]).astype(np.float32))
+    out = torch.zeros(5001, device="cuda")
+    ops.pointwise_forward(d[1:], POINTWISE_OP.RELU, out=out[1:])
+    assert np.array_equal(out.cpu().numpy()[1:], np.maximum(x, 0))
+    assert out[0].item() == 0.0
+    # binary16: fp32 arithmetic, one rounding
+    h = x.astype(np.float16)
+    got = ops.pointwise_forward(dev(h, torch.float16), POINTWISE_OP.TANH)
+    ref = np.tanh(h.astype(np.float32)).astype(np.float16)
+    assert_close_f16(got.float().cpu().numpy(), ref.astype(np.float32),
+                     "tanh f16")
+    g = ops.pointwise_grad(dev(h, torch.float16), dev(h, torch.float16),
+                           POINTWISE_OP.RELU)
+    assert np.array_equal(g.cpu().numpy(), np.where(h > 0, h, 0).astype(np.float16))
+
+
+BINARY = {"add": np.add, "sub": np.subtract, "mul": np.multiply,
+          "div": np.divide}
+
+
+@pytest.mark.parametrize("op", list(BINARY))
+@pytest.mark.parametrize("dims", [
+    ([32, 56, 56, 64], [64]),           # bias add over NHWC: periodic operand
+    ([64], [32, 56, 56, 64]),           # ... on the left
+    ([3, 5, 7, 9], [3, 5, 7, 9]),       # same shape, odd size (tail)
+    ([1000003], []),                    # scalar right operand
+    ([], [257]),                        # scalar left operand
+    ([4, 1, 6, 1], [1, 5, 1, 7]),       # general broadcasting both ways
+    ([2, 3, 4, 6], [4, 6]),             # period 24, not a multiple of 4 x 8? (f32: 24 % 4 == 0)
+    ([2, 3, 4, 5], [5]),                # period 5: general kernel
+    ([6, 1, 5], [2, 1, 7, 1]),          # different ranks
+])
+def test_binaryop_shapes(op, dims):
+    lhs_dims, rhs_dims = dims
+    rng = np.random.default_rng(960 + len(lhs_dims) * 7 + len(rhs_dims))
+    lhs = uniform(rng, int(np.prod(lhs_dims)))
+    rhs = uniform(rng, int(np.prod(rhs_dims))) + 2.0  # keep div well away from 0
+    ref = BINARY[op](lhs.reshape(lhs_dims), rhs.reshape(rhs_dims)).reshape(-1)
+    assert np.array_equal(oracle.binaryop(op, lhs, rhs, lhs_dims, rhs_dims),
+                          ref)
+    got = ops.binaryop(dev(lhs), dev(rhs), lhs_dims, rhs_dims,
+                       getattr(BINARY_OP, op.upper())).cpu().numpy()
+    # add, sub, mul are exactly rounded on both sides; div within 1 ULP
+    if op == "div":
+        assert_ulp(got, ref, 1, (op, dims))
+    else:
+        assert np.array_equal(got, ref), (op, dims)
+
+
+def test_binaryop_f16_in_place_and_errors():
+    rng = np.random.default_rng(970)
+    x = uniform(rng, 32 * 14 * 14 * 256).astype(np.float16)
+    b = uniform(rng, 256).astype(np.float16)
+    d = dev(x, torch.float16)
+    ops.binaryop(d, dev(b, torch.float16), [32, 14, 14, 256], [256],
+                 BINARY_OP.ADD, out=d)
+    ref = (x.astype(np.float32).reshape(-1, 256) +
+           b.astype(np.float32)).astype(np.float16).reshape(-1)
+    assert np.array_equal(d.cpu().numpy(), ref)
+    a = dev(uniform(rng, 6))
+    out = torch.empty(12, device="cuda")
+    # include/portdnn/internal/binaryop/launch.h:52-56: not broadcastable
+    assert ops.binaryop_raw(a, a, out, [2, 3], [3, 2], BINARY_OP.ADD) == \
+        STATUS.INVALID_PARAMETER
+    assert ops.binaryop_raw(a, a, out, [1, 1, 1, 2, 3], [3], BINARY_OP.ADD) == \
+        STATUS.INVALID_PARAMETER
+    assert ops.binaryop_raw(a, a, out, [2, 3], [3], 9) == \
+        STATUS.INVALID_PARAMETER
