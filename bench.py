@@ -365,6 +365,35 @@ def main():
         del xs, ys
         detail["elementwise"] = elem
 
+        # convolution + bias + ReLU: three launches (the reference's
+        # composition) against the entry point that folds bias and
+        # activation into the convolution's output stage
+        fused = []
+        for name, p in layers:
+            algo = default_algo(p)
+            n_in, n_fil, n_out = ops.conv_sizes(p, DIRECTION.FORWARD)
+            x, f, b = uniform(n_in), uniform(n_fil), uniform(p.features)
+            y = torch.empty(n_out, device="cuda")
+            _, rec = ops.workspace_size(p, DIRECTION.FORWARD, algo)
+            ws = torch.empty(max(rec, 1), device="cuda")
+            out_dims = [p.batch, p.out_rows, p.out_cols, p.features]
+
+            def three():
+                ops.conv2d(x, f, p, DIRECTION.FORWARD, algo, workspace=ws,
+                           out=y)
+                ops.binaryop(y, b, out_dims, [p.features], BINARY_OP.ADD,
+                             out=y)
+                ops.pointwise_forward(y, POINTWISE_OP.RELU, out=y)
+
+            def one():
+                ops.conv2d_bias_act(x, f, b, p, algo, relu=True, workspace=ws,
+                                    out=y)
+            fused.append({"layer": name,
+                          "three_launches_ms": round(
+                              event_time_ms(three, reps=30), 5),
+                          "fused_ms": round(event_time_ms(one, reps=30), 5)})
+        detail["conv_bias_relu"] = fused
+
         # gradients of the memory-bound operators (same byte accounting:
         # every operand read or written once)
         grads = []

@@ -262,6 +262,24 @@ SNN_HIP_API int snn_hip_matmul_f32(const float* lhs, const float* rhs,
                                    int n, int transpose_lhs, int transpose_rhs,
                                    float beta, void* stream);
 
+/* ---- convolution with bias and activation ---------------------------------
+ * No single counterpart in the reference, which runs three launches for this
+ * (conv2d::launch, binaryop::launch<Add> with the bias as a [features]
+ * operand, pointwise::launch<Relu, Forward>; e.g. the layers of
+ * tools/layer.h).  Here the bias add and the activation are folded into the
+ * convolution's output stage wherever the chosen kernel writes each output
+ * once, and run as one in-place pass otherwise; the result equals the three
+ * launches.  `bias` holds one value per feature or is NULL; `activation` is a
+ * snn_hip_activation.  Everything else as snn_hip_conv2d_forward_f32. */
+typedef enum snn_hip_activation {
+  SNN_HIP_ACTIVATION_NONE = 0,
+  SNN_HIP_ACTIVATION_RELU = 1
+} snn_hip_activation;
+SNN_HIP_API int snn_hip_conv2d_forward_bias_act_f32(
+    const float* input, const float* filter, const float* bias, float* output,
+    const snn_hip_conv2d_params* params, int algorithm, int activation,
+    float* workspace, size_t workspace_elems, void* stream);
+
 /* ---- pointwise -------------------------------------------------------------
  * Stand-ins for sycldnn::pointwise::internal::launch_pointwise
  * (src/pointwise/launch_pointwise_forward.cc, launch_pointwise_grad.cc)

@@ -348,14 +348,21 @@ __global__ void __launch_bounds__(kThreads)
 //   * weight and output accesses use a per-lane constant offset plus a scalar
 //     offset operand, LDS addresses are constants plus immediates (the chunk
 //     loop is unrolled by the two LDS stages).
-template <int BM, int BN, int WM, int WN, bool B_K_INNER, bool ATOMIC>
+//
+// EPI: the forward convolution's optional epilogue, out = act(acc +
+// bias[feature]), applied to the accumulators before they are stored.
+template <int BM, int BN, int WM, int WN, bool B_K_INNER, bool ATOMIC,
+          bool EPI = false>
 __global__ void __launch_bounds__(kThreads)
     conv_igemm_fast_kernel(const float* __restrict__ src,
                            const float* __restrict__ wgt,
                            float* __restrict__ dst, Gather g,
                            unsigned src_bytes, unsigned wgt_bytes,
                            unsigned dst_bytes, unsigned n_tiles_n,
-                           unsigned n_tiles, int chunks_per_split) {
+                           unsigned n_tiles, int chunks_per_split,
+                           const float* __restrict__ bias = nullptr,
+                           int relu = 0) {
+  static_assert(!(EPI && ATOMIC), "partial sums cannot take the epilogue");
   static_assert(WM * WN == 4, "four waves per work-group");
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -578,6 +585,10 @@ __global__ void __launch_bounds__(kThreads)
               ? static_cast<unsigned>(m_base) * row_bytes +
                     static_cast<unsigned>(col) * 4u
               : kOob;
+      float bias_col = 0.f;
+      if (EPI) {
+        if (bias != nullptr && col < g.n_total) bias_col = bias[col];
+      }
       // The row offset goes into the vector offset, not the scalar offset
       // operand: hipcc (ROCm 7.2) treats buffer stores that differ only in
       // their scalar offset as stores to one address and forwards the first
@@ -586,7 +597,11 @@ __global__ void __launch_bounds__(kThreads)
       for (int v = 0; v < 16; ++v) {
         const unsigned off =
             voff + static_cast<unsigned>(8 * (v >> 2) + (v & 3)) * row_bytes;
-        const float val = acc[i][j][v];
+        float val = acc[i][j][v];
+        if (EPI) {
+          val += bias_col;
+          if (relu) val = fmaxf(val, 0.f);
+        }
         if (ATOMIC) {
           __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(val, dst_rsrc, off, 0,
                                                           0);
@@ -1007,7 +1022,8 @@ template <int BM, int BN, int WM, int WN, bool B_K_INNER, bool STRIDED>
 void launch_tile(const float* src, const float* wgt, float* dst,
                  const Gather& g, size_t src_elems, size_t wgt_elems,
                  int splits, hipStream_t stream, int batches = 1,
-                 bool accumulate = false) {
+                 bool accumulate = false,
+                 const ConvEpilogue* epilogue = nullptr) {
   // accumulate: add the product to what dst holds (atomic kernel, no zero
   // fill) instead of overwriting it.
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(g.m_total, BM));
@@ -1046,7 +1062,7 @@ void launch_tile(const float* src, const float* wgt, float* dst,
       hipLaunchKernelGGL(kernel, dim3(n_tiles, splits, batches),
                          dim3(kThreads), kLdsBytes, stream, src, wgt, dst, g,
                          src_bytes, wgt_bytes, dst_bytes, tiles_n, n_tiles,
-                         per_split);
+                         per_split, static_cast<const float*>(nullptr), 0);
       return;
     }
     auto kernel = conv_igemm_kernel<BM, BN, WM, WN, B_K_INNER, STRIDED, true>;
@@ -1059,6 +1075,20 @@ void launch_tile(const float* src, const float* wgt, float* dst,
                        wgt_bytes, tiles_n, n_tiles, per_split);
   } else {
     KernelTimer timer(stream);
+    if (fast && epilogue != nullptr && epilogue->wanted() && batches == 1) {
+      auto kernel =
+          conv_igemm_fast_kernel<BM, BN, WM, WN, B_K_INNER, false, true>;
+      static const hipError_t attr = hipFuncSetAttribute(
+          reinterpret_cast<const void*>(kernel),
+          hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+      (void)attr;
+      hipLaunchKernelGGL(kernel, dim3(n_tiles, 1, 1), dim3(kThreads),
+                         kLdsBytes, stream, src, wgt, dst, g, src_bytes,
+                         wgt_bytes, dst_bytes, tiles_n, n_tiles, per_split,
+                         epilogue->bias, epilogue->relu ? 1 : 0);
+      if (epilogue->applied != nullptr) *epilogue->applied = true;
+      return;
+    }
     if (fast) {
       auto kernel = conv_igemm_fast_kernel<BM, BN, WM, WN, B_K_INNER, false>;
       static const hipError_t attr = hipFuncSetAttribute(
@@ -1067,7 +1097,8 @@ void launch_tile(const float* src, const float* wgt, float* dst,
       (void)attr;
       hipLaunchKernelGGL(kernel, dim3(n_tiles, 1, batches), dim3(kThreads),
                          kLdsBytes, stream, src, wgt, dst, g, src_bytes,
-                         wgt_bytes, dst_bytes, tiles_n, n_tiles, per_split);
+                         wgt_bytes, dst_bytes, tiles_n, n_tiles, per_split,
+                         static_cast<const float*>(nullptr), 0);
       return;
     }
     auto kernel = conv_igemm_kernel<BM, BN, WM, WN, B_K_INNER, STRIDED, false>;
@@ -1098,7 +1129,7 @@ constexpr int kMinChunksPerSplit = 8;
 template <bool B_K_INNER, bool STRIDED>
 void launch_auto(const float* src, const float* wgt, float* dst,
                  const Gather& g, size_t src_elems, size_t wgt_elems,
-                 hipStream_t stream) {
+                 hipStream_t stream, const ConvEpilogue* epilogue = nullptr) {
   auto tiles = [&](int bm, int bn) {
     return static_cast<long>(ceil_div(g.m_total, bm)) * ceil_div(g.n_total, bn);
   };
@@ -1123,8 +1154,8 @@ void launch_auto(const float* src, const float* wgt, float* dst,
     return;
   }
   if (g.n_total > 64 && tiles(128, 128) >= 4 * kResidentSlots) {
-    launch_tile<128, 128, 2, 2, B_K_INNER, STRIDED>(src, wgt, dst, g, src_elems,
-                                                    wgt_elems, 1, stream);
+    launch_tile<128, 128, 2, 2, B_K_INNER, STRIDED>(
+        src, wgt, dst, g, src_elems, wgt_elems, 1, stream, 1, false, epilogue);
     return;
   }
   const long t = tiles(64, 64);
@@ -1134,8 +1165,9 @@ void launch_auto(const float* src, const float* wgt, float* dst,
     splits = static_cast<int>((kSplitUnits + t - 1) / t);
     splits = max(1, min(splits, n_chunks / kMinChunksPerSplit));
   }
-  launch_tile<64, 64, 2, 2, B_K_INNER, STRIDED>(src, wgt, dst, g, src_elems,
-                                                wgt_elems, splits, stream);
+  launch_tile<64, 64, 2, 2, B_K_INNER, STRIDED>(
+      src, wgt, dst, g, src_elems, wgt_elems, splits, stream, 1, false,
+      epilogue);
 }
 
 // Forward convolution whose channel count is not a multiple of 4: 64x64
@@ -1392,7 +1424,8 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
                             const float* filter, float* output,
                             const snn_hip_conv2d_params& p,
                             hipStream_t stream, float* workspace,
-                            size_t workspace_elems) {
+                            size_t workspace_elems,
+                            const ConvEpilogue* epilogue) {
   if (direction == SNN_HIP_INPUT_BACKPROP && p.channels < 16 &&
       p.features % kBK == 0 &&
       static_cast<size_t>(p.out_rows) * p.out_cols * p.window_rows *
@@ -1440,7 +1473,7 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
                                  wgt_elems, stream);
   } else if (direction == SNN_HIP_FORWARD) {
     launch_auto<false, false>(input, filter, output, g, src_elems, wgt_elems,
-                              stream);
+                              stream, epilogue);
   } else if (g.div_rows != 1 || g.div_cols != 1) {
     launch_auto<true, true>(input, filter, output, g, src_elems, wgt_elems,
                             stream);

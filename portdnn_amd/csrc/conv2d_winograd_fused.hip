@@ -159,7 +159,8 @@ __global__ void __launch_bounds__(512)
                          const float* __restrict__ u, float* __restrict__ out,
                          FusedGeom g, unsigned in_bytes, unsigned u_bytes,
                          unsigned out_bytes, UnitGrid ug,
-                         int chunks_per_split) {
+                         int chunks_per_split,
+                         const float* __restrict__ bias, int relu) {
   __shared__ __align__(16) float lds_v[2 * kVBuf];
   __shared__ int lds_tile_off[kTiles];
   __shared__ int lds_tile_flags[kTiles];
@@ -352,10 +353,24 @@ __global__ void __launch_bounds__(512)
     for (int i = 0; i < 4; ++i)
       s[i] = *reinterpret_cast<const float4*>(
           lds_v + ((i * 2 + b) * 16 + v) * 64 + 4 * q);
-    const float4 y0 = s[0] + s[1] + s[2];
-    const float4 y1 = s[1] - s[2] - s[3];
+    float4 y0 = s[0] + s[1] + s[2];
+    float4 y1 = s[1] - s[2] - s[3];
     const int m = 8 * (v >> 2) + 4 * (q >> 3) + (v & 3);
     const int f = static_cast<int>(fb) * kFeat + 4 * (q & 7);
+    if (!ATOMIC) {
+      // Optional epilogue of the forward convolution: bias per feature, ReLU.
+      if (bias != nullptr) {
+        const float4 b4 = *reinterpret_cast<const float4*>(bias + f);
+        y0 = y0 + b4;
+        y1 = y1 + b4;
+      }
+      if (relu) {
+        y0 = make_float4(fmaxf(y0.x, 0.f), fmaxf(y0.y, 0.f), fmaxf(y0.z, 0.f),
+                         fmaxf(y0.w, 0.f));
+        y1 = make_float4(fmaxf(y1.x, 0.f), fmaxf(y1.y, 0.f), fmaxf(y1.z, 0.f),
+                         fmaxf(y1.w, 0.f));
+      }
+    }
     const int tile_off = lds_tile_off[m];
     const int flags = lds_tile_flags[m];
     const bool col_ok = tile_off >= 0 && (b == 0 || (flags & 2) != 0);
@@ -408,7 +423,8 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
                                      const float* filter, float* output,
                                      const snn_hip_conv2d_params& p,
                                      float* workspace, size_t workspace_elems,
-                                     hipStream_t stream) {
+                                     hipStream_t stream,
+                                     const ConvEpilogue* epilogue) {
   const bool backprop = direction == SNN_HIP_INPUT_BACKPROP;
   FusedGeom g;
   g.in_rows = backprop ? p.out_rows : p.in_rows;
@@ -505,12 +521,19 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
     KernelTimer timer(stream);
     hipLaunchKernelGGL(wino_fused_kernel<true>, dim3(grid_x, splits),
                        dim3(512), 0, stream, input, workspace, output, g,
-                       in_bytes, u_bytes, out_bytes, ug, per_split);
+                       in_bytes, u_bytes, out_bytes, ug, per_split,
+                       static_cast<const float*>(nullptr), 0);
   } else {
+    // The bias vector is read 16 bytes at a time.
+    const bool fuse = epilogue != nullptr && epilogue->wanted() && !backprop &&
+                      (epilogue->bias == nullptr || aligned16(epilogue->bias));
     KernelTimer timer(stream);
     hipLaunchKernelGGL(wino_fused_kernel<false>, dim3(grid_x, 1), dim3(512),
                        0, stream, input, workspace, output, g, in_bytes,
-                       u_bytes, out_bytes, ug, per_split);
+                       u_bytes, out_bytes, ug, per_split,
+                       fuse ? epilogue->bias : nullptr,
+                       fuse && epilogue->relu ? 1 : 0);
+    if (fuse && epilogue->applied != nullptr) *epilogue->applied = true;
   }
   SNN_HIP_CHECK_LAUNCH();
   return SNN_HIP_OK;

@@ -365,7 +365,81 @@ int launch_binaryop_t(int op, const T* lhs, const T* rhs, T* out,
   }
 }
 
+// data = act(data + bias[feature]) in place; VEC lanes of one vector share a
+// pixel (features % 4 == 0) or the kernel runs element by element.
+template <bool VEC>
+__global__ void __launch_bounds__(kThreads)
+    bias_act_kernel(float* data, const float* __restrict__ bias,
+                    unsigned features, size_t n_items, int relu) {
+  typedef Vec16<float>::type V;
+  const size_t i = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i >= n_items) return;
+  if (VEC) {
+    V v = reinterpret_cast<V*>(data)[i];
+    if (bias != nullptr) {
+      const V b = *reinterpret_cast<const V*>(
+          bias + static_cast<unsigned>((i * 4) % features));
+      v += b;
+    }
+    if (relu) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k] = fmaxf(v[k], 0.f);
+    }
+    reinterpret_cast<V*>(data)[i] = v;
+  } else {
+    float v = data[i];
+    if (bias != nullptr) v += bias[i % features];
+    if (relu) v = fmaxf(v, 0.f);
+    data[i] = v;
+  }
+}
+
+template <bool BLEND>
+__global__ void __launch_bounds__(kThreads)
+    scale_blend_kernel(float* data, const float* prior, float alpha,
+                       float beta, size_t n) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i >= n) return;
+  float v = alpha * data[i];
+  if (BLEND) v += beta * prior[i];
+  data[i] = v;
+}
+
 }  // namespace
+
+int launch_bias_act_f32(float* data, const float* bias, int features, size_t n,
+                        bool relu, hipStream_t stream) {
+  const bool vec = features % 4 == 0 && aligned16(data) &&
+                   (bias == nullptr || aligned16(bias));
+  if (vec) {
+    const size_t n_vec = n / 4;
+    hipLaunchKernelGGL(bias_act_kernel<true>,
+                       dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{kThreads}))),
+                       dim3(kThreads), 0, stream, data, bias,
+                       static_cast<unsigned>(features), n_vec, relu ? 1 : 0);
+  } else {
+    hipLaunchKernelGGL(bias_act_kernel<false>,
+                       dim3(static_cast<unsigned>(ceil_div(n, size_t{kThreads}))),
+                       dim3(kThreads), 0, stream, data, bias,
+                       static_cast<unsigned>(features), n, relu ? 1 : 0);
+  }
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? SNN_HIP_OK : report_hip_error(e, "bias_act_kernel");
+}
+
+int launch_scale_blend_f32(float* data, const float* prior, float alpha,
+                           float beta, size_t n, hipStream_t stream) {
+  const dim3 grid(static_cast<unsigned>(ceil_div(n, size_t{kThreads})));
+  if (beta != 0.f && prior != nullptr)
+    hipLaunchKernelGGL(scale_blend_kernel<true>, grid, dim3(kThreads), 0,
+                       stream, data, prior, alpha, beta, n);
+  else
+    hipLaunchKernelGGL(scale_blend_kernel<false>, grid, dim3(kThreads), 0,
+                       stream, data, prior, alpha, beta, n);
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? SNN_HIP_OK
+                         : report_hip_error(e, "scale_blend_kernel");
+}
 
 int launch_pointwise_forward_f32(int op, const float* in, float* out, size_t n,
                                  hipStream_t stream) {

@@ -291,12 +291,14 @@ inline bool aligned16(const void* p) {
 template <typename T>
 int launch_gemm_path(int direction, const T* input, const T* filter, T* output,
                      const snn_hip_conv2d_params& p, hipStream_t s,
-                     T* workspace = nullptr, size_t workspace_elems = 0);
+                     T* workspace = nullptr, size_t workspace_elems = 0,
+                     const ConvEpilogue* epilogue = nullptr);
 template <>
 int launch_gemm_path<_Float16>(int direction, const _Float16* input,
                                const _Float16* filter, _Float16* output,
                                const snn_hip_conv2d_params& p, hipStream_t s,
-                               _Float16* workspace, size_t workspace_elems) {
+                               _Float16* workspace, size_t workspace_elems,
+                               const ConvEpilogue*) {
   if (direction == SNN_HIP_FORWARD && conv2d_igemm_f16_supports(p) &&
       aligned16(input) && aligned16(filter) && aligned16(output))
     return launch_conv2d_igemm_f16(input, filter, output, p, workspace,
@@ -307,11 +309,12 @@ template <>
 int launch_gemm_path<float>(int direction, const float* input,
                             const float* filter, float* output,
                             const snn_hip_conv2d_params& p, hipStream_t s,
-                            float* workspace, size_t workspace_elems) {
+                            float* workspace, size_t workspace_elems,
+                            const ConvEpilogue* epilogue) {
   if (conv2d_igemm_supports(direction, p) && aligned16(input) &&
       aligned16(filter) && aligned16(output))
     return launch_conv2d_igemm_f32(direction, input, filter, output, p, s,
-                                   workspace, workspace_elems);
+                                   workspace, workspace_elems, epilogue);
   return launch_conv2d_direct<float>(direction, input, filter, output, p, s);
 }
 
@@ -323,7 +326,8 @@ int launch_gemm_path<float>(int direction, const float* input,
 template <typename T>
 int launch_winograd_path(int direction, const T* input, const T* filter,
                          T* output, const snn_hip_conv2d_params& p,
-                         T* workspace, size_t workspace_elems, hipStream_t s) {
+                         T* workspace, size_t workspace_elems, hipStream_t s,
+                         const ConvEpilogue* epilogue = nullptr) {
   return launch_gemm_path<T>(direction, input, filter, output, p, s);
 }
 template <>
@@ -331,24 +335,27 @@ int launch_winograd_path<float>(int direction, const float* input,
                                 const float* filter, float* output,
                                 const snn_hip_conv2d_params& p,
                                 float* workspace, size_t workspace_elems,
-                                hipStream_t s) {
+                                hipStream_t s, const ConvEpilogue* epilogue) {
   // SNN_HIP_WINO_UNFUSED is a development switch that forces the three-stage
   // chain on shapes the fused kernel would take.
   if (conv2d_winograd_fused_supports(direction, p) && aligned16(input) &&
       aligned16(output) && aligned16(workspace) &&
       std::getenv("SNN_HIP_WINO_UNFUSED") == nullptr)
     return launch_conv2d_winograd_fused_f32(direction, input, filter, output,
-                                            p, workspace, workspace_elems, s);
+                                            p, workspace, workspace_elems, s,
+                                            epilogue);
   if (conv2d_winograd_supports(direction, p))
     return launch_conv2d_winograd_f32(direction, input, filter, output, p,
                                       workspace, workspace_elems, s);
-  return launch_gemm_path<float>(direction, input, filter, output, p, s);
+  return launch_gemm_path<float>(direction, input, filter, output, p, s,
+                                 nullptr, 0, epilogue);
 }
 
 template <typename T>
 int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
                     const snn_hip_conv2d_params* params, int algorithm,
-                    T* workspace, size_t workspace_elems, void* stream) {
+                    T* workspace, size_t workspace_elems, void* stream,
+                    const ConvEpilogue* epilogue = nullptr) {
   if (params == nullptr) return SNN_HIP_INVALID_PARAMETER;
   const snn_hip_conv2d_params& p = *params;
   const int v = validate(p);
@@ -370,12 +377,12 @@ int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
       if (workspace == nullptr || workspace_elems == 0)
         return SNN_HIP_INSUFFICIENT_WORKSPACE;
       return launch_winograd_path<T>(direction, input, filter, output, p,
-                                     workspace, workspace_elems, s);
+                                     workspace, workspace_elems, s, epilogue);
     case SNN_HIP_ALGO_TILED:
     case SNN_HIP_ALGO_IM2COL:
     case SNN_HIP_ALGO_MATMUL:
       return launch_gemm_path<T>(direction, input, filter, output, p, s,
-                                 workspace, workspace_elems);
+                                 workspace, workspace_elems, epilogue);
     default:
       return launch_conv2d_direct<T>(direction, input, filter, output, p, s);
   }
@@ -630,6 +637,32 @@ int snn_hip_matmul_f32(const float* lhs, const float* rhs, float* output,
   return launch_matmul_f32(lhs, rhs, output, batches, m, k, n,
                            transpose_lhs != 0, transpose_rhs != 0, beta,
                            as_stream(stream));
+}
+
+int snn_hip_conv2d_forward_bias_act_f32(
+    const float* input, const float* filter, const float* bias, float* output,
+    const snn_hip_conv2d_params* params, int algorithm, int activation,
+    float* workspace, size_t workspace_elems, void* stream) {
+  if (activation != SNN_HIP_ACTIVATION_NONE &&
+      activation != SNN_HIP_ACTIVATION_RELU)
+    return SNN_HIP_INVALID_PARAMETER;
+  bool applied = false;
+  ConvEpilogue epilogue;
+  epilogue.bias = bias;
+  epilogue.relu = activation == SNN_HIP_ACTIVATION_RELU;
+  epilogue.applied = &applied;
+  const int status =
+      conv2d_dispatch<float>(SNN_HIP_FORWARD, input, filter, output, params,
+                             algorithm, workspace, workspace_elems, stream,
+                             &epilogue);
+  if (status != SNN_HIP_OK || applied || !epilogue.wanted()) return status;
+  // The chosen kernel could not fold the epilogue into its stores (partial
+  // sums meeting through atomics, the direct and three-stage kernels): one
+  // in-place pass over the finished output.
+  const size_t n = static_cast<size_t>(params->batch) * params->out_rows *
+                   params->out_cols * params->features;
+  return launch_bias_act_f32(output, bias, params->features, n, epilogue.relu,
+                             as_stream(stream));
 }
 
 int snn_hip_pointwise_forward_f32(const float* input, float* output,

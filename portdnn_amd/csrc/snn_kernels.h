@@ -14,6 +14,16 @@ int launch_conv2d_direct(int direction, const T* input, const T* filter,
                          T* output, const snn_hip_conv2d_params& p,
                          hipStream_t stream);
 
+// Work a forward convolution may fold into its last stage: out = act(conv +
+// bias[feature]).  A launcher that applies it sets *applied; otherwise the
+// caller runs launch_bias_act_f32 over the finished output.
+struct ConvEpilogue {
+  const float* bias = nullptr;  // one value per feature, or none
+  bool relu = false;
+  bool* applied = nullptr;
+  bool wanted() const { return bias != nullptr || relu; }
+};
+
 // Implicit-GEMM convolution on MFMA (conv2d_igemm.hip): the path behind the
 // Tiled and Im2col algorithm tags.  `supports` tells whether the shape meets
 // the kernel's vector-width requirements; pointers must be 16-byte aligned.
@@ -22,7 +32,8 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
                             const float* filter, float* output,
                             const snn_hip_conv2d_params& p, hipStream_t stream,
                             float* workspace = nullptr,
-                            size_t workspace_elems = 0);
+                            size_t workspace_elems = 0,
+                            const ConvEpilogue* epilogue = nullptr);
 
 // Batched row-major GEMM C[z] = A[z] (m x k) * op(B[z]) on the same MFMA
 // kernel, op(B) = B (k x n) or B^T with B stored n x k; operands of
@@ -55,7 +66,8 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
                                      const float* filter, float* output,
                                      const snn_hip_conv2d_params& p,
                                      float* workspace, size_t workspace_elems,
-                                     hipStream_t stream);
+                                     hipStream_t stream,
+                                     const ConvEpilogue* epilogue = nullptr);
 
 // Half-precision forward convolution on MFMA (conv2d_igemm_f16.hip).  The
 // workspace, when large enough, receives the re-laid-out filter.
@@ -115,6 +127,14 @@ int launch_binaryop_f32(int op, const float* lhs, const float* rhs, float* out,
 int launch_binaryop_f16(int op, const _Float16* lhs, const _Float16* rhs,
                         _Float16* out, const int* lhs_dims, int n_lhs,
                         const int* rhs_dims, int n_rhs, hipStream_t stream);
+// data[i] = act(data[i] + bias[i % features]) in place over n elements
+// (n % features == 0); bias may be null, act is max(., 0) when relu.
+int launch_bias_act_f32(float* data, const float* bias, int features, size_t n,
+                        bool relu, hipStream_t stream);
+// data[i] = alpha * data[i] + beta * prior[i] (prior may be null when beta is
+// 0): the blend of the compatibility layer's alpha / beta scaling.
+int launch_scale_blend_f32(float* data, const float* prior, float alpha,
+                           float beta, size_t n, hipStream_t stream);
 
 }  // namespace snn
 

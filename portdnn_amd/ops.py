@@ -127,6 +127,22 @@ def conv2d(inp, fil, p, direction=DIRECTION.FORWARD, algorithm=ALGO.DIRECT,
     return out
 
 
+def conv2d_bias_act(inp, fil, bias, p, algorithm, relu=True, workspace=None,
+                    out=None):
+    """snn_hip_conv2d_forward_bias_act_f32: act(conv(inp, fil) + bias)."""
+    _, _, n_out = conv_sizes(p, DIRECTION.FORWARD)
+    if out is None:
+        out = torch.empty(n_out, dtype=inp.dtype, device=inp.device)
+    if workspace is None and algorithm in (ALGO.WINOGRAD, ALGO.WINOGRAD_LARGE):
+        _, rec = workspace_size(p, DIRECTION.FORWARD, algorithm)
+        workspace = torch.empty(rec, dtype=inp.dtype, device=inp.device)
+    ws_elems = 0 if workspace is None else workspace.numel()
+    capi.check(capi.lib().snn_hip_conv2d_forward_bias_act_f32(
+        _ptr(inp), _ptr(fil), _ptr(bias), _ptr(out), ctypes.byref(p),
+        algorithm, 1 if relu else 0, _ptr(workspace), ws_elems, _stream()))
+    return out
+
+
 _DW_FN = {
     (DIRECTION.FORWARD, torch.float32): "snn_hip_depthwise_conv2d_forward_f32",
     (DIRECTION.INPUT_BACKPROP, torch.float32):
@@ -248,6 +264,7 @@ __all__ = [
     "ALGO", "BINARY_OP", "DIRECTION", "POINTWISE_OP", "POOL_OP", "STATUS",
     "ConvParams", "DepthwiseParams", "PoolParams", "add_padding_to",
     "binaryop", "binaryop_raw", "calculate_padding", "conv2d",
+    "conv2d_bias_act",
     "conv2d_raw", "conv_flops", "conv_params", "conv_sizes",
     "depthwise_conv2d", "depthwise_params", "depthwise_sizes", "matmul",
     "pointwise_forward", "pointwise_grad", "pool_params", "pooling_avg_grad",

@@ -711,3 +711,58 @@ def test_binaryop_f16_in_place_and_errors():
         STATUS.INVALID_PARAMETER
     assert ops.binaryop_raw(a, a, out, [2, 3], [3], 9) == \
         STATUS.INVALID_PARAMETER
+
+
+# ---- convolution with bias and activation ------------------------------------
+
+@pytest.mark.parametrize("shape", [
+    # batch, size, channels, features, window, stride
+    (4, 28, 64, 64, 3, 1),      # fused Winograd epilogue
+    (2, 14, 256, 256, 3, 1),    # Winograd with a channel split: separate pass
+    (4, 28, 64, 256, 1, 1),     # implicit GEMM, epilogue in the kernel
+    (1, 7, 512, 2048, 1, 1),    # implicit GEMM with a reduction split
+    (2, 15, 24, 40, 3, 2),      # strided, ragged
+    (1, 9, 3, 6, 5, 1),         # direct kernel, features % 4 != 0
+])
+@pytest.mark.parametrize("relu", [True, False])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_conv2d_bias_activation(shape, relu, with_bias):
+    """snn_hip_conv2d_forward_bias_act_f32 against the composition it stands
+    for: oracle convolution, oracle binaryop add of the [features] bias,
+    oracle relu."""
+    batch, size, ch, feats, window, stride = shape
+    p = ops.conv_params(batch, size, size, ch, feats, window, stride, True)
+    rng = np.random.default_rng(1000 + size + feats)
+    n_in, n_fil, n_out = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x, w = uniform(rng, n_in), uniform(rng, n_fil)
+    bias = uniform(rng, feats) * 4 if with_bias else None
+    ref = oracle.conv2d_forward(x, w, oracle_params(p, feats), acc64=True)
+    if with_bias:
+        ref = oracle.binaryop("add", ref, bias,
+                              [batch, p.out_rows, p.out_cols, feats], [feats])
+    if relu:
+        ref = oracle.pointwise_forward("relu", ref)
+    d_bias = dev(bias) if with_bias else None
+    n_run = 0
+    for algo in FWD_ALGOS:
+        if not supported(p, DIRECTION.FORWARD, algo):
+            continue
+        got = ops.conv2d_bias_act(dev(x), dev(w), d_bias, p, algo,
+                                  relu=relu).cpu().numpy()
+        # an output within rounding of zero may land on either side of the
+        # ReLU: the absolute part of the tolerance covers it
+        assert_close(got, ref, ("bias_act", ALGO_NAME[algo], shape, relu,
+                                with_bias))
+        n_run += 1
+    assert n_run >= 2
+
+
+def test_conv2d_bias_activation_rejects_unknown_activation():
+    p = ops.conv_params(1, 8, 8, 4, 4, 3, 1, True)
+    x = torch.zeros(ops.conv_sizes(p, 0)[0], device="cuda")
+    w = torch.zeros(ops.conv_sizes(p, 0)[1], device="cuda")
+    y = torch.zeros(ops.conv_sizes(p, 0)[2], device="cuda")
+    rc = capi.lib().snn_hip_conv2d_forward_bias_act_f32(
+        x.data_ptr(), w.data_ptr(), None, y.data_ptr(), ctypes.byref(p),
+        ALGO.DIRECT, 7, None, 0, None)
+    assert rc == STATUS.INVALID_PARAMETER
