@@ -300,6 +300,39 @@ SNNStatus launch(typename Backend::template pointer_type<T const> input,
       stream);
 }
 
+// Not in portDNN, which runs three launches for this (conv2d::launch,
+// binaryop::launch<Add> with the bias as a [features] operand,
+// pointwise::launch<Relu, Forward>): output = act(conv(input, filter) +
+// bias[feature]) with the bias add and the activation folded into the
+// convolution's output stage where the chosen kernel allows it.  `bias` may
+// be null.  Forward, float, NHWC only.
+enum class Activation {
+  None = SNN_HIP_ACTIVATION_NONE,
+  Relu = SNN_HIP_ACTIVATION_RELU
+};
+template <typename T, typename Backend>
+SNNStatus launch_forward_bias_activation(
+    typename Backend::template pointer_type<T const> input,
+    typename Backend::template pointer_type<T const> filter,
+    typename Backend::template pointer_type<T const> bias,
+    typename Backend::template pointer_type<T> output,
+    Conv2DParams const& params, Selector& selector, Backend& backend,
+    typename Backend::template pointer_type<T> workspace,
+    size_t workspace_size, Activation activation,
+    const std::vector<hip::Event>& events = {}) {
+  static_assert(std::is_same<T, float>::value,
+                "launch_forward_bias_activation is provided for float");
+  const snn_hip_conv2d_params c = internal::to_c(params);
+  const Algorithm algo = selector.select<conv_type::Forward>(params);
+  hipStream_t stream = backend.get_stream();
+  hip::detail::wait_for(stream, events);
+  return hip::detail::finish(
+      snn_hip_conv2d_forward_bias_act_f32(
+          input, filter, bias, output, &c, static_cast<int>(algo),
+          static_cast<int>(activation), workspace, workspace_size, stream),
+      stream);
+}
+
 }  // namespace conv2d
 }  // namespace sycldnn
 

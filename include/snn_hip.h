@@ -280,6 +280,16 @@ SNN_HIP_API int snn_hip_conv2d_forward_bias_act_f32(
     const snn_hip_conv2d_params* params, int algorithm, int activation,
     float* workspace, size_t workspace_elems, void* stream);
 
+/* ---- alpha / beta blend ----------------------------------------------------
+ * data[i] = alpha * data[i] + beta * prior[i] over n_items elements: the
+ * scaling step of the cuDNN-style layer (ScalingParams::applyScaling,
+ * include/portdnn/compat/scaling.hpp:150-262, which composes binaryop
+ * launches for it).  `prior` may be NULL when beta is 0; a zero alpha drops
+ * the data term outright. */
+SNN_HIP_API int snn_hip_scale_blend_f32(float* data, const float* prior,
+                                        float alpha, float beta,
+                                        size_t n_items, void* stream);
+
 /* ---- pointwise -------------------------------------------------------------
  * Stand-ins for sycldnn::pointwise::internal::launch_pointwise
  * (src/pointwise/launch_pointwise_forward.cc, launch_pointwise_grad.cc)

@@ -400,7 +400,9 @@ __global__ void __launch_bounds__(kThreads)
                        float beta, size_t n) {
   const size_t i = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i >= n) return;
-  float v = alpha * data[i];
+  // A zero factor drops its term outright (NaN or Inf in it do not survive),
+  // as the reference does by skipping the convolution / zeroing the output.
+  float v = alpha == 0.f ? 0.f : alpha * data[i];
   if (BLEND) v += beta * prior[i];
   data[i] = v;
 }

@@ -355,22 +355,96 @@ template <typename T>
 int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
                     const snn_hip_conv2d_params* params, int algorithm,
                     T* workspace, size_t workspace_elems, void* stream,
-                    const ConvEpilogue* epilogue = nullptr) {
+                    const ConvEpilogue* epilogue = nullptr);
+
+// NCHW activations with an FCHW filter (the only filter layout portDNN
+// accepts with NCHW, include/portdnn/internal/conv2d/launch.h:86-88): the
+// operands are rewritten as NHWC / HWCF into stream-ordered temporaries, the
+// convolution runs on them and the result is written back in the caller's
+// layout.  Only fp32.
+template <typename T>
+int conv2d_nchw(int, const T*, const T*, T*, const snn_hip_conv2d_params&,
+                int, hipStream_t) {
+  return SNN_HIP_INVALID_ALGORITHM;
+}
+template <>
+int conv2d_nchw<float>(int direction, const float* input, const float* filter,
+                       float* output, const snn_hip_conv2d_params& p,
+                       int algorithm, hipStream_t s) {
+  const ConvSizes sz = conv_sizes(p, direction);
+  const int taps = p.window_rows * p.window_cols;
+  const int in_hw = p.in_rows * p.in_cols, out_hw = p.out_rows * p.out_cols;
+  float* tmp = nullptr;
+  if (hipMallocAsync(reinterpret_cast<void**>(&tmp),
+                     (sz.input + sz.filter + sz.output) * sizeof(float), s) !=
+      hipSuccess)
+    return SNN_HIP_ALLOCATION_PROBLEM;
+  float* t_in = tmp;
+  float* t_fil = tmp + sz.input;
+  float* t_out = t_fil + sz.filter;
+  // operand roles per direction (include/snn_hip.h): tensor shapes as
+  // (batches, channels, pixels) for the activations
+  struct Act { int c, hw; };
+  const Act x{p.channels, in_hw}, y{p.features, out_hw};
+  const Act in_a = direction == SNN_HIP_INPUT_BACKPROP ? y : x;
+  const bool fil_is_filter = direction != SNN_HIP_FILTER_BACKPROP;
+  const Act out_a = direction == SNN_HIP_FORWARD ? y : x;
+  int rc = launch_transpose_batched_f32(input, t_in, p.batch, in_a.c, in_a.hw,
+                                        s);
+  if (rc == SNN_HIP_OK)
+    rc = fil_is_filter
+             ? launch_permute_filter_f32(filter, t_fil, p.features, p.channels,
+                                         taps, true, s)
+             : launch_transpose_batched_f32(filter, t_fil, p.batch, y.c, y.hw,
+                                            s);
+  if (rc == SNN_HIP_OK) {
+    snn_hip_conv2d_params q = p;
+    q.input_format = 0;
+    q.filter_format = 0;
+    rc = conv2d_dispatch<float>(direction, t_in, t_fil, t_out, &q, algorithm,
+                                nullptr, 0, s);
+  }
+  if (rc == SNN_HIP_OK)
+    rc = direction == SNN_HIP_FILTER_BACKPROP
+             ? launch_permute_filter_f32(t_out, output, p.features, p.channels,
+                                         taps, false, s)
+             : launch_transpose_batched_f32(t_out, output, p.batch, out_a.hw,
+                                            out_a.c, s);
+  (void)hipFreeAsync(tmp, s);
+  return rc;
+}
+
+template <typename T>
+int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
+                    const snn_hip_conv2d_params* params, int algorithm,
+                    T* workspace, size_t workspace_elems, void* stream,
+                    const ConvEpilogue* epilogue) {
   if (params == nullptr) return SNN_HIP_INVALID_PARAMETER;
   const snn_hip_conv2d_params& p = *params;
   const int v = validate(p);
   if (v != SNN_HIP_OK) return v;
   if (input == nullptr || filter == nullptr || output == nullptr)
     return SNN_HIP_INVALID_PARAMETER;
-  // Grouped, NCHW and FHWC convolutions are outside this library.
-  if (p.groups != 1 || p.input_format != 0 || p.filter_format != 0)
-    return SNN_HIP_INVALID_ALGORITHM;
+  // Grouped and FHWC convolutions are outside this library.
+  if (p.groups != 1 || p.filter_format == 2) return SNN_HIP_INVALID_ALGORITHM;
+  // include/portdnn/internal/conv2d/launch.h:81-88: NHWC goes with HWCF,
+  // NCHW with FCHW.
+  if ((p.input_format == 0) != (p.filter_format == 0))
+    return SNN_HIP_INVALID_PARAMETER;
   if (algorithm_supports(p, direction, algorithm) == SNN_HIP_ALGO_NOT_SUPPORTED)
     return SNN_HIP_INVALID_ALGORITHM;
   const ConvSizes sz = conv_sizes(p, direction);
   if (!fits_int32(sz.input) || !fits_int32(sz.filter) || !fits_int32(sz.output))
     return SNN_HIP_INDEX_EXCEEDED;
   hipStream_t s = as_stream(stream);
+  if (p.input_format != 0) {
+    // include/portdnn/internal/conv2d/launch.h:191-194: NCHW is served by the
+    // Direct algorithm only.
+    if (algorithm != SNN_HIP_ALGO_DIRECT) return SNN_HIP_INVALID_ALGORITHM;
+    if (epilogue != nullptr && epilogue->wanted())
+      return SNN_HIP_INVALID_ALGORITHM;  // bias is indexed by the last dim
+    return conv2d_nchw<T>(direction, input, filter, output, p, algorithm, s);
+  }
   switch (algorithm) {
     case SNN_HIP_ALGO_WINOGRAD:
     case SNN_HIP_ALGO_WINOGRAD_LARGE:
@@ -663,6 +737,14 @@ int snn_hip_conv2d_forward_bias_act_f32(
                    params->out_cols * params->features;
   return launch_bias_act_f32(output, bias, params->features, n, epilogue.relu,
                              as_stream(stream));
+}
+
+int snn_hip_scale_blend_f32(float* data, const float* prior, float alpha,
+                            float beta, size_t n_items, void* stream) {
+  if (data == nullptr || n_items == 0 || (beta != 0.f && prior == nullptr))
+    return SNN_HIP_INVALID_PARAMETER;
+  return launch_scale_blend_f32(data, prior, alpha, beta, n_items,
+                                as_stream(stream));
 }
 
 int snn_hip_pointwise_forward_f32(const float* input, float* output,

@@ -136,6 +136,15 @@ int launch_bias_act_f32(float* data, const float* bias, int features, size_t n,
 int launch_scale_blend_f32(float* data, const float* prior, float alpha,
                            float beta, size_t n, hipStream_t stream);
 
+// Layout conversions (layout.hip).  out[b][c][r] = in[b][r][c] for every
+// batch b (NCHW -> NHWC with rows = C, cols = H * W, and back with the two
+// swapped); FCHW <-> HWCF filters with taps = R * S.
+int launch_transpose_batched_f32(const float* in, float* out, int batches,
+                                 int rows, int cols, hipStream_t stream);
+int launch_permute_filter_f32(const float* in, float* out, int features,
+                              int channels, int taps, bool to_hwcf,
+                              hipStream_t stream);
+
 }  // namespace snn
 
 #endif  // PORTDNN_AMD_CSRC_SNN_KERNELS_H_

@@ -6,6 +6,7 @@
 // with the CPU oracle (which the golden tests pin to the reference's vectors).
 #include <portdnn/backend/hip_backend.h>
 #include <portdnn/binaryop/launch.h>
+#include <portdnn/compat/convolution.hpp>
 #include <portdnn/conv2d/launch.h>
 #include <portdnn/conv2d/selector/default_selector.h>
 #include <portdnn/conv2d/selector/direct_selector.h>
@@ -401,6 +402,193 @@ static void test_elementwise(backend::HIPBackend& backend) {
              backend).status == StatusCode::InvalidParameter));
 }
 
+// test/compat/conv2d_forward_compat.cc:77-172 (fixture) with its hand-written
+// cases :174-446: operands and the initial output are 1,2,3,... (max 2048).
+static void compat_case(compat::SNNHandle& handle, std::vector<int> in_sizes,
+                        std::vector<int> filt_sizes, std::vector<int> conv,
+                        std::vector<float> expect, DataFormat format,
+                        conv2d::Algorithm algo, float alpha, float beta,
+                        StatusCode want = StatusCode::OK, int groups = 1) {
+  using namespace compat;
+  backend::HIPBackend& backend = handle.getBackend();
+  TensorDescriptor x_desc, y_desc;
+  FilterDescriptor w_desc;
+  ConvolutionDescriptor c_desc;
+  CHECK(x_desc.set4d(format, in_sizes[0], in_sizes[1], in_sizes[2],
+                     in_sizes[3]) == StatusCode::OK);
+  CHECK(w_desc.set4d(format, filt_sizes[0], filt_sizes[1], filt_sizes[2],
+                     filt_sizes[3]) == StatusCode::OK);
+  CHECK(c_desc.set2d(conv[0], conv[1], conv[2], conv[3], conv[4], conv[5]) ==
+        StatusCode::OK);
+  if (groups > 1) CHECK(setConvolutionGroupCount(c_desc, groups) == StatusCode::OK);
+  int n, c, h, w;
+  CHECK(getConvolution2dForwardOutputDim(c_desc, x_desc, w_desc, &n, &c, &h,
+                                         &w) == StatusCode::OK);
+  CHECK(y_desc.set4d(format, n, c, h, w) == StatusCode::OK);
+  DeviceBuffer d_x(backend, iota_data(x_desc.getSize(), 2048));
+  DeviceBuffer d_w(backend, iota_data(w_desc.getSize(), 2048));
+  DeviceBuffer d_y(backend, iota_data(y_desc.getSize(), 2048));
+  SNNStatus st = convolutionForward(handle, &alpha, x_desc, d_x.ptr, w_desc,
+                                    d_w.ptr, c_desc, algo, nullptr, 0, &beta,
+                                    y_desc, d_y.ptr);
+  CHECK(st.status == want);
+  if (want != StatusCode::OK) return;
+  st.event.wait_and_throw();
+  const bool ok = close(d_y.host(), expect, true);
+  if (!ok) std::printf("  compat case alpha %g beta %g\n", alpha, beta);
+  CHECK(ok);
+}
+
+// conv + bias + ReLU in one launch against the reference's three.
+static void test_bias_activation(backend::HIPBackend& backend) {
+  Conv2DParams p{};
+  p.channels = 64; p.features = 96; p.batch = 2;
+  p.in_rows = p.in_cols = 14;
+  p.window_rows = p.window_cols = 3;
+  p.stride_rows = p.stride_cols = 1;
+  p = helpers::add_padding_to(p, PaddingMode::SAME);
+  const auto sizes = conv2d::get_sizes<ct::Forward>(p);
+  const auto x = uniform_data(sizes.input_size, 21);
+  const auto w = uniform_data(sizes.filter_size, 22);
+  const auto b = uniform_data(p.features, 23);
+  DeviceBuffer d_x(backend, x), d_w(backend, w), d_b(backend, b);
+  DeviceBuffer d_fused(backend, sizes.output_size),
+      d_three(backend, sizes.output_size);
+  conv2d::WinogradSelector wino;
+  const auto ws = conv2d::query_workspace_size<ct::Forward>(p, wino);
+  DeviceBuffer d_ws(backend, ws.recommended_size);
+  auto st = conv2d::launch_forward_bias_activation<float>(
+      d_x.ptr, d_w.ptr, d_b.ptr, d_fused.ptr, p, wino, backend, d_ws.ptr,
+      ws.recommended_size, conv2d::Activation::Relu);
+  CHECK(st.status == StatusCode::OK);
+  st = conv2d::launch<float, ct::Forward>(d_x.ptr, d_w.ptr, d_three.ptr, p,
+                                          wino, backend, d_ws.ptr,
+                                          ws.recommended_size);
+  CHECK(st.status == StatusCode::OK);
+  st = binaryop::launch<float, binaryop::Add>(
+      d_three.ptr, d_b.ptr, d_three.ptr,
+      binaryop::BinaryParams{{p.batch, p.out_rows, p.out_cols, p.features},
+                             {p.features}},
+      backend);
+  CHECK(st.status == StatusCode::OK);
+  st = pointwise::launch<float, pointwise::Relu, pointwise::Forward>(
+      d_three.ptr, d_three.ptr, sizes.output_size, backend);
+  CHECK(st.status == StatusCode::OK);
+  st.event.wait_and_throw();
+  CHECK(close(d_fused.host(), d_three.host(), true));
+}
+
+static void test_compat(hipStream_t stream) {
+  using namespace compat;
+  using A = conv2d::Algorithm;
+  // test/compat/conv2d_forward_compat.cc:25-67
+  ConvolutionDescriptor desc;
+  CHECK(setConvolution2dDescriptor(desc, 1, 2, 3, 4, 1, 1,
+                                   ConvolutionMode::CROSS_CORRELATION) ==
+        StatusCode::OK);
+  CHECK(desc.getPadH() == 1 && desc.getPadW() == 2 && desc.getStrideH() == 3 &&
+        desc.getStrideW() == 4 && desc.getDilationH() == 1 &&
+        desc.getMode() == ConvolutionMode::CROSS_CORRELATION);
+  CHECK(desc.set2d(-1, 0, 1, 1, 1, 1) == StatusCode::InvalidParameter);
+  CHECK(desc.set2d(0, 0, 1, 1, 1, 1, ConvolutionMode::CONVOLUTION) ==
+        StatusCode::InvalidParameter);
+  setConvolutionGroupCount(desc, 5);
+  CHECK(desc.getGroupCount() == 5);
+
+  SNNHandle handle;
+  CHECK(SNNCreate(handle, stream) == StatusCode::OK);
+  const DataFormat nhwc = DataFormat::NHWC, nchw = DataFormat::NCHW;
+  const std::vector<int> unit = {0, 0, 1, 1, 1, 1};
+  compat_case(handle, {1, 1, 4, 4}, {1, 1, 3, 3}, unit, {348, 393, 528, 573},
+              nhwc, A::Direct, 1.f, 0.f);
+  compat_case(handle, {2, 3, 1, 1}, {1, 3, 1, 1}, unit, {14, 32}, nhwc,
+              A::Direct, 1.f, 0.f);
+  compat_case(handle, {1, 1, 1, 1}, {1, 1, 3, 3}, {1, 1, 1, 1, 1, 1}, {5},
+              nhwc, A::Direct, 1.f, 0.f);
+  compat_case(handle, {1, 3, 1, 1}, {1, 3, 3, 3}, {1, 1, 1, 1, 1, 1}, {86},
+              nhwc, A::Direct, 1.f, 0.f);
+  compat_case(handle, {1, 1, 5, 5}, {1, 1, 3, 3}, {0, 0, 2, 2, 1, 1},
+              {411, 501, 861, 951}, nchw, A::Direct, 1.f, 0.f);
+  compat_case(handle, {1, 1, 11, 11}, {2, 1, 7, 7}, {2, 2, 4, 4, 1, 1},
+              {48425., 49050., 72800., 73780., 55075., 55850., 125230.,
+               127260., 177037., 180026., 126980., 129220., 91975., 94250.,
+               126210., 129500., 87825., 90250.},
+              nhwc, A::Im2col, 1.f, 0.f);
+  // alpha / beta, :285-446
+  compat_case(handle, {1, 1, 4, 4}, {1, 1, 3, 3}, unit, {696, 786, 1056, 1146},
+              nhwc, A::Direct, 2.f, 0.f);
+  compat_case(handle, {1, 1, 4, 4}, {1, 1, 3, 3}, unit, {0, 0, 0, 0}, nhwc,
+              A::Direct, 0.f, 0.f);
+  compat_case(handle, {1, 1, 4, 4}, {1, 1, 3, 3}, unit,
+              {-696, -786, -1056, -1146}, nhwc, A::Direct, -2.f, 0.f);
+  compat_case(handle, {1, 1, 4, 4}, {1, 1, 3, 3}, unit, {349, 395, 531, 577},
+              nhwc, A::Direct, 1.f, 1.f);
+  compat_case(handle, {1, 1, 4, 4}, {1, 1, 3, 3}, unit, {1, 2, 3, 4}, nhwc,
+              A::Direct, 0.f, 1.f);
+  compat_case(handle, {1, 1, 4, 4}, {1, 1, 3, 3}, unit, {2, 4, 6, 8}, nhwc,
+              A::Direct, 0.f, 2.f);
+  compat_case(handle, {1, 1, 4, 4}, {1, 1, 3, 3}, unit, {-2, -4, -6, -8}, nhwc,
+              A::Direct, 0.f, -2.f);
+  // both factors at once: 3 * conv - 2 * prior
+  compat_case(handle, {1, 1, 4, 4}, {1, 1, 3, 3}, unit,
+              {3 * 348 - 2, 3 * 393 - 4, 3 * 528 - 6, 3 * 573 - 8}, nhwc,
+              A::Direct, 3.f, -2.f);
+  // grouped convolutions are not provided
+  compat_case(handle, {1, 2, 5, 5}, {2, 1, 2, 2}, unit, {}, nhwc, A::Im2col,
+              1.f, 0.f, StatusCode::InvalidAlgorithm, 2);
+  // NCHW runs on Direct only (internal/conv2d/launch.h:191-194)
+  compat_case(handle, {1, 1, 5, 5}, {1, 1, 3, 3}, {0, 0, 2, 2, 1, 1}, {}, nchw,
+              A::Im2col, 1.f, 0.f, StatusCode::InvalidAlgorithm);
+
+  // workspace size in bytes = recommended elements * sizeof(float)
+  TensorDescriptor x_desc, y_desc;
+  FilterDescriptor w_desc;
+  ConvolutionDescriptor c_desc;
+  x_desc.set4d(nhwc, 2, 64, 28, 28);
+  w_desc.set4d(nhwc, 64, 64, 3, 3);
+  c_desc.set2d(1, 1, 1, 1, 1, 1);
+  int n, c, h, w;
+  getConvolution2dForwardOutputDim(c_desc, x_desc, w_desc, &n, &c, &h, &w);
+  CHECK(n == 2 && c == 64 && h == 28 && w == 28);
+  y_desc.set4d(nhwc, n, c, h, w);
+  size_t bytes = 0;
+  CHECK(getConvolutionForwardWorkspaceSize(handle, x_desc, w_desc, c_desc,
+                                           y_desc, A::Winograd, &bytes) ==
+        StatusCode::OK);
+  conv2d::WinogradSelector wino;
+  const auto ws = conv2d::query_workspace_size<ct::Forward>(
+      compat::internal::descToSnnParams(x_desc, y_desc, w_desc, c_desc), wino);
+  CHECK(bytes == ws.recommended_size * sizeof(float) && bytes > 0);
+
+  // backward data / filter against the oracle, NHWC, with a blend
+  const auto x = uniform_data(x_desc.getSize(), 11);
+  const auto wt = uniform_data(w_desc.getSize(), 12);
+  const auto dy = uniform_data(y_desc.getSize(), 13);
+  backend::HIPBackend& backend = handle.getBackend();
+  DeviceBuffer d_x(backend, x), d_w(backend, wt), d_dy(backend, dy);
+  const auto dx0 = uniform_data(x_desc.getSize(), 14);
+  const auto dw0 = uniform_data(w_desc.getSize(), 15);
+  DeviceBuffer d_dx(backend, dx0), d_dw(backend, dw0);
+  const float alpha = 0.5f, beta = 2.f;
+  auto st = convolutionBackwardData(handle, &alpha, w_desc, d_w.ptr, y_desc,
+                                    d_dy.ptr, c_desc, A::Im2col, nullptr, 0,
+                                    &beta, x_desc, d_dx.ptr);
+  CHECK(st.status == StatusCode::OK);
+  st = convolutionBackwardFilter(handle, &alpha, x_desc, d_x.ptr, y_desc,
+                                 d_dy.ptr, c_desc, A::Im2col, nullptr, 0, &beta,
+                                 w_desc, d_dw.ptr);
+  CHECK(st.status == StatusCode::OK);
+  st.event.wait_and_throw();
+  oracle_params op{64, 64, 2, 28, 28, 3, 3, 1, 1, 28, 28, 1, 1};
+  std::vector<float> dx(x.size()), dw(wt.size());
+  oracle_conv2d_input_backprop(dy.data(), wt.data(), dx.data(), &op, 1);
+  oracle_conv2d_filter_backprop(x.data(), dy.data(), dw.data(), &op, 1);
+  for (size_t i = 0; i < dx.size(); ++i) dx[i] = alpha * dx[i] + beta * dx0[i];
+  for (size_t i = 0; i < dw.size(); ++i) dw[i] = alpha * dw[i] + beta * dw0[i];
+  CHECK(close(d_dx.host(), dx, false));
+  CHECK(close(d_dw.host(), dw, false));
+}
+
 int main() {
   int n = 0;
   if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
@@ -417,7 +605,9 @@ int main() {
     test_event_dependencies(backend);
     test_matmul(backend);
     test_elementwise(backend);
+    test_bias_activation(backend);
   }
+  test_compat(stream);
   (void)hipStreamDestroy(stream);
   return report("gpu_api_test");
 }

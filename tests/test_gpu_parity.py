@@ -766,3 +766,80 @@ def test_conv2d_bias_activation_rejects_unknown_activation():
         x.data_ptr(), w.data_ptr(), None, y.data_ptr(), ctypes.byref(p),
         ALGO.DIRECT, 7, None, 0, None)
     assert rc == STATUS.INVALID_PARAMETER
+
+
+# ---- NCHW / FCHW operands ------------------------------------------------------
+
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, window, stride, same
+    (2, 9, 11, 5, 7, 3, 1, True),
+    (3, 12, 8, 16, 24, 3, 2, True),
+    (1, 37, 41, 3, 8, 7, 2, True),      # tiles of the transposes are ragged
+    (2, 6, 6, 40, 33, 1, 1, False),
+])
+@pytest.mark.parametrize("direction", [DIRECTION.FORWARD,
+                                       DIRECTION.INPUT_BACKPROP,
+                                       DIRECTION.FILTER_BACKPROP])
+def test_conv2d_nchw_fchw(shape, direction):
+    """DataFormat::NCHW with FilterFormat::FCHW through the Direct algorithm
+    (include/portdnn/internal/conv2d/launch.h:86-88, :191-194) against the
+    NHWC / HWCF oracle on permuted operands."""
+    batch, rows, cols, ch, feats, window, stride, same = shape
+    p = ops.add_padding_to(ops.ConvParams(
+        channels=ch, features=feats, batch=batch, in_rows=rows, in_cols=cols,
+        window_rows=window, window_cols=window, stride_rows=stride,
+        stride_cols=stride), same)
+    rng = np.random.default_rng(1100 + rows)
+    x = uniform(rng, batch * rows * cols * ch).reshape(batch, rows, cols, ch)
+    w = uniform(rng, window * window * ch * feats).reshape(window, window, ch,
+                                                           feats)
+    dy = uniform(rng, batch * p.out_rows * p.out_cols * feats).reshape(
+        batch, p.out_rows, p.out_cols, feats)
+    op = oracle_params(p, feats)
+    nchw = lambda t: np.ascontiguousarray(t.transpose(0, 3, 1, 2)).reshape(-1)
+    fchw = lambda t: np.ascontiguousarray(t.transpose(3, 2, 0, 1)).reshape(-1)
+    if direction == DIRECTION.FORWARD:
+        a, b = nchw(x), fchw(w)
+        ref = nchw(oracle.conv2d_forward(x, w, op).reshape(dy.shape))
+    elif direction == DIRECTION.INPUT_BACKPROP:
+        a, b = nchw(dy), fchw(w)
+        ref = nchw(oracle.conv2d_input_backprop(dy, w, op).reshape(x.shape))
+    else:
+        a, b = nchw(x), nchw(dy)
+        ref = fchw(oracle.conv2d_filter_backprop(x, dy, op).reshape(w.shape))
+    q = ops.ConvParams(**{f: getattr(p, f) for f, _ in p._fields_})
+    q.input_format, q.filter_format = 1, 1
+    got = ops.conv2d(dev(a), dev(b), q, direction, ALGO.DIRECT).cpu().numpy()
+    assert_close(got, ref, ("nchw", shape, direction))
+    # any other algorithm is refused for NCHW
+    out = torch.empty(ref.size, device="cuda")
+    assert ops.conv2d_raw(dev(a), dev(b), out, q, direction, ALGO.IM2COL) == \
+        STATUS.INVALID_ALGORITHM
+    # NCHW with an HWCF filter is an invalid combination
+    q.filter_format = 0
+    assert ops.conv2d_raw(dev(a), dev(b), out, q, direction, ALGO.DIRECT) == \
+        STATUS.INVALID_PARAMETER
+
+
+def test_scale_blend():
+    """snn_hip_scale_blend_f32: y = alpha * y + beta * prior, the scaling step
+    of the cuDNN-style layer (include/portdnn/compat/scaling.hpp:150-262)."""
+    rng = np.random.default_rng(1200)
+    y, prior = uniform(rng, 4099), uniform(rng, 4099)
+    L = capi.lib()
+    for alpha, beta in ((2.0, 0.0), (1.0, 1.0), (-0.5, 3.0), (0.0, 2.0)):
+        d = dev(y)
+        rc = L.snn_hip_scale_blend_f32(d.data_ptr(), dev(prior).data_ptr(),
+                                       alpha, beta, y.size, None)
+        assert rc == STATUS.OK
+        torch.cuda.synchronize()
+        ref = (np.float32(alpha) * y if alpha else 0 * y) + \
+            np.float32(beta) * prior
+        assert np.allclose(d.cpu().numpy(), ref, rtol=1e-6, atol=1e-7)
+    # a zero alpha drops the data term even when it holds NaN
+    d = dev(np.full(16, np.nan, dtype=np.float32))
+    assert L.snn_hip_scale_blend_f32(d.data_ptr(), None, 0.0, 0.0, 16,
+                                     None) == STATUS.OK
+    assert np.array_equal(d.cpu().numpy(), np.zeros(16, dtype=np.float32))
+    assert L.snn_hip_scale_blend_f32(d.data_ptr(), None, 1.0, 1.0, 16,
+                                     None) == STATUS.INVALID_PARAMETER
