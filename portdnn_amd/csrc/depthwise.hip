@@ -538,41 +538,66 @@ __global__ void __launch_bounds__(kStrip* kSlices)
   }
 }
 
-// Launches the 3x3 strip kernel with V channels per lane.  Output rows per
-// lane: as many as still leave every CU a few thousand lanes (measured best:
-// 8 rows x 1 column for the large layers).
+// Launches the 3x3 strip kernel with V channels per lane and a TH x TW block
+// of outputs per lane.  A lane loads (TH + 2)(TW + 2) input vectors for
+// TH * TW outputs (stride 1), so larger blocks cut the L1 traffic, but fewer
+// lanes remain and, with TW = 2, a wave's loads spread over twice as many
+// cache lines.  Measured best on MI355X at batch 32 / 128:
+//   stride 1: TW = 2 once a pixel's channel vectors fill a 128-byte line,
+//             TH = 4 for images of 28 rows and more, else 8 (4 with V = 8);
+//   stride 2: TW = 1, TH = 2 for outputs of 56 rows and more, else 8 (4).
 template <typename T, int V, bool FLIP>
 void launch_dw_strip(const T* input, const T* filter, T* output,
                      const snn_hip_depthwise_params& p, hipStream_t stream) {
   constexpr int kBlock = 256;
-  constexpr int kTw = 1;
-  const int n_col_blocks = ceil_div(p.out_cols, kTw);
-  const size_t per_row = static_cast<size_t>(p.batch) * n_col_blocks *
-                         (p.channels / V);
-  int th = V == 8 ? 4 : 8;  // 8 rows x 8 channels would need ~250 registers
-  while (th > 1 && per_row * ceil_div(p.out_rows, th) < 150000) th /= 2;
-  // Developer override for tuning runs: SNN_HIP_DW_TH=<1|2|4|8>.
-  static const char* tune = getenv("SNN_HIP_DW_TH");
-  if (tune != nullptr && tune[0] != 0) th = max(1, min(8, atoi(tune)));
-  if (th != 1 && th != 2 && th != 4) th = th >= 8 ? 8 : 4;
-  const int n_strips = ceil_div(p.out_rows, th);
-  const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
-  const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
-#define SNN_DW_STRIP(STRIDE, TH)                                               \
-  hipLaunchKernelGGL((dw_forward_3x3_strip_kernel<T, STRIDE, TH, kTw, FLIP, V>), \
-                     grid, dim3(kBlock), 0, stream, input, filter, output, p,  \
-                     n_strips, n_col_blocks, n_items)
+  const int cv = p.channels / V;
+  const int th_max = V == 8 ? 4 : 8;  // 8 rows x 8 channels: ~250 registers
+  int th, tw;
   if (p.stride_rows == 1) {
-    if (th == 8) SNN_DW_STRIP(1, 8);
-    else if (th == 4) SNN_DW_STRIP(1, 4);
-    else if (th == 2) SNN_DW_STRIP(1, 2);
-    else SNN_DW_STRIP(1, 1);
+    tw = cv * 16 >= 128 ? 2 : 1;
+    th = p.out_rows >= 28 ? 4 : th_max;
   } else {
-    if (th == 8) SNN_DW_STRIP(2, 8);
-    else if (th == 4) SNN_DW_STRIP(2, 4);
-    else if (th == 2) SNN_DW_STRIP(2, 2);
-    else SNN_DW_STRIP(2, 1);
+    tw = 1;
+    th = p.out_rows >= 56 ? 2 : th_max;
   }
+  // Developer overrides for tuning runs: SNN_HIP_DW_TH=<1|2|4|8>,
+  // SNN_HIP_DW_TW=<1|2>.
+  static const char* tune_th = getenv("SNN_HIP_DW_TH");
+  static const char* tune_tw = getenv("SNN_HIP_DW_TW");
+  if (tune_th != nullptr && tune_th[0] != 0) th = atoi(tune_th);
+  if (tune_tw != nullptr && tune_tw[0] != 0) tw = atoi(tune_tw);
+  tw = tw >= 2 ? 2 : 1;
+  th = th >= 8 ? 8 : th >= 4 ? 4 : th >= 2 ? 2 : 1;
+  if (th > th_max) th = th_max;
+  const int n_col_blocks = ceil_div(p.out_cols, tw);
+  const int n_strips = ceil_div(p.out_rows, th);
+  const unsigned n_items = static_cast<unsigned>(
+      static_cast<size_t>(p.batch) * n_col_blocks * cv * n_strips);
+  const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
+#define SNN_DW_STRIP(STRIDE, TH, TW)                                            \
+  hipLaunchKernelGGL((dw_forward_3x3_strip_kernel<T, STRIDE, TH, TW, FLIP, V>), \
+                     grid, dim3(kBlock), 0, stream, input, filter, output, p,   \
+                     n_strips, n_col_blocks, n_items)
+#define SNN_DW_STRIP_TH(STRIDE, TW)                      \
+  do {                                                   \
+    if (th == 8) {                                       \
+      if constexpr (V != 8) SNN_DW_STRIP(STRIDE, 8, TW); \
+    } else if (th == 4) {                                \
+      SNN_DW_STRIP(STRIDE, 4, TW);                       \
+    } else if (th == 2) {                                \
+      SNN_DW_STRIP(STRIDE, 2, TW);                       \
+    } else {                                             \
+      SNN_DW_STRIP(STRIDE, 1, TW);                       \
+    }                                                    \
+  } while (0)
+  if (p.stride_rows == 1) {
+    if (tw == 2) SNN_DW_STRIP_TH(1, 2);
+    else SNN_DW_STRIP_TH(1, 1);
+  } else {
+    if (tw == 2) SNN_DW_STRIP_TH(2, 2);
+    else SNN_DW_STRIP_TH(2, 1);
+  }
+#undef SNN_DW_STRIP_TH
 #undef SNN_DW_STRIP
 }
 
