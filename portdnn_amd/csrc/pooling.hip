@@ -565,6 +565,147 @@ int launch_forward_op(const T* input, T* output,
   return SNN_HIP_OK;
 }
 
+// Max gradient for small square windows (WIN x WIN, stride STRIDE), four
+// channels per lane.  The per-element kernel above re-scans a window for
+// every input element that ties with its maximum; here a work-group owns a
+// 16 x 16 tile of input pixels and up to 64 channels:
+//   1. every window that touches the tile is scanned once (row-major, clipped
+//      to the image) for the first element equal to the forward output -- the
+//      reference's tie rule (src/pooling/kernels.h:197-239) -- and the
+//      position WIN * r + c (255: none) of each channel goes to LDS;
+//   2. every input element of the tile looks up the windows that cover it and
+//      takes dY of those whose recorded position is its own.
+// Windows on the tile border are scanned by both neighbouring tiles; nothing
+// is accumulated across work-groups, so no atomics and no zero fill.
+constexpr int kGradTile = 16;
+template <int WIN, int STRIDE>
+__global__ void __launch_bounds__(256)
+    pool_max_grad_tile_kernel(const float* __restrict__ in,
+                              const float* __restrict__ out,
+                              const float* __restrict__ dy,
+                              float* __restrict__ dx, snn_hip_pooling_params p,
+                              bool nan_mode, int tiles_x, int tiles_y,
+                              int cv_per_group) {
+  // windows per dimension that can touch 16 consecutive input rows / columns
+  constexpr int NW = (kGradTile + WIN - 2) / STRIDE + 2;
+  constexpr int kMaxCv = 16;
+  __shared__ unsigned int first_pos[NW * NW * kMaxCv];  // 4 channel bytes each
+
+  const int C = p.channels;
+  int t = blockIdx.x;
+  const int tx = t % tiles_x;
+  t /= tiles_x;
+  const int ty = t % tiles_y;
+  const int n = t / tiles_y;
+  const int cv0 = blockIdx.y * cv_per_group;
+  const int cvl = threadIdx.x % cv_per_group;
+  const int lane_w = threadIdx.x / cv_per_group;
+  const int n_lanes_w = 256 / cv_per_group;
+  const int ch = (cv0 + cvl) * 4;
+  const bool ch_ok = ch < C;
+
+  const int iy0 = ty * kGradTile, ix0 = tx * kGradTile;
+  // first window (per dimension) whose unclipped extent reaches the tile
+  auto first_window = [](int i0, int pad) {
+    const int v = i0 + pad - WIN + 1;  // smallest o with o*STRIDE - pad + WIN - 1 >= i0
+    return v <= 0 ? 0 : (v + STRIDE - 1) / STRIDE;
+  };
+  const int oy0 = first_window(iy0, p.pad_rows);
+  const int ox0 = first_window(ix0, p.pad_cols);
+  const size_t in_base =
+      static_cast<size_t>(n) * p.in_rows * p.in_cols * C + ch;
+  const size_t out_base =
+      static_cast<size_t>(n) * p.out_rows * p.out_cols * C + ch;
+
+  for (int w = lane_w; w < NW * NW; w += n_lanes_w) {
+    const int oy = oy0 + w / NW, ox = ox0 + w % NW;
+    unsigned int packed = 0xFFFFFFFFu;
+    if (ch_ok && oy < p.out_rows && ox < p.out_cols) {
+      float target[4];
+      GradVec<4>::load(
+          out + out_base + (static_cast<size_t>(oy) * p.out_cols + ox) * C,
+          target);
+      unsigned int pos[4] = {255u, 255u, 255u, 255u};
+      const int r_in = oy * STRIDE - p.pad_rows;
+      const int c_in = ox * STRIDE - p.pad_cols;
+#pragma unroll
+      for (int r = 0; r < WIN; ++r) {
+#pragma unroll
+        for (int c = 0; c < WIN; ++c) {
+          const int iy = r_in + r, ix = c_in + c;
+          if (static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_rows) &&
+              static_cast<unsigned>(ix) < static_cast<unsigned>(p.in_cols)) {
+            float v[4];
+            GradVec<4>::load(
+                in + in_base + (static_cast<size_t>(iy) * p.in_cols + ix) * C,
+                v);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (pos[i] == 255u && pool_equal(v[i], target[i], nan_mode))
+                pos[i] = static_cast<unsigned>(r * WIN + c);
+          }
+        }
+      }
+      packed = pos[0] | (pos[1] << 8) | (pos[2] << 16) | (pos[3] << 24);
+    }
+    first_pos[w * kMaxCv + cvl] = packed;
+  }
+  __syncthreads();
+
+  if (!ch_ok) return;
+  for (int pix = lane_w; pix < kGradTile * kGradTile; pix += n_lanes_w) {
+    const int iy = iy0 + pix / kGradTile, ix = ix0 + pix % kGradTile;
+    if (iy >= p.in_rows || ix >= p.in_cols) continue;
+    float grad[4] = {0.f, 0.f, 0.f, 0.f};
+    // windows whose unclipped extent contains (iy, ix)
+    const int py = iy + p.pad_rows, px = ix + p.pad_cols;
+    const int oy_begin = py < WIN ? 0 : (py - WIN) / STRIDE + 1;
+    const int oy_end = min(py / STRIDE + 1, p.out_rows);
+    const int ox_begin = px < WIN ? 0 : (px - WIN) / STRIDE + 1;
+    const int ox_end = min(px / STRIDE + 1, p.out_cols);
+    for (int oy = oy_begin; oy < oy_end; ++oy) {
+      for (int ox = ox_begin; ox < ox_end; ++ox) {
+        const unsigned int mine = static_cast<unsigned>(
+            (py - oy * STRIDE) * WIN + (px - ox * STRIDE));
+        const unsigned int packed =
+            first_pos[((oy - oy0) * NW + (ox - ox0)) * kMaxCv + cvl];
+        bool hit[4];
+        bool any = false;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          hit[i] = ((packed >> (8 * i)) & 255u) == mine;
+          any |= hit[i];
+        }
+        if (!any) continue;
+        float g[4];
+        GradVec<4>::load(
+            dy + out_base + (static_cast<size_t>(oy) * p.out_cols + ox) * C, g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (hit[i]) grad[i] += g[i];
+      }
+    }
+    GradVec<4>::store(
+        dx + in_base + (static_cast<size_t>(iy) * p.in_cols + ix) * C, grad);
+  }
+}
+
+template <int WIN, int STRIDE>
+void launch_max_grad_tile(const float* in, const float* out, const float* dy,
+                          float* dx, const snn_hip_pooling_params& p,
+                          bool nan_mode, hipStream_t stream) {
+  const int cv = p.channels / 4;
+  int cv_per_group = 16;
+  while (cv_per_group > 1 && cv_per_group / 2 >= cv) cv_per_group /= 2;
+  const int tiles_x = ceil_div(p.in_cols, kGradTile);
+  const int tiles_y = ceil_div(p.in_rows, kGradTile);
+  const dim3 grid(static_cast<unsigned>(p.batch * tiles_y * tiles_x),
+                  static_cast<unsigned>(ceil_div(cv, cv_per_group)));
+  hipLaunchKernelGGL((pool_max_grad_tile_kernel<WIN, STRIDE>), grid, dim3(256),
+                     0, stream, in, out, dy, dx, p, nan_mode, tiles_x, tiles_y,
+                     cv_per_group);
+}
+
 }  // namespace
 
 template <typename T>
@@ -603,9 +744,26 @@ int launch_pooling_max_grad(const float* input_data, const float* output_data,
   const size_t n_in =
       static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
   const bool nan_mode = op == SNN_HIP_POOL_MAX_WITH_NAN;
-  if (p.channels % 4 == 0 && grad_aligned16(input_data) &&
-      grad_aligned16(output_data) && grad_aligned16(input_backprop) &&
-      grad_aligned16(output_backprop)) {
+  const bool vec4 = p.channels % 4 == 0 && grad_aligned16(input_data) &&
+                    grad_aligned16(output_data) &&
+                    grad_aligned16(input_backprop) &&
+                    grad_aligned16(output_backprop);
+  const bool square = p.window_rows == p.window_cols &&
+                      p.stride_rows == p.stride_cols &&
+                      static_cast<size_t>(p.batch) *
+                              ceil_div(p.in_rows, kGradTile) *
+                              ceil_div(p.in_cols, kGradTile) < 0x7FFFFFFFu &&
+                      ceil_div(p.channels / 4, 16) <= 65535;
+  if (vec4 && square && p.window_rows == 3 && p.stride_rows == 2) {
+    launch_max_grad_tile<3, 2>(input_data, output_data, input_backprop,
+                               output_backprop, p, nan_mode, stream);
+  } else if (vec4 && square && p.window_rows == 3 && p.stride_rows == 1) {
+    launch_max_grad_tile<3, 1>(input_data, output_data, input_backprop,
+                               output_backprop, p, nan_mode, stream);
+  } else if (vec4 && square && p.window_rows == 2 && p.stride_rows == 2) {
+    launch_max_grad_tile<2, 2>(input_data, output_data, input_backprop,
+                               output_backprop, p, nan_mode, stream);
+  } else if (vec4) {
     const size_t n_vec = n_in / 4;
     hipLaunchKernelGGL(pool_max_grad_kernel<4>,
                        dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{kBlock}))),

@@ -397,6 +397,34 @@ def test_pooling_ragged(shape):
                  oracle.pool_avg_grad(dy, op), ("avg grad", shape))
 
 
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, window, stride, same
+    (2, 37, 41, 12, 3, 2, True),     # ragged 16 x 16 tiles, 3 channel vectors
+    (1, 33, 17, 72, 3, 2, False),    # two channel groups, VALID
+    (3, 19, 23, 8, 3, 1, True),      # stride 1: every element in 9 windows
+    (2, 30, 18, 20, 2, 2, False),    # disjoint windows
+    (1, 16, 16, 4, 3, 2, True),      # exactly one tile
+])
+@pytest.mark.parametrize("nan_mode", [False, True])
+def test_maxpool_grad_tiled_kernel(shape, nan_mode):
+    """The work-group-tiled max gradient (3x3 s2, 3x3 s1, 2x2 s2 with
+    channels % 4 == 0): small integers make most windows tie, some NaNs test
+    both NaN rules; results must equal the oracle exactly."""
+    n, h, w_, c, win, st, same = shape
+    p = ops.pool_params(n, h, w_, c, win, st, same)
+    op = oracle_params(p, 0)
+    rng = np.random.default_rng(1300 + h * w_ + c)
+    x = rng.integers(-2, 3, n * h * w_ * c).astype(np.float32)
+    x[rng.integers(0, x.size, x.size // 50)] = np.nan
+    gpu_op = POOL_OP.MAX_WITH_NAN if nan_mode else POOL_OP.MAX
+    y = ops.pooling_forward(dev(x), p, gpu_op)
+    ref_y = oracle.pool_max_forward(x, op, nan_mode)
+    assert np.array_equal(y.cpu().numpy(), ref_y, equal_nan=True)
+    dy = rng.integers(1, 9, ref_y.size).astype(np.float32)
+    got = ops.pooling_max_grad(dev(x), y, dev(dy), p, gpu_op).cpu().numpy()
+    assert np.array_equal(got, oracle.pool_max_grad(x, ref_y, dy, op, nan_mode))
+
+
 def test_maxpool_nan_rules():
     """test/pooling/max_pooling_with_nan.cc: Max drops NaNs, MaxWithNan
     propagates them (forward and gradient)."""
