@@ -8,6 +8,8 @@
 // average divides by the clipped element count.
 #include <cfloat>
 
+#include <cstdlib>
+
 #include "snn_kernels.h"
 
 namespace snn {
@@ -524,6 +526,10 @@ int launch_forward_op(const T* input, T* output,
         static_cast<size_t>(p.batch) * p.out_cols * (p.channels / 4);
     int th = 4;
     while (th > 1 && per_row * ceil_div(p.out_rows, th) < 150000) th /= 2;
+    // Developer override for tuning runs: SNN_HIP_POOL_TH=<1|2|4>.
+    static const char* tune = getenv("SNN_HIP_POOL_TH");
+    if (tune != nullptr && tune[0] != 0) th = atoi(tune);
+    th = th >= 4 ? 4 : th >= 2 ? 2 : 1;
     const int n_strips = ceil_div(p.out_rows, th);
     const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
     const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
