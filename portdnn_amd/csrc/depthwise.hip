@@ -485,6 +485,173 @@ __global__ void __launch_bounds__(kDwFilbkThreads)
   }
 }
 
+// The same reduction with the input window kept in registers: a pixel lane
+// walks TH consecutive output rows of one output column and loads every input
+// row of that strip once (three column taps), so an output pixel costs
+// STRIDE * 3 + 1 vector loads instead of 10.  Strips are numbered column
+// fastest, (image, row block, column), and dealt to the pixel lanes in that
+// order; rows past the end of the image read zeros through the buffer range
+// check and add nothing.
+template <int STRIDE, int TH>
+__global__ void __launch_bounds__(kDwFilbkThreads)
+    dw_filter_backprop_3x3_strip_kernel(const float* __restrict__ in,
+                                        const float* __restrict__ dy,
+                                        float* __restrict__ dw,
+                                        float* __restrict__ part,
+                                        snn_hip_depthwise_params p, int cvw,
+                                        int strips_per_group, int n_strips,
+                                        int n_row_blocks) {
+  constexpr int RING = 3;  // input rows alive at once
+  __shared__ float partial[kDwFilbkThreads][37];
+  const int C = p.channels;
+  const int tid = threadIdx.x;
+  const int cl = tid % cvw;
+  const int pl = tid / cvw;
+  const int n_pl = kDwFilbkThreads / cvw;
+  const int c = (blockIdx.y * cvw + cl) * 4;
+  const int strip_begin = blockIdx.x * strips_per_group;
+  const int strip_end = min(n_strips, strip_begin + strips_per_group);
+  const size_t in_elems =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * C;
+  const size_t dy_elems =
+      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * C;
+  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_elems * 4);
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, dy_elems * 4);
+  float acc[9][4];
+#pragma unroll
+  for (int t = 0; t < 9; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[t][i] = 0.f;
+  if (c < C) {
+    for (int strip = strip_begin + pl; strip < strip_end; strip += n_pl) {
+      const int ox = strip % p.out_cols;
+      const int t2 = strip / p.out_cols;
+      const int rb = t2 % n_row_blocks;
+      const int n = t2 / n_row_blocks;
+      const int oy0 = rb * TH;
+      const int y0 = oy0 * STRIDE - p.pad_rows;
+      const int x0 = ox * STRIDE - p.pad_cols;
+      // byte offsets of the three column taps in input row 0 of the image, or
+      // out of range for a padding column
+      unsigned col_off[3];
+#pragma unroll
+      for (int sc = 0; sc < 3; ++sc)
+        col_off[sc] = static_cast<unsigned>(x0 + sc) <
+                              static_cast<unsigned>(p.in_cols)
+                          ? static_cast<unsigned>((x0 + sc) * C + c) * 4u
+                          : kOobOffset;
+      const unsigned image_off =
+          static_cast<unsigned>(n * p.in_rows * p.in_cols * C) * 4u;
+      const unsigned row_bytes = static_cast<unsigned>(p.in_cols * C) * 4u;
+      float win[RING][3][4];
+      auto load_row = [&](int rel, float (&dst)[3][4]) {
+        const int y = y0 + rel;
+        const bool ok =
+            static_cast<unsigned>(y) < static_cast<unsigned>(p.in_rows);
+        const unsigned base =
+            image_off + static_cast<unsigned>(y) * row_bytes;
+#pragma unroll
+        for (int sc = 0; sc < 3; ++sc)
+          BufVec4<float>::load(
+              in_rsrc,
+              (ok && col_off[sc] != kOobOffset) ? base + col_off[sc]
+                                                : kOobOffset,
+              dst[sc]);
+      };
+#pragma unroll
+      for (int rel = 0; rel < 3 - STRIDE; ++rel) load_row(rel, win[rel % RING]);
+      const unsigned dy_off0 =
+          static_cast<unsigned>(((n * p.out_rows + oy0) * p.out_cols + ox) * C +
+                                c) * 4u;
+      const unsigned dy_row_bytes = static_cast<unsigned>(p.out_cols * C) * 4u;
+#pragma unroll
+      for (int i = 0; i < TH; ++i) {
+        // the input rows this output row adds that the previous one lacked
+#pragma unroll
+        for (int rel = 3 - STRIDE; rel < 3; ++rel)
+          load_row(i * STRIDE + rel, win[(i * STRIDE + rel) % RING]);
+        float g[4];
+        BufVec4<float>::load(
+            dy_rsrc,
+            oy0 + i < p.out_rows ? dy_off0 + static_cast<unsigned>(i) * dy_row_bytes
+                                 : kOobOffset,
+            g);
+        // (a row block may run past the last output row: nothing to add,
+        // whatever the input rows below it hold)
+        if (oy0 + i < p.out_rows) {
+#pragma unroll
+          for (int r = 0; r < 3; ++r)
+#pragma unroll
+            for (int sc = 0; sc < 3; ++sc)
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                acc[r * 3 + sc][e] = fmaf(win[(i * STRIDE + r) % RING][sc][e],
+                                          g[e], acc[r * 3 + sc][e]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < 9; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) partial[tid][t * 4 + i] = acc[t][i];
+  __syncthreads();
+  for (int e = tid; e < cvw * 36; e += kDwFilbkThreads) {
+    const int ecl = e % cvw, comp = e / cvw;  // comp = tap * 4 + i
+    float sum = 0.f;
+    for (int q = 0; q < n_pl; ++q) sum += partial[q * cvw + ecl][comp];
+    const int ch = (blockIdx.y * cvw + ecl) * 4 + (comp & 3);
+    if (ch >= C) continue;
+    if (part != nullptr) {
+      part[static_cast<size_t>(blockIdx.x) * 9 * C + (comp >> 2) * C + ch] =
+          sum;
+      // the kernel that adds the partial filters up expects dF zero-filled
+      if (blockIdx.x == 0) dw[(comp >> 2) * C + ch] = 0.f;
+    } else {
+      atomicAdd(dw + (comp >> 2) * C + ch, sum);
+    }
+  }
+}
+
+// dF += the work-groups' partial filters part[group][e], four elements per
+// lane; blockIdx.y and the four waves of a work-group split the groups, the
+// waves combine through LDS and one float atomic per element and work-group
+// goes to dF, which the strip kernel has zero-filled.
+constexpr int kDwFilbkReduceY = 16;
+
+__global__ void __launch_bounds__(256)
+    dw_filbk_reduce_kernel(const float4* __restrict__ part,
+                           float* __restrict__ dw, int n_vec, int n_groups) {
+  __shared__ float4 sums[4][64];
+  const int lane = threadIdx.x & 63, sub = threadIdx.x >> 6;
+  const int v = blockIdx.x * 64 + lane;
+  const int n_slices = gridDim.y * 4;
+  float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+  if (v < n_vec) {
+    int g = blockIdx.y * 4 + sub;
+    for (; g + n_slices < n_groups; g += 2 * n_slices) {
+      const float4 x = part[static_cast<size_t>(g) * n_vec + v];
+      const float4 y = part[static_cast<size_t>(g + n_slices) * n_vec + v];
+      a = make_float4(a.x + x.x, a.y + x.y, a.z + x.z, a.w + x.w);
+      b = make_float4(b.x + y.x, b.y + y.y, b.z + y.z, b.w + y.w);
+    }
+    if (g < n_groups) {
+      const float4 x = part[static_cast<size_t>(g) * n_vec + v];
+      a = make_float4(a.x + x.x, a.y + x.y, a.z + x.z, a.w + x.w);
+    }
+  }
+  sums[sub][lane] = make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
+  __syncthreads();
+  if (sub == 0 && v < n_vec) {
+    const float4 s0 = sums[0][lane], s1 = sums[1][lane], s2 = sums[2][lane],
+                 s3 = sums[3][lane];
+    atomicAdd(dw + 4 * v + 0, (s0.x + s1.x) + (s2.x + s3.x));
+    atomicAdd(dw + 4 * v + 1, (s0.y + s1.y) + (s2.y + s3.y));
+    atomicAdd(dw + 4 * v + 2, (s0.z + s1.z) + (s2.z + s3.z));
+    atomicAdd(dw + 4 * v + 3, (s0.w + s1.w) + (s2.w + s3.w));
+  }
+}
+
 __global__ void __launch_bounds__(256)
     dw_zero_kernel(float* __restrict__ p, int n) {
   const int i = blockIdx.x * 256 + threadIdx.x;
@@ -603,6 +770,74 @@ void launch_dw_strip(const T* input, const T* filter, T* output,
 
 }  // namespace
 
+// Picks the strip height (4 or 8 output rows, whichever wastes fewer rows of
+// the last row block; 8 on a tie) and deals the strips to the work-groups.
+// Large problems use about 2048 work-groups whose partial filters go to a
+// stream-ordered temporary that a second kernel adds up; small ones (or no
+// temporary) use up to 1024 work-groups that add into the zero-filled dF
+// with float atomics, which serialise per address.
+static void launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
+                                  const snn_hip_depthwise_params& p, int cvw,
+                                  int grid_y, hipStream_t stream) {
+  const int n_pl = kDwFilbkThreads / cvw;
+  const int th =
+      ceil_div(p.out_rows, 8) * 8 <= ceil_div(p.out_rows, 4) * 4 ? 8 : 4;
+  const int n_rb = ceil_div(p.out_rows, th);
+  const int n_strips = p.batch * n_rb * p.out_cols;
+  const int dw_elems = 9 * p.channels;
+  static const char* tune = getenv("SNN_HIP_DW_FILBK_GROUPS");
+  auto plan = [&](int target_groups, int* spg) {
+    *spg = max(n_pl, ceil_div(n_strips, max(1, target_groups / grid_y)));
+    *spg = ceil_div(*spg, n_pl) * n_pl;
+    return ceil_div(n_strips, *spg);
+  };
+  const size_t in_bytes = static_cast<size_t>(p.batch) * p.in_rows *
+                          p.in_cols * p.channels * sizeof(float);
+  constexpr size_t kTwoStageBytes = size_t{32} << 20;
+  int spg = 0, grid_x = 0;
+  float* part = nullptr;
+  if (in_bytes >= kTwoStageBytes) {
+    grid_x = plan(tune != nullptr ? max(1, atoi(tune)) : 2048, &spg);
+    if (hipMallocAsync(reinterpret_cast<void**>(&part),
+                       static_cast<size_t>(grid_x) * dw_elems * sizeof(float),
+                       stream) != hipSuccess) {
+      (void)hipGetLastError();
+      part = nullptr;
+    }
+  }
+  if (part == nullptr) {
+    grid_x = plan(1024, &spg);
+    hipLaunchKernelGGL(dw_zero_kernel, dim3(ceil_div(dw_elems, 256)),
+                       dim3(256), 0, stream, dw, dw_elems);
+  }
+  const dim3 grid(static_cast<unsigned>(grid_x),
+                  static_cast<unsigned>(grid_y));
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(kDwFilbkThreads), 0, stream, x, dy,
+                       dw, part, p, cvw, spg, n_strips, n_rb);
+  };
+  if (p.stride_rows == 1) {
+    if (th == 8)
+      launch(dw_filter_backprop_3x3_strip_kernel<1, 8>);
+    else
+      launch(dw_filter_backprop_3x3_strip_kernel<1, 4>);
+  } else {
+    if (th == 8)
+      launch(dw_filter_backprop_3x3_strip_kernel<2, 8>);
+    else
+      launch(dw_filter_backprop_3x3_strip_kernel<2, 4>);
+  }
+  if (part != nullptr) {
+    const int n_vec = dw_elems / 4;
+    hipLaunchKernelGGL(
+        dw_filbk_reduce_kernel,
+        dim3(static_cast<unsigned>(ceil_div(n_vec, 64)), kDwFilbkReduceY),
+        dim3(256), 0, stream, reinterpret_cast<const float4*>(part), dw, n_vec,
+        grid_x);
+    (void)hipFreeAsync(part, stream);
+  }
+}
+
 template <typename T>
 int launch_depthwise(int direction, const T* input, const T* filter, T* output,
                      const snn_hip_depthwise_params& p, hipStream_t stream) {
@@ -695,13 +930,21 @@ int launch_depthwise(int direction, const T* input, const T* filter, T* output,
         ppg = ceil_div(ppg, n_pl) * n_pl;
         const int grid_x = ceil_div(n_pix, ppg);
         const int dw_elems = 9 * p.channels;
-        hipLaunchKernelGGL(dw_zero_kernel, dim3(ceil_div(dw_elems, 256)),
-                           dim3(256), 0, stream, output, dw_elems);
-        hipLaunchKernelGGL(dw_filter_backprop_3x3_kernel,
-                           dim3(static_cast<unsigned>(grid_x),
-                                static_cast<unsigned>(grid_y)),
-                           dim3(kDwFilbkThreads), 0, stream, input, filter,
-                           output, p, cvw, ppg);
+        const bool strip_ok =
+            p.stride_rows == p.stride_cols &&
+            (p.stride_rows == 1 || p.stride_rows == 2) &&
+            getenv("SNN_HIP_DW_FILBK_PIXEL") == nullptr;
+        if (strip_ok) {
+          launch_dw_filbk_strip(input, filter, output, p, cvw, grid_y, stream);
+        } else {
+          hipLaunchKernelGGL(dw_zero_kernel, dim3(ceil_div(dw_elems, 256)),
+                             dim3(256), 0, stream, output, dw_elems);
+          hipLaunchKernelGGL(dw_filter_backprop_3x3_kernel,
+                             dim3(static_cast<unsigned>(grid_x),
+                                  static_cast<unsigned>(grid_y)),
+                             dim3(kDwFilbkThreads), 0, stream, input, filter,
+                             output, p, cvw, ppg);
+        }
         done = true;
       }
     }

@@ -318,6 +318,36 @@ def test_depthwise_ragged(shape):
                  ("dw filbk", shape))
 
 
+@pytest.mark.parametrize("shape", [(2, 13, 11, 8, 1, True),
+                                   (3, 14, 14, 64, 2, True),
+                                   (1, 12, 10, 4, 2, False),
+                                   (2, 33, 20, 12, 1, False),
+                                   (5, 5, 37, 16, 2, True),
+                                   (1, 3, 3, 256, 1, True),
+                                   (2, 29, 6, 132, 1, True)])
+def test_depthwise_filter_backprop_row_strips(shape):
+    """3x3 filter gradient with four channels per lane: row blocks that run
+    past the last output row, odd sizes, both strides and paddings."""
+    n, h, w_, c, st, same = shape
+    p = ops.depthwise_params(n, h, w_, c, 1, 3, st, same)
+    op = oracle_params(p, 1)
+    rng = np.random.default_rng(900 + h * w_ + c)
+    x = rng.standard_normal(n * h * w_ * c).astype(np.float32)
+    dy = rng.standard_normal(n * p.out_rows * p.out_cols * c).astype(
+        np.float32)
+    # rows and columns no window touches must not leak in, whatever they hold
+    if not same and st == 2:
+        xv = x.reshape(n, h, w_, c)
+        last_r = (p.out_rows - 1) * st + 3
+        last_c = (p.out_cols - 1) * st + 3
+        xv[:, last_r:, :, :] = np.inf
+        xv[:, :, last_c:, :] = np.inf
+    got = ops.depthwise_conv2d(dev(x), dev(dy), p,
+                               DIRECTION.FILTER_BACKPROP).cpu().numpy()
+    assert_close(got, oracle.depthwise_filter_backprop(x, dy, op),
+                 ("dw filbk strips", shape))
+
+
 @pytest.mark.parametrize("size,ch,stride", MOBILENET)
 def test_depthwise_full_batch_matches_oracle(size, ch, stride):
     """Batch 32: the depthwise oracle is cheap enough to run in full."""
