@@ -503,6 +503,73 @@ __global__ void __launch_bounds__(256)
   GradVec<VEC>::store(dx + idx * VEC, grad);
 }
 
+// The same gradient with TH consecutive input rows of one column per lane
+// (four channels): the index arithmetic and the column range are computed once
+// per strip, and every contributing dY / count is formed once and added to
+// each of the strip's rows its window covers, in the same output-row,
+// output-column order as above.
+template <int TH>
+__global__ void __launch_bounds__(256)
+    pool_avg_grad_strip_kernel(const float* __restrict__ dy,
+                               float* __restrict__ dx, snn_hip_pooling_params p,
+                               int n_strips, unsigned n_items) {
+  const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+  if (idx >= n_items) return;
+  const int C = p.channels;
+  const unsigned cv = static_cast<unsigned>(C) / 4u;
+  const int ch = static_cast<int>(idx % cv) * 4;
+  unsigned t = idx / cv;
+  const int x = static_cast<int>(t % static_cast<unsigned>(p.in_cols));
+  t /= static_cast<unsigned>(p.in_cols);
+  const int y0 = static_cast<int>(t % static_cast<unsigned>(n_strips)) * TH;
+  const int n = static_cast<int>(t / static_cast<unsigned>(n_strips));
+  const int y_last = min(y0 + TH, p.in_rows) - 1;
+  const int px = x + p.pad_cols;
+  const int ox_begin =
+      px < p.window_cols ? 0 : (px - p.window_cols) / p.stride_cols + 1;
+  const int ox_end = min(px / p.stride_cols + 1, p.out_cols);
+  const int py0 = y0 + p.pad_rows;
+  const int oy_begin =
+      py0 < p.window_rows ? 0 : (py0 - p.window_rows) / p.stride_rows + 1;
+  const int oy_end = min((y_last + p.pad_rows) / p.stride_rows + 1, p.out_rows);
+  const float* dy_n =
+      dy + static_cast<size_t>(n) * p.out_rows * p.out_cols * C + ch;
+  float grad[TH][4];
+#pragma unroll
+  for (int i = 0; i < TH; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) grad[i][e] = 0.f;
+  for (int oy = oy_begin; oy < oy_end; ++oy) {
+    int r0 = oy * p.stride_rows - p.pad_rows;
+    const int r1 = min(r0 + p.window_rows, p.in_rows);
+    r0 = max(r0, 0);
+    for (int ox = ox_begin; ox < ox_end; ++ox) {
+      int c0 = ox * p.stride_cols - p.pad_cols;
+      const int c1 = min(c0 + p.window_cols, p.in_cols);
+      c0 = max(c0, 0);
+      const float count = static_cast<float>((r1 - r0) * (c1 - c0));
+      float g[4];
+      GradVec<4>::load(dy_n + (static_cast<size_t>(oy) * p.out_cols + ox) * C,
+                       g);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) g[e] = g[e] / count;
+#pragma unroll
+      for (int i = 0; i < TH; ++i) {
+        if (y0 + i >= r0 && y0 + i < r1) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) grad[i][e] += g[e];
+        }
+      }
+    }
+  }
+  float* dx_p =
+      dx + ((static_cast<size_t>(n) * p.in_rows + y0) * p.in_cols + x) * C + ch;
+  const size_t row_elems = static_cast<size_t>(p.in_cols) * C;
+#pragma unroll
+  for (int i = 0; i < TH; ++i)
+    if (y0 + i <= y_last) GradVec<4>::store(dx_p + i * row_elems, grad[i]);
+}
+
 template <typename T, typename Op>
 int launch_forward_op(const T* input, T* output,
                       const snn_hip_pooling_params& p, hipStream_t stream) {
@@ -795,10 +862,31 @@ int launch_pooling_avg_grad(const float* input_backprop,
   if (p.channels % 4 == 0 && grad_aligned16(input_backprop) &&
       grad_aligned16(output_backprop)) {
     const size_t n_vec = n_in / 4;
-    hipLaunchKernelGGL(pool_avg_grad_kernel<4>,
-                       dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{kBlock}))),
-                       dim3(kBlock), 0, stream, input_backprop,
-                       output_backprop, p, n_vec);
+    // row strips when they still give every CU a few thousand lanes
+    const size_t per_row =
+        static_cast<size_t>(p.batch) * p.in_cols * (p.channels / 4);
+    int th = 8;
+    while (th > 1 && per_row * ceil_div(p.in_rows, th) < 150000) th /= 2;
+    static const char* tune = getenv("SNN_HIP_POOL_GRAD_TH");
+    if (tune != nullptr && tune[0] != 0) th = atoi(tune);
+    const int n_strips = ceil_div(p.in_rows, th >= 8 ? 8 : 4);
+    const size_t n_items = per_row * n_strips;
+    if (th >= 4 && n_items < 0x7FFFFFFFu) {
+      const dim3 grid(static_cast<unsigned>(ceil_div(n_items, size_t{kBlock})));
+      if (th >= 8)
+        hipLaunchKernelGGL(pool_avg_grad_strip_kernel<8>, grid, dim3(kBlock), 0,
+                           stream, input_backprop, output_backprop, p, n_strips,
+                           static_cast<unsigned>(n_items));
+      else
+        hipLaunchKernelGGL(pool_avg_grad_strip_kernel<4>, grid, dim3(kBlock), 0,
+                           stream, input_backprop, output_backprop, p, n_strips,
+                           static_cast<unsigned>(n_items));
+    } else {
+      hipLaunchKernelGGL(
+          pool_avg_grad_kernel<4>,
+          dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{kBlock}))),
+          dim3(kBlock), 0, stream, input_backprop, output_backprop, p, n_vec);
+    }
   } else {
     hipLaunchKernelGGL(pool_avg_grad_kernel<1>,
                        dim3(static_cast<unsigned>(ceil_div(n_in, size_t{kBlock}))),

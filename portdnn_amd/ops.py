@@ -186,17 +186,19 @@ def pooling_forward(inp, p, op, out=None):
     return out
 
 
-def pooling_max_grad(inp, out, dy, p, op=POOL_OP.MAX):
-    dx = torch.empty_like(inp)
+def pooling_max_grad(inp, out, dy, p, op=POOL_OP.MAX, dx=None):
+    if dx is None:
+        dx = torch.empty_like(inp)
     capi.check(capi.lib().snn_hip_pooling_max_grad_f32(
         _ptr(inp), _ptr(out), _ptr(dy), _ptr(dx), ctypes.byref(p), op,
         _stream()))
     return dx
 
 
-def pooling_avg_grad(dy, p):
-    dx = torch.empty(p.batch * p.in_rows * p.in_cols * p.channels,
-                     dtype=dy.dtype, device=dy.device)
+def pooling_avg_grad(dy, p, dx=None):
+    if dx is None:
+        dx = torch.empty(p.batch * p.in_rows * p.in_cols * p.channels,
+                         dtype=dy.dtype, device=dy.device)
     capi.check(capi.lib().snn_hip_pooling_avg_grad_f32(
         _ptr(dy), _ptr(dx), ctypes.byref(p), _stream()))
     return dx

@@ -405,6 +405,24 @@ def test_avgpool_resnet_full_batch():
                  oracle.pool_avg_grad(dy, oracle_params(p, 0)), "avg grad")
 
 
+@pytest.mark.parametrize("shape", [(32, 75, 70, 64, 3, 2, True),
+                                   (16, 61, 59, 64, 3, 2, False),
+                                   (24, 40, 40, 128, 5, 1, True),
+                                   (20, 30, 33, 256, 2, 2, False),
+                                   (32, 112, 112, 64, 3, 2, True)])
+def test_avgpool_grad_row_strips(shape):
+    """Average-pool gradient on tensors large enough for the kernel that
+    gives a lane a strip of input rows (8 or 4 rows, ragged last strip)."""
+    n, h, w_, c, win, st, same = shape
+    p = ops.pool_params(n, h, w_, c, win, st, same)
+    rng = np.random.default_rng(700 + h + c)
+    dy = rng.standard_normal(n * p.out_rows * p.out_cols * c).astype(
+        np.float32)
+    got = ops.pooling_avg_grad(dev(dy), p).cpu().numpy()
+    assert_close(got, oracle.pool_avg_grad(dy, oracle_params(p, 0)),
+                 ("avg grad strips", shape))
+
+
 @pytest.mark.parametrize("shape", [(2, 9, 7, 5, 3, 2, True),
                                    (1, 11, 11, 3, 5, 1, True),
                                    (3, 8, 8, 8, 2, 2, False),
