@@ -150,7 +150,8 @@ SNN_HIP_API const char* snn_hip_last_error(void);
  * launches return a cl::sycl::event that carries profiling information).
  * While enabled, every convolution launch brackets its dominant kernel -- the
  * implicit-GEMM or fused Winograd kernel, not the filter preparation or zero
- * fill around it -- with HIP events recorded on the launch stream.
+ * fill around it -- with HIP events recorded on the launch stream; depthwise
+ * and pooling launches bracket everything they enqueue.
  * snn_hip_kernel_timing_read waits for the recorded events, returns the summed
  * kernel time in milliseconds and the number of kernels, and clears the
  * record.  Not thread safe; meant for a single benchmarking thread. */

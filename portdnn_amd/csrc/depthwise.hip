@@ -841,6 +841,7 @@ static void launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
 template <typename T>
 int launch_depthwise(int direction, const T* input, const T* filter, T* output,
                      const snn_hip_depthwise_params& p, hipStream_t stream) {
+  KernelTimer timer(stream);
   constexpr int kBlock = 256;
   const size_t CM = static_cast<size_t>(p.channels) * p.channel_multiplier;
   if (direction == SNN_HIP_FORWARD) {

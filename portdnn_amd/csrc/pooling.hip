@@ -785,6 +785,7 @@ template <typename T>
 int launch_pooling_forward(const T* input, T* output,
                            const snn_hip_pooling_params& p, int op,
                            hipStream_t stream) {
+  KernelTimer timer(stream);
   switch (op) {
     case SNN_HIP_POOL_MAX:
       return launch_forward_op<T, MaxOp>(input, output, p, stream);
@@ -813,6 +814,7 @@ int launch_pooling_max_grad(const float* input_data, const float* output_data,
                             float* output_backprop,
                             const snn_hip_pooling_params& p, int op,
                             hipStream_t stream) {
+  KernelTimer timer(stream);
   constexpr int kBlock = 256;
   const size_t n_in =
       static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
@@ -856,6 +858,7 @@ int launch_pooling_avg_grad(const float* input_backprop,
                             float* output_backprop,
                             const snn_hip_pooling_params& p,
                             hipStream_t stream) {
+  KernelTimer timer(stream);
   constexpr int kBlock = 256;
   const size_t n_in =
       static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;

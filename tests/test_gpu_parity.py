@@ -549,6 +549,9 @@ def test_f16_conv_forward(size, ch, window):
     (1, 9, 9, 64, 200, 5, 1, False),     # VALID, 25 taps
     (5, 7, 7, 192, 8, 1, 1, False),      # 1x1, three chunks per tap
     (2, 33, 31, 64, 130, 3, 2, False),   # features just past two tiles
+    (2, 17, 9, 128, 80, 3, 2, True),     # 16-byte stores, half a block masked
+    (5, 7, 7, 192, 48, 1, 1, False),     # 1x1, 16-byte stores, ragged rows
+    (3, 10, 10, 64, 272, 3, 2, True),    # 16-byte stores past two tiles
 ])
 def test_f16_conv_forward_ragged(shape):
     batch, rows, cols, ch, feats, window, stride, same = shape
