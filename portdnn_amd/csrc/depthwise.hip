@@ -405,6 +405,117 @@ __global__ void __launch_bounds__(256)
   BufVec4<T>::store(dx_rsrc, idx * 4u * static_cast<unsigned>(sizeof(T)), acc);
 }
 
+// Input backprop, 3x3 stride 2, multiplier == 1, four channels per lane.
+// In padded coordinates t = y + pad a dX pixel with even t takes filter rows
+// 0 and 2 (from dY rows t / 2 and t / 2 - 1) and one with odd t takes row 1
+// (from dY row t / 2); columns alike.  A lane owns the 2 x 2 dX pixels of
+// TH consecutive block rows of one block column: four dY vectors feed the
+// four pixels of a block, two of them carried over from the block row above,
+// and the nine filter taps stay in registers.  Every dX pixel still adds its
+// taps in filter-row, filter-column order.
+template <typename T, int TH>
+__global__ void __launch_bounds__(256)
+    dw_input_backprop_3x3_s2_kernel(const T* __restrict__ dy,
+                                    const T* __restrict__ fil,
+                                    T* __restrict__ dx,
+                                    snn_hip_depthwise_params p, int n_bcols,
+                                    int n_strips, unsigned n_items) {
+  const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+  if (idx >= n_items) return;
+  const int C = p.channels;
+  const unsigned cv = static_cast<unsigned>(C) / 4u;
+  const int c = static_cast<int>(idx % cv) * 4;
+  unsigned t = idx / cv;
+  const int bc = static_cast<int>(t % static_cast<unsigned>(n_bcols)) +
+                 p.pad_cols / 2;
+  t /= static_cast<unsigned>(n_bcols);
+  const int br0 = static_cast<int>(t % static_cast<unsigned>(n_strips)) * TH +
+                  p.pad_rows / 2;
+  const int n = static_cast<int>(t / static_cast<unsigned>(n_strips));
+  const size_t dy_elems =
+      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * C;
+  const size_t dx_elems =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * C;
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, dy_elems * sizeof(T));
+  const __amdgpu_buffer_rsrc_t fil_rsrc =
+      make_rsrc(fil, static_cast<size_t>(9) * C * sizeof(T));
+  const __amdgpu_buffer_rsrc_t dx_rsrc = make_rsrc(dx, dx_elems * sizeof(T));
+  float f[9][4];
+#pragma unroll
+  for (int k = 0; k < 9; ++k)
+    BufVec4<T>::load(fil_rsrc,
+                     static_cast<unsigned>(k * C + c) * sizeof(T), f[k]);
+  // dY columns bc - 1 and bc of one dY row; out of range reads zeros
+  const bool col_ok[2] = {bc >= 1 && bc - 1 < p.out_cols, bc < p.out_cols};
+  auto load_row = [&](int oy, float (&g)[2][4]) {
+    const bool row_ok =
+        static_cast<unsigned>(oy) < static_cast<unsigned>(p.out_rows);
+    const unsigned base =
+        static_cast<unsigned>(((n * p.out_rows + oy) * p.out_cols + bc - 1) *
+                                  C + c) * sizeof(T);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      BufVec4<T>::load(dy_rsrc,
+                       (row_ok && col_ok[j])
+                           ? base + static_cast<unsigned>(j * C) * sizeof(T)
+                           : kOobOffset,
+                       g[j]);
+  };
+  // dX pixel (2 * br - pad + i, 2 * bc - pad + j) of the current block
+  const int x0 = 2 * bc - p.pad_cols;
+  const bool x_ok[2] = {
+      static_cast<unsigned>(x0) < static_cast<unsigned>(p.in_cols),
+      static_cast<unsigned>(x0 + 1) < static_cast<unsigned>(p.in_cols)};
+  float above[2][4], here[2][4];
+  load_row(br0 - 1, above);
+#pragma unroll
+  for (int i = 0; i < TH; ++i) {
+    const int br = br0 + i;
+    load_row(br, here);
+    float even_even[4], even_odd[4], odd_even[4], odd_odd[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      // taps in (r, s) order: (0,0) (0,2) (2,0) (2,2)
+      float v = here[1][e] * f[0][e];
+      v = fmaf(here[0][e], f[2][e], v);
+      v = fmaf(above[1][e], f[6][e], v);
+      even_even[e] = fmaf(above[0][e], f[8][e], v);
+      // (0,1) (2,1)
+      even_odd[e] = fmaf(above[1][e], f[7][e], here[1][e] * f[1][e]);
+      // (1,0) (1,2)
+      odd_even[e] = fmaf(here[0][e], f[5][e], here[1][e] * f[3][e]);
+      // (1,1)
+      odd_odd[e] = here[1][e] * f[4][e];
+    }
+    const int y0 = 2 * br - p.pad_rows;
+    const bool y_ok[2] = {
+        static_cast<unsigned>(y0) < static_cast<unsigned>(p.in_rows),
+        static_cast<unsigned>(y0 + 1) < static_cast<unsigned>(p.in_rows)};
+    const unsigned base =
+        static_cast<unsigned>(((n * p.in_rows + y0) * p.in_cols + x0) * C + c) *
+        sizeof(T);
+    const unsigned row_bytes =
+        static_cast<unsigned>(p.in_cols * C) * sizeof(T);
+    const unsigned col_bytes = static_cast<unsigned>(C) * sizeof(T);
+    BufVec4<T>::store(dx_rsrc, (y_ok[0] && x_ok[0]) ? base : kOobOffset,
+                      even_even);
+    BufVec4<T>::store(dx_rsrc,
+                      (y_ok[0] && x_ok[1]) ? base + col_bytes : kOobOffset,
+                      even_odd);
+    BufVec4<T>::store(dx_rsrc,
+                      (y_ok[1] && x_ok[0]) ? base + row_bytes : kOobOffset,
+                      odd_even);
+    BufVec4<T>::store(
+        dx_rsrc,
+        (y_ok[1] && x_ok[1]) ? base + row_bytes + col_bytes : kOobOffset,
+        odd_odd);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) above[j][e] = here[j][e];
+  }
+}
+
 // Filter backprop, 3x3, multiplier == 1, C % 4 == 0.  A work-group covers
 // `cvw` channel vectors x (256 / cvw) pixels at a time and walks a range of
 // output pixels; each lane keeps the 9 x 4 partial sums of its channels, the
@@ -898,6 +1009,26 @@ int launch_depthwise(int direction, const T* input, const T* filter, T* output,
         }
       }
       if (!wide) launch_dw_strip<T, 4, true>(input, filter, output, q, stream);
+    } else if (vec_ok && p.window_rows == 3 && p.window_cols == 3 &&
+               p.stride_rows == 2 && p.stride_cols == 2 && p.pad_rows <= 2 &&
+               p.pad_cols <= 2 && getenv("SNN_HIP_DW_INBK_GATHER") == nullptr) {
+      // block rows / columns: padded coordinates pad .. in + pad - 1, halved
+      const int n_brows = (p.in_rows + p.pad_rows - 1) / 2 - p.pad_rows / 2 + 1;
+      const int n_bcols = (p.in_cols + p.pad_cols - 1) / 2 - p.pad_cols / 2 + 1;
+      const size_t per_row =
+          static_cast<size_t>(p.batch) * n_bcols * (p.channels / 4);
+      const int th = per_row * ceil_div(n_brows, 4) >= 150000 ? 4 : 2;
+      const int n_strips = ceil_div(n_brows, th);
+      const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
+      const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
+      if (th == 4)
+        hipLaunchKernelGGL((dw_input_backprop_3x3_s2_kernel<T, 4>), grid,
+                           dim3(kBlock), 0, stream, input, filter, output, p,
+                           n_bcols, n_strips, n_items);
+      else
+        hipLaunchKernelGGL((dw_input_backprop_3x3_s2_kernel<T, 2>), grid,
+                           dim3(kBlock), 0, stream, input, filter, output, p,
+                           n_bcols, n_strips, n_items);
     } else if (vec_ok) {
       const unsigned n_vec = static_cast<unsigned>(n_out / 4);
       hipLaunchKernelGGL(dw_input_backprop_vec4_kernel<T>,

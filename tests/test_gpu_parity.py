@@ -348,6 +348,28 @@ def test_depthwise_filter_backprop_row_strips(shape):
                  ("dw filbk strips", shape))
 
 
+@pytest.mark.parametrize("shape", [(2, 9, 7, 8, True),      # pad 1
+                                   (3, 14, 14, 64, True),    # pad 0
+                                   (1, 12, 10, 4, False),    # unused last row
+                                   (2, 33, 21, 12, False),
+                                   (5, 5, 37, 16, True),
+                                   (1, 3, 3, 256, True),
+                                   (40, 30, 31, 128, True)])  # 4-row strips
+def test_depthwise_input_backprop_stride2_blocks(shape):
+    """3x3 stride-2 input gradient, one 2 x 2 block of dX pixels at a time."""
+    n, h, w_, c, same = shape
+    p = ops.depthwise_params(n, h, w_, c, 1, 3, 2, same)
+    op = oracle_params(p, 1)
+    rng = np.random.default_rng(950 + h * w_ + c)
+    w = rng.standard_normal(9 * c).astype(np.float32)
+    dy = rng.standard_normal(n * p.out_rows * p.out_cols * c).astype(
+        np.float32)
+    got = ops.depthwise_conv2d(dev(dy), dev(w), p,
+                               DIRECTION.INPUT_BACKPROP).cpu().numpy()
+    assert_close(got, oracle.depthwise_input_backprop(dy, w, op),
+                 ("dw inbk s2", shape))
+
+
 @pytest.mark.parametrize("size,ch,stride", MOBILENET)
 def test_depthwise_full_batch_matches_oracle(size, ch, stride):
     """Batch 32: the depthwise oracle is cheap enough to run in full."""
