@@ -763,6 +763,199 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// Max gradient, 3x3 windows, stride 2, four channels per lane, without LDS.
+// In padded coordinates t = y + pad window o covers t = 2 * o .. 2 * o + 2,
+// so the 2 x 2 dX pixels of block (br, bc) (t rows 2 * br, 2 * br + 1, columns
+// alike) are covered by windows (br - 1 .. br) x (bc - 1 .. bc) only.  A lane
+// walks TH consecutive block rows of one block column: per block row it loads
+// two input rows of five columns (the third row of the two new windows is the
+// first row of the next block row and is carried in registers), finds for the
+// windows (br, bc - 1) and (br, bc) the first element equal to the forward
+// output in row-major order -- the reference's tie rule
+// (src/pooling/kernels.h:197-239) -- and carries those two positions and dY
+// values down as the "windows above" of the next block row.  Each dX pixel
+// adds its windows in output-row, output-column order.
+template <int TH>
+__global__ void __launch_bounds__(256)
+    pool_max_grad_3x3_s2_kernel(const float* __restrict__ in,
+                                const float* __restrict__ out,
+                                const float* __restrict__ dy,
+                                float* __restrict__ dx, snn_hip_pooling_params p,
+                                bool nan_mode, int n_bcols, int n_strips,
+                                unsigned n_items) {
+  const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+  if (idx >= n_items) return;
+  const int C = p.channels;
+  const unsigned cv = static_cast<unsigned>(C) / 4u;
+  const int ch = static_cast<int>(idx % cv) * 4;
+  unsigned t = idx / cv;
+  const int bc = static_cast<int>(t % static_cast<unsigned>(n_bcols)) +
+                 p.pad_cols / 2;
+  t /= static_cast<unsigned>(n_bcols);
+  const int br0 = static_cast<int>(t % static_cast<unsigned>(n_strips)) * TH +
+                  p.pad_rows / 2;
+  const int n = static_cast<int>(t / static_cast<unsigned>(n_strips));
+  const size_t in_elems =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * C;
+  const size_t out_elems =
+      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * C;
+  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_elems * 4);
+  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_elems * 4);
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, out_elems * 4);
+  const __amdgpu_buffer_rsrc_t dx_rsrc = make_rsrc(dx, in_elems * 4);
+
+  // input columns 2 * bc - 2 .. 2 * bc + 2 (padded), image column x0 + j
+  const int x0 = 2 * bc - 2 - p.pad_cols;
+  bool x_ok[5];
+#pragma unroll
+  for (int j = 0; j < 5; ++j)
+    x_ok[j] = static_cast<unsigned>(x0 + j) < static_cast<unsigned>(p.in_cols);
+  // windows bc - 1 and bc
+  const bool w_ok[2] = {bc >= 1 && bc - 1 < p.out_cols, bc < p.out_cols};
+  const unsigned in_row_bytes = static_cast<unsigned>(p.in_cols * C) * 4u;
+  const unsigned in_image = static_cast<unsigned>(n * p.in_rows) * in_row_bytes;
+  const unsigned in_col0 = static_cast<unsigned>(x0 * C + ch) * 4u;
+  auto load_in_row = [&](int y, float (&v)[5][4]) {
+    const bool ok = static_cast<unsigned>(y) < static_cast<unsigned>(p.in_rows);
+    const unsigned base =
+        in_image + static_cast<unsigned>(y) * in_row_bytes + in_col0;
+#pragma unroll
+    for (int j = 0; j < 5; ++j)
+      BufVec4<float>::load(
+          in_rsrc,
+          (ok && x_ok[j]) ? base + static_cast<unsigned>(j * C) * 4u
+                          : kOobOffset,
+          v[j]);
+  };
+  auto load_out_pair = [&](__amdgpu_buffer_rsrc_t rsrc, int oy,
+                           float (&v)[2][4]) {
+    const bool ok =
+        static_cast<unsigned>(oy) < static_cast<unsigned>(p.out_rows);
+    const unsigned base = static_cast<unsigned>(
+        ((n * p.out_rows + oy) * p.out_cols + bc - 1) * C + ch) * 4u;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      BufVec4<float>::load(
+          rsrc,
+          (ok && w_ok[j]) ? base + static_cast<unsigned>(j * C) * 4u
+                          : kOobOffset,
+          v[j]);
+  };
+
+  // windows of the block row above: first-maximum position (9: none) and dY
+  int up_pos[2][4];
+  float up_g[2][4];
+  float rows[3][5][4];  // rows[0] is carried from the block row above
+  {
+    // block row br0 - 1, needed only for its windows: scan it in full
+    const int y = 2 * (br0 - 1) - p.pad_rows;
+    float target[2][4];
+    load_out_pair(out_rsrc, br0 - 1, target);
+    load_out_pair(dy_rsrc, br0 - 1, up_g);
+    load_in_row(y, rows[0]);
+    load_in_row(y + 1, rows[1]);
+    load_in_row(y + 2, rows[2]);
+    const bool win_row_ok = static_cast<unsigned>(br0 - 1) <
+                            static_cast<unsigned>(p.out_rows);
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        int pos = 9;
+#pragma unroll
+        for (int k = 8; k >= 0; --k) {
+          const int r = k / 3, c = k % 3;
+          const bool y_ok = static_cast<unsigned>(y + r) <
+                            static_cast<unsigned>(p.in_rows);
+          if (y_ok && x_ok[2 * w + c] &&
+              pool_equal(rows[r][2 * w + c][e], target[w][e], nan_mode))
+            pos = k;
+        }
+        up_pos[w][e] = (win_row_ok && w_ok[w]) ? pos : 9;
+      }
+#pragma unroll
+    for (int j = 0; j < 5; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) rows[0][j][e] = rows[2][j][e];
+  }
+
+#pragma unroll
+  for (int i = 0; i < TH; ++i) {
+    const int br = br0 + i;
+    const int y = 2 * br - p.pad_rows;  // image row of padded row 2 * br
+    float target[2][4], g[2][4];
+    load_out_pair(out_rsrc, br, target);
+    load_out_pair(dy_rsrc, br, g);
+    load_in_row(y + 1, rows[1]);
+    load_in_row(y + 2, rows[2]);
+    bool y_ok[3];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+      y_ok[r] = static_cast<unsigned>(y + r) < static_cast<unsigned>(p.in_rows);
+    const bool win_row_ok =
+        static_cast<unsigned>(br) < static_cast<unsigned>(p.out_rows);
+    int pos[2][4];
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        int first = 9;
+#pragma unroll
+        for (int k = 8; k >= 0; --k) {
+          const int r = k / 3, c = k % 3;
+          if (y_ok[r] && x_ok[2 * w + c] &&
+              pool_equal(rows[r][2 * w + c][e], target[w][e], nan_mode))
+            first = k;
+        }
+        pos[w][e] = (win_row_ok && w_ok[w]) ? first : 9;
+      }
+    // the four dX pixels; windows in (output row, output column) order
+    float ee[4], eo[4], oe[4], oo[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float v = 0.f;
+      if (up_pos[0][e] == 8) v += up_g[0][e];
+      if (up_pos[1][e] == 6) v += up_g[1][e];
+      if (pos[0][e] == 2) v += g[0][e];
+      if (pos[1][e] == 0) v += g[1][e];
+      ee[e] = v;
+      v = 0.f;
+      if (up_pos[1][e] == 7) v += up_g[1][e];
+      if (pos[1][e] == 1) v += g[1][e];
+      eo[e] = v;
+      v = 0.f;
+      if (pos[0][e] == 5) v += g[0][e];
+      if (pos[1][e] == 3) v += g[1][e];
+      oe[e] = v;
+      oo[e] = pos[1][e] == 4 ? 0.f + g[1][e] : 0.f;
+    }
+    const unsigned base = in_image + static_cast<unsigned>(y) * in_row_bytes +
+                          in_col0 + static_cast<unsigned>(2 * C) * 4u;
+    const unsigned col_bytes = static_cast<unsigned>(C) * 4u;
+    BufVec4<float>::store(dx_rsrc, (y_ok[0] && x_ok[2]) ? base : kOobOffset,
+                          ee);
+    BufVec4<float>::store(
+        dx_rsrc, (y_ok[0] && x_ok[3]) ? base + col_bytes : kOobOffset, eo);
+    BufVec4<float>::store(
+        dx_rsrc, (y_ok[1] && x_ok[2]) ? base + in_row_bytes : kOobOffset, oe);
+    BufVec4<float>::store(
+        dx_rsrc,
+        (y_ok[1] && x_ok[3]) ? base + in_row_bytes + col_bytes : kOobOffset,
+        oo);
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        up_pos[w][e] = pos[w][e];
+        up_g[w][e] = g[w][e];
+      }
+#pragma unroll
+    for (int j = 0; j < 5; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) rows[0][j][e] = rows[2][j][e];
+  }
+}
+
 template <int WIN, int STRIDE>
 void launch_max_grad_tile(const float* in, const float* out, const float* dy,
                           float* dx, const snn_hip_pooling_params& p,
@@ -829,7 +1022,31 @@ int launch_pooling_max_grad(const float* input_data, const float* output_data,
                               ceil_div(p.in_rows, kGradTile) *
                               ceil_div(p.in_cols, kGradTile) < 0x7FFFFFFFu &&
                       ceil_div(p.channels / 4, 16) <= 65535;
-  if (vec4 && square && p.window_rows == 3 && p.stride_rows == 2) {
+  const size_t n_out =
+      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * p.channels;
+  static const bool use_tiles = getenv("SNN_HIP_POOL_GRAD_TILES") != nullptr;
+  if (vec4 && square && p.window_rows == 3 && p.stride_rows == 2 &&
+      !use_tiles && n_in * 4 < 0x7FFFFFF0u && n_out * 4 < 0x7FFFFFF0u) {
+    // block rows / columns: padded coordinates pad .. in + pad - 1, halved
+    const int n_brows = (p.in_rows + p.pad_rows - 1) / 2 - p.pad_rows / 2 + 1;
+    const int n_bcols = (p.in_cols + p.pad_cols - 1) / 2 - p.pad_cols / 2 + 1;
+    const size_t per_row =
+        static_cast<size_t>(p.batch) * n_bcols * (p.channels / 4);
+    const int th = per_row * ceil_div(n_brows, 4) >= 150000 ? 4 : 2;
+    const int n_strips = ceil_div(n_brows, th);
+    const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
+    const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
+    if (th == 4)
+      hipLaunchKernelGGL(pool_max_grad_3x3_s2_kernel<4>, grid, dim3(kBlock), 0,
+                         stream, input_data, output_data, input_backprop,
+                         output_backprop, p, nan_mode, n_bcols, n_strips,
+                         n_items);
+    else
+      hipLaunchKernelGGL(pool_max_grad_3x3_s2_kernel<2>, grid, dim3(kBlock), 0,
+                         stream, input_data, output_data, input_backprop,
+                         output_backprop, p, nan_mode, n_bcols, n_strips,
+                         n_items);
+  } else if (vec4 && square && p.window_rows == 3 && p.stride_rows == 2) {
     launch_max_grad_tile<3, 2>(input_data, output_data, input_backprop,
                                output_backprop, p, nan_mode, stream);
   } else if (vec4 && square && p.window_rows == 3 && p.stride_rows == 1) {

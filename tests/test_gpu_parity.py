@@ -474,12 +474,15 @@ def test_pooling_ragged(shape):
     (3, 19, 23, 8, 3, 1, True),      # stride 1: every element in 9 windows
     (2, 30, 18, 20, 2, 2, False),    # disjoint windows
     (1, 16, 16, 4, 3, 2, True),      # exactly one tile
+    (32, 90, 75, 64, 3, 2, True),    # 3x3 s2 with four block rows per lane
+    (3, 21, 20, 16, 3, 2, False),    # 3x3 s2 VALID, unused last column
 ])
 @pytest.mark.parametrize("nan_mode", [False, True])
 def test_maxpool_grad_tiled_kernel(shape, nan_mode):
-    """The work-group-tiled max gradient (3x3 s2, 3x3 s1, 2x2 s2 with
-    channels % 4 == 0): small integers make most windows tie, some NaNs test
-    both NaN rules; results must equal the oracle exactly."""
+    """The specialised max gradients (3x3 s2 by 2 x 2 blocks of dX pixels,
+    3x3 s1 and 2x2 s2 by work-group tiles, channels % 4 == 0): small integers
+    make most windows tie, some NaNs test both NaN rules; results must equal
+    the oracle exactly."""
     n, h, w_, c, win, st, same = shape
     p = ops.pool_params(n, h, w_, c, win, st, same)
     op = oracle_params(p, 0)
