@@ -400,12 +400,24 @@ __global__ void __launch_bounds__(kThreads)
   const int a_r0 = tid >> 3;
   unsigned a_voff[A_PASSES];
   unsigned a_inval[A_PASSES];  // bit t set: filter tap t is padding
+  // A 1x1 window at stride 1 without padding reads row m of the source as it
+  // is (plain GEMM): no pixel decomposition, no tap masks.  The test is
+  // uniform, so a launch pays for one of the two set-ups only.
+  const bool plain_rows = g.win_rows == 1 && g.win_cols == 1 &&
+                          g.step_rows == 1 && g.step_cols == 1 &&
+                          g.off_rows == 0 && g.off_cols == 0 &&
+                          g.src_rows == g.p_rows && g.src_cols == g.p_cols;
 #pragma unroll
   for (int i = 0; i < A_PASSES; ++i) {
     const int m = m0 + a_r0 + 32 * i;
     unsigned inval = 0xFFFFFFFFu;
     int off = 0;
-    if (m < g.m_total) {
+    if (plain_rows) {
+      if (m < g.m_total) {
+        inval = 0;
+        off = m * g.src_ch + 4 * a_cc;
+      }
+    } else if (m < g.m_total) {
       const int px = m % g.p_cols;
       const int t = m / g.p_cols;
       const int py = t % g.p_rows;
