@@ -377,9 +377,6 @@ __global__ void __launch_bounds__(kThreads)
   const int wave = tid >> 6;
   const int wave_m = wave / WN, wave_n = wave % WN;
 
-  const unsigned tile = xcd_remap(blockIdx.x, n_tiles);
-  const int m0 = static_cast<int>(tile / n_tiles_n) * BM;
-  const int n0 = static_cast<int>(tile % n_tiles_n) * BN;
   const int chunks_per_tap = g.src_ch / kBK;
   const int n_chunks_total = g.win_rows * g.win_cols * chunks_per_tap;
   const int chunk_begin = blockIdx.y * chunks_per_split;
@@ -390,6 +387,12 @@ __global__ void __launch_bounds__(kThreads)
   dst += static_cast<size_t>(blockIdx.z) * g.z_dst;
   const __amdgpu_buffer_rsrc_t src_rsrc = make_rsrc(src, src_bytes);
   const __amdgpu_buffer_rsrc_t wgt_rsrc = make_rsrc(wgt, wgt_bytes);
+  const __amdgpu_buffer_rsrc_t dst_rsrc = make_rsrc(dst, dst_bytes);
+
+  // A work-group walks the tiles blockIdx.x, blockIdx.x + gridDim.x, ... (the
+  // launcher starts no more work-groups than fit on the GPU at once), so the
+  // hardware does not have to retire and dispatch a work-group per tile and
+  // the first loads of a tile are in flight while the previous one is stored.
 
   // ---- A gather: lane copies 16 bytes at chunk column a_cc of tile rows
   // a_r0 + 32 * i.  a_voff = byte offset of (n, iy0, ix0, 4 * a_cc) in two's
@@ -407,43 +410,6 @@ __global__ void __launch_bounds__(kThreads)
                           g.step_rows == 1 && g.step_cols == 1 &&
                           g.off_rows == 0 && g.off_cols == 0 &&
                           g.src_rows == g.p_rows && g.src_cols == g.p_cols;
-#pragma unroll
-  for (int i = 0; i < A_PASSES; ++i) {
-    const int m = m0 + a_r0 + 32 * i;
-    unsigned inval = 0xFFFFFFFFu;
-    int off = 0;
-    if (plain_rows) {
-      if (m < g.m_total) {
-        inval = 0;
-        off = m * g.src_ch + 4 * a_cc;
-      }
-    } else if (m < g.m_total) {
-      const int px = m % g.p_cols;
-      const int t = m / g.p_cols;
-      const int py = t % g.p_rows;
-      const int n = t / g.p_rows;
-      const int iy0 = py * g.step_rows + g.off_rows;
-      const int ix0 = px * g.step_cols + g.off_cols;
-      off = ((n * g.src_rows + iy0) * g.src_cols + ix0) * g.src_ch + 4 * a_cc;
-      // bit c of col_bad: tap column c falls outside the source row
-      unsigned col_bad = 0;
-      for (int c = 0; c < g.win_cols; ++c) {
-        const unsigned ix = static_cast<unsigned>(ix0 + g.tap_sign * c);
-        col_bad |= (ix < static_cast<unsigned>(g.src_cols) ? 0u : 1u) << c;
-      }
-      const unsigned all_cols = (1u << g.win_cols) - 1u;  // win_cols <= 31
-      inval = 0;
-      int shift = 0;
-      for (int r = 0; r < g.win_rows; ++r, shift += g.win_cols) {
-        const unsigned iy = static_cast<unsigned>(iy0 + g.tap_sign * r);
-        const unsigned row =
-            iy < static_cast<unsigned>(g.src_rows) ? col_bad : all_cols;
-        inval |= row << shift;
-      }
-    }
-    a_voff[i] = static_cast<unsigned>(off) * 4u;
-    a_inval[i] = inval;
-  }
 
   // ---- B copy: per-lane constant offsets, scalar chunk offsets
   constexpr int B_VEC_PER_ROW = B_K_INNER ? kBK / 4 : BN / 4;
@@ -452,20 +418,6 @@ __global__ void __launch_bounds__(kThreads)
   const int b_vec = tid % B_VEC_PER_ROW;
   const int b_row0 = tid / B_VEC_PER_ROW;
   unsigned b_voff[B_K_INNER ? B_PASSES : 1];
-  if (B_K_INNER) {
-#pragma unroll
-    for (int i = 0; i < B_PASSES; ++i) {
-      const int col = n0 + b_row0 + B_ROWS_PER_PASS * i;
-      b_voff[i] = col < g.n_total
-                      ? static_cast<unsigned>(col * g.src_ch + 4 * b_vec) * 4u
-                      : kOob;
-    }
-  } else {
-    const int col = n0 + 4 * b_vec;
-    b_voff[0] = col < g.n_total
-                    ? static_cast<unsigned>(b_row0 * g.n_total + col) * 4u
-                    : kOob;
-  }
   // scalar byte strides
   const unsigned b_pass_stride =
       static_cast<unsigned>(B_ROWS_PER_PASS * g.n_total) * 4u;  // NN only
@@ -473,18 +425,80 @@ __global__ void __launch_bounds__(kThreads)
       static_cast<unsigned>(g.n_total * g.src_ch) * 4u;  // K-inner only
 
   // wave-uniform reduction position: tap index, its (row, col), channel base
-  int tap = chunk_begin / chunks_per_tap;
-  int c0 = (chunk_begin - tap * chunks_per_tap) * kBK;
-  int tap_r = tap / g.win_cols;
-  int tap_c = tap - tap_r * g.win_cols;
-  int chunk = chunk_begin;
+  int tap, c0, tap_r, tap_c, chunk;
+  const int chunk_end = chunk_begin + n_chunks;
+
+  // Per-tile set-up of the load side: addresses of tile `logical` and the
+  // reduction position back at the start of this work-group's chunk range.
+  auto setup_tile = [&](unsigned logical, int* m0_out, int* n0_out) {
+    const unsigned tile = xcd_remap(logical, n_tiles);
+    const int m0 = static_cast<int>(tile / n_tiles_n) * BM;
+    const int n0 = static_cast<int>(tile % n_tiles_n) * BN;
+    *m0_out = m0;
+    *n0_out = n0;
+#pragma unroll
+    for (int i = 0; i < A_PASSES; ++i) {
+      const int m = m0 + a_r0 + 32 * i;
+      unsigned inval = 0xFFFFFFFFu;
+      int off = 0;
+      if (plain_rows) {
+        if (m < g.m_total) {
+          inval = 0;
+          off = m * g.src_ch + 4 * a_cc;
+        }
+      } else if (m < g.m_total) {
+        const int px = m % g.p_cols;
+        const int t = m / g.p_cols;
+        const int py = t % g.p_rows;
+        const int n = t / g.p_rows;
+        const int iy0 = py * g.step_rows + g.off_rows;
+        const int ix0 = px * g.step_cols + g.off_cols;
+        off = ((n * g.src_rows + iy0) * g.src_cols + ix0) * g.src_ch + 4 * a_cc;
+        // bit c of col_bad: tap column c falls outside the source row
+        unsigned col_bad = 0;
+        for (int c = 0; c < g.win_cols; ++c) {
+          const unsigned ix = static_cast<unsigned>(ix0 + g.tap_sign * c);
+          col_bad |= (ix < static_cast<unsigned>(g.src_cols) ? 0u : 1u) << c;
+        }
+        const unsigned all_cols = (1u << g.win_cols) - 1u;  // win_cols <= 31
+        inval = 0;
+        int shift = 0;
+        for (int r = 0; r < g.win_rows; ++r, shift += g.win_cols) {
+          const unsigned iy = static_cast<unsigned>(iy0 + g.tap_sign * r);
+          const unsigned row =
+              iy < static_cast<unsigned>(g.src_rows) ? col_bad : all_cols;
+          inval |= row << shift;
+        }
+      }
+      a_voff[i] = static_cast<unsigned>(off) * 4u;
+      a_inval[i] = inval;
+    }
+    if (B_K_INNER) {
+#pragma unroll
+      for (int i = 0; i < B_PASSES; ++i) {
+        const int col = n0 + b_row0 + B_ROWS_PER_PASS * i;
+        b_voff[i] = col < g.n_total
+                        ? static_cast<unsigned>(col * g.src_ch + 4 * b_vec) * 4u
+                        : kOob;
+      }
+    } else {
+      const int col = n0 + 4 * b_vec;
+      b_voff[0] = col < g.n_total
+                      ? static_cast<unsigned>(b_row0 * g.n_total + col) * 4u
+                      : kOob;
+    }
+    tap = chunk_begin / chunks_per_tap;
+    c0 = (chunk_begin - tap * chunks_per_tap) * kBK;
+    tap_r = tap / g.win_cols;
+    tap_c = tap - tap_r * g.win_cols;
+    chunk = chunk_begin;
+  };
 
   // Two register sets: the global loads of a chunk are issued two chunks
   // before its data is written to LDS, so their latency is covered by two
   // chunks of MFMA work (a wave of a 64x64 tile has only 16 MFMAs per chunk).
   float4 a_reg[2][A_PASSES];
   float4 b_reg[2][B_PASSES];
-  const int chunk_end = chunk_begin + n_chunks;
 
   auto load_global = [&](int set) {
     if (chunk >= chunk_end) return;  // wave-uniform
@@ -547,82 +561,102 @@ __global__ void __launch_bounds__(kThreads)
   };
 
   float16v acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
   auto compute = [&](int stage) {
     mma_chunk<TM, TN, true, B_K_INNER, BM, BN>(
         lds + stage * STAGE_FLOATS, lds + stage * STAGE_FLOATS + A_FLOATS,
         wave_m * WTM, wave_n * WTN, lane, acc);
   };
 
-  // Chunk j is loaded into register set j % 2 and staged in LDS stage j % 2.
-  // The loop is unrolled by two so that stage and set are literals (every LDS
-  // address is then a per-lane constant plus an immediate).
-  load_global(0);  // chunk 0
-  store_tiles(0, 0);
-  __syncthreads();
-  load_global(1);  // chunk 1
-  for (int done = 0;; done += 2) {
-    load_global(0);  // chunk done + 2
-    compute(0);      // chunk done
-    if (done + 1 >= n_chunks) break;
-    store_tiles(1, 1);  // chunk done + 1
-    __syncthreads();
-    load_global(1);  // chunk done + 3
-    compute(1);      // chunk done + 1
-    if (done + 2 >= n_chunks) break;
-    store_tiles(0, 0);  // chunk done + 2
-    __syncthreads();
-  }
-
-  // ---- epilogue through a buffer descriptor: rows past the end fall outside
-  // it and are dropped; per-lane constant offset + scalar row offsets.
-  const __amdgpu_buffer_rsrc_t dst_rsrc = make_rsrc(dst, dst_bytes);
   const int col_l = lane & 31;
   const int row_l = 4 * (lane >> 5);
   const unsigned row_bytes = static_cast<unsigned>(g.n_total) * 4u;
+
+  unsigned logical = blockIdx.x;
+  int m0, n0;
+  setup_tile(logical, &m0, &n0);
+  load_global(0);  // chunk 0 of the first tile
+  while (true) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int col = n0 + wave_n * WTN + 32 * j + col_l;
-      const int m_base = m0 + wave_m * WTM + 32 * i + row_l;
-      const unsigned voff =
-          (col < g.n_total && m_base < g.m_total)
-              ? static_cast<unsigned>(m_base) * row_bytes +
-                    static_cast<unsigned>(col) * 4u
-              : kOob;
-      float bias_col = 0.f;
-      if (EPI) {
-        if (bias != nullptr && col < g.n_total) bias_col = bias[col];
-      }
-      // The row offset goes into the vector offset, not the scalar offset
-      // operand: hipcc (ROCm 7.2) treats buffer stores that differ only in
-      // their scalar offset as stores to one address and forwards the first
-      // value to all of them.
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const unsigned off =
-            voff + static_cast<unsigned>(8 * (v >> 2) + (v & 3)) * row_bytes;
-        float val = acc[i][j][v];
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    // Chunk j is loaded into register set j % 2 and staged in LDS stage
+    // j % 2.  The loop is unrolled by two so that stage and set are literals
+    // (every LDS address is then a per-lane constant plus an immediate).
+    store_tiles(0, 0);
+    __syncthreads();
+    load_global(1);  // chunk 1
+    for (int done = 0;; done += 2) {
+      load_global(0);  // chunk done + 2
+      compute(0);      // chunk done
+      if (done + 1 >= n_chunks) break;
+      store_tiles(1, 1);  // chunk done + 1
+      __syncthreads();
+      load_global(1);  // chunk done + 3
+      compute(1);      // chunk done + 1
+      if (done + 2 >= n_chunks) break;
+      store_tiles(0, 0);  // chunk done + 2
+      __syncthreads();
+    }
+
+    // The next tile's addresses and its first chunk's loads, so that they
+    // are in flight during the stores below.
+    const int m0_done = m0, n0_done = n0;
+    logical += gridDim.x;
+    const bool more = logical < n_tiles;  // uniform
+    if (more) {
+      setup_tile(logical, &m0, &n0);
+      load_global(0);
+    }
+
+    // ---- epilogue through a buffer descriptor: rows past the end fall
+    // outside it and are dropped; per-lane constant offset + scalar row
+    // offsets.
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = n0_done + wave_n * WTN + 32 * j + col_l;
+        const int m_base = m0_done + wave_m * WTM + 32 * i + row_l;
+        const unsigned voff =
+            (col < g.n_total && m_base < g.m_total)
+                ? static_cast<unsigned>(m_base) * row_bytes +
+                      static_cast<unsigned>(col) * 4u
+                : kOob;
+        float bias_col = 0.f;
         if (EPI) {
-          val += bias_col;
-          if (relu) val = fmaxf(val, 0.f);
+          if (bias != nullptr && col < g.n_total) bias_col = bias[col];
         }
-        if (ATOMIC) {
-          __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(val, dst_rsrc, off, 0,
-                                                          0);
-        } else {
-          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), dst_rsrc,
-                                                off, 0, 0);
+        // The row offset goes into the vector offset, not the scalar offset
+        // operand: hipcc (ROCm 7.2) treats buffer stores that differ only in
+        // their scalar offset as stores to one address and forwards the first
+        // value to all of them.
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const unsigned off =
+              voff + static_cast<unsigned>(8 * (v >> 2) + (v & 3)) * row_bytes;
+          float val = acc[i][j][v];
+          if (EPI) {
+            val += bias_col;
+            if (relu) val = fmaxf(val, 0.f);
+          }
+          if (ATOMIC) {
+            __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(val, dst_rsrc, off,
+                                                            0, 0);
+          } else {
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val),
+                                                  dst_rsrc, off, 0, 0);
+          }
         }
       }
     }
+    if (!more) break;
+    // every wave is done reading the last LDS stage of this tile before the
+    // next tile's first chunk is written
+    __syncthreads();
   }
 }
 
@@ -1030,6 +1064,39 @@ __global__ void __launch_bounds__(256)
   if (i < n_vec) p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
+// Number of work-groups along x for the fast kernel, which walks tiles
+// x, x + gridDim.x, ...: as many as the GPU holds at once (CUs times the
+// work-groups of this kernel one CU can host), shared between the `yz`
+// reduction splits and batches of the launch, in whole rounds of the 8 XCDs;
+// one work-group per tile when there are fewer than four tiles for each.
+template <typename Kernel>
+unsigned resident_groups(Kernel kernel, size_t lds_bytes) {
+  int per_cu = 0, device = 0, cus = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(
+          &per_cu, reinterpret_cast<const void*>(kernel), kThreads,
+          lds_bytes) != hipSuccess ||
+      hipGetDevice(&device) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount,
+                            device) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return static_cast<unsigned>(max(per_cu, 1)) * static_cast<unsigned>(cus);
+}
+
+inline unsigned persistent_grid_x(unsigned resident, unsigned n_tiles,
+                                  unsigned yz) {
+  static const bool off = getenv("SNN_HIP_IGEMM_ONE_TILE") != nullptr;
+  if (off || resident == 0) return n_tiles;
+  unsigned gx = resident / max(yz, 1u);
+  gx -= gx % 8u;
+  if (gx < 8u) gx = 8u;
+  // Tiles are dealt round-robin, so with only a few per work-group the
+  // uneven shares cost more than the saved dispatches (measured: 1.5 tiles
+  // per work-group ran 20 % slower than one work-group per tile).
+  return n_tiles >= 4u * gx ? gx : n_tiles;
+}
+
 template <int BM, int BN, int WM, int WN, bool B_K_INNER, bool STRIDED>
 void launch_tile(const float* src, const float* wgt, float* dst,
                  const Gather& g, size_t src_elems, size_t wgt_elems,
@@ -1071,7 +1138,10 @@ void launch_tile(const float* src, const float* wgt, float* dst,
           reinterpret_cast<const void*>(kernel),
           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
       (void)attr;
-      hipLaunchKernelGGL(kernel, dim3(n_tiles, splits, batches),
+      static const unsigned resident = resident_groups(kernel, kLdsBytes);
+      const unsigned gx = persistent_grid_x(
+          resident, n_tiles, static_cast<unsigned>(splits * batches));
+      hipLaunchKernelGGL(kernel, dim3(gx, splits, batches),
                          dim3(kThreads), kLdsBytes, stream, src, wgt, dst, g,
                          src_bytes, wgt_bytes, dst_bytes, tiles_n, n_tiles,
                          per_split, static_cast<const float*>(nullptr), 0);
@@ -1094,7 +1164,9 @@ void launch_tile(const float* src, const float* wgt, float* dst,
           reinterpret_cast<const void*>(kernel),
           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
       (void)attr;
-      hipLaunchKernelGGL(kernel, dim3(n_tiles, 1, 1), dim3(kThreads),
+      static const unsigned resident = resident_groups(kernel, kLdsBytes);
+      const unsigned gx = persistent_grid_x(resident, n_tiles, 1u);
+      hipLaunchKernelGGL(kernel, dim3(gx, 1, 1), dim3(kThreads),
                          kLdsBytes, stream, src, wgt, dst, g, src_bytes,
                          wgt_bytes, dst_bytes, tiles_n, n_tiles, per_split,
                          epilogue->bias, epilogue->relu ? 1 : 0);
@@ -1107,7 +1179,10 @@ void launch_tile(const float* src, const float* wgt, float* dst,
           reinterpret_cast<const void*>(kernel),
           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
       (void)attr;
-      hipLaunchKernelGGL(kernel, dim3(n_tiles, 1, batches), dim3(kThreads),
+      static const unsigned resident = resident_groups(kernel, kLdsBytes);
+      const unsigned gx = persistent_grid_x(
+          resident, n_tiles, static_cast<unsigned>(batches));
+      hipLaunchKernelGGL(kernel, dim3(gx, 1, batches), dim3(kThreads),
                          kLdsBytes, stream, src, wgt, dst, g, src_bytes,
                          wgt_bytes, dst_bytes, tiles_n, n_tiles, per_split,
                          static_cast<const float*>(nullptr), 0);
