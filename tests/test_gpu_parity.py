@@ -537,6 +537,45 @@ def test_matmul(trans_a, trans_b, shape):
         assert_close(got, ref, ("matmul", shape, trans_a, trans_b, beta))
 
 
+def test_many_tiles_per_work_group_epilogue_and_accumulate():
+    """Launches with thousands of 64 x 64 tiles make the implicit-GEMM
+    work-groups walk several tiles each.  At that size: the fused bias + ReLU
+    epilogue must equal the Direct convolution followed by the two element-wise
+    steps, and a matmul that accumulates (beta = 1) must equal the plain
+    product plus the previous contents; a small slice is checked against the
+    oracle as well."""
+    p = ops.conv_params(32, 56, 56, 64, 256, 1, 1, False)
+    rng = np.random.default_rng(4242)
+    n_in, n_fil, n_out = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x, w = uniform(rng, n_in), uniform(rng, n_fil)
+    bias = uniform(rng, 256) * 4
+    dx, dw, db = dev(x), dev(w), dev(bias)
+    base = ops.conv2d(dx, dw, p, DIRECTION.FORWARD, ALGO.DIRECT)
+    want = torch.relu(base.view(-1, 256) + db).view(-1)
+    scale = max(1.0, float(base.pow(2).mean().sqrt()))
+    for algo in (ALGO.MATMUL, ALGO.IM2COL, ALGO.TILED):
+        got = ops.conv2d_bias_act(dx, dw, db, p, algo, relu=True)
+        diff = (got - want).abs()
+        assert bool((diff <= 2 * (RTOL * want.abs() + ATOL * scale)).all()), (
+            ALGO_NAME[algo], diff.max().item())
+    # first 64 pixels against the oracle (1x1: rows of a GEMM)
+    ref = oracle.matmul(x[:64 * 64], w, 1, 64, 64, 256, False, False, 0.0)
+    ref = np.maximum(ref.reshape(64, 256) + bias, 0).reshape(-1)
+    got = ops.conv2d_bias_act(dx, dw, db, p, ALGO.MATMUL, relu=True)
+    assert_close(got[:64 * 256].cpu().numpy(), ref, "bias_act slice")
+
+    m, k, n = 100352, 64, 256
+    c0 = dev(uniform(rng, m * n))
+    plain = ops.matmul(dx, dw, 1, m, k, n, False, False, 0.0,
+                       out=torch.empty(m * n, device="cuda"))
+    acc = ops.matmul(dx, dw, 1, m, k, n, False, False, 1.0, out=c0.clone())
+    diff = (acc - (plain + c0)).abs()
+    assert bool((diff <= 2 * (RTOL * (plain + c0).abs() + ATOL * scale)).all())
+    assert_close(plain[:64 * 256].cpu().numpy(),
+                 oracle.matmul(x[:64 * 64], w, 1, 64, 64, 256, False, False,
+                               0.0), "matmul slice")
+
+
 # ---- f16 ---------------------------------------------------------------------
 
 def assert_close_f16(got, ref, what):
