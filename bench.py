@@ -253,6 +253,22 @@ def main():
                     window, window, size, size, ch, feats), "ms": round(ms, 4),
                     "tflops": round(fl / ms / 1e9, 1),
                     "frac_f16_mfma_peak": round(fl / ms / 1e9 / 2500.0, 4)})
+                if window == 3:
+                    # input gradient: the same kernel on dY (o) with the
+                    # filter's taps mirrored and its roles swapped
+                    dx = torch.empty(n_a, device="cuda", dtype=torch.float16)
+                    o.copy_(uniform(n_o).half())
+                    ms = event_time_ms(lambda: ops.conv2d(
+                        o, b, p, DIRECTION.INPUT_BACKPROP, ALGO.IM2COL,
+                        workspace=ws, out=dx), reps=10, warm=2, repeats=3)
+                    fl = ops.conv_flops(p, DIRECTION.INPUT_BACKPROP)
+                    h.append({"op": "conv3x3_%dx%dx%d_k%d_b128_f16_input_"
+                              "backprop" % (size, size, ch, feats),
+                              "ms": round(ms, 4),
+                              "tflops": round(fl / ms / 1e9, 1),
+                              "frac_f16_mfma_peak": round(
+                                  fl / ms / 1e9 / 2500.0, 4)})
+                    del dx
                 del a, b, o, ws
         for size, ch, stride in MOBILENET:
             p = ops.depthwise_params(128, size, size, ch, 1, 3, stride, True)

@@ -271,7 +271,11 @@ inline int call(T const* input, T const* filter, T* output,
     if (dir == SNN_HIP_FORWARD)
       return snn_hip_conv2d_forward_f16(input, filter, output, &c, algo,
                                         workspace, workspace_size, stream);
-    return SNN_HIP_INVALID_ALGORITHM;  // half backprop is not provided
+    if (dir == SNN_HIP_INPUT_BACKPROP)
+      return snn_hip_conv2d_input_backprop_f16(
+          input, filter, output, &c, algo, workspace, workspace_size, stream);
+    return snn_hip_conv2d_filter_backprop_f16(
+        input, filter, output, &c, algo, workspace, workspace_size, stream);
   }
 }
 

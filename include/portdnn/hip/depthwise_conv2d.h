@@ -81,7 +81,11 @@ SNNStatus launch(typename Backend::template pointer_type<T const> input,
     code = dir == SNN_HIP_FORWARD
                ? snn_hip_depthwise_conv2d_forward_f16(input, filter, output,
                                                       &c, stream)
-               : SNN_HIP_INVALID_ALGORITHM;
+           : dir == SNN_HIP_INPUT_BACKPROP
+               ? snn_hip_depthwise_conv2d_input_backprop_f16(
+                     input, filter, output, &c, stream)
+               : snn_hip_depthwise_conv2d_filter_backprop_f16(
+                     input, filter, output, &c, stream);
   }
   return hip::detail::finish(code, stream);
 }

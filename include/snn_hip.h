@@ -190,6 +190,19 @@ SNN_HIP_API int snn_hip_conv2d_forward_f16(
     const void* input, const void* filter, void* output,
     const snn_hip_conv2d_params* params, int algorithm, void* workspace,
     size_t workspace_elems, void* stream);
+/* The two gradients in half precision (fp32 accumulation), the reference's
+ * launch<half, conv_type::InputBackprop / FilterBackprop>.  Stride-1 input
+ * gradients with channel and feature counts in multiples of 64 run on the
+ * matrix cores; everything else, and the filter gradient, on the direct
+ * kernels. */
+SNN_HIP_API int snn_hip_conv2d_input_backprop_f16(
+    const void* input, const void* filter, void* output,
+    const snn_hip_conv2d_params* params, int algorithm, void* workspace,
+    size_t workspace_elems, void* stream);
+SNN_HIP_API int snn_hip_conv2d_filter_backprop_f16(
+    const void* input, const void* filter, void* output,
+    const snn_hip_conv2d_params* params, int algorithm, void* workspace,
+    size_t workspace_elems, void* stream);
 
 /* sycldnn::conv2d::query_workspace_size<ConvType>(params, selector)
  * (include/portdnn/conv2d/workspace_size.h:158-163) for an already selected
@@ -227,6 +240,12 @@ SNN_HIP_API int snn_hip_depthwise_conv2d_filter_backprop_f32(
     const float* input, const float* filter, float* output,
     const snn_hip_depthwise_params* params, void* stream);
 SNN_HIP_API int snn_hip_depthwise_conv2d_forward_f16(
+    const void* input, const void* filter, void* output,
+    const snn_hip_depthwise_params* params, void* stream);
+SNN_HIP_API int snn_hip_depthwise_conv2d_input_backprop_f16(
+    const void* input, const void* filter, void* output,
+    const snn_hip_depthwise_params* params, void* stream);
+SNN_HIP_API int snn_hip_depthwise_conv2d_filter_backprop_f16(
     const void* input, const void* filter, void* output,
     const snn_hip_depthwise_params* params, void* stream);
 

@@ -116,6 +116,8 @@ SIGNATURES = {
     "snn_hip_conv2d_input_backprop_f32": [_P, _P, _P, _P, _I, _P, _SZ, _P],
     "snn_hip_conv2d_filter_backprop_f32": [_P, _P, _P, _P, _I, _P, _SZ, _P],
     "snn_hip_conv2d_forward_f16": [_P, _P, _P, _P, _I, _P, _SZ, _P],
+    "snn_hip_conv2d_input_backprop_f16": [_P, _P, _P, _P, _I, _P, _SZ, _P],
+    "snn_hip_conv2d_filter_backprop_f16": [_P, _P, _P, _P, _I, _P, _SZ, _P],
     "snn_hip_conv2d_forward_bias_act_f32": [_P, _P, _P, _P, _P, _I, _I, _P,
                                             _SZ, _P],
     "snn_hip_conv2d_workspace_size": [_P, _I, _I, ctypes.POINTER(_SZ),
@@ -126,6 +128,8 @@ SIGNATURES = {
     "snn_hip_depthwise_conv2d_input_backprop_f32": [_P, _P, _P, _P, _P],
     "snn_hip_depthwise_conv2d_filter_backprop_f32": [_P, _P, _P, _P, _P],
     "snn_hip_depthwise_conv2d_forward_f16": [_P, _P, _P, _P, _P],
+    "snn_hip_depthwise_conv2d_input_backprop_f16": [_P, _P, _P, _P, _P],
+    "snn_hip_depthwise_conv2d_filter_backprop_f16": [_P, _P, _P, _P, _P],
     "snn_hip_pooling_forward_f32": [_P, _P, _P, _I, _P],
     "snn_hip_pooling_forward_f16": [_P, _P, _P, _I, _P],
     "snn_hip_pooling_max_grad_f32": [_P, _P, _P, _P, _P, _I, _P],

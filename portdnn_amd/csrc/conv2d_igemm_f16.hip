@@ -345,4 +345,87 @@ int launch_conv2d_igemm_f16(const _Float16* input, const _Float16* filter,
   return SNN_HIP_OK;
 }
 
+// The input gradient of a stride-1 convolution as a forward convolution of
+// dY: channels and features trade places, padding becomes window - 1 - pad.
+static bool as_forward_of_dy(const snn_hip_conv2d_params& p,
+                             snn_hip_conv2d_params* q) {
+  if (p.stride_rows != 1 || p.stride_cols != 1) return false;
+  if (p.pad_rows > p.window_rows - 1 || p.pad_cols > p.window_cols - 1)
+    return false;
+  *q = p;
+  q->channels = p.features;
+  q->features = p.channels;
+  q->in_rows = p.out_rows;
+  q->in_cols = p.out_cols;
+  q->out_rows = p.in_rows;
+  q->out_cols = p.in_cols;
+  q->pad_rows = p.window_rows - 1 - p.pad_rows;
+  q->pad_cols = p.window_cols - 1 - p.pad_cols;
+  return true;
+}
+
+bool conv2d_input_backprop_f16_supports(const snn_hip_conv2d_params& p) {
+  snn_hip_conv2d_params q;
+  if (!as_forward_of_dy(p, &q)) return false;
+  if (conv2d_rowtile_f16_supports(q)) return true;
+  // 1x1: W[c][k] already is the gradient's filter with the reduction index
+  // (k) contiguous, the layout the implicit-GEMM kernel wants
+  return p.window_rows == 1 && p.window_cols == 1 &&
+         conv2d_igemm_f16_supports(q);
+}
+
+int launch_conv2d_input_backprop_f16(const _Float16* dy,
+                                     const _Float16* filter, _Float16* dx,
+                                     const snn_hip_conv2d_params& p,
+                                     _Float16* workspace,
+                                     size_t workspace_elems,
+                                     hipStream_t stream) {
+  snn_hip_conv2d_params q;
+  if (!as_forward_of_dy(p, &q)) return SNN_HIP_INVALID_ALGORITHM;
+  const size_t wgt_elems = static_cast<size_t>(p.window_rows) * p.window_cols *
+                           p.channels * p.features;
+  if (conv2d_rowtile_f16_supports(q)) {
+    _Float16* packed = workspace;
+    bool temporary = false;
+    if (workspace == nullptr || workspace_elems < wgt_elems ||
+        (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) {
+      void* ptr = nullptr;
+      if (hipMallocAsync(&ptr, wgt_elems * sizeof(_Float16), stream) !=
+          hipSuccess)
+        return SNN_HIP_ALLOCATION_PROBLEM;
+      packed = static_cast<_Float16*>(ptr);
+      temporary = true;
+    }
+    const int status =
+        launch_conv2d_rowtile_f16(dy, filter, dx, q, packed, stream, true);
+    if (temporary) (void)hipFreeAsync(packed, stream);
+    return status;
+  }
+  if (p.window_rows != 1 || p.window_cols != 1 || !conv2d_igemm_f16_supports(q))
+    return SNN_HIP_INVALID_ALGORITHM;
+  GatherH g;
+  g.p_rows = q.out_rows; g.p_cols = q.out_cols;
+  g.src_rows = q.in_rows; g.src_cols = q.in_cols;
+  g.src_ch = q.channels;
+  g.win_rows = 1; g.win_cols = 1;
+  g.step_rows = 1; g.step_cols = 1;
+  g.off_rows = -q.pad_rows; g.off_cols = -q.pad_cols;
+  g.m_total = q.batch * q.out_rows * q.out_cols;
+  g.n_total = q.features;
+  const size_t src_elems =
+      static_cast<size_t>(q.batch) * q.in_rows * q.in_cols * q.channels;
+  const long big = static_cast<long>(ceil_div(g.m_total, 128)) *
+                   ceil_div(g.n_total, 128);
+  if (g.n_total > 64 && big >= 512)
+    launch_f16_tile<128, 128, 2, 2>(dy, filter, dx, g, src_elems, wgt_elems,
+                                    stream);
+  else
+    launch_f16_tile<64, 64, 2, 2>(dy, filter, dx, g, src_elems, wgt_elems,
+                                  stream);
+  const hipError_t launch_err = hipGetLastError();
+  if (launch_err != hipSuccess)
+    return report_hip_error(launch_err, "conv_igemm_f16_kernel");
+  return SNN_HIP_OK;
+}
+
 }  // namespace snn

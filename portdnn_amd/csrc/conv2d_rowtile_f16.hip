@@ -76,11 +76,15 @@ __device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* p,
 // (KC / 16) + ks, c = chunk * KC + ks * 16 + 8 * (lane / 32) + e and, for
 // MFMA row rho = lane % 32, f = fb * 32 + 16 * ((rho / 4) % 2) + 4 * (rho / 8)
 // + rho % 4: the accumulator rows 8g + 4h + i a lane holds (h = lane / 32)
-// are then features 16h + 4g + i, 16 consecutive ones.
+// are then features 16h + 4g + i, 16 consecutive ones.  `transposed`: the
+// input gradient's filter, w[taps - 1 - tap][f][c] of the HWCF tensor of a
+// convolution with `features` input channels and `channels` features
+// (mirrored taps, channel and feature roles swapped).
 __global__ void __launch_bounds__(256)
     pack_filter_rowtile_kernel(const _Float16* __restrict__ w,
                                _Float16* __restrict__ wpk, int channels,
-                               int features, int taps, int kc, int n_lanes) {
+                               int features, int taps, int kc, int n_lanes,
+                               bool transposed) {
   // One thread per (step, fb, lane): eight channel values of one feature.
   // The 32 lanes of a half-wave read 32 permuted but adjacent features.
   const int idx = blockIdx.x * 256 + threadIdx.x;
@@ -98,10 +102,14 @@ __global__ void __launch_bounds__(256)
   const int c = chunk * kc + ks * 16 + 8 * (lane >> 5);
   const int rho = lane & 31;
   const int f = fb * 32 + 16 * ((rho >> 2) & 1) + 4 * (rho >> 3) + (rho & 3);
-  const _Float16* src = w + (static_cast<size_t>(tap) * channels + c) * features + f;
+  const _Float16* src =
+      transposed
+          ? w + (static_cast<size_t>(taps - 1 - tap) * features + f) * channels + c
+          : w + (static_cast<size_t>(tap) * channels + c) * features + f;
+  const size_t stride = transposed ? 1 : static_cast<size_t>(features);
   half8 v;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) v[e] = src[static_cast<size_t>(e) * features];
+  for (int e = 0; e < 8; ++e) v[e] = src[static_cast<size_t>(e) * stride];
   *reinterpret_cast<half8*>(wpk + static_cast<size_t>(idx) * 8) = v;
 }
 
@@ -658,7 +666,8 @@ bool conv2d_rowtile_f16_supports(const snn_hip_conv2d_params& p) {
 
 int launch_conv2d_rowtile_f16(const _Float16* input, const _Float16* filter,
                               _Float16* output, const snn_hip_conv2d_params& p,
-                              _Float16* packed, hipStream_t stream) {
+                              _Float16* packed, hipStream_t stream,
+                              bool transposed_filter) {
   const RowTilePlan plan = make_plan(p);
   if (plan.lds_bytes == 0) return SNN_HIP_INVALID_ALGORITHM;
   static const bool print_plan = getenv("SNN_HIP_F16_PLAN") != nullptr;
@@ -675,7 +684,7 @@ int launch_conv2d_rowtile_f16(const _Float16* input, const _Float16* filter,
       pack_filter_rowtile_kernel,
       dim3(static_cast<unsigned>(ceil_div(wgt_elems / 8, size_t{256}))),
       dim3(256), 0, stream, filter, packed, p.channels, p.features, taps,
-      plan.kc, static_cast<int>(wgt_elems / 8));
+      plan.kc, static_cast<int>(wgt_elems / 8), transposed_filter);
   const bool launched =
       launch_shape<1, 2, 2>(input, packed, output, p, plan, wgt_elems, stream) ||
       launch_shape<1, 2, 4>(input, packed, output, p, plan, wgt_elems, stream) ||

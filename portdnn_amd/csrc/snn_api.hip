@@ -303,6 +303,11 @@ int launch_gemm_path<_Float16>(int direction, const _Float16* input,
       aligned16(input) && aligned16(filter) && aligned16(output))
     return launch_conv2d_igemm_f16(input, filter, output, p, workspace,
                                    workspace_elems, s);
+  if (direction == SNN_HIP_INPUT_BACKPROP &&
+      conv2d_input_backprop_f16_supports(p) && aligned16(input) &&
+      aligned16(filter) && aligned16(output))
+    return launch_conv2d_input_backprop_f16(input, filter, output, p,
+                                            workspace, workspace_elems, s);
   return launch_conv2d_direct<_Float16>(direction, input, filter, output, p, s);
 }
 template <>
@@ -590,6 +595,30 @@ int snn_hip_conv2d_forward_f16(const void* input, const void* filter,
       stream);
 }
 
+int snn_hip_conv2d_input_backprop_f16(const void* input, const void* filter,
+                                      void* output,
+                                      const snn_hip_conv2d_params* params,
+                                      int algorithm, void* workspace,
+                                      size_t workspace_elems, void* stream) {
+  return conv2d_dispatch<_Float16>(
+      SNN_HIP_INPUT_BACKPROP, static_cast<const _Float16*>(input),
+      static_cast<const _Float16*>(filter), static_cast<_Float16*>(output),
+      params, algorithm, static_cast<_Float16*>(workspace), workspace_elems,
+      stream);
+}
+
+int snn_hip_conv2d_filter_backprop_f16(const void* input, const void* filter,
+                                       void* output,
+                                       const snn_hip_conv2d_params* params,
+                                       int algorithm, void* workspace,
+                                       size_t workspace_elems, void* stream) {
+  return conv2d_dispatch<_Float16>(
+      SNN_HIP_FILTER_BACKPROP, static_cast<const _Float16*>(input),
+      static_cast<const _Float16*>(filter), static_cast<_Float16*>(output),
+      params, algorithm, static_cast<_Float16*>(workspace), workspace_elems,
+      stream);
+}
+
 int snn_hip_conv2d_workspace_size(const snn_hip_conv2d_params* params,
                                   int direction, int algorithm,
                                   size_t* required_elems,
@@ -641,6 +670,24 @@ int snn_hip_depthwise_conv2d_forward_f16(
     const snn_hip_depthwise_params* params, void* stream) {
   return depthwise_dispatch<_Float16>(
       SNN_HIP_FORWARD, static_cast<const _Float16*>(input),
+      static_cast<const _Float16*>(filter), static_cast<_Float16*>(output),
+      params, stream);
+}
+
+int snn_hip_depthwise_conv2d_input_backprop_f16(
+    const void* input, const void* filter, void* output,
+    const snn_hip_depthwise_params* params, void* stream) {
+  return depthwise_dispatch<_Float16>(
+      SNN_HIP_INPUT_BACKPROP, static_cast<const _Float16*>(input),
+      static_cast<const _Float16*>(filter), static_cast<_Float16*>(output),
+      params, stream);
+}
+
+int snn_hip_depthwise_conv2d_filter_backprop_f16(
+    const void* input, const void* filter, void* output,
+    const snn_hip_depthwise_params* params, void* stream) {
+  return depthwise_dispatch<_Float16>(
+      SNN_HIP_FILTER_BACKPROP, static_cast<const _Float16*>(input),
       static_cast<const _Float16*>(filter), static_cast<_Float16*>(output),
       params, stream);
 }

@@ -76,15 +76,29 @@ int launch_conv2d_igemm_f16(const _Float16* input, const _Float16* filter,
                             _Float16* output, const snn_hip_conv2d_params& p,
                             _Float16* workspace, size_t workspace_elems,
                             hipStream_t stream);
+// Stride-1 input gradient in half precision: the forward kernels above run on
+// dY with the filter's taps mirrored and its channel / feature roles swapped.
+// `supports` is false when neither kernel takes the shape.
+bool conv2d_input_backprop_f16_supports(const snn_hip_conv2d_params& p);
+int launch_conv2d_input_backprop_f16(const _Float16* dy,
+                                     const _Float16* filter, _Float16* dx,
+                                     const snn_hip_conv2d_params& p,
+                                     _Float16* workspace,
+                                     size_t workspace_elems,
+                                     hipStream_t stream);
 
 // Half-precision stride-1 forward convolution with the input tile resident
 // in LDS (conv2d_rowtile_f16.hip).  `packed` receives the filter in MFMA
 // operand order: window_rows * window_cols * channels * features halves,
-// 16-byte aligned.
+// 16-byte aligned.  With `transposed_filter` the filter is read as the input
+// gradient's: `p` then describes the gradient as a forward convolution of dY
+// (channels = the original features and vice versa, padding window - 1 - pad)
+// and `filter` is still the original HWCF tensor.
 bool conv2d_rowtile_f16_supports(const snn_hip_conv2d_params& p);
 int launch_conv2d_rowtile_f16(const _Float16* input, const _Float16* filter,
                               _Float16* output, const snn_hip_conv2d_params& p,
-                              _Float16* packed, hipStream_t stream);
+                              _Float16* packed, hipStream_t stream,
+                              bool transposed_filter = false);
 
 // Depthwise convolution, all three directions (depthwise.hip).
 template <typename T>

@@ -100,6 +100,10 @@ _CONV_FN = {
     (DIRECTION.FILTER_BACKPROP, torch.float32):
         "snn_hip_conv2d_filter_backprop_f32",
     (DIRECTION.FORWARD, torch.float16): "snn_hip_conv2d_forward_f16",
+    (DIRECTION.INPUT_BACKPROP, torch.float16):
+        "snn_hip_conv2d_input_backprop_f16",
+    (DIRECTION.FILTER_BACKPROP, torch.float16):
+        "snn_hip_conv2d_filter_backprop_f16",
 }
 
 
@@ -150,6 +154,10 @@ _DW_FN = {
     (DIRECTION.FILTER_BACKPROP, torch.float32):
         "snn_hip_depthwise_conv2d_filter_backprop_f32",
     (DIRECTION.FORWARD, torch.float16): "snn_hip_depthwise_conv2d_forward_f16",
+    (DIRECTION.INPUT_BACKPROP, torch.float16):
+        "snn_hip_depthwise_conv2d_input_backprop_f16",
+    (DIRECTION.FILTER_BACKPROP, torch.float16):
+        "snn_hip_depthwise_conv2d_filter_backprop_f16",
 }
 
 

@@ -688,6 +688,79 @@ def test_f16_conv_forward_full_batch_sampled(size, ch, feats, window):
     assert_close_f16(got[flat], ref, ("f16 batch 128 sampled", size, window))
 
 
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, win_rows, win_cols, stride, same
+    (3, 14, 14, 64, 128, 3, 3, 1, True),    # LDS-tile kernel on dY
+    (2, 28, 28, 192, 64, 3, 3, 1, True),    # three feature blocks reduced
+    (2, 11, 13, 64, 64, 3, 3, 1, False),    # VALID: padding 2 on dY
+    (3, 12, 10, 128, 128, 5, 5, 1, True),   # 25 mirrored taps
+    (2, 9, 20, 128, 256, 1, 3, 1, True),    # 1 x 3 window
+    (7, 5, 5, 256, 320, 1, 1, 1, False),    # 1x1: implicit-GEMM kernel
+    (2, 28, 28, 128, 512, 1, 1, 1, False),  # 1x1, 128 x 128 tiles
+    (2, 17, 9, 128, 64, 3, 3, 2, True),     # stride 2: direct kernel
+    (2, 8, 8, 24, 40, 3, 3, 1, True),       # few channels: direct kernel
+])
+def test_f16_conv_input_backprop(shape):
+    """Half-precision input gradient (fp32 accumulation) against the oracle in
+    double precision on the same half-rounded operands."""
+    batch, rows, cols, ch, feats, wr, wc, stride, same = shape
+    p = ops.add_padding_to(ops.ConvParams(
+        channels=ch, features=feats, batch=batch, in_rows=rows, in_cols=cols,
+        window_rows=wr, window_cols=wc, stride_rows=stride,
+        stride_cols=stride), same)
+    rng = np.random.default_rng(780 + rows * cols + feats)
+    n_dy, n_fil, _ = ops.conv_sizes(p, DIRECTION.INPUT_BACKPROP)
+    dy = uniform(rng, n_dy).astype(np.float16)
+    w = uniform(rng, n_fil).astype(np.float16)
+    ref = oracle.conv2d_input_backprop(dy.astype(np.float32),
+                                       w.astype(np.float32),
+                                       oracle_params(p, feats), acc64=True)
+    for algo in (ALGO.IM2COL, ALGO.DIRECT):
+        got = ops.conv2d(dev(dy, torch.float16), dev(w, torch.float16), p,
+                         DIRECTION.INPUT_BACKPROP, algo).float().cpu().numpy()
+        assert_close_f16(got, ref, ("f16 inbk", ALGO_NAME[algo], shape))
+
+
+def test_f16_conv_filter_backprop():
+    p = ops.conv_params(3, 10, 9, 16, 24, 3, 1, True)
+    rng = np.random.default_rng(781)
+    n_x, n_dy, _ = ops.conv_sizes(p, DIRECTION.FILTER_BACKPROP)
+    x = uniform(rng, n_x).astype(np.float16)
+    dy = uniform(rng, n_dy).astype(np.float16)
+    ref = oracle.conv2d_filter_backprop(x.astype(np.float32),
+                                        dy.astype(np.float32),
+                                        oracle_params(p, 24), acc64=True)
+    got = ops.conv2d(dev(x, torch.float16), dev(dy, torch.float16), p,
+                     DIRECTION.FILTER_BACKPROP,
+                     ALGO.IM2COL).float().cpu().numpy()
+    assert_close_f16(got, ref, "f16 filbk")
+
+
+@pytest.mark.parametrize("shape", [(2, 28, 28, 64, 1), (2, 28, 28, 64, 2),
+                                   (3, 13, 11, 8, 2), (1, 9, 9, 6, 1)])
+def test_f16_depthwise_backprops(shape):
+    n, h, w_, c, stride = shape
+    p = ops.depthwise_params(n, h, w_, c, 1, 3, stride, True)
+    op = oracle_params(p, 1)
+    rng = np.random.default_rng(790 + h + c)
+    x = rng.standard_normal(n * h * w_ * c).astype(np.float16)
+    w = rng.standard_normal(9 * c).astype(np.float16)
+    dy = rng.standard_normal(n * p.out_rows * p.out_cols * c).astype(
+        np.float16)
+    got = ops.depthwise_conv2d(dev(dy, torch.float16), dev(w, torch.float16),
+                               p, DIRECTION.INPUT_BACKPROP)
+    assert_close_f16(got.float().cpu().numpy(),
+                     oracle.depthwise_input_backprop(
+                         dy.astype(np.float32), w.astype(np.float32), op),
+                     ("f16 dw inbk", shape))
+    got = ops.depthwise_conv2d(dev(x, torch.float16), dev(dy, torch.float16),
+                               p, DIRECTION.FILTER_BACKPROP)
+    assert_close_f16(got.float().cpu().numpy(),
+                     oracle.depthwise_filter_backprop(
+                         x.astype(np.float32), dy.astype(np.float32), op),
+                     ("f16 dw filbk", shape))
+
+
 @pytest.mark.parametrize("size,ch,stride", MOBILENET)
 def test_f16_depthwise_forward(size, ch, stride):
     p = ops.depthwise_params(2, size, size, ch, 1, 3, stride, True)
