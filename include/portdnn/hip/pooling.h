@@ -108,10 +108,11 @@ SNNStatus launch(typename Backend::template pointer_type<T const> input,
       code = snn_hip_pooling_forward_f16(
           input, output, &c, internal::OpCode<PoolType>::value, stream);
     }
-  } else {
-    static_assert(std::is_same<T, float>::value,
-                  "pooling gradients are provided for float");
+  } else if constexpr (std::is_same<T, float>::value) {
     code = snn_hip_pooling_avg_grad_f32(input, output, &c, stream);
+  } else {
+    static_assert(sizeof(T) == 2, "supported data types: float and half");
+    code = snn_hip_pooling_avg_grad_f16(input, output, &c, stream);
   }
   return hip::detail::finish(code, stream);
 }
@@ -127,16 +128,23 @@ SNNStatus launch(typename Backend::template pointer_type<T const> input_data,
                  typename Backend::template pointer_type<T> output_backprop,
                  PoolingParams const& pp, Backend& backend,
                  const std::vector<hip::Event>& events = {}) {
-  static_assert(std::is_same<T, float>::value,
-                "pooling gradients are provided for float");
   const snn_hip_pooling_params c = internal::to_c(pp);
   hipStream_t stream = backend.get_stream();
   hip::detail::wait_for(stream, events);
-  return hip::detail::finish(
-      snn_hip_pooling_max_grad_f32(input_data, output_data, input_backprop,
-                                   output_backprop, &c,
-                                   internal::OpCode<PoolType>::value, stream),
-      stream);
+  int code;
+  if constexpr (std::is_same<T, float>::value) {
+    code = snn_hip_pooling_max_grad_f32(input_data, output_data,
+                                        input_backprop, output_backprop, &c,
+                                        internal::OpCode<PoolType>::value,
+                                        stream);
+  } else {
+    static_assert(sizeof(T) == 2, "supported data types: float and half");
+    code = snn_hip_pooling_max_grad_f16(input_data, output_data,
+                                        input_backprop, output_backprop, &c,
+                                        internal::OpCode<PoolType>::value,
+                                        stream);
+  }
+  return hip::detail::finish(code, stream);
 }
 
 }  // namespace pooling

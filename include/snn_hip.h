@@ -271,6 +271,14 @@ SNN_HIP_API int snn_hip_pooling_max_grad_f32(
 SNN_HIP_API int snn_hip_pooling_avg_grad_f32(
     const float* input_backprop, float* output_backprop,
     const snn_hip_pooling_params* params, void* stream);
+/* The two gradients on half-precision tensors (same operands). */
+SNN_HIP_API int snn_hip_pooling_max_grad_f16(
+    const void* input_data, const void* output_data,
+    const void* input_backprop, void* output_backprop,
+    const snn_hip_pooling_params* params, int op, void* stream);
+SNN_HIP_API int snn_hip_pooling_avg_grad_f16(
+    const void* input_backprop, void* output_backprop,
+    const snn_hip_pooling_params* params, void* stream);
 
 /* ---- matmul ----------------------------------------------------------------
  * Stand-in for sycldnn::matmul::internal::launch (src/matmul/launch.cc) as the

@@ -134,6 +134,8 @@ SIGNATURES = {
     "snn_hip_pooling_forward_f16": [_P, _P, _P, _I, _P],
     "snn_hip_pooling_max_grad_f32": [_P, _P, _P, _P, _P, _I, _P],
     "snn_hip_pooling_avg_grad_f32": [_P, _P, _P, _P],
+    "snn_hip_pooling_max_grad_f16": [_P, _P, _P, _P, _P, _I, _P],
+    "snn_hip_pooling_avg_grad_f16": [_P, _P, _P, _P],
     "snn_hip_matmul_f32": [_P, _P, _P, _I, _I, _I, _I, _I, _I,
                            ctypes.c_float, _P],
     "snn_hip_scale_blend_f32": [_P, _P, ctypes.c_float, ctypes.c_float, _SZ,

@@ -358,9 +358,16 @@ template <>
 struct GradVec<1> {
   __device__ static void load(const float* p, float (&v)[1]) { v[0] = *p; }
   __device__ static void store(float* p, const float (&v)[1]) { *p = v[0]; }
+  __device__ static void load(const _Float16* p, float (&v)[1]) {
+    v[0] = static_cast<float>(*p);
+  }
+  __device__ static void store(_Float16* p, const float (&v)[1]) {
+    *p = static_cast<_Float16>(v[0]);
+  }
 };
 template <>
 struct GradVec<4> {
+  typedef _Float16 half4 __attribute__((ext_vector_type(4)));
   __device__ static void load(const float* p, float (&v)[4]) {
     const float4 t = *reinterpret_cast<const float4*>(p);
     v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
@@ -368,15 +375,25 @@ struct GradVec<4> {
   __device__ static void store(float* p, const float (&v)[4]) {
     *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
   }
+  __device__ static void load(const _Float16* p, float (&v)[4]) {
+    const half4 t = *reinterpret_cast<const half4*>(p);
+    v[0] = static_cast<float>(t.x); v[1] = static_cast<float>(t.y);
+    v[2] = static_cast<float>(t.z); v[3] = static_cast<float>(t.w);
+  }
+  __device__ static void store(_Float16* p, const float (&v)[4]) {
+    half4 t;
+    t.x = static_cast<_Float16>(v[0]); t.y = static_cast<_Float16>(v[1]);
+    t.z = static_cast<_Float16>(v[2]); t.w = static_cast<_Float16>(v[3]);
+    *reinterpret_cast<half4*>(p) = t;
+  }
 };
 
 // VEC channels per lane (4 when the channel count and the pointers allow
 // 16-byte accesses).
-template <int VEC>
+template <int VEC, typename T = float>
 __global__ void __launch_bounds__(256)
-    pool_max_grad_kernel(const float* __restrict__ in,
-                         const float* __restrict__ out,
-                         const float* __restrict__ dy, float* __restrict__ dx,
+    pool_max_grad_kernel(const T* __restrict__ in, const T* __restrict__ out,
+                         const T* __restrict__ dy, T* __restrict__ dx,
                          snn_hip_pooling_params p, bool nan_mode, size_t n_vec) {
   const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (idx >= n_vec) return;
@@ -390,8 +407,7 @@ __global__ void __launch_bounds__(256)
   const int n = static_cast<int>(pix / p.in_rows);
   float mine[VEC];
   GradVec<VEC>::load(in + idx * VEC, mine);
-  const float* in_n =
-      in + static_cast<size_t>(n) * p.in_rows * p.in_cols * C + ch;
+  const T* in_n = in + static_cast<size_t>(n) * p.in_rows * p.in_cols * C + ch;
   const size_t out_base =
       static_cast<size_t>(n) * p.out_rows * p.out_cols * C + ch;
   // outputs whose (unclipped) window contains y / x
@@ -458,9 +474,9 @@ __global__ void __launch_bounds__(256)
 
 // Average gradient: every covering output contributes dY / clipped window
 // size (src/pooling/kernels.h:291-414).
-template <int VEC>
+template <int VEC, typename T = float>
 __global__ void __launch_bounds__(256)
-    pool_avg_grad_kernel(const float* __restrict__ dy, float* __restrict__ dx,
+    pool_avg_grad_kernel(const T* __restrict__ dy, T* __restrict__ dx,
                          snn_hip_pooling_params p, size_t n_vec) {
   const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (idx >= n_vec) return;
@@ -1109,6 +1125,67 @@ int launch_pooling_avg_grad(const float* input_backprop,
     }
   } else {
     hipLaunchKernelGGL(pool_avg_grad_kernel<1>,
+                       dim3(static_cast<unsigned>(ceil_div(n_in, size_t{kBlock}))),
+                       dim3(kBlock), 0, stream, input_backprop,
+                       output_backprop, p, n_in);
+  }
+  SNN_HIP_CHECK_LAUNCH();
+  return SNN_HIP_OK;
+}
+
+// Half-precision gradients (fp32 arithmetic inside a lane): the
+// one-lane-per-element kernels, four channels per lane when the channel count
+// and the pointers allow 8-byte accesses.
+static inline bool grad_aligned8(const void* ptr) {
+  return (reinterpret_cast<uintptr_t>(ptr) & 7u) == 0;
+}
+
+int launch_pooling_max_grad_f16(const _Float16* input_data,
+                                const _Float16* output_data,
+                                const _Float16* input_backprop,
+                                _Float16* output_backprop,
+                                const snn_hip_pooling_params& p, int op,
+                                hipStream_t stream) {
+  KernelTimer timer(stream);
+  constexpr int kBlock = 256;
+  const size_t n_in =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
+  const bool nan_mode = op == SNN_HIP_POOL_MAX_WITH_NAN;
+  if (p.channels % 4 == 0 && grad_aligned8(input_data) &&
+      grad_aligned8(output_data) && grad_aligned8(input_backprop) &&
+      grad_aligned8(output_backprop)) {
+    const size_t n_vec = n_in / 4;
+    hipLaunchKernelGGL((pool_max_grad_kernel<4, _Float16>),
+                       dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{kBlock}))),
+                       dim3(kBlock), 0, stream, input_data, output_data,
+                       input_backprop, output_backprop, p, nan_mode, n_vec);
+  } else {
+    hipLaunchKernelGGL((pool_max_grad_kernel<1, _Float16>),
+                       dim3(static_cast<unsigned>(ceil_div(n_in, size_t{kBlock}))),
+                       dim3(kBlock), 0, stream, input_data, output_data,
+                       input_backprop, output_backprop, p, nan_mode, n_in);
+  }
+  SNN_HIP_CHECK_LAUNCH();
+  return SNN_HIP_OK;
+}
+
+int launch_pooling_avg_grad_f16(const _Float16* input_backprop,
+                                _Float16* output_backprop,
+                                const snn_hip_pooling_params& p,
+                                hipStream_t stream) {
+  KernelTimer timer(stream);
+  constexpr int kBlock = 256;
+  const size_t n_in =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
+  if (p.channels % 4 == 0 && grad_aligned8(input_backprop) &&
+      grad_aligned8(output_backprop)) {
+    const size_t n_vec = n_in / 4;
+    hipLaunchKernelGGL((pool_avg_grad_kernel<4, _Float16>),
+                       dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{kBlock}))),
+                       dim3(kBlock), 0, stream, input_backprop,
+                       output_backprop, p, n_vec);
+  } else {
+    hipLaunchKernelGGL((pool_avg_grad_kernel<1, _Float16>),
                        dim3(static_cast<unsigned>(ceil_div(n_in, size_t{kBlock}))),
                        dim3(kBlock), 0, stream, input_backprop,
                        output_backprop, p, n_in);

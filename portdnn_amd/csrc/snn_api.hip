@@ -743,6 +743,40 @@ int snn_hip_pooling_avg_grad_f32(const float* input_backprop,
                                  as_stream(stream));
 }
 
+int snn_hip_pooling_max_grad_f16(const void* input_data,
+                                 const void* output_data,
+                                 const void* input_backprop,
+                                 void* output_backprop,
+                                 const snn_hip_pooling_params* params, int op,
+                                 void* stream) {
+  const int v = pooling_check(params, false);
+  if (v != SNN_HIP_OK) return v;
+  if (input_data == nullptr || output_data == nullptr ||
+      input_backprop == nullptr || output_backprop == nullptr)
+    return SNN_HIP_INVALID_PARAMETER;
+  if (op != SNN_HIP_POOL_MAX && op != SNN_HIP_POOL_MAX_WITH_NAN)
+    return SNN_HIP_INVALID_PARAMETER;
+  return launch_pooling_max_grad_f16(
+      static_cast<const _Float16*>(input_data),
+      static_cast<const _Float16*>(output_data),
+      static_cast<const _Float16*>(input_backprop),
+      static_cast<_Float16*>(output_backprop), *params, op,
+      as_stream(stream));
+}
+
+int snn_hip_pooling_avg_grad_f16(const void* input_backprop,
+                                 void* output_backprop,
+                                 const snn_hip_pooling_params* params,
+                                 void* stream) {
+  const int v = pooling_check(params, false);
+  if (v != SNN_HIP_OK) return v;
+  if (input_backprop == nullptr || output_backprop == nullptr)
+    return SNN_HIP_INVALID_PARAMETER;
+  return launch_pooling_avg_grad_f16(
+      static_cast<const _Float16*>(input_backprop),
+      static_cast<_Float16*>(output_backprop), *params, as_stream(stream));
+}
+
 int snn_hip_matmul_f32(const float* lhs, const float* rhs, float* output,
                        int batches, int m, int k, int n, int transpose_lhs,
                        int transpose_rhs, float beta, void* stream) {

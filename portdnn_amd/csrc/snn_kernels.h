@@ -119,6 +119,16 @@ int launch_pooling_avg_grad(const float* input_backprop,
                             float* output_backprop,
                             const snn_hip_pooling_params& p,
                             hipStream_t stream);
+int launch_pooling_max_grad_f16(const _Float16* input_data,
+                                const _Float16* output_data,
+                                const _Float16* input_backprop,
+                                _Float16* output_backprop,
+                                const snn_hip_pooling_params& p, int op,
+                                hipStream_t stream);
+int launch_pooling_avg_grad_f16(const _Float16* input_backprop,
+                                _Float16* output_backprop,
+                                const snn_hip_pooling_params& p,
+                                hipStream_t stream);
 
 // Batched row-major GEMM on MFMA (matmul.hip).
 int launch_matmul_f32(const float* lhs, const float* rhs, float* output,

@@ -197,7 +197,9 @@ def pooling_forward(inp, p, op, out=None):
 def pooling_max_grad(inp, out, dy, p, op=POOL_OP.MAX, dx=None):
     if dx is None:
         dx = torch.empty_like(inp)
-    capi.check(capi.lib().snn_hip_pooling_max_grad_f32(
+    name = ("snn_hip_pooling_max_grad_f32" if inp.dtype == torch.float32 else
+            "snn_hip_pooling_max_grad_f16")
+    capi.check(getattr(capi.lib(), name)(
         _ptr(inp), _ptr(out), _ptr(dy), _ptr(dx), ctypes.byref(p), op,
         _stream()))
     return dx
@@ -207,7 +209,9 @@ def pooling_avg_grad(dy, p, dx=None):
     if dx is None:
         dx = torch.empty(p.batch * p.in_rows * p.in_cols * p.channels,
                          dtype=dy.dtype, device=dy.device)
-    capi.check(capi.lib().snn_hip_pooling_avg_grad_f32(
+    name = ("snn_hip_pooling_avg_grad_f32" if dy.dtype == torch.float32 else
+            "snn_hip_pooling_avg_grad_f16")
+    capi.check(getattr(capi.lib(), name)(
         _ptr(dy), _ptr(dx), ctypes.byref(p), _stream()))
     return dx
 

@@ -517,6 +517,33 @@ def test_maxpool_nan_rules():
                                                         nan_mode))
 
 
+@pytest.mark.parametrize("shape", [(2, 13, 11, 8, 3, 2, True),
+                                   (1, 12, 12, 5, 2, 2, False),
+                                   (2, 9, 9, 16, 3, 1, True)])
+def test_f16_pooling_gradients(shape):
+    """Half-precision pooling gradients: the maximum is exact in half, so the
+    max gradient must equal the oracle on the same half values bit for bit;
+    the average gradient within the half tolerance."""
+    n, h, w_, c, win, st, same = shape
+    p = ops.pool_params(n, h, w_, c, win, st, same)
+    op = oracle_params(p, 0)
+    rng = np.random.default_rng(1400 + h + c)
+    x = rng.integers(-3, 4, n * h * w_ * c).astype(np.float16)
+    y = ops.pooling_forward(dev(x, torch.float16), p, POOL_OP.MAX)
+    ref_y = oracle.pool_max_forward(x.astype(np.float32), op)
+    assert np.array_equal(y.float().cpu().numpy(), ref_y)
+    dy = rng.integers(1, 9, ref_y.size).astype(np.float16)
+    got = ops.pooling_max_grad(dev(x, torch.float16), y,
+                               dev(dy, torch.float16), p)
+    assert np.array_equal(got.float().cpu().numpy(),
+                          oracle.pool_max_grad(x.astype(np.float32), ref_y,
+                                               dy.astype(np.float32), op))
+    got = ops.pooling_avg_grad(dev(dy, torch.float16), p)
+    assert_close_f16(got.float().cpu().numpy(),
+                     oracle.pool_avg_grad(dy.astype(np.float32), op),
+                     ("f16 avg grad", shape))
+
+
 # ---- matmul ------------------------------------------------------------------
 
 @pytest.mark.parametrize("trans_a", [False, True])
