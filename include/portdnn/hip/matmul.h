@@ -35,17 +35,22 @@ SNNStatus launch(typename Backend::template pointer_type<T const> lhs,
                  typename Backend::template pointer_type<T> output,
                  MatmulParams const& params, Backend& backend,
                  const std::vector<hip::Event>& events = {}) {
-  static_assert(std::is_same<T, float>::value,
-                "matmul::launch is provided for float");
   hipStream_t stream = backend.get_stream();
   if (params.batch_type != sycldnn::BatchFormat::STRIDED)
     return hip::detail::finish(SNN_HIP_INVALID_ALGORITHM, stream);
   hip::detail::wait_for(stream, events);
-  return hip::detail::finish(
-      snn_hip_matmul_f32(lhs, rhs, output, params.batches, params.m, params.k,
-                         params.n, TransposeLHS, TransposeRHS, params.beta,
-                         stream),
-      stream);
+  int code;
+  if constexpr (std::is_same<T, float>::value) {
+    code = snn_hip_matmul_f32(lhs, rhs, output, params.batches, params.m,
+                              params.k, params.n, TransposeLHS, TransposeRHS,
+                              params.beta, stream);
+  } else {
+    static_assert(sizeof(T) == 2, "supported data types: float and half");
+    code = snn_hip_matmul_f16(lhs, rhs, output, params.batches, params.m,
+                              params.k, params.n, TransposeLHS, TransposeRHS,
+                              params.beta, stream);
+  }
+  return hip::detail::finish(code, stream);
 }
 
 }  // namespace matmul

@@ -289,6 +289,11 @@ SNN_HIP_API int snn_hip_matmul_f32(const float* lhs, const float* rhs,
                                    float* output, int batches, int m, int k,
                                    int n, int transpose_lhs, int transpose_rhs,
                                    float beta, void* stream);
+/* The same on half-precision matrices (products and sums in fp32). */
+SNN_HIP_API int snn_hip_matmul_f16(const void* lhs, const void* rhs,
+                                   void* output, int batches, int m, int k,
+                                   int n, int transpose_lhs, int transpose_rhs,
+                                   float beta, void* stream);
 
 /* ---- convolution with bias and activation ---------------------------------
  * No single counterpart in the reference, which runs three launches for this

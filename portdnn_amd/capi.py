@@ -138,6 +138,8 @@ SIGNATURES = {
     "snn_hip_pooling_avg_grad_f16": [_P, _P, _P, _P],
     "snn_hip_matmul_f32": [_P, _P, _P, _I, _I, _I, _I, _I, _I,
                            ctypes.c_float, _P],
+    "snn_hip_matmul_f16": [_P, _P, _P, _I, _I, _I, _I, _I, _I,
+                           ctypes.c_float, _P],
     "snn_hip_scale_blend_f32": [_P, _P, ctypes.c_float, ctypes.c_float, _SZ,
                                 _P],
     "snn_hip_pointwise_forward_f32": [_P, _P, _SZ, _I, _P],

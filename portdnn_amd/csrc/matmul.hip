@@ -14,11 +14,11 @@ namespace {
 constexpr int kTile = 64;
 constexpr int kTileK = 16;
 
-template <bool TransA, bool TransB>
+// T = float or _Float16 (products and sums in fp32 either way).
+template <bool TransA, bool TransB, typename T = float>
 __global__ void __launch_bounds__(256)
-    matmul_general_kernel(const float* __restrict__ a,
-                          const float* __restrict__ b, float* __restrict__ c,
-                          int m, int k, int n, float beta) {
+    matmul_general_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                          T* __restrict__ c, int m, int k, int n, float beta) {
   __shared__ float sa[kTileK][kTile + 4];  // [kk][row]
   __shared__ float sb[kTileK][kTile + 4];  // [kk][col]
   const int batch = blockIdx.z;
@@ -44,8 +44,8 @@ __global__ void __launch_bounds__(256)
       const int gr = row0 + r, gk = k0 + kk;
       float v = 0.f;
       if (gr < m && gk < k) {
-        v = TransA ? a[static_cast<size_t>(gk) * m + gr]
-                   : a[static_cast<size_t>(gr) * k + gk];
+        v = static_cast<float>(TransA ? a[static_cast<size_t>(gk) * m + gr]
+                                      : a[static_cast<size_t>(gr) * k + gk]);
       }
       sa[kk][r] = v;
       // B tile element (depth kk2, col cc)
@@ -60,8 +60,8 @@ __global__ void __launch_bounds__(256)
       const int gc = col0 + cc, gk2 = k0 + kk2;
       float w = 0.f;
       if (gc < n && gk2 < k) {
-        w = TransB ? b[static_cast<size_t>(gc) * k + gk2]
-                   : b[static_cast<size_t>(gk2) * n + gc];
+        w = static_cast<float>(TransB ? b[static_cast<size_t>(gc) * k + gk2]
+                                      : b[static_cast<size_t>(gk2) * n + gc]);
       }
       sb[kk2][cc] = w;
     }
@@ -89,7 +89,9 @@ __global__ void __launch_bounds__(256)
       const int gc = col0 + tx * 4 + j;
       if (gc >= n) continue;
       const size_t o = static_cast<size_t>(gr) * n + gc;
-      c[o] = (beta == 0.f) ? acc[i][j] : fmaf(beta, c[o], acc[i][j]);
+      c[o] = static_cast<T>(
+          (beta == 0.f) ? acc[i][j]
+                        : fmaf(beta, static_cast<float>(c[o]), acc[i][j]));
     }
   }
 }
@@ -140,6 +142,64 @@ int launch_matmul_f32(const float* lhs, const float* rhs, float* output,
     else
       hipLaunchKernelGGL((matmul_general_kernel<false, false>), grid, block, 0,
                          stream, lhs, rhs, output, m, k, n, beta);
+  }
+  SNN_HIP_CHECK_LAUNCH();
+  return SNN_HIP_OK;
+}
+
+int launch_matmul_f16(const _Float16* lhs, const _Float16* rhs,
+                      _Float16* output, int batches, int m, int k, int n,
+                      bool transpose_lhs, bool transpose_rhs, float beta,
+                      hipStream_t stream) {
+  // Matrix-core path: one problem, A not transposed, beta == 0 and operands
+  // the half-precision 1x1 convolution kernels take.  A [m x k] * B [k x n]
+  // is the forward 1x1 convolution of m pixels with k channels and n
+  // features (B is its HWCF filter); A * B^T with B stored [n x k] is the
+  // input gradient of the 1x1 convolution with n channels and k features.
+  const bool aligned =
+      ((reinterpret_cast<uintptr_t>(lhs) | reinterpret_cast<uintptr_t>(rhs) |
+        reinterpret_cast<uintptr_t>(output)) & 15u) == 0;
+  if (!transpose_lhs && batches == 1 && beta == 0.f && aligned && m >= 32) {
+    snn_hip_conv2d_params p = {};
+    p.batch = 1;
+    p.in_rows = p.out_rows = 1;
+    p.in_cols = p.out_cols = m;
+    p.window_rows = p.window_cols = 1;
+    p.stride_rows = p.stride_cols = 1;
+    p.dilation_rows = p.dilation_cols = 1;
+    p.groups = 1;
+    if (!transpose_rhs) {
+      p.channels = k;
+      p.features = n;
+      if (conv2d_igemm_f16_supports(p))
+        return launch_conv2d_igemm_f16(lhs, rhs, output, p, nullptr, 0,
+                                       stream);
+    } else {
+      p.channels = n;
+      p.features = k;
+      if (conv2d_input_backprop_f16_supports(p))
+        return launch_conv2d_input_backprop_f16(lhs, rhs, output, p, nullptr,
+                                                0, stream);
+    }
+  }
+  const dim3 grid(static_cast<unsigned>(ceil_div(m, kTile)),
+                  static_cast<unsigned>(ceil_div(n, kTile)),
+                  static_cast<unsigned>(batches));
+  const dim3 block(256);
+  if (transpose_lhs) {
+    if (transpose_rhs)
+      hipLaunchKernelGGL((matmul_general_kernel<true, true, _Float16>), grid,
+                         block, 0, stream, lhs, rhs, output, m, k, n, beta);
+    else
+      hipLaunchKernelGGL((matmul_general_kernel<true, false, _Float16>), grid,
+                         block, 0, stream, lhs, rhs, output, m, k, n, beta);
+  } else {
+    if (transpose_rhs)
+      hipLaunchKernelGGL((matmul_general_kernel<false, true, _Float16>), grid,
+                         block, 0, stream, lhs, rhs, output, m, k, n, beta);
+    else
+      hipLaunchKernelGGL((matmul_general_kernel<false, false, _Float16>), grid,
+                         block, 0, stream, lhs, rhs, output, m, k, n, beta);
   }
   SNN_HIP_CHECK_LAUNCH();
   return SNN_HIP_OK;

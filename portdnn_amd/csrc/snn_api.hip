@@ -794,6 +794,24 @@ int snn_hip_matmul_f32(const float* lhs, const float* rhs, float* output,
                            as_stream(stream));
 }
 
+int snn_hip_matmul_f16(const void* lhs, const void* rhs, void* output,
+                       int batches, int m, int k, int n, int transpose_lhs,
+                       int transpose_rhs, float beta, void* stream) {
+  if (lhs == nullptr || rhs == nullptr || output == nullptr)
+    return SNN_HIP_INVALID_PARAMETER;
+  if (batches <= 0 || m <= 0 || k <= 0 || n <= 0)
+    return SNN_HIP_INVALID_PARAMETER;
+  if (!fits_int32(static_cast<size_t>(batches) * m * k) ||
+      !fits_int32(static_cast<size_t>(batches) * k * n) ||
+      !fits_int32(static_cast<size_t>(batches) * m * n))
+    return SNN_HIP_INDEX_EXCEEDED;
+  return launch_matmul_f16(static_cast<const _Float16*>(lhs),
+                           static_cast<const _Float16*>(rhs),
+                           static_cast<_Float16*>(output), batches, m, k, n,
+                           transpose_lhs != 0, transpose_rhs != 0, beta,
+                           as_stream(stream));
+}
+
 int snn_hip_conv2d_forward_bias_act_f32(
     const float* input, const float* filter, const float* bias, float* output,
     const snn_hip_conv2d_params* params, int algorithm, int activation,

@@ -134,6 +134,10 @@ int launch_pooling_avg_grad_f16(const _Float16* input_backprop,
 int launch_matmul_f32(const float* lhs, const float* rhs, float* output,
                       int batches, int m, int k, int n, bool transpose_lhs,
                       bool transpose_rhs, float beta, hipStream_t stream);
+int launch_matmul_f16(const _Float16* lhs, const _Float16* rhs,
+                      _Float16* output, int batches, int m, int k, int n,
+                      bool transpose_lhs, bool transpose_rhs, float beta,
+                      hipStream_t stream);
 
 // Element-wise operators (elementwise.hip).  `op` is a snn_hip_pointwise_op
 // or snn_hip_binary_op; operands may alias the output element for element.

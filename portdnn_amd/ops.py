@@ -221,7 +221,9 @@ def matmul(a, b, batches, m, k, n, trans_a=False, trans_b=False, beta=0.0,
     assert a.numel() == batches * m * k and b.numel() == batches * k * n
     if out is None:
         out = torch.zeros(batches * m * n, dtype=a.dtype, device=a.device)
-    capi.check(capi.lib().snn_hip_matmul_f32(
+    name = ("snn_hip_matmul_f32" if a.dtype == torch.float32 else
+            "snn_hip_matmul_f16")
+    capi.check(getattr(capi.lib(), name)(
         _ptr(a), _ptr(b), _ptr(out), batches, m, k, n, int(trans_a),
         int(trans_b), float(beta), _stream()))
     return out

@@ -603,6 +603,29 @@ def test_many_tiles_per_work_group_epilogue_and_accumulate():
                                0.0), "matmul slice")
 
 
+@pytest.mark.parametrize("shape", [(1, 256, 128, 192), (1, 100, 64, 64),
+                                   (3, 33, 20, 17), (1, 2048, 256, 512)])
+@pytest.mark.parametrize("trans_a", [False, True])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_matmul_f16(trans_a, trans_b, shape):
+    """Half-precision matmul (fp32 accumulation): matrix-core shapes and the
+    general kernel, against the oracle on the same half-rounded operands."""
+    b_, m, k, n = shape
+    rng = np.random.default_rng(sum(shape) + 7)
+    a = uniform(rng, b_ * m * k).astype(np.float16)
+    b = uniform(rng, b_ * k * n).astype(np.float16)
+    c0 = uniform(rng, b_ * m * n).astype(np.float16)
+    for beta in (0.0, 1.0):
+        ref = oracle.matmul(a.astype(np.float32), b.astype(np.float32), b_, m,
+                            k, n, trans_a, trans_b, beta,
+                            c=c0.astype(np.float32))
+        got = ops.matmul(dev(a, torch.float16), dev(b, torch.float16), b_, m,
+                         k, n, trans_a, trans_b, beta,
+                         out=dev(c0, torch.float16).clone())
+        assert_close_f16(got.float().cpu().numpy(), ref,
+                         ("matmul f16", shape, trans_a, trans_b, beta))
+
+
 # ---- f16 ---------------------------------------------------------------------
 
 def assert_close_f16(got, ref, what):
