@@ -749,6 +749,9 @@ def test_f16_conv_forward_full_batch_sampled(size, ch, feats, window):
     (2, 28, 28, 128, 512, 1, 1, 1, False),  # 1x1, 128 x 128 tiles
     (2, 17, 9, 128, 64, 3, 3, 2, True),     # stride 2: direct kernel
     (2, 8, 8, 24, 40, 3, 3, 1, True),       # few channels: direct kernel
+    (2, 9, 10, 64, 64, 2, 2, 1, True),      # even window: padding 0 before, 1 after
+    (2, 12, 9, 64, 128, 4, 4, 1, True),     # even window: padding 1 before, 2 after
+    (2, 10, 10, 64, 64, 2, 4, 1, False),    # VALID, rectangular even window
 ])
 def test_f16_conv_input_backprop(shape):
     """Half-precision input gradient (fp32 accumulation) against the oracle in
