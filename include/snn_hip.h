@@ -239,6 +239,21 @@ SNN_HIP_API int snn_hip_depthwise_conv2d_input_backprop_f32(
 SNN_HIP_API int snn_hip_depthwise_conv2d_filter_backprop_f32(
     const float* input, const float* filter, float* output,
     const snn_hip_depthwise_params* params, void* stream);
+/* The fp32 filter gradient for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  Same operands and result as
+ * snn_hip_depthwise_conv2d_filter_backprop_f32, whose large-input path keeps
+ * the work-groups' partial filters in a stream-ordered temporary; here they
+ * live in a 9 MiB device array inside the library (held by every GPU the
+ * library runs on until the process ends), sized for the largest plan that
+ * path makes, so no hipMalloc / hipFree in any form is called.  A shape whose
+ * partial filters would not fit is rejected with SNN_HIP_INVALID_PARAMETER
+ * and a message in snn_hip_last_error().  All calls on one GPU share that
+ * array: calls that overlap on one GPU (different streams or threads) race;
+ * stream-ordered calls are safe.  The stream's device must be current. */
+SNN_HIP_API int snn_hip_depthwise_conv2d_filter_backprop_noalloc_f32(
+    const float* input, const float* filter, float* output,
+    const snn_hip_depthwise_params* params, void* stream);
 SNN_HIP_API int snn_hip_depthwise_conv2d_forward_f16(
     const void* input, const void* filter, void* output,
     const snn_hip_depthwise_params* params, void* stream);

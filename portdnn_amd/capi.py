@@ -127,6 +127,8 @@ SIGNATURES = {
     "snn_hip_depthwise_conv2d_forward_f32": [_P, _P, _P, _P, _P],
     "snn_hip_depthwise_conv2d_input_backprop_f32": [_P, _P, _P, _P, _P],
     "snn_hip_depthwise_conv2d_filter_backprop_f32": [_P, _P, _P, _P, _P],
+    "snn_hip_depthwise_conv2d_filter_backprop_noalloc_f32": [_P, _P, _P, _P,
+                                                             _P],
     "snn_hip_depthwise_conv2d_forward_f16": [_P, _P, _P, _P, _P],
     "snn_hip_depthwise_conv2d_input_backprop_f16": [_P, _P, _P, _P, _P],
     "snn_hip_depthwise_conv2d_filter_backprop_f16": [_P, _P, _P, _P, _P],

@@ -11,6 +11,8 @@
 // and the window taps of neighbouring lanes/pixels are served from L1/L2.
 // Everything else goes through the scalar kernel.
 #include <cstdlib>
+#include <mutex>
+#include <string>
 #include <type_traits>
 
 #include "gemm_tile.h"
@@ -881,22 +883,58 @@ void launch_dw_strip(const T* input, const T* filter, T* output,
 
 }  // namespace
 
+// Device memory for the entry point that allocates nothing
+// (snn_hip_depthwise_conv2d_filter_backprop_noalloc_f32): the work-groups'
+// partial filters.  The strip kernel runs at most 2048 / grid_y groups along
+// x, each writing 9 * C floats with C <= 128 * grid_y, so 2048 * 1152 floats
+// (9 MiB) hold the partial filters of every shape that kernel takes.  Every
+// device the library runs on holds its own copy until the process ends.
+constexpr size_t kDwScratchElems = size_t{2048} * 1152;
+static __device__ __align__(256) float scratch[kDwScratchElems];
+
+namespace {
+
+// The address of `scratch` on the current device, looked up once per device.
+// In host code the array's name is only a handle for hipGetSymbolAddress;
+// kernels and copies must be given the pointer this returns.
+int dw_scratch_on_current_device(float** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mutex;
+  static float* address[kMaxDevices] = {};
+  int device = 0;
+  SNN_HIP_TRY(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices)
+    return report_error(SNN_HIP_INVALID_PARAMETER,
+                        "device ordinal beyond the per-device scratch table");
+  std::lock_guard<std::mutex> lock(mutex);
+  if (address[device] == nullptr) {
+    void* p = nullptr;
+    SNN_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    address[device] = static_cast<float*>(p);
+  }
+  *out = address[device];
+  return SNN_HIP_OK;
+}
+
+}  // namespace
+
 // Picks the strip height (4 or 8 output rows, whichever wastes fewer rows of
 // the last row block; 8 on a tie) and deals the strips to the work-groups.
-// Large problems use about 2048 work-groups whose partial filters go to a
-// stream-ordered temporary that a second kernel adds up; small ones (or no
-// temporary) use up to 1024 work-groups that add into the zero-filled dF
-// with float atomics, which serialise per address.
-static void launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
-                                  const snn_hip_depthwise_params& p, int cvw,
-                                  int grid_y, hipStream_t stream) {
+// Large problems use about 2048 work-groups whose partial filters go to
+// `static_scratch` when the caller brings it (kDwScratchElems floats), else to
+// a stream-ordered temporary, and a second kernel adds them up; small ones (or
+// a failed allocation) use up to 1024 work-groups that add into the
+// zero-filled dF with float atomics, which serialise per address.
+static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
+                                 const snn_hip_depthwise_params& p, int cvw,
+                                 int grid_y, hipStream_t stream,
+                                 float* static_scratch) {
   const int n_pl = kDwFilbkThreads / cvw;
   const int th =
       ceil_div(p.out_rows, 8) * 8 <= ceil_div(p.out_rows, 4) * 4 ? 8 : 4;
   const int n_rb = ceil_div(p.out_rows, th);
   const int n_strips = p.batch * n_rb * p.out_cols;
   const int dw_elems = 9 * p.channels;
-  static const char* tune = getenv("SNN_HIP_DW_FILBK_GROUPS");
   auto plan = [&](int target_groups, int* spg) {
     *spg = max(n_pl, ceil_div(n_strips, max(1, target_groups / grid_y)));
     *spg = ceil_div(*spg, n_pl) * n_pl;
@@ -907,11 +945,24 @@ static void launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
   constexpr size_t kTwoStageBytes = size_t{32} << 20;
   int spg = 0, grid_x = 0;
   float* part = nullptr;
+  bool temporary = false;
   if (in_bytes >= kTwoStageBytes) {
-    grid_x = plan(tune != nullptr ? max(1, atoi(tune)) : 2048, &spg);
-    if (hipMallocAsync(reinterpret_cast<void**>(&part),
-                       static_cast<size_t>(grid_x) * dw_elems * sizeof(float),
-                       stream) != hipSuccess) {
+    grid_x = plan(2048, &spg);
+    const size_t part_elems = static_cast<size_t>(grid_x) * dw_elems;
+    if (static_scratch != nullptr) {
+      if (part_elems > kDwScratchElems)
+        return report_error(
+            SNN_HIP_INVALID_PARAMETER,
+            "depthwise filter backprop without allocation: the partial "
+            "filters need " + std::to_string(part_elems * sizeof(float)) +
+            " bytes, the library's scratch array holds " +
+            std::to_string(kDwScratchElems * sizeof(float)));
+      part = static_scratch;
+    } else if (hipMallocAsync(reinterpret_cast<void**>(&part),
+                              part_elems * sizeof(float),
+                              stream) == hipSuccess) {
+      temporary = true;
+    } else {
       (void)hipGetLastError();
       part = nullptr;
     }
@@ -945,13 +996,15 @@ static void launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
         dim3(static_cast<unsigned>(ceil_div(n_vec, 64)), kDwFilbkReduceY),
         dim3(256), 0, stream, reinterpret_cast<const float4*>(part), dw, n_vec,
         grid_x);
-    (void)hipFreeAsync(part, stream);
+    if (temporary) (void)hipFreeAsync(part, stream);
   }
+  return SNN_HIP_OK;
 }
 
 template <typename T>
 int launch_depthwise(int direction, const T* input, const T* filter, T* output,
-                     const snn_hip_depthwise_params& p, hipStream_t stream) {
+                     const snn_hip_depthwise_params& p, hipStream_t stream,
+                     float* static_scratch) {
   KernelTimer timer(stream);
   constexpr int kBlock = 256;
   const size_t CM = static_cast<size_t>(p.channels) * p.channel_multiplier;
@@ -1067,7 +1120,9 @@ int launch_depthwise(int direction, const T* input, const T* filter, T* output,
             (p.stride_rows == 1 || p.stride_rows == 2) &&
             getenv("SNN_HIP_DW_FILBK_PIXEL") == nullptr;
         if (strip_ok) {
-          launch_dw_filbk_strip(input, filter, output, p, cvw, grid_y, stream);
+          const int status = launch_dw_filbk_strip(
+              input, filter, output, p, cvw, grid_y, stream, static_scratch);
+          if (status != SNN_HIP_OK) return status;
         } else {
           hipLaunchKernelGGL(dw_zero_kernel, dim3(ceil_div(dw_elems, 256)),
                              dim3(256), 0, stream, output, dw_elems);
@@ -1094,10 +1149,20 @@ int launch_depthwise(int direction, const T* input, const T* filter, T* output,
 
 template int launch_depthwise<float>(int, const float*, const float*, float*,
                                      const snn_hip_depthwise_params&,
-                                     hipStream_t);
+                                     hipStream_t, float*);
 template int launch_depthwise<_Float16>(int, const _Float16*, const _Float16*,
                                         _Float16*,
                                         const snn_hip_depthwise_params&,
-                                        hipStream_t);
+                                        hipStream_t, float*);
+
+int launch_depthwise_filter_backprop_noalloc_f32(
+    const float* input, const float* dy, float* dw,
+    const snn_hip_depthwise_params& p, hipStream_t stream) {
+  float* scratch_ptr = nullptr;
+  const int status = dw_scratch_on_current_device(&scratch_ptr);
+  if (status != SNN_HIP_OK) return status;
+  return launch_depthwise<float>(SNN_HIP_FILTER_BACKPROP, input, dy, dw, p,
+                                 stream, scratch_ptr);
+}
 
 }  // namespace snn

@@ -42,6 +42,11 @@ int report_hip_error(hipError_t err, const char* what) {
   return SNN_HIP_DEVICE_ERROR;
 }
 
+int report_error(int status, const std::string& text) {
+  g_last_error = text;
+  return status;
+}
+
 // include/portdnn/internal/conv2d/launch.h:42-97.  groups == 0 passes the
 // reference's `>= 0` check and then divides by zero there; it is rejected here.
 int validate(const snn_hip_conv2d_params& p) {
@@ -663,6 +668,24 @@ int snn_hip_depthwise_conv2d_filter_backprop_f32(
     const snn_hip_depthwise_params* params, void* stream) {
   return depthwise_dispatch<float>(SNN_HIP_FILTER_BACKPROP, input, filter,
                                    output, params, stream);
+}
+
+int snn_hip_depthwise_conv2d_filter_backprop_noalloc_f32(
+    const float* input, const float* filter, float* output,
+    const snn_hip_depthwise_params* params, void* stream) {
+  if (params == nullptr) return SNN_HIP_INVALID_PARAMETER;
+  const int v = validate(*params);
+  if (v != SNN_HIP_OK) return v;
+  if (input == nullptr || filter == nullptr || output == nullptr)
+    return SNN_HIP_INVALID_PARAMETER;
+  const snn_hip_depthwise_params& p = *params;
+  const size_t cm = static_cast<size_t>(p.channels) * p.channel_multiplier;
+  if (!fits_int32(static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                  p.channels) ||
+      !fits_int32(static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * cm))
+    return SNN_HIP_INDEX_EXCEEDED;
+  return launch_depthwise_filter_backprop_noalloc_f32(input, filter, output, p,
+                                                      as_stream(stream));
 }
 
 int snn_hip_depthwise_conv2d_forward_f16(

@@ -8,6 +8,7 @@
 #include <climits>
 #include <cstddef>
 #include <cstdint>
+#include <string>
 
 #include "snn_hip.h"
 
@@ -16,6 +17,9 @@ namespace snn {
 // Records the HIP error text for snn_hip_last_error() and returns
 // SNN_HIP_DEVICE_ERROR.
 int report_hip_error(hipError_t err, const char* what);
+
+// Records `text` for snn_hip_last_error() and returns `status`.
+int report_error(int status, const std::string& text);
 
 #define SNN_HIP_TRY(expr)                                   \
   do {                                                      \

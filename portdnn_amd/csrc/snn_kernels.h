@@ -100,10 +100,18 @@ int launch_conv2d_rowtile_f16(const _Float16* input, const _Float16* filter,
                               _Float16* packed, hipStream_t stream,
                               bool transposed_filter = false);
 
-// Depthwise convolution, all three directions (depthwise.hip).
+// Depthwise convolution, all three directions (depthwise.hip).  With
+// `static_scratch` (the library's own scratch array) the filter gradient
+// takes its partial-filter buffer from there and allocates nothing.
 template <typename T>
 int launch_depthwise(int direction, const T* input, const T* filter, T* output,
-                     const snn_hip_depthwise_params& p, hipStream_t stream);
+                     const snn_hip_depthwise_params& p, hipStream_t stream,
+                     float* static_scratch = nullptr);
+// The fp32 filter gradient with the partial filters in the library's
+// file-scope device array: no allocation of any kind.
+int launch_depthwise_filter_backprop_noalloc_f32(
+    const float* input, const float* dy, float* dw,
+    const snn_hip_depthwise_params& p, hipStream_t stream);
 
 // Pooling (pooling.hip).
 template <typename T>
