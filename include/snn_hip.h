@@ -154,7 +154,10 @@ SNN_HIP_API const char* snn_hip_last_error(void);
  * and pooling launches bracket everything they enqueue.
  * snn_hip_kernel_timing_read waits for the recorded events, returns the summed
  * kernel time in milliseconds and the number of kernels, and clears the
- * record.  Not thread safe; meant for a single benchmarking thread. */
+ * record.  Launches from several threads may record concurrently (the record
+ * is mutex-guarded and stops growing at 65536 kernels until it is read); a
+ * read waits for every recorded kernel, so call it from one thread once the
+ * timed launches have been enqueued. */
 SNN_HIP_API int snn_hip_kernel_timing_enable(int enable);
 SNN_HIP_API int snn_hip_kernel_timing_read(double* total_ms, int* kernels);
 

@@ -1086,7 +1086,7 @@ unsigned resident_groups(Kernel kernel, size_t lds_bytes) {
 
 inline unsigned persistent_grid_x(unsigned resident, unsigned n_tiles,
                                   unsigned yz) {
-  static const bool off = getenv("SNN_HIP_IGEMM_ONE_TILE") != nullptr;
+  static const bool off = SNN_TUNING_ENV("SNN_HIP_IGEMM_ONE_TILE") != nullptr;
   if (off || resident == 0) return n_tiles;
   unsigned gx = resident / max(yz, 1u);
   gx -= gx % 8u;
@@ -1223,7 +1223,7 @@ void launch_auto(const float* src, const float* wgt, float* dst,
   const int n_chunks = ceil_div(g.k_total, kBK);
   // Developer override for tuning runs: SNN_HIP_IGEMM="<tile>,<splits>" with
   // tile 0 = 128x128, 1 = 128x64, 2 = 64x64.
-  static const char* tune = getenv("SNN_HIP_IGEMM");
+  static const char* tune = SNN_TUNING_ENV("SNN_HIP_IGEMM");
   if (tune != nullptr) {
     int tile = 2, splits = 1;
     sscanf(tune, "%d,%d", &tile, &splits);

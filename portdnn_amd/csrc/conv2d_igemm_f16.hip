@@ -308,7 +308,7 @@ int launch_conv2d_igemm_f16(const _Float16* input, const _Float16* filter,
     wgt_t = static_cast<_Float16*>(ptr);
     temporary = true;
   }
-  static const bool no_rowtile = getenv("SNN_HIP_F16_IGEMM") != nullptr;
+  static const bool no_rowtile = SNN_TUNING_ENV("SNN_HIP_F16_IGEMM") != nullptr;
   if (!no_rowtile && conv2d_rowtile_f16_supports(p)) {
     const int status =
         launch_conv2d_rowtile_f16(input, filter, output, p, wgt_t, stream);

@@ -670,7 +670,7 @@ int launch_conv2d_rowtile_f16(const _Float16* input, const _Float16* filter,
                               bool transposed_filter) {
   const RowTilePlan plan = make_plan(p);
   if (plan.lds_bytes == 0) return SNN_HIP_INVALID_ALGORITHM;
-  static const bool print_plan = getenv("SNN_HIP_F16_PLAN") != nullptr;
+  static const bool print_plan = SNN_TUNING_ENV("SNN_HIP_F16_PLAN") != nullptr;
   if (print_plan)
     fprintf(stderr,
             "rowtile f16: waves %dx%d, %d pixel blocks, %d channels/tile, "

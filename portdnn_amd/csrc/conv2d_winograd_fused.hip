@@ -481,7 +481,7 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
       }
     }
   }
-  if (const char* tune = std::getenv("SNN_HIP_WINO_XCDF")) {
+  if (const char* tune = SNN_TUNING_ENV("SNN_HIP_WINO_XCDF")) {
     const int xf = std::atoi(tune);
     if (xf == 1 || xf == 2 || xf == 4 || xf == 8) {
       ug.xcd_f = xf;
@@ -503,7 +503,7 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
   if (n_units < kFewUnits)
     splits = static_cast<int>(ceil_div(kTargetGroups, n_units));
   splits = max(1, min(splits, n_chunks / kMinChunks));
-  if (const char* tune = std::getenv("SNN_HIP_WINO")) {
+  if (const char* tune = SNN_TUNING_ENV("SNN_HIP_WINO")) {
     if (tune[0] != 0) splits = max(1, min(std::atoi(tune), n_chunks));
   }
   const int per_split = ceil_div(n_chunks, splits);

@@ -842,8 +842,8 @@ void launch_dw_strip(const T* input, const T* filter, T* output,
   }
   // Developer overrides for tuning runs: SNN_HIP_DW_TH=<1|2|4|8>,
   // SNN_HIP_DW_TW=<1|2>.
-  static const char* tune_th = getenv("SNN_HIP_DW_TH");
-  static const char* tune_tw = getenv("SNN_HIP_DW_TW");
+  static const char* tune_th = SNN_TUNING_ENV("SNN_HIP_DW_TH");
+  static const char* tune_tw = SNN_TUNING_ENV("SNN_HIP_DW_TW");
   if (tune_th != nullptr && tune_th[0] != 0) th = atoi(tune_th);
   if (tune_tw != nullptr && tune_tw[0] != 0) tw = atoi(tune_tw);
   tw = tw >= 2 ? 2 : 1;
@@ -1064,7 +1064,7 @@ int launch_depthwise(int direction, const T* input, const T* filter, T* output,
       if (!wide) launch_dw_strip<T, 4, true>(input, filter, output, q, stream);
     } else if (vec_ok && p.window_rows == 3 && p.window_cols == 3 &&
                p.stride_rows == 2 && p.stride_cols == 2 && p.pad_rows <= 2 &&
-               p.pad_cols <= 2 && getenv("SNN_HIP_DW_INBK_GATHER") == nullptr) {
+               p.pad_cols <= 2 && SNN_TUNING_ENV("SNN_HIP_DW_INBK_GATHER") == nullptr) {
       // block rows / columns: padded coordinates pad .. in + pad - 1, halved
       const int n_brows = (p.in_rows + p.pad_rows - 1) / 2 - p.pad_rows / 2 + 1;
       const int n_bcols = (p.in_cols + p.pad_cols - 1) / 2 - p.pad_cols / 2 + 1;
@@ -1118,7 +1118,7 @@ int launch_depthwise(int direction, const T* input, const T* filter, T* output,
         const bool strip_ok =
             p.stride_rows == p.stride_cols &&
             (p.stride_rows == 1 || p.stride_rows == 2) &&
-            getenv("SNN_HIP_DW_FILBK_PIXEL") == nullptr;
+            SNN_TUNING_ENV("SNN_HIP_DW_FILBK_PIXEL") == nullptr;
         if (strip_ok) {
           const int status = launch_dw_filbk_strip(
               input, filter, output, p, cvw, grid_y, stream, static_scratch);

@@ -610,7 +610,7 @@ int launch_forward_op(const T* input, T* output,
     int th = 4;
     while (th > 1 && per_row * ceil_div(p.out_rows, th) < 150000) th /= 2;
     // Developer override for tuning runs: SNN_HIP_POOL_TH=<1|2|4>.
-    static const char* tune = getenv("SNN_HIP_POOL_TH");
+    static const char* tune = SNN_TUNING_ENV("SNN_HIP_POOL_TH");
     if (tune != nullptr && tune[0] != 0) th = atoi(tune);
     th = th >= 4 ? 4 : th >= 2 ? 2 : 1;
     const int n_strips = ceil_div(p.out_rows, th);
@@ -1040,7 +1040,7 @@ int launch_pooling_max_grad(const float* input_data, const float* output_data,
                       ceil_div(p.channels / 4, 16) <= 65535;
   const size_t n_out =
       static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * p.channels;
-  static const bool use_tiles = getenv("SNN_HIP_POOL_GRAD_TILES") != nullptr;
+  static const bool use_tiles = SNN_TUNING_ENV("SNN_HIP_POOL_GRAD_TILES") != nullptr;
   if (vec4 && square && p.window_rows == 3 && p.stride_rows == 2 &&
       !use_tiles && n_in * 4 < 0x7FFFFFF0u && n_out * 4 < 0x7FFFFFF0u) {
     // block rows / columns: padded coordinates pad .. in + pad - 1, halved
@@ -1103,7 +1103,7 @@ int launch_pooling_avg_grad(const float* input_backprop,
         static_cast<size_t>(p.batch) * p.in_cols * (p.channels / 4);
     int th = 8;
     while (th > 1 && per_row * ceil_div(p.in_rows, th) < 150000) th /= 2;
-    static const char* tune = getenv("SNN_HIP_POOL_GRAD_TH");
+    static const char* tune = SNN_TUNING_ENV("SNN_HIP_POOL_GRAD_TH");
     if (tune != nullptr && tune[0] != 0) th = atoi(tune);
     const int n_strips = ceil_div(p.in_rows, th >= 8 ? 8 : 4);
     const size_t n_items = per_row * n_strips;

@@ -1,7 +1,9 @@
 // The C ABI of libsnn_hip.so: parameter validation, algorithm support rules,
 // workspace sizing and dispatch to the kernel launchers.
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <utility>
 #include <vector>
@@ -14,13 +16,23 @@ namespace {
 thread_local std::string g_last_error;
 }
 
+// The opt-in kernel-timing record: the only process-wide state of the
+// library.  The switch is atomic and the list of event pairs is guarded by a
+// mutex, so launches from several threads may record concurrently; the list
+// stops growing at kMaxTimedKernels pairs until it is read.
 namespace {
-bool g_timing_enabled = false;
+std::atomic<bool> g_timing_enabled{false};
+std::mutex g_timing_mutex;
 std::vector<std::pair<hipEvent_t, hipEvent_t>> g_timed_kernels;
+constexpr size_t kMaxTimedKernels = 1u << 16;
 }  // namespace
 
 KernelTimer::KernelTimer(hipStream_t stream) : stream_(stream), stop_(nullptr) {
-  if (!g_timing_enabled) return;
+  if (!g_timing_enabled.load(std::memory_order_relaxed)) return;
+  {
+    std::lock_guard<std::mutex> lock(g_timing_mutex);
+    if (g_timed_kernels.size() >= kMaxTimedKernels) return;
+  }
   hipEvent_t start = nullptr;
   if (hipEventCreate(&start) != hipSuccess) return;
   if (hipEventCreate(&stop_) != hipSuccess) {
@@ -29,6 +41,7 @@ KernelTimer::KernelTimer(hipStream_t stream) : stream_(stream), stop_(nullptr) {
     return;
   }
   (void)hipEventRecord(start, stream_);
+  std::lock_guard<std::mutex> lock(g_timing_mutex);
   g_timed_kernels.emplace_back(start, stop_);
 }
 
@@ -238,6 +251,12 @@ void im2col_workspace(const snn_hip_conv2d_params& p, int direction,
   *recommended = static_cast<size_t>(p.batch) * in_t + filter_t;
 }
 
+// What a launch with `algorithm` needs.  Winograd forward / input backprop
+// follow the reference's F(2x2,3x3) formula (the three-stage chain uses all of
+// it, the fused kernel its transformed-filter part).  WinogradLarge runs the
+// same F(2x2,3x3) kernels here, so it reports their size, not the reference's
+// F(4x4,3x3) one; the filter gradient under either Winograd tag runs on the
+// implicit-GEMM kernel and needs nothing.
 int workspace_size(const snn_hip_conv2d_params& p, int direction,
                    int algorithm, size_t* required, size_t* recommended) {
   *required = 0;
@@ -245,18 +264,10 @@ int workspace_size(const snn_hip_conv2d_params& p, int direction,
   const bool filbk = direction == SNN_HIP_FILTER_BACKPROP;
   switch (algorithm) {
     case SNN_HIP_ALGO_WINOGRAD:
-      // F(2x2,3x3), or F(3x3,2x2) for the filter gradient
-      // (workspace_size.h:78-87).
-      if (filbk)
-        winograd_workspace(p, direction, 3, 3, 2, 2, required, recommended);
-      else
-        winograd_workspace(p, direction, 2, 2, 3, 3, required, recommended);
-      break;
     case SNN_HIP_ALGO_WINOGRAD_LARGE:
-      if (filbk)
-        winograd_workspace(p, direction, 3, 3, 3, 3, required, recommended);
-      else
-        winograd_workspace(p, direction, 4, 4, 3, 3, required, recommended);
+      // (1x3 / 3x1 windows are computed by the implicit-GEMM kernel too)
+      if (!filbk && p.window_rows == 3 && p.window_cols == 3)
+        winograd_workspace(p, direction, 2, 2, 3, 3, required, recommended);
       break;
     case SNN_HIP_ALGO_IM2COL:
       im2col_workspace(p, direction, required, recommended);
@@ -350,7 +361,7 @@ int launch_winograd_path<float>(int direction, const float* input,
   // chain on shapes the fused kernel would take.
   if (conv2d_winograd_fused_supports(direction, p) && aligned16(input) &&
       aligned16(output) && aligned16(workspace) &&
-      std::getenv("SNN_HIP_WINO_UNFUSED") == nullptr)
+      SNN_TUNING_ENV("SNN_HIP_WINO_UNFUSED") == nullptr)
     return launch_conv2d_winograd_fused_f32(direction, input, filter, output,
                                             p, workspace, workspace_elems, s,
                                             epilogue);
@@ -457,11 +468,16 @@ int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
   }
   switch (algorithm) {
     case SNN_HIP_ALGO_WINOGRAD:
-    case SNN_HIP_ALGO_WINOGRAD_LARGE:
-      if (workspace == nullptr || workspace_elems == 0)
+    case SNN_HIP_ALGO_WINOGRAD_LARGE: {
+      // internal/conv2d/winograd/launch.h:271-286: a Winograd launch without
+      // the workspace its transforms need reports InsufficientWorkspace.
+      size_t required = 0, recommended = 0;
+      workspace_size(p, direction, algorithm, &required, &recommended);
+      if (required > 0 && (workspace == nullptr || workspace_elems < required))
         return SNN_HIP_INSUFFICIENT_WORKSPACE;
       return launch_winograd_path<T>(direction, input, filter, output, p,
                                      workspace, workspace_elems, s, epilogue);
+    }
     case SNN_HIP_ALGO_TILED:
     case SNN_HIP_ALGO_IM2COL:
     case SNN_HIP_ALGO_MATMUL:
@@ -529,7 +545,7 @@ const char* snn_hip_status_string(int status) {
 const char* snn_hip_last_error(void) { return g_last_error.c_str(); }
 
 int snn_hip_kernel_timing_enable(int enable) {
-  snn::g_timing_enabled = enable != 0;
+  snn::g_timing_enabled.store(enable != 0);
   return SNN_HIP_OK;
 }
 
@@ -539,7 +555,12 @@ int snn_hip_kernel_timing_read(double* total_ms, int* kernels) {
   double sum = 0.0;
   int n = 0;
   int status = SNN_HIP_OK;
-  for (auto& pair : snn::g_timed_kernels) {
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> pairs;
+  {
+    std::lock_guard<std::mutex> lock(snn::g_timing_mutex);
+    pairs.swap(snn::g_timed_kernels);
+  }
+  for (auto& pair : pairs) {
     float ms = 0.f;
     hipError_t err = hipEventSynchronize(pair.second);
     if (err == hipSuccess)
@@ -553,7 +574,6 @@ int snn_hip_kernel_timing_read(double* total_ms, int* kernels) {
     (void)hipEventDestroy(pair.first);
     (void)hipEventDestroy(pair.second);
   }
-  snn::g_timed_kernels.clear();
   *total_ms = sum;
   *kernels = n;
   return status;

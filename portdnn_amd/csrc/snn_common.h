@@ -8,6 +8,7 @@
 #include <climits>
 #include <cstddef>
 #include <cstdint>
+#include <cstdlib>
 #include <string>
 
 #include "snn_hip.h"
@@ -38,6 +39,20 @@ int report_error(int status, const std::string& text);
   do {                                            \
     if (!(cond)) return SNN_HIP_INVALID_PARAMETER; \
   } while (0)
+
+// Developer switches (tile shapes, kernel choices) are read from the
+// environment only in builds made with -DSNN_HIP_TUNING, once per switch; the
+// shipped library reads no environment variable and every SNN_TUNING_ENV is a
+// null constant the compiler folds away.
+#ifdef SNN_HIP_TUNING
+#define SNN_TUNING_ENV(name)                     \
+  ([]() -> const char* {                         \
+    static const char* const value = std::getenv(name); \
+    return value;                                \
+  }())
+#else
+#define SNN_TUNING_ENV(name) (static_cast<const char*>(nullptr))
+#endif
 
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 

@@ -109,10 +109,10 @@ def test_conv2d_invalid_algorithm():
 
 def test_winograd_needs_workspace():
     """internal/conv2d/winograd/launch.h:271-286"""
-    for d in (DIRECTION.FORWARD, DIRECTION.INPUT_BACKPROP,
-              DIRECTION.FILTER_BACKPROP):
-        assert _call_conv(_conv(), ALGO.WINOGRAD,
-                          d) == STATUS.INSUFFICIENT_WORKSPACE
+    for algo in (ALGO.WINOGRAD, ALGO.WINOGRAD_LARGE):
+        for d in (DIRECTION.FORWARD, DIRECTION.INPUT_BACKPROP):
+            assert _call_conv(_conv(), algo,
+                              d) == STATUS.INSUFFICIENT_WORKSPACE
 
 
 def test_index_exceeded():
@@ -239,10 +239,18 @@ def test_workspace_sizes_reference_bounds():
     ab = 16
     t = 112 * 112 * 64
     f = 64 * 64
-    for d in range(3):
-        req, rec = ops.workspace_size(p, d, ALGO.WINOGRAD)
-        assert req >= ab * (t + f + t)
-        assert rec >= ab * (32 * (t + t) + f)
+    for d in (DIRECTION.FORWARD, DIRECTION.INPUT_BACKPROP):
+        for algo in (ALGO.WINOGRAD, ALGO.WINOGRAD_LARGE):
+            req, rec = ops.workspace_size(p, d, algo)
+            assert req >= ab * (t + f + t)
+            assert rec >= ab * (32 * (t + t) + f)
+    # WinogradLarge runs the F(2x2,3x3) kernels: it asks for their size
+    assert ops.workspace_size(p, DIRECTION.FORWARD, ALGO.WINOGRAD_LARGE) == \
+        ops.workspace_size(p, DIRECTION.FORWARD, ALGO.WINOGRAD)
+    # the filter gradient under the Winograd tags runs on the implicit-GEMM
+    # kernel, which needs no caller scratch
+    assert ops.workspace_size(p, DIRECTION.FILTER_BACKPROP,
+                              ALGO.WINOGRAD) == (0, 0)
     # figures quoted for the benchmark layers (Winograd F(2x2,3x3), batch 32)
     p56 = ops.conv_params(32, 56, 56, 64, 64, 3, 1, True)
     req, rec = ops.workspace_size(p56, DIRECTION.FORWARD, ALGO.WINOGRAD)
