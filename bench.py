@@ -12,11 +12,18 @@ algorithm).  The same JSON line carries
 
   roofline      the main kernel of the 3x3 convolutions against the fp32 MFMA
                 peak: algorithmic flops per launch over its average duration,
-                timed with HIP events on the launch stream,
-  cpu_baseline  the reference's tiled algorithm restated in C (oracle/), timed
-                on the host cores on a bounded sample of the same layers,
-  detail        per-layer / per-algorithm TFLOP/s and the depthwise / pooling
-                GB/s against the HBM peak.
+                timed with HIP events on the launch stream; `traffic` is read
+                from the committed rocprofv3 summary named in `traffic_source`;
+                `hbm` lists the memory-bound half of the metric (depthwise and
+                pooling kernels against the HBM peak), `config0` the
+                single-image 56x56x64 layer through the Tiled algorithm,
+  cpu_baseline  the reference's algorithms restated in C (oracle/), timed on
+                the host cores on bounded samples: the tiled convolution on
+                the same eight layers (`value`), the depthwise and pooling
+                loops (`memory_bound`) and the single-image layer (`config0`),
+  detail        per-layer / per-algorithm TFLOP/s, gradients, half precision.
+
+No printed fraction of a peak may exceed 1: `frac()` raises if one does.
 """
 import argparse
 import json
@@ -29,10 +36,40 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch of the fused Winograd kernel, mean over the four 3x3
-# layers, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (FETCH_SIZE scaled
-# by the factor a plain copy kernel of known size shows, 2.0; WRITE_SIZE 1.0).
-WINOGRAD_TRAFFIC_BYTES = 42.5e6
+# HBM bytes per launch of the dominant kernel come from this committed
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary (its header says how the
+# counters were scaled): the "HBM MB / launch" column of the rows of the
+# kernel, averaged over the four 3x3 layers.
+TRAFFIC_PROFILE = os.path.join("profiles",
+                               "conv2d_forward_resnet_batch32_hbm_traffic.md")
+
+
+def profiled_traffic_bytes(kernel_prefix):
+    """Mean of the 'HBM MB / launch' column over the table rows whose kernel
+    name starts with `kernel_prefix`, in bytes; None if there is no such row."""
+    path = os.path.join(ROOT, TRAFFIC_PROFILE)
+    if not os.path.exists(path):
+        return None
+    column = None
+    values = []
+    with open(path) as f:
+        for line in f:
+            cells = [c.strip() for c in line.strip().strip("|").split("|")]
+            if "HBM MB / launch" in cells:
+                column = cells.index("HBM MB / launch")
+            elif (column is not None and cells and
+                  cells[0].strip("`").startswith(kernel_prefix) and
+                  len(cells) > column):
+                values.append(float(cells[column]))
+    return sum(values) / len(values) * 1e6 if values else None
+
+
+def frac(value, peak):
+    """value / peak, rounded; a fraction above 1 means the accounting is wrong."""
+    f = value / peak
+    if f > 1.0:
+        raise AssertionError("fraction of peak above 1: %r / %r" % (value, peak))
+    return round(f, 4)
 
 RESNET = [(56, 64), (28, 128), (14, 256), (7, 512)]
 MOBILENET = [(112, 32, 1), (112, 64, 2), (56, 128, 1), (28, 256, 2),
@@ -157,7 +194,7 @@ def main():
         per_layer.append({"layer": w["name"], "algorithm": algo_names[w["algo"]],
                           "ms": round(ms, 4), "kernel_ms": round(kernel_ms, 4),
                           "tflops": round(tf, 2),
-                          "frac_mfma_peak": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)})
+                          "frac_mfma_peak": frac(tf, PEAK_FP32_MFMA_TFLOPS)})
         if w["name"].startswith("3x3"):
             k3_flops += w["flops"] * kt.kernels
             k3_kernel_ms += kt.total_ms
@@ -170,19 +207,122 @@ def main():
         "kernel": "main kernel of the 3x3 s1 forward convolution (%s), the four "
                   "ResNet stages, one launch each per step" % "/".join(k3_algos),
         "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
-        "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+        "unit": "TFLOP/s", "frac": frac(achieved, PEAK_FP32_MFMA_TFLOPS),
         "avg_kernel_ms": round(k3_kernel_ms / k3_kernels, 5),
         "algorithmic_gflop_per_launch": round(k3_flops / k3_kernels / 1e9, 4),
         # Winograd F(2x2,3x3) executes 16/36 of the algorithmic flops on the
         # matrix cores; this is the MFMA pipe's own utilisation
         "mfma_executed_tflops": round(
             achieved * (4.0 / 9.0 if k3_algos == ["winograd"] else 1.0), 2),
-        "mfma_executed_frac": round(
-            achieved * (4.0 / 9.0 if k3_algos == ["winograd"] else 1.0) /
-            PEAK_FP32_MFMA_TFLOPS, 4),
-        "traffic": WINOGRAD_TRAFFIC_BYTES if k3_algos == ["winograd"] else None}
+        "mfma_executed_frac": frac(
+            achieved * (4.0 / 9.0 if k3_algos == ["winograd"] else 1.0),
+            PEAK_FP32_MFMA_TFLOPS),
+        "traffic": (profiled_traffic_bytes("wino_fused_kernel")
+                    if k3_algos == ["winograd"] else None),
+        "traffic_source": TRAFFIC_PROFILE}
 
-    detail = {"layers": per_layer}
+    # ---- memory-bound half of the metric: depthwise and pooling against HBM ----
+    # Buffer sets rotate so that the 256 MB last-level cache cannot hold the
+    # working set between launches.
+    def rotate_sets(nbytes):
+        return max(3, int(600e6 // nbytes) + 1)
+
+    def device_ms(fn, calls):
+        """Mean device time of one call: HIP events the library records on the
+        launch stream around the kernels of each call (what rocprofv3 reports
+        per kernel), free of the host's launch rate, which bounds `ms` for
+        the smallest layers."""
+        with ops.kernel_timing() as kt:
+            for _ in range(calls):
+                fn()
+        return kt.total_ms / max(1, kt.kernels)
+
+    def mem_entry(name, nbytes, ms, kernel_ms):
+        gbs = nbytes / ms / 1e6
+        kgbs = nbytes / kernel_ms / 1e6
+        return {"op": name, "bytes": nbytes, "ms": round(ms, 5),
+                "gbs": round(gbs, 1),
+                "frac_hbm_peak": frac(gbs, PEAK_HBM_GBS),
+                "kernel_ms": round(kernel_ms, 5),
+                "kernel_gbs": round(kgbs, 1),
+                "kernel_frac_hbm_peak": frac(kgbs, PEAK_HBM_GBS)}
+
+    def depthwise_entry(size, ch, stride):
+        p = ops.depthwise_params(BATCH, size, size, ch, 1, 3, stride, True)
+        n_in, n_fil, n_out = ops.depthwise_sizes(p, DIRECTION.FORWARD)
+        nbytes = 4 * (n_in + n_fil + n_out)
+        sets = rotate_sets(nbytes)
+        xs = [normal(n_in) for _ in range(sets)]
+        ys = [torch.empty(n_out, device="cuda") for _ in range(sets)]
+        f = normal(n_fil)
+        state = {"i": 0}
+
+        def run():
+            i = state["i"] % sets
+            state["i"] += 1
+            ops.depthwise_conv2d(xs[i], f, p, out=ys[i])
+        ms = event_time_ms(run, reps=5 * sets, warm=sets, repeats=3)
+        return mem_entry("depthwise3x3_%dx%dx%d_s%d" % (size, size, ch, stride),
+                         nbytes, ms, device_ms(run, 5 * sets))
+
+    def pooling_entry(name, p, op):
+        n_in = p.batch * p.in_rows * p.in_cols * p.channels
+        n_out = p.batch * p.out_rows * p.out_cols * p.channels
+        nbytes = 4 * (n_in + n_out)
+        sets = rotate_sets(nbytes)
+        xs = [normal(n_in) for _ in range(sets)]
+        ys = [torch.empty(n_out, device="cuda") for _ in range(sets)]
+        state = {"i": 0}
+
+        def run():
+            i = state["i"] % sets
+            state["i"] += 1
+            ops.pooling_forward(xs[i], p, op, out=ys[i])
+        ms = event_time_ms(run, reps=5 * sets, warm=sets, repeats=3)
+        return mem_entry(name, nbytes, ms, device_ms(run, 5 * sets))
+
+    POOLS = (("maxpool3x3_s2_112x112x64",
+              ops.pool_params(BATCH, 112, 112, 64, 3, 2, True), POOL_OP.MAX),
+             ("avgpool7x7_7x7x2048",
+              ops.pool_params(BATCH, 7, 7, 2048, 7, 1, False), POOL_OP.AVERAGE))
+    mem = [depthwise_entry(*layer) for layer in MOBILENET]
+    mem += [pooling_entry(*pool) for pool in POOLS]
+    # The entries a reader needs beside the convolution figure: kernel = what
+    # ran, bytes_per_launch = (input + filter + output) * 4, the time of one
+    # launch and the fraction of the 8 TB/s peak.  ms_per_launch is the mean
+    # over back-to-back launches between two stream events (an upper bound of
+    # the kernel's own duration, which rocprofv3 reports; the per-launch event
+    # pairs behind `kernel_ms` in detail.memory_bound add 2-3 us to kernels
+    # this short).
+    roofline["hbm"] = [
+        {"kernel": e["op"], "bytes_per_launch": e["bytes"],
+         "ms_per_launch": e["ms"], "achieved_gbs": e["gbs"],
+         "frac": e["frac_hbm_peak"]}
+        for e in mem if e["op"] in (
+            "depthwise3x3_112x112x64_s2", "depthwise3x3_56x56x128_s1",
+            "maxpool3x3_s2_112x112x64", "avgpool7x7_7x7x2048")]
+
+    # ---- configuration 0: one 56x56x64 image, 3x3 s1 SAME, Tiled -------------
+    p0 = ops.conv_params(1, 56, 56, 64, 64, 3, 1, True)
+    x0, w0 = uniform(56 * 56 * 64), uniform(9 * 64 * 64)
+    y0 = torch.empty(56 * 56 * 64, device="cuda")
+
+    def call0():
+        ops.conv2d(x0, w0, p0, DIRECTION.FORWARD, ALGO.TILED, out=y0)
+    ms0 = event_time_ms(call0, reps=50)
+    with ops.kernel_timing() as kt:
+        for _ in range(50):
+            call0()
+    kms0 = kt.total_ms / max(1, kt.kernels)
+    fl0 = ops.conv_flops(p0, DIRECTION.FORWARD)
+    roofline["config0"] = {
+        "workload": "conv2d forward fp32 [1,56,56,64] x [3,3,64,64], s1 SAME, "
+                    "Tiled", "gflop": round(fl0 / 1e9, 4), "ms": round(ms0, 5),
+        "tflops": round(fl0 / ms0 / 1e9, 2), "kernel_ms": round(kms0, 5),
+        "kernel_tflops": round(fl0 / kms0 / 1e9, 2),
+        "kernel_frac_mfma_peak": frac(fl0 / kms0 / 1e9, PEAK_FP32_MFMA_TFLOPS)}
+
+    detail = {"layers": per_layer, "memory_bound": mem}
     if not args.no_detail:
         # every algorithm on every 3x3 / 1x1 layer
         algo_table = []
@@ -203,9 +343,13 @@ def main():
                 del ws
         detail["algorithms"] = algo_table
 
-        # backprops of the 3x3 layers and the 7x7 s2 stem in all directions
-        # (flops as the reference's benchmarks count them: by input pixels
-        # for the two gradients)
+        # backprops of the 3x3 layers and the 7x7 s2 stem in all directions.
+        # `tflops_reference_accounting` counts the two gradients by input
+        # pixels, 2*N*H*W*R*S*C*K, as the reference's benchmarks do
+        # (bench/conv2d/base_convolution_fixture.h:91-109), which at stride 2
+        # is four times the multiplies a gradient needs; `tflops` and the
+        # fraction of the peak count the multiply-adds of the convolution
+        # itself, 2*N*OH*OW*R*S*C*K, in every direction.
         bk = []
         stem = ops.conv_params(BATCH, 224, 224, 3, 64, 7, 2, True)
         cases = [("stem7x7_s2_224x224x3_k64", stem, d) for d in (
@@ -228,10 +372,15 @@ def main():
             ms = event_time_ms(lambda: ops.conv2d(
                 a, b, p, direction, algo, workspace=ws, out=o), reps=10,
                 warm=2, repeats=3)
-            fl = ops.conv_flops(p, direction)
+            fl_ref = ops.conv_flops(p, direction)
+            fl = ops.conv_flops(p, DIRECTION.FORWARD)
             bk.append({"layer": name, "direction": dir_names[direction],
                        "algorithm": algo_names[algo], "ms": round(ms, 4),
-                       "tflops": round(fl / ms / 1e9, 2)})
+                       "tflops": round(fl / ms / 1e9, 2),
+                       "frac_mfma_peak": frac(fl / ms / 1e9,
+                                              PEAK_FP32_MFMA_TFLOPS),
+                       "tflops_reference_accounting": round(
+                           fl_ref / ms / 1e9, 2)})
             del a, b, o, ws
         detail["backprop_and_stem"] = bk
 
@@ -252,7 +401,7 @@ def main():
                 h.append({"op": "conv%dx%d_%dx%dx%d_k%d_b128_f16" % (
                     window, window, size, size, ch, feats), "ms": round(ms, 4),
                     "tflops": round(fl / ms / 1e9, 1),
-                    "frac_f16_mfma_peak": round(fl / ms / 1e9 / 2500.0, 4)})
+                    "frac_f16_mfma_peak": frac(fl / ms / 1e9, 2500.0)})
                 if window == 3:
                     # input gradient: the same kernel on dY (o) with the
                     # filter's taps mirrored and its roles swapped
@@ -266,8 +415,8 @@ def main():
                               "backprop" % (size, size, ch, feats),
                               "ms": round(ms, 4),
                               "tflops": round(fl / ms / 1e9, 1),
-                              "frac_f16_mfma_peak": round(
-                                  fl / ms / 1e9 / 2500.0, 4)})
+                              "frac_f16_mfma_peak": frac(
+                                  fl / ms / 1e9, 2500.0)})
                     del dx
                 del a, b, o, ws
         for size, ch, stride in MOBILENET:
@@ -290,78 +439,9 @@ def main():
             h.append({"op": "depthwise3x3_%dx%dx%d_s%d_b128_f16" % (
                 size, size, ch, stride), "bytes": nbytes, "ms": round(ms, 5),
                 "gbs": round(gbs, 1),
-                "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)})
+                "frac_hbm_peak": frac(gbs, PEAK_HBM_GBS)})
             del xs, ys
         detail["f16_batch128"] = h
-
-        # memory-bound operators: rotate buffer sets so that the 256 MB
-        # last-level cache cannot hold the working set between launches
-        mem = []
-
-        def rotate_sets(nbytes):
-            return max(3, int(600e6 // nbytes) + 1)
-
-        def device_ms(fn, calls):
-            """Mean device time of one call: HIP events the library records
-            on the launch stream around the kernels of each call (what
-            rocprofv3 reports per kernel), free of the host's launch rate,
-            which bounds `ms` for the smallest layers."""
-            with ops.kernel_timing() as kt:
-                for _ in range(calls):
-                    fn()
-            return kt.total_ms / max(1, kt.kernels)
-
-        def mem_entry(name, nbytes, ms, kernel_ms):
-            gbs = nbytes / ms / 1e6
-            kgbs = nbytes / kernel_ms / 1e6
-            return {"op": name, "bytes": nbytes, "ms": round(ms, 5),
-                    "gbs": round(gbs, 1),
-                    "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
-                    "kernel_ms": round(kernel_ms, 5),
-                    "kernel_gbs": round(kgbs, 1),
-                    "kernel_frac_hbm_peak": round(kgbs / PEAK_HBM_GBS, 4)}
-
-        for size, ch, stride in MOBILENET:
-            p = ops.depthwise_params(BATCH, size, size, ch, 1, 3, stride, True)
-            n_in, n_fil, n_out = ops.depthwise_sizes(p, DIRECTION.FORWARD)
-            nbytes = 4 * (n_in + n_fil + n_out)
-            sets = rotate_sets(nbytes)
-            xs = [normal(n_in) for _ in range(sets)]
-            ys = [torch.empty(n_out, device="cuda") for _ in range(sets)]
-            f = normal(n_fil)
-            state = {"i": 0}
-
-            def run():
-                i = state["i"] % sets
-                state["i"] += 1
-                ops.depthwise_conv2d(xs[i], f, p, out=ys[i])
-            ms = event_time_ms(run, reps=5 * sets, warm=sets, repeats=3)
-            mem.append(mem_entry(
-                "depthwise3x3_%dx%dx%d_s%d" % (size, size, ch, stride), nbytes,
-                ms, device_ms(run, 5 * sets)))
-            del xs, ys
-        for name, p, op in (
-                ("maxpool3x3_s2_112x112x64",
-                 ops.pool_params(BATCH, 112, 112, 64, 3, 2, True), POOL_OP.MAX),
-                ("avgpool7x7_7x7x2048",
-                 ops.pool_params(BATCH, 7, 7, 2048, 7, 1, False),
-                 POOL_OP.AVERAGE)):
-            n_in = p.batch * p.in_rows * p.in_cols * p.channels
-            n_out = p.batch * p.out_rows * p.out_cols * p.channels
-            nbytes = 4 * (n_in + n_out)
-            sets = rotate_sets(nbytes)
-            xs = [normal(n_in) for _ in range(sets)]
-            ys = [torch.empty(n_out, device="cuda") for _ in range(sets)]
-            state = {"i": 0}
-
-            def run():
-                i = state["i"] % sets
-                state["i"] += 1
-                ops.pooling_forward(xs[i], p, op, out=ys[i])
-            ms = event_time_ms(run, reps=5 * sets, warm=sets, repeats=3)
-            mem.append(mem_entry(name, nbytes, ms, device_ms(run, 5 * sets)))
-            del xs, ys
-        detail["memory_bound"] = mem
 
         # element-wise operators on the 56x56x256 activation of the first
         # ResNet stage: ReLU (read + write) and bias add (read + write + bias)
@@ -391,7 +471,7 @@ def main():
             gbs = nbytes / ms / 1e6
             elem.append({"op": name, "bytes": nbytes, "ms": round(ms, 5),
                          "gbs": round(gbs, 1),
-                         "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)})
+                         "frac_hbm_peak": frac(gbs, PEAK_HBM_GBS)})
         del xs, ys
         detail["elementwise"] = elem
 
@@ -498,7 +578,7 @@ def main():
             mm.append({"op": "matmul b%d %dx%dx%d%s" % (
                 batches, m, k, n, " rhs^T" if tb else ""), "ms": round(ms, 4),
                 "tflops": round(tf, 2),
-                "frac_mfma_peak": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)})
+                "frac_mfma_peak": frac(tf, PEAK_FP32_MFMA_TFLOPS)})
         detail["matmul"] = mm
 
     # ---- CPU baseline: the reference's tiled algorithm, restated --------------
@@ -537,6 +617,63 @@ def main():
                          "portDNN tiled algorithm (2x2x4 register tiles) "
                          "restated in C with OpenMP; %.1f s of CPU time"
                          % (passes, cpu_batch, cpu_s)}
+
+        def cpu_time(fn, budget_s, max_runs=10):
+            """Median wall time of fn() after one warm-up run, at most
+            `max_runs` runs or `budget_s` seconds."""
+            fn()
+            times, spent = [], 0.0
+            while len(times) < max_runs and (spent < budget_s or not times):
+                t = time.perf_counter()
+                fn()
+                times.append(time.perf_counter() - t)
+                spent += times[-1]
+            times.sort()
+            return times[len(times) // 2], len(times)
+
+        # configuration 0 on the CPU: the single 56x56x64 image, tiled
+        p = oracle.make_params(1, 56, 56, 64, 64, 3, 1, True)
+        x = rng.uniform(-1, 1, 56 * 56 * 64).astype(np.float32)
+        w = rng.uniform(-1, 1, 9 * 64 * 64).astype(np.float32)
+        sec, runs = cpu_time(lambda: oracle.conv2d_tiled_forward(x, w, p), 2.0)
+        cpu["config0"] = {
+            "value": round(2.0 * 56 * 56 * 9 * 64 * 64 / sec / 1e12, 5),
+            "unit": "TFLOP/s", "ms": round(sec * 1e3, 3), "cores": cores,
+            "sample": "median of %d runs of the tiled restatement on "
+                      "[1,56,56,64] x [3,3,64,64]" % runs}
+
+        # depthwise and pooling in the reference's loop order
+        # (src/depthwise_conv2d/kernels.h:58-125, src/pooling/kernels.h:61-99:
+        # one work-item per output element, window rows then columns, fp32),
+        # work-items spread over the host threads; batch 8 of each layer
+        mem_cpu = []
+        cb = 8
+        for size, ch, stride in MOBILENET:
+            p = oracle.make_params(cb, size, size, ch, 1, 3, stride, True)
+            x = rng.standard_normal(cb * size * size * ch).astype(np.float32)
+            w = rng.standard_normal(9 * ch).astype(np.float32)
+            sec, runs = cpu_time(
+                lambda: oracle.depthwise_forward(x, w, p, acc64=False), 1.0, 5)
+            nbytes = 4 * (x.size + w.size + cb * p.out_rows * p.out_cols * ch)
+            mem_cpu.append({"op": "depthwise3x3_%dx%dx%d_s%d" % (
+                size, size, ch, stride), "batch": cb, "bytes": nbytes,
+                "ms": round(sec * 1e3, 3),
+                "gbs": round(nbytes / sec / 1e9, 2), "runs": runs})
+        for name, args_, fn in (
+                ("maxpool3x3_s2_112x112x64", (cb, 112, 112, 64, 0, 3, 2, True),
+                 lambda x, p: oracle.pool_max_forward(x, p)),
+                ("avgpool7x7_7x7x2048", (cb, 7, 7, 2048, 0, 7, 1, False),
+                 lambda x, p: oracle.pool_avg_forward(x, p, acc64=False))):
+            p = oracle.make_params(*args_)
+            x = rng.standard_normal(
+                cb * args_[1] * args_[2] * args_[3]).astype(np.float32)
+            sec, runs = cpu_time(lambda: fn(x, p), 1.0, 5)
+            nbytes = 4 * (x.size + cb * p.out_rows * p.out_cols * args_[3])
+            mem_cpu.append({"op": name, "batch": cb, "bytes": nbytes,
+                            "ms": round(sec * 1e3, 3),
+                            "gbs": round(nbytes / sec / 1e9, 2), "runs": runs})
+        cpu["memory_bound"] = mem_cpu
+        cpu["memory_bound_unit"] = "GB/s"
 
     line = {
         "metric": "conv2d fwd TFLOP/s + %MFMA peak; depthwise/pool GB/s + "
