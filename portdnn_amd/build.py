@@ -1,6 +1,11 @@
 """Builds libsnn_hip.so (the HIP kernels + C ABI) in-tree with hipcc for gfx950.
 
-    python -m portdnn_amd.build
+    python -m portdnn_amd.build [-v] [--define NAME[=VALUE]]... [--output PATH]
+
+--define adds a preprocessor definition (-DSNN_HIP_TUNING turns on the
+developer switches read from the environment); --output writes the library
+somewhere else than portdnn_amd/libsnn_hip.so, with its objects in a
+directory of their own, and skips the C++ test programs.
 """
 import concurrent.futures
 import glob
@@ -25,9 +30,10 @@ FLAGS = [
 ]
 
 
-def _compile(src):
-    obj = os.path.join(OBJ_DIR, os.path.basename(src) + ".o")
-    cmd = [HIPCC] + FLAGS + ["-c", src, "-o", obj]
+def _compile(src, obj_dir=OBJ_DIR, defines=()):
+    obj = os.path.join(obj_dir, os.path.basename(src) + ".o")
+    cmd = ([HIPCC] + FLAGS + ["-D" + d for d in defines] +
+           ["-c", src, "-o", obj])
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
                           text=True)
     out = "\n".join(l for l in proc.stdout.splitlines()
@@ -37,22 +43,25 @@ def _compile(src):
     return obj, out
 
 
-def build_library(verbose=False, jobs=8):
+def build_library(verbose=False, jobs=8, defines=(), output=None):
     """Compiles every csrc/*.hip and links libsnn_hip.so. Always rebuilds."""
-    os.makedirs(OBJ_DIR, exist_ok=True)
+    lib_path = LIB_PATH if output is None else os.path.abspath(output)
+    obj_dir = OBJ_DIR if output is None else lib_path + ".objs"
+    os.makedirs(obj_dir, exist_ok=True)
     sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
     if not sources:
         raise RuntimeError("no HIP sources under " + CSRC)
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        results = list(pool.map(_compile, sources))
+        results = list(pool.map(
+            lambda src: _compile(src, obj_dir, defines), sources))
     for obj, out in results:
         if verbose and out:
             print(out)
     objs = [obj for obj, _ in results]
     cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=" + ARCH, "-o",
-           LIB_PATH] + objs
+           lib_path] + objs
     subprocess.check_call(cmd)
-    return LIB_PATH
+    return lib_path
 
 
 CPP_TEST_DIR = os.path.join(ROOT, "tests", "cpp")
@@ -87,5 +96,12 @@ def build_cpp_tests():
 
 
 if __name__ == "__main__":
-    print(build_library(verbose="-v" in sys.argv))
-    print(build_cpp_tests())
+    import argparse
+    ap = argparse.ArgumentParser()
+    ap.add_argument("-v", action="store_true")
+    ap.add_argument("--define", action="append", default=[])
+    ap.add_argument("--output")
+    a = ap.parse_args()
+    print(build_library(verbose=a.v, defines=a.define, output=a.output))
+    if a.output is None:
+        print(build_cpp_tests())

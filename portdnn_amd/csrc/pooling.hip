@@ -10,6 +10,7 @@
 
 #include <cstdlib>
 
+#include "gemm_tile.h"
 #include "snn_kernels.h"
 
 namespace snn {
@@ -201,7 +202,11 @@ __global__ void __launch_bounds__(256)
     pool_forward_3x3_strip_kernel(const T* __restrict__ in, T* __restrict__ out,
                                   snn_hip_pooling_params p, int n_strips,
                                   unsigned n_items) {
-  const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+  // Work-groups go round-robin to the 8 XCDs; the remap gives every XCD one
+  // contiguous run of the index space, so vertically adjacent strips (which
+  // share an input row at stride 2, two at stride 1) meet in the same L2.
+  const unsigned idx =
+      gemm::xcd_remap(blockIdx.x, gridDim.x) * 256u + threadIdx.x;
   if (idx >= n_items) return;
   const int C = p.channels;
   const unsigned cv = static_cast<unsigned>(C) / 4u;
@@ -284,17 +289,23 @@ __global__ void __launch_bounds__(256)
 }
 
 // ---- windows covering most of a small image (global pooling) ---------------
-// One work-group per (image, 64-channel-vector group, output pixel); the
-// window rows are spread over the 4 waves and combined through LDS, so the 49
-// taps of a 7x7 global average are 13 loads deep instead of 49.
+// One work-group per (image, output pixel, group of 16 channel vectors).  The
+// window taps are dealt to 16 tap slices -- four per wave, lane = slice * 16 +
+// channel vector -- so the 49 taps of a 7x7 global average are at most four
+// independent 16-byte loads per lane, all in flight together, and 16 lanes
+// read one contiguous 256-byte run of a pixel's channels.  The slices of a
+// wave are combined with two cross-lane exchanges (no LDS memory), the four
+// waves through 1 KiB of LDS.
 template <typename T, typename Op>
 __global__ void __launch_bounds__(256)
-    pool_forward_rowsplit_kernel(const T* __restrict__ in, T* __restrict__ out,
+    pool_forward_tapsplit_kernel(const T* __restrict__ in, T* __restrict__ out,
                                  snn_hip_pooling_params p, int n_groups) {
-  __shared__ float part[4][64][4];
+  __shared__ float part[4][16][4];
   const int C = p.channels;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
+  const int cvl = lane & 15;
+  const int slice = wave * 4 + (lane >> 4);  // 0 .. 15
   unsigned b = blockIdx.x;
   const int grp = static_cast<int>(b % static_cast<unsigned>(n_groups));
   b /= static_cast<unsigned>(n_groups);
@@ -302,7 +313,7 @@ __global__ void __launch_bounds__(256)
   b /= static_cast<unsigned>(p.out_cols);
   const int oy = static_cast<int>(b % static_cast<unsigned>(p.out_rows));
   const int n = static_cast<int>(b / static_cast<unsigned>(p.out_rows));
-  const int c = (grp * 64 + lane) * 4;
+  const int c = (grp * 16 + cvl) * 4;
   const bool active = c < C;
   int r0 = oy * p.stride_rows - p.pad_rows;
   const int r1 = min(r0 + p.window_rows, p.in_rows);
@@ -310,32 +321,51 @@ __global__ void __launch_bounds__(256)
   int c0 = ox * p.stride_cols - p.pad_cols;
   const int c1 = min(c0 + p.window_cols, p.in_cols);
   c0 = max(c0, 0);
+  const int width = c1 - c0;
+  const int n_taps = (r1 - r0) * width;
   Op acc[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) acc[i].init(lowest_of<T>());
-  if (active) {
+  if (active && n_taps > 0) {
     const T* base =
         in + static_cast<size_t>(n) * p.in_rows * p.in_cols * C + c;
-    for (int r = r0 + wave; r < r1; r += 4) {
-      for (int col = c0; col < c1; ++col) {
-        float v[4];
-        VecIO<T, 4>::load(base + (static_cast<size_t>(r) * p.in_cols + col) * C,
-                          v);
+    for (int t0 = slice; t0 < n_taps; t0 += 64) {
+      float v[4][4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i].accumulate(v[i]);
+      for (int k = 0; k < 4; ++k) {
+        // a tap index past the end re-reads the last tap and is not counted
+        const int t = min(t0 + 16 * k, n_taps - 1);
+        const int r = r0 + t / width, col = c0 + t % width;
+        VecIO<T, 4>::load(base + (static_cast<size_t>(r) * p.in_cols + col) * C,
+                          v[k]);
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (t0 + 16 * k < n_taps) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[i].accumulate(v[k][i]);
+        }
       }
     }
   }
+  // the four tap slices of this wave: lanes l, l ^ 16, l ^ 32, l ^ 48
 #pragma unroll
-  for (int i = 0; i < 4; ++i) part[wave][lane][i] = acc[i].v;
+  for (int i = 0; i < 4; ++i) {
+    acc[i].merge(__shfl_xor(acc[i].v, 16));
+    acc[i].merge(__shfl_xor(acc[i].v, 32));
+  }
+  if (lane < 16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part[wave][lane][i] = acc[i].v;
+  }
   __syncthreads();
-  if (wave == 0 && active) {
+  if (wave == 0 && lane < 16 && active) {
     float res[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       Op total = acc[i];
       for (int w = 1; w < 4; ++w) total.merge(part[w][lane][i]);
-      res[i] = total.value((r1 - r0) * (c1 - c0));
+      res[i] = total.value(n_taps);
     }
     VecIO<T, 4>::store(
         out + ((static_cast<size_t>(n) * p.out_rows + oy) * p.out_cols + ox) * C +
@@ -607,7 +637,12 @@ int launch_forward_op(const T* input, T* output,
       n_out * sizeof(T) < 0x7FFFFFF0u) {
     const size_t per_row =
         static_cast<size_t>(p.batch) * p.out_cols * (p.channels / 4);
-    int th = 4;
+    // Two output rows per lane: measured on MI355X with the XCD-contiguous
+    // order above, the 112x112x64 stride-2 max pool runs in 24.4 us with one
+    // or two rows per lane against 26.0 us with four (the rows that strips
+    // share come from the XCD's L2 either way, and shorter strips leave more
+    // lanes to keep loads in flight).
+    int th = 2;
     while (th > 1 && per_row * ceil_div(p.out_rows, th) < 150000) th /= 2;
     // Developer override for tuning runs: SNN_HIP_POOL_TH=<1|2|4>.
     static const char* tune = SNN_TUNING_ENV("SNN_HIP_POOL_TH");
@@ -630,15 +665,13 @@ int launch_forward_op(const T* input, T* output,
       else SNN_POOL_STRIP(2, 1);
     }
 #undef SNN_POOL_STRIP
-  } else if (p.channels % 4 == 0 && p.window_rows >= 4 &&
-             static_cast<size_t>(p.batch) * p.out_rows * p.out_cols *
-                     ceil_div(p.channels, 256) >= 256 &&
+  } else if (p.channels % 4 == 0 && p.window_rows * p.window_cols >= 16 &&
              n_out / 4 < 200000) {
-    // few, large windows: split the window rows over the waves
-    const int n_groups = ceil_div(p.channels, 256);
+    // few, large windows: split the window taps over the lanes
+    const int n_groups = ceil_div(p.channels, 64);
     const unsigned blocks = static_cast<unsigned>(
         static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * n_groups);
-    hipLaunchKernelGGL((pool_forward_rowsplit_kernel<T, Op>), dim3(blocks),
+    hipLaunchKernelGGL((pool_forward_tapsplit_kernel<T, Op>), dim3(blocks),
                        dim3(kBlock), 0, stream, input, output, p, n_groups);
   } else if (p.channels % 4 == 0) {
     const size_t n_vec = n_out / 4;
