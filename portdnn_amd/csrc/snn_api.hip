@@ -254,9 +254,11 @@ void im2col_workspace(const snn_hip_conv2d_params& p, int direction,
 // What a launch with `algorithm` needs.  Winograd forward / input backprop
 // follow the reference's F(2x2,3x3) formula (the three-stage chain uses all of
 // it, the fused kernel its transformed-filter part).  WinogradLarge runs the
-// same F(2x2,3x3) kernels here, so it reports their size, not the reference's
-// F(4x4,3x3) one; the filter gradient under either Winograd tag runs on the
-// implicit-GEMM kernel and needs nothing.
+// same F(2x2,3x3) / F(3x3,2x2) kernels here, so it reports their sizes, not
+// the reference's F(4x4,3x3) ones.  The fused F(3x3,2x2) filter gradient keeps
+// no transformed tensors, only one partial filter per slice of the tile
+// range; shapes it does not take run on the implicit-GEMM kernel and need
+// nothing.
 int workspace_size(const snn_hip_conv2d_params& p, int direction,
                    int algorithm, size_t* required, size_t* recommended) {
   *required = 0;
@@ -266,8 +268,12 @@ int workspace_size(const snn_hip_conv2d_params& p, int direction,
     case SNN_HIP_ALGO_WINOGRAD:
     case SNN_HIP_ALGO_WINOGRAD_LARGE:
       // (1x3 / 3x1 windows are computed by the implicit-GEMM kernel too)
-      if (!filbk && p.window_rows == 3 && p.window_cols == 3)
+      if (!filbk && p.window_rows == 3 && p.window_cols == 3) {
         winograd_workspace(p, direction, 2, 2, 3, 3, required, recommended);
+      } else if (filbk && conv2d_winograd_filter_backprop_supports(p)) {
+        *required = conv2d_winograd_filter_backprop_workspace(p);
+        *recommended = *required;
+      }
       break;
     case SNN_HIP_ALGO_IM2COL:
       im2col_workspace(p, direction, required, recommended);
@@ -292,6 +298,15 @@ int default_algorithm(const snn_hip_conv2d_params& p, int direction) {
   if (algorithm_supports(p, direction, SNN_HIP_ALGO_WINOGRAD) &&
       conv2d_winograd_fused_supports(direction, p) &&
       static_cast<long long>(p.batch) * p.out_rows * p.out_cols >= 1024)
+    return SNN_HIP_ALGO_WINOGRAD;
+  // The fused F(3x3,2x2) filter gradient: measured 1.2-1.6x faster than the
+  // implicit GEMM on the batch-32 ResNet shapes once the tile range gives
+  // every work-group a few steps.
+  if (direction == SNN_HIP_FILTER_BACKPROP &&
+      algorithm_supports(p, direction, SNN_HIP_ALGO_WINOGRAD) &&
+      conv2d_winograd_filter_backprop_supports(p) && p.channels % 32 == 0 &&
+      p.features % 32 == 0 &&
+      static_cast<long long>(p.batch) * p.out_rows * p.out_cols >= 4096)
     return SNN_HIP_ALGO_WINOGRAD;
   if (algorithm_supports(p, direction, SNN_HIP_ALGO_TILED))
     return SNN_HIP_ALGO_TILED;
@@ -368,6 +383,11 @@ int launch_winograd_path<float>(int direction, const float* input,
   if (conv2d_winograd_supports(direction, p))
     return launch_conv2d_winograd_f32(direction, input, filter, output, p,
                                       workspace, workspace_elems, s);
+  if (direction == SNN_HIP_FILTER_BACKPROP &&
+      conv2d_winograd_filter_backprop_supports(p) && aligned16(input) &&
+      aligned16(filter) && aligned16(output) && aligned16(workspace))
+    return launch_conv2d_winograd_filter_backprop_f32(
+        input, filter, output, p, workspace, workspace_elems, s);
   return launch_gemm_path<float>(direction, input, filter, output, p, s,
                                  nullptr, 0, epilogue);
 }

@@ -69,6 +69,17 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
                                      hipStream_t stream,
                                      const ConvEpilogue* epilogue = nullptr);
 
+// Winograd F(3x3,2x2) filter gradient of a 3x3 stride-1 convolution in one
+// fused kernel (conv2d_winograd_filter.hip).  `workspace` receives one
+// partial filter per slice of the tile range; `..._workspace` tells how many
+// elements that takes (0 when one work-group per filter block is enough).
+bool conv2d_winograd_filter_backprop_supports(const snn_hip_conv2d_params& p);
+size_t conv2d_winograd_filter_backprop_workspace(
+    const snn_hip_conv2d_params& p);
+int launch_conv2d_winograd_filter_backprop_f32(
+    const float* x, const float* dy, float* dw, const snn_hip_conv2d_params& p,
+    float* workspace, size_t workspace_elems, hipStream_t stream);
+
 // Half-precision forward convolution on MFMA (conv2d_igemm_f16.hip).  The
 // workspace, when large enough, receives the re-laid-out filter.
 bool conv2d_igemm_f16_supports(const snn_hip_conv2d_params& p);

@@ -176,6 +176,25 @@ def test_winograd_fused_shapes(shape, direction):
     conv_case(p, direction, [ALGO.WINOGRAD], seed=1300 + rows + ch)
 
 
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, same
+    (3, 13, 11, 32, 64, True),    # odd sizes: clipped dY tiles on both edges
+    (2, 9, 10, 16, 32, False),    # VALID, half-empty channel and feature blocks
+    (1, 7, 7, 512, 512, True),    # 128 filter blocks, tile range in two slices
+    (5, 6, 5, 48, 96, True),      # ragged channel block, ragged feature block
+    (2, 30, 4, 64, 36, False),    # narrow image, features not a multiple of 32
+    (7, 33, 29, 64, 64, True),    # many slices, ragged last step of a slice
+    (4, 16, 16, 18, 20, True),    # channels x2 only, features x4 only
+])
+def test_winograd_filter_backprop_shapes(shape):
+    """The fused F(3x3,2x2) filter gradient: tile-range slices, partial
+    channel / feature blocks, images with odd sizes."""
+    batch, rows, cols, ch, feats, same = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, 3, 1, same)
+    conv_case(p, DIRECTION.FILTER_BACKPROP, [ALGO.WINOGRAD],
+              seed=1350 + rows + ch)
+
+
 @pytest.mark.parametrize("direction", [DIRECTION.FORWARD,
                                        DIRECTION.INPUT_BACKPROP,
                                        DIRECTION.FILTER_BACKPROP])
