@@ -173,8 +173,8 @@ def test_default_algorithm_is_launchable():
 
 def test_default_algorithm_policy_on_benchmark_layers():
     """1x1 stride-1 layers are one GEMM; 3x3 stride-1 layers whose channel
-    counts fit the fused Winograd kernel take it for forward and input
-    backprop; everything else is the implicit GEMM (Tiled / Im2col tags)."""
+    counts fit the fused Winograd kernels take them in all three directions;
+    everything else is the implicit GEMM (Tiled / Im2col tags)."""
     L = capi.lib()
 
     def default(p, d):
@@ -184,14 +184,14 @@ def test_default_algorithm_policy_on_benchmark_layers():
         p3 = ops.conv_params(32, size, size, ch, ch, 3, 1, True)
         assert default(p3, DIRECTION.FORWARD) == ALGO.WINOGRAD
         assert default(p3, DIRECTION.INPUT_BACKPROP) == ALGO.WINOGRAD
-        assert default(p3, DIRECTION.FILTER_BACKPROP) in (ALGO.TILED,
-                                                          ALGO.IM2COL)
+        assert default(p3, DIRECTION.FILTER_BACKPROP) == ALGO.WINOGRAD
         p1 = ops.conv_params(32, size, size, ch, 4 * ch, 1, 1, False)
         assert default(p1, DIRECTION.FORWARD) == ALGO.MATMUL
     stem = ops.conv_params(32, 224, 224, 3, 64, 7, 2, True)
     assert default(stem, DIRECTION.FORWARD) in (ALGO.TILED, ALGO.IM2COL)
     odd = ops.conv_params(32, 28, 28, 24, 40, 3, 1, True)
     assert default(odd, DIRECTION.FORWARD) in (ALGO.TILED, ALGO.IM2COL)
+    assert default(odd, DIRECTION.FILTER_BACKPROP) == ALGO.IM2COL
 
 
 def test_kernel_timing_argument_checks():
