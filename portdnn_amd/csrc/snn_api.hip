@@ -306,7 +306,7 @@ int default_algorithm(const snn_hip_conv2d_params& p, int direction) {
       algorithm_supports(p, direction, SNN_HIP_ALGO_WINOGRAD) &&
       conv2d_winograd_filter_backprop_supports(p) && p.channels % 32 == 0 &&
       p.features % 32 == 0 &&
-      static_cast<long long>(p.batch) * p.out_rows * p.out_cols >= 4096)
+      static_cast<long long>(p.batch) * p.out_rows * p.out_cols >= 1024)
     return SNN_HIP_ALGO_WINOGRAD;
   if (algorithm_supports(p, direction, SNN_HIP_ALGO_TILED))
     return SNN_HIP_ALGO_TILED;
