@@ -207,6 +207,29 @@ SNN_HIP_API int snn_hip_conv2d_filter_backprop_f16(
     const snn_hip_conv2d_params* params, int algorithm, void* workspace,
     size_t workspace_elems, void* stream);
 
+/* Run-to-run reproducibility.  The reference's kernels add every output's
+ * terms in one fixed order, so its results repeat bit for bit.  The entry
+ * points above do not always: where a launch would otherwise fill only part
+ * of the GPU they split a reduction across work-groups whose partial sums
+ * meet through float atomics -- the implicit-GEMM filter gradient (Im2col /
+ * Tiled / Direct-fallback tags) always, forward and input gradients of small
+ * problems (fewer than ~640 64x64 output tiles) and the fused Winograd
+ * kernel below 128 work units -- and the order of those additions, hence the
+ * last bits of the result, can change between runs.  The Winograd filter
+ * gradient and every launch without such a split are reproducible.
+ *
+ * snn_hip_conv2d_deterministic_f32 is the same operation as the three fp32
+ * entry points (`direction` is a snn_hip_direction) with a fixed order of
+ * additions: no reduction splits (small problems run on fewer work-groups),
+ * and a filter gradient outside the Winograd algorithm runs on the direct
+ * kernel, one lane per filter element.  Two calls with the same arguments
+ * return bit-identical results.  Workspace sizes are those of
+ * snn_hip_conv2d_workspace_size. */
+SNN_HIP_API int snn_hip_conv2d_deterministic_f32(
+    int direction, const float* input, const float* filter, float* output,
+    const snn_hip_conv2d_params* params, int algorithm, float* workspace,
+    size_t workspace_elems, void* stream);
+
 /* sycldnn::conv2d::query_workspace_size<ConvType>(params, selector)
  * (include/portdnn/conv2d/workspace_size.h:158-163) for an already selected
  * algorithm.  Sizes in elements. */

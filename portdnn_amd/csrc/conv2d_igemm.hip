@@ -1102,7 +1102,7 @@ void launch_tile(const float* src, const float* wgt, float* dst,
                  const Gather& g, size_t src_elems, size_t wgt_elems,
                  int splits, hipStream_t stream, int batches = 1,
                  bool accumulate = false,
-                 const ConvEpilogue* epilogue = nullptr) {
+                 const LaunchOptions* epilogue = nullptr) {
   // accumulate: add the product to what dst holds (atomic kernel, no zero
   // fill) instead of overwriting it.
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(g.m_total, BM));
@@ -1216,7 +1216,7 @@ constexpr int kMinChunksPerSplit = 8;
 template <bool B_K_INNER, bool STRIDED>
 void launch_auto(const float* src, const float* wgt, float* dst,
                  const Gather& g, size_t src_elems, size_t wgt_elems,
-                 hipStream_t stream, const ConvEpilogue* epilogue = nullptr) {
+                 hipStream_t stream, const LaunchOptions* epilogue = nullptr) {
   auto tiles = [&](int bm, int bn) {
     return static_cast<long>(ceil_div(g.m_total, bm)) * ceil_div(g.n_total, bn);
   };
@@ -1251,7 +1251,8 @@ void launch_auto(const float* src, const float* wgt, float* dst,
   // n_total % 4 == 0 is needed by the zero fill of the split path
   // (measured: 800 tiles run 5 % faster unsplit than in two halves plus the
   // zero fill, so a launch that nearly fills the slots is left alone)
-  if (t < kResidentSlots * 5 / 8 && g.n_total % 4 == 0) {
+  const bool deterministic = epilogue != nullptr && epilogue->deterministic;
+  if (t < kResidentSlots * 5 / 8 && g.n_total % 4 == 0 && !deterministic) {
     splits = static_cast<int>((kSplitUnits + t - 1) / t);
     splits = max(1, min(splits, n_chunks / kMinChunksPerSplit));
   }
@@ -1466,7 +1467,7 @@ bool batched_gemm_mfma_supports(int m, int k, int n, const void* a,
 int launch_batched_gemm_mfma_f32(const float* a, const float* b, float* c,
                                  int batches, int m, int k, int n,
                                  hipStream_t stream, bool transpose_b,
-                                 bool accumulate) {
+                                 bool accumulate, bool deterministic) {
   // C[z] (+)= A[z] (m x k) * op(B[z]): a 1x1 "convolution" over m pixels.  B
   // as k x n is the forward filter layout, B as n x k (transpose_b) the
   // K-contiguous layout of the input-gradient kernel.
@@ -1492,7 +1493,7 @@ int launch_batched_gemm_mfma_f32(const float* a, const float* b, float* c,
   // the zero fill of a split launch writes float4s
   const bool can_split =
       accumulate || (static_cast<size_t>(batches) * m * n) % 4 == 0;
-  if (tiles < kResidentSlots && can_split) {
+  if (tiles < kResidentSlots && can_split && !deterministic) {
     splits = static_cast<int>((kSplitUnits + tiles - 1) / tiles);
     splits = max(1, min(splits, n_chunks / kMinChunksPerSplit));
   }
@@ -1515,7 +1516,7 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
                             const snn_hip_conv2d_params& p,
                             hipStream_t stream, float* workspace,
                             size_t workspace_elems,
-                            const ConvEpilogue* epilogue) {
+                            const LaunchOptions* epilogue) {
   if (direction == SNN_HIP_INPUT_BACKPROP && p.channels < 16 &&
       p.features % kBK == 0 &&
       static_cast<size_t>(p.out_rows) * p.out_cols * p.window_rows *
@@ -1566,10 +1567,10 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
                               stream, epilogue);
   } else if (g.div_rows != 1 || g.div_cols != 1) {
     launch_auto<true, true>(input, filter, output, g, src_elems, wgt_elems,
-                            stream);
+                            stream, epilogue);
   } else {
     launch_auto<true, false>(input, filter, output, g, src_elems, wgt_elems,
-                             stream);
+                             stream, epilogue);
   }
   SNN_HIP_CHECK_LAUNCH();
   return SNN_HIP_OK;

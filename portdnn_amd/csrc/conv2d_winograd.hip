@@ -207,7 +207,7 @@ int launch_conv2d_winograd_f32(int direction, const float* input,
                                const float* filter, float* output,
                                const snn_hip_conv2d_params& p,
                                float* workspace, size_t workspace_elems,
-                               hipStream_t stream) {
+                               hipStream_t stream, bool deterministic) {
   const bool backprop = direction == SNN_HIP_INPUT_BACKPROP;
   WinoGeom g;
   g.in_rows = backprop ? p.out_rows : p.in_rows;
@@ -261,7 +261,8 @@ int launch_conv2d_winograd_f32(int direction, const float* input,
     if (vec_ok &&
         batched_gemm_mfma_supports(g.n_tiles, g.in_ch, g.out_ch, v, u, m)) {
       rc = launch_batched_gemm_mfma_f32(v, u, m, 16, g.n_tiles, g.in_ch,
-                                        g.out_ch, stream);
+                                        g.out_ch, stream, false, false,
+                                        deterministic);
     } else {
       rc = launch_matmul_f32(v, u, m, 16, g.n_tiles, g.in_ch, g.out_ch, false,
                              false, 0.f, stream);

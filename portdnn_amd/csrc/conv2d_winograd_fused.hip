@@ -424,7 +424,7 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
                                      const snn_hip_conv2d_params& p,
                                      float* workspace, size_t workspace_elems,
                                      hipStream_t stream,
-                                     const ConvEpilogue* epilogue) {
+                                     const LaunchOptions* epilogue) {
   const bool backprop = direction == SNN_HIP_INPUT_BACKPROP;
   FusedGeom g;
   g.in_rows = backprop ? p.out_rows : p.in_rows;
@@ -500,7 +500,8 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
   constexpr unsigned kTargetGroups = 512;
   constexpr int kMinChunks = 4;
   int splits = 1;
-  if (n_units < kFewUnits)
+  const bool deterministic = epilogue != nullptr && epilogue->deterministic;
+  if (n_units < kFewUnits && !deterministic)
     splits = static_cast<int>(ceil_div(kTargetGroups, n_units));
   splits = max(1, min(splits, n_chunks / kMinChunks));
   if (const char* tune = SNN_TUNING_ENV("SNN_HIP_WINO")) {

@@ -323,13 +323,13 @@ template <typename T>
 int launch_gemm_path(int direction, const T* input, const T* filter, T* output,
                      const snn_hip_conv2d_params& p, hipStream_t s,
                      T* workspace = nullptr, size_t workspace_elems = 0,
-                     const ConvEpilogue* epilogue = nullptr);
+                     const LaunchOptions* epilogue = nullptr);
 template <>
 int launch_gemm_path<_Float16>(int direction, const _Float16* input,
                                const _Float16* filter, _Float16* output,
                                const snn_hip_conv2d_params& p, hipStream_t s,
                                _Float16* workspace, size_t workspace_elems,
-                               const ConvEpilogue*) {
+                               const LaunchOptions*) {
   if (direction == SNN_HIP_FORWARD && conv2d_igemm_f16_supports(p) &&
       aligned16(input) && aligned16(filter) && aligned16(output))
     return launch_conv2d_igemm_f16(input, filter, output, p, workspace,
@@ -346,24 +346,30 @@ int launch_gemm_path<float>(int direction, const float* input,
                             const float* filter, float* output,
                             const snn_hip_conv2d_params& p, hipStream_t s,
                             float* workspace, size_t workspace_elems,
-                            const ConvEpilogue* epilogue) {
+                            const LaunchOptions* epilogue) {
+  // The implicit-GEMM filter gradient always meets its partial tiles through
+  // float atomics; a launch that must be reproducible takes the direct kernel
+  // (one lane per filter element, fixed order) instead.
+  const bool atomics_only = direction == SNN_HIP_FILTER_BACKPROP &&
+                            epilogue != nullptr && epilogue->deterministic;
   if (conv2d_igemm_supports(direction, p) && aligned16(input) &&
-      aligned16(filter) && aligned16(output))
+      aligned16(filter) && aligned16(output) && !atomics_only)
     return launch_conv2d_igemm_f32(direction, input, filter, output, p, s,
                                    workspace, workspace_elems, epilogue);
   return launch_conv2d_direct<float>(direction, input, filter, output, p, s);
 }
 
 // Winograd / WinogradLarge: F(2x2,3x3) for forward and input backprop of 3x3
-// stride-1 convolutions.  The filter gradient and the 1x3 / 3x1 windows the
-// selector also accepts are computed by the implicit-GEMM kernels (the result
-// is the same convolution; no Winograd tiling exists for them here), and so
-// is WinogradLarge's F(4x4,3x3), whose larger constants cost accuracy.
+// stride-1 convolutions and F(3x3,2x2) for their filter gradient.  The 1x3 /
+// 3x1 windows the selector also accepts, and shapes the Winograd kernels do
+// not take, are computed by the implicit-GEMM kernels (the result is the same
+// convolution); WinogradLarge runs the same kernels as Winograd, because the
+// larger constants of F(4x4,3x3) cost accuracy against the fp32 bar.
 template <typename T>
 int launch_winograd_path(int direction, const T* input, const T* filter,
                          T* output, const snn_hip_conv2d_params& p,
                          T* workspace, size_t workspace_elems, hipStream_t s,
-                         const ConvEpilogue* epilogue = nullptr) {
+                         const LaunchOptions* epilogue = nullptr) {
   return launch_gemm_path<T>(direction, input, filter, output, p, s);
 }
 template <>
@@ -371,7 +377,7 @@ int launch_winograd_path<float>(int direction, const float* input,
                                 const float* filter, float* output,
                                 const snn_hip_conv2d_params& p,
                                 float* workspace, size_t workspace_elems,
-                                hipStream_t s, const ConvEpilogue* epilogue) {
+                                hipStream_t s, const LaunchOptions* epilogue) {
   // SNN_HIP_WINO_UNFUSED is a development switch that forces the three-stage
   // chain on shapes the fused kernel would take.
   if (conv2d_winograd_fused_supports(direction, p) && aligned16(input) &&
@@ -381,8 +387,9 @@ int launch_winograd_path<float>(int direction, const float* input,
                                             p, workspace, workspace_elems, s,
                                             epilogue);
   if (conv2d_winograd_supports(direction, p))
-    return launch_conv2d_winograd_f32(direction, input, filter, output, p,
-                                      workspace, workspace_elems, s);
+    return launch_conv2d_winograd_f32(
+        direction, input, filter, output, p, workspace, workspace_elems, s,
+        epilogue != nullptr && epilogue->deterministic);
   if (direction == SNN_HIP_FILTER_BACKPROP &&
       conv2d_winograd_filter_backprop_supports(p) && aligned16(input) &&
       aligned16(filter) && aligned16(output) && aligned16(workspace))
@@ -396,7 +403,7 @@ template <typename T>
 int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
                     const snn_hip_conv2d_params* params, int algorithm,
                     T* workspace, size_t workspace_elems, void* stream,
-                    const ConvEpilogue* epilogue = nullptr);
+                    const LaunchOptions* epilogue = nullptr);
 
 // NCHW activations with an FCHW filter (the only filter layout portDNN
 // accepts with NCHW, include/portdnn/internal/conv2d/launch.h:86-88): the
@@ -459,7 +466,7 @@ template <typename T>
 int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
                     const snn_hip_conv2d_params* params, int algorithm,
                     T* workspace, size_t workspace_elems, void* stream,
-                    const ConvEpilogue* epilogue) {
+                    const LaunchOptions* epilogue) {
   if (params == nullptr) return SNN_HIP_INVALID_PARAMETER;
   const snn_hip_conv2d_params& p = *params;
   const int v = validate(p);
@@ -662,6 +669,20 @@ int snn_hip_conv2d_filter_backprop_f16(const void* input, const void* filter,
       static_cast<const _Float16*>(filter), static_cast<_Float16*>(output),
       params, algorithm, static_cast<_Float16*>(workspace), workspace_elems,
       stream);
+}
+
+int snn_hip_conv2d_deterministic_f32(int direction, const float* input,
+                                     const float* filter, float* output,
+                                     const snn_hip_conv2d_params* params,
+                                     int algorithm, float* workspace,
+                                     size_t workspace_elems, void* stream) {
+  if (direction < SNN_HIP_FORWARD || direction > SNN_HIP_FILTER_BACKPROP)
+    return SNN_HIP_INVALID_PARAMETER;
+  LaunchOptions options;
+  options.deterministic = true;
+  return conv2d_dispatch<float>(direction, input, filter, output, params,
+                                algorithm, workspace, workspace_elems, stream,
+                                &options);
 }
 
 int snn_hip_conv2d_workspace_size(const snn_hip_conv2d_params* params,
@@ -883,7 +904,7 @@ int snn_hip_conv2d_forward_bias_act_f32(
       activation != SNN_HIP_ACTIVATION_RELU)
     return SNN_HIP_INVALID_PARAMETER;
   bool applied = false;
-  ConvEpilogue epilogue;
+  LaunchOptions epilogue;
   epilogue.bias = bias;
   epilogue.relu = activation == SNN_HIP_ACTIVATION_RELU;
   epilogue.applied = &applied;

@@ -14,13 +14,17 @@ int launch_conv2d_direct(int direction, const T* input, const T* filter,
                          T* output, const snn_hip_conv2d_params& p,
                          hipStream_t stream);
 
-// Work a forward convolution may fold into its last stage: out = act(conv +
-// bias[feature]).  A launcher that applies it sets *applied; otherwise the
-// caller runs launch_bias_act_f32 over the finished output.
-struct ConvEpilogue {
+// Per-launch options handed down to the kernel launchers.
+//  * Work a forward convolution may fold into its last stage: out = act(conv +
+//    bias[feature]).  A launcher that applies it sets *applied; otherwise the
+//    caller runs launch_bias_act_f32 over the finished output.
+//  * deterministic: the launcher must not combine partial sums through float
+//    atomics (whose order varies from run to run): no reduction splits.
+struct LaunchOptions {
   const float* bias = nullptr;  // one value per feature, or none
   bool relu = false;
   bool* applied = nullptr;
+  bool deterministic = false;
   bool wanted() const { return bias != nullptr || relu; }
 };
 
@@ -33,7 +37,7 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
                             const snn_hip_conv2d_params& p, hipStream_t stream,
                             float* workspace = nullptr,
                             size_t workspace_elems = 0,
-                            const ConvEpilogue* epilogue = nullptr);
+                            const LaunchOptions* epilogue = nullptr);
 
 // Batched row-major GEMM C[z] = A[z] (m x k) * op(B[z]) on the same MFMA
 // kernel, op(B) = B (k x n) or B^T with B stored n x k; operands of
@@ -46,7 +50,8 @@ bool batched_gemm_mfma_supports(int m, int k, int n, const void* a,
 int launch_batched_gemm_mfma_f32(const float* a, const float* b, float* c,
                                  int batches, int m, int k, int n,
                                  hipStream_t stream, bool transpose_b = false,
-                                 bool accumulate = false);
+                                 bool accumulate = false,
+                                 bool deterministic = false);
 
 // Winograd F(2x2,3x3) convolution, forward and input backprop
 // (conv2d_winograd.hip).  `workspace` holds the three transform buffers.
@@ -55,7 +60,7 @@ int launch_conv2d_winograd_f32(int direction, const float* input,
                                const float* filter, float* output,
                                const snn_hip_conv2d_params& p,
                                float* workspace, size_t workspace_elems,
-                               hipStream_t stream);
+                               hipStream_t stream, bool deterministic = false);
 
 // The same convolution in one fused kernel (conv2d_winograd_fused.hip): needs
 // channel counts that are multiples of 16 (reduced) and 32 (produced), 16-byte
@@ -67,7 +72,7 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
                                      const snn_hip_conv2d_params& p,
                                      float* workspace, size_t workspace_elems,
                                      hipStream_t stream,
-                                     const ConvEpilogue* epilogue = nullptr);
+                                     const LaunchOptions* epilogue = nullptr);
 
 // Winograd F(3x3,2x2) filter gradient of a 3x3 stride-1 convolution in one
 // fused kernel (conv2d_winograd_filter.hip).  `workspace` receives one

@@ -131,6 +131,24 @@ def conv2d(inp, fil, p, direction=DIRECTION.FORWARD, algorithm=ALGO.DIRECT,
     return out
 
 
+def conv2d_deterministic(inp, fil, p, direction, algorithm, workspace=None,
+                         out=None):
+    """snn_hip_conv2d_deterministic_f32: fixed order of additions."""
+    n_in, n_fil, n_out = conv_sizes(p, direction)
+    assert inp.numel() == n_in and fil.numel() == n_fil
+    if out is None:
+        out = torch.empty(n_out, dtype=inp.dtype, device=inp.device)
+    if workspace is None:
+        _, rec = workspace_size(p, direction, algorithm)
+        if rec:
+            workspace = torch.empty(rec, dtype=inp.dtype, device=inp.device)
+    capi.check(capi.lib().snn_hip_conv2d_deterministic_f32(
+        direction, _ptr(inp), _ptr(fil), _ptr(out), ctypes.byref(p), algorithm,
+        _ptr(workspace), 0 if workspace is None else workspace.numel(),
+        _stream()))
+    return out
+
+
 def conv2d_bias_act(inp, fil, bias, p, algorithm, relu=True, workspace=None,
                     out=None):
     """snn_hip_conv2d_forward_bias_act_f32: act(conv(inp, fil) + bias)."""

@@ -231,6 +231,36 @@ def test_winograd_runs_with_exactly_the_queried_workspace(algo, batch,
             STATUS.INSUFFICIENT_WORKSPACE
 
 
+# ---- reproducible launches ----------------------------------------------------
+
+@pytest.mark.parametrize("case", [
+    # batch, size, channels, features, window, direction, algorithm
+    (2, 14, 256, 256, 3, DIRECTION.FORWARD, ALGO.IM2COL),        # would split
+    (2, 14, 256, 256, 3, DIRECTION.INPUT_BACKPROP, ALGO.IM2COL),
+    (1, 7, 512, 512, 3, DIRECTION.FORWARD, ALGO.WINOGRAD),       # < 128 units
+    (1, 7, 512, 512, 3, DIRECTION.INPUT_BACKPROP, ALGO.WINOGRAD),
+    (4, 28, 64, 64, 3, DIRECTION.FILTER_BACKPROP, ALGO.IM2COL),  # direct kernel
+    (8, 28, 128, 128, 3, DIRECTION.FILTER_BACKPROP, ALGO.WINOGRAD),
+    (2, 14, 256, 1024, 1, DIRECTION.FORWARD, ALGO.MATMUL),
+    (2, 20, 24, 40, 3, DIRECTION.FORWARD, ALGO.WINOGRAD),        # 3-stage chain
+])
+def test_deterministic_entry_point_repeats_bit_for_bit(case):
+    batch, size, ch, feats, window, direction, algo = case
+    p = ops.conv_params(batch, size, size, ch, feats, window, 1, window == 3)
+    rng = np.random.default_rng(3700 + size + direction + algo)
+    n_a, n_b, _ = ops.conv_sizes(p, direction)
+    a, b = uniform(rng, n_a), uniform(rng, n_b)
+    ref = ORACLE_FN[direction](a, b, oracle_params(p, feats), acc64=True)
+    da, db = dev(a), dev(b)
+    first = ops.conv2d_deterministic(da, db, p, direction, algo)
+    assert_close(first.cpu().numpy(), ref, ("deterministic", case))
+    for _ in range(4):
+        # other work in between changes the timing of the next launch
+        ops.conv2d(da, db, p, direction, algo)
+        again = ops.conv2d_deterministic(da, db, p, direction, algo)
+        assert torch.equal(first.view(torch.int32), again.view(torch.int32))
+
+
 # ---- half-precision kernels: ragged feature counts, unaligned workspace ------
 
 @pytest.mark.parametrize("n", [5, 10, 72])
