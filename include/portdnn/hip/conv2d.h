@@ -337,6 +337,32 @@ SNNStatus launch_forward_bias_activation(
       stream);
 }
 
+// Not in portDNN, whose kernels always add in one fixed order: the same
+// convolution as launch<float, ConvType> with run-to-run bit-identical
+// results (no reduction split across work-groups, whose partial sums would
+// meet through float atomics in varying order).  Slower for small problems
+// and for filter gradients outside the Winograd algorithm.
+template <typename T, typename ConvType, typename Backend>
+SNNStatus launch_deterministic(
+    typename Backend::template pointer_type<T const> input,
+    typename Backend::template pointer_type<T const> filter,
+    typename Backend::template pointer_type<T> output,
+    Conv2DParams const& params, Selector& selector, Backend& backend,
+    typename Backend::template pointer_type<T> workspace,
+    size_t workspace_size, const std::vector<hip::Event>& events = {}) {
+  static_assert(std::is_same<T, float>::value,
+                "launch_deterministic is provided for float");
+  const snn_hip_conv2d_params c = internal::to_c(params);
+  const Algorithm algo = selector.select<ConvType>(params);
+  hipStream_t stream = backend.get_stream();
+  hip::detail::wait_for(stream, events);
+  return hip::detail::finish(
+      snn_hip_conv2d_deterministic_f32(
+          internal::Direction<ConvType>::value, input, filter, output, &c,
+          static_cast<int>(algo), workspace, workspace_size, stream),
+      stream);
+}
+
 }  // namespace conv2d
 }  // namespace sycldnn
 

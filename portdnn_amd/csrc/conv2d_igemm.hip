@@ -57,28 +57,48 @@ typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
 constexpr unsigned kOob = 0x7FFFFFF0u;       // beyond any accepted tensor
 constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
 
-__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const float* p,
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* p,
                                                    unsigned bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p), 0, bytes,
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes,
                                            0x00020000);
 }
 __device__ inline float4 buffer_load4(__amdgpu_buffer_rsrc_t r, unsigned off) {
   const uint4v v = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
   return __builtin_bit_cast(float4, v);
 }
+// Four consecutive elements of storage type T at byte offset `off`, as floats
+// (half-precision tensors are multiplied on the fp32 matrix instructions, so
+// every product and sum is exactly what an f16 instruction with fp32
+// accumulation would give).
+template <typename T>
+__device__ inline float4 buffer_load4_as_float(__amdgpu_buffer_rsrc_t r,
+                                               unsigned off) {
+  if constexpr (sizeof(T) == 4) {
+    return buffer_load4(r, off);
+  } else {
+    typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+    typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
+    const uint2v v = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+    const half4 h = __builtin_bit_cast(half4, v);
+    return make_float4(static_cast<float>(h.x), static_cast<float>(h.y),
+                       static_cast<float>(h.z), static_cast<float>(h.w));
+  }
+}
 
 // SCALAR_A: the gathered tensor's channel count is not a multiple of 4 (e.g.
 // the 3-channel stem), so four consecutive reduction indices are not four
 // consecutive floats of one tap; each is located and loaded on its own.
 template <int BM, int BN, int WM, int WN, bool B_K_INNER, bool STRIDED,
-          bool ATOMIC, bool SCALAR_A = false>
+          bool ATOMIC, bool SCALAR_A = false, typename T = float>
 __global__ void __launch_bounds__(kThreads)
-    conv_igemm_kernel(const float* __restrict__ src,
-                      const float* __restrict__ wgt, float* __restrict__ dst,
-                      Gather g, unsigned src_bytes, unsigned wgt_bytes,
-                      unsigned n_tiles_n, unsigned n_tiles,
+    conv_igemm_kernel(const T* __restrict__ src, const T* __restrict__ wgt,
+                      T* __restrict__ dst, Gather g, unsigned src_bytes,
+                      unsigned wgt_bytes, unsigned n_tiles_n, unsigned n_tiles,
                       int chunks_per_split) {
   static_assert(WM * WN == 4, "four waves per work-group");
+  static_assert(sizeof(T) == 4 || (!ATOMIC && !SCALAR_A),
+                "half-precision tensors: plain stores, vector gather");
+  constexpr unsigned kEsz = sizeof(T);
   constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
   constexpr int TM = WTM / 32, TN = WTN / 32;  // MFMA blocks per wave
   static_assert(TM >= 1 && TN >= 1, "wave tile must hold a 32x32 block");
@@ -219,8 +239,8 @@ __global__ void __launch_bounds__(kThreads)
       ok = ok &
            (static_cast<unsigned>(iy) < static_cast<unsigned>(g.src_rows)) &
            (static_cast<unsigned>(ix) < static_cast<unsigned>(g.src_cols));
-      a_reg[i] = buffer_load4(src_rsrc,
-                              ok ? static_cast<unsigned>(off) * 4u : kOob);
+      a_reg[i] = buffer_load4_as_float<T>(
+          src_rsrc, ok ? static_cast<unsigned>(off) * kEsz : kOob);
     }
   };
   auto advance_a = [&]() {
@@ -252,7 +272,7 @@ __global__ void __launch_bounds__(kThreads)
           const int tap = q / g.src_ch;
           const int kk = q - tap * g.src_ch;
           off = static_cast<unsigned>((tap * g.n_total + col) * g.src_ch + kk) *
-                4u;
+                kEsz;
         }
       } else {
         // W[q][col], col contiguous; q >= k_total is past the end of the
@@ -260,9 +280,9 @@ __global__ void __launch_bounds__(kThreads)
         const int q = k0 + b_row0 + B_ROWS_PER_PASS * i;
         const int col = n0 + 4 * b_vec;
         if (col < g.n_total)
-          off = static_cast<unsigned>(q * g.n_total + col) * 4u;
+          off = static_cast<unsigned>(q * g.n_total + col) * kEsz;
       }
-      b_reg[i] = buffer_load4(wgt_rsrc, off);
+      b_reg[i] = buffer_load4_as_float<T>(wgt_rsrc, off);
     }
   };
   auto store_tiles = [&](int stage) {
@@ -324,11 +344,11 @@ __global__ void __launch_bounds__(kThreads)
       for (int v = 0; v < 16; ++v) {
         const int m = m0 + wave_m * WTM + 32 * i + 8 * (v >> 2) + row_l + (v & 3);
         if (m < g.m_total) {
-          float* o = dst + static_cast<size_t>(m) * g.n_total + col;
-          if (ATOMIC)
+          T* o = dst + static_cast<size_t>(m) * g.n_total + col;
+          if constexpr (ATOMIC)
             unsafeAtomicAdd(o, acc[i][j][v]);
           else
-            *o = acc[i][j][v];
+            *o = static_cast<T>(acc[i][j][v]);
         }
       }
     }
@@ -675,9 +695,10 @@ struct FilterBackpropGeom {
   int m_total;  // batch * out_rows * out_cols
 };
 
+template <typename T>
 __global__ void __launch_bounds__(kThreads)
-    conv_filter_backprop_kernel(const float* __restrict__ x,
-                                const float* __restrict__ dy,
+    conv_filter_backprop_kernel(const T* __restrict__ x,
+                                const T* __restrict__ dy,
                                 float* __restrict__ dw, FilterBackpropGeom g,
                                 unsigned x_bytes, unsigned dy_bytes,
                                 unsigned dw_bytes, int chunks_per_split) {
@@ -727,7 +748,8 @@ __global__ void __launch_bounds__(kThreads)
     x_off[i] = ((n * g.in_rows + iy[i]) * g.in_cols + o * g.stride_cols -
                 g.pad_cols + tap_c) * g.channels + c0 + 4 * vec;
     dy_off[i] = (n0 + 4 * vec < g.features)
-                    ? static_cast<unsigned>(m * g.features + n0 + 4 * vec) * 4u
+                    ? static_cast<unsigned>(m * g.features + n0 + 4 * vec) *
+                          static_cast<unsigned>(sizeof(T))
                     : kOob;
   }
   // element-offset deltas of the pixel walk
@@ -747,9 +769,11 @@ __global__ void __launch_bounds__(kThreads)
       const bool ok =
           (static_cast<unsigned>(iy[i]) < static_cast<unsigned>(g.in_rows)) &
           (static_cast<unsigned>(ix) < static_cast<unsigned>(g.in_cols));
-      a_reg[i] = buffer_load4(
-          x_rsrc, ok ? static_cast<unsigned>(x_off[i]) * 4u : kOob);
-      b_reg[i] = buffer_load4(dy_rsrc, dy_off[i]);
+      a_reg[i] = buffer_load4_as_float<T>(
+          x_rsrc, ok ? static_cast<unsigned>(x_off[i]) *
+                           static_cast<unsigned>(sizeof(T))
+                     : kOob);
+      b_reg[i] = buffer_load4_as_float<T>(dy_rsrc, dy_off[i]);
       // advance this row by one chunk (32 pixels)
       ox[i] += kBK;
       x_off[i] += kBK * step_px;
@@ -762,7 +786,8 @@ __global__ void __launch_bounds__(kThreads)
           x_off[i] += step_img;
         }
       }
-      if (dy_off[i] != kOob) dy_off[i] += kBK * g.features * 4u;
+      if (dy_off[i] != kOob)
+        dy_off[i] += kBK * g.features * static_cast<unsigned>(sizeof(T));
     }
   };
   float* const a_store = lds + row0 * (BM + kPad) + 4 * vec;
@@ -1425,11 +1450,176 @@ static int launch_filter_backprop(const float* x, const float* dy, float* dw,
                      dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
                      dim3(256), 0, stream, reinterpret_cast<float4*>(dw), n_vec);
   KernelTimer timer(stream);
-  hipLaunchKernelGGL(conv_filter_backprop_kernel, dim3(tiles, splits),
+  hipLaunchKernelGGL(conv_filter_backprop_kernel<float>, dim3(tiles, splits),
                      dim3(kThreads), 0, stream, x, dy, dw, g,
                      static_cast<unsigned>(x_elems * 4),
                      static_cast<unsigned>(dy_elems * 4),
                      static_cast<unsigned>(dw_elems * 4), per_split);
+  return SNN_HIP_OK;
+}
+
+namespace {
+
+__global__ void __launch_bounds__(256)
+    f32_to_f16_kernel(const float* __restrict__ in, _Float16* __restrict__ out,
+                      size_t n) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i < n) out[i] = static_cast<_Float16>(in[i]);
+}
+
+void fill_gather(const snn_hip_conv2d_params& p, int direction, Gather* g) {
+  g->batch = p.batch;
+  g->win_rows = p.window_rows;
+  g->win_cols = p.window_cols;
+  if (direction == SNN_HIP_FORWARD) {
+    g->p_rows = p.out_rows;  g->p_cols = p.out_cols;
+    g->src_rows = p.in_rows; g->src_cols = p.in_cols;
+    g->src_ch = p.channels;
+    g->step_rows = p.stride_rows; g->step_cols = p.stride_cols;
+    g->off_rows = -p.pad_rows;    g->off_cols = -p.pad_cols;
+    g->tap_sign = 1;
+    g->div_rows = g->div_cols = 1;
+    g->n_total = p.features;
+  } else {
+    g->p_rows = p.in_rows;    g->p_cols = p.in_cols;
+    g->src_rows = p.out_rows; g->src_cols = p.out_cols;
+    g->src_ch = p.features;
+    g->step_rows = g->step_cols = 1;
+    g->off_rows = p.pad_rows; g->off_cols = p.pad_cols;
+    g->tap_sign = -1;
+    g->div_rows = p.stride_rows; g->div_cols = p.stride_cols;
+    g->n_total = p.channels;
+  }
+  g->m_total = g->batch * g->p_rows * g->p_cols;
+  g->k_total = g->win_rows * g->win_cols * g->src_ch;
+  g->z_src = g->z_wgt = g->z_dst = 0;
+}
+
+}  // namespace
+
+// Half-precision filter gradient on the matrix cores: the fp32 kernel reads
+// binary16 operands (converted on the way into LDS, so every product and sum
+// is what an f16 matrix instruction with fp32 accumulation would give),
+// accumulates dW in an fp32 buffer -- the workspace when it holds 2 * R*S*C*K
+// halves, else a stream-ordered temporary -- and one pass rounds it to
+// binary16.
+bool conv2d_filter_backprop_f16_supports(const snn_hip_conv2d_params& p) {
+  const size_t x = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                   p.channels;
+  const size_t y = static_cast<size_t>(p.batch) * p.out_rows * p.out_cols *
+                   p.features;
+  return p.channels % 64 == 0 && p.features % 4 == 0 &&
+         max(x, y) * sizeof(_Float16) <= kMaxBufferBytes &&
+         static_cast<size_t>(p.window_rows) * p.window_cols * p.channels *
+                 p.features * sizeof(float) <= kMaxBufferBytes;
+}
+
+int launch_conv2d_filter_backprop_f16(const _Float16* x, const _Float16* dy,
+                                      _Float16* dw,
+                                      const snn_hip_conv2d_params& p,
+                                      _Float16* workspace,
+                                      size_t workspace_elems,
+                                      hipStream_t stream) {
+  FilterBackpropGeom g;
+  g.batch = p.batch; g.in_rows = p.in_rows; g.in_cols = p.in_cols;
+  g.channels = p.channels; g.out_rows = p.out_rows; g.out_cols = p.out_cols;
+  g.features = p.features; g.win_rows = p.window_rows;
+  g.win_cols = p.window_cols; g.stride_rows = p.stride_rows;
+  g.stride_cols = p.stride_cols; g.pad_rows = p.pad_rows;
+  g.pad_cols = p.pad_cols;
+  g.m_total = p.batch * p.out_rows * p.out_cols;
+  const size_t x_elems =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
+  const size_t dy_elems = static_cast<size_t>(g.m_total) * p.features;
+  const size_t dw_elems = static_cast<size_t>(p.window_rows) * p.window_cols *
+                          p.channels * p.features;
+  float* acc32 = reinterpret_cast<float*>(workspace);
+  bool temporary = false;
+  if (workspace == nullptr || workspace_elems < 2 * dw_elems ||
+      (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) {
+    void* ptr = nullptr;
+    if (hipMallocAsync(&ptr, dw_elems * sizeof(float), stream) != hipSuccess)
+      return SNN_HIP_ALLOCATION_PROBLEM;
+    acc32 = static_cast<float*>(ptr);
+    temporary = true;
+  }
+  const int tiles = (p.window_rows * p.window_cols * p.channels / 64) *
+                    ceil_div(p.features, 64);
+  const int n_chunks = ceil_div(g.m_total, kBK);
+  int splits = max(1, min(ceil_div(kSplitUnits, tiles),
+                          n_chunks / kMinChunksPerSplit));
+  const int per_split = ceil_div(n_chunks, splits);
+  splits = ceil_div(n_chunks, per_split);
+  const size_t n_vec = dw_elems / 4;
+  hipLaunchKernelGGL(zero_fill_kernel,
+                     dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
+                     dim3(256), 0, stream, reinterpret_cast<float4*>(acc32),
+                     n_vec);
+  {
+    KernelTimer timer(stream);
+    hipLaunchKernelGGL(conv_filter_backprop_kernel<_Float16>,
+                       dim3(tiles, splits), dim3(kThreads), 0, stream, x, dy,
+                       acc32, g, static_cast<unsigned>(x_elems * 2),
+                       static_cast<unsigned>(dy_elems * 2),
+                       static_cast<unsigned>(dw_elems * 4), per_split);
+  }
+  hipLaunchKernelGGL(f32_to_f16_kernel,
+                     dim3(static_cast<unsigned>(ceil_div(dw_elems, size_t{256}))),
+                     dim3(256), 0, stream, acc32, dw, dw_elems);
+  const hipError_t err = hipGetLastError();
+  if (temporary) (void)hipFreeAsync(acc32, stream);
+  if (err != hipSuccess) return report_hip_error(err, "f16 filter backprop");
+  return SNN_HIP_OK;
+}
+
+// Half-precision input gradient for the shapes the LDS-tile kernel does not
+// take (strides, channel counts that are not multiples of 64): the general
+// implicit-GEMM kernel reading binary16 operands, one work-group per 64 x 64
+// tile of dX and no reduction split, so every output is stored once.
+bool conv2d_input_backprop_general_f16_supports(
+    const snn_hip_conv2d_params& p) {
+  const size_t x = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                   p.channels;
+  const size_t y = static_cast<size_t>(p.batch) * p.out_rows * p.out_cols *
+                   p.features;
+  const size_t w = static_cast<size_t>(p.window_rows) * p.window_cols *
+                   p.channels * p.features;
+  return p.features % 4 == 0 &&
+         max(max(x, y), w) * sizeof(_Float16) <= kMaxBufferBytes;
+}
+
+int launch_conv2d_input_backprop_general_f16(const _Float16* dy,
+                                             const _Float16* filter,
+                                             _Float16* dx,
+                                             const snn_hip_conv2d_params& p,
+                                             hipStream_t stream) {
+  Gather g;
+  fill_gather(p, SNN_HIP_INPUT_BACKPROP, &g);
+  constexpr int BM = 64, BN = 64;
+  const unsigned tiles_m = static_cast<unsigned>(ceil_div(g.m_total, BM));
+  const unsigned tiles_n = static_cast<unsigned>(ceil_div(g.n_total, BN));
+  const unsigned n_tiles = tiles_m * tiles_n;
+  const int n_chunks = ceil_div(g.k_total, kBK);
+  constexpr size_t kLdsBytes =
+      2 * sizeof(float) * (k_inner_floats(BM) + k_inner_floats(BN));
+  const unsigned src_bytes = static_cast<unsigned>(
+      static_cast<size_t>(g.batch) * g.src_rows * g.src_cols * g.src_ch * 2);
+  const unsigned wgt_bytes = static_cast<unsigned>(
+      static_cast<size_t>(p.window_rows) * p.window_cols * p.channels *
+      p.features * 2);
+  KernelTimer timer(stream);
+  if (g.div_rows != 1 || g.div_cols != 1) {
+    hipLaunchKernelGGL(
+        (conv_igemm_kernel<BM, BN, 2, 2, true, true, false, false, _Float16>),
+        dim3(n_tiles, 1), dim3(kThreads), kLdsBytes, stream, dy, filter, dx, g,
+        src_bytes, wgt_bytes, tiles_n, n_tiles, n_chunks);
+  } else {
+    hipLaunchKernelGGL(
+        (conv_igemm_kernel<BM, BN, 2, 2, true, false, false, false, _Float16>),
+        dim3(n_tiles, 1), dim3(kThreads), kLdsBytes, stream, dy, filter, dx, g,
+        src_bytes, wgt_bytes, tiles_n, n_tiles, n_chunks);
+  }
+  SNN_HIP_CHECK_LAUNCH();
   return SNN_HIP_OK;
 }
 

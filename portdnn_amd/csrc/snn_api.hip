@@ -339,6 +339,16 @@ int launch_gemm_path<_Float16>(int direction, const _Float16* input,
       aligned16(filter) && aligned16(output))
     return launch_conv2d_input_backprop_f16(input, filter, output, p,
                                             workspace, workspace_elems, s);
+  if (direction == SNN_HIP_INPUT_BACKPROP &&
+      conv2d_input_backprop_general_f16_supports(p) && aligned16(input) &&
+      aligned16(filter))
+    return launch_conv2d_input_backprop_general_f16(input, filter, output, p,
+                                                    s);
+  if (direction == SNN_HIP_FILTER_BACKPROP &&
+      conv2d_filter_backprop_f16_supports(p) && aligned16(input) &&
+      aligned16(filter))
+    return launch_conv2d_filter_backprop_f16(input, filter, output, p,
+                                             workspace, workspace_elems, s);
   return launch_conv2d_direct<_Float16>(direction, input, filter, output, p, s);
 }
 template <>

@@ -103,6 +103,26 @@ int launch_conv2d_input_backprop_f16(const _Float16* dy,
                                      size_t workspace_elems,
                                      hipStream_t stream);
 
+// Half-precision gradients on the fp32 matrix instructions
+// (conv2d_igemm.hip): the filter gradient for channel counts in multiples of
+// 64 (fp32 accumulation buffer in the workspace when it holds twice the
+// filter's element count, else a stream-ordered temporary), and the input
+// gradient for the shapes launch_conv2d_input_backprop_f16 does not take.
+bool conv2d_filter_backprop_f16_supports(const snn_hip_conv2d_params& p);
+int launch_conv2d_filter_backprop_f16(const _Float16* x, const _Float16* dy,
+                                      _Float16* dw,
+                                      const snn_hip_conv2d_params& p,
+                                      _Float16* workspace,
+                                      size_t workspace_elems,
+                                      hipStream_t stream);
+bool conv2d_input_backprop_general_f16_supports(
+    const snn_hip_conv2d_params& p);
+int launch_conv2d_input_backprop_general_f16(const _Float16* dy,
+                                             const _Float16* filter,
+                                             _Float16* dx,
+                                             const snn_hip_conv2d_params& p,
+                                             hipStream_t stream);
+
 // Half-precision stride-1 forward convolution with the input tile resident
 // in LDS (conv2d_rowtile_f16.hip).  `packed` receives the filter in MFMA
 // operand order: window_rows * window_cols * channels * features halves,

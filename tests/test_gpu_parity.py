@@ -766,8 +766,10 @@ def test_f16_conv_forward_full_batch_sampled(size, ch, feats, window):
     (2, 9, 20, 128, 256, 1, 3, 1, True),    # 1 x 3 window
     (7, 5, 5, 256, 320, 1, 1, 1, False),    # 1x1: implicit-GEMM kernel
     (2, 28, 28, 128, 512, 1, 1, 1, False),  # 1x1, 128 x 128 tiles
-    (2, 17, 9, 128, 64, 3, 3, 2, True),     # stride 2: direct kernel
-    (2, 8, 8, 24, 40, 3, 3, 1, True),       # few channels: direct kernel
+    (2, 17, 9, 128, 64, 3, 3, 2, True),     # stride 2: general MFMA kernel
+    (2, 8, 8, 24, 40, 3, 3, 1, True),       # few channels: general MFMA kernel
+    (3, 31, 29, 64, 132, 3, 3, 2, False),   # stride 2, VALID, ragged tiles
+    (2, 16, 16, 6, 10, 3, 3, 2, True),      # features not x4: direct kernel
     (2, 9, 10, 64, 64, 2, 2, 1, True),      # even window: padding 0 before, 1 after
     (2, 12, 9, 64, 128, 4, 4, 1, True),     # even window: padding 1 before, 2 after
     (2, 10, 10, 64, 64, 2, 4, 1, False),    # VALID, rectangular even window
@@ -791,6 +793,39 @@ def test_f16_conv_input_backprop(shape):
         got = ops.conv2d(dev(dy, torch.float16), dev(w, torch.float16), p,
                          DIRECTION.INPUT_BACKPROP, algo).float().cpu().numpy()
         assert_close_f16(got, ref, ("f16 inbk", ALGO_NAME[algo], shape))
+
+
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, window, stride, same
+    (4, 56, 56, 64, 64, 3, 1, True),      # the four ResNet 3x3 layers
+    (4, 28, 28, 128, 128, 3, 1, True),
+    (4, 14, 14, 256, 256, 3, 1, True),
+    (4, 7, 7, 512, 512, 3, 1, True),
+    (4, 28, 28, 128, 512, 1, 1, False),   # 1x1 K = 4C
+    (3, 17, 9, 128, 72, 3, 2, True),      # stride 2, ragged feature tile
+    (2, 9, 9, 64, 200, 5, 1, False),      # VALID, 25 taps
+    (128, 28, 28, 128, 128, 3, 1, True),  # configuration 4's batch
+])
+def test_f16_conv_filter_backprop_on_matrix_cores(shape):
+    """Half-precision filter gradient (channel counts in multiples of 64: the
+    implicit-GEMM kernel reading binary16, fp32 accumulation) against the
+    oracle in double precision on the same half-rounded operands; with and
+    without a caller workspace for the fp32 accumulation buffer."""
+    batch, rows, cols, ch, feats, window, stride, same = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, window, stride, same)
+    rng = np.random.default_rng(782 + rows + feats)
+    n_x, n_dy, n_dw = ops.conv_sizes(p, DIRECTION.FILTER_BACKPROP)
+    x = uniform(rng, n_x).astype(np.float16)
+    dy = uniform(rng, n_dy).astype(np.float16)
+    ref = oracle.conv2d_filter_backprop(x.astype(np.float32),
+                                        dy.astype(np.float32),
+                                        oracle_params(p, feats), acc64=True)
+    dx_, ddy = dev(x, torch.float16), dev(dy, torch.float16)
+    for ws in (None, torch.empty(2 * n_dw, dtype=torch.float16,
+                                 device="cuda")):
+        got = ops.conv2d(dx_, ddy, p, DIRECTION.FILTER_BACKPROP, ALGO.IM2COL,
+                         workspace=ws).float().cpu().numpy()
+        assert_close_f16(got, ref, ("f16 filbk mfma", shape, ws is None))
 
 
 def test_f16_conv_filter_backprop():
