@@ -681,6 +681,203 @@ __global__ void __launch_bounds__(kThreads)
 }
 
 // ---------------------------------------------------------------------------
+// Plain rows: C[m][n] = sum_k A[m][k] * B[k][n] with A read row by row -- the
+// 1x1 stride-1 unpadded convolution (m = pixel, k = channel, n = feature) and
+// the row-major matmul.  The general kernels above spend one LDS fetch
+// instruction per matrix instruction on these shapes (the B operand, n
+// contiguous, is fetched word by word) and store the result one word per
+// lane; this kernel is built around 16-byte accesses on both sides:
+//
+//   * v_mfma_f32_16x16x4_f32: lane l supplies A[row l % 16][k = l / 16] and
+//     B[k = l / 16][column l % 16], the 16 x 16 result sits in four registers
+//     (row 4 (l / 16) + v, column l % 16);
+//   * A tile [64][32 + 4], k contiguous: one ds_read_b128 gives a lane the
+//     four k = 16 s + 4 (l / 16) + t, t = 0 .. 3, of its row;
+//   * B tile [32][128 + 4], n contiguous: for each of those k one ds_read_b128
+//     gives the lane B[k][4 (l % 16) .. + 3], which feeds FOUR matrix
+//     instructions whose column blocks interleave: instruction u computes the
+//     columns 4 i + u.  A lane therefore ends with four consecutive columns
+//     of each of its rows and stores them with one 16-byte store;
+//   * a wave owns 32 rows x 64 columns (2 x 4 blocks, 32 accumulators): per 16
+//     reduction steps 6 LDS fetches feed 32 matrix instructions;
+//   * a work-group is 2 x 2 waves on a 64 x 128 tile, 51 KiB of LDS in two
+//     stages (three work-groups per CU).
+//
+// Needs k % 32 == 0, n % 4 == 0 and 16-byte aligned operands.  EPI as above.
+constexpr int kRowsBM = 64, kRowsBN = 128;
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+// RK: reduction steps per LDS stage, 32 (51 KiB of LDS, three work-groups per
+// CU) or 16 (27 KiB, five per CU, twice the barriers).
+template <bool EPI, int RK>
+__global__ void __launch_bounds__(kThreads)
+    gemm_rows_kernel(const float* __restrict__ a_ptr,
+                     const float* __restrict__ b_ptr, float* __restrict__ c_ptr,
+                     int m_total, int k_total, int n_total, int z_a, int z_b,
+                     int z_c, unsigned n_tiles_n, unsigned n_tiles,
+                     const float* __restrict__ bias, int relu) {
+  constexpr int kRowsAFloats = kRowsBM * (RK + kPad);
+  constexpr int kRowsBFloats = RK * (kRowsBN + kPad);
+  constexpr int kRowsStage = kRowsAFloats + kRowsBFloats;
+  constexpr int A_VEC = RK / 4;                 // 16-byte pieces per A row
+  constexpr int A_ROWS = kThreads / A_VEC;      // A rows per copy pass
+  constexpr int A_PASSES = kRowsBM / A_ROWS;
+  constexpr int B_PASSES = RK / 8;
+  __shared__ __align__(16) float lds[2 * kRowsStage];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int r16 = lane & 15, g4 = lane >> 4;
+
+  a_ptr += static_cast<size_t>(blockIdx.z) * z_a;
+  b_ptr += static_cast<size_t>(blockIdx.z) * z_b;
+  c_ptr += static_cast<size_t>(blockIdx.z) * z_c;
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(
+      a_ptr, static_cast<unsigned>(static_cast<size_t>(m_total) * k_total * 4));
+  const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(
+      b_ptr, static_cast<unsigned>(static_cast<size_t>(k_total) * n_total * 4));
+  const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(
+      c_ptr, static_cast<unsigned>(static_cast<size_t>(m_total) * n_total * 4));
+
+  const unsigned tile = xcd_remap(blockIdx.x, n_tiles);
+  const int m0 = static_cast<int>(tile / n_tiles_n) * kRowsBM;
+  const int n0 = static_cast<int>(tile % n_tiles_n) * kRowsBN;
+
+  // global -> register -> LDS copies: A rows tid / A_VEC + A_ROWS i, 16 bytes
+  // at k quad tid % A_VEC; B rows tid / 32 + 8 i, 16 bytes at column quad
+  // tid % 32
+  unsigned a_off[A_PASSES], b_off[B_PASSES];
+#pragma unroll
+  for (int i = 0; i < A_PASSES; ++i) {
+    const int m = m0 + tid / A_VEC + A_ROWS * i;
+    a_off[i] = m < m_total
+                   ? static_cast<unsigned>(m * k_total + 4 * (tid % A_VEC)) * 4u
+                   : kOob;
+  }
+  {
+    const int col = n0 + 4 * (tid & 31);
+#pragma unroll
+    for (int i = 0; i < B_PASSES; ++i)
+      b_off[i] = col < n_total
+                     ? static_cast<unsigned>(((tid >> 5) + 8 * i) * n_total +
+                                             col) * 4u
+                     : kOob;
+  }
+  // One register set: the loads of chunk c + 1 are issued before chunk c is
+  // multiplied and written to the other LDS stage after it.  (A second set,
+  // loads two chunks ahead, measured 3 - 8 % slower: the extra registers cost
+  // more occupancy than the longer prefetch gains.)
+  float4 a_reg[A_PASSES], b_reg[B_PASSES];
+  const int n_chunks = k_total / RK;
+  auto load_global = [&](int chunk) {
+    const unsigned a_s = static_cast<unsigned>(chunk * RK) * 4u;
+    const unsigned b_s = static_cast<unsigned>(chunk * RK * n_total) * 4u;
+#pragma unroll
+    for (int i = 0; i < A_PASSES; ++i)
+      a_reg[i] = __builtin_bit_cast(
+          float4, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_off[i], a_s, 0));
+#pragma unroll
+    for (int i = 0; i < B_PASSES; ++i)
+      b_reg[i] = __builtin_bit_cast(
+          float4, __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_off[i], b_s, 0));
+  };
+  float* const a_store =
+      lds + (tid / A_VEC) * (RK + kPad) + 4 * (tid % A_VEC);
+  float* const b_store =
+      lds + kRowsAFloats + (tid >> 5) * (kRowsBN + kPad) + 4 * (tid & 31);
+  auto store_tiles = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < A_PASSES; ++i)
+      *reinterpret_cast<float4*>(a_store + stage * kRowsStage +
+                                 A_ROWS * i * (RK + kPad)) = a_reg[i];
+#pragma unroll
+    for (int i = 0; i < B_PASSES; ++i)
+      *reinterpret_cast<float4*>(b_store + stage * kRowsStage +
+                                 8 * i * (kRowsBN + kPad)) = b_reg[i];
+  };
+
+  float4v acc[2][4];
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc[rb][u] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  const float* const a_fetch =
+      lds + (32 * wm + r16) * (RK + kPad) + 4 * g4;
+  const float* const b_fetch =
+      lds + kRowsAFloats + (4 * g4) * (kRowsBN + kPad) + 64 * wn + 4 * r16;
+  auto compute = [&](int stage) {
+    const float* const a_tile = a_fetch + stage * kRowsStage;
+    const float* const b_tile = b_fetch + stage * kRowsStage;
+#pragma unroll
+    for (int s = 0; s < RK / 16; ++s) {
+      float4 a[2], b[4];
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb)
+        a[rb] = *reinterpret_cast<const float4*>(
+            a_tile + 16 * rb * (RK + kPad) + 16 * s);
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        b[t] = *reinterpret_cast<const float4*>(
+            b_tile + (16 * s + t) * (kRowsBN + kPad));
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            acc[rb][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                comp(a[rb], t), comp(b[t], u), acc[rb][u], 0, 0, 0);
+    }
+  };
+
+  load_global(0);
+  store_tiles(0);
+  __syncthreads();
+  for (int c = 0; c < n_chunks; ++c) {
+    const bool more = c + 1 < n_chunks;
+    if (more) load_global(c + 1);
+    compute(c & 1);
+    if (more) store_tiles((c + 1) & 1);
+    __syncthreads();
+  }
+
+  // lane holds C[m0 + 32 wm + 16 rb + 4 g4 + v][n0 + 64 wn + 4 r16 + u]
+  const int col = n0 + 64 * wn + 4 * r16;
+  float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (EPI) {
+    if (bias != nullptr && col < n_total)
+      bias4 = *reinterpret_cast<const float4*>(bias + col);
+  }
+  const unsigned row_bytes = static_cast<unsigned>(n_total) * 4u;
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb) {
+    const int row = m0 + 32 * wm + 16 * rb + 4 * g4;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      float4 out = make_float4(acc[rb][0][v], acc[rb][1][v], acc[rb][2][v],
+                               acc[rb][3][v]);
+      if (EPI) {
+        out = make_float4(out.x + bias4.x, out.y + bias4.y, out.z + bias4.z,
+                          out.w + bias4.w);
+        if (relu)
+          out = make_float4(fmaxf(out.x, 0.f), fmaxf(out.y, 0.f),
+                            fmaxf(out.z, 0.f), fmaxf(out.w, 0.f));
+      }
+      const unsigned off =
+          (row + v < m_total && col < n_total)
+              ? static_cast<unsigned>(row + v) * row_bytes +
+                    static_cast<unsigned>(col) * 4u
+              : kOob;
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, out),
+                                             c_rsrc, off, 0, 0);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Filter backprop: dW[q][k] = sum_m A[m][q] * dY[m][k], q = (r, s, c),
 // m = (n, oy, ox).  The reduction runs over every output pixel, so both
 // operands are read with the reduction index as the slow dimension and both
@@ -1238,6 +1435,72 @@ constexpr int kResidentSlots = 1024;  // 256 CUs x 4 work-groups of 64x64
 constexpr int kSplitUnits = 2048;
 constexpr int kMinChunksPerSplit = 8;
 
+// The plain-rows kernel: one work-group per 64 x 128 tile, `batches`
+// independent problems along blockIdx.z.  Stages of 32 reduction steps fit
+// three work-groups on a CU (768 on the GPU), stages of 16 five (1280) at
+// twice the barriers; the shorter stage is taken when it saves a round of
+// work-groups.
+template <bool EPI, int RK>
+void launch_gemm_rows_as(const float* a, const float* b, float* c, int m,
+                         int k, int n, int batches, int z_a, int z_b, int z_c,
+                         unsigned tiles_n, unsigned n_tiles, const float* bias,
+                         int relu, hipStream_t stream) {
+  hipLaunchKernelGGL((gemm_rows_kernel<EPI, RK>),
+                     dim3(n_tiles, 1, static_cast<unsigned>(batches)),
+                     dim3(kThreads), 0, stream, a, b, c, m, k, n, z_a, z_b, z_c,
+                     tiles_n, n_tiles, bias, relu);
+}
+
+void launch_gemm_rows(const float* a, const float* b, float* c, int m, int k,
+                      int n, int batches, int z_a, int z_b, int z_c,
+                      hipStream_t stream, const LaunchOptions* epilogue) {
+  const unsigned tiles_m = static_cast<unsigned>(ceil_div(m, kRowsBM));
+  const unsigned tiles_n = static_cast<unsigned>(ceil_div(n, kRowsBN));
+  const unsigned n_tiles = tiles_m * tiles_n;
+  const long groups = static_cast<long>(n_tiles) * batches;
+  bool short_stage = (groups + 1279) / 1280 < (groups + 767) / 768;
+  if (const char* tune = SNN_TUNING_ENV("SNN_HIP_GEMM_ROWS_RK")) {
+    if (tune[0] != 0) short_stage = std::atoi(tune) == 16;
+  }
+  KernelTimer timer(stream);
+  // the bias vector is read 16 bytes at a time
+  const bool fuse = epilogue != nullptr && epilogue->wanted() && batches == 1 &&
+                    (epilogue->bias == nullptr ||
+                     (reinterpret_cast<uintptr_t>(epilogue->bias) & 15u) == 0);
+  const float* bias = fuse ? epilogue->bias : nullptr;
+  const int relu = fuse && epilogue->relu ? 1 : 0;
+  if (fuse) {
+    if (short_stage)
+      launch_gemm_rows_as<true, 16>(a, b, c, m, k, n, batches, z_a, z_b, z_c,
+                                    tiles_n, n_tiles, bias, relu, stream);
+    else
+      launch_gemm_rows_as<true, 32>(a, b, c, m, k, n, batches, z_a, z_b, z_c,
+                                    tiles_n, n_tiles, bias, relu, stream);
+    if (epilogue->applied != nullptr) *epilogue->applied = true;
+  } else {
+    if (short_stage)
+      launch_gemm_rows_as<false, 16>(a, b, c, m, k, n, batches, z_a, z_b, z_c,
+                                     tiles_n, n_tiles, bias, relu, stream);
+    else
+      launch_gemm_rows_as<false, 32>(a, b, c, m, k, n, batches, z_a, z_b, z_c,
+                                     tiles_n, n_tiles, bias, relu, stream);
+  }
+}
+
+// Shapes the plain-rows kernel takes and is the better choice for: rows read
+// as they are, k in whole chunks, 16-byte columns, and enough 64 x 128 tiles
+// to give every CU a work-group (smaller problems keep the 64 x 64 tiles and
+// the reduction split of the general kernel).
+constexpr long kRowsMinTiles = 256;
+bool gemm_rows_wanted(int m, int k, int n, int batches) {
+  static const char* tune = SNN_TUNING_ENV("SNN_HIP_GEMM_ROWS");
+  if (tune != nullptr && tune[0] == '0') return false;
+  const long tiles = static_cast<long>(ceil_div(m, kRowsBM)) *
+                     ceil_div(n, kRowsBN) * batches;
+  const long min_tiles = (tune != nullptr && tune[0] == '1') ? 1 : kRowsMinTiles;
+  return k % kBK == 0 && n % 4 == 0 && tiles >= min_tiles;
+}
+
 template <bool B_K_INNER, bool STRIDED>
 void launch_auto(const float* src, const float* wgt, float* dst,
                  const Gather& g, size_t src_elems, size_t wgt_elems,
@@ -1246,6 +1509,17 @@ void launch_auto(const float* src, const float* wgt, float* dst,
     return static_cast<long>(ceil_div(g.m_total, bm)) * ceil_div(g.n_total, bn);
   };
   const int n_chunks = ceil_div(g.k_total, kBK);
+  if constexpr (!B_K_INNER && !STRIDED) {
+    const bool plain_rows = g.win_rows == 1 && g.win_cols == 1 &&
+                            g.step_rows == 1 && g.step_cols == 1 &&
+                            g.off_rows == 0 && g.off_cols == 0 &&
+                            g.src_rows == g.p_rows && g.src_cols == g.p_cols;
+    if (plain_rows && gemm_rows_wanted(g.m_total, g.k_total, g.n_total, 1)) {
+      launch_gemm_rows(src, wgt, dst, g.m_total, g.k_total, g.n_total, 1, 0, 0,
+                       0, stream, epilogue);
+      return;
+    }
+  }
   // Developer override for tuning runs: SNN_HIP_IGEMM="<tile>,<splits>" with
   // tile 0 = 128x128, 1 = 128x64, 2 = 64x64.
   static const char* tune = SNN_TUNING_ENV("SNN_HIP_IGEMM");
@@ -1686,6 +1960,12 @@ int launch_batched_gemm_mfma_f32(const float* a, const float* b, float* c,
   if (tiles < kResidentSlots && can_split && !deterministic) {
     splits = static_cast<int>((kSplitUnits + tiles - 1) / tiles);
     splits = max(1, min(splits, n_chunks / kMinChunksPerSplit));
+  }
+  if (!transpose_b && !accumulate && gemm_rows_wanted(m, k, n, batches)) {
+    launch_gemm_rows(a, b, c, m, k, n, batches, m * k, k * n, m * n, stream,
+                     nullptr);
+    SNN_HIP_CHECK_LAUNCH();
+    return SNN_HIP_OK;
   }
   if (transpose_b)
     launch_tile<64, 64, 2, 2, true, false>(a, b, c, g,
