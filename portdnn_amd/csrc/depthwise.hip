@@ -98,6 +98,11 @@ __global__ void __launch_bounds__(256)
 typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
 typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
 constexpr unsigned kOobOffset = 0x7FFFFFF0u;
+// Cache policy bits of the input loads (0 = default; a build-time switch for
+// experiments, e.g. -DSNN_MEM_LOAD_AUX=2 for streaming loads).
+#ifndef SNN_MEM_LOAD_AUX
+#define SNN_MEM_LOAD_AUX 0
+#endif
 // Output is written once and not re-read by the kernel: stream it (slc).
 constexpr int kStoreAux = 2;
 
@@ -114,7 +119,7 @@ struct BufVec4<float> {
   __device__ static void load(__amdgpu_buffer_rsrc_t r, unsigned off,
                               float (&v)[4]) {
     const float4 t = __builtin_bit_cast(
-        float4, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0));
+        float4, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, SNN_MEM_LOAD_AUX));
     v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
   }
   __device__ static void store(__amdgpu_buffer_rsrc_t r, unsigned off,
@@ -130,7 +135,7 @@ struct BufVec4<_Float16> {
   __device__ static void load(__amdgpu_buffer_rsrc_t r, unsigned off,
                               float (&v)[4]) {
     const half4 t = __builtin_bit_cast(
-        half4, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0));
+        half4, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, SNN_MEM_LOAD_AUX));
     v[0] = static_cast<float>(t.x); v[1] = static_cast<float>(t.y);
     v[2] = static_cast<float>(t.z); v[3] = static_cast<float>(t.w);
   }
@@ -154,7 +159,7 @@ struct BufVecN<_Float16, 8> {
   __device__ static void load(__amdgpu_buffer_rsrc_t r, unsigned off,
                               float (&v)[8]) {
     const half8 t = __builtin_bit_cast(
-        half8, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0));
+        half8, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, SNN_MEM_LOAD_AUX));
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = static_cast<float>(t[i]);
   }

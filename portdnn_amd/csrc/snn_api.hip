@@ -267,9 +267,13 @@ int workspace_size(const snn_hip_conv2d_params& p, int direction,
   switch (algorithm) {
     case SNN_HIP_ALGO_WINOGRAD:
     case SNN_HIP_ALGO_WINOGRAD_LARGE:
-      // (1x3 / 3x1 windows are computed by the implicit-GEMM kernel too)
       if (!filbk && p.window_rows == 3 && p.window_cols == 3) {
         winograd_workspace(p, direction, 2, 2, 3, 3, required, recommended);
+      } else if (algorithm == SNN_HIP_ALGO_WINOGRAD &&
+                 conv2d_winograd_1d_supports(direction, p)) {
+        // 1x3 / 3x1: F(2,3) along the window's axis, four planes
+        *required = conv2d_winograd_1d_workspace(direction, p, 1);
+        *recommended = conv2d_winograd_1d_workspace(direction, p, p.batch);
       } else if (filbk && conv2d_winograd_filter_backprop_supports(p)) {
         *required = conv2d_winograd_filter_backprop_workspace(p);
         *recommended = *required;
@@ -370,11 +374,13 @@ int launch_gemm_path<float>(int direction, const float* input,
 }
 
 // Winograd / WinogradLarge: F(2x2,3x3) for forward and input backprop of 3x3
-// stride-1 convolutions and F(3x3,2x2) for their filter gradient.  The 1x3 /
-// 3x1 windows the selector also accepts, and shapes the Winograd kernels do
-// not take, are computed by the implicit-GEMM kernels (the result is the same
-// convolution); WinogradLarge runs the same kernels as Winograd, because the
-// larger constants of F(4x4,3x3) cost accuracy against the fp32 bar.
+// stride-1 convolutions and F(3x3,2x2) for their filter gradient; F(2,3)
+// along the window's axis for the 1x3 / 3x1 windows the selector also accepts
+// (forward and input backprop; their filter gradient, a reduction over every
+// tile with 3 results per (channel, feature), gains nothing over the implicit
+// GEMM and runs there, as do shapes the Winograd kernels do not take).
+// WinogradLarge runs the same kernels as Winograd, because the larger
+// constants of F(4x4,3x3) cost accuracy against the fp32 bar.
 template <typename T>
 int launch_winograd_path(int direction, const T* input, const T* filter,
                          T* output, const snn_hip_conv2d_params& p,
@@ -398,6 +404,10 @@ int launch_winograd_path<float>(int direction, const float* input,
                                             epilogue);
   if (conv2d_winograd_supports(direction, p))
     return launch_conv2d_winograd_f32(
+        direction, input, filter, output, p, workspace, workspace_elems, s,
+        epilogue != nullptr && epilogue->deterministic);
+  if (conv2d_winograd_1d_supports(direction, p) && aligned16(workspace))
+    return launch_conv2d_winograd_1d_f32(
         direction, input, filter, output, p, workspace, workspace_elems, s,
         epilogue != nullptr && epilogue->deterministic);
   if (direction == SNN_HIP_FILTER_BACKPROP &&

@@ -62,6 +62,19 @@ int launch_conv2d_winograd_f32(int direction, const float* input,
                                float* workspace, size_t workspace_elems,
                                hipStream_t stream, bool deterministic = false);
 
+// One-dimensional Winograd F(2,3) for 1x3 / 3x1 stride-1 windows, forward and
+// input backprop (conv2d_winograd_1d.hip).  `..._workspace` is the element
+// count needed to run `images` images per pass.
+bool conv2d_winograd_1d_supports(int direction, const snn_hip_conv2d_params& p);
+size_t conv2d_winograd_1d_workspace(int direction,
+                                    const snn_hip_conv2d_params& p, int images);
+int launch_conv2d_winograd_1d_f32(int direction, const float* input,
+                                  const float* filter, float* output,
+                                  const snn_hip_conv2d_params& p,
+                                  float* workspace, size_t workspace_elems,
+                                  hipStream_t stream,
+                                  bool deterministic = false);
+
 // The same convolution in one fused kernel (conv2d_winograd_fused.hip): needs
 // channel counts that are multiples of 16 (reduced) and 32 (produced), 16-byte
 // aligned pointers and only the transformed-filter part of the workspace.

@@ -176,6 +176,38 @@ def test_winograd_fused_shapes(shape, direction):
     conv_case(p, direction, [ALGO.WINOGRAD], seed=1300 + rows + ch)
 
 
+@pytest.mark.parametrize("direction", [DIRECTION.FORWARD,
+                                       DIRECTION.INPUT_BACKPROP])
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, win_rows, win_cols, same
+    (3, 9, 20, 64, 96, 1, 3, True),     # along columns, MFMA GEMMs
+    (3, 20, 9, 64, 96, 3, 1, True),     # along rows
+    (2, 7, 13, 32, 64, 1, 3, False),    # VALID, odd output length
+    (2, 13, 7, 32, 64, 3, 1, False),
+    (4, 6, 11, 5, 7, 1, 3, True),       # channel counts off the MFMA path
+    (4, 11, 6, 5, 7, 3, 1, True),
+])
+def test_winograd_one_dimensional_windows(shape, direction):
+    """F(2,3) along the window's axis for 1x3 / 3x1 windows, with the
+    recommended workspace (all images in one pass) and with the required one
+    (one image per pass)."""
+    batch, rows, cols, ch, feats, wr, wc, same = shape
+    p = ops.add_padding_to(ops.ConvParams(
+        channels=ch, features=feats, batch=batch, in_rows=rows, in_cols=cols,
+        window_rows=wr, window_cols=wc, stride_rows=1, stride_cols=1), same)
+    rng = np.random.default_rng(1360 + rows * cols + ch)
+    n_a, n_b, n_out = ops.conv_sizes(p, direction)
+    a, b = uniform(rng, n_a), uniform(rng, n_b)
+    ref = ORACLE_FN[direction](a, b, oracle_params(p, feats), acc64=True)
+    required, recommended = ops.workspace_size(p, direction, ALGO.WINOGRAD)
+    assert 0 < required < recommended
+    for elems in (recommended, required):
+        ws = torch.empty(elems, dtype=torch.float32, device="cuda")
+        got = ops.conv2d(dev(a), dev(b), p, direction, ALGO.WINOGRAD,
+                         workspace=ws).cpu().numpy()
+        assert_close(got, ref, ("winograd 1-D", shape, direction, elems))
+
+
 @pytest.mark.parametrize("shape", [
     # batch, rows, cols, channels, features, same
     (3, 13, 11, 32, 64, True),    # odd sizes: clipped dY tiles on both edges
