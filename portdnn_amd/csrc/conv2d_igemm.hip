@@ -1490,7 +1490,10 @@ void launch_gemm_rows(const float* a, const float* b, float* c, int m, int k,
 // Shapes the plain-rows kernel takes and is the better choice for: rows read
 // as they are, k in whole chunks, 16-byte columns, and enough 64 x 128 tiles
 // to give every CU a work-group (smaller problems keep the 64 x 64 tiles and
-// the reduction split of the general kernel).
+// the reduction split of the general kernel).  (The same kernel with the
+// im2col gather of conv_igemm_fast_kernel in front was measured on the 3x3
+// ResNet layers: within 3 % of that kernel either way, so convolutions with a
+// window keep the general kernel.)
 constexpr long kRowsMinTiles = 256;
 bool gemm_rows_wanted(int m, int k, int n, int batches) {
   static const char* tune = SNN_TUNING_ENV("SNN_HIP_GEMM_ROWS");
@@ -1498,7 +1501,11 @@ bool gemm_rows_wanted(int m, int k, int n, int batches) {
   const long tiles = static_cast<long>(ceil_div(m, kRowsBM)) *
                      ceil_div(n, kRowsBN) * batches;
   const long min_tiles = (tune != nullptr && tune[0] == '1') ? 1 : kRowsMinTiles;
-  return k % kBK == 0 && n % 4 == 0 && tiles >= min_tiles;
+  // columns past n in the last 128-wide tile are computed and dropped: at
+  // most a fifth of the work
+  const int n_padded = ceil_div(n, kRowsBN) * kRowsBN;
+  return k % kBK == 0 && n % 4 == 0 && tiles >= min_tiles &&
+         5 * (n_padded - n) <= n_padded;
 }
 
 template <bool B_K_INNER, bool STRIDED>
