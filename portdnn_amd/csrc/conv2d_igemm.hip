@@ -703,32 +703,61 @@ __global__ void __launch_bounds__(kThreads)
 //   * a work-group is 2 x 2 waves on a 64 x 128 tile, 51 KiB of LDS in two
 //     stages (three work-groups per CU).
 //
+//   * BM = 112 is the second tiling: 7 blocks of 16 rows, the four waves side
+//     by side on 32 columns each (8-byte B fetches feeding two interleaved
+//     column blocks, 56 accumulators, 8-byte stores).  The ResNet layers have
+//     49 * 2^k rows; 112-row tiles divide them into counts that spread evenly
+//     over the 256 CUs where 64-row tiles leave a quarter of the CUs one tile
+//     more than the rest (784 tiles: 3.06 per CU).
+//
 // Needs k % 32 == 0, n % 4 == 0 and 16-byte aligned operands.  EPI as above.
-constexpr int kRowsBM = 64, kRowsBN = 128;
+constexpr int kRowsBN = 128;
 
 typedef float float4v __attribute__((ext_vector_type(4)));
 
-// RK: reduction steps per LDS stage, 32 (51 KiB of LDS, three work-groups per
-// CU) or 16 (27 KiB, five per CU, twice the barriers).
-template <bool EPI, int RK>
+template <int U>
+struct RowVec;
+template <>
+struct RowVec<4> {
+  using type = float4;
+  __device__ static float get(const float4& v, int u) { return comp(v, u); }
+};
+template <>
+struct RowVec<2> {
+  using type = float2;
+  __device__ static float get(const float2& v, int u) {
+    return u == 0 ? v.x : v.y;
+  }
+};
+
+// RK: reduction steps per LDS stage, 32 or 16 (half the LDS, more work-groups
+// per CU, twice the barriers).  BM: 64 (2 x 2 waves of 32 x 64) or 112 (1 x 4
+// waves of 112 x 32).
+template <bool EPI, int RK, int BM>
 __global__ void __launch_bounds__(kThreads)
     gemm_rows_kernel(const float* __restrict__ a_ptr,
                      const float* __restrict__ b_ptr, float* __restrict__ c_ptr,
                      int m_total, int k_total, int n_total, int z_a, int z_b,
                      int z_c, unsigned n_tiles_n, unsigned n_tiles,
                      const float* __restrict__ bias, int relu) {
-  constexpr int kRowsAFloats = kRowsBM * (RK + kPad);
+  static_assert(BM == 64 || BM == 112, "tilings built: 64 and 112 rows");
+  constexpr int WN = BM == 64 ? 2 : 4;       // waves along n
+  constexpr int RB = BM == 64 ? 2 : 7;       // 16-row blocks per wave
+  constexpr int U = kRowsBN / WN / 16;       // interleaved column blocks: 4 / 2
+  constexpr int A_LDS_ROWS = BM == 64 ? 64 : 128;  // copy passes of 32+ rows
+  constexpr int kRowsAFloats = A_LDS_ROWS * (RK + kPad);
   constexpr int kRowsBFloats = RK * (kRowsBN + kPad);
   constexpr int kRowsStage = kRowsAFloats + kRowsBFloats;
   constexpr int A_VEC = RK / 4;                 // 16-byte pieces per A row
   constexpr int A_ROWS = kThreads / A_VEC;      // A rows per copy pass
-  constexpr int A_PASSES = kRowsBM / A_ROWS;
+  constexpr int A_PASSES = A_LDS_ROWS / A_ROWS;
   constexpr int B_PASSES = RK / 8;
+  using BVec = typename RowVec<U>::type;
   __shared__ __align__(16) float lds[2 * kRowsStage];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
   const int r16 = lane & 15, g4 = lane >> 4;
 
   a_ptr += static_cast<size_t>(blockIdx.z) * z_a;
@@ -742,17 +771,18 @@ __global__ void __launch_bounds__(kThreads)
       c_ptr, static_cast<unsigned>(static_cast<size_t>(m_total) * n_total * 4));
 
   const unsigned tile = xcd_remap(blockIdx.x, n_tiles);
-  const int m0 = static_cast<int>(tile / n_tiles_n) * kRowsBM;
+  const int m0 = static_cast<int>(tile / n_tiles_n) * BM;
   const int n0 = static_cast<int>(tile % n_tiles_n) * kRowsBN;
 
   // global -> register -> LDS copies: A rows tid / A_VEC + A_ROWS i, 16 bytes
-  // at k quad tid % A_VEC; B rows tid / 32 + 8 i, 16 bytes at column quad
-  // tid % 32
+  // at k quad tid % A_VEC (rows past the tile or the matrix read zeros); B
+  // rows tid / 32 + 8 i, 16 bytes at column quad tid % 32
   unsigned a_off[A_PASSES], b_off[B_PASSES];
 #pragma unroll
   for (int i = 0; i < A_PASSES; ++i) {
-    const int m = m0 + tid / A_VEC + A_ROWS * i;
-    a_off[i] = m < m_total
+    const int row = tid / A_VEC + A_ROWS * i;
+    const int m = m0 + row;
+    a_off[i] = (row < BM && m < m_total)
                    ? static_cast<unsigned>(m * k_total + 4 * (tid % A_VEC)) * 4u
                    : kOob;
   }
@@ -798,38 +828,40 @@ __global__ void __launch_bounds__(kThreads)
                                  8 * i * (kRowsBN + kPad)) = b_reg[i];
   };
 
-  float4v acc[2][4];
+  float4v acc[RB][U];
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb)
+  for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-    for (int u = 0; u < 4; ++u) acc[rb][u] = float4v{0.f, 0.f, 0.f, 0.f};
+    for (int u = 0; u < U; ++u) acc[rb][u] = float4v{0.f, 0.f, 0.f, 0.f};
 
   const float* const a_fetch =
-      lds + (32 * wm + r16) * (RK + kPad) + 4 * g4;
-  const float* const b_fetch =
-      lds + kRowsAFloats + (4 * g4) * (kRowsBN + kPad) + 64 * wn + 4 * r16;
+      lds + (16 * RB * wm + r16) * (RK + kPad) + 4 * g4;
+  const float* const b_fetch = lds + kRowsAFloats +
+                               (4 * g4) * (kRowsBN + kPad) +
+                               (kRowsBN / WN) * wn + U * r16;
   auto compute = [&](int stage) {
     const float* const a_tile = a_fetch + stage * kRowsStage;
     const float* const b_tile = b_fetch + stage * kRowsStage;
 #pragma unroll
     for (int s = 0; s < RK / 16; ++s) {
-      float4 a[2], b[4];
+      float4 a[RB];
+      BVec b[4];
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb)
+      for (int rb = 0; rb < RB; ++rb)
         a[rb] = *reinterpret_cast<const float4*>(
             a_tile + 16 * rb * (RK + kPad) + 16 * s);
 #pragma unroll
       for (int t = 0; t < 4; ++t)
-        b[t] = *reinterpret_cast<const float4*>(
+        b[t] = *reinterpret_cast<const BVec*>(
             b_tile + (16 * s + t) * (kRowsBN + kPad));
 #pragma unroll
       for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
+        for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-          for (int u = 0; u < 4; ++u)
+          for (int u = 0; u < U; ++u)
             acc[rb][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                comp(a[rb], t), comp(b[t], u), acc[rb][u], 0, 0, 0);
+                comp(a[rb], t), RowVec<U>::get(b[t], u), acc[rb][u], 0, 0, 0);
     }
   };
 
@@ -844,35 +876,49 @@ __global__ void __launch_bounds__(kThreads)
     __syncthreads();
   }
 
-  // lane holds C[m0 + 32 wm + 16 rb + 4 g4 + v][n0 + 64 wn + 4 r16 + u]
-  const int col = n0 + 64 * wn + 4 * r16;
-  float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  // lane holds C[m0 + 16 RB wm + 16 rb + 4 g4 + v][col + u], u = 0 .. U - 1
+  const int col = n0 + (kRowsBN / WN) * wn + U * r16;
+  float bias_u[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) bias_u[u] = 0.f;
   if (EPI) {
-    if (bias != nullptr && col < n_total)
-      bias4 = *reinterpret_cast<const float4*>(bias + col);
+    if (bias != nullptr && col < n_total) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) bias_u[u] = bias[col + u];
+    }
   }
   const unsigned row_bytes = static_cast<unsigned>(n_total) * 4u;
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
-    const int row = m0 + 32 * wm + 16 * rb + 4 * g4;
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row_l = 16 * RB * wm + 16 * rb + 4 * g4;  // row inside the tile
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      float4 out = make_float4(acc[rb][0][v], acc[rb][1][v], acc[rb][2][v],
-                               acc[rb][3][v]);
-      if (EPI) {
-        out = make_float4(out.x + bias4.x, out.y + bias4.y, out.z + bias4.z,
-                          out.w + bias4.w);
-        if (relu)
-          out = make_float4(fmaxf(out.x, 0.f), fmaxf(out.y, 0.f),
-                            fmaxf(out.z, 0.f), fmaxf(out.w, 0.f));
+      float out[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        out[u] = acc[rb][u][v];
+        if (EPI) {
+          out[u] += bias_u[u];
+          if (relu) out[u] = fmaxf(out[u], 0.f);
+        }
       }
+      const int row = m0 + row_l + v;
       const unsigned off =
-          (row + v < m_total && col < n_total)
-              ? static_cast<unsigned>(row + v) * row_bytes +
+          (row_l + v < BM && row < m_total && col < n_total)
+              ? static_cast<unsigned>(row) * row_bytes +
                     static_cast<unsigned>(col) * 4u
               : kOob;
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, out),
-                                             c_rsrc, off, 0, 0);
+      if constexpr (U == 4) {
+        __builtin_amdgcn_raw_buffer_store_b128(
+            __builtin_bit_cast(uint4v,
+                               make_float4(out[0], out[1], out[2], out[3])),
+            c_rsrc, off, 0, 0);
+      } else {
+        typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
+        __builtin_amdgcn_raw_buffer_store_b64(
+            __builtin_bit_cast(uint2v, make_float2(out[0], out[1])), c_rsrc,
+            off, 0, 0);
+      }
     }
   }
 }
@@ -1435,17 +1481,23 @@ constexpr int kResidentSlots = 1024;  // 256 CUs x 4 work-groups of 64x64
 constexpr int kSplitUnits = 2048;
 constexpr int kMinChunksPerSplit = 8;
 
-// The plain-rows kernel: one work-group per 64 x 128 tile, `batches`
-// independent problems along blockIdx.z.  Stages of 32 reduction steps fit
-// three work-groups on a CU (768 on the GPU), stages of 16 five (1280) at
-// twice the barriers; the shorter stage is taken when it saves a round of
-// work-groups.
-template <bool EPI, int RK>
+// The plain-rows kernel: one work-group per BM x 128 tile, `batches`
+// independent problems along blockIdx.z.
+//  * BM: the work-groups spread over the 256 CUs, so a launch lasts about
+//    ceil(tiles / 256) * BM row-steps; 112-row tiles are taken when that is
+//    smaller than for 64-row tiles (49 * 2^k rows: 3.06 tiles per CU become
+//    1.75).
+//  * RK: stages of 32 reduction steps or of 16 (more work-groups resident per
+//    CU at twice the barriers); the shorter stage when it saves a round of
+//    work-groups.
+template <bool EPI, int RK, int BM>
 void launch_gemm_rows_as(const float* a, const float* b, float* c, int m,
                          int k, int n, int batches, int z_a, int z_b, int z_c,
-                         unsigned tiles_n, unsigned n_tiles, const float* bias,
-                         int relu, hipStream_t stream) {
-  hipLaunchKernelGGL((gemm_rows_kernel<EPI, RK>),
+                         const float* bias, int relu, hipStream_t stream) {
+  const unsigned tiles_m = static_cast<unsigned>(ceil_div(m, BM));
+  const unsigned tiles_n = static_cast<unsigned>(ceil_div(n, kRowsBN));
+  const unsigned n_tiles = tiles_m * tiles_n;
+  hipLaunchKernelGGL((gemm_rows_kernel<EPI, RK, BM>),
                      dim3(n_tiles, 1, static_cast<unsigned>(batches)),
                      dim3(kThreads), 0, stream, a, b, c, m, k, n, z_a, z_b, z_c,
                      tiles_n, n_tiles, bias, relu);
@@ -1454,37 +1506,51 @@ void launch_gemm_rows_as(const float* a, const float* b, float* c, int m,
 void launch_gemm_rows(const float* a, const float* b, float* c, int m, int k,
                       int n, int batches, int z_a, int z_b, int z_c,
                       hipStream_t stream, const LaunchOptions* epilogue) {
-  const unsigned tiles_m = static_cast<unsigned>(ceil_div(m, kRowsBM));
-  const unsigned tiles_n = static_cast<unsigned>(ceil_div(n, kRowsBN));
-  const unsigned n_tiles = tiles_m * tiles_n;
-  const long groups = static_cast<long>(n_tiles) * batches;
-  bool short_stage = (groups + 1279) / 1280 < (groups + 767) / 768;
+  const long tiles_n = ceil_div(n, kRowsBN);
+  const long groups64 = static_cast<long>(ceil_div(m, 64)) * tiles_n * batches;
+  const long groups112 =
+      static_cast<long>(ceil_div(m, 112)) * tiles_n * batches;
+  // (measured: a 6 % shorter estimate -- 56x56x64 -> 256 -- changes nothing,
+  // and 224 work-groups of four waves cannot fill 256 CUs -- 7x7x512 -> 2048 --
+  // so the tall tile needs a tenth less and at least 320 work-groups)
+  bool tall = 10 * ((groups112 + 255) / 256) * 112 <=
+                  9 * ((groups64 + 255) / 256) * 64 &&
+              groups112 >= 320;
+  if (const char* tune = SNN_TUNING_ENV("SNN_HIP_GEMM_ROWS_BM")) {
+    if (tune[0] != 0) tall = std::atoi(tune) == 112;
+  }
+  const long groups = tall ? groups112 : groups64;
+  // resident work-groups on 256 CUs: 64-row tiles 3 / 5 per CU (stage of 32 /
+  // 16 steps), 112-row tiles 2 / 4
+  const long slots32 = tall ? 512 : 768, slots16 = tall ? 1024 : 1280;
+  bool short_stage =
+      (groups + slots16 - 1) / slots16 < (groups + slots32 - 1) / slots32;
   if (const char* tune = SNN_TUNING_ENV("SNN_HIP_GEMM_ROWS_RK")) {
     if (tune[0] != 0) short_stage = std::atoi(tune) == 16;
   }
   KernelTimer timer(stream);
-  // the bias vector is read 16 bytes at a time
-  const bool fuse = epilogue != nullptr && epilogue->wanted() && batches == 1 &&
-                    (epilogue->bias == nullptr ||
-                     (reinterpret_cast<uintptr_t>(epilogue->bias) & 15u) == 0);
+  // bias is added per column from the bias vector
+  const bool fuse = epilogue != nullptr && epilogue->wanted() && batches == 1;
   const float* bias = fuse ? epilogue->bias : nullptr;
   const int relu = fuse && epilogue->relu ? 1 : 0;
+#define SNN_ROWS(EPI, RK, BM)                                                 \
+  launch_gemm_rows_as<EPI, RK, BM>(a, b, c, m, k, n, batches, z_a, z_b, z_c, \
+                                   bias, relu, stream)
   if (fuse) {
-    if (short_stage)
-      launch_gemm_rows_as<true, 16>(a, b, c, m, k, n, batches, z_a, z_b, z_c,
-                                    tiles_n, n_tiles, bias, relu, stream);
-    else
-      launch_gemm_rows_as<true, 32>(a, b, c, m, k, n, batches, z_a, z_b, z_c,
-                                    tiles_n, n_tiles, bias, relu, stream);
+    if (tall) {
+      if (short_stage) SNN_ROWS(true, 16, 112); else SNN_ROWS(true, 32, 112);
+    } else {
+      if (short_stage) SNN_ROWS(true, 16, 64); else SNN_ROWS(true, 32, 64);
+    }
     if (epilogue->applied != nullptr) *epilogue->applied = true;
   } else {
-    if (short_stage)
-      launch_gemm_rows_as<false, 16>(a, b, c, m, k, n, batches, z_a, z_b, z_c,
-                                     tiles_n, n_tiles, bias, relu, stream);
-    else
-      launch_gemm_rows_as<false, 32>(a, b, c, m, k, n, batches, z_a, z_b, z_c,
-                                     tiles_n, n_tiles, bias, relu, stream);
+    if (tall) {
+      if (short_stage) SNN_ROWS(false, 16, 112); else SNN_ROWS(false, 32, 112);
+    } else {
+      if (short_stage) SNN_ROWS(false, 16, 64); else SNN_ROWS(false, 32, 64);
+    }
   }
+#undef SNN_ROWS
 }
 
 // Shapes the plain-rows kernel takes and is the better choice for: rows read
@@ -1498,7 +1564,7 @@ constexpr long kRowsMinTiles = 256;
 bool gemm_rows_wanted(int m, int k, int n, int batches) {
   static const char* tune = SNN_TUNING_ENV("SNN_HIP_GEMM_ROWS");
   if (tune != nullptr && tune[0] == '0') return false;
-  const long tiles = static_cast<long>(ceil_div(m, kRowsBM)) *
+  const long tiles = static_cast<long>(ceil_div(m, 64)) *
                      ceil_div(n, kRowsBN) * batches;
   const long min_tiles = (tune != nullptr && tune[0] == '1') ? 1 : kRowsMinTiles;
   // columns past n in the last 128-wide tile are computed and dropped: at

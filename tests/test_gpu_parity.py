@@ -615,6 +615,43 @@ def test_matmul(trans_a, trans_b, shape):
         assert_close(got, ref, ("matmul", shape, trans_a, trans_b, beta))
 
 
+@pytest.mark.parametrize("shape", [
+    # batches, m, k, n: shapes that take the plain-rows kernel
+    (1, 6390, 256, 1000),   # 112-row tiles: 57 full + 6 rows, 24 columns short
+    (1, 16390, 64, 252),    # 64-row tiles, ragged last row tile and column tile
+    (3, 6272, 128, 128),    # batched, short LDS stages
+    (1, 25088, 96, 512),    # three chunks
+])
+def test_matmul_plain_rows_kernel(shape):
+    """The 16x16x4 MFMA kernel behind A * B with 16-byte fetches and stores:
+    both tilings, ragged rows and columns, batches."""
+    b_, m, k, n = shape
+    rng = np.random.default_rng(sum(shape) + 11)
+    a, b = uniform(rng, b_ * m * k), uniform(rng, b_ * k * n)
+    ref = oracle.matmul(a, b, b_, m, k, n, False, False, 0.0)
+    got = ops.matmul(dev(a), dev(b), b_, m, k, n, False, False, 0.0)
+    assert_close(got.cpu().numpy(), ref, ("matmul rows", shape))
+
+
+def test_plain_rows_kernel_bias_relu_on_tall_tiles():
+    """14x14x256 -> 1024 at batch 32 runs on 112-row tiles; the fused bias +
+    ReLU epilogue must equal the convolution followed by the two steps."""
+    p = ops.conv_params(32, 14, 14, 256, 1024, 1, 1, False)
+    rng = np.random.default_rng(4343)
+    n_in, n_fil, _ = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x, w = uniform(rng, n_in), uniform(rng, n_fil)
+    bias = uniform(rng, 1024) * 4
+    dx, dw, db = dev(x), dev(w), dev(bias)
+    plain = ops.conv2d(dx, dw, p, DIRECTION.FORWARD, ALGO.MATMUL)
+    ref = oracle.conv2d_forward(x, w, oracle_params(p, 1024), acc64=True)
+    assert_close(plain.cpu().numpy(), ref, "1x1 on tall tiles")
+    want = torch.relu(plain.view(-1, 1024) + db).view(-1)
+    got = ops.conv2d_bias_act(dx, dw, db, p, ALGO.MATMUL, relu=True)
+    assert torch.equal(got, want)
+    got = ops.conv2d_bias_act(dx, dw, db, p, ALGO.MATMUL, relu=False)
+    assert torch.equal(got, (plain.view(-1, 1024) + db).view(-1))
+
+
 def test_many_tiles_per_work_group_epilogue_and_accumulate():
     """Launches with thousands of 64 x 64 tiles make the implicit-GEMM
     work-groups walk several tiles each.  At that size: the fused bias + ReLU
