@@ -398,10 +398,19 @@ def main():
                     a, b, p, DIRECTION.FORWARD, ALGO.IM2COL, workspace=ws,
                     out=o), reps=10, warm=2, repeats=3)
                 fl = ops.conv_flops(p, DIRECTION.FORWARD)
-                h.append({"op": "conv%dx%d_%dx%dx%d_k%d_b128_f16" % (
+                entry = {"op": "conv%dx%d_%dx%dx%d_k%d_b128_f16" % (
                     window, window, size, size, ch, feats), "ms": round(ms, 4),
                     "tflops": round(fl / ms / 1e9, 1),
-                    "frac_f16_mfma_peak": frac(fl / ms / 1e9, 2500.0)})
+                    "frac_f16_mfma_peak": frac(fl / ms / 1e9, 2500.0)}
+                if window == 1:
+                    # the 1x1 layers move (input + filter + output) x 2 bytes
+                    # for little arithmetic: the large ones are HBM bound
+                    nbytes = 2 * (n_a + n_b + n_o)
+                    entry["bytes"] = nbytes
+                    entry["gbs"] = round(nbytes / ms / 1e6, 1)
+                    entry["frac_hbm_peak"] = frac(nbytes / ms / 1e6,
+                                                  PEAK_HBM_GBS)
+                h.append(entry)
                 if window == 3:
                     # input gradient: the same kernel on dY (o) with the
                     # filter's taps mirrored and its roles swapped

@@ -298,6 +298,21 @@ int launch_conv2d_igemm_f16(const _Float16* input, const _Float16* filter,
                             hipStream_t stream) {
   const size_t wgt_elems = static_cast<size_t>(p.window_rows) * p.window_cols *
                            p.channels * p.features;
+  // 1x1, stride 1, no padding: a plain row-major GEMM over the pixels
+  if (p.window_rows == 1 && p.window_cols == 1 && p.stride_rows == 1 &&
+      p.stride_cols == 1 && p.pad_rows == 0 && p.pad_cols == 0 &&
+      p.out_rows == p.in_rows && p.out_cols == p.in_cols &&
+      ((reinterpret_cast<uintptr_t>(input) |
+        reinterpret_cast<uintptr_t>(filter) |
+        reinterpret_cast<uintptr_t>(output)) & 15u) == 0) {
+    const size_t pixels = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols;
+    if (pixels <= static_cast<size_t>(INT_MAX) &&
+        gemm_rows_f16_supports(static_cast<int>(pixels), p.channels,
+                               p.features))
+      return launch_gemm_rows_f16(input, filter, output,
+                                  static_cast<int>(pixels), p.channels,
+                                  p.features, stream);
+  }
   _Float16* wgt_t = workspace;
   bool temporary = false;
   if (workspace == nullptr || workspace_elems < wgt_elems ||

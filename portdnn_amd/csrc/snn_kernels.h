@@ -105,6 +105,12 @@ int launch_conv2d_igemm_f16(const _Float16* input, const _Float16* filter,
                             _Float16* output, const snn_hip_conv2d_params& p,
                             _Float16* workspace, size_t workspace_elems,
                             hipStream_t stream);
+// Row-major binary16 GEMM y[m][n] = sum_k x[m][k] w[k][n] with the filter slab
+// resident in LDS (gemm_rows_f16.hip): 1x1 stride-1 convolutions and matmul
+// with k a multiple of 64 and n a multiple of 64; needs no workspace.
+bool gemm_rows_f16_supports(int m, int k, int n);
+int launch_gemm_rows_f16(const _Float16* x, const _Float16* w, _Float16* y,
+                         int m, int k, int n, hipStream_t stream);
 // Stride-1 input gradient in half precision: the forward kernels above run on
 // dY with the filter's taps mirrored and its channel / feature roles swapped.
 // `supports` is false when neither kernel takes the shape.

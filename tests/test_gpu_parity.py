@@ -714,6 +714,40 @@ def test_matmul_f16(trans_a, trans_b, shape):
                          ("matmul f16", shape, trans_a, trans_b, beta))
 
 
+@pytest.mark.parametrize("shape", [
+    # rows, reduction, columns of the row-major half-precision GEMM
+    (6272, 64, 256),     # one slab, X kept in registers for both column groups
+    (3136, 128, 512),    # two chunks resident, four column groups, tail jobs
+    (1000, 128, 384),    # three column groups, rows not a multiple of 32
+    (1568, 256, 1024),   # streamed X, four slabs
+    (490, 512, 2048),    # sixteen slabs of 128 columns
+    (777, 192, 192),     # 64-column groups (two interleaved features per lane)
+    (65, 64, 64),        # a single 64-column group
+    (1, 64, 128),        # one row
+    (4097, 1024, 64),    # long reduction, narrow slab
+])
+def test_f16_rows_gemm_slab_kernel(shape):
+    """1x1 stride-1 half-precision convolution / matmul on the kernel that
+    keeps the filter slab in LDS: every driver (X resident for 64 and 128
+    channels, streamed above), both column-group widths, ragged row counts and
+    several slabs, against the fp64 product of the same half-rounded operands.
+    Tolerance 1e-2 relative (rms-floored), the half-precision bar."""
+    m, k, n = shape
+    rng = np.random.default_rng(m + k + n)
+    a = uniform(rng, m * k).astype(np.float16)
+    b = uniform(rng, k * n).astype(np.float16)
+    ref = (a.astype(np.float64).reshape(m, k) @
+           b.astype(np.float64).reshape(k, n)).reshape(-1)
+    got = ops.matmul(dev(a, torch.float16), dev(b, torch.float16), 1, m, k, n,
+                     False, False, 0.0)
+    assert_close_f16(got.float().cpu().numpy(), ref, ("rows f16 matmul", shape))
+    # the same product as a convolution over an image of m pixels
+    p = ops.conv_params(1, 1, m, k, n, 1, 1, False)
+    out = ops.conv2d(dev(a, torch.float16), dev(b, torch.float16), p,
+                     DIRECTION.FORWARD, ALGO.MATMUL)
+    assert_close_f16(out.float().cpu().numpy(), ref, ("rows f16 conv", shape))
+
+
 # ---- f16 ---------------------------------------------------------------------
 
 def assert_close_f16(got, ref, what):
