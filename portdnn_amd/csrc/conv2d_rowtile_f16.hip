@@ -12,9 +12,9 @@
 //
 //   * the input rows those outputs need (the tile plus its halo, zero padding
 //     included as explicit zero pixels) are loaded into LDS once per block of
-//     KC channels, [pixel slot][KC halves] with the 16-byte pieces of a slot
-//     XOR-swizzled, by buffer loads that write LDS directly; every filter tap
-//     then reads the same LDS tile at a slot offset of r * Wh + s;
+//     KC channels, [pixel slot][KC halves + 16 bytes of padding], by buffer
+//     loads that write LDS directly; every filter tap then reads the same LDS
+//     tile at a slot offset of r * Wh + s;
 //   * the filter never touches LDS: it is pre-packed in MFMA A-operand order,
 //     [k-step][feature block of 32][lane][8 halves], and streams from global
 //     memory (L2-resident) straight into registers, prefetched two units of
@@ -124,11 +124,15 @@ constexpr int kWaitVm8 = 0x0F78;
 // window, whose reduction loop is unrolled over a filter row with all tap
 // bookkeeping resolved at compile time.
 //
-// LDS tile: [pixel slot][KC halves], no padding; the 16-byte pieces of a slot
-// are stored at piece position (piece ^ swizzle(slot)), which keeps the
-// ds_read_b128 of 32 consecutive slots free of bank conflicts.  Tiles are
-// filled by buffer loads that write LDS directly (64 lanes x 16 bytes = 1 KB
-// of consecutive LDS per instruction), so a whole tile is in flight without
+// LDS tile: [pixel slot][KC halves + one 16-byte pad piece].  A slot is then
+// an odd number of 16-byte pieces (5 or 9), so the ds_read_b128 of 16
+// consecutive slots at the same piece touch 16 different bank groups, and a
+// slot's address is linear in its index: the three taps of a filter row and
+// the reduction steps of a tap are compile-time offsets of one address per
+// pixel block, which leaves the reduction loop without address arithmetic.
+// Tiles are filled by buffer loads that write LDS directly (64 lanes x 16
+// bytes = 1 KB of consecutive LDS per instruction; the lanes that fall on pad
+// pieces load from out of range), so a whole tile is in flight without
 // holding registers; out-of-range offsets (padding pixels) store zeros.
 template <int WF, int WP, int PB, int KC, bool MULTI, bool WIN3>
 __global__ void __launch_bounds__(64 * WF * WP)
@@ -142,9 +146,8 @@ __global__ void __launch_bounds__(64 * WF * WP)
   constexpr int NW = WF * WP;
   constexpr int KS = KC / 16;        // MFMA reduction steps per tap
   constexpr int UPT = KS / 2;        // units of two steps per tap
-  constexpr int ROWB = KC * 2;       // bytes per LDS pixel slot
-  constexpr int PPS = KC / 8;        // 16-byte pieces per slot
-  constexpr int SPB = 64 / PPS;      // slots per 1 KB block
+  constexpr int PPS = KC / 8;        // 16-byte pieces of data per slot
+  constexpr int SLOTB = KC * 2 + 16; // bytes per LDS pixel slot (one pad piece)
   extern __shared__ __align__(16) unsigned char lds[];
   typedef __attribute__((address_space(3))) void* lds_ptr;
 
@@ -163,19 +166,17 @@ __global__ void __launch_bounds__(64 * WF * WP)
   const int first_padded =
       (row0 / g.out_rows) * g.padded_rows + row0 % g.out_rows;
 
-  const int n_blocks = (g.n_slots + SPB - 1) / SPB;  // 1 KB blocks per tile
+  // 1 KB blocks per tile, and the slots they reach into
+  const int n_blocks = (g.n_slots * SLOTB + 1023) / 1024;
+  const int n_table = n_blocks * 1024 / SLOTB + 1;
   const int buf_bytes = n_blocks * 1024;
   unsigned char* const bufs = lds;
   unsigned* const table =
       reinterpret_cast<unsigned*>(lds + (MULTI ? 2 : 1) * buf_bytes);
 
-  auto swizzle = [](int slot) {
-    return PPS == 4 ? (slot >> 1) & 3 : slot & 7;
-  };
-
   // Global byte offset of channel 0 of every pixel slot (kOob for padding
   // and for the slots that only fill up the last block).
-  for (int slot = tid; slot < n_blocks * SPB; slot += NT) {
+  for (int slot = tid; slot < n_table; slot += NT) {
     const int lrow = slot / g.halo_cols;
     const int hx = slot - lrow * g.halo_cols;
     const int padded = first_padded + lrow;
@@ -197,17 +198,19 @@ __global__ void __launch_bounds__(64 * WF * WP)
   const __amdgpu_buffer_rsrc_t wpk_rsrc = make_rsrc(wpk, wpk_bytes);
 
   // Starts the loads of one channel block into an LDS tile: wave w takes the
-  // 1 KB blocks w, w + NW, ...; lane l fills piece position l % PPS of slot
-  // block * SPB + l / PPS.  `soff` (in range by construction) selects the
-  // channel block; padding goes out of range through the vector offset,
-  // which is the only one the hardware range-checks.
-  const int fill_slot = lane / PPS;
-  const int fill_pos = lane % PPS;
+  // 1 KB blocks w, w + NW, ...; lane l fills bytes 16 l .. 16 l + 15 of its
+  // block, which belong to piece (position % SLOTB) / 16 of slot position /
+  // SLOTB; the pad piece of a slot loads from out of range (zeros).  `soff`
+  // (in range by construction) selects the channel block; padding pixels go
+  // out of range through the vector offset, the only one the hardware
+  // range-checks.
   auto start_tile = [&](unsigned char* buf, unsigned soff) {
     for (int block = wave; block < n_blocks; block += NW) {
-      const int slot = block * SPB + fill_slot;
+      const int pos = block * 1024 + lane * 16;
+      const int slot = pos / SLOTB;
+      const int piece = (pos - slot * SLOTB) >> 4;
       const unsigned voff =
-          table[slot] + static_cast<unsigned>(fill_pos ^ swizzle(slot)) * 16u;
+          piece < PPS ? table[slot] + static_cast<unsigned>(piece) * 16u : kOob;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           src_rsrc, (lds_ptr)(buf + block * 1024), 16, voff, soff, 0, 0);
     }
@@ -300,35 +303,34 @@ __global__ void __launch_bounds__(64 * WF * WP)
     // with the three taps of a row (UPT units each) unrolled, which also
     // keeps the rotation of the three filter buffers static.
     int cur_off = 0, nxt_off = buf_bytes;
-    // LDS byte offset of this lane's fragment of step 0 of a tap; step ks is
-    // at the same offset with ks * 32 XOR-ed in (the swizzle only permutes
-    // 16-byte pieces inside a slot).
-    auto tap_base = [&](int (&base)[PB], int buf_off, int slots) {
+    // Byte offset inside a tile of this lane's fragment of tap (0, 0), step 0.
+    // Slots are SLOTB bytes apart, so the taps of a filter row and the steps
+    // of a tap are compile-time offsets from the row's address.
+    int lane_base[PB];
 #pragma unroll
-      for (int j = 0; j < PB; ++j) {
-        const int slot = b_slot[j] + slots;
-        base[j] = buf_off + slot * ROWB + ((khalf ^ swizzle(slot)) << 4);
-      }
-    };
-    auto read_b = [&](half8 (&b)[PB], const int (&base)[PB], int ks) {
+    for (int j = 0; j < PB; ++j) lane_base[j] = b_slot[j] * SLOTB + khalf * 16;
+    const int row_step = g.halo_cols * SLOTB;
+    auto read_b = [&](half8 (&b)[PB], const int (&rb)[PB], int offset) {
 #pragma unroll
       for (int j = 0; j < PB; ++j)
-        b[j] = *reinterpret_cast<const half8*>(bufs + (base[j] ^ (ks * 32)));
+        b[j] = *reinterpret_cast<const half8*>(bufs + rb[j] + offset);
     };
-    int base[PB];
-    tap_base(base, cur_off, 0);
-    read_b(b_even, base, 0);
+    int rb[PB];  // filter row r of the current tile
+#pragma unroll
+    for (int j = 0; j < PB; ++j) rb[j] = cur_off + lane_base[j];
+    read_b(b_even, rb, 0);
 #pragma unroll 1
     for (int c = 0; c < n_chunks; ++c) {
 #pragma unroll 1
       for (int r = 0; r < 3; ++r) {
+        // the next filter row (after the last one the tiles swap and the
+        // fragment is read again; the tile's first row will do here)
+        int rb_next[PB];
+#pragma unroll
+        for (int j = 0; j < PB; ++j)
+          rb_next[j] = r < 2 ? rb[j] + row_step : cur_off + lane_base[j];
 #pragma unroll
         for (int sc = 0; sc < 3; ++sc) {
-          // first step of the next tap (after the last tap the tiles swap
-          // and the fragment is read again; slot 0 will do here)
-          const int next_slots =
-              sc < 2 ? r * g.halo_cols + sc + 1
-                     : (r < 2 ? (r + 1) * g.halo_cols : 0);
 #pragma unroll
           for (int u = 0; u < UPT; ++u) {
             constexpr int kRot = 3;
@@ -342,33 +344,38 @@ __global__ void __launch_bounds__(64 * WF * WP)
                              static_cast<unsigned>((c + 1) * KC * 2));
               }
             }
-            read_b(b_odd, base, 2 * u + 1);
+            read_b(b_odd, rb, sc * SLOTB + (2 * u + 1) * 32);
             __builtin_amdgcn_sched_barrier(0);
-            // Address arithmetic shares a scheduling region with MFMAs so
-            // that it issues in their shadow: the filter prefetch and, in
-            // the last unit of a tap, the next tap's LDS offsets (the
-            // current ones are dead once the odd step's reads are issued).
+            // The filter prefetch issues in the shadow of the MFMAs.
             load_a(a_fill, step + 4);
             step += 2;
             mfma_step(a_use[0], b_even);
-            if (u + 1 == UPT) tap_base(base, cur_off, next_slots);
             __builtin_amdgcn_sched_barrier(0);
-            read_b(b_even, base, u + 1 < UPT ? 2 * u + 2 : 0);
+            if (u + 1 < UPT)
+              read_b(b_even, rb, sc * SLOTB + (2 * u + 2) * 32);
+            else if (sc < 2)
+              read_b(b_even, rb, (sc + 1) * SLOTB);
+            else
+              read_b(b_even, rb_next, 0);
             __builtin_amdgcn_sched_barrier(0);
             mfma_step(a_use[1], b_odd);
             __builtin_amdgcn_sched_barrier(0);
           }
         }
+#pragma unroll
+        for (int j = 0; j < PB; ++j) rb[j] = rb_next[j];
       }
       if constexpr (MULTI) {
-        // End of the channel block; the compiler waits for the LDS-direct
-        // loads of the next tile before the barrier.
+        // End of the channel block.  Vector-memory loads complete in order,
+        // so the next tile, issued at the block's start, has landed once the
+        // filter loads of the block's later units have been waited for.
         __syncthreads();
         const int t = cur_off;
         cur_off = nxt_off;
         nxt_off = t;
-        tap_base(base, cur_off, 0);
-        read_b(b_even, base, 0);
+#pragma unroll
+        for (int j = 0; j < PB; ++j) rb[j] = cur_off + lane_base[j];
+        read_b(b_even, rb, 0);
       }
     }
   } else {
@@ -378,12 +385,10 @@ __global__ void __launch_bounds__(64 * WF * WP)
     int tap_slots = 0;  // slot offset of the current tap: r * Wh + s
     // Pixel fragments of reduction step `ks` (0 .. KS-1) of a tap.
     auto load_b = [&](half8 (&b)[PB], int slots, int ks) {
+      const int offset = slots * SLOTB + (2 * ks + khalf) * 16;
 #pragma unroll
-      for (int j = 0; j < PB; ++j) {
-        const int slot = b_slot[j] + slots;
-        const int pos = (2 * ks + khalf) ^ swizzle(slot);
-        b[j] = *reinterpret_cast<const half8*>(cur + slot * ROWB + pos * 16);
-      }
+      for (int j = 0; j < PB; ++j)
+        b[j] = *reinterpret_cast<const half8*>(cur + b_slot[j] * SLOTB + offset);
     };
     load_b(b_even, 0, 0);
 
@@ -543,10 +548,11 @@ RowTilePlan plan_tile(const snn_hip_conv2d_params& p, int wf, int wp, int pb,
   g.n_slots = static_cast<int>(lds_rows) * g.halo_cols;
   g.n_fslices = p.features / (64 * wf);
   const int n_chunks = p.channels / kc;
-  const int slots_per_block = 64 / (kc / 8);  // slots per 1 KB of LDS
-  const size_t n_blocks = ceil_div(g.n_slots, slots_per_block);
-  const size_t lds_bytes = (n_chunks > 1 ? 2 : 1) * n_blocks * 1024 +
-                           n_blocks * slots_per_block * 4;
+  const size_t slot_bytes = static_cast<size_t>(kc) * 2 + 16;
+  const size_t n_blocks = ceil_div(g.n_slots * slot_bytes, size_t{1024});
+  const size_t n_table = n_blocks * 1024 / slot_bytes + 1;
+  const size_t lds_bytes =
+      (n_chunks > 1 ? 2 : 1) * n_blocks * 1024 + n_table * 4;
   if (lds_bytes > kMaxLdsBytes) return plan;
   plan.wf = wf; plan.wp = wp; plan.pb = pb; plan.kc = kc;
   plan.lds_bytes = lds_bytes;
