@@ -621,6 +621,122 @@ __global__ void __launch_bounds__(256)
     if (y0 + i <= y_last) GradVec<4>::store(dx_p + i * row_elems, grad[i]);
 }
 
+// The average gradient for 3x3 windows at stride 2 (no LDS, all loads of a
+// block row issued together).  In padded coordinates an input pixel with an
+// even row lies in the last row of window row (row / 2 - 1) and the first of
+// (row / 2), one with an odd row only in the middle of (row / 2); columns
+// alike.  So the 2x2 input pixels of block (br, bc) take their gradient from
+// the windows (br - 1 .. br) x (bc - 1 .. bc) only: a lane walks TH block rows
+// of one block column, loads the two dY vectors of a window row once, divides
+// them by the windows' in-image element counts and carries them down as the
+// next block row's "windows above".  The terms are added in the reference's
+// order (window row, then window column, starting from zero;
+// src/pooling/kernels.h:291-375); a window that does not exist contributes
+// +0, which leaves every sum as it is.
+template <int TH>
+__global__ void __launch_bounds__(256)
+    pool_avg_grad_3x3_s2_kernel(const float* __restrict__ dy,
+                                float* __restrict__ dx,
+                                snn_hip_pooling_params p, int n_bcols,
+                                int n_strips, unsigned n_items) {
+  const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+  if (idx >= n_items) return;
+  const int C = p.channels;
+  const unsigned cv = static_cast<unsigned>(C) / 4u;
+  const int ch = static_cast<int>(idx % cv) * 4;
+  unsigned t = idx / cv;
+  const int bc = static_cast<int>(t % static_cast<unsigned>(n_bcols)) +
+                 p.pad_cols / 2;
+  t /= static_cast<unsigned>(n_bcols);
+  const int br0 = static_cast<int>(t % static_cast<unsigned>(n_strips)) * TH +
+                  p.pad_rows / 2;
+  const int n = static_cast<int>(t / static_cast<unsigned>(n_strips));
+  const size_t in_elems =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * C;
+  const size_t out_elems =
+      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * C;
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, out_elems * 4);
+  const __amdgpu_buffer_rsrc_t dx_rsrc = make_rsrc(dx, in_elems * 4);
+
+  // windows bc - 1 and bc: present, and their number of in-image columns
+  bool w_ok[2];
+  int w_cols[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int ox = bc - 1 + j;
+    w_ok[j] = static_cast<unsigned>(ox) < static_cast<unsigned>(p.out_cols);
+    const int c0 = 2 * ox - p.pad_cols;
+    w_cols[j] = max(min(c0 + 3, p.in_cols) - max(c0, 0), 1);
+  }
+  // dY[oy][bc - 1 .. bc] / count, zeros for windows that do not exist
+  auto load_row = [&](int oy, float (&g)[2][4]) {
+    const bool row_ok =
+        static_cast<unsigned>(oy) < static_cast<unsigned>(p.out_rows);
+    const unsigned base =
+        static_cast<unsigned>(((n * p.out_rows + oy) * p.out_cols + bc - 1) *
+                                  C + ch) * 4u;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      BufVec4<float>::load(dy_rsrc,
+                           (row_ok && w_ok[j])
+                               ? base + static_cast<unsigned>(j * C) * 4u
+                               : kOobOffset,
+                           g[j]);
+  };
+  auto divide_row = [&](int oy, float (&g)[2][4]) {
+    const int r0 = 2 * oy - p.pad_rows;
+    const int w_rows = max(min(r0 + 3, p.in_rows) - max(r0, 0), 1);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const float count = static_cast<float>(w_rows * w_cols[j]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) g[j][e] = g[j][e] / count;
+    }
+  };
+  const int x0 = 2 * bc - p.pad_cols;
+  const bool x_ok[2] = {
+      static_cast<unsigned>(x0) < static_cast<unsigned>(p.in_cols),
+      static_cast<unsigned>(x0 + 1) < static_cast<unsigned>(p.in_cols)};
+  const unsigned row_bytes = static_cast<unsigned>(p.in_cols * C) * 4u;
+  const unsigned col_bytes = static_cast<unsigned>(C) * 4u;
+
+  float rows[TH + 1][2][4];
+#pragma unroll
+  for (int i = 0; i <= TH; ++i) load_row(br0 - 1 + i, rows[i]);
+#pragma unroll
+  for (int i = 0; i <= TH; ++i) divide_row(br0 - 1 + i, rows[i]);
+#pragma unroll
+  for (int i = 0; i < TH; ++i) {
+    const int br = br0 + i;
+    const float (&above)[2][4] = rows[i];
+    const float (&here)[2][4] = rows[i + 1];
+    float ee[4], eo[4], oe[4], oo[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      ee[e] = (((0.f + above[0][e]) + above[1][e]) + here[0][e]) + here[1][e];
+      eo[e] = (0.f + above[1][e]) + here[1][e];
+      oe[e] = (0.f + here[0][e]) + here[1][e];
+      oo[e] = 0.f + here[1][e];
+    }
+    const int y0 = 2 * br - p.pad_rows;
+    const bool y_ok[2] = {
+        static_cast<unsigned>(y0) < static_cast<unsigned>(p.in_rows),
+        static_cast<unsigned>(y0 + 1) < static_cast<unsigned>(p.in_rows)};
+    const unsigned base =
+        static_cast<unsigned>(((n * p.in_rows + y0) * p.in_cols + x0) * C + ch) *
+        4u;
+    BufVec4<float>::store(dx_rsrc, (y_ok[0] && x_ok[0]) ? base : kOobOffset,
+                          ee);
+    BufVec4<float>::store(
+        dx_rsrc, (y_ok[0] && x_ok[1]) ? base + col_bytes : kOobOffset, eo);
+    BufVec4<float>::store(
+        dx_rsrc, (y_ok[1] && x_ok[0]) ? base + row_bytes : kOobOffset, oe);
+    BufVec4<float>::store(
+        dx_rsrc,
+        (y_ok[1] && x_ok[1]) ? base + row_bytes + col_bytes : kOobOffset, oo);
+  }
+}
+
 template <typename T, typename Op>
 int launch_forward_op(const T* input, T* output,
                       const snn_hip_pooling_params& p, hipStream_t stream) {
@@ -1133,8 +1249,32 @@ int launch_pooling_avg_grad(const float* input_backprop,
   constexpr int kBlock = 256;
   const size_t n_in =
       static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
+  const size_t n_out =
+      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * p.channels;
+  static const bool no_s2 = SNN_TUNING_ENV("SNN_HIP_POOL_AVG_GRAD_GENERIC") != nullptr;
   if (p.channels % 4 == 0 && grad_aligned16(input_backprop) &&
-      grad_aligned16(output_backprop)) {
+      grad_aligned16(output_backprop) && p.window_rows == 3 &&
+      p.window_cols == 3 && p.stride_rows == 2 && p.stride_cols == 2 &&
+      n_in * 4 < 0x7FFFFFF0u && n_out * 4 < 0x7FFFFFF0u && !no_s2) {
+    // block rows / columns: padded coordinates pad .. in + pad - 1, halved
+    const int n_brows = (p.in_rows + p.pad_rows - 1) / 2 - p.pad_rows / 2 + 1;
+    const int n_bcols = (p.in_cols + p.pad_cols - 1) / 2 - p.pad_cols / 2 + 1;
+    const size_t per_row =
+        static_cast<size_t>(p.batch) * n_bcols * (p.channels / 4);
+    const int th = per_row * ceil_div(n_brows, 4) >= 150000 ? 4 : 2;
+    const int n_strips = ceil_div(n_brows, th);
+    const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
+    const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
+    if (th == 4)
+      hipLaunchKernelGGL(pool_avg_grad_3x3_s2_kernel<4>, grid, dim3(kBlock), 0,
+                         stream, input_backprop, output_backprop, p, n_bcols,
+                         n_strips, n_items);
+    else
+      hipLaunchKernelGGL(pool_avg_grad_3x3_s2_kernel<2>, grid, dim3(kBlock), 0,
+                         stream, input_backprop, output_backprop, p, n_bcols,
+                         n_strips, n_items);
+  } else if (p.channels % 4 == 0 && grad_aligned16(input_backprop) &&
+             grad_aligned16(output_backprop)) {
     const size_t n_vec = n_in / 4;
     // row strips when they still give every CU a few thousand lanes
     const size_t per_row =

@@ -496,6 +496,30 @@ def test_avgpool_grad_row_strips(shape):
                  ("avg grad strips", shape))
 
 
+@pytest.mark.parametrize("shape", [(32, 112, 112, 64, True),
+                                   (16, 61, 59, 64, False),
+                                   (3, 75, 70, 8, True),
+                                   (2, 8, 9, 4, True),
+                                   (2, 7, 7, 12, False),
+                                   (1, 3, 3, 4, False),
+                                   (5, 30, 31, 32, True)])
+def test_avgpool_grad_3x3_stride2_bit_exact(shape):
+    """The block-row kernel for the 3x3 stride-2 average gradient adds the
+    window terms in the reference's order, so it must reproduce the oracle's
+    fp32 reference-order mode bit for bit (even / odd sizes, SAME and VALID
+    padding, both strip heights, signed zeros in dY)."""
+    n, h, w_, c, same = shape
+    p = ops.pool_params(n, h, w_, c, 3, 2, same)
+    rng = np.random.default_rng(900 + h + w_ + c)
+    dy = rng.standard_normal(n * p.out_rows * p.out_cols * c).astype(
+        np.float32)
+    dy[::97] = 0.0
+    dy[5::89] = -0.0
+    got = ops.pooling_avg_grad(dev(dy), p).cpu().numpy()
+    ref = oracle.pool_avg_grad(dy, oracle_params(p, 0), acc64=False)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), shape
+
+
 @pytest.mark.parametrize("shape", [(2, 9, 7, 5, 3, 2, True),
                                    (1, 11, 11, 3, 5, 1, True),
                                    (3, 8, 8, 8, 2, 2, False),
