@@ -397,6 +397,351 @@ __global__ void __launch_bounds__(512)
   }
 }
 
+// At m A along xi's row index (across the multiplying waves, through `xch`)
+// and the stores of one unit; all 512 lanes take part.
+__device__ __forceinline__ void wino_stream_store(
+    const float* xch, const int* tile_off_tab, const int* tile_flags_tab,
+    int count, int fb, int tid, const FusedGeom& g, float* out,
+    unsigned out_bytes, const float* bias, int relu) {
+  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_bytes);
+  const unsigned out_row_bytes =
+      static_cast<unsigned>(g.out_cols) * g.out_ch * 4u;
+  const int ob = tid >> 8;
+  const int q = tid & 15;
+  const int v = (tid >> 4) & 15;
+  float4 s[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    s[i] = *reinterpret_cast<const float4*>(xch + ((i * 2 + ob) * 16 + v) * 64 +
+                                            4 * q);
+  float4 y0 = s[0] + s[1] + s[2];
+  float4 y1 = s[1] - s[2] - s[3];
+  const int m = 8 * (v >> 2) + 4 * (q >> 3) + (v & 3);
+  const int f = fb * kFeat + 4 * (q & 7);
+  if (bias != nullptr) {
+    const float4 b4 = *reinterpret_cast<const float4*>(bias + f);
+    y0 = y0 + b4;
+    y1 = y1 + b4;
+  }
+  if (relu) {
+    y0 = make_float4(fmaxf(y0.x, 0.f), fmaxf(y0.y, 0.f), fmaxf(y0.z, 0.f),
+                     fmaxf(y0.w, 0.f));
+    y1 = make_float4(fmaxf(y1.x, 0.f), fmaxf(y1.y, 0.f), fmaxf(y1.z, 0.f),
+                     fmaxf(y1.w, 0.f));
+  }
+  const int tile_off = tile_off_tab[(count & 3) * kTiles + m];
+  const int flags = tile_flags_tab[(count & 3) * kTiles + m];
+  const bool col_ok = tile_off >= 0 && (ob == 0 || (flags & 2) != 0);
+  const unsigned off0 = col_ok ? static_cast<unsigned>(tile_off) +
+                                     static_cast<unsigned>(ob * g.out_ch + f) *
+                                         4u
+                               : kOob;
+  const unsigned off1 =
+      (col_ok && (flags & 1) != 0) ? off0 + out_row_bytes : kOob;
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y0),
+                                         out_rsrc, off0, 0, 0);
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y1),
+                                         out_rsrc, off1, 0, 0);
+}
+
+// ---------------------------------------------------------------------------
+// Stream kernel: wino_fused_kernel's unit (32 tiles x 32 features), wave roles
+// (waves 0-3 multiply, waves 4-7 gather and transform) and LDS / operand
+// layouts, run by persistent work-groups.
+//
+// Timestamps inside wino_fused_kernel show that its chunk loop keeps the
+// vector ALUs busy (the fp32 matrix instructions run on them, so the
+// transform's additions and the multiplications share one resource) as long
+// as two work-groups overlap on a CU, but that a unit's prologue (tile index
+// arithmetic, first gather from memory, first transform: 2.7 - 6.7 us) and
+// epilogue (1.3 us) are nearly half of its 14 us on a 64-channel layer.
+// Here a work-group walks the units slot, slot + G, ... of its XCD as one
+// stream of 16-channel chunks: the transforming waves run ahead of the
+// multiplying ones across unit boundaries (gather two chunks ahead,
+// transform one ahead), so the next unit's index arithmetic and first loads
+// happen while the current one is being multiplied.  One barrier per chunk;
+// at the end of a unit At m A goes through the LDS buffer that was
+// multiplied last (two more barriers).  Requires an even number of chunks.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(512)
+    __attribute__((amdgpu_waves_per_eu(4, 4)))
+    wino_stream_kernel(const float* __restrict__ in,
+                       const float* __restrict__ u, float* __restrict__ out,
+                       FusedGeom g, unsigned in_bytes, unsigned u_bytes,
+                       unsigned out_bytes, UnitGrid ug, float inv_tile_cols,
+                       float inv_tile_rows, const float* __restrict__ bias,
+                       int relu) {
+  __shared__ __align__(16) float lds_v[2 * kVBuf];
+  __shared__ int lds_tile_off[4][kTiles];
+  __shared__ int lds_tile_flags[4][kTiles];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int xcd = static_cast<int>(blockIdx.x & 7u);
+  const int slot = static_cast<int>(blockIdx.x >> 3);
+  const int stride = static_cast<int>(gridDim.x >> 3);
+  const int xa = xcd / ug.xcd_f, xc = xcd % ug.xcd_f;
+  const int m_lo = xa * ug.n_mblocks / ug.xcd_m;
+  const int m_hi = (xa + 1) * ug.n_mblocks / ug.xcd_m;
+  const int f_lo = xc * ug.n_fblocks / ug.xcd_f;
+  const int f_hi = (xc + 1) * ug.n_fblocks / ug.xcd_f;
+  const int f_cnt = f_hi - f_lo;
+  const int n_local = (m_hi - m_lo) * f_cnt;
+  if (slot >= n_local) return;  // whole group, before any barrier
+  const int n_chunks = g.in_ch / kChunk;
+
+  if (wave >= 4) {
+    // ---- gather + transform waves ----------------------------------------
+    const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_bytes);
+    const int ptid = tid - 256;
+    const int tile_l = ptid >> 3, pair = ptid & 7;
+    unsigned p_off[16];
+    int g_unit = slot;   // unit (index within the XCD) the gather is in
+    int g_count = 0;     // units the gather has entered before it
+    int g_chunk = 0;     // next chunk to load
+    // Patch offsets of this lane's tile in unit `unit`; every offset is out
+    // of range (loads return zero, nothing is fetched) past the last unit.
+    auto enter_unit = [&](int unit, int count) {
+      const bool any = unit < n_local;
+      const int mb = m_lo + unit / f_cnt;
+      const int tile = mb * kTiles + tile_l;
+      const bool live = any && tile < g.n_tiles;
+      // tile = (n * tile_rows + ty) * tile_cols + tx with tile < 2^23: the
+      // float quotient is at most one off.
+      int t2 = static_cast<int>(static_cast<float>(tile) * inv_tile_cols);
+      int tx = tile - t2 * g.tile_cols;
+      if (tx < 0) { tx += g.tile_cols; --t2; }
+      if (tx >= g.tile_cols) { tx -= g.tile_cols; ++t2; }
+      int n = static_cast<int>(static_cast<float>(t2) * inv_tile_rows);
+      int ty = t2 - n * g.tile_rows;
+      if (ty < 0) { ty += g.tile_rows; --n; }
+      if (ty >= g.tile_rows) { ty -= g.tile_rows; ++n; }
+      const int y0 = 2 * ty - g.pad_rows, x0 = 2 * tx - g.pad_cols;
+      unsigned row_off[4], col_off[4];
+      bool row_ok[4], col_ok[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int y = y0 + i, x = x0 + i;
+        row_ok[i] = live && static_cast<unsigned>(y) <
+                                static_cast<unsigned>(g.in_rows);
+        col_ok[i] =
+            static_cast<unsigned>(x) < static_cast<unsigned>(g.in_cols);
+        row_off[i] = static_cast<unsigned>((n * g.in_rows + y) * g.in_cols) *
+                     static_cast<unsigned>(g.in_ch) * 4u;
+        col_off[i] = static_cast<unsigned>(x * g.in_ch + 2 * pair) * 4u;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          p_off[i * 4 + j] =
+              (row_ok[i] && col_ok[j]) ? row_off[i] + col_off[j] : kOob;
+      if (pair == 0) {
+        lds_tile_off[count & 3][tile_l] =
+            live ? ((n * g.out_rows + 2 * ty) * g.out_cols + 2 * tx) *
+                       g.out_ch * 4
+                 : -1;
+        lds_tile_flags[count & 3][tile_l] =
+            (2 * ty + 1 < g.out_rows ? 1 : 0) |
+            (2 * tx + 1 < g.out_cols ? 2 : 0);
+      }
+    };
+    auto load_patch = [&](float2 (&d)[16]) {
+      const unsigned soff = static_cast<unsigned>(g_chunk * kChunk * 4);
+#pragma unroll
+      for (int q = 0; q < 16; ++q)
+        d[q] = __builtin_bit_cast(
+            float2,
+            __builtin_amdgcn_raw_buffer_load_b64(in_rsrc, p_off[q], soff, 0));
+      if (++g_chunk == n_chunks) {
+        g_chunk = 0;
+        g_unit += stride;
+        ++g_count;
+        enter_unit(g_unit, g_count);
+      }
+    };
+    float* const v_store =
+        lds_v + tile_l * kChunk + 4 * ((pair >> 1) ^ ((tile_l >> 1) & 3)) +
+        2 * (pair & 1);
+    auto transform_store = [&](const float2 (&d)[16], int buf) {
+      float* const dst = v_store + buf * kVBuf;
+      float2 t[4][4];  // Bt d
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        t[0][j] = d[0 * 4 + j] - d[2 * 4 + j];
+        t[1][j] = d[1 * 4 + j] + d[2 * 4 + j];
+        t[2][j] = d[2 * 4 + j] - d[1 * 4 + j];
+        t[3][j] = d[1 * 4 + j] - d[3 * 4 + j];
+      }
+      constexpr int kXi = kTiles * kChunk;  // floats per xi plane
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        *reinterpret_cast<float2*>(dst + (i * 4 + 0) * kXi) =
+            t[i][0] - t[i][2];
+        *reinterpret_cast<float2*>(dst + (i * 4 + 1) * kXi) =
+            t[i][1] + t[i][2];
+        *reinterpret_cast<float2*>(dst + (i * 4 + 2) * kXi) =
+            t[i][2] - t[i][1];
+        *reinterpret_cast<float2*>(dst + (i * 4 + 3) * kXi) =
+            t[i][1] - t[i][3];
+      }
+    };
+    // The fences keep every load where it is written: left alone, the
+    // compiler moves loads across the transforms into spare registers and
+    // then waits for the newest loads instead of the oldest.
+    float2 d_even[16], d_odd[16];
+    enter_unit(g_unit, 0);
+    load_patch(d_even);
+    __builtin_amdgcn_sched_barrier(0);
+    transform_store(d_even, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    load_patch(d_odd);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    for (int unit = slot; unit < n_local; unit += stride) {
+      for (int c = 0; c < n_chunks; c += 2) {
+        // An even chunk is being multiplied from buffer 0.  The loads of the
+        // chunk after next are issued first, right behind the barrier, so
+        // that they queue up in the memory pipeline while the multiplying
+        // waves hold the ALUs; the transform then only has its additions and
+        // LDS writes between the moment those waves stop and the barrier.
+        load_patch(d_even);
+        __builtin_amdgcn_sched_barrier(0);
+        transform_store(d_odd, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        // an odd chunk is being multiplied from buffer 1; the last one of a
+        // unit leaves the next unit's first chunk in buffer 0
+        load_patch(d_odd);
+        __builtin_amdgcn_sched_barrier(0);
+        transform_store(d_even, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+      }
+      __syncthreads();  // multiplying waves write At m A (columns) to buffer 1
+      wino_stream_store(lds_v + kVBuf, lds_tile_off[0], lds_tile_flags[0],
+                        (unit - slot) / stride, f_lo + unit % f_cnt, tid, g,
+                        out, out_bytes, bias, relu);
+      __syncthreads();  // buffer 1 is free again
+    }
+  } else {
+    // ---- multiplying waves -----------------------------------------------
+    const __amdgpu_buffer_rsrc_t u_rsrc = make_rsrc(u, u_bytes);
+    const unsigned n_fblocks = static_cast<unsigned>(ug.n_fblocks);
+    const unsigned u_lane = static_cast<unsigned>(lane) * 16u;
+    const unsigned cgroups = static_cast<unsigned>(g.in_ch) / 8u;
+    // Byte offset of U[xi = 4 wave][feature block of `unit`][channel group 0].
+    auto u_base_of = [&](int unit) {
+      const unsigned fb = static_cast<unsigned>(f_lo + unit % f_cnt);
+      return static_cast<unsigned>(__builtin_amdgcn_readfirstlane(
+          ((static_cast<unsigned>(4 * wave) * n_fblocks + fb) * cgroups) *
+          1024u));
+    };
+    const unsigned u_xi_stride = n_fblocks * cgroups * 1024u;
+    auto load_b = [&](unsigned base, int cgroup, int j) {
+      return __builtin_bit_cast(
+          float4, __builtin_amdgcn_raw_buffer_load_b128(
+                      u_rsrc, u_lane,
+                      base + static_cast<unsigned>(j) * u_xi_stride +
+                          static_cast<unsigned>(cgroup) * 1024u,
+                      0));
+    };
+    const int tile_r = lane & 31;
+    const int swz = (tile_r >> 1) & 3;
+    constexpr int kXi = kTiles * kChunk;
+    const float* const a_base = lds_v + (4 * wave * kTiles + tile_r) * kChunk;
+    const int a_grp0 = 4 * ((0 + (lane >> 5)) ^ swz);
+    const int a_grp1 = 4 * ((2 + (lane >> 5)) ^ swz);
+    auto load_a = [&](const float* a_ptr, int j) {
+      return *reinterpret_cast<const float4*>(a_ptr + j * kXi);
+    };
+    float16v acc[4];
+    // Eight matrix instructions: two xi planes, four reduction steps each.
+    auto mma_pair = [&](int j, const float4& a0, const float4& a1,
+                        const float4& b0, const float4& b1) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(comp(a0, t), comp(b0, t),
+                                                      acc[j], 0, 0, 0);
+        acc[j + 1] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+            comp(a1, t), comp(b1, t), acc[j + 1], 0, 0, 0);
+      }
+    };
+    float4 b[2][4];
+    // One chunk: four quarters (channel half, xi pair).  The B registers of a
+    // quarter are refilled for the chunk after (nb_base, nb_cg) as soon as
+    // its matrix instructions have been issued; the fences keep the compiler
+    // from sinking those loads to the end of the chunk.
+    auto multiply = [&](int buf, unsigned nb_base, int nb_cg) {
+      const float* const a_buf = a_base + buf * kVBuf;
+      float4 a[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) a[j] = load_a(a_buf + a_grp0, j);
+      __builtin_amdgcn_sched_barrier(0);
+      mma_pair(0, a[0], a[1], b[0][0], b[0][1]);
+      __builtin_amdgcn_sched_barrier(0);
+      a[0] = load_a(a_buf + a_grp1, 0);
+      a[1] = load_a(a_buf + a_grp1, 1);
+      b[0][0] = load_b(nb_base, nb_cg, 0);
+      b[0][1] = load_b(nb_base, nb_cg, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mma_pair(2, a[2], a[3], b[0][2], b[0][3]);
+      __builtin_amdgcn_sched_barrier(0);
+      a[2] = load_a(a_buf + a_grp1, 2);
+      a[3] = load_a(a_buf + a_grp1, 3);
+      b[0][2] = load_b(nb_base, nb_cg, 2);
+      b[0][3] = load_b(nb_base, nb_cg, 3);
+      __builtin_amdgcn_sched_barrier(0);
+      mma_pair(0, a[0], a[1], b[1][0], b[1][1]);
+      __builtin_amdgcn_sched_barrier(0);
+      b[1][0] = load_b(nb_base, nb_cg + 1, 0);
+      b[1][1] = load_b(nb_base, nb_cg + 1, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mma_pair(2, a[2], a[3], b[1][2], b[1][3]);
+      __builtin_amdgcn_sched_barrier(0);
+      b[1][2] = load_b(nb_base, nb_cg + 1, 2);
+      b[1][3] = load_b(nb_base, nb_cg + 1, 3);
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+    };
+    unsigned u_base = u_base_of(slot);
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[h][j] = load_b(u_base, h, j);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    for (int unit = slot; unit < n_local; unit += stride) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+      const int next_unit = unit + stride < n_local ? unit + stride : unit;
+      const unsigned u_next = u_base_of(next_unit);
+      for (int c = 0; c < n_chunks; c += 2) {
+        multiply(0, u_base, 2 * (c + 1));
+        const bool last = c + 2 >= n_chunks;
+        multiply(1, last ? u_next : u_base, last ? 0 : 2 * (c + 2));
+      }
+      // At m A along xi's column index, inside the lane, into buffer 1 (every
+      // wave is past its reads of it).
+      float* const s_base = lds_v + kVBuf + (wave * 2 * 16) * 64 + lane;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        s_base[v * 64] = acc[0][v] + acc[1][v] + acc[2][v];
+        s_base[(16 + v) * 64] = acc[1][v] - acc[2][v] - acc[3][v];
+      }
+      __syncthreads();
+      wino_stream_store(lds_v + kVBuf, lds_tile_off[0], lds_tile_flags[0],
+                        (unit - slot) / stride, f_lo + unit % f_cnt, tid, g,
+                        out, out_bytes, bias, relu);
+      __syncthreads();
+      u_base = u_next;
+    }
+  }
+}
+
 inline bool aligned16(const void* p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }
@@ -524,6 +869,23 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
                        dim3(512), 0, stream, input, workspace, output, g,
                        in_bytes, u_bytes, out_bytes, ug, per_split,
                        static_cast<const float*>(nullptr), 0);
+  } else if (n_chunks % 2 == 0) {
+    // The bias vector is read 16 bytes at a time.
+    const bool fuse = epilogue != nullptr && epilogue->wanted() && !backprop &&
+                      (epilogue->bias == nullptr || aligned16(epilogue->bias));
+    // Persistent work-groups, two per CU (32 CUs per XCD), fewer when an XCD
+    // has fewer units.
+    const unsigned per_xcd = grid_x / 8u;
+    const unsigned groups_per_xcd = per_xcd < 64u ? per_xcd : 64u;
+    KernelTimer timer(stream);
+    hipLaunchKernelGGL(wino_stream_kernel, dim3(8u * groups_per_xcd),
+                       dim3(512), 0, stream, input, workspace, output, g,
+                       in_bytes, u_bytes, out_bytes, ug,
+                       1.0f / static_cast<float>(g.tile_cols),
+                       1.0f / static_cast<float>(g.tile_rows),
+                       fuse ? epilogue->bias : nullptr,
+                       fuse && epilogue->relu ? 1 : 0);
+    if (fuse && epilogue->applied != nullptr) *epilogue->applied = true;
   } else {
     // The bias vector is read 16 bytes at a time.
     const bool fuse = epilogue != nullptr && epilogue->wanted() && !backprop &&

@@ -169,6 +169,11 @@ def test_ragged_shapes(shape, direction):
     (1, 7, 7, 512, 512, True),    # channel range split across work-groups
     (5, 6, 5, 48, 96, True),      # three chunks, three feature blocks
     (2, 30, 4, 64, 32, False),    # narrow image
+    # persistent work-groups that walk several units: 680 units of two
+    # chunks (a unit boundary every other chunk), clipped tiles, a ragged
+    # last tile block
+    (40, 33, 31, 32, 64, True),
+    (21, 45, 47, 96, 64, False),  # 666 units of six chunks, VALID
 ])
 def test_winograd_fused_shapes(shape, direction):
     batch, rows, cols, ch, feats, same = shape
@@ -1020,6 +1025,22 @@ def test_f16_pooling_forward():
     ref = oracle.pool_avg_forward(x.astype(np.float32), oracle_params(q, 0))
     got = ops.pooling_forward(dev(x, torch.float16), q, POOL_OP.AVERAGE)
     assert_close_f16(got.float().cpu().numpy(), ref, "f16 avg")
+
+
+def test_winograd_stream_bias_relu_matches_separate_launches():
+    """Bias and ReLU applied by the persistent Winograd kernel's stores give
+    the bits of convolution, bias add and ReLU run as three launches."""
+    p = ops.conv_params(40, 33, 31, 32, 64, 3, 1, True)
+    rng = np.random.default_rng(1717)
+    n_in, n_fil, n_out = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x, w = dev(uniform(rng, n_in)), dev(uniform(rng, n_fil))
+    bias = dev(uniform(rng, 64))
+    plain = ops.conv2d(x, w, p, DIRECTION.FORWARD, ALGO.WINOGRAD)
+    want = torch.relu(plain.view(-1, 64) + bias).view(-1)
+    got = ops.conv2d_bias_act(x, w, bias, p, ALGO.WINOGRAD, relu=True)
+    assert torch.equal(got, want)
+    got = ops.conv2d_bias_act(x, w, bias, p, ALGO.WINOGRAD, relu=False)
+    assert torch.equal(got, (plain.view(-1, 64) + bias).view(-1))
 
 
 def test_kernel_timing_brackets_the_main_kernel():
