@@ -85,7 +85,8 @@ __device__ inline float4 operator-(float4 a, float4 b) {
 // and feature roles swapped).
 __global__ void __launch_bounds__(256)
     wino_filter_pack_kernel(const float* __restrict__ w, float* __restrict__ u,
-                            int channels, int features, bool backprop) {
+                            int channels, int features, bool backprop,
+                            bool halves) {
   const int cin = backprop ? features : channels;
   const int cout = backprop ? channels : features;
   const int idx = blockIdx.x * 256 + threadIdx.x;
@@ -125,9 +126,16 @@ __global__ void __launch_bounds__(256)
   }
   const int fblocks = cout / kFeat;
   const int cgroups = cin / 8;
-  const int lane = co % kFeat + 32 * (cq & 1);
+  // Channel quad cq = ci / 4 goes to (channel group, lane half).  Default:
+  // group cq / 2, half cq % 2 (a group is 8 consecutive channels).  `halves`
+  // (cin % 16 == 0): within 16 channels the lower lane half takes channels
+  // 0 - 7 and the upper 8 - 15, so quad cq = 4 c16 + 2 half + q is group
+  // 2 c16 + q.
+  const int half = halves ? (cq >> 1) & 1 : cq & 1;
+  const int group = halves ? 2 * (cq >> 2) + (cq & 1) : cq >> 1;
+  const int lane = co % kFeat + 32 * half;
   const size_t base =
-      ((static_cast<size_t>(co / kFeat) * cgroups + cq / 2) * 64 + lane) * 4;
+      ((static_cast<size_t>(co / kFeat) * cgroups + group) * 64 + lane) * 4;
   const size_t xi_stride = static_cast<size_t>(fblocks) * cgroups * 256;
 #pragma unroll
   for (int xi = 0; xi < 16; ++xi) {
@@ -397,83 +405,67 @@ __global__ void __launch_bounds__(512)
   }
 }
 
-// At m A along xi's row index (across the multiplying waves, through `xch`)
-// and the stores of one unit; all 512 lanes take part.
-__device__ __forceinline__ void wino_stream_store(
-    const float* xch, const int* tile_off_tab, const int* tile_flags_tab,
-    int count, int fb, int tid, const FusedGeom& g, float* out,
-    unsigned out_bytes, const float* bias, int relu) {
-  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_bytes);
-  const unsigned out_row_bytes =
-      static_cast<unsigned>(g.out_cols) * g.out_ch * 4u;
-  const int ob = tid >> 8;
-  const int q = tid & 15;
-  const int v = (tid >> 4) & 15;
-  float4 s[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-    s[i] = *reinterpret_cast<const float4*>(xch + ((i * 2 + ob) * 16 + v) * 64 +
-                                            4 * q);
-  float4 y0 = s[0] + s[1] + s[2];
-  float4 y1 = s[1] - s[2] - s[3];
-  const int m = 8 * (v >> 2) + 4 * (q >> 3) + (v & 3);
-  const int f = fb * kFeat + 4 * (q & 7);
-  if (bias != nullptr) {
-    const float4 b4 = *reinterpret_cast<const float4*>(bias + f);
-    y0 = y0 + b4;
-    y1 = y1 + b4;
-  }
-  if (relu) {
-    y0 = make_float4(fmaxf(y0.x, 0.f), fmaxf(y0.y, 0.f), fmaxf(y0.z, 0.f),
-                     fmaxf(y0.w, 0.f));
-    y1 = make_float4(fmaxf(y1.x, 0.f), fmaxf(y1.y, 0.f), fmaxf(y1.z, 0.f),
-                     fmaxf(y1.w, 0.f));
-  }
-  const int tile_off = tile_off_tab[(count & 3) * kTiles + m];
-  const int flags = tile_flags_tab[(count & 3) * kTiles + m];
-  const bool col_ok = tile_off >= 0 && (ob == 0 || (flags & 2) != 0);
-  const unsigned off0 = col_ok ? static_cast<unsigned>(tile_off) +
-                                     static_cast<unsigned>(ob * g.out_ch + f) *
-                                         4u
-                               : kOob;
-  const unsigned off1 =
-      (col_ok && (flags & 1) != 0) ? off0 + out_row_bytes : kOob;
-  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y0),
-                                         out_rsrc, off0, 0, 0);
-  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y1),
-                                         out_rsrc, off1, 0, 0);
-}
-
 // ---------------------------------------------------------------------------
-// Stream kernel: wino_fused_kernel's unit (32 tiles x 32 features), wave roles
-// (waves 0-3 multiply, waves 4-7 gather and transform) and LDS / operand
-// layouts, run by persistent work-groups.
+// Persistent direct-to-LDS kernel: wino_fused_kernel's unit (32 tiles x 32
+// features) and xi-row-per-wave multiplication, organised around what was
+// measured on this GPU:
 //
-// Timestamps inside wino_fused_kernel show that its chunk loop keeps the
-// vector ALUs busy (the fp32 matrix instructions run on them, so the
-// transform's additions and the multiplications share one resource) as long
-// as two work-groups overlap on a CU, but that a unit's prologue (tile index
-// arithmetic, first gather from memory, first transform: 2.7 - 6.7 us) and
-// epilogue (1.3 us) are nearly half of its 14 us on a 64-channel layer.
-// Here a work-group walks the units slot, slot + G, ... of its XCD as one
-// stream of 16-channel chunks: the transforming waves run ahead of the
-// multiplying ones across unit boundaries (gather two chunks ahead,
-// transform one ahead), so the next unit's index arithmetic and first loads
-// happen while the current one is being multiplied.  One barrier per chunk;
-// at the end of a unit At m A goes through the LDS buffer that was
-// multiplied last (two more barriers).  Requires an even number of chunks.
+//   * Timestamps inside wino_fused_kernel: a unit's prologue (tile index
+//     arithmetic, first gather from memory, first transform: 2.7 - 6.7 us)
+//     and epilogue (1.3 us) are nearly half of its 14 us on a 64-channel
+//     layer.  Here a work-group is persistent: it walks the units slot,
+//     slot + G, ... of its XCD as one stream of 16-channel chunks, and the
+//     next unit's index arithmetic and first loads happen while the current
+//     one is being multiplied.
+//   * The fp32 matrix instructions run on the vector ALUs: a wave of plain
+//     v_add_f32 next to a wave streaming v_mfma_f32_32x32x2_f32 on the same
+//     SIMD is issued nothing until that wave stops (whatever the waves' age
+//     or priority).  Waves that only transform therefore take turns with the
+//     multiplying waves instead of working alongside them.  Here no wave only
+//     transforms: the additions sit in the multiplying wave's own
+//     instruction stream.
+//   * Per wave-level load of an L2-resident buffer: an 8-byte-per-lane gather
+//     of 8 tiles x 64 bytes into registers costs 32 CU-cycles (16 B/clk), a
+//     contiguous 16-byte register load 28, a 16-byte load that writes LDS
+//     directly 13.5 (76 B/clk) whatever its address pattern.  64 register
+//     gathers and 32 B loads per chunk are about 2900 CU-cycles of
+//     vector-memory time per 2048 cycles of matrix instructions.  Here the
+//     patches go from memory to LDS with buffer_load ... lds.
+//
+//   A work-group is 4 waves; wave w owns the xi = 4w .. 4w+3 planes and
+//   fetches patch row w: 32 instructions per chunk and work-group, two 32 KiB
+//   raw buffers, the chunk after the current one in flight.
+//   raw[p][T][piece][t] is 16 bytes: pixel p of the 4x4 patch, tile 16 T + t,
+//   channels 4 piece .. 4 piece + 3.  Each wave reads the two patch rows its
+//   xi row combines (Bt d: d0 - d2, d1 + d2, d2 - d1, d1 - d3), applies the
+//   column transform in registers and feeds the results to the matrix
+//   instructions as the A operand: lane (tile, half) covers channels
+//   8 half .. 8 half + 7 of the chunk (the filter pack orders U to match).
+//   The transformed input never exists in memory.  One barrier per chunk; at
+//   the end of a unit At m A goes through the raw buffer that was multiplied
+//   last (two more barriers).
+//
+// Two work-groups per CU (2 x 65 KiB LDS, up to 256 registers).  Requires an
+// even number of chunks.
 // ---------------------------------------------------------------------------
-__global__ void __launch_bounds__(512)
-    __attribute__((amdgpu_waves_per_eu(4, 4)))
-    wino_stream_kernel(const float* __restrict__ in,
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+constexpr int kWaitVm8 = 0x0F78;  // s_waitcnt vmcnt(8)
+
+__global__ void __launch_bounds__(256)
+    __attribute__((amdgpu_waves_per_eu(2, 2)))
+    wino_direct_kernel(const float* __restrict__ in,
                        const float* __restrict__ u, float* __restrict__ out,
                        FusedGeom g, unsigned in_bytes, unsigned u_bytes,
                        unsigned out_bytes, UnitGrid ug, float inv_tile_cols,
                        float inv_tile_rows, const float* __restrict__ bias,
                        int relu) {
-  __shared__ __align__(16) float lds_v[2 * kVBuf];
-  __shared__ int lds_tile_off[4][kTiles];
-  __shared__ int lds_tile_flags[4][kTiles];
+  // Two raw buffers as two objects: the compiler then knows that the loads
+  // that fill one do not touch the one being read, and does not make the
+  // reads wait for them.
+  __shared__ __align__(16) float lds_raw0[kVBuf];
+  __shared__ __align__(16) float lds_raw1[kVBuf];
+  __shared__ int lds_tile_off[2][kTiles];
+  __shared__ int lds_tile_flags[2][kTiles];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -491,20 +483,21 @@ __global__ void __launch_bounds__(512)
   if (slot >= n_local) return;  // whole group, before any barrier
   const int n_chunks = g.in_ch / kChunk;
 
-  if (wave >= 4) {
-    // ---- gather + transform waves ----------------------------------------
-    const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_bytes);
-    const int ptid = tid - 256;
-    const int tile_l = ptid >> 3, pair = ptid & 7;
-    unsigned p_off[16];
-    int g_unit = slot;   // unit (index within the XCD) the gather is in
-    int g_count = 0;     // units the gather has entered before it
-    int g_chunk = 0;     // next chunk to load
-    // Patch offsets of this lane's tile in unit `unit`; every offset is out
-    // of range (loads return zero, nothing is fetched) past the last unit.
-    auto enter_unit = [&](int unit, int count) {
-      const bool any = unit < n_local;
-      const int mb = m_lo + unit / f_cnt;
+  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_bytes);
+  const __amdgpu_buffer_rsrc_t u_rsrc = make_rsrc(u, u_bytes);
+
+  // ---- gather: lane (piece, t) of instruction (patch column pc, T) --------
+  const int g_piece = lane >> 4, g_t = lane & 15;
+  unsigned p_off[2][4];
+  // Offsets of patch row `wave` of tiles t and 16 + t of unit `unit`, all out
+  // of range (the loads then write zeros and fetch nothing) past the last
+  // unit.  Wave 0 also notes where the unit's tiles go in the output.
+  auto enter_unit = [&](int unit, int count) {
+    const bool any = unit < n_local;
+    const int mb = m_lo + unit / f_cnt;
+#pragma unroll
+    for (int T = 0; T < 2; ++T) {
+      const int tile_l = 16 * T + g_t;
       const int tile = mb * kTiles + tile_l;
       const bool live = any && tile < g.n_tiles;
       // tile = (n * tile_rows + ty) * tile_cols + tx with tile < 2^23: the
@@ -517,228 +510,243 @@ __global__ void __launch_bounds__(512)
       int ty = t2 - n * g.tile_rows;
       if (ty < 0) { ty += g.tile_rows; --n; }
       if (ty >= g.tile_rows) { ty -= g.tile_rows; ++n; }
-      const int y0 = 2 * ty - g.pad_rows, x0 = 2 * tx - g.pad_cols;
-      unsigned row_off[4], col_off[4];
-      bool row_ok[4], col_ok[4];
+      const int y = 2 * ty - g.pad_rows + wave;
+      const int x0 = 2 * tx - g.pad_cols;
+      const bool row_ok = live && static_cast<unsigned>(y) <
+                                      static_cast<unsigned>(g.in_rows);
+      const unsigned row_off =
+          static_cast<unsigned>((n * g.in_rows + y) * g.in_cols) *
+              static_cast<unsigned>(g.in_ch) * 4u +
+          static_cast<unsigned>(g_piece) * 16u;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int y = y0 + i, x = x0 + i;
-        row_ok[i] = live && static_cast<unsigned>(y) <
-                                static_cast<unsigned>(g.in_rows);
-        col_ok[i] =
-            static_cast<unsigned>(x) < static_cast<unsigned>(g.in_cols);
-        row_off[i] = static_cast<unsigned>((n * g.in_rows + y) * g.in_cols) *
-                     static_cast<unsigned>(g.in_ch) * 4u;
-        col_off[i] = static_cast<unsigned>(x * g.in_ch + 2 * pair) * 4u;
+      for (int pc = 0; pc < 4; ++pc) {
+        const int x = x0 + pc;
+        const bool ok = row_ok && static_cast<unsigned>(x) <
+                                      static_cast<unsigned>(g.in_cols);
+        p_off[T][pc] =
+            ok ? row_off + static_cast<unsigned>(x * g.in_ch) * 4u : kOob;
       }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          p_off[i * 4 + j] =
-              (row_ok[i] && col_ok[j]) ? row_off[i] + col_off[j] : kOob;
-      if (pair == 0) {
-        lds_tile_off[count & 3][tile_l] =
+      if (wave == 0 && g_piece == 0) {
+        lds_tile_off[count & 1][tile_l] =
             live ? ((n * g.out_rows + 2 * ty) * g.out_cols + 2 * tx) *
                        g.out_ch * 4
                  : -1;
-        lds_tile_flags[count & 3][tile_l] =
+        lds_tile_flags[count & 1][tile_l] =
             (2 * ty + 1 < g.out_rows ? 1 : 0) |
             (2 * tx + 1 < g.out_cols ? 2 : 0);
       }
-    };
-    auto load_patch = [&](float2 (&d)[16]) {
-      const unsigned soff = static_cast<unsigned>(g_chunk * kChunk * 4);
-#pragma unroll
-      for (int q = 0; q < 16; ++q)
-        d[q] = __builtin_bit_cast(
-            float2,
-            __builtin_amdgcn_raw_buffer_load_b64(in_rsrc, p_off[q], soff, 0));
-      if (++g_chunk == n_chunks) {
-        g_chunk = 0;
-        g_unit += stride;
-        ++g_count;
-        enter_unit(g_unit, g_count);
-      }
-    };
-    float* const v_store =
-        lds_v + tile_l * kChunk + 4 * ((pair >> 1) ^ ((tile_l >> 1) & 3)) +
-        2 * (pair & 1);
-    auto transform_store = [&](const float2 (&d)[16], int buf) {
-      float* const dst = v_store + buf * kVBuf;
-      float2 t[4][4];  // Bt d
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        t[0][j] = d[0 * 4 + j] - d[2 * 4 + j];
-        t[1][j] = d[1 * 4 + j] + d[2 * 4 + j];
-        t[2][j] = d[2 * 4 + j] - d[1 * 4 + j];
-        t[3][j] = d[1 * 4 + j] - d[3 * 4 + j];
-      }
-      constexpr int kXi = kTiles * kChunk;  // floats per xi plane
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        *reinterpret_cast<float2*>(dst + (i * 4 + 0) * kXi) =
-            t[i][0] - t[i][2];
-        *reinterpret_cast<float2*>(dst + (i * 4 + 1) * kXi) =
-            t[i][1] + t[i][2];
-        *reinterpret_cast<float2*>(dst + (i * 4 + 2) * kXi) =
-            t[i][2] - t[i][1];
-        *reinterpret_cast<float2*>(dst + (i * 4 + 3) * kXi) =
-            t[i][1] - t[i][3];
-      }
-    };
-    // The fences keep every load where it is written: left alone, the
-    // compiler moves loads across the transforms into spare registers and
-    // then waits for the newest loads instead of the oldest.
-    float2 d_even[16], d_odd[16];
-    enter_unit(g_unit, 0);
-    load_patch(d_even);
-    __builtin_amdgcn_sched_barrier(0);
-    transform_store(d_even, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    load_patch(d_odd);
-    __builtin_amdgcn_sched_barrier(0);
-    __syncthreads();
-    for (int unit = slot; unit < n_local; unit += stride) {
-      for (int c = 0; c < n_chunks; c += 2) {
-        // An even chunk is being multiplied from buffer 0.  The loads of the
-        // chunk after next are issued first, right behind the barrier, so
-        // that they queue up in the memory pipeline while the multiplying
-        // waves hold the ALUs; the transform then only has its additions and
-        // LDS writes between the moment those waves stop and the barrier.
-        load_patch(d_even);
-        __builtin_amdgcn_sched_barrier(0);
-        transform_store(d_odd, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
-        // an odd chunk is being multiplied from buffer 1; the last one of a
-        // unit leaves the next unit's first chunk in buffer 0
-        load_patch(d_odd);
-        __builtin_amdgcn_sched_barrier(0);
-        transform_store(d_even, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
-      }
-      __syncthreads();  // multiplying waves write At m A (columns) to buffer 1
-      wino_stream_store(lds_v + kVBuf, lds_tile_off[0], lds_tile_flags[0],
-                        (unit - slot) / stride, f_lo + unit % f_cnt, tid, g,
-                        out, out_bytes, bias, relu);
-      __syncthreads();  // buffer 1 is free again
     }
-  } else {
-    // ---- multiplying waves -----------------------------------------------
-    const __amdgpu_buffer_rsrc_t u_rsrc = make_rsrc(u, u_bytes);
-    const unsigned n_fblocks = static_cast<unsigned>(ug.n_fblocks);
-    const unsigned u_lane = static_cast<unsigned>(lane) * 16u;
-    const unsigned cgroups = static_cast<unsigned>(g.in_ch) / 8u;
-    // Byte offset of U[xi = 4 wave][feature block of `unit`][channel group 0].
-    auto u_base_of = [&](int unit) {
-      const unsigned fb = static_cast<unsigned>(f_lo + unit % f_cnt);
-      return static_cast<unsigned>(__builtin_amdgcn_readfirstlane(
-          ((static_cast<unsigned>(4 * wave) * n_fblocks + fb) * cgroups) *
-          1024u));
-    };
-    const unsigned u_xi_stride = n_fblocks * cgroups * 1024u;
-    auto load_b = [&](unsigned base, int cgroup, int j) {
-      return __builtin_bit_cast(
-          float4, __builtin_amdgcn_raw_buffer_load_b128(
-                      u_rsrc, u_lane,
-                      base + static_cast<unsigned>(j) * u_xi_stride +
-                          static_cast<unsigned>(cgroup) * 1024u,
-                      0));
-    };
-    const int tile_r = lane & 31;
-    const int swz = (tile_r >> 1) & 3;
-    constexpr int kXi = kTiles * kChunk;
-    const float* const a_base = lds_v + (4 * wave * kTiles + tile_r) * kChunk;
-    const int a_grp0 = 4 * ((0 + (lane >> 5)) ^ swz);
-    const int a_grp1 = 4 * ((2 + (lane >> 5)) ^ swz);
-    auto load_a = [&](const float* a_ptr, int j) {
-      return *reinterpret_cast<const float4*>(a_ptr + j * kXi);
-    };
-    float16v acc[4];
-    // Eight matrix instructions: two xi planes, four reduction steps each.
-    auto mma_pair = [&](int j, const float4& a0, const float4& a1,
-                        const float4& b0, const float4& b1) {
+  };
+  // One of the eight loads of patch row `wave` of chunk `chunk` into a raw
+  // buffer: instruction i = (pc, T) fills the 1 KiB block (4 wave + pc) * 2 + T.
+  auto gather = [&](float* raw, int chunk, int i) {
+    const unsigned soff = static_cast<unsigned>(chunk * kChunk * 4);
+    char* const dst = reinterpret_cast<char*>(raw) + wave * 8 * 1024;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        in_rsrc, (lds_void_ptr)(dst + i * 1024), 16, p_off[i & 1][i >> 1],
+        soff, 0, 0);
+  };
+
+  // ---- multiply: lane (tile, half) ---------------------------------------
+  const int tile_r = lane & 31, half = lane >> 5;
+  const unsigned n_fblocks = static_cast<unsigned>(ug.n_fblocks);
+  const unsigned u_lane = static_cast<unsigned>(lane) * 16u;
+  const unsigned cgroups = static_cast<unsigned>(g.in_ch) / 8u;
+  // Byte offset of U[xi = 4 wave][feature block of `unit`][channel group 0].
+  auto u_base_of = [&](int unit) {
+    const unsigned fb = static_cast<unsigned>(f_lo + unit % f_cnt);
+    return static_cast<unsigned>(__builtin_amdgcn_readfirstlane(
+        ((static_cast<unsigned>(4 * wave) * n_fblocks + fb) * cgroups) *
+        1024u));
+  };
+  const unsigned u_xi_stride = n_fblocks * cgroups * 1024u;
+  auto load_b = [&](unsigned base, int cgroup, int j) {
+    return __builtin_bit_cast(
+        float4, __builtin_amdgcn_raw_buffer_load_b128(
+                    u_rsrc, u_lane,
+                    base + static_cast<unsigned>(j) * u_xi_stride +
+                        static_cast<unsigned>(cgroup) * 1024u,
+                    0));
+  };
+  // Bt d for xi row `wave`: patch rows ra and rb, t = d[ra] + sgn d[rb].
+  const int ra = wave == 0 ? 0 : (wave == 2 ? 2 : 1);
+  const int rb = wave == 0 ? 2 : (wave == 1 ? 2 : (wave == 2 ? 1 : 3));
+  const float sgn = wave == 1 ? 1.f : -1.f;
+  // 16-byte piece (row r, column 0, this lane's tile, channel quad 2 half)
+  // of a raw buffer; columns are 128 pieces apart, the second quad 16.
+  const int piece_t = ((tile_r >> 4) * 4 + 2 * half) * 16 + (tile_r & 15);
+  const int raw_a = (ra * 4 * 128 + piece_t) * 4;
+  const int raw_b = (rb * 4 * 128 + piece_t) * 4;
+  auto read_rows = [&](const float* raw, int q, float4 (&da)[4],
+                       float4 (&db)[4]) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(comp(a0, t), comp(b0, t),
-                                                      acc[j], 0, 0, 0);
-        acc[j + 1] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-            comp(a1, t), comp(b1, t), acc[j + 1], 0, 0, 0);
-      }
-    };
-    float4 b[2][4];
-    // One chunk: four quarters (channel half, xi pair).  The B registers of a
-    // quarter are refilled for the chunk after (nb_base, nb_cg) as soon as
-    // its matrix instructions have been issued; the fences keep the compiler
-    // from sinking those loads to the end of the chunk.
-    auto multiply = [&](int buf, unsigned nb_base, int nb_cg) {
-      const float* const a_buf = a_base + buf * kVBuf;
-      float4 a[4];
+    for (int pc = 0; pc < 4; ++pc) {
+      da[pc] = *reinterpret_cast<const float4*>(raw + raw_a +
+                                                (pc * 128 + q * 16) * 4);
+      db[pc] = *reinterpret_cast<const float4*>(raw + raw_b +
+                                                (pc * 128 + q * 16) * 4);
+    }
+  };
+  auto fma4 = [&](const float4& x, const float4& y) {
+    return make_float4(fmaf(y.x, sgn, x.x), fmaf(y.y, sgn, x.y),
+                       fmaf(y.z, sgn, x.z), fmaf(y.w, sgn, x.w));
+  };
+  // (Bt d B) for this wave's xi row: a[j], four channels each.
+  auto transform = [&](const float4 (&da)[4], const float4 (&db)[4],
+                       float4 (&a)[4]) {
+    const float4 t0 = fma4(da[0], db[0]), t1 = fma4(da[1], db[1]);
+    const float4 t2 = fma4(da[2], db[2]), t3 = fma4(da[3], db[3]);
+    a[0] = t0 - t2;
+    a[1] = t1 + t2;
+    a[2] = t2 - t1;
+    a[3] = t1 - t3;
+  };
+  float16v acc[4];
+  // Four matrix instructions: reduction step e of the four xi planes.
+  auto mma_group = [&](const float4 (&a)[4], const float4 (&b)[4], int e) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) a[j] = load_a(a_buf + a_grp0, j);
-      __builtin_amdgcn_sched_barrier(0);
-      mma_pair(0, a[0], a[1], b[0][0], b[0][1]);
-      __builtin_amdgcn_sched_barrier(0);
-      a[0] = load_a(a_buf + a_grp1, 0);
-      a[1] = load_a(a_buf + a_grp1, 1);
-      b[0][0] = load_b(nb_base, nb_cg, 0);
-      b[0][1] = load_b(nb_base, nb_cg, 1);
-      __builtin_amdgcn_sched_barrier(0);
-      mma_pair(2, a[2], a[3], b[0][2], b[0][3]);
-      __builtin_amdgcn_sched_barrier(0);
-      a[2] = load_a(a_buf + a_grp1, 2);
-      a[3] = load_a(a_buf + a_grp1, 3);
-      b[0][2] = load_b(nb_base, nb_cg, 2);
-      b[0][3] = load_b(nb_base, nb_cg, 3);
-      __builtin_amdgcn_sched_barrier(0);
-      mma_pair(0, a[0], a[1], b[1][0], b[1][1]);
-      __builtin_amdgcn_sched_barrier(0);
-      b[1][0] = load_b(nb_base, nb_cg + 1, 0);
-      b[1][1] = load_b(nb_base, nb_cg + 1, 1);
-      __builtin_amdgcn_sched_barrier(0);
-      mma_pair(2, a[2], a[3], b[1][2], b[1][3]);
-      __builtin_amdgcn_sched_barrier(0);
-      b[1][2] = load_b(nb_base, nb_cg + 1, 2);
-      b[1][3] = load_b(nb_base, nb_cg + 1, 3);
-      __builtin_amdgcn_sched_barrier(0);
-      __syncthreads();
-    };
-    unsigned u_base = u_base_of(slot);
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) b[h][j] = load_b(u_base, h, j);
+    for (int j = 0; j < 4; ++j)
+      acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(comp(a[j], e),
+                                                    comp(b[j], e), acc[j], 0,
+                                                    0, 0);
+  };
+  // B operand: b0 for the first channel quad of a chunk, b1x / b1y in turn
+  // for the second.
+  float4 b0[4], b1x[4], b1y[4];
+  // One chunk from `raw`.  Every vector-memory instruction sits behind a
+  // group of four matrix instructions (256 cycles of matrix work), so the
+  // texture path takes them one at a time and the wave never stands at a
+  // full queue: the eight gather loads of the next chunk of the stream
+  // (chunk g_chunk of the unit the offsets are set for; into the other raw
+  // buffer, which every wave finished reading before the barrier) behind
+  // the groups of the first quad, and behind those of the second quad the
+  // refills of b0 (used up by then) and of the idle b1 for the chunk after
+  // (nb_base, nb_cg).  The fences keep the compiler from collecting the
+  // loads in one place.
+  auto step = [&](const float* raw, float* raw_next, int g_chunk,
+                  float4 (&b1)[4], float4 (&b1_idle)[4], unsigned nb_base,
+                  int nb_cg) {
+    float4 da[4], db[4], a0[4], a1[4];
+    read_rows(raw, 0, da, db);
     __builtin_amdgcn_sched_barrier(0);
+    transform(da, db, a0);
+    __builtin_amdgcn_sched_barrier(0);
+    read_rows(raw, 1, da, db);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      mma_group(a0, b0, e);
+      __builtin_amdgcn_sched_barrier(0);
+      gather(raw_next, g_chunk, 2 * e);
+      gather(raw_next, g_chunk, 2 * e + 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    transform(da, db, a1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      mma_group(a1, b1, e);
+      __builtin_amdgcn_sched_barrier(0);
+      b0[e] = load_b(nb_base, nb_cg, e);
+      b1_idle[e] = load_b(nb_base, nb_cg + 1, e);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // The gather (eight loads, issued before the eight B loads) has landed.
+    __builtin_amdgcn_s_waitcnt(kWaitVm8);
     __syncthreads();
-    for (int unit = slot; unit < n_local; unit += stride) {
+  };
+
+  // ---- start of the stream ------------------------------------------------
+  enter_unit(slot, 0);
+  unsigned u_base = u_base_of(slot);
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+  for (int i = 0; i < 8; ++i) gather(lds_raw0, 0, i);
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
-      const int next_unit = unit + stride < n_local ? unit + stride : unit;
-      const unsigned u_next = u_base_of(next_unit);
-      for (int c = 0; c < n_chunks; c += 2) {
-        multiply(0, u_base, 2 * (c + 1));
-        const bool last = c + 2 >= n_chunks;
-        multiply(1, last ? u_next : u_base, last ? 0 : 2 * (c + 2));
-      }
-      // At m A along xi's column index, inside the lane, into buffer 1 (every
-      // wave is past its reads of it).
-      float* const s_base = lds_v + kVBuf + (wave * 2 * 16) * 64 + lane;
+  for (int j = 0; j < 4; ++j) {
+    b0[j] = load_b(u_base, 0, j);
+    b1x[j] = load_b(u_base, 1, j);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_waitcnt(kWaitVm8);
+  __syncthreads();
+
+  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_bytes);
+  const unsigned out_row_bytes =
+      static_cast<unsigned>(g.out_cols) * g.out_ch * 4u;
+  int count = 0;
+  for (int unit = slot; unit < n_local; unit += stride, ++count) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+    const int next_unit = unit + stride < n_local ? unit + stride : unit;
+    const unsigned u_next = u_base_of(next_unit);
+    // The unit's bias is fetched now: a load issued at the end of the unit
+    // would have to wait for every load issued before it, the next unit's
+    // first gather among them.
+    const int fb = f_lo + unit % f_cnt;
+    const int f = fb * kFeat + 4 * (tid & 7);
+    float4 b4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (bias != nullptr) b4 = *reinterpret_cast<const float4*>(bias + f);
+    for (int c = 0; c < n_chunks; c += 2) {
+      step(lds_raw0, lds_raw1, c + 1, b1x, b1y, u_base, 2 * (c + 1));
+      const bool last = c + 2 >= n_chunks;
+      // The last chunk of a unit gathers the first one of the next unit.
+      if (last) enter_unit(unit + stride, count + 1);
+      step(lds_raw1, lds_raw0, last ? 0 : c + 2, b1y, b1x,
+           last ? u_next : u_base, last ? 0 : 2 * (c + 2));
+    }
+    // At m A: along xi's column index inside the lane, into raw buffer 1
+    // (every wave is past its reads of it; buffer 0 is being filled) ...
+    {
+      float* const s_base = lds_raw1 + (wave * 2 * 16) * 64 + lane;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         s_base[v * 64] = acc[0][v] + acc[1][v] + acc[2][v];
         s_base[(16 + v) * 64] = acc[1][v] - acc[2][v] - acc[3][v];
       }
-      __syncthreads();
-      wino_stream_store(lds_v + kVBuf, lds_tile_off[0], lds_tile_flags[0],
-                        (unit - slot) / stride, f_lo + unit % f_cnt, tid, g,
-                        out, out_bytes, bias, relu);
-      __syncthreads();
-      u_base = u_next;
     }
+    __syncthreads();
+    // ... then along its row index across the waves.
+    const int q = tid & 15;
+    const int v = (tid >> 4) & 15;
+    const int m = 8 * (v >> 2) + 4 * (q >> 3) + (v & 3);
+    const int tile_off = lds_tile_off[count & 1][m];
+    const int flags = lds_tile_flags[count & 1][m];
+#pragma unroll
+    for (int ob = 0; ob < 2; ++ob) {
+      float4 s[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        s[i] = *reinterpret_cast<const float4*>(
+            lds_raw1 + ((i * 2 + ob) * 16 + v) * 64 + 4 * q);
+      float4 y0 = s[0] + s[1] + s[2];
+      float4 y1 = s[1] - s[2] - s[3];
+      if (bias != nullptr) {
+        y0 = y0 + b4;
+        y1 = y1 + b4;
+      }
+      if (relu) {
+        y0 = make_float4(fmaxf(y0.x, 0.f), fmaxf(y0.y, 0.f), fmaxf(y0.z, 0.f),
+                         fmaxf(y0.w, 0.f));
+        y1 = make_float4(fmaxf(y1.x, 0.f), fmaxf(y1.y, 0.f), fmaxf(y1.z, 0.f),
+                         fmaxf(y1.w, 0.f));
+      }
+      const bool col_ok = tile_off >= 0 && (ob == 0 || (flags & 2) != 0);
+      const unsigned off0 =
+          col_ok ? static_cast<unsigned>(tile_off) +
+                       static_cast<unsigned>(ob * g.out_ch + f) * 4u
+                 : kOob;
+      const unsigned off1 =
+          (col_ok && (flags & 1) != 0) ? off0 + out_row_bytes : kOob;
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y0),
+                                             out_rsrc, off0, 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y1),
+                                             out_rsrc, off1, 0, 0);
+    }
+    __syncthreads();  // raw buffer 1 is free for the next unit's second chunk
+    u_base = u_next;
   }
 }
 
@@ -797,11 +805,6 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
   const size_t out_elems = static_cast<size_t>(p.batch) * g.out_rows *
                            g.out_cols * g.out_ch;
 
-  hipLaunchKernelGGL(wino_filter_pack_kernel,
-                     dim3(ceil_div((g.in_ch / 4) * g.out_ch, 256)), dim3(256),
-                     0, stream, filter, workspace, p.channels, p.features,
-                     backprop);
-
   UnitGrid ug;
   ug.n_mblocks = ceil_div(g.n_tiles, kTiles);
   ug.n_fblocks = g.out_ch / kFeat;
@@ -858,6 +861,14 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
   const unsigned in_bytes = static_cast<unsigned>(in_elems * 4);
   const unsigned u_bytes = static_cast<unsigned>(u_elems * 4);
   const unsigned out_bytes = static_cast<unsigned>(out_elems * 4);
+  // The persistent kernel takes every launch that is not split and has an
+  // even number of chunks; it wants U with the channels of a chunk dealt to
+  // the lane halves eight at a time.
+  const bool persistent = splits == 1 && n_chunks % 2 == 0;
+  hipLaunchKernelGGL(wino_filter_pack_kernel,
+                     dim3(ceil_div((g.in_ch / 4) * g.out_ch, 256)), dim3(256),
+                     0, stream, filter, workspace, p.channels, p.features,
+                     backprop, persistent);
   if (splits > 1) {
     const size_t n_vec = out_elems / 4;  // out_ch % 32 == 0
     hipLaunchKernelGGL(wino_zero_fill_kernel,
@@ -869,7 +880,7 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
                        dim3(512), 0, stream, input, workspace, output, g,
                        in_bytes, u_bytes, out_bytes, ug, per_split,
                        static_cast<const float*>(nullptr), 0);
-  } else if (n_chunks % 2 == 0) {
+  } else if (persistent) {
     // The bias vector is read 16 bytes at a time.
     const bool fuse = epilogue != nullptr && epilogue->wanted() && !backprop &&
                       (epilogue->bias == nullptr || aligned16(epilogue->bias));
@@ -878,8 +889,8 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
     const unsigned per_xcd = grid_x / 8u;
     const unsigned groups_per_xcd = per_xcd < 64u ? per_xcd : 64u;
     KernelTimer timer(stream);
-    hipLaunchKernelGGL(wino_stream_kernel, dim3(8u * groups_per_xcd),
-                       dim3(512), 0, stream, input, workspace, output, g,
+    hipLaunchKernelGGL(wino_direct_kernel, dim3(8u * groups_per_xcd),
+                       dim3(256), 0, stream, input, workspace, output, g,
                        in_bytes, u_bytes, out_bytes, ug,
                        1.0f / static_cast<float>(g.tile_cols),
                        1.0f / static_cast<float>(g.tile_rows),
