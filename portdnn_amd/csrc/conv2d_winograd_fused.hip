@@ -93,6 +93,18 @@ __global__ void __launch_bounds__(256)
   if (idx >= (cin / 4) * cout) return;
   const int co = idx % cout, cq = idx / cout;
   float uu[16][4];
+  // The four channels of the quad are contiguous in W for the input gradient
+  // (W[2-r][2-s][co][ci]): one 16-byte load per tap.
+  float4 gq[3][3];
+  if (backprop) {
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+      for (int s = 0; s < 3; ++s)
+        gq[r][s] = *reinterpret_cast<const float4*>(
+            w + ((static_cast<size_t>(2 - r) * 3 + (2 - s)) * channels + co) *
+                    features + 4 * cq);
+  }
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
     const int ci = 4 * cq + t;
@@ -103,8 +115,7 @@ __global__ void __launch_bounds__(256)
       for (int s = 0; s < 3; ++s) {
         g[r][s] =
             backprop
-                ? w[((static_cast<size_t>(2 - r) * 3 + (2 - s)) * channels +
-                     co) * features + ci]
+                ? comp(gq[r][s], t)
                 : w[((static_cast<size_t>(r) * 3 + s) * channels + ci) *
                         features + co];
       }
@@ -798,7 +809,8 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
                            g.tile_cols * (g.in_ch + g.out_ch);
   if (workspace == nullptr || workspace_elems < u_elems + per_image)
     return SNN_HIP_INSUFFICIENT_WORKSPACE;
-  if (!aligned16(workspace) || !aligned16(input) || !aligned16(output))
+  if (!aligned16(workspace) || !aligned16(input) || !aligned16(output) ||
+      (backprop && !aligned16(filter)))
     return SNN_HIP_INVALID_PARAMETER;
   const size_t in_elems = static_cast<size_t>(p.batch) * g.in_rows *
                           g.in_cols * g.in_ch;

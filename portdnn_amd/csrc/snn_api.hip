@@ -396,8 +396,10 @@ int launch_winograd_path<float>(int direction, const float* input,
                                 hipStream_t s, const LaunchOptions* epilogue) {
   // SNN_HIP_WINO_UNFUSED is a development switch that forces the three-stage
   // chain on shapes the fused kernel would take.
+  // (the input gradient's filter transform reads the filter 16 bytes at a time)
   if (conv2d_winograd_fused_supports(direction, p) && aligned16(input) &&
       aligned16(output) && aligned16(workspace) &&
+      (direction != SNN_HIP_INPUT_BACKPROP || aligned16(filter)) &&
       SNN_TUNING_ENV("SNN_HIP_WINO_UNFUSED") == nullptr)
     return launch_conv2d_winograd_fused_f32(direction, input, filter, output,
                                             p, workspace, workspace_elems, s,
