@@ -1027,6 +1027,35 @@ def test_f16_pooling_forward():
     assert_close_f16(got.float().cpu().numpy(), ref, "f16 avg")
 
 
+def _winograd_sweep_shapes():
+    """Seeded shapes for the persistent Winograd kernel: even numbers of
+    16-channel chunks, odd image sizes, both paddings, tile counts that leave
+    ragged last tile blocks, enough units for a work-group to walk several."""
+    rng = np.random.default_rng(20261125)
+    shapes = []
+    while len(shapes) < 14:
+        ch = int(rng.choice([32, 64, 96, 128]))
+        feats = int(rng.choice([32, 64, 96, 160]))
+        rows, cols = int(rng.integers(5, 40)), int(rng.integers(5, 40))
+        same = bool(rng.integers(0, 2))
+        if not same and min(rows, cols) < 4:
+            continue
+        # keep the oracle to about a second per case
+        batch = int(max(1, min(48, 1.2e9 // (rows * cols * 18 * ch * feats))))
+        shapes.append((batch, rows, cols, ch, feats, same))
+    return shapes
+
+
+@pytest.mark.parametrize("direction", [DIRECTION.FORWARD,
+                                       DIRECTION.INPUT_BACKPROP])
+@pytest.mark.parametrize("shape", _winograd_sweep_shapes())
+def test_winograd_persistent_kernel_sweep(shape, direction):
+    batch, rows, cols, ch, feats, same = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, 3, 1, same)
+    conv_case(p, direction, [ALGO.WINOGRAD],
+              seed=4000 + 7 * rows + 3 * cols + ch + feats)
+
+
 def test_winograd_stream_bias_relu_matches_separate_launches():
     """Bias and ReLU applied by the persistent Winograd kernel's stores give
     the bits of convolution, bias add and ReLU run as three launches."""
