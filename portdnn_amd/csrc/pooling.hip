@@ -945,14 +945,14 @@ __global__ void __launch_bounds__(256)
 // (src/pooling/kernels.h:197-239) -- and carries those two positions and dY
 // values down as the "windows above" of the next block row.  Each dX pixel
 // adds its windows in output-row, output-column order.
-template <int TH>
+template <int TH, bool NAN_MODE>
 __global__ void __launch_bounds__(256)
     pool_max_grad_3x3_s2_kernel(const float* __restrict__ in,
                                 const float* __restrict__ out,
                                 const float* __restrict__ dy,
                                 float* __restrict__ dx, snn_hip_pooling_params p,
-                                bool nan_mode, int n_bcols, int n_strips,
-                                unsigned n_items) {
+                                int n_bcols, int n_strips, unsigned n_items) {
+  constexpr bool nan_mode = NAN_MODE;
   const unsigned idx = blockIdx.x * 256u + threadIdx.x;
   if (idx >= n_items) return;
   const int C = p.channels;
@@ -1027,22 +1027,40 @@ __global__ void __launch_bounds__(256)
     load_in_row(y + 2, rows[2]);
     const bool win_row_ok = static_cast<unsigned>(br0 - 1) <
                             static_cast<unsigned>(p.out_rows);
+    const bool interior =
+        y >= 0 && y + 2 < p.in_rows && x_ok[0] && x_ok[1] && x_ok[2] &&
+        x_ok[3] && x_ok[4] && win_row_ok && w_ok[0] && w_ok[1];
+    if (__builtin_amdgcn_ballot_w64(!interior) == 0) {
 #pragma unroll
-    for (int w = 0; w < 2; ++w)
+      for (int w = 0; w < 2; ++w)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        int pos = 9;
+        for (int e = 0; e < 4; ++e) {
+          int pos = 9;
 #pragma unroll
-        for (int k = 8; k >= 0; --k) {
-          const int r = k / 3, c = k % 3;
-          const bool y_ok = static_cast<unsigned>(y + r) <
-                            static_cast<unsigned>(p.in_rows);
-          if (y_ok && x_ok[2 * w + c] &&
-              pool_equal(rows[r][2 * w + c][e], target[w][e], nan_mode))
-            pos = k;
+          for (int k = 8; k >= 0; --k)
+            if (pool_equal(rows[k / 3][2 * w + k % 3][e], target[w][e],
+                           nan_mode))
+              pos = k;
+          up_pos[w][e] = pos;
         }
-        up_pos[w][e] = (win_row_ok && w_ok[w]) ? pos : 9;
-      }
+    } else {
+#pragma unroll
+      for (int w = 0; w < 2; ++w)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          int pos = 9;
+#pragma unroll
+          for (int k = 8; k >= 0; --k) {
+            const int r = k / 3, c = k % 3;
+            const bool y_ok = static_cast<unsigned>(y + r) <
+                              static_cast<unsigned>(p.in_rows);
+            if (y_ok && x_ok[2 * w + c] &&
+                pool_equal(rows[r][2 * w + c][e], target[w][e], nan_mode))
+              pos = k;
+          }
+          up_pos[w][e] = (win_row_ok && w_ok[w]) ? pos : 9;
+        }
+    }
 #pragma unroll
     for (int j = 0; j < 5; ++j)
 #pragma unroll
@@ -1065,20 +1083,42 @@ __global__ void __launch_bounds__(256)
     const bool win_row_ok =
         static_cast<unsigned>(br) < static_cast<unsigned>(p.out_rows);
     int pos[2][4];
+    // Away from the image border every element of both windows exists for
+    // every lane of the wave: the search then is a compare and a select per
+    // element, with none of the per-element validity masks (scalar mask
+    // arithmetic that outnumbered the vector instructions of this kernel).
+    const bool interior = y_ok[0] && y_ok[1] && y_ok[2] && x_ok[0] &&
+                          x_ok[1] && x_ok[2] && x_ok[3] && x_ok[4] &&
+                          win_row_ok && w_ok[0] && w_ok[1];
+    if (__builtin_amdgcn_ballot_w64(!interior) == 0) {
 #pragma unroll
-    for (int w = 0; w < 2; ++w)
+      for (int w = 0; w < 2; ++w)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        int first = 9;
+        for (int e = 0; e < 4; ++e) {
+          int first = 9;
 #pragma unroll
-        for (int k = 8; k >= 0; --k) {
-          const int r = k / 3, c = k % 3;
-          if (y_ok[r] && x_ok[2 * w + c] &&
-              pool_equal(rows[r][2 * w + c][e], target[w][e], nan_mode))
-            first = k;
+          for (int k = 8; k >= 0; --k)
+            if (pool_equal(rows[k / 3][2 * w + k % 3][e], target[w][e],
+                           nan_mode))
+              first = k;
+          pos[w][e] = first;
         }
-        pos[w][e] = (win_row_ok && w_ok[w]) ? first : 9;
-      }
+    } else {
+#pragma unroll
+      for (int w = 0; w < 2; ++w)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          int first = 9;
+#pragma unroll
+          for (int k = 8; k >= 0; --k) {
+            const int r = k / 3, c = k % 3;
+            if (y_ok[r] && x_ok[2 * w + c] &&
+                pool_equal(rows[r][2 * w + c][e], target[w][e], nan_mode))
+              first = k;
+          }
+          pos[w][e] = (win_row_ok && w_ok[w]) ? first : 9;
+        }
+    }
     // the four dX pixels; windows in (output row, output column) order
     float ee[4], eo[4], oe[4], oo[4];
 #pragma unroll
@@ -1206,16 +1246,22 @@ int launch_pooling_max_grad(const float* input_data, const float* output_data,
     const int n_strips = ceil_div(n_brows, th);
     const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
     const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
-    if (th == 4)
-      hipLaunchKernelGGL(pool_max_grad_3x3_s2_kernel<4>, grid, dim3(kBlock), 0,
-                         stream, input_data, output_data, input_backprop,
-                         output_backprop, p, nan_mode, n_bcols, n_strips,
-                         n_items);
-    else
-      hipLaunchKernelGGL(pool_max_grad_3x3_s2_kernel<2>, grid, dim3(kBlock), 0,
-                         stream, input_data, output_data, input_backprop,
-                         output_backprop, p, nan_mode, n_bcols, n_strips,
-                         n_items);
+    auto launch = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, grid, dim3(kBlock), 0, stream, input_data,
+                         output_data, input_backprop, output_backprop, p,
+                         n_bcols, n_strips, n_items);
+    };
+    if (th == 4) {
+      if (nan_mode)
+        launch(pool_max_grad_3x3_s2_kernel<4, true>);
+      else
+        launch(pool_max_grad_3x3_s2_kernel<4, false>);
+    } else {
+      if (nan_mode)
+        launch(pool_max_grad_3x3_s2_kernel<2, true>);
+      else
+        launch(pool_max_grad_3x3_s2_kernel<2, false>);
+    }
   } else if (vec4 && square && p.window_rows == 3 && p.stride_rows == 2) {
     launch_max_grad_tile<3, 2>(input_data, output_data, input_backprop,
                                output_backprop, p, nan_mode, stream);
