@@ -234,8 +234,7 @@ def main():
         "mfma_executed_frac": frac(
             achieved * (WINOGRAD_SHARE if k3_algos == ["winograd"] else 1.0),
             PEAK_FP32_MFMA_TFLOPS),
-        "traffic": ((profiled_traffic_bytes("wino_stream_kernel") or
-                     profiled_traffic_bytes("wino_fused_kernel"))
+        "traffic": (profiled_traffic_bytes("wino_direct_kernel")
                     if k3_algos == ["winograd"] else None),
         "traffic_source": TRAFFIC_PROFILE}
 
