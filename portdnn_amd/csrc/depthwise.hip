@@ -604,13 +604,14 @@ __global__ void __launch_bounds__(kDwFilbkThreads)
 }
 
 // The same reduction with the input window kept in registers: a pixel lane
-// walks TH consecutive output rows of one output column and loads every input
-// row of that strip once (three column taps), so an output pixel costs
-// STRIDE * 3 + 1 vector loads instead of 10.  Strips are numbered column
-// fastest, (image, row block, column), and dealt to the pixel lanes in that
-// order; rows past the end of the image read zeros through the buffer range
-// check and add nothing.
-template <int STRIDE, int TH>
+// walks TH consecutive output rows of TW adjacent output columns and loads
+// every input row of that strip once, so two stride-1 output pixels cost
+// 4 + 2 vector loads instead of 20.  Strips are numbered column block
+// fastest, (image, row block, column block), and dealt to the pixel lanes in
+// that order; rows and columns past the end of the image read zeros through
+// the buffer range check and add nothing.  The pixel lanes of a wave are added
+// up across lanes, the four waves through LDS.
+template <int STRIDE, int TH, int TW, int AHEAD>
 __global__ void __launch_bounds__(kDwFilbkThreads)
     dw_filter_backprop_3x3_strip_kernel(const float* __restrict__ in,
                                         const float* __restrict__ dy,
@@ -618,9 +619,14 @@ __global__ void __launch_bounds__(kDwFilbkThreads)
                                         float* __restrict__ part,
                                         snn_hip_depthwise_params p, int cvw,
                                         int strips_per_group, int n_strips,
-                                        int n_row_blocks) {
-  constexpr int RING = 3;  // input rows alive at once
-  __shared__ float partial[kDwFilbkThreads][37];
+                                        int n_row_blocks, int n_col_blocks) {
+  // A strip is TH output rows of TW adjacent output columns, so an input row
+  // costs NC column loads for TW outputs.  The loads of output row i + AHEAD
+  // are issued before the products of row i.
+  constexpr int NC = (TW - 1) * STRIDE + 3;  // input columns of a strip
+  constexpr int RING = AHEAD * STRIDE + 3;   // input rows alive at once
+  constexpr int GRING = AHEAD + 1;           // dY rows alive at once
+  __shared__ float partial[4][32][37];       // [wave][channel vector][tap * 4 + i]
   const int C = p.channels;
   const int tid = threadIdx.x;
   const int cl = tid % cvw;
@@ -642,18 +648,18 @@ __global__ void __launch_bounds__(kDwFilbkThreads)
     for (int i = 0; i < 4; ++i) acc[t][i] = 0.f;
   if (c < C) {
     for (int strip = strip_begin + pl; strip < strip_end; strip += n_pl) {
-      const int ox = strip % p.out_cols;
-      const int t2 = strip / p.out_cols;
+      const int ox = (strip % n_col_blocks) * TW;
+      const int t2 = strip / n_col_blocks;
       const int rb = t2 % n_row_blocks;
       const int n = t2 / n_row_blocks;
       const int oy0 = rb * TH;
       const int y0 = oy0 * STRIDE - p.pad_rows;
       const int x0 = ox * STRIDE - p.pad_cols;
-      // byte offsets of the three column taps in input row 0 of the image, or
+      // byte offsets of the strip's input columns in row 0 of the image, or
       // out of range for a padding column
-      unsigned col_off[3];
+      unsigned col_off[NC];
 #pragma unroll
-      for (int sc = 0; sc < 3; ++sc)
+      for (int sc = 0; sc < NC; ++sc)
         col_off[sc] = static_cast<unsigned>(x0 + sc) <
                               static_cast<unsigned>(p.in_cols)
                           ? static_cast<unsigned>((x0 + sc) * C + c) * 4u
@@ -661,63 +667,88 @@ __global__ void __launch_bounds__(kDwFilbkThreads)
       const unsigned image_off =
           static_cast<unsigned>(n * p.in_rows * p.in_cols * C) * 4u;
       const unsigned row_bytes = static_cast<unsigned>(p.in_cols * C) * 4u;
-      float win[RING][3][4];
-      auto load_row = [&](int rel, float (&dst)[3][4]) {
+      float win[RING][NC][4];
+      auto load_row = [&](int rel, float (&dst)[NC][4]) {
         const int y = y0 + rel;
         const bool ok =
             static_cast<unsigned>(y) < static_cast<unsigned>(p.in_rows);
         const unsigned base =
             image_off + static_cast<unsigned>(y) * row_bytes;
 #pragma unroll
-        for (int sc = 0; sc < 3; ++sc)
+        for (int sc = 0; sc < NC; ++sc)
           BufVec4<float>::load(
               in_rsrc,
               (ok && col_off[sc] != kOobOffset) ? base + col_off[sc]
                                                 : kOobOffset,
               dst[sc]);
       };
-#pragma unroll
-      for (int rel = 0; rel < 3 - STRIDE; ++rel) load_row(rel, win[rel % RING]);
       const unsigned dy_off0 =
           static_cast<unsigned>(((n * p.out_rows + oy0) * p.out_cols + ox) * C +
                                 c) * 4u;
       const unsigned dy_row_bytes = static_cast<unsigned>(p.out_cols * C) * 4u;
-#pragma unroll
-      for (int i = 0; i < TH; ++i) {
-        // the input rows this output row adds that the previous one lacked
+      float g[GRING][TW][4];
+      // the input rows output row i adds that row i - 1 lacked, and its dY
+      auto load_out_row = [&](int i) {
 #pragma unroll
         for (int rel = 3 - STRIDE; rel < 3; ++rel)
           load_row(i * STRIDE + rel, win[(i * STRIDE + rel) % RING]);
-        float g[4];
-        BufVec4<float>::load(
-            dy_rsrc,
-            oy0 + i < p.out_rows ? dy_off0 + static_cast<unsigned>(i) * dy_row_bytes
-                                 : kOobOffset,
-            g);
-        // (a row block may run past the last output row: nothing to add,
-        // whatever the input rows below it hold)
-        if (oy0 + i < p.out_rows) {
 #pragma unroll
-          for (int r = 0; r < 3; ++r)
+        for (int tw = 0; tw < TW; ++tw)
+          BufVec4<float>::load(
+              dy_rsrc,
+              (oy0 + i < p.out_rows && ox + tw < p.out_cols)
+                  ? dy_off0 + static_cast<unsigned>(i) * dy_row_bytes +
+                        static_cast<unsigned>(tw * C) * 4u
+                  : kOobOffset,
+              g[i % GRING][tw]);
+      };
 #pragma unroll
-            for (int sc = 0; sc < 3; ++sc)
+      for (int rel = 0; rel < 3 - STRIDE; ++rel) load_row(rel, win[rel % RING]);
 #pragma unroll
-              for (int e = 0; e < 4; ++e)
-                acc[r * 3 + sc][e] = fmaf(win[(i * STRIDE + r) % RING][sc][e],
-                                          g[e], acc[r * 3 + sc][e]);
+      for (int i = 0; i < AHEAD && i < TH; ++i) load_out_row(i);
+#pragma unroll
+      for (int i = 0; i < TH; ++i) {
+        if (i + AHEAD < TH) load_out_row(i + AHEAD);
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw) {
+          // (a strip may run past the last output row or column: nothing to
+          // add there, whatever the input under it holds)
+          if (oy0 + i < p.out_rows && ox + tw < p.out_cols) {
+#pragma unroll
+            for (int r = 0; r < 3; ++r)
+#pragma unroll
+              for (int sc = 0; sc < 3; ++sc)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  acc[r * 3 + sc][e] =
+                      fmaf(win[(i * STRIDE + r) % RING][tw * STRIDE + sc][e],
+                           g[i % GRING][tw][e], acc[r * 3 + sc][e]);
+          }
         }
       }
     }
   }
+  // The lanes of a wave that share a channel vector are l, l ^ cvw,
+  // l ^ 2 cvw, ...: add them up across lanes, then the four waves through LDS.
+  for (int m = cvw; m < 64; m <<= 1) {
 #pragma unroll
-  for (int t = 0; t < 9; ++t)
+    for (int t = 0; t < 9; ++t)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) partial[tid][t * 4 + i] = acc[t][i];
+      for (int i = 0; i < 4; ++i) acc[t][i] += __shfl_xor(acc[t][i], m);
+  }
+  const int lane = tid & 63, wave = tid >> 6;
+  if (lane < cvw) {
+#pragma unroll
+    for (int t = 0; t < 9; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) partial[wave][lane][t * 4 + i] = acc[t][i];
+  }
   __syncthreads();
+  // lane e of the first cvw * 36 adds up one (channel vector, tap, component)
   for (int e = tid; e < cvw * 36; e += kDwFilbkThreads) {
     const int ecl = e % cvw, comp = e / cvw;  // comp = tap * 4 + i
-    float sum = 0.f;
-    for (int q = 0; q < n_pl; ++q) sum += partial[q * cvw + ecl][comp];
+    const float sum = (partial[0][ecl][comp] + partial[1][ecl][comp]) +
+                      (partial[2][ecl][comp] + partial[3][ecl][comp]);
     const int ch = (blockIdx.y * cvw + ecl) * 4 + (comp & 3);
     if (ch >= C) continue;
     if (part != nullptr) {
@@ -732,10 +763,12 @@ __global__ void __launch_bounds__(kDwFilbkThreads)
 }
 
 // dF += the work-groups' partial filters part[group][e], four elements per
-// lane; blockIdx.y and the four waves of a work-group split the groups, the
-// waves combine through LDS and one float atomic per element and work-group
-// goes to dF, which the strip kernel has zero-filled.
-constexpr int kDwFilbkReduceY = 16;
+// lane.  blockIdx.y and the four waves of a work-group split the groups into
+// gridDim.y * 4 slices; the launcher sizes gridDim.y so that a lane has at most
+// kDwFilbkReduceLoads groups to add, and their loads are all issued before the
+// first addition.  The waves combine through LDS and one float atomic per
+// element and work-group goes to dF, which the strip kernel has zero-filled.
+constexpr int kDwFilbkReduceLoads = 8;
 
 __global__ void __launch_bounds__(256)
     dw_filbk_reduce_kernel(const float4* __restrict__ part,
@@ -744,21 +777,26 @@ __global__ void __launch_bounds__(256)
   const int lane = threadIdx.x & 63, sub = threadIdx.x >> 6;
   const int v = blockIdx.x * 64 + lane;
   const int n_slices = gridDim.y * 4;
-  float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+  float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
   if (v < n_vec) {
-    int g = blockIdx.y * 4 + sub;
-    for (; g + n_slices < n_groups; g += 2 * n_slices) {
-      const float4 x = part[static_cast<size_t>(g) * n_vec + v];
-      const float4 y = part[static_cast<size_t>(g + n_slices) * n_vec + v];
-      a = make_float4(a.x + x.x, a.y + x.y, a.z + x.z, a.w + x.w);
-      b = make_float4(b.x + y.x, b.y + y.y, b.z + y.z, b.w + y.w);
-    }
-    if (g < n_groups) {
-      const float4 x = part[static_cast<size_t>(g) * n_vec + v];
-      a = make_float4(a.x + x.x, a.y + x.y, a.z + x.z, a.w + x.w);
+    for (int g0 = blockIdx.y * 4 + sub; g0 < n_groups;
+         g0 += kDwFilbkReduceLoads * n_slices) {
+      float4 x[kDwFilbkReduceLoads];
+#pragma unroll
+      for (int k = 0; k < kDwFilbkReduceLoads; ++k) {
+        // a group index past the end re-reads the last group and is not added
+        const int g = min(g0 + k * n_slices, n_groups - 1);
+        x[k] = part[static_cast<size_t>(g) * n_vec + v];
+      }
+#pragma unroll
+      for (int k = 0; k < kDwFilbkReduceLoads; ++k) {
+        if (g0 + k * n_slices < n_groups)
+          a = make_float4(a.x + x[k].x, a.y + x[k].y, a.z + x[k].z,
+                          a.w + x[k].w);
+      }
     }
   }
-  sums[sub][lane] = make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
+  sums[sub][lane] = a;
   __syncthreads();
   if (sub == 0 && v < n_vec) {
     const float4 s0 = sums[0][lane], s1 = sums[1][lane], s2 = sums[2][lane],
@@ -890,9 +928,10 @@ void launch_dw_strip(const T* input, const T* filter, T* output,
 
 // Device memory for the entry point that allocates nothing
 // (snn_hip_depthwise_conv2d_filter_backprop_noalloc_f32): the work-groups'
-// partial filters.  The strip kernel runs at most 2048 / grid_y groups along
-// x, each writing 9 * C floats with C <= 128 * grid_y, so 2048 * 1152 floats
-// (9 MiB) hold the partial filters of every shape that kernel takes.  Every
+// partial filters.  The strip kernel runs at most 1024 / grid_y + 1 groups
+// along x, each writing 9 * C floats with C <= 128 * grid_y, so 2048 * 1152
+// floats (9 MiB) hold the partial filters of every shape that kernel takes
+// with room to spare.  Every
 // device the library runs on holds its own copy until the process ends.
 constexpr size_t kDwScratchElems = size_t{2048} * 1152;
 static __device__ __align__(256) float scratch[kDwScratchElems];
@@ -925,11 +964,11 @@ int dw_scratch_on_current_device(float** out) {
 
 // Picks the strip height (4 or 8 output rows, whichever wastes fewer rows of
 // the last row block; 8 on a tie) and deals the strips to the work-groups.
-// Large problems use about 2048 work-groups whose partial filters go to
-// `static_scratch` when the caller brings it (kDwScratchElems floats), else to
-// a stream-ordered temporary, and a second kernel adds them up; small ones (or
-// a failed allocation) use up to 1024 work-groups that add into the
-// zero-filled dF with float atomics, which serialise per address.
+// The work-groups add their sums into the zero-filled dF with float atomics
+// while those stay few; otherwise their partial filters go to `static_scratch`
+// when the caller brings it (kDwScratchElems floats), else to a stream-ordered
+// temporary, and a second kernel adds them up (also the fallback when the
+// allocation fails).
 static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
                                  const snn_hip_depthwise_params& p, int cvw,
                                  int grid_y, hipStream_t stream,
@@ -937,8 +976,10 @@ static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
   const int n_pl = kDwFilbkThreads / cvw;
   const int th =
       ceil_div(p.out_rows, 8) * 8 <= ceil_div(p.out_rows, 4) * 4 ? 8 : 4;
+  constexpr int tw = 2;
   const int n_rb = ceil_div(p.out_rows, th);
-  const int n_strips = p.batch * n_rb * p.out_cols;
+  const int n_cb = ceil_div(p.out_cols, tw);
+  const int n_strips = p.batch * n_rb * n_cb;
   const int dw_elems = 9 * p.channels;
   auto plan = [&](int target_groups, int* spg) {
     *spg = max(n_pl, ceil_div(n_strips, max(1, target_groups / grid_y)));
@@ -947,13 +988,20 @@ static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
   };
   const size_t in_bytes = static_cast<size_t>(p.batch) * p.in_rows *
                           p.in_cols * p.channels * sizeof(float);
-  constexpr size_t kTwoStageBytes = size_t{32} << 20;
-  int spg = 0, grid_x = 0;
+  // Large inputs: about 448 work-groups, every lane two or more strips (more,
+  // shorter work-groups lose to their own start and end).  Small ones: up to
+  // 1024, for the sake of parallelism.
+  constexpr size_t kLargeInputBytes = size_t{32} << 20;
+  // Above this many float atomics into dF the partial filters and a second
+  // kernel are cheaper (measured: about 45 atomics per nanosecond).
+  constexpr size_t kMaxAtomics = size_t{1} << 18;
+  int spg = 0;
+  const int grid_x =
+      plan(in_bytes >= kLargeInputBytes ? 448 : 1024, &spg);
+  const size_t part_elems = static_cast<size_t>(grid_x) * dw_elems;
   float* part = nullptr;
   bool temporary = false;
-  if (in_bytes >= kTwoStageBytes) {
-    grid_x = plan(2048, &spg);
-    const size_t part_elems = static_cast<size_t>(grid_x) * dw_elems;
+  if (part_elems > kMaxAtomics) {
     if (static_scratch != nullptr) {
       if (part_elems > kDwScratchElems)
         return report_error(
@@ -973,7 +1021,6 @@ static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
     }
   }
   if (part == nullptr) {
-    grid_x = plan(1024, &spg);
     hipLaunchKernelGGL(dw_zero_kernel, dim3(ceil_div(dw_elems, 256)),
                        dim3(256), 0, stream, dw, dw_elems);
   }
@@ -981,24 +1028,33 @@ static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
                   static_cast<unsigned>(grid_y));
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, dim3(kDwFilbkThreads), 0, stream, x, dy,
-                       dw, part, p, cvw, spg, n_strips, n_rb);
+                       dw, part, p, cvw, spg, n_strips, n_rb, n_cb);
   };
+  // Loads one output row ahead of the arithmetic pay everywhere except in
+  // the large stride-2 launches, whose five-column rows then cost occupancy.
   if (p.stride_rows == 1) {
     if (th == 8)
-      launch(dw_filter_backprop_3x3_strip_kernel<1, 8>);
+      launch(dw_filter_backprop_3x3_strip_kernel<1, 8, tw, 1>);
     else
-      launch(dw_filter_backprop_3x3_strip_kernel<1, 4>);
+      launch(dw_filter_backprop_3x3_strip_kernel<1, 4, tw, 1>);
+  } else if (in_bytes >= kLargeInputBytes) {
+    if (th == 8)
+      launch(dw_filter_backprop_3x3_strip_kernel<2, 8, tw, 0>);
+    else
+      launch(dw_filter_backprop_3x3_strip_kernel<2, 4, tw, 0>);
   } else {
     if (th == 8)
-      launch(dw_filter_backprop_3x3_strip_kernel<2, 8>);
+      launch(dw_filter_backprop_3x3_strip_kernel<2, 8, tw, 1>);
     else
-      launch(dw_filter_backprop_3x3_strip_kernel<2, 4>);
+      launch(dw_filter_backprop_3x3_strip_kernel<2, 4, tw, 1>);
   }
   if (part != nullptr) {
     const int n_vec = dw_elems / 4;
     hipLaunchKernelGGL(
         dw_filbk_reduce_kernel,
-        dim3(static_cast<unsigned>(ceil_div(n_vec, 64)), kDwFilbkReduceY),
+        dim3(static_cast<unsigned>(ceil_div(n_vec, 64)),
+             static_cast<unsigned>(
+                 ceil_div(grid_x, 4 * kDwFilbkReduceLoads))),
         dim3(256), 0, stream, reinterpret_cast<const float4*>(part), dw, n_vec,
         grid_x);
     if (temporary) (void)hipFreeAsync(part, stream);

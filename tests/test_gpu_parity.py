@@ -377,6 +377,7 @@ def test_depthwise_ragged(shape):
 @pytest.mark.parametrize("shape", [(2, 13, 11, 8, 1, True),
                                    (3, 14, 14, 64, 2, True),
                                    (1, 12, 10, 4, 2, False),
+                                   (2, 12, 12, 8, 2, False),
                                    (2, 33, 20, 12, 1, False),
                                    (5, 5, 37, 16, 2, True),
                                    (1, 3, 3, 256, 1, True),
