@@ -1533,6 +1533,13 @@ void launch_gemm_rows(const float* a, const float* b, float* c, int m, int k,
   const bool fuse = epilogue != nullptr && epilogue->wanted() && batches == 1;
   const float* bias = fuse ? epilogue->bias : nullptr;
   const int relu = fuse && epilogue->relu ? 1 : 0;
+  // short reductions: the kernel that keeps the filter in registers
+  if (batches == 1 && gemm_wreg_supports(m, k, n) &&
+      SNN_TUNING_ENV("SNN_HIP_GEMM_WREG_OFF") == nullptr) {
+    launch_gemm_wreg(a, b, c, m, k, n, fuse, bias, relu != 0, stream);
+    if (fuse && epilogue->applied != nullptr) *epilogue->applied = true;
+    return;
+  }
 #define SNN_ROWS(EPI, RK, BM)                                                 \
   launch_gemm_rows_as<EPI, RK, BM>(a, b, c, m, k, n, batches, z_a, z_b, z_c, \
                                    bias, relu, stream)

@@ -98,6 +98,16 @@ int launch_conv2d_winograd_filter_backprop_f32(
     const float* x, const float* dy, float* dw, const snn_hip_conv2d_params& p,
     float* workspace, size_t workspace_elems, hipStream_t stream);
 
+// Row-major fp32 GEMM Y = X (m x k) * W (k x n) with the filter in registers
+// (gemm_wreg.hip): k = 64, 128 or 256, n in whole feature slices, enough rows
+// to keep 256 persistent work-groups busy.  Operands 16-byte aligned.  With
+// `epilogue`, bias (one value per column, may be null) is added and relu
+// applied on the way out.
+bool gemm_wreg_supports(int m, int k, int n);
+void launch_gemm_wreg(const float* x, const float* w, float* y, int m, int k,
+                      int n, bool epilogue, const float* bias, bool relu,
+                      hipStream_t stream);
+
 // Half-precision forward convolution on MFMA (conv2d_igemm_f16.hip).  The
 // workspace, when large enough, receives the re-laid-out filter.
 bool conv2d_igemm_f16_supports(const snn_hip_conv2d_params& p);

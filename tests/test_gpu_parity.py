@@ -663,10 +663,68 @@ def test_matmul_plain_rows_kernel(shape):
     assert_close(got.cpu().numpy(), ref, ("matmul rows", shape))
 
 
+@pytest.mark.parametrize("shape", [
+    # m, k, n -> (pixel blocks per tile, feature blocks per wave) of the plan
+    (16390, 64, 256),    # (2, 1), ragged last tile
+    (40000, 64, 512),    # (2, 2)
+    (12005, 128, 256),   # (1, 1), ragged
+    (28923, 128, 128),   # (2, 1)
+    (14965, 128, 256),   # (1, 2)
+    (20000, 128, 512),   # (2, 2)
+    (4100, 256, 1024),   # (1, 1), eight feature slices
+    (28923, 256, 128),   # (2, 1)
+    (14965, 256, 256),   # (1, 2)
+    (30917, 256, 256),   # (2, 2)
+    (3000, 512, 1024),   # 512 reduction steps
+    (3137, 128, 2048),   # sixteen feature slices
+])
+def test_matmul_filter_in_registers_kernel(shape):
+    """A * B with k = 64 / 128 / 256 / 512 and n in whole feature slices runs on
+    the persistent kernel that keeps B in registers: every tiling it builds,
+    row counts that end inside a tile, 1 to 16 feature slices."""
+    m, k, n = shape
+    rng = np.random.default_rng(sum(shape) + 17)
+    a, b = uniform(rng, m * k), uniform(rng, k * n)
+    ref = oracle.matmul(a, b, 1, m, k, n, False, False, 0.0)
+    out = torch.full((m * n + 64,), 7.0, device="cuda")
+    got = ops.matmul(dev(a), dev(b), 1, m, k, n, False, False, 0.0,
+                     out=out[:m * n])
+    assert_close(got.cpu().numpy(), ref, ("matmul, filter in registers", shape))
+    # nothing is written past the last row
+    assert torch.all(out[m * n:] == 7.0)
+
+
+@pytest.mark.parametrize("shape", [(4, 56, 56, 64, 256), (6, 28, 28, 128, 512),
+                                   (12, 14, 14, 256, 1024),
+                                   (32, 7, 7, 512, 2048)])
+def test_conv1x1_filter_in_registers_bias_relu(shape):
+    """1x1 convolutions on the same kernel with its fused epilogue: equal to
+    the plain launch followed by the bias addition and the ReLU, and to the
+    oracle."""
+    batch, rows, cols, ch, feats = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, 1, 1, False)
+    rng = np.random.default_rng(5151 + ch)
+    n_in, n_fil, _ = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x, w = uniform(rng, n_in), uniform(rng, n_fil)
+    bias = uniform(rng, feats) * 4
+    dx, dw, db = dev(x), dev(w), dev(bias)
+    plain = ops.conv2d(dx, dw, p, DIRECTION.FORWARD, ALGO.MATMUL)
+    ref = oracle.conv2d_forward(x, w, oracle_params(p, feats), acc64=True)
+    assert_close(plain.cpu().numpy(), ref, ("1x1, filter in registers", shape))
+    want = torch.relu(plain.view(-1, feats) + db).view(-1)
+    got = ops.conv2d_bias_act(dx, dw, db, p, ALGO.MATMUL, relu=True)
+    assert torch.equal(got, want)
+    got = ops.conv2d_bias_act(dx, dw, db, p, ALGO.MATMUL, relu=False)
+    assert torch.equal(got, (plain.view(-1, feats) + db).view(-1))
+    got = ops.conv2d_bias_act(dx, dw, None, p, ALGO.MATMUL, relu=True)
+    assert torch.equal(got, torch.relu(plain))
+
+
 def test_plain_rows_kernel_bias_relu_on_tall_tiles():
-    """14x14x256 -> 1024 at batch 32 runs on 112-row tiles; the fused bias +
-    ReLU epilogue must equal the convolution followed by the two steps."""
-    p = ops.conv_params(32, 14, 14, 256, 1024, 1, 1, False)
+    """14x14x192 -> 1024 at batch 32 runs on 112-row tiles of the plain-rows
+    kernel; the fused bias + ReLU epilogue must equal the convolution followed
+    by the two steps."""
+    p = ops.conv_params(32, 14, 14, 192, 1024, 1, 1, False)
     rng = np.random.default_rng(4343)
     n_in, n_fil, _ = ops.conv_sizes(p, DIRECTION.FORWARD)
     x, w = uniform(rng, n_in), uniform(rng, n_fil)
