@@ -415,7 +415,7 @@ def main():
                 ws = torch.empty(n_b, device="cuda", dtype=torch.float16)
                 ms = event_time_ms(lambda: ops.conv2d(
                     a, b, p, DIRECTION.FORWARD, ALGO.IM2COL, workspace=ws,
-                    out=o), reps=10, warm=2, repeats=3)
+                    out=o), reps=30, warm=5, repeats=3)
                 fl = ops.conv_flops(p, DIRECTION.FORWARD)
                 entry = {"op": "conv%dx%d_%dx%dx%d_k%d_b128_f16" % (
                     window, window, size, size, ch, feats), "ms": round(ms, 4),
@@ -437,7 +437,7 @@ def main():
                     o.copy_(uniform(n_o).half())
                     ms = event_time_ms(lambda: ops.conv2d(
                         o, b, p, DIRECTION.INPUT_BACKPROP, ALGO.IM2COL,
-                        workspace=ws, out=dx), reps=10, warm=2, repeats=3)
+                        workspace=ws, out=dx), reps=30, warm=5, repeats=3)
                     fl = ops.conv_flops(p, DIRECTION.INPUT_BACKPROP)
                     h.append({"op": "conv3x3_%dx%dx%d_k%d_b128_f16_input_"
                               "backprop" % (size, size, ch, feats),

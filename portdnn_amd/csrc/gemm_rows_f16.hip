@@ -398,16 +398,21 @@ int launch_rows_tj(const _Float16* x, const _Float16* w, _Float16* y,
 bool gemm_rows_f16_supports(int m, int k, int n) {
   static const bool off = SNN_TUNING_ENV("SNN_HIP_F16_ROWS_OFF") != nullptr;
   RowsPlan plan;
-  return !off && plan_rows(m, k, n, &plan);
+  return !off && (gemm_wreg_f16_supports(m, k, n) || plan_rows(m, k, n, &plan));
 }
 
 int launch_gemm_rows_f16(const _Float16* x, const _Float16* w, _Float16* y,
                          int m, int k, int n, hipStream_t stream) {
-  RowsPlan plan;
-  if (!plan_rows(m, k, n, &plan)) return SNN_HIP_INVALID_ALGORITHM;
   if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) |
         reinterpret_cast<uintptr_t>(y)) & 15u) != 0)
     return SNN_HIP_INVALID_PARAMETER;
+  // short reductions: the kernel that keeps the filter in registers
+  if (gemm_wreg_f16_supports(m, k, n)) {
+    launch_gemm_wreg_f16(x, w, y, m, k, n, stream);
+    return SNN_HIP_OK;
+  }
+  RowsPlan plan;
+  if (!plan_rows(m, k, n, &plan)) return SNN_HIP_INVALID_ALGORITHM;
   return plan.tj == 4 ? launch_rows_tj<4>(x, w, y, plan, stream)
                       : launch_rows_tj<2>(x, w, y, plan, stream);
 }

@@ -107,6 +107,11 @@ bool gemm_wreg_supports(int m, int k, int n);
 void launch_gemm_wreg(const float* x, const float* w, float* y, int m, int k,
                       int n, bool epilogue, const float* bias, bool relu,
                       hipStream_t stream);
+// The same in half precision with fp32 accumulation (gemm_wreg_f16.hip):
+// k = 64, 128, 256 or 512.
+bool gemm_wreg_f16_supports(int m, int k, int n);
+void launch_gemm_wreg_f16(const _Float16* x, const _Float16* w, _Float16* y,
+                          int m, int k, int n, hipStream_t stream);
 
 // Half-precision forward convolution on MFMA (conv2d_igemm_f16.hip).  The
 // workspace, when large enough, receives the re-laid-out filter.

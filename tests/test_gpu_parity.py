@@ -779,6 +779,39 @@ def test_many_tiles_per_work_group_epilogue_and_accumulate():
                                0.0), "matmul slice")
 
 
+@pytest.mark.parametrize("shape", [
+    # m, k, n -> (k / 32, pixel blocks per tile, feature blocks per wave)
+    (50977, 64, 256),    # (2, 4, 2), ragged last tile
+    (58973, 64, 512),    # (2, 4, 4)
+    (24990, 128, 256),   # (4, 2, 2)
+    (28988, 128, 512),   # (4, 2, 4)
+    (12996, 256, 256),   # (8, 1, 2)
+    (14995, 256, 512),   # (8, 1, 4)
+    (28988, 256, 256),   # (8, 2, 2)
+    (30987, 256, 512),   # (8, 2, 4)
+    (12996, 512, 256),   # (16, 1, 2)
+    (28988, 512, 256),   # (16, 2, 2)
+    (6272, 512, 2048),   # eight feature slices, one XCD per slice
+])
+def test_matmul_f16_filter_in_registers_kernel(shape):
+    """Half-precision A * B with k = 64 / 128 / 256 / 512 on the persistent kernel
+    that keeps B in registers (transposed there from its feature-contiguous
+    layout): every tiling it builds, row counts that end inside a tile."""
+    m, k, n = shape
+    rng = np.random.default_rng(sum(shape) + 23)
+    a = uniform(rng, m * k).astype(np.float16)
+    b = uniform(rng, k * n).astype(np.float16)
+    ref = oracle.matmul(a.astype(np.float32), b.astype(np.float32), 1, m, k, n,
+                        False, False, 0.0)
+    out = torch.full((m * n + 64,), 7.0, device="cuda", dtype=torch.float16)
+    got = ops.matmul(dev(a, torch.float16), dev(b, torch.float16), 1, m, k, n,
+                     False, False, 0.0, out=out[:m * n])
+    assert_close_f16(got.float().cpu().numpy(), ref,
+                     ("matmul f16, filter in registers", shape))
+    # nothing is written past the last row
+    assert torch.all(out[m * n:] == 7.0)
+
+
 @pytest.mark.parametrize("shape", [(1, 256, 128, 192), (1, 100, 64, 64),
                                    (3, 33, 20, 17), (1, 2048, 256, 512)])
 @pytest.mark.parametrize("trans_a", [False, True])
