@@ -571,7 +571,11 @@ def main():
                     state["i"] += 1
                     ops.depthwise_conv2d(a_s[i], b_s[i], p, direction,
                                          out=o_s[i])
-                ms = event_time_ms(run, reps=5 * sets, warm=sets, repeats=3)
+                # (the calls that take a stream-ordered temporary pay a fixed
+                # cost after every synchronisation: long runs, so that the
+                # figure is the steady state)
+                ms = event_time_ms(run, reps=max(5 * sets, 100), warm=sets,
+                                   repeats=3)
                 grads.append(mem_entry(
                     "depthwise3x3_%dx%dx%d_s%d_%s" % (size, size, ch, stride,
                                                       tag),

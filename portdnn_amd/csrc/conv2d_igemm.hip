@@ -1694,7 +1694,7 @@ static int launch_input_backprop_col2im(const float* dy, const float* filter,
     const size_t cap = max(z_per_image, (size_t{64} << 20) / sizeof(float));
     z_elems = min(cap, z_per_image * p.batch);
     void* ptr = nullptr;
-    if (hipMallocAsync(&ptr, z_elems * sizeof(float), stream) != hipSuccess)
+    if (temp_malloc_async(&ptr, z_elems * sizeof(float), stream) != hipSuccess)
       return SNN_HIP_ALLOCATION_PROBLEM;
     z = static_cast<float*>(ptr);
     temporary = true;
@@ -1744,7 +1744,7 @@ static int launch_input_backprop_col2im(const float* dy, const float* filter,
                        dim3(256), 0, stream, z, dx_mb, fg, images);
   }
   const hipError_t err = hipGetLastError();
-  if (temporary) (void)hipFreeAsync(z, stream);
+  if (temporary) temp_free_async(z, stream);
   if (err != hipSuccess) return report_hip_error(err, "input backprop col2im");
   return SNN_HIP_OK;
 }
@@ -1892,7 +1892,7 @@ int launch_conv2d_filter_backprop_f16(const _Float16* x, const _Float16* dy,
   if (workspace == nullptr || workspace_elems < 2 * dw_elems ||
       (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) {
     void* ptr = nullptr;
-    if (hipMallocAsync(&ptr, dw_elems * sizeof(float), stream) != hipSuccess)
+    if (temp_malloc_async(&ptr, dw_elems * sizeof(float), stream) != hipSuccess)
       return SNN_HIP_ALLOCATION_PROBLEM;
     acc32 = static_cast<float*>(ptr);
     temporary = true;
@@ -1921,7 +1921,7 @@ int launch_conv2d_filter_backprop_f16(const _Float16* x, const _Float16* dy,
                      dim3(static_cast<unsigned>(ceil_div(dw_elems, size_t{256}))),
                      dim3(256), 0, stream, acc32, dw, dw_elems);
   const hipError_t err = hipGetLastError();
-  if (temporary) (void)hipFreeAsync(acc32, stream);
+  if (temporary) temp_free_async(acc32, stream);
   if (err != hipSuccess) return report_hip_error(err, "f16 filter backprop");
   return SNN_HIP_OK;
 }

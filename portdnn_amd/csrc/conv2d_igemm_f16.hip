@@ -318,7 +318,7 @@ int launch_conv2d_igemm_f16(const _Float16* input, const _Float16* filter,
   if (workspace == nullptr || workspace_elems < wgt_elems ||
       (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) {
     void* ptr = nullptr;
-    if (hipMallocAsync(&ptr, wgt_elems * sizeof(_Float16), stream) != hipSuccess)
+    if (temp_malloc_async(&ptr, wgt_elems * sizeof(_Float16), stream) != hipSuccess)
       return SNN_HIP_ALLOCATION_PROBLEM;
     wgt_t = static_cast<_Float16*>(ptr);
     temporary = true;
@@ -327,7 +327,7 @@ int launch_conv2d_igemm_f16(const _Float16* input, const _Float16* filter,
   if (!no_rowtile && conv2d_rowtile_f16_supports(p)) {
     const int status =
         launch_conv2d_rowtile_f16(input, filter, output, p, wgt_t, stream);
-    if (temporary) (void)hipFreeAsync(wgt_t, stream);
+    if (temporary) temp_free_async(wgt_t, stream);
     return status;
   }
   hipLaunchKernelGGL(repack_filter_kernel,
@@ -354,7 +354,7 @@ int launch_conv2d_igemm_f16(const _Float16* input, const _Float16* filter,
     launch_f16_tile<64, 64, 2, 2>(input, wgt_t, output, g, src_elems,
                                   wgt_elems, stream);
   const hipError_t launch_err = hipGetLastError();
-  if (temporary) (void)hipFreeAsync(wgt_t, stream);
+  if (temporary) temp_free_async(wgt_t, stream);
   if (launch_err != hipSuccess)
     return report_hip_error(launch_err, "conv_igemm_f16_kernel");
   return SNN_HIP_OK;
@@ -405,7 +405,7 @@ int launch_conv2d_input_backprop_f16(const _Float16* dy,
     if (workspace == nullptr || workspace_elems < wgt_elems ||
         (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) {
       void* ptr = nullptr;
-      if (hipMallocAsync(&ptr, wgt_elems * sizeof(_Float16), stream) !=
+      if (temp_malloc_async(&ptr, wgt_elems * sizeof(_Float16), stream) !=
           hipSuccess)
         return SNN_HIP_ALLOCATION_PROBLEM;
       packed = static_cast<_Float16*>(ptr);
@@ -413,7 +413,7 @@ int launch_conv2d_input_backprop_f16(const _Float16* dy,
     }
     const int status =
         launch_conv2d_rowtile_f16(dy, filter, dx, q, packed, stream, true);
-    if (temporary) (void)hipFreeAsync(packed, stream);
+    if (temporary) temp_free_async(packed, stream);
     return status;
   }
   if (p.window_rows != 1 || p.window_cols != 1 || !conv2d_igemm_f16_supports(q))

@@ -1011,7 +1011,7 @@ static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
             " bytes, the library's scratch array holds " +
             std::to_string(kDwScratchElems * sizeof(float)));
       part = static_scratch;
-    } else if (hipMallocAsync(reinterpret_cast<void**>(&part),
+    } else if (temp_malloc_async(reinterpret_cast<void**>(&part),
                               part_elems * sizeof(float),
                               stream) == hipSuccess) {
       temporary = true;
@@ -1057,7 +1057,7 @@ static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
                  ceil_div(grid_x, 4 * kDwFilbkReduceLoads))),
         dim3(256), 0, stream, reinterpret_cast<const float4*>(part), dw, n_vec,
         grid_x);
-    if (temporary) (void)hipFreeAsync(part, stream);
+    if (temporary) temp_free_async(part, stream);
   }
   return SNN_HIP_OK;
 }

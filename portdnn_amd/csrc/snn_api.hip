@@ -27,6 +27,54 @@ std::vector<std::pair<hipEvent_t, hipEvent_t>> g_timed_kernels;
 constexpr size_t kMaxTimedKernels = 1u << 16;
 }  // namespace
 
+namespace {
+constexpr int kMaxPoolDevices = 64;
+std::mutex g_pool_mutex;
+hipMemPool_t g_pools[kMaxPoolDevices] = {};
+bool g_pool_failed[kMaxPoolDevices] = {};
+
+// The current device's pool, created at first use; null when there is none.
+hipMemPool_t temp_pool() {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 ||
+      device >= kMaxPoolDevices) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_pool_mutex);
+  if (g_pools[device] == nullptr && !g_pool_failed[device]) {
+    hipMemPoolProps props = {};
+    props.allocType = hipMemAllocationTypePinned;
+    props.handleTypes = hipMemHandleTypeNone;
+    props.location.type = hipMemLocationTypeDevice;
+    props.location.id = device;
+    hipMemPool_t pool = nullptr;
+    if (hipMemPoolCreate(&pool, &props) == hipSuccess) {
+      uint64_t keep = uint64_t{512} << 20;
+      (void)hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep);
+      g_pools[device] = pool;
+    } else {
+      (void)hipGetLastError();
+      g_pool_failed[device] = true;
+    }
+  }
+  return g_pools[device];
+}
+}  // namespace
+
+hipError_t temp_malloc_async(void** ptr, size_t bytes, hipStream_t stream) {
+  if (hipMemPool_t pool = temp_pool()) {
+    if (hipMallocFromPoolAsync(ptr, bytes, pool, stream) == hipSuccess)
+      return hipSuccess;
+    (void)hipGetLastError();
+  }
+  return hipMallocAsync(ptr, bytes, stream);
+}
+
+void temp_free_async(void* ptr, hipStream_t stream) {
+  (void)hipFreeAsync(ptr, stream);
+}
+
 KernelTimer::KernelTimer(hipStream_t stream) : stream_(stream), stop_(nullptr) {
   if (!g_timing_enabled.load(std::memory_order_relaxed)) return;
   {
@@ -445,7 +493,7 @@ int conv2d_nchw<float>(int direction, const float* input, const float* filter,
   const int taps = p.window_rows * p.window_cols;
   const int in_hw = p.in_rows * p.in_cols, out_hw = p.out_rows * p.out_cols;
   float* tmp = nullptr;
-  if (hipMallocAsync(reinterpret_cast<void**>(&tmp),
+  if (temp_malloc_async(reinterpret_cast<void**>(&tmp),
                      (sz.input + sz.filter + sz.output) * sizeof(float), s) !=
       hipSuccess)
     return SNN_HIP_ALLOCATION_PROBLEM;
@@ -480,7 +528,7 @@ int conv2d_nchw<float>(int direction, const float* input, const float* filter,
                                          taps, false, s)
              : launch_transpose_batched_f32(t_out, output, p.batch, out_a.hw,
                                             out_a.c, s);
-  (void)hipFreeAsync(tmp, s);
+  temp_free_async(tmp, s);
   return rc;
 }
 

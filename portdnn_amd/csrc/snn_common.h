@@ -106,6 +106,15 @@ struct Elem<_Float16> {
   }
 };
 
+// Stream-ordered temporaries (partial results, re-laid-out filters) for calls
+// that bring no workspace.  They come from a memory pool of the library's own,
+// one per device, that keeps up to 512 MiB of freed blocks instead of handing
+// them back at every synchronisation -- the default pool does, and the next
+// allocation after a hipStreamSynchronize then costs tens of microseconds.
+// Falls back to the device's default pool when a pool cannot be created.
+hipError_t temp_malloc_async(void** ptr, size_t bytes, hipStream_t stream);
+void temp_free_async(void* ptr, hipStream_t stream);
+
 // Validated, normalised views of the three parameter records.
 int validate(const snn_hip_conv2d_params& p);
 int validate(const snn_hip_depthwise_params& p);
