@@ -912,12 +912,12 @@ __global__ void __launch_bounds__(kThreads)
         __builtin_amdgcn_raw_buffer_store_b128(
             __builtin_bit_cast(uint4v,
                                make_float4(out[0], out[1], out[2], out[3])),
-            c_rsrc, off, 0, 0);
+            c_rsrc, off, 0, 2);  // written once: streaming store (slc)
       } else {
         typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
         __builtin_amdgcn_raw_buffer_store_b64(
             __builtin_bit_cast(uint2v, make_float2(out[0], out[1])), c_rsrc,
-            off, 0, 0);
+            off, 0, 2);
       }
     }
   }

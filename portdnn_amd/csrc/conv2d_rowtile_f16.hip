@@ -50,6 +50,7 @@ using gemm::xcd_remap;
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
 constexpr unsigned kOob = 0x7FFFFFF0u;
+constexpr int kStoreAux = 2;  // the output is written once: stream it (slc)
 constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
 constexpr int kFA = 2;  // feature blocks (of 32) per wave
 constexpr size_t kMaxLdsBytes = 160 * 1024;
@@ -490,9 +491,9 @@ __global__ void __launch_bounds__(64 * WF * WP)
         hi[v] = static_cast<_Float16>(acc[i][j][8 + v]);
       }
       __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, lo),
-                                             dst_rsrc, off, 0, 0);
+                                             dst_rsrc, off, 0, kStoreAux);
       __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, hi),
-                                             dst_rsrc, off + 16u, 0, 0);
+                                             dst_rsrc, off + 16u, 0, kStoreAux);
     }
   }
 }

@@ -460,6 +460,9 @@ __global__ void __launch_bounds__(512)
 // even number of chunks.
 // ---------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
+// The output is written once and not read again by the kernel: stream it
+// (slc).  -1 ... -2 us on the 56x56x64 layer.
+constexpr int kStoreAux = 2;
 constexpr int kWaitVm8 = 0x0F78;  // s_waitcnt vmcnt(8)
 
 __global__ void __launch_bounds__(256)
@@ -752,9 +755,9 @@ __global__ void __launch_bounds__(256)
       const unsigned off1 =
           (col_ok && (flags & 1) != 0) ? off0 + out_row_bytes : kOob;
       __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y0),
-                                             out_rsrc, off0, 0, 0);
+                                             out_rsrc, off0, 0, kStoreAux);
       __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, y1),
-                                             out_rsrc, off1, 0, 0);
+                                             out_rsrc, off1, 0, kStoreAux);
     }
     __syncthreads();  // raw buffer 1 is free for the next unit's second chunk
     u_base = u_next;
