@@ -234,8 +234,7 @@ __global__ void __launch_bounds__(64 * WAVES)
           }
           __builtin_amdgcn_raw_buffer_store_b128(
               __builtin_bit_cast(uint4v, v8), y_rsrc,
-              voff + static_cast<unsigned>(a * 16 * TJ + e * 32), 0,
-              2);  // written once: streaming store (slc)
+              voff + static_cast<unsigned>(a * 16 * TJ + e * 32), 0, 0);
         }
       }
     }
