@@ -36,7 +36,11 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
 constexpr int kWaves = 8;
-constexpr int kStoreAux = 2;  // the output is written once: stream it (slc)
+// The output is written once: stream it (slc) -- unless it is larger than the
+// 256 MiB last-level cache, where ordinary stores measured 3-6 %
+// faster (the launcher decides: stream_stores).
+constexpr int kStoreAux = 2;
+constexpr size_t kStreamStoreMaxBytes = size_t{256} << 20;
 constexpr int kGroups = 2048 / kWaves;  // persistent work-groups: 8 waves per CU
 constexpr unsigned kOobOffset = 0x7FFFFFF0u;  // beyond every buffer's range
 constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
@@ -60,7 +64,8 @@ template <int KSTEPS, int PB, int FB, bool EPI>
 __device__ __forceinline__ void gemm_wreg_body(
     const float* __restrict__ x, const float* __restrict__ w,
     float* __restrict__ y, int m, int n, int n_cols, int m_tiles,
-    int cols_by_xcd, const float* __restrict__ bias, int relu) {
+    int cols_by_xcd, int stream_stores, const float* __restrict__ bias,
+    int relu) {
   constexpr int K = 4 * KSTEPS;
   constexpr int TP = 16 * PB;                     // pixels per tile
   constexpr int TILE_FLOATS = TP * K;
@@ -197,10 +202,12 @@ __device__ __forceinline__ void gemm_wreg_body(
             v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f);
           }
         }
-        __builtin_amdgcn_raw_buffer_store_b128(
-            v, y_rsrc,
-            base + static_cast<unsigned>(16 * pb * n + 16 * fb) * 4u, 0,
-            kStoreAux);
+        const unsigned off =
+            base + static_cast<unsigned>(16 * pb * n + 16 * fb) * 4u;
+        if (stream_stores)
+          __builtin_amdgcn_raw_buffer_store_b128(v, y_rsrc, off, 0, kStoreAux);
+        else
+          __builtin_amdgcn_raw_buffer_store_b128(v, y_rsrc, off, 0, 0);
       }
   };
 
@@ -277,9 +284,11 @@ bool make_plan(int m, int k, int n, Plan* plan) {
       gemm_wreg_k##KSTEPS##_p##PB##_f##FB##_e##E(                              \
           const float* __restrict__ x, const float* __restrict__ w,            \
           float* __restrict__ y, int m, int n, int n_cols, int m_tiles,        \
-          int cols_by_xcd, const float* __restrict__ bias, int relu) {         \
+          int cols_by_xcd, int stream_stores, const float* __restrict__ bias,  \
+          int relu) {                                                          \
     gemm_wreg_body<KSTEPS, PB, FB, E != 0>(x, w, y, m, n, n_cols, m_tiles,     \
-                                           cols_by_xcd, bias, relu);           \
+                                           cols_by_xcd, stream_stores, bias,   \
+                                           relu);                              \
   }
 #define SNN_WREG_KERNELS(KSTEPS, PB, FB) \
   SNN_WREG_KERNEL(KSTEPS, PB, FB, 0)     \
@@ -297,7 +306,7 @@ SNN_WREG_KERNELS(128, 1, 1)
 #undef SNN_WREG_KERNEL
 
 using WregKernel = void (*)(const float*, const float*, float*, int, int, int,
-                            int, int, const float*, int);
+                            int, int, int, const float*, int);
 
 WregKernel pick_kernel(int k, const Plan& plan, bool epilogue) {
 #define SNN_WREG_PICK(KSTEPS, PB, FB)                     \
@@ -334,6 +343,10 @@ void launch_gemm_wreg(const float* x, const float* w, float* y, int m, int k,
   hipLaunchKernelGGL(kernel, dim3(kGroups), dim3(64 * kWaves), 0, stream, x, w,
                      y, m, n, plan.n_cols, plan.m_tiles,
                      plan.n_cols >= 8 && n > m ? 1 : 0,
+                     static_cast<size_t>(m) * n * sizeof(float) <=
+                             kStreamStoreMaxBytes
+                         ? 1
+                         : 0,
                      epilogue ? bias : nullptr, epilogue && relu ? 1 : 0);
 }
 
