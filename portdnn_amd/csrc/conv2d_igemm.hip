@@ -2109,6 +2109,12 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
                            g.src_cols * g.src_ch;
   const size_t wgt_elems = static_cast<size_t>(p.window_rows) * p.window_cols *
                            p.channels * p.features;
+  if (direction == SNN_HIP_FORWARD && conv2d_stem_supports(p) &&
+      (reinterpret_cast<uintptr_t>(output) & 15u) == 0 &&
+      SNN_TUNING_ENV("SNN_HIP_STEM_OFF") == nullptr) {
+    // three channels, 7x7 stride 2, 64 features: the kernel built for it
+    return launch_conv2d_stem_f32(input, filter, output, p, stream);
+  }
   if (direction == SNN_HIP_FORWARD && g.src_ch % 4 != 0) {
     launch_scalar_gather_forward(input, filter, output, g, src_elems,
                                  wgt_elems, stream);

@@ -1,0 +1,364 @@
+// Forward convolution of an image with three channels: 7x7 window, stride 2,
+// 64 features, fp32 NHWC x HWCF -- the ResNet stem (the forward case of
+// include/portdnn/conv2d/launch.h:59-118 that the reference runs on its Direct /
+// Tiled kernels, src/conv2d/direct/kernels.h, src/conv2d/tiled/kernels.h).
+// As an implicit GEMM this layer has a reduction of 7 * 7 * 3 = 147 with the
+// three channels innermost, which neither 16-byte gathers nor whole chunks of
+// 32 fit; the general kernel locates and loads every reduction index on its
+// own.  Here the structure of the layer is used instead:
+//
+//   * a work-group owns a band of consecutive output rows of one image and
+//     keeps every input row the band touches in LDS, each loaded once with
+//     `buffer_load_dword ... lds` (no registers; rows and columns of the
+//     padding arrive as zeros through the buffer range check).  An input row
+//     is stored from its left padding on, so the 7 * 3 = 21 reduction values
+//     of one filter row are 21 consecutive floats at 6 * ox for output column
+//     ox, and 16 neighbouring output pixels read them without bank conflicts
+//     (stride 6 words);
+//   * the filter sits in registers, a quarter (16 features) per wave: 37 matrix
+//     instructions of 4 reduction indices (148, the last one a zero weight
+//     whose operand comes from a word of LDS that holds zero);
+//   * a wave multiplies blocks of 16 output pixels against its 16 features,
+//     v_mfma_f32_16x16x4_f32 with features as rows, so a lane ends with four
+//     consecutive features of its pixel (16-byte stores).
+//
+// Reduction order inside an output: k = 4 t + q for instruction t and lane
+// quarter q, summed by the matrix unit over q and accumulated over t in order.
+#include "snn_kernels.h"
+
+namespace snn {
+namespace {
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+constexpr int kWaves = 8;
+constexpr int kWin = 7, kCh = 3, kStride = 2, kFeatures = 64;
+constexpr int kRowK = kWin * kCh;                 // 21 reduction values per filter row
+constexpr int kK = kWin * kRowK;                  // 147
+constexpr int kSteps = (kK + 3) / 4;              // 37 matrix instructions per block
+constexpr int kFb = kFeatures / 16;               // 4 feature blocks
+constexpr unsigned kOobOffset = 0x7FFFFFF0u;
+constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
+constexpr size_t kMaxLdsBytes = 150 * 1024;
+constexpr int kStoreAux = 2;  // the output is written once: stream it (slc)
+
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* p,
+                                                   size_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0,
+                                           static_cast<unsigned>(bytes),
+                                           0x00020000);
+}
+
+constexpr int vmcnt_imm(int n) {
+  return 0x0F70 | (n & 15) | ((n >> 4) << 14);
+}
+
+struct StemGeom {
+  int batch, in_rows, in_cols, out_rows, out_cols, pad_rows, pad_cols;
+  int band;        // output rows per work-group (even)
+  int n_bands;     // bands per image
+  int row_floats;  // LDS floats per input row (a multiple of 64)
+  int lds_rows;    // 2 * band + 5
+  int loads_per_row;   // row_floats / 64
+};
+
+constexpr int kNpb = 7;              // 16-pixel blocks of an output row
+constexpr int kUnits = kNpb;         // (output row, pixel block) pairs per wave and step
+constexpr int kRowsPerStep = 2;      // output rows per step
+constexpr int kNewRows = kStride * kRowsPerStep;  // input rows a step adds
+constexpr int kGroup = 4;            // matrix instructions per operand fetch
+// LDS floats per input row, fixed so that operand addresses are immediates:
+// 11 x 64 floats hold the 224 + 6 columns a 112-pixel output row reads.
+constexpr int kRowFloats = 704;
+// Fewest output rows (over the batch) the kernel is used for.
+constexpr long kMinOutputRows = 224;
+
+// Reduction index k = 4 t + q sits k / 21 rows down and k % 21 floats along.
+// For most t the four lane quarters stay in one filter row, so the offset is
+// a constant plus q and the constant goes into the instruction; where a row
+// ends inside the group (and in the last group, which has one index past
+// the reduction) a lane needs an offset of its own.
+constexpr bool group_straddles(int t) {
+  return (4 * t) / kRowK != (4 * t + 3) / kRowK || 4 * t + 3 >= kK;
+}
+constexpr int group_offset(int t) {
+  return ((4 * t) / kRowK) * kRowFloats + (4 * t) % kRowK;
+}
+constexpr int count_straddles() {
+  int n = 0;
+  for (int t = 0; t < kSteps; ++t) n += group_straddles(t) ? 1 : 0;
+  return n;
+}
+constexpr int straddle_index(int t) {
+  int n = 0;
+  for (int u = 0; u < t; ++u) n += group_straddles(u) ? 1 : 0;
+  return n;
+}
+constexpr int kStraddles = count_straddles();
+
+// Input rows of the band go to LDS row 0 ...; LDS column i of a row holds the
+// input float i - 3 * pad_cols of that image row.
+//
+// A step is two output rows = 2 x 7 pixel blocks x 4 feature blocks = 56
+// blocks of 16 x 16 outputs, seven per wave: wave w takes blocks w, w + 8, ...,
+// in (row, pixel block, feature block) order, which gives it the feature block
+// w % 4 every time -- it keeps that quarter of the filter (37 registers) -- and
+// the four SIMDs the same work (with one output row per step and one pixel
+// block per wave the eighth wave idled).
+__global__ void __launch_bounds__(64 * kWaves)
+    __attribute__((amdgpu_waves_per_eu(2, 2)))
+    conv_stem_7x7s2_kernel(const float* __restrict__ x,
+                           const float* __restrict__ w, float* __restrict__ y,
+                           StemGeom g) {
+  extern __shared__ __align__(16) float lds[];
+  // one word past the rows that always holds zero
+  const int zero_word = g.lds_rows * kRowFloats;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int q = lane >> 4;
+  const int px = lane & 15;
+  const int fb = wave & 3;
+  const int n = blockIdx.x / g.n_bands;
+  const int band = blockIdx.x % g.n_bands;
+  const int oy0 = band * g.band;
+  const int n_rows = min(g.band, g.out_rows - oy0);
+  const int n_steps = (n_rows + kRowsPerStep - 1) / kRowsPerStep;
+  const int y_first = kStride * oy0 - g.pad_rows;
+
+  const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(
+      x, static_cast<size_t>(g.batch) * g.in_rows * g.in_cols * kCh * 4);
+  const __amdgpu_buffer_rsrc_t y_rsrc = make_rsrc(
+      y, static_cast<size_t>(g.batch) * g.out_rows * g.out_cols * kFeatures * 4);
+
+  if (threadIdx.x == 0) lds[zero_word] = 0.f;
+
+  // Load instruction `i` of LDS row `row`: 64 consecutive floats.  A row or a
+  // column outside the image is out of the buffer's range: zeros.
+  const int row_bytes_in = g.in_cols * kCh * 4;
+  auto issue_row_piece = [&](int row, int i, bool live) {
+    const int yy = y_first + row;
+    const int f = i * 64 + lane - kCh * g.pad_cols;  // float index in the image row
+    const bool ok = live &&
+                    static_cast<unsigned>(yy) < static_cast<unsigned>(g.in_rows) &&
+                    static_cast<unsigned>(f) <
+                        static_cast<unsigned>(g.in_cols * kCh);
+    const unsigned off =
+        ok ? static_cast<unsigned>((n * g.in_rows + yy)) *
+                     static_cast<unsigned>(row_bytes_in) +
+                 static_cast<unsigned>(f) * 4u
+           : kOobOffset;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        x_rsrc, (lds_ptr)(lds + row * kRowFloats + i * 64), 4, off, 0, 0, 0);
+  };
+  // this wave's quarter of the filter, in matrix-operand order: k = 4 t + q,
+  // feature 16 fb + px
+  float wreg[kSteps];
+#pragma unroll
+  for (int t = 0; t < kSteps; ++t) {
+    const int k = 4 * t + q;
+    wreg[t] = k < kK ? w[k * kFeatures + 16 * fb + px] : 0.f;
+  }
+  // the lanes' own offsets for the groups that straddle a filter row, relative
+  // to a block's base (which already includes q); the index past the
+  // reduction reads the zero word instead: its weight is zero, but zero times a
+  // stray infinity would not be
+  int kspec[kStraddles];
+#pragma unroll
+  for (int t = 0; t < kSteps; ++t) {
+    if (group_straddles(t)) {
+      const int k = 4 * t + q;
+      kspec[straddle_index(t)] =
+          k < kK ? (k / kRowK) * kRowFloats + k % kRowK - q : 0;
+    }
+  }
+  const bool last_is_pad = 4 * (kSteps - 1) + q >= kK;
+  // this wave's blocks of a step: output row u / 28 of the step, pixel block
+  // (u % 28) / 4 for u = wave + 8 i
+  int unit_row[kUnits], unit_pb[kUnits];
+#pragma unroll
+  for (int i = 0; i < kUnits; ++i) {
+    const int u = wave + kWaves * i;
+    unit_row[i] = u / (4 * kNpb);
+    unit_pb[i] = (u % (4 * kNpb)) >> 2;
+  }
+
+  // ---- start: the rows of the first two steps are waited for; every other
+  // row of the band is issued behind them and has two steps to arrive.  The
+  // band's rows all have a place of their own in LDS, so nothing is ever
+  // overwritten and two barriers serve the whole band.
+  constexpr int kFirstRows = kWin - kStride + 2 * kNewRows;
+  __builtin_amdgcn_sched_barrier(0);
+  for (int row = 0; row < kFirstRows && row < g.lds_rows; ++row)
+    for (int i = wave; i < g.loads_per_row; i += kWaves)
+      issue_row_piece(row, i, true);
+  __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+  __syncthreads();
+  for (int row = kFirstRows; row < g.lds_rows; ++row)
+    for (int i = wave; i < g.loads_per_row; i += kWaves)
+      issue_row_piece(row, i, true);
+
+  for (int s = 0; s < n_steps; ++s) {
+    if (s == 2) {
+      // Vector-memory operations retire in order: once at most the stores of
+      // the first two steps are outstanding, every load has landed.
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(2 * kUnits));
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // where each block's windows start in LDS; a block outside the image or
+    // the band computes on the first block's data and is not stored
+    const float* base[kUnits];
+    bool live[kUnits];
+#pragma unroll
+    for (int i = 0; i < kUnits; ++i) {
+      live[i] = kRowsPerStep * s + unit_row[i] < n_rows &&
+                16 * unit_pb[i] < g.out_cols;
+      const int row0 = live[i] ? kNewRows * s + kStride * unit_row[i]
+                               : kNewRows * s;
+      const int pb = live[i] ? unit_pb[i] : 0;
+      base[i] = lds + row0 * kRowFloats + kStride * kCh * (16 * pb + px) + q;
+    }
+    float4v acc[kUnits];
+#pragma unroll
+    for (int i = 0; i < kUnits; ++i) acc[i] = float4v{0.f, 0.f, 0.f, 0.f};
+    // operands are fetched one group of matrix instructions ahead; the seven
+    // blocks take turns, so consecutive instructions never share an
+    // accumulator
+    float xv[2][kGroup][kUnits];
+    auto fetch = [&](int t0, float (&dst)[kGroup][kUnits]) {
+#pragma unroll
+      for (int e = 0; e < kGroup; ++e) {
+        const int t = t0 + e;
+        if (t < kSteps) {
+#pragma unroll
+          for (int i = 0; i < kUnits; ++i) {
+            const float* src = group_straddles(t)
+                                   ? base[i] + kspec[straddle_index(t)]
+                                   : base[i] + group_offset(t);
+            if (t == kSteps - 1) src = last_is_pad ? lds + zero_word : src;
+            dst[e][i] = *src;
+          }
+        }
+      }
+    };
+    fetch(0, xv[0]);
+#pragma unroll
+    for (int t0 = 0; t0 < kSteps; t0 += kGroup) {
+      // (fences: the compiler otherwise sinks each fetch to its use)
+      __builtin_amdgcn_sched_barrier(0);
+      if (t0 + kGroup < kSteps) fetch(t0 + kGroup, xv[(t0 / kGroup + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int e = 0; e < kGroup; ++e) {
+        const int t = t0 + e;
+        if (t < kSteps) {
+#pragma unroll
+          for (int i = 0; i < kUnits; ++i)
+            acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                wreg[t], xv[(t0 / kGroup) & 1][e][i], acc[i], 0, 0, 0);
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kUnits; ++i) {
+      const int oy = oy0 + kRowsPerStep * s + unit_row[i];
+      const int ox = 16 * unit_pb[i] + px;
+      const unsigned off =
+          (live[i] && ox < g.out_cols)
+              ? static_cast<unsigned>(((n * g.out_rows + oy) * g.out_cols + ox) *
+                                          kFeatures +
+                                      16 * fb + 4 * q) *
+                    4u
+              : kOobOffset;
+      __builtin_amdgcn_raw_buffer_store_b128(acc[i], y_rsrc, off, 0, kStoreAux);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+}
+
+bool make_geom(const snn_hip_conv2d_params& p, StemGeom* g) {
+  if (p.channels != kCh || p.features != kFeatures || p.window_rows != kWin ||
+      p.window_cols != kWin || p.stride_rows != kStride ||
+      p.stride_cols != kStride)
+    return false;
+  if (p.pad_rows < 0 || p.pad_cols < 0 || p.pad_rows >= kWin ||
+      p.pad_cols >= kWin || p.out_cols > 16 * kNpb || p.out_rows < 1)
+    return false;
+  const size_t in_bytes = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                          kCh * sizeof(float);
+  const size_t out_bytes = static_cast<size_t>(p.batch) * p.out_rows *
+                           p.out_cols * kFeatures * sizeof(float);
+  if (in_bytes > kMaxBufferBytes || out_bytes > kMaxBufferBytes) return false;
+  g->batch = p.batch; g->in_rows = p.in_rows; g->in_cols = p.in_cols;
+  g->out_rows = p.out_rows; g->out_cols = p.out_cols;
+  g->pad_rows = p.pad_rows; g->pad_cols = p.pad_cols;
+  // a row holds every column a window of the last output pixel block reads
+  const int cols_read = kStride * (16 * ceil_div(p.out_cols, 16) - 1) + kWin;
+  if (max(cols_read, p.in_cols + p.pad_cols) * kCh > kRowFloats) return false;
+  g->row_floats = kRowFloats;
+  g->loads_per_row = g->row_floats / 64;
+  // Below two images' worth of rows a band is a single step and the
+  // work-group's start-up (filter, first rows) is most of its time: the
+  // general kernels are quicker there.
+  if (static_cast<long>(p.batch) * p.out_rows < kMinOutputRows) return false;
+  // Bands per image: the count whose rounds of work-groups over the CUs,
+  // times the steps (plus start-up) of one work-group, come to the least,
+  // among those whose rows fit LDS and that give every CU a work-group when
+  // the layer has that many steps at all.
+  const int n_cus = 256;
+  const int max_bands = ceil_div(p.out_rows, kRowsPerStep);
+  long best_cost = -1;
+  for (int n_bands = 1; n_bands <= max_bands; ++n_bands) {
+    // whole steps of two output rows
+    const int band =
+        ceil_div(ceil_div(p.out_rows, n_bands), kRowsPerStep) * kRowsPerStep;
+    const int bands = ceil_div(p.out_rows, band);
+    const int lds_rows = kStride * band + kWin - kStride;
+    const size_t bytes =
+        (static_cast<size_t>(lds_rows + 1) * g->row_floats + 64) * sizeof(float);
+    if (bytes > kMaxLdsBytes) continue;
+    const size_t groups = static_cast<size_t>(p.batch) * bands;
+    const long rounds =
+        static_cast<long>(ceil_div(groups, static_cast<size_t>(n_cus)));
+    // start-up counted as a step and a half (in half steps)
+    const long cost = rounds * (band + 3);
+    if (best_cost < 0 || cost < best_cost) {
+      best_cost = cost;
+      g->band = band;
+      g->n_bands = bands;
+      g->lds_rows = lds_rows;
+    }
+  }
+  return best_cost >= 0;
+}
+
+}  // namespace
+
+bool conv2d_stem_supports(const snn_hip_conv2d_params& p) {
+  StemGeom g;
+  return make_geom(p, &g);
+}
+
+// The output must be 16-byte aligned (the loads need nothing beyond 4).
+int launch_conv2d_stem_f32(const float* x, const float* w, float* y,
+                           const snn_hip_conv2d_params& p,
+                           hipStream_t stream) {
+  StemGeom g;
+  if (!make_geom(p, &g)) return SNN_HIP_INVALID_ALGORITHM;
+  const size_t lds_bytes =
+      (static_cast<size_t>(g.lds_rows + 1) * g.row_floats + 64) * sizeof(float);
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(conv_stem_7x7s2_kernel),
+      hipFuncAttributeMaxDynamicSharedMemorySize,
+      static_cast<int>(kMaxLdsBytes));
+  (void)attr;
+  KernelTimer timer(stream);
+  hipLaunchKernelGGL(conv_stem_7x7s2_kernel,
+                     dim3(static_cast<unsigned>(p.batch * g.n_bands)),
+                     dim3(64 * kWaves), lds_bytes, stream, x, w, y, g);
+  return SNN_HIP_OK;
+}
+
+}  // namespace snn

@@ -107,6 +107,13 @@ bool gemm_wreg_supports(int m, int k, int n);
 void launch_gemm_wreg(const float* x, const float* w, float* y, int m, int k,
                       int n, bool epilogue, const float* bias, bool relu,
                       hipStream_t stream);
+// Forward convolution of a three-channel image with a 7x7 window, stride 2 and
+// 64 features (conv2d_stem.hip): input rows of a band of output rows in LDS,
+// the filter in registers.  Output 16-byte aligned, at most 128 output columns.
+bool conv2d_stem_supports(const snn_hip_conv2d_params& p);
+int launch_conv2d_stem_f32(const float* x, const float* w, float* y,
+                           const snn_hip_conv2d_params& p, hipStream_t stream);
+
 // The same in half precision with fp32 accumulation (gemm_wreg_f16.hip):
 // k = 64, 128, 256 or 512.
 bool gemm_wreg_f16_supports(int m, int k, int n);

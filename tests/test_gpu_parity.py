@@ -119,6 +119,22 @@ def test_stem_7x7_stride2(direction):
     conv_case(p, direction, [ALGO.DIRECT, ALGO.IM2COL], seed=300 + direction)
 
 
+@pytest.mark.parametrize("batch,rows,cols,same", [
+    (40, 64, 64, True),     # bands of three steps, two-row last band
+    (5, 97, 61, True),      # 49 x 31 output: ragged pixel block, odd rows
+    (6, 85, 100, False),    # no padding
+    (3, 223, 221, True),    # odd image, padding 3
+    (9, 224, 224, True),    # the stem layer itself, bands of two steps
+])
+def test_stem_rows_in_lds_kernel(batch, rows, cols, same):
+    """The 7x7 stride-2, 3 -> 64 channel forward kernel that keeps a band of
+    input rows in LDS (used from 224 output rows over the batch upwards)."""
+    p = ops.conv_params(batch, rows, cols, 3, 64, 7, 2, same)
+    assert batch * p.out_rows >= 224
+    conv_case(p, DIRECTION.FORWARD, [ALGO.IM2COL, ALGO.TILED],
+              seed=350 + batch + rows)
+
+
 def test_config0_single_image_tiled():
     """Benchmark configuration 0: N=1, 56x56x64 -> 64, 3x3 s1 SAME, Tiled;
     also checked against the reference-loop-nest restatement in fp32."""

@@ -126,7 +126,8 @@ def test_full_batch_backprop_3x3(size, ch, direction):
                                        DIRECTION.INPUT_BACKPROP,
                                        DIRECTION.FILTER_BACKPROP])
 def test_full_batch_stem_7x7_stride2(direction):
-    """[32,224,224,3] -> [32,112,112,64]: scalar gather forward, the
+    """[32,224,224,3] -> [32,112,112,64]: the rows-in-LDS forward kernel
+    (Im2col) beside the scalar gather forward (Direct), the
     one-work-group-per-64-features filter gradient, and the input gradient as a
     GEMM per output pixel + tap gather, whose temporary (112*112*147 floats
     per image) makes it run in minibatches of 9 images."""
