@@ -1,0 +1,413 @@
+// Half-precision filter gradient of 3x3 stride-1 SAME convolutions on the
+// binary16 matrix cores (gfx950).
+//
+//   dW[r][s][c][k] = sum over (n, oy, ox) of X[n][oy+r-1][ox+s-1][c] * dY[n][oy][ox][k]
+//
+// (the FilterBackprop direction of sycldnn::conv2d::launch,
+// include/portdnn/conv2d/launch.h:59-118; products of binary16 values summed
+// in fp32 and rounded to binary16 once).
+//
+// The reduction runs over pixels, which is the slow dimension of both
+// operands in memory (NHWC), while v_mfma_f32_32x32x16_f16 wants eight
+// consecutive reduction indices per lane.  ds_read_b64_tr_b16 does that
+// transposition on the way out of LDS: within 16 lanes, lane 4 j + i supplies
+// the address of four consecutive halves (columns 4 i ... 4 i + 3) of row j,
+// and lane t receives column t of rows 0 ... 3.  Two such reads make one
+// operand.
+//
+//   * A work-group (4 waves, one per SIMD, one work-group per CU) owns a
+//     64-channel x 64-feature tile of dW for all nine taps -- wave w a 32 x 32
+//     quarter of it, nine 32 x 32 accumulator blocks -- and walks a run of
+//     consecutive bands of output rows.  (A single wave issues the 32 x 32 x 16
+//     instruction at its full rate, the 16 x 16 x 32 one at 0.56 of it.)
+//   * A band's input rows (with the halo and zero padding, row pitch
+//     cols + 2 pixels) and dY rows (same pitch, zeros in the two extra
+//     columns) are loaded into LDS with 16-byte LDS-direct loads, padding
+//     through the buffer bounds.  With equal pitches the tap (r, s) operand of
+//     pixel m is the input pixel m + r * pitch + s: one flat run of pixels per
+//     band, cut into chunks of 16, whatever the image width.  Two LDS
+//     buffers: the next band arrives while this one is multiplied.
+//   * Per chunk and wave: one dY operand + 9 input operands (20 transposing
+//     reads, fetched one chunk ahead) feed 9 matrix instructions.
+//   * 16-byte pieces of a pixel are XOR-swizzled on the way in so that the 16
+//     lanes of a transposing read (4 pixels x 32 bytes) fall into distinct
+//     banks.
+//   * Float atomics retire one lane at a time (measured: 19 M of them cost
+//     60 us), so the partial tiles are stored, and a second kernel sums them
+//     and rounds to binary16.
+
+#include "snn_common.h"
+#include "snn_kernels.h"
+
+namespace snn {
+
+namespace {
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) void* lds_ptr;
+typedef __attribute__((address_space(3))) short4v* lds_short4_ptr;
+
+constexpr int kWaves = 4;
+constexpr int kTile = 64;         // channels and features per work-group
+constexpr int kTaps = 9;
+constexpr int kChunk = 16;        // pixels per matrix instruction
+constexpr int kPixelBytes = 128;  // 64 halves
+constexpr int kTileFloats = kTaps * kTile * kTile;
+constexpr int kBufBytes = 78 * 1024;  // one of the two LDS buffers
+constexpr int kNumCus = 256;
+constexpr int kReduceGroups = 16;  // partial sums per output in the reduction
+constexpr unsigned kOobOffset = 0x7FFFFFF0u;  // beyond every buffer's range
+constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
+
+struct FbGeom {
+  int batch, rows, cols, channels, features;
+  int pitch;            // cols + 2
+  unsigned pitch_magic; // ceil(2^32 / pitch)
+  int band;             // output rows per band
+  int bands_per_image;
+  int n_subbands;       // batch * bands_per_image
+  int group;            // bands per task (several whole images when small)
+  int n_tasks;
+  int x_px;             // LDS pixels of a band's input rows (multiple of 32)
+  int y_px;             // LDS pixels of a band's dY rows (multiple of 32)
+  int c_tiles, k_tiles, n_splits;
+  int per_split;        // consecutive tasks per work-group
+};
+
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* p,
+                                                   size_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0,
+                                           static_cast<unsigned>(bytes),
+                                           0x00020000);
+}
+
+constexpr int vmcnt_imm(int n) {
+  return 0x0F70 | (n & 15) | ((n >> 4) << 14);
+}
+
+// Which 16-byte position of LDS pixel p holds 16-byte piece c: c ^ swz(p).
+// Four consecutive pixels get four different piece pairs, and pixels 8 apart
+// swap the pairs of even and odd pixels.
+__device__ __forceinline__ unsigned swz(unsigned p) {
+  return ((p & 3u) ^ ((p >> 3) & 1u)) << 1;
+}
+
+__device__ __forceinline__ half8 read_transposed(const char* at_lo,
+                                                 const char* at_hi) {
+  const short4v lo =
+      __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(at_lo));
+  const short4v hi =
+      __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(at_hi));
+  const short8v both =
+      __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(half8, both);
+}
+
+// part: [split][tile][tap][64 channels][64 features] floats, each written once.
+__global__ void __launch_bounds__(64 * kWaves)
+    conv_filter_backprop_3x3_f16_kernel(const _Float16* __restrict__ x,
+                                        const _Float16* __restrict__ dy,
+                                        float* __restrict__ part, FbGeom g) {
+  // two objects, so that the compiler ties an LDS read to the loads of its
+  // own buffer only
+  __shared__ __align__(1024) char buf0[kBufBytes];
+  __shared__ __align__(1024) char buf1[kBufBytes];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int n_tiles = g.c_tiles * g.k_tiles;
+  const int tile = blockIdx.x % n_tiles;
+  const int split = blockIdx.x / n_tiles;
+  const int ct = tile % g.c_tiles;
+  const int kt = tile / g.c_tiles;
+
+  const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(
+      x, static_cast<size_t>(g.batch) * g.rows * g.cols * g.channels * 2);
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(
+      dy, static_cast<size_t>(g.batch) * g.rows * g.cols * g.features * 2);
+
+  const int sb_px = g.x_px + g.y_px;  // LDS pixels per band
+
+  // ---- transposing-read offsets, relative to the chunk's first pixel ------
+  // v_mfma_f32_32x32x16_f16: lane l holds row (or column) l % 32 at reduction
+  // indices 8 (l / 32) ... + 7.  Of lane = 16 gq + 4 j + e, as a source of the
+  // transposing read: pixel 8 (gq / 2) + j (+ 4 for the second read), halves
+  // 4 e ... 4 e + 3 of the 16-wide block gq % 2 of this wave's 32.
+  const unsigned gq = lane >> 4, j = (lane >> 2) & 3, e = lane & 3;
+  const unsigned c32 = wave & 1, k32 = wave >> 1;
+  unsigned off_x[kTaps][2];
+  unsigned off_y[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const unsigned p0 = 8 * (gq >> 1) + 4 * h + j;
+#pragma unroll
+    for (int tap = 0; tap < kTaps; ++tap) {
+      const unsigned p = (tap / 3) * g.pitch + (tap % 3) + p0;
+      off_x[tap][h] =
+          p * kPixelBytes +
+          (((4 * c32 + 2 * (gq & 1) + (e >> 1)) ^ swz(p)) << 4) + ((e & 1) << 3);
+    }
+    off_y[h] = (g.x_px + p0) * kPixelBytes +
+               (((4 * k32 + 2 * (gq & 1) + (e >> 1)) ^ swz(p0)) << 4) +
+               ((e & 1) << 3);
+  }
+
+  // acc[tap][i]: feature 32 k32 + 8 (i / 4) + 4 (lane / 32) + i % 4,
+  // channel 32 c32 + lane % 32
+  float16v acc[kTaps];
+#pragma unroll
+  for (int tap = 0; tap < kTaps; ++tap)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[tap][i] = 0.f;
+
+  const unsigned lane_px = lane >> 3;   // pixel of a load instruction's eight
+  const unsigned lane_piece = lane & 7; // 16-byte position within the pixel
+  const int n_chunks = g.y_px / kChunk;
+
+  auto issue_task = [&](int task, char* buf) {
+    for (int i = 0; i < g.group; ++i) {
+      const int sb = task * g.group + i;
+      const bool live = sb < g.n_subbands;
+      const int n = sb / g.bands_per_image;
+      const int oy0 = (sb - n * g.bands_per_image) * g.band;
+      char* base = buf + i * sb_px * kPixelBytes;
+      for (int l = wave; l < g.x_px / 8; l += kWaves) {
+        const unsigned p = 8 * l + lane_px;
+        const unsigned row = __umulhi(p, g.pitch_magic);
+        const int col = static_cast<int>(p - row * g.pitch);
+        const int iy = oy0 - 1 + static_cast<int>(row);
+        const int ix = col - 1;
+        const bool ok = live && row < static_cast<unsigned>(g.band + 2) &&
+                        iy >= 0 && iy < g.rows && ix >= 0 && ix < g.cols;
+        const unsigned off =
+            (static_cast<unsigned>((n * g.rows + iy) * g.cols + ix) *
+                 g.channels + ct * kTile) * 2u +
+            ((lane_piece ^ swz(p)) << 4);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            x_rsrc, (lds_ptr)(base + l * 1024), 16, ok ? off : kOobOffset, 0, 0,
+            0);
+      }
+      char* ybase = base + g.x_px * kPixelBytes;
+      for (int l = wave; l < g.y_px / 8; l += kWaves) {
+        const unsigned p = 8 * l + lane_px;
+        const unsigned row = __umulhi(p, g.pitch_magic);
+        const int col = static_cast<int>(p - row * g.pitch);
+        const int oy = oy0 + static_cast<int>(row);
+        const bool ok = live && row < static_cast<unsigned>(g.band) &&
+                        oy < g.rows && col < g.cols;
+        const unsigned off =
+            (static_cast<unsigned>((n * g.rows + oy) * g.cols + col) *
+                 g.features + kt * kTile) * 2u +
+            ((lane_piece ^ swz(p)) << 4);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            dy_rsrc, (lds_ptr)(ybase + l * 1024), 16, ok ? off : kOobOffset, 0,
+            0, 0);
+      }
+    }
+  };
+
+  auto fetch = [&](const char* at, half8& ya, half8 (&xb)[kTaps]) {
+    ya = read_transposed(at + off_y[0], at + off_y[1]);
+#pragma unroll
+    for (int tap = 0; tap < kTaps; ++tap)
+      xb[tap] = read_transposed(at + off_x[tap][0], at + off_x[tap][1]);
+  };
+  auto multiply = [&](const half8& ya, const half8 (&xb)[kTaps]) {
+#pragma unroll
+    for (int tap = 0; tap < kTaps; ++tap)
+      acc[tap] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ya, xb[tap], acc[tap],
+                                                        0, 0, 0);
+  };
+
+  // Chunks of the task's live bands, operands fetched one chunk ahead (the
+  // last fetch repeats the last chunk).
+  auto multiply_task = [&](int task, const char* buf) {
+    const int live = min(g.group, g.n_subbands - task * g.group);
+    const int total = live * n_chunks;
+    half8 ya0, xb0[kTaps], ya1, xb1[kTaps];
+    int next_px = 0, next_chunk = 0, fetched = 0;
+    auto advance = [&]() {
+      if (fetched + 1 < total) {
+        ++fetched;
+        next_px += kChunk;
+        if (++next_chunk == n_chunks) {
+          next_chunk = 0;
+          next_px += g.x_px;
+        }
+      }
+    };
+    fetch(buf, ya0, xb0);
+    for (int f = 0; f < total; f += 2) {
+      advance();
+      fetch(buf + next_px * kPixelBytes, ya1, xb1);
+      multiply(ya0, xb0);
+      if (f + 1 >= total) break;
+      advance();
+      fetch(buf + next_px * kPixelBytes, ya0, xb0);
+      multiply(ya1, xb1);
+    }
+  };
+
+  // ---- bands: load one ahead ------------------------------------------------
+#define SNN_FILBK_STEP(cur, nxt)                              \
+  {                                                           \
+    if (task >= task_end) break;                              \
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));                 \
+    __syncthreads();                                          \
+    if (task + 1 < task_end) issue_task(task + 1, nxt);       \
+    multiply_task(task, cur);                                 \
+    ++task;                                                   \
+  }
+  // consecutive bands: the halo rows a band shares with the one before it
+  // are still in this XCD's L2
+  int task = split * g.per_split;
+  const int task_end = min(g.n_tasks, task + g.per_split);
+  if (task < task_end) issue_task(task, buf0);
+  for (;;) {
+    SNN_FILBK_STEP(buf0, buf1)
+    SNN_FILBK_STEP(buf1, buf0)
+  }
+#undef SNN_FILBK_STEP
+
+  // ---- store the partial tile ------------------------------------------------
+  float* out = part + (static_cast<size_t>(split) * n_tiles + tile) * kTileFloats;
+  const unsigned c = 32 * c32 + (lane & 31);
+#pragma unroll
+  for (int tap = 0; tap < kTaps; ++tap)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const unsigned k = 32 * k32 + 8 * i4 + 4 * (lane >> 5);
+      const float4v v = {acc[tap][4 * i4], acc[tap][4 * i4 + 1],
+                         acc[tap][4 * i4 + 2], acc[tap][4 * i4 + 3]};
+      *reinterpret_cast<float4v*>(out + (tap * kTile + c) * kTile + k) = v;
+    }
+}
+
+// Sums the partial tiles and rounds: a work-group is 256 / n_groups
+// consecutive float4 of the filter x n_groups groups of splits (a power of two
+// up to 16).
+__global__ void __launch_bounds__(256)
+    filter_backprop_f16_reduce_kernel(const float4v* __restrict__ part,
+                                      _Float16* __restrict__ dw, int n_tiles,
+                                      int c_tiles, int n_splits, int n_groups,
+                                      int channels, int features) {
+  __shared__ float4v sums[256];
+  constexpr int kTileVecs = kTileFloats / 4;
+  const int width = 256 / n_groups;
+  const int lane_o = threadIdx.x % width;
+  const int group = threadIdx.x / width;
+  const unsigned o = blockIdx.x * width + lane_o;  // float4 of the whole filter
+  const unsigned tile = o / kTileVecs;
+  const unsigned local = o - tile * kTileVecs;
+  float4v sum = {0.f, 0.f, 0.f, 0.f};
+  for (int sp = group; sp < n_splits; sp += n_groups)
+    sum += part[(static_cast<size_t>(sp) * n_tiles + tile) * kTileVecs + local];
+  sums[threadIdx.x] = sum;
+  __syncthreads();
+  if (group != 0) return;
+  for (int i = 1; i < n_groups; ++i) sum += sums[i * width + lane_o];
+  const unsigned tap = local / (kTile * kTile / 4);
+  const unsigned c = (local / (kTile / 4)) % kTile;
+  const unsigned k4 = local % (kTile / 4);
+  const unsigned ct = tile % c_tiles, kt = tile / c_tiles;
+  typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+  half4v r;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) r[v] = static_cast<_Float16>(sum[v]);
+  *reinterpret_cast<half4v*>(
+      dw + (static_cast<size_t>(tap) * channels + ct * kTile + c) * features +
+      kt * kTile + 4 * k4) = r;
+}
+
+int round_up(int a, int b) { return ceil_div(a, b) * b; }
+
+bool make_geom(const snn_hip_conv2d_params& p, FbGeom* g) {
+  if (p.window_rows != 3 || p.window_cols != 3 || p.stride_rows != 1 ||
+      p.stride_cols != 1 || p.pad_rows != 1 || p.pad_cols != 1 ||
+      p.out_rows != p.in_rows || p.out_cols != p.in_cols)
+    return false;
+  if (p.channels % kTile != 0 || p.features % kTile != 0 || p.batch < 1)
+    return false;
+  const size_t x_bytes = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                         p.channels * 2;
+  const size_t y_bytes = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                         p.features * 2;
+  if (x_bytes > kMaxBufferBytes || y_bytes > kMaxBufferBytes) return false;
+  g->batch = p.batch; g->rows = p.in_rows; g->cols = p.in_cols;
+  g->channels = p.channels; g->features = p.features;
+  g->pitch = p.in_cols + 2;
+  g->pitch_magic = 0xFFFFFFFFu / static_cast<unsigned>(g->pitch) + 1u;
+  // the most rows whose band fits a buffer, then evened out over the image
+  auto band_px = [&](int band, int* x_px, int* y_px) {
+    *y_px = round_up(band * g->pitch, kChunk);
+    *x_px = round_up(*y_px + 2 * g->pitch + 2, kChunk);
+    return *x_px + *y_px;
+  };
+  int x_px = 0, y_px = 0, band = 0;
+  for (int r = 1; r <= p.in_rows; ++r) {
+    if (band_px(r, &x_px, &y_px) * kPixelBytes > kBufBytes) break;
+    band = r;
+  }
+  if (band == 0) return false;
+  g->bands_per_image = ceil_div(p.in_rows, band);
+  g->band = ceil_div(p.in_rows, g->bands_per_image);
+  const int sb_px = band_px(g->band, &x_px, &y_px);
+  g->x_px = x_px; g->y_px = y_px;
+  g->n_subbands = p.batch * g->bands_per_image;
+  g->group = 1;
+  if (g->bands_per_image == 1)
+    g->group = max(1, min(p.batch, kBufBytes / (sb_px * kPixelBytes)));
+  g->n_tasks = ceil_div(g->n_subbands, g->group);
+  g->c_tiles = p.channels / kTile;
+  g->k_tiles = p.features / kTile;
+  const int n_tiles = g->c_tiles * g->k_tiles;
+  const int want = max(1, min(g->n_tasks, kNumCus / n_tiles));
+  g->per_split = ceil_div(g->n_tasks, want);
+  g->n_splits = ceil_div(g->n_tasks, g->per_split);
+  return true;
+}
+
+}  // namespace
+
+bool conv2d_filter_backprop_3x3_f16_supports(const snn_hip_conv2d_params& p) {
+  FbGeom g;
+  return make_geom(p, &g);
+}
+
+size_t conv2d_filter_backprop_3x3_f16_partial_floats(
+    const snn_hip_conv2d_params& p) {
+  FbGeom g;
+  if (!make_geom(p, &g)) return 0;
+  return static_cast<size_t>(g.n_splits) * g.c_tiles * g.k_tiles * kTileFloats;
+}
+
+// x, dy, dw 16-byte aligned; part holds
+// conv2d_filter_backprop_3x3_f16_partial_floats(p) floats.
+int launch_conv2d_filter_backprop_3x3_f16(const _Float16* x,
+                                          const _Float16* dy, _Float16* dw,
+                                          float* part,
+                                          const snn_hip_conv2d_params& p,
+                                          hipStream_t stream) {
+  FbGeom g;
+  if (!make_geom(p, &g)) return SNN_HIP_INVALID_ALGORITHM;
+  const int n_tiles = g.c_tiles * g.k_tiles;
+  {
+    KernelTimer timer(stream);
+    hipLaunchKernelGGL(conv_filter_backprop_3x3_f16_kernel,
+                       dim3(static_cast<unsigned>(n_tiles * g.n_splits)),
+                       dim3(64 * kWaves), 0, stream, x, dy, part, g);
+  }
+  const unsigned vecs = static_cast<unsigned>(n_tiles) * (kTileFloats / 4);
+  int n_groups = 1;
+  while (n_groups < kReduceGroups && 2 * n_groups <= g.n_splits) n_groups *= 2;
+  hipLaunchKernelGGL(filter_backprop_f16_reduce_kernel,
+                     dim3(vecs / (256 / n_groups)), dim3(256), 0, stream,
+                     reinterpret_cast<const float4v*>(part), dw, n_tiles,
+                     g.c_tiles, g.n_splits, n_groups, p.channels, p.features);
+  return SNN_HIP_OK;
+}
+
+}  // namespace snn

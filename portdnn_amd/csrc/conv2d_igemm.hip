@@ -1887,6 +1887,31 @@ int launch_conv2d_filter_backprop_f16(const _Float16* x, const _Float16* dy,
   const size_t dy_elems = static_cast<size_t>(g.m_total) * p.features;
   const size_t dw_elems = static_cast<size_t>(p.window_rows) * p.window_cols *
                           p.channels * p.features;
+  const bool ws_aligned =
+      workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0;
+  if (conv2d_filter_backprop_3x3_f16_supports(p) &&
+      (reinterpret_cast<uintptr_t>(dw) & 7u) == 0 &&
+      SNN_TUNING_ENV("SNN_HIP_FILBK_F16_OFF") == nullptr) {
+    // binary16 matrix instructions; the partial tiles go to the workspace
+    // when it holds them, else to a stream-ordered temporary
+    const size_t part_floats = conv2d_filter_backprop_3x3_f16_partial_floats(p);
+    float* part = reinterpret_cast<float*>(workspace);
+    const bool own = !ws_aligned || workspace_elems < 2 * part_floats;
+    if (own) {
+      void* ptr = nullptr;
+      if (temp_malloc_async(&ptr, part_floats * sizeof(float), stream) !=
+          hipSuccess)
+        return SNN_HIP_ALLOCATION_PROBLEM;
+      part = static_cast<float*>(ptr);
+    }
+    const int status =
+        launch_conv2d_filter_backprop_3x3_f16(x, dy, dw, part, p, stream);
+    const hipError_t err = hipGetLastError();
+    if (own) temp_free_async(part, stream);
+    if (status != SNN_HIP_OK) return status;
+    if (err != hipSuccess) return report_hip_error(err, "f16 filter backprop");
+    return SNN_HIP_OK;
+  }
   float* acc32 = reinterpret_cast<float*>(workspace);
   bool temporary = false;
   if (workspace == nullptr || workspace_elems < 2 * dw_elems ||

@@ -149,6 +149,17 @@ int launch_conv2d_input_backprop_f16(const _Float16* dy,
 // 64 (fp32 accumulation buffer in the workspace when it holds twice the
 // filter's element count, else a stream-ordered temporary), and the input
 // gradient for the shapes launch_conv2d_input_backprop_f16 does not take.
+// conv2d_filter_backprop_f16.hip: 3x3 stride-1 SAME filter gradient on the
+// binary16 matrix cores (channels and features multiples of 64).  `part` is
+// scratch of ..._partial_floats(p) floats for the partial tiles.
+bool conv2d_filter_backprop_3x3_f16_supports(const snn_hip_conv2d_params& p);
+size_t conv2d_filter_backprop_3x3_f16_partial_floats(
+    const snn_hip_conv2d_params& p);
+int launch_conv2d_filter_backprop_3x3_f16(const _Float16* x,
+                                          const _Float16* dy, _Float16* dw,
+                                          float* part,
+                                          const snn_hip_conv2d_params& p,
+                                          hipStream_t stream);
 bool conv2d_filter_backprop_f16_supports(const snn_hip_conv2d_params& p);
 int launch_conv2d_filter_backprop_f16(const _Float16* x, const _Float16* dy,
                                       _Float16* dw,

@@ -1068,6 +1068,37 @@ def test_f16_conv_filter_backprop_on_matrix_cores(shape):
         assert_close_f16(got, ref, ("f16 filbk mfma", shape, ws is None))
 
 
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features
+    (3, 17, 9, 64, 128),     # odd image, two feature tiles
+    (2, 10, 30, 128, 64),    # two channel tiles
+    (1, 20, 120, 64, 64),    # wide rows: bands of one row
+    (5, 7, 7, 64, 64),       # several images per LDS buffer, ragged last task
+    (7, 14, 14, 192, 64),    # three channel tiles
+    (300, 7, 7, 64, 64),     # more tasks than work-groups
+    (9, 56, 56, 64, 64),     # runs of consecutive bands across images
+])
+def test_f16_filter_backprop_3x3_transposing_reads(shape):
+    """The 3x3 stride-1 SAME half-precision filter gradient on the binary16
+    matrix cores (LDS transposing reads, partial tiles + reduction) against
+    the oracle in double precision on the same half-rounded operands."""
+    batch, rows, cols, ch, feats = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, 3, 1, True)
+    rng = np.random.default_rng(795 + rows + feats + batch)
+    n_x, n_dy, n_dw = ops.conv_sizes(p, DIRECTION.FILTER_BACKPROP)
+    x = uniform(rng, n_x).astype(np.float16)
+    dy = uniform(rng, n_dy).astype(np.float16)
+    ref = oracle.conv2d_filter_backprop(x.astype(np.float32),
+                                        dy.astype(np.float32),
+                                        oracle_params(p, feats), acc64=True)
+    dx_, ddy = dev(x, torch.float16), dev(dy, torch.float16)
+    for ws in (None, torch.empty(2 * 256 * 9 * 64 * 64, dtype=torch.float16,
+                                 device="cuda")):
+        got = ops.conv2d(dx_, ddy, p, DIRECTION.FILTER_BACKPROP, ALGO.IM2COL,
+                         workspace=ws).float().cpu().numpy()
+        assert_close_f16(got, ref, ("f16 filbk 3x3", shape, ws is None))
+
+
 def test_f16_conv_filter_backprop():
     p = ops.conv_params(3, 10, 9, 16, 24, 3, 1, True)
     rng = np.random.default_rng(781)
