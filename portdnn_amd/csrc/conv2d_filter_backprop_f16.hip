@@ -27,8 +27,12 @@
 //     pixel m is the input pixel m + r * pitch + s: one flat run of pixels per
 //     band, cut into chunks of 16, whatever the image width.  Two LDS
 //     buffers: the next band arrives while this one is multiplied.
-//   * Per chunk and wave: one dY operand + 9 input operands (20 transposing
-//     reads, fetched one chunk ahead) feed 9 matrix instructions.
+//   * Per chunk and wave: one dY operand (2 transposing reads) + per filter
+//     row 12 consecutive input pixels (3 reads), whose windows at pixel 0, 1
+//     and 2 are the row's three taps (one funnel shift per register for the
+//     middle one): 11 reads, fetched one chunk ahead, feed 9 matrix
+//     instructions.  A wave issues one such read per 32 cycles (measured), a
+//     32x32x16 instruction takes 32.
 //   * 16-byte pieces of a pixel are XOR-swizzled on the way in so that the 16
 //     lanes of a transposing read (4 pixels x 32 bytes) fall into distinct
 //     banks.
@@ -48,6 +52,8 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef short short8v __attribute__((ext_vector_type(8)));
+typedef unsigned uint2v __attribute__((ext_vector_type(2)));
+typedef unsigned uint4v __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void* lds_ptr;
 typedef __attribute__((address_space(3))) short4v* lds_short4_ptr;
 
@@ -107,7 +113,13 @@ __device__ __forceinline__ half8 read_transposed(const char* at_lo,
   return __builtin_bit_cast(half8, both);
 }
 
-// part: [split][tile][tap][64 channels][64 features] floats, each written once.
+__device__ __forceinline__ uint2v read_transposed4(const char* at) {
+  return __builtin_bit_cast(
+      uint2v, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(at)));
+}
+
+// part: [split][tile] tiles of 9 x 64 x 64 floats in accumulator order, each
+// written once.
 __global__ void __launch_bounds__(64 * kWaves)
     conv_filter_backprop_3x3_f16_kernel(const _Float16* __restrict__ x,
                                         const _Float16* __restrict__ dy,
@@ -138,21 +150,26 @@ __global__ void __launch_bounds__(64 * kWaves)
   // 4 e ... 4 e + 3 of the 16-wide block gq % 2 of this wave's 32.
   const unsigned gq = lane >> 4, j = (lane >> 2) & 3, e = lane & 3;
   const unsigned c32 = wave & 1, k32 = wave >> 1;
-  unsigned off_x[kTaps][2];
+  // Input operands: per filter row three reads of 4 pixels (12 consecutive
+  // pixels per lane); the three taps of the row are the 8-pixel windows at
+  // pixel 0, 1 and 2 of them.  (A wave can issue one such read per 32 cycles:
+  // 11 reads per chunk instead of 20 keep it near the matrix rate.)
+  unsigned off_x[3][3];
   unsigned off_y[2];
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
+  for (int h = 0; h < 3; ++h) {
     const unsigned p0 = 8 * (gq >> 1) + 4 * h + j;
 #pragma unroll
-    for (int tap = 0; tap < kTaps; ++tap) {
-      const unsigned p = (tap / 3) * g.pitch + (tap % 3) + p0;
-      off_x[tap][h] =
+    for (int r = 0; r < 3; ++r) {
+      const unsigned p = r * g.pitch + p0;
+      off_x[r][h] =
           p * kPixelBytes +
           (((4 * c32 + 2 * (gq & 1) + (e >> 1)) ^ swz(p)) << 4) + ((e & 1) << 3);
     }
-    off_y[h] = (g.x_px + p0) * kPixelBytes +
-               (((4 * k32 + 2 * (gq & 1) + (e >> 1)) ^ swz(p0)) << 4) +
-               ((e & 1) << 3);
+    if (h < 2)
+      off_y[h] = (g.x_px + p0) * kPixelBytes +
+                 (((4 * k32 + 2 * (gq & 1) + (e >> 1)) ^ swz(p0)) << 4) +
+                 ((e & 1) << 3);
   }
 
   // acc[tap][i]: feature 32 k32 + 8 (i / 4) + 4 (lane / 32) + i % 4,
@@ -209,17 +226,34 @@ __global__ void __launch_bounds__(64 * kWaves)
     }
   };
 
-  auto fetch = [&](const char* at, half8& ya, half8 (&xb)[kTaps]) {
+  // xw[r][h]: pixels 4 h ... 4 h + 3 of filter row r's 12, two halves a register
+  auto fetch = [&](const char* at, half8& ya, uint2v (&xw)[3][3]) {
     ya = read_transposed(at + off_y[0], at + off_y[1]);
 #pragma unroll
-    for (int tap = 0; tap < kTaps; ++tap)
-      xb[tap] = read_transposed(at + off_x[tap][0], at + off_x[tap][1]);
-  };
-  auto multiply = [&](const half8& ya, const half8 (&xb)[kTaps]) {
+    for (int r = 0; r < 3; ++r)
 #pragma unroll
-    for (int tap = 0; tap < kTaps; ++tap)
-      acc[tap] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ya, xb[tap], acc[tap],
-                                                        0, 0, 0);
+      for (int h = 0; h < 3; ++h) xw[r][h] = read_transposed4(at + off_x[r][h]);
+  };
+  // The windows are cut out of the 12 pixels here, a chunk after the reads
+  // were issued, so that nothing waits on them.
+  auto multiply = [&](const half8& ya, const uint2v (&xw)[3][3]) {
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      const unsigned w0 = xw[r][0][0], w1 = xw[r][0][1], w2 = xw[r][1][0],
+                     w3 = xw[r][1][1], w4 = xw[r][2][0];
+      const uint4v s0 = {w0, w1, w2, w3};
+      const uint4v s1 = {__builtin_amdgcn_alignbit(w1, w0, 16),
+                         __builtin_amdgcn_alignbit(w2, w1, 16),
+                         __builtin_amdgcn_alignbit(w3, w2, 16),
+                         __builtin_amdgcn_alignbit(w4, w3, 16)};
+      const uint4v s2 = {w1, w2, w3, w4};
+      acc[3 * r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+          ya, __builtin_bit_cast(half8, s0), acc[3 * r], 0, 0, 0);
+      acc[3 * r + 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+          ya, __builtin_bit_cast(half8, s1), acc[3 * r + 1], 0, 0, 0);
+      acc[3 * r + 2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+          ya, __builtin_bit_cast(half8, s2), acc[3 * r + 2], 0, 0, 0);
+    }
   };
 
   // Chunks of the task's live bands, operands fetched one chunk ahead (the
@@ -227,7 +261,8 @@ __global__ void __launch_bounds__(64 * kWaves)
   auto multiply_task = [&](int task, const char* buf) {
     const int live = min(g.group, g.n_subbands - task * g.group);
     const int total = live * n_chunks;
-    half8 ya0, xb0[kTaps], ya1, xb1[kTaps];
+    half8 ya0, ya1;
+    uint2v xb0[3][3], xb1[3][3];
     int next_px = 0, next_chunk = 0, fetched = 0;
     auto advance = [&]() {
       if (fetched + 1 < total) {
@@ -239,14 +274,20 @@ __global__ void __launch_bounds__(64 * kWaves)
         }
       }
     };
+    // (fences: the compiler otherwise sinks the reads next to their uses and
+    // waits out the LDS latency twice per chunk)
     fetch(buf, ya0, xb0);
     for (int f = 0; f < total; f += 2) {
       advance();
+      __builtin_amdgcn_sched_barrier(0);
       fetch(buf + next_px * kPixelBytes, ya1, xb1);
+      __builtin_amdgcn_sched_barrier(0);
       multiply(ya0, xb0);
       if (f + 1 >= total) break;
       advance();
+      __builtin_amdgcn_sched_barrier(0);
       fetch(buf + next_px * kPixelBytes, ya0, xb0);
+      __builtin_amdgcn_sched_barrier(0);
       multiply(ya1, xb1);
     }
   };
@@ -274,15 +315,16 @@ __global__ void __launch_bounds__(64 * kWaves)
 
   // ---- store the partial tile ------------------------------------------------
   float* out = part + (static_cast<size_t>(split) * n_tiles + tile) * kTileFloats;
-  const unsigned c = 32 * c32 + (lane & 31);
+  // in accumulator order, [tap][wave][i4][lane] float4: every store
+  // instruction writes 1 KB of consecutive memory
 #pragma unroll
   for (int tap = 0; tap < kTaps; ++tap)
 #pragma unroll
     for (int i4 = 0; i4 < 4; ++i4) {
-      const unsigned k = 32 * k32 + 8 * i4 + 4 * (lane >> 5);
       const float4v v = {acc[tap][4 * i4], acc[tap][4 * i4 + 1],
                          acc[tap][4 * i4 + 2], acc[tap][4 * i4 + 3]};
-      *reinterpret_cast<float4v*>(out + (tap * kTile + c) * kTile + k) = v;
+      *reinterpret_cast<float4v*>(
+          out + (((tap * kWaves + wave) * 4 + i4) * 64 + lane) * 4) = v;
     }
 }
 
@@ -309,9 +351,13 @@ __global__ void __launch_bounds__(256)
   __syncthreads();
   if (group != 0) return;
   for (int i = 1; i < n_groups; ++i) sum += sums[i * width + lane_o];
-  const unsigned tap = local / (kTile * kTile / 4);
-  const unsigned c = (local / (kTile / 4)) % kTile;
-  const unsigned k4 = local % (kTile / 4);
+  // accumulator order of the partial tiles: local = ((tap * 4 + wave) * 4 +
+  // i4) * 64 + lane holds channel 32 (wave & 1) + lane % 32 and features
+  // 32 (wave >> 1) + 8 i4 + 4 (lane / 32) ... + 3
+  const unsigned ln = local & 63, i4 = (local >> 6) & 3, wv = (local >> 8) & 3;
+  const unsigned tap = local >> 10;
+  const unsigned c = 32 * (wv & 1) + (ln & 31);
+  const unsigned k4 = 8 * (wv >> 1) + 2 * i4 + (ln >> 5);
   const unsigned ct = tile % c_tiles, kt = tile / c_tiles;
   typedef _Float16 half4v __attribute__((ext_vector_type(4)));
   half4v r;
@@ -343,7 +389,8 @@ bool make_geom(const snn_hip_conv2d_params& p, FbGeom* g) {
   // the most rows whose band fits a buffer, then evened out over the image
   auto band_px = [&](int band, int* x_px, int* y_px) {
     *y_px = round_up(band * g->pitch, kChunk);
-    *x_px = round_up(*y_px + 2 * g->pitch + 2, kChunk);
+    // (the third read of a row reaches two pixels past the last window)
+    *x_px = round_up(*y_px + 2 * g->pitch + 4, kChunk);
     return *x_px + *y_px;
   };
   int x_px = 0, y_px = 0, band = 0;
