@@ -1795,7 +1795,11 @@ static int launch_filter_backprop(const float* x, const float* dy, float* dw,
   const int tiles = (p.window_rows * p.window_cols * p.channels / 64) *
                     ceil_div(p.features, 64);
   const int n_chunks = ceil_div(g.m_total, kBK);
-  int splits = max(1, min(ceil_div(kSplitUnits, tiles),
+  // (1x1 windows: half as many units measured 2-14 % faster on the four
+  // batch-32 K = 4C layers, 3x3 windows up to 13 % slower on the deeper two)
+  const int units =
+      p.window_rows * p.window_cols == 1 ? kSplitUnits / 2 : kSplitUnits;
+  int splits = max(1, min(ceil_div(units, tiles),
                           n_chunks / kMinChunksPerSplit));
   const int per_split = ceil_div(n_chunks, splits);
   splits = ceil_div(n_chunks, per_split);
