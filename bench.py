@@ -360,7 +360,8 @@ def main():
                 del ws
         detail["algorithms"] = algo_table
 
-        # backprops of the 3x3 layers and the 7x7 s2 stem in all directions.
+        # backprops of the 3x3 and 1x1 layers and the 7x7 s2 stem in all
+        # directions.
         # `tflops_reference_accounting` counts the two gradients by input
         # pixels, 2*N*H*W*R*S*C*K, as the reference's benchmarks do
         # (bench/conv2d/base_convolution_fixture.h:91-109), which at stride 2
@@ -372,7 +373,7 @@ def main():
         cases = [("stem7x7_s2_224x224x3_k64", stem, d) for d in (
             DIRECTION.FORWARD, DIRECTION.INPUT_BACKPROP,
             DIRECTION.FILTER_BACKPROP)]
-        for w in work[:4]:
+        for w in work[:8]:  # the four 3x3 layers, then the four 1x1 layers
             cases += [(w["name"], w["p"], DIRECTION.INPUT_BACKPROP),
                       (w["name"], w["p"], DIRECTION.FILTER_BACKPROP)]
         dir_names = {DIRECTION.FORWARD: "forward",

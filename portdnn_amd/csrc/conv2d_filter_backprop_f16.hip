@@ -1,5 +1,5 @@
-// Half-precision filter gradient of 3x3 stride-1 SAME convolutions on the
-// binary16 matrix cores (gfx950).
+// Half-precision filter gradient of 3x3 stride-1 SAME convolutions (and, at
+// the end of the file, of 1x1 ones) on the binary16 matrix cores (gfx950).
 //
 //   dW[r][s][c][k] = sum over (n, oy, ox) of X[n][oy+r-1][ox+s-1][c] * dY[n][oy][ox][k]
 //
@@ -417,6 +417,263 @@ bool make_geom(const snn_hip_conv2d_params& p, FbGeom* g) {
   return true;
 }
 
+// ---------------------------------------------------------------------------
+// 1x1 (stride 1, no padding): dW[c][k] = sum over pixels m of X[m][c] * dY[m][k],
+// one flat stream of pixels.  A work-group (4 waves, 2 x 2) owns a tile of
+// (64 A) channels x (64 B) features of dW and a range of the pixels; wave
+// (wc, wk) its quarter at (wc, wk), A x B blocks of 32 x 32.  Stages of 64
+// pixels, [pixel][64 A channels] and [pixel][64 B features], arrive in two
+// LDS buffers by LDS-direct loads (swizzled as
+// above); per chunk of 16 pixels a wave fetches A + B operands for A x B
+// matrix instructions.  The layers are bound by the bytes moved (the tile has
+// 32 A B / (A + B) flop per loaded byte, and each work-group stores one
+// partial tile), so the tile shape is picked to make loads plus partial
+// tiles least.
+struct Fb1Geom {
+  int pixels, channels, features;
+  int c_tiles, k_tiles, n_splits;
+  int n_stages, per_split;  // stages of kStagePx pixels; consecutive per split
+};
+constexpr int kStagePx = 64;
+
+template <int A, int B>
+__device__ __forceinline__ void filter_backprop_1x1_body(
+    const _Float16* __restrict__ x, const _Float16* __restrict__ dy,
+    float* __restrict__ part, const Fb1Geom& g, char* buf0, char* buf1) {
+  constexpr int kXBytes = 128 * A;  // per pixel
+  constexpr int kYBytes = 128 * B;
+  constexpr int kXStage = kStagePx * kXBytes;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wc = wave & 1, wk = wave >> 1;
+  const int n_tiles = g.c_tiles * g.k_tiles;
+  const int tile = blockIdx.x % n_tiles;
+  const int split = blockIdx.x / n_tiles;
+  const int ct = tile % g.c_tiles;
+  const int kt = tile / g.c_tiles;
+  const __amdgpu_buffer_rsrc_t x_rsrc =
+      make_rsrc(x, static_cast<size_t>(g.pixels) * g.channels * 2);
+  const __amdgpu_buffer_rsrc_t dy_rsrc =
+      make_rsrc(dy, static_cast<size_t>(g.pixels) * g.features * 2);
+
+  // transposing-read offsets within a chunk (see the 3x3 kernel)
+  const unsigned gq = lane >> 4, j = (lane >> 2) & 3, e = lane & 3;
+  unsigned off_x[A][2], off_y[B][2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const unsigned p = 8 * (gq >> 1) + 4 * h + j;
+#pragma unroll
+    for (int i = 0; i < A; ++i) {
+      const unsigned piece = 4 * (wc * A + i) + 2 * (gq & 1) + (e >> 1);
+      off_x[i][h] = p * kXBytes + ((piece ^ swz(p)) << 4) + ((e & 1) << 3);
+    }
+#pragma unroll
+    for (int i = 0; i < B; ++i) {
+      const unsigned piece = 4 * (wk * B + i) + 2 * (gq & 1) + (e >> 1);
+      off_y[i][h] =
+          kXStage + p * kYBytes + ((piece ^ swz(p)) << 4) + ((e & 1) << 3);
+    }
+  }
+
+  float16v acc[A][B];
+#pragma unroll
+  for (int ia = 0; ia < A; ++ia)
+#pragma unroll
+    for (int ib = 0; ib < B; ++ib)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[ia][ib][i] = 0.f;
+
+  // a 1 KB load covers 8 / A pixels of X (8 / B of dY)
+  auto issue_stage = [&](int stage, char* buf) {
+    const unsigned m0 = static_cast<unsigned>(stage) * kStagePx;
+    constexpr int kXPieces = 8 * A, kYPieces = 8 * B;
+    for (int l = wave; l < kStagePx * kXPieces / 64; l += kWaves) {
+      const unsigned p = (64 * l + lane) / kXPieces;
+      const unsigned piece = (64 * l + lane) % kXPieces;
+      const unsigned m = m0 + p;
+      const unsigned off =
+          (m * g.channels + ct * 64 * A) * 2u + ((piece ^ swz(p)) << 4);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          x_rsrc, (lds_ptr)(buf + l * 1024), 16,
+          m < static_cast<unsigned>(g.pixels) ? off : kOobOffset, 0, 0, 0);
+    }
+    for (int l = wave; l < kStagePx * kYPieces / 64; l += kWaves) {
+      const unsigned p = (64 * l + lane) / kYPieces;
+      const unsigned piece = (64 * l + lane) % kYPieces;
+      const unsigned m = m0 + p;
+      const unsigned off =
+          (m * g.features + kt * 64 * B) * 2u + ((piece ^ swz(p)) << 4);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          dy_rsrc, (lds_ptr)(buf + kXStage + l * 1024), 16,
+          m < static_cast<unsigned>(g.pixels) ? off : kOobOffset, 0, 0, 0);
+    }
+  };
+
+  auto multiply_stage = [&](const char* buf) {
+    half8 xa[2][A], yb[2][B];
+    auto fetch = [&](int chunk, half8 (&xo)[A], half8 (&yo)[B]) {
+      const char* xat = buf + chunk * kChunk * kXBytes;
+      const char* yat = buf + chunk * kChunk * kYBytes;
+#pragma unroll
+      for (int i = 0; i < A; ++i)
+        xo[i] = read_transposed(xat + off_x[i][0], xat + off_x[i][1]);
+#pragma unroll
+      for (int i = 0; i < B; ++i)
+        yo[i] = read_transposed(yat + off_y[i][0], yat + off_y[i][1]);
+    };
+    fetch(0, xa[0], yb[0]);
+#pragma unroll
+    for (int chunk = 0; chunk < kStagePx / kChunk; ++chunk) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (chunk + 1 < kStagePx / kChunk)
+        fetch(chunk + 1, xa[(chunk + 1) & 1], yb[(chunk + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ia = 0; ia < A; ++ia)
+#pragma unroll
+        for (int ib = 0; ib < B; ++ib)
+          acc[ia][ib] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+              yb[chunk & 1][ib], xa[chunk & 1][ia], acc[ia][ib], 0, 0, 0);
+    }
+  };
+
+#define SNN_FILBK1_STEP(cur, nxt)                               \
+  {                                                             \
+    if (stage >= stage_end) break;                              \
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));                   \
+    __syncthreads();                                            \
+    if (stage + 1 < stage_end) issue_stage(stage + 1, nxt);     \
+    multiply_stage(cur);                                        \
+    ++stage;                                                    \
+  }
+  int stage = split * g.per_split;
+  const int stage_end = min(g.n_stages, stage + g.per_split);
+  if (stage < stage_end) issue_stage(stage, buf0);
+  for (;;) {
+    SNN_FILBK1_STEP(buf0, buf1)
+    SNN_FILBK1_STEP(buf1, buf0)
+  }
+#undef SNN_FILBK1_STEP
+
+  // partial tile in accumulator order: [wave][ia][ib][i4][lane] float4
+  float* out = part + (static_cast<size_t>(split) * n_tiles + tile) *
+                          (4096 * A * B);
+#pragma unroll
+  for (int ia = 0; ia < A; ++ia)
+#pragma unroll
+    for (int ib = 0; ib < B; ++ib)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const float4v v = {acc[ia][ib][4 * i4], acc[ia][ib][4 * i4 + 1],
+                           acc[ia][ib][4 * i4 + 2], acc[ia][ib][4 * i4 + 3]};
+        *reinterpret_cast<float4v*>(
+            out + ((((wave * A + ia) * B + ib) * 4 + i4) * 64 + lane) * 4) = v;
+      }
+}
+
+// (plain functions around the template body: the compiler drops the host side
+// of a kernel template whose body names the LDS-direct load)
+#define SNN_FILBK1_KERNEL(A, B)                                              \
+  __global__ void __launch_bounds__(64 * kWaves)                             \
+      filter_backprop_1x1_f16_a##A##_b##B(const _Float16* __restrict__ x,    \
+                                          const _Float16* __restrict__ dy,   \
+                                          float* __restrict__ part,          \
+                                          Fb1Geom g) {                       \
+    __shared__ __align__(1024) char buf0[kStagePx * 128 * (A + B)];          \
+    __shared__ __align__(1024) char buf1[kStagePx * 128 * (A + B)];          \
+    filter_backprop_1x1_body<A, B>(x, dy, part, g, buf0, buf1);              \
+  }
+SNN_FILBK1_KERNEL(1, 1)
+SNN_FILBK1_KERNEL(1, 2)
+SNN_FILBK1_KERNEL(1, 4)
+SNN_FILBK1_KERNEL(2, 2)
+SNN_FILBK1_KERNEL(2, 4)
+#undef SNN_FILBK1_KERNEL
+
+// Sums the partial tiles of the 1x1 kernel and rounds.  Thread o of the
+// filter's float4s, in accumulator order within a tile.
+__global__ void __launch_bounds__(256)
+    filter_backprop_1x1_f16_reduce_kernel(const float4v* __restrict__ part,
+                                          _Float16* __restrict__ dw,
+                                          int n_tiles, int c_tiles,
+                                          int n_splits, int n_groups, int a,
+                                          int b, int features) {
+  __shared__ float4v sums[256];
+  const int tile_vecs = 1024 * a * b;
+  const int width = 256 / n_groups;
+  const int lane_o = threadIdx.x % width;
+  const int group = threadIdx.x / width;
+  const unsigned o = blockIdx.x * width + lane_o;
+  const unsigned tile = o / tile_vecs;
+  const unsigned local = o - tile * tile_vecs;
+  float4v sum = {0.f, 0.f, 0.f, 0.f};
+  for (int sp = group; sp < n_splits; sp += n_groups)
+    sum += part[(static_cast<size_t>(sp) * n_tiles + tile) * tile_vecs + local];
+  sums[threadIdx.x] = sum;
+  __syncthreads();
+  if (group != 0) return;
+  for (int i = 1; i < n_groups; ++i) sum += sums[i * width + lane_o];
+  const unsigned ln = local & 63, i4 = (local >> 6) & 3;
+  unsigned idx = local >> 8;
+  const unsigned ib = idx % b; idx /= b;
+  const unsigned ia = idx % a; idx /= a;
+  const unsigned wc = idx & 1, wk = idx >> 1;
+  const unsigned ct = tile % c_tiles, kt = tile / c_tiles;
+  const unsigned c = ct * 64 * a + (wc * a + ia) * 32 + (ln & 31);
+  const unsigned k = kt * 64 * b + (wk * b + ib) * 32 + 8 * i4 + 4 * (ln >> 5);
+  typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+  half4v r;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) r[v] = static_cast<_Float16>(sum[v]);
+  *reinterpret_cast<half4v*>(dw + static_cast<size_t>(c) * features + k) = r;
+}
+
+struct Fb1Plan {
+  int a = 0, b = 0;
+  Fb1Geom g;
+};
+
+// The tile shape whose loads plus partial tiles (written and read back) come
+// to the fewest bytes.
+bool make_plan_1x1(const snn_hip_conv2d_params& p, Fb1Plan* plan) {
+  if (p.window_rows != 1 || p.window_cols != 1 || p.stride_rows != 1 ||
+      p.stride_cols != 1 || p.pad_rows != 0 || p.pad_cols != 0 ||
+      p.out_rows != p.in_rows || p.out_cols != p.in_cols)
+    return false;
+  if (p.channels % 64 != 0 || p.features % 64 != 0 || p.batch < 1) return false;
+  const size_t pixels = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols;
+  if (pixels * p.channels * 2 > kMaxBufferBytes ||
+      pixels * p.features * 2 > kMaxBufferBytes)
+    return false;
+  static const int shapes[5][2] = {{1, 1}, {1, 2}, {1, 4}, {2, 2}, {2, 4}};
+  double best = -1;
+  for (const auto& sh : shapes) {
+    const int a = sh[0], b = sh[1];
+    if (p.channels % (64 * a) != 0 || p.features % (64 * b) != 0) continue;
+    Fb1Geom g;
+    g.pixels = static_cast<int>(pixels);
+    g.channels = p.channels; g.features = p.features;
+    g.c_tiles = p.channels / (64 * a);
+    g.k_tiles = p.features / (64 * b);
+    g.n_stages = ceil_div(g.pixels, kStagePx);
+    const int n_tiles = g.c_tiles * g.k_tiles;
+    const int want = max(1, min(g.n_stages, kNumCus / n_tiles));
+    g.per_split = ceil_div(g.n_stages, want);
+    g.n_splits = ceil_div(g.n_stages, g.per_split);
+    const double loads = 2.0 * pixels *
+                         (static_cast<double>(p.channels) * g.k_tiles +
+                          static_cast<double>(p.features) * g.c_tiles);
+    const double partials =
+        2.0 * 4.0 * 4096.0 * a * b * n_tiles * g.n_splits;
+    const double cost = loads + partials;
+    if (best < 0 || cost < best) {
+      best = cost;
+      plan->a = a; plan->b = b; plan->g = g;
+    }
+  }
+  return best >= 0;
+}
+
 }  // namespace
 
 bool conv2d_filter_backprop_3x3_f16_supports(const snn_hip_conv2d_params& p) {
@@ -454,6 +711,52 @@ int launch_conv2d_filter_backprop_3x3_f16(const _Float16* x,
                      dim3(vecs / (256 / n_groups)), dim3(256), 0, stream,
                      reinterpret_cast<const float4v*>(part), dw, n_tiles,
                      g.c_tiles, g.n_splits, n_groups, p.channels, p.features);
+  return SNN_HIP_OK;
+}
+
+bool conv2d_filter_backprop_1x1_f16_supports(const snn_hip_conv2d_params& p) {
+  Fb1Plan plan;
+  return make_plan_1x1(p, &plan);
+}
+
+size_t conv2d_filter_backprop_1x1_f16_partial_floats(
+    const snn_hip_conv2d_params& p) {
+  Fb1Plan plan;
+  if (!make_plan_1x1(p, &plan)) return 0;
+  return static_cast<size_t>(plan.g.n_splits) * plan.g.c_tiles *
+         plan.g.k_tiles * 4096 * plan.a * plan.b;
+}
+
+int launch_conv2d_filter_backprop_1x1_f16(const _Float16* x,
+                                          const _Float16* dy, _Float16* dw,
+                                          float* part,
+                                          const snn_hip_conv2d_params& p,
+                                          hipStream_t stream) {
+  Fb1Plan plan;
+  if (!make_plan_1x1(p, &plan)) return SNN_HIP_INVALID_ALGORITHM;
+  const Fb1Geom& g = plan.g;
+  const int n_tiles = g.c_tiles * g.k_tiles;
+  void (*kernel)(const _Float16*, const _Float16*, float*, Fb1Geom) = nullptr;
+  if (plan.a == 1 && plan.b == 1) kernel = filter_backprop_1x1_f16_a1_b1;
+  if (plan.a == 1 && plan.b == 2) kernel = filter_backprop_1x1_f16_a1_b2;
+  if (plan.a == 1 && plan.b == 4) kernel = filter_backprop_1x1_f16_a1_b4;
+  if (plan.a == 2 && plan.b == 2) kernel = filter_backprop_1x1_f16_a2_b2;
+  if (plan.a == 2 && plan.b == 4) kernel = filter_backprop_1x1_f16_a2_b4;
+  if (kernel == nullptr) return SNN_HIP_INVALID_ALGORITHM;
+  {
+    KernelTimer timer(stream);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(n_tiles * g.n_splits)),
+                       dim3(64 * kWaves), 0, stream, x, dy, part, g);
+  }
+  const int tile_vecs = 1024 * plan.a * plan.b;
+  const unsigned vecs = static_cast<unsigned>(n_tiles) * tile_vecs;
+  int n_groups = 1;
+  while (n_groups < kReduceGroups && 2 * n_groups <= g.n_splits) n_groups *= 2;
+  hipLaunchKernelGGL(filter_backprop_1x1_f16_reduce_kernel,
+                     dim3(vecs / (256 / n_groups)), dim3(256), 0, stream,
+                     reinterpret_cast<const float4v*>(part), dw, n_tiles,
+                     g.c_tiles, g.n_splits, n_groups, plan.a, plan.b,
+                     p.features);
   return SNN_HIP_OK;
 }
 

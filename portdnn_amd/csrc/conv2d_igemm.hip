@@ -1893,12 +1893,15 @@ int launch_conv2d_filter_backprop_f16(const _Float16* x, const _Float16* dy,
                           p.channels * p.features;
   const bool ws_aligned =
       workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0;
-  if (conv2d_filter_backprop_3x3_f16_supports(p) &&
+  const bool is_3x3 = conv2d_filter_backprop_3x3_f16_supports(p);
+  if ((is_3x3 || conv2d_filter_backprop_1x1_f16_supports(p)) &&
       (reinterpret_cast<uintptr_t>(dw) & 7u) == 0 &&
       SNN_TUNING_ENV("SNN_HIP_FILBK_F16_OFF") == nullptr) {
     // binary16 matrix instructions; the partial tiles go to the workspace
     // when it holds them, else to a stream-ordered temporary
-    const size_t part_floats = conv2d_filter_backprop_3x3_f16_partial_floats(p);
+    const size_t part_floats =
+        is_3x3 ? conv2d_filter_backprop_3x3_f16_partial_floats(p)
+               : conv2d_filter_backprop_1x1_f16_partial_floats(p);
     float* part = reinterpret_cast<float*>(workspace);
     const bool own = !ws_aligned || workspace_elems < 2 * part_floats;
     if (own) {
@@ -1909,7 +1912,9 @@ int launch_conv2d_filter_backprop_f16(const _Float16* x, const _Float16* dy,
       part = static_cast<float*>(ptr);
     }
     const int status =
-        launch_conv2d_filter_backprop_3x3_f16(x, dy, dw, part, p, stream);
+        is_3x3
+            ? launch_conv2d_filter_backprop_3x3_f16(x, dy, dw, part, p, stream)
+            : launch_conv2d_filter_backprop_1x1_f16(x, dy, dw, part, p, stream);
     const hipError_t err = hipGetLastError();
     if (own) temp_free_async(part, stream);
     if (status != SNN_HIP_OK) return status;

@@ -160,6 +160,15 @@ int launch_conv2d_filter_backprop_3x3_f16(const _Float16* x,
                                           float* part,
                                           const snn_hip_conv2d_params& p,
                                           hipStream_t stream);
+// The same for 1x1 stride-1 unpadded layers (one flat stream of pixels).
+bool conv2d_filter_backprop_1x1_f16_supports(const snn_hip_conv2d_params& p);
+size_t conv2d_filter_backprop_1x1_f16_partial_floats(
+    const snn_hip_conv2d_params& p);
+int launch_conv2d_filter_backprop_1x1_f16(const _Float16* x,
+                                          const _Float16* dy, _Float16* dw,
+                                          float* part,
+                                          const snn_hip_conv2d_params& p,
+                                          hipStream_t stream);
 bool conv2d_filter_backprop_f16_supports(const snn_hip_conv2d_params& p);
 int launch_conv2d_filter_backprop_f16(const _Float16* x, const _Float16* dy,
                                       _Float16* dw,

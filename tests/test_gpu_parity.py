@@ -1099,6 +1099,37 @@ def test_f16_filter_backprop_3x3_transposing_reads(shape):
         assert_close_f16(got, ref, ("f16 filbk 3x3", shape, ws is None))
 
 
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features
+    (3, 7, 9, 64, 64),        # one 64 x 64 tile, 189 pixels (ragged stage)
+    (2, 14, 14, 64, 128),
+    (32, 28, 28, 64, 256),    # 64 x 256 tiles
+    (5, 8, 8, 128, 256),      # 128 x 256 tiles
+    (2, 28, 28, 192, 320),    # channel and feature counts in odd multiples of 64
+    (32, 7, 7, 512, 2048),    # many tiles, few splits
+    (64, 28, 28, 128, 512),   # 256 splits
+])
+def test_f16_filter_backprop_1x1_transposing_reads(shape):
+    """The 1x1 half-precision filter gradient on the binary16 matrix cores
+    against the oracle in double precision on the same half-rounded
+    operands."""
+    batch, rows, cols, ch, feats = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, 1, 1, False)
+    rng = np.random.default_rng(796 + rows + feats + batch)
+    n_x, n_dy, n_dw = ops.conv_sizes(p, DIRECTION.FILTER_BACKPROP)
+    x = uniform(rng, n_x).astype(np.float16)
+    dy = uniform(rng, n_dy).astype(np.float16)
+    ref = oracle.conv2d_filter_backprop(x.astype(np.float32),
+                                        dy.astype(np.float32),
+                                        oracle_params(p, feats), acc64=True)
+    dx_, ddy = dev(x, torch.float16), dev(dy, torch.float16)
+    for ws in (None, torch.empty(2 * 256 * 4096 * 8, dtype=torch.float16,
+                                 device="cuda")):
+        got = ops.conv2d(dx_, ddy, p, DIRECTION.FILTER_BACKPROP, ALGO.MATMUL,
+                         workspace=ws).float().cpu().numpy()
+        assert_close_f16(got, ref, ("f16 filbk 1x1", shape, ws is None))
+
+
 def test_f16_conv_filter_backprop():
     p = ops.conv_params(3, 10, 9, 16, 24, 3, 1, True)
     rng = np.random.default_rng(781)
