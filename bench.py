@@ -431,6 +431,31 @@ def main():
                     entry["frac_hbm_peak"] = frac(nbytes / ms / 1e6,
                                                   PEAK_HBM_GBS)
                 h.append(entry)
+                if window == 1:
+                    # gradients of the 1x1 layers (same byte accounting)
+                    o.copy_(uniform(n_o).half())
+                    dx = torch.empty(n_a, device="cuda", dtype=torch.float16)
+                    dw = torch.empty(n_b, device="cuda", dtype=torch.float16)
+                    ws2 = torch.empty(2 * 256 * 128 * 256, device="cuda",
+                                      dtype=torch.float16)
+                    for direction, tag, bufs in (
+                            (DIRECTION.INPUT_BACKPROP, "input_backprop",
+                             (o, b, dx)),
+                            (DIRECTION.FILTER_BACKPROP, "filter_backprop",
+                             (a, o, dw))):
+                        ms = event_time_ms(lambda: ops.conv2d(
+                            bufs[0], bufs[1], p, direction, ALGO.MATMUL,
+                            workspace=ws2, out=bufs[2]), reps=20, warm=3,
+                            repeats=3)
+                        h.append({"op": "conv1x1_%dx%dx%d_k%d_b128_f16_%s" % (
+                            size, size, ch, feats, tag), "ms": round(ms, 4),
+                            "tflops": round(fl / ms / 1e9, 1),
+                            "frac_f16_mfma_peak": frac(fl / ms / 1e9, 2500.0),
+                            "bytes": nbytes,
+                            "gbs": round(nbytes / ms / 1e6, 1),
+                            "frac_hbm_peak": frac(nbytes / ms / 1e6,
+                                                  PEAK_HBM_GBS)})
+                    del dx, dw, ws2
                 if window == 3:
                     # input gradient: the same kernel on dY (o) with the
                     # filter's taps mirrored and its roles swapped
