@@ -1764,6 +1764,10 @@ static int launch_filter_backprop(const float* x, const float* dy, float* dw,
   const size_t dy_elems = static_cast<size_t>(g.m_total) * p.features;
   const size_t dw_elems = static_cast<size_t>(p.window_rows) * p.window_cols *
                           p.channels * p.features;
+  if (conv2d_stem_filter_backprop_supports(p) &&
+      (reinterpret_cast<uintptr_t>(dw) & 15u) == 0 &&
+      SNN_TUNING_ENV("SNN_HIP_STEM_OFF") == nullptr)
+    return launch_conv2d_stem_filter_backprop_f32(x, dy, dw, p, stream);
   if (p.channels % 64 != 0) {
     // few (tap, channel) pairs: one work-group column per 64 features, the
     // pixel range split over about two work-groups per CU

@@ -24,6 +24,8 @@
 //
 // Reduction order inside an output: k = 4 t + q for instruction t and lane
 // quarter q, summed by the matrix unit over q and accumulated over t in order.
+#include <algorithm>
+
 #include "snn_kernels.h"
 
 namespace snn {
@@ -334,6 +336,204 @@ bool make_geom(const snn_hip_conv2d_params& p, StemGeom* g) {
   return best_cost >= 0;
 }
 
+// ---------------------------------------------------------------------------
+// Filter gradient of the same layer:
+//   dW[rho][k] = sum over (n, oy, ox) of X[n][2 oy + r - pad][2 ox + s - pad][c] * dY[n][oy][ox][k],
+// rho = 21 r + 3 s + c (147 values, ten row blocks of 16, the last 13 rows
+// unused).  The work-group and its band of input rows in LDS are the forward
+// kernel's.  Matrix instruction: D[rho][k] (16 x 16) += A[rho][4 pixels] *
+// B[4 pixels][k]; the A operand of lane l is one LDS float at
+// (row 2 (oy - oy0) + rho / 21, column 6 ox + rho % 21), i.e. a per-lane
+// constant plus 24 floats per step of four pixels -- an immediate offset; the
+// B operand is one float of dY, loaded from global memory a whole output row
+// ahead (56 registers).  Wave w: row blocks 5 (w & 1) ... + 4, feature blocks
+// 2 ((w >> 1) & 1) ... + 1, output rows of the band of parity w >> 2: 7 loads
+// per 10 matrix instructions.  The two parities meet through LDS, the
+// work-groups through partial filters that a second kernel sums.
+constexpr int kRhoBlocks = 5;   // per wave (ten in all)
+constexpr int kMaxTSteps = 28;  // four-pixel steps of an output row
+constexpr int kPartFloats = kK * kFeatures;
+
+__global__ void __launch_bounds__(64 * kWaves)
+    __attribute__((amdgpu_waves_per_eu(2, 2)))
+    conv_stem_filter_backprop_kernel(const float* __restrict__ x,
+                                     const float* __restrict__ dy,
+                                     float* __restrict__ part, StemGeom g) {
+  extern __shared__ __align__(16) float lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int q = lane >> 4;
+  const int l16 = lane & 15;
+  const int rh = wave & 1, kp = (wave >> 1) & 1, ph = wave >> 2;
+  const int n = blockIdx.x / g.n_bands;
+  const int band = blockIdx.x % g.n_bands;
+  const int oy0 = band * g.band;
+  const int oy_end = min(oy0 + g.band, g.out_rows);
+  const int y_first = kStride * oy0 - g.pad_rows;
+
+  const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(
+      x, static_cast<size_t>(g.batch) * g.in_rows * g.in_cols * kCh * 4);
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(
+      dy, static_cast<size_t>(g.batch) * g.out_rows * g.out_cols * kFeatures * 4);
+
+  // every input row of the band (rows and columns outside the image: zeros)
+  const int row_bytes_in = g.in_cols * kCh * 4;
+  for (int row = 0; row < g.lds_rows; ++row)
+    for (int i = wave; i < g.loads_per_row; i += kWaves) {
+      const int yy = y_first + row;
+      const int f = i * 64 + lane - kCh * g.pad_cols;
+      const bool ok =
+          static_cast<unsigned>(yy) < static_cast<unsigned>(g.in_rows) &&
+          static_cast<unsigned>(f) < static_cast<unsigned>(g.in_cols * kCh);
+      const unsigned off =
+          ok ? static_cast<unsigned>((n * g.in_rows + yy)) *
+                       static_cast<unsigned>(row_bytes_in) +
+                   static_cast<unsigned>(f) * 4u
+             : kOobOffset;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          x_rsrc, (lds_ptr)(lds + row * kRowFloats + i * 64), 4, off, 0, 0, 0);
+    }
+
+  // A operand: where this lane's rho sits relative to (first LDS row of the
+  // output row, pixel 4 t)
+  int a_off[kRhoBlocks];
+#pragma unroll
+  for (int b = 0; b < kRhoBlocks; ++b) {
+    const int rho = 16 * (kRhoBlocks * rh + b) + l16;
+    a_off[b] = (rho / kRowK) * kRowFloats + 6 * q + rho % kRowK;
+  }
+  const int n_tsteps = (g.out_cols + 3) >> 2;
+  const int n_iter = (g.band + 1) >> 1;  // output rows per parity
+
+  float4v acc[kRhoBlocks][2];
+#pragma unroll
+  for (int b = 0; b < kRhoBlocks; ++b)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[b][j] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  // dY of one output row for this lane: pixel 4 t + q, features
+  // 16 (2 kp + j) + l16; zeros past the row's end and past the band's.  One
+  // per-lane offset per row, the step and the feature block in the scalar
+  // offset, so that a row's 56 loads cost no vector arithmetic; only the last
+  // step of a row can run past its end and has an offset of its own.
+  auto issue_dy = [&](int oy, float (&bv)[kMaxTSteps][2]) {
+    const bool row_ok = oy < oy_end;
+    const unsigned lane_off =
+        (static_cast<unsigned>((n * g.out_rows + oy) * g.out_cols + q) *
+             kFeatures + 32 * kp + l16) * 4u;
+    const unsigned v_main = row_ok ? lane_off : kOobOffset;
+    const unsigned v_last =
+        row_ok && 4 * (n_tsteps - 1) + q < g.out_cols ? lane_off : kOobOffset;
+#pragma unroll
+    for (int t = 0; t < kMaxTSteps; ++t) {
+      if (t < n_tsteps) {
+        const unsigned v = t == n_tsteps - 1 ? v_last : v_main;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          bv[t][j] = __builtin_bit_cast(
+              float, __builtin_amdgcn_raw_buffer_load_b32(
+                         dy_rsrc, v, (4 * t * kFeatures + 16 * j) * 4, 0));
+      }
+    }
+  };
+  // The A operands of a step are fetched during the step before it (fenced:
+  // left alone, the compiler reads one operand, waits for it and issues two
+  // matrix instructions, and the LDS latency shows every time).
+  auto multiply_row = [&](int oy, const float (&bv)[kMaxTSteps][2]) {
+    const float* base = lds + kStride * (oy - oy0) * kRowFloats;
+    float a[2][kRhoBlocks];
+#pragma unroll
+    for (int b = 0; b < kRhoBlocks; ++b) a[0][b] = base[a_off[b]];
+#pragma unroll
+    for (int t = 0; t < kMaxTSteps; ++t) {
+      if (t < n_tsteps) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < kMaxTSteps) {
+#pragma unroll
+          for (int b = 0; b < kRhoBlocks; ++b)
+            a[(t + 1) & 1][b] = base[a_off[b] + 24 * (t + 1)];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int b = 0; b < kRhoBlocks; ++b)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[b][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                a[t & 1][b], bv[t][j], acc[b][j], 0, 0, 0);
+      }
+    }
+  };
+
+  float bv0[kMaxTSteps][2], bv1[kMaxTSteps][2];
+  issue_dy(oy0 + ph, bv0);
+  __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+  __syncthreads();  // the band's rows are in LDS
+#define SNN_STEM_FILBK_STEP(cur, nxt)                                  \
+  {                                                                    \
+    if (i >= n_iter) break;                                            \
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));                          \
+    if (i + 1 < n_iter) issue_dy(oy0 + ph + 2 * (i + 1), nxt);         \
+    multiply_row(oy0 + ph + 2 * i, cur);                               \
+    ++i;                                                               \
+  }
+  int i = 0;
+  for (;;) {
+    SNN_STEM_FILBK_STEP(bv0, bv1)
+    SNN_STEM_FILBK_STEP(bv1, bv0)
+  }
+#undef SNN_STEM_FILBK_STEP
+
+  // the two row parities meet in LDS (the input rows are no longer needed)
+  __syncthreads();
+  constexpr int kWaveAcc = kRhoBlocks * 2 * 4 * 64;
+  if (ph == 1) {
+    float* dst = lds + (wave - 4) * kWaveAcc;
+#pragma unroll
+    for (int b = 0; b < kRhoBlocks; ++b)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          dst[((b * 2 + j) * 4 + v) * 64 + lane] = acc[b][j][v];
+  }
+  __syncthreads();
+  if (ph == 1) return;
+  const float* src = lds + wave * kWaveAcc;
+  float* out = part + static_cast<size_t>(blockIdx.x) * kPartFloats;
+#pragma unroll
+  for (int b = 0; b < kRhoBlocks; ++b)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        // accumulator element v of lane l: row 4 (l / 16) + v, column l % 16
+        const int rho = 16 * (kRhoBlocks * rh + b) + 4 * q + v;
+        const int k = 16 * (2 * kp + j) + l16;
+        if (rho < kK)
+          out[rho * kFeatures + k] =
+              acc[b][j][v] + src[((b * 2 + j) * 4 + v) * 64 + lane];
+      }
+}
+
+// dW = sum of the work-groups' partial filters: 16 consecutive float4 x 16
+// groups of partials per work-group.
+__global__ void __launch_bounds__(256)
+    stem_filter_backprop_reduce_kernel(const float4v* __restrict__ part,
+                                       float4v* __restrict__ dw, int n_parts) {
+  __shared__ float4v sums[16][16];
+  const int o16 = threadIdx.x & 15, group = threadIdx.x >> 4;
+  const int o = blockIdx.x * 16 + o16;
+  float4v sum = {0.f, 0.f, 0.f, 0.f};
+  for (int sp = group; sp < n_parts; sp += 16)
+    sum += part[static_cast<size_t>(sp) * (kPartFloats / 4) + o];
+  sums[group][o16] = sum;
+  __syncthreads();
+  if (group != 0) return;
+#pragma unroll
+  for (int i = 1; i < 16; ++i) sum += sums[i][o16];
+  dw[o] = sum;
+}
+
 }  // namespace
 
 bool conv2d_stem_supports(const snn_hip_conv2d_params& p) {
@@ -358,6 +558,52 @@ int launch_conv2d_stem_f32(const float* x, const float* w, float* y,
   hipLaunchKernelGGL(conv_stem_7x7s2_kernel,
                      dim3(static_cast<unsigned>(p.batch * g.n_bands)),
                      dim3(64 * kWaves), lds_bytes, stream, x, w, y, g);
+  return SNN_HIP_OK;
+}
+
+bool conv2d_stem_filter_backprop_supports(const snn_hip_conv2d_params& p) {
+  StemGeom g;
+  return make_geom(p, &g) && p.out_cols <= 4 * kMaxTSteps;
+}
+
+// dw 16-byte aligned.  The partial filters (one of 147 x 64 floats per
+// work-group) live in a stream-ordered temporary.
+int launch_conv2d_stem_filter_backprop_f32(const float* x, const float* dy,
+                                           float* dw,
+                                           const snn_hip_conv2d_params& p,
+                                           hipStream_t stream) {
+  StemGeom g;
+  if (!make_geom(p, &g) || p.out_cols > 4 * kMaxTSteps)
+    return SNN_HIP_INVALID_ALGORITHM;
+  const unsigned n_groups = static_cast<unsigned>(p.batch * g.n_bands);
+  void* ptr = nullptr;
+  if (temp_malloc_async(&ptr, static_cast<size_t>(n_groups) * kPartFloats *
+                                  sizeof(float),
+                        stream) != hipSuccess)
+    return SNN_HIP_ALLOCATION_PROBLEM;
+  float* part = static_cast<float*>(ptr);
+  // the band's rows, and at the end the accumulators of four waves
+  const size_t lds_bytes = std::max(
+      (static_cast<size_t>(g.lds_rows + 1) * g.row_floats + 64) * sizeof(float),
+      static_cast<size_t>(4 * kRhoBlocks * 2 * 4 * 64) * sizeof(float));
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(conv_stem_filter_backprop_kernel),
+      hipFuncAttributeMaxDynamicSharedMemorySize,
+      static_cast<int>(kMaxLdsBytes));
+  (void)attr;
+  {
+    KernelTimer timer(stream);
+    hipLaunchKernelGGL(conv_stem_filter_backprop_kernel, dim3(n_groups),
+                       dim3(64 * kWaves), lds_bytes, stream, x, dy, part, g);
+  }
+  static_assert(kPartFloats % 64 == 0, "whole groups of 16 float4");
+  hipLaunchKernelGGL(stem_filter_backprop_reduce_kernel,
+                     dim3(kPartFloats / 64), dim3(256), 0, stream,
+                     reinterpret_cast<const float4v*>(part),
+                     reinterpret_cast<float4v*>(dw), static_cast<int>(n_groups));
+  const hipError_t err = hipGetLastError();
+  temp_free_async(part, stream);
+  if (err != hipSuccess) return report_hip_error(err, "stem filter backprop");
   return SNN_HIP_OK;
 }
 

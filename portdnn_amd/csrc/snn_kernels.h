@@ -113,6 +113,13 @@ void launch_gemm_wreg(const float* x, const float* w, float* y, int m, int k,
 bool conv2d_stem_supports(const snn_hip_conv2d_params& p);
 int launch_conv2d_stem_f32(const float* x, const float* w, float* y,
                            const snn_hip_conv2d_params& p, hipStream_t stream);
+// ... and its filter gradient (dw 16-byte aligned; partial filters in a
+// stream-ordered temporary).
+bool conv2d_stem_filter_backprop_supports(const snn_hip_conv2d_params& p);
+int launch_conv2d_stem_filter_backprop_f32(const float* x, const float* dy,
+                                           float* dw,
+                                           const snn_hip_conv2d_params& p,
+                                           hipStream_t stream);
 
 // The same in half precision with fp32 accumulation (gemm_wreg_f16.hip):
 // k = 64, 128, 256 or 512.

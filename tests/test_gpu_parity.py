@@ -127,12 +127,15 @@ def test_stem_7x7_stride2(direction):
     (9, 224, 224, True),    # the stem layer itself, bands of two steps
 ])
 def test_stem_rows_in_lds_kernel(batch, rows, cols, same):
-    """The 7x7 stride-2, 3 -> 64 channel forward kernel that keeps a band of
-    input rows in LDS (used from 224 output rows over the batch upwards)."""
+    """The 7x7 stride-2, 3 -> 64 channel forward and filter-gradient kernels
+    that keep a band of input rows in LDS (used from 224 output rows over the
+    batch upwards)."""
     p = ops.conv_params(batch, rows, cols, 3, 64, 7, 2, same)
     assert batch * p.out_rows >= 224
     conv_case(p, DIRECTION.FORWARD, [ALGO.IM2COL, ALGO.TILED],
               seed=350 + batch + rows)
+    conv_case(p, DIRECTION.FILTER_BACKPROP, [ALGO.IM2COL],
+              seed=360 + batch + rows)
 
 
 def test_config0_single_image_tiled():
