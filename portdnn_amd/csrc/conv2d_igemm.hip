@@ -2105,6 +2105,14 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
                             hipStream_t stream, float* workspace,
                             size_t workspace_elems,
                             const LaunchOptions* epilogue) {
+  if (direction == SNN_HIP_INPUT_BACKPROP &&
+      conv2d_stem_input_backprop_supports(p) &&
+      (reinterpret_cast<uintptr_t>(output) & 15u) == 0 &&
+      SNN_TUNING_ENV("SNN_HIP_STEM_OFF") == nullptr) {
+    // three channels, 7x7 stride 2, 64 features: the kernel built for it
+    return launch_conv2d_stem_input_backprop_f32(input, filter, output, p,
+                                                 stream);
+  }
   if (direction == SNN_HIP_INPUT_BACKPROP && p.channels < 16 &&
       p.features % kBK == 0 &&
       static_cast<size_t>(p.out_rows) * p.out_cols * p.window_rows *

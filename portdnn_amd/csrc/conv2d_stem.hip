@@ -534,6 +534,200 @@ __global__ void __launch_bounds__(256)
   dw[o] = sum;
 }
 
+// ---------------------------------------------------------------------------
+// Input gradient of the same layer:
+//   dX[n][2 oy + r - pad][2 ox + s - pad][c] += sum over k of dY[n][oy][ox][k] * W[r][s][c][k].
+// Per block of 16 output pixels, Z[rho][pixel] = W[rho][.] * dY[pixel][.] (ten
+// row blocks of 16 x 16 reduction steps of 4) is computed on the matrix cores
+// and added straight into the band's input rows in LDS (the layout is the
+// forward kernel's), so the [pixels][147] intermediate never
+// reaches memory.  The filter is the B operand and stays in registers (wave
+// w: row blocks 5 (w & 1) ..., 80 registers); reduction index 16 q + t sits
+// in lane group q at step t, which makes both operands runs of 16 consecutive
+// floats per lane.  At the end the band's rows are written out: rows no other band touches with
+// plain stores, the five rows shared with each neighbouring band with float
+// atomics into the zero-filled output (two addends, so the result does not
+// depend on their order).
+
+__global__ void __launch_bounds__(64 * kWaves)
+    __attribute__((amdgpu_waves_per_eu(2, 2)))
+    conv_stem_input_backprop_kernel(const float* __restrict__ dy,
+                                    const float* __restrict__ w,
+                                    float* __restrict__ dx, StemGeom g) {
+  extern __shared__ __align__(16) float lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int q = lane >> 4;
+  const int l16 = lane & 15;
+  const int rh = wave & 1;
+  const int n = blockIdx.x / g.n_bands;
+  const int band = blockIdx.x % g.n_bands;
+  const int oy0 = band * g.band;
+  const int n_rows = min(g.band, g.out_rows - oy0);
+  const int y_first = kStride * oy0 - g.pad_rows;
+
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(
+      dy, static_cast<size_t>(g.batch) * g.out_rows * g.out_cols * kFeatures * 4);
+  const __amdgpu_buffer_rsrc_t dx_rsrc = make_rsrc(
+      dx, static_cast<size_t>(g.batch) * g.in_rows * g.in_cols * kCh * 4);
+
+  for (int i = threadIdx.x; i < g.lds_rows * kRowFloats; i += 64 * kWaves)
+    lds[i] = 0.f;
+
+  // filter rows 16 (5 rh + b) + l16, reduction indices 16 q + t
+  float wreg[kRhoBlocks][16];
+#pragma unroll
+  for (int b = 0; b < kRhoBlocks; ++b) {
+    const int rho = 16 * (kRhoBlocks * rh + b) + l16;
+#pragma unroll
+    for (int t4 = 0; t4 < 4; ++t4) {
+      float4v v = {0.f, 0.f, 0.f, 0.f};
+      if (rho < kK)
+        v = *reinterpret_cast<const float4v*>(w + rho * kFeatures + 16 * q +
+                                              4 * t4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) wreg[b][4 * t4 + e] = v[e];
+    }
+  }
+  // Pixels are the rows of the product and rho its columns: accumulator
+  // element v of row block b belongs to pixel 4 q + v and this lane's rho, and
+  // lands at row rho / 21, float rho % 21 + 6 (4 q + v) relative to (first LDS
+  // row of the output row, pixel block).  The 64 lanes of one LDS add then hit
+  // 64 different floats (with rho down the rows, lanes two pixels and three
+  // lane groups apart met in the same float and an add took ~100 cycles).
+  int z_off[kRhoBlocks];
+#pragma unroll
+  for (int b = 0; b < kRhoBlocks; ++b) {
+    const int rho = 16 * (kRhoBlocks * rh + b) + l16;
+    z_off[b] = rho < kK ? (rho / kRowK) * kRowFloats + rho % kRowK + 24 * q : -1;
+  }
+
+  const int n_pb = (g.out_cols + 15) >> 4;
+  // dY of a block for this lane: pixel 16 pb + l16, features 16 q ... + 15
+  auto issue_dy = [&](int row, int pb, bool live, float4v (&bv)[4]) {
+    const int ox = 16 * pb + l16;
+    const bool ok = live && row < n_rows && ox < g.out_cols;
+    const unsigned off =
+        (static_cast<unsigned>((n * g.out_rows + oy0 + row) * g.out_cols + ox) *
+             kFeatures + 16 * q) * 4u;
+#pragma unroll
+    for (int t4 = 0; t4 < 4; ++t4)
+      bv[t4] = __builtin_bit_cast(
+          float4v, __builtin_amdgcn_raw_buffer_load_b128(
+                       dy_rsrc, ok ? off : kOobOffset, 16 * t4, 0));
+  };
+  // Z of one block, added into the band's rows.  Plain read-add-write: the 64
+  // lanes of an instruction hit 64 different floats, and the schedule below
+  // keeps the waves' blocks apart.  (LDS float atomics measured ~180 cycles
+  // per instruction, four times the rest of the kernel.)
+  auto multiply_add = [&](int row, int pb, const float4v (&bv)[4]) {
+    float4v acc[kRhoBlocks];
+#pragma unroll
+    for (int b = 0; b < kRhoBlocks; ++b) acc[b] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < 16; ++t)
+#pragma unroll
+      for (int b = 0; b < kRhoBlocks; ++b)
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(bv[t >> 2][t & 3], wreg[b][t],
+                                                      acc[b], 0, 0, 0);
+    // A float one lane updates for pixel 4 q + v is another lane's for pixel
+    // 4 q + v + 1 (two taps to the left), so the four v must stay in program
+    // order: volatile, and the LDS serves a wave's accesses in order.  The
+    // five row blocks of one v never meet (their rho differ by less than the
+    // 24 floats between lane groups, or sit in different LDS rows) and go as
+    // one batch of reads and one of writes.
+    volatile float* base = lds + kStride * row * kRowFloats + 96 * pb;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      float old[kRhoBlocks];
+#pragma unroll
+      for (int b = 0; b < kRhoBlocks; ++b)
+        old[b] = base[(z_off[b] >= 0 ? z_off[b] : 0) + 6 * v];
+#pragma unroll
+      for (int b = 0; b < kRhoBlocks; ++b)
+        if (z_off[b] >= 0) base[z_off[b] + 6 * v] = old[b] + acc[b][v];
+    }
+  };
+
+  // A block (output row, pixel block) touches LDS rows 2 row ... 2 row + 6 and
+  // floats 96 pb ... 96 pb + 110: blocks four rows or two pixel blocks apart
+  // are disjoint.  A step gives the eight waves eight such slots -- rows
+  // i + 4 m (m = 0 ... 3) x pixel blocks {2 cs, 2 cs + 1} or {4 + 2 cs,
+  // 5 + 2 cs} -- and a barrier ends it; every slot is visited twice, once by a
+  // wave of each half of the rho range.
+  const int wj = wave >> 1;
+  const int n_steps = 16 * ((n_rows + 15) >> 4);
+  auto decode = [&](int st, int& row, int& pb0) {
+    const int sub = st & 1, cs = (st >> 1) & 1, i = (st >> 2) & 3, rg = st >> 4;
+    const int slot = 2 * wj + (rh ^ sub);
+    row = 16 * rg + i + 4 * (slot >> 1);
+    pb0 = 4 * (slot & 1) + 2 * cs;
+  };
+  auto issue_item = [&](int st, float4v (&bv)[2][4]) {
+    int row, pb0;
+    decode(st, row, pb0);
+#pragma unroll
+    for (int d = 0; d < 2; ++d)
+      issue_dy(row, pb0 + d, st < n_steps && pb0 + d < n_pb, bv[d]);
+  };
+  auto do_item = [&](int st, const float4v (&bv)[2][4]) {
+    int row, pb0;
+    decode(st, row, pb0);
+#pragma unroll
+    for (int d = 0; d < 2; ++d)
+      if (row < n_rows && pb0 + d < n_pb) multiply_add(row, pb0 + d, bv[d]);
+  };
+
+  float4v bv0[2][4], bv1[2][4];
+  issue_item(0, bv0);
+  __syncthreads();  // the band's rows are zero
+#define SNN_STEM_INBK_STEP(cur, nxt)                    \
+  {                                                     \
+    if (st >= n_steps) break;                           \
+    issue_item(st + 1, nxt);                            \
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(8));           \
+    do_item(st, cur);                                   \
+    __syncthreads();                                    \
+    ++st;                                               \
+  }
+  int st = 0;
+  for (;;) {
+    SNN_STEM_INBK_STEP(bv0, bv1)
+    SNN_STEM_INBK_STEP(bv1, bv0)
+  }
+#undef SNN_STEM_INBK_STEP
+  __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+  __syncthreads();
+
+  // ---- write the band's rows ------------------------------------------------
+  const int row_floats_in = g.in_cols * kCh;
+  const int first_col = kCh * g.pad_cols;
+  for (int row = wave; row < g.lds_rows; row += kWaves) {
+    const int yy = y_first + row;
+    if (yy < 0 || yy >= g.in_rows) continue;
+    const bool shared = (band > 0 && row < kWin - kStride) ||
+                        (band + 1 < g.n_bands && row >= kStride * g.band);
+    const unsigned row_off =
+        static_cast<unsigned>(n * g.in_rows + yy) *
+        static_cast<unsigned>(row_floats_in) * 4u;
+    for (int f = lane; f < row_floats_in; f += 64) {
+      const float v = lds[row * kRowFloats + first_col + f];
+      const unsigned off = row_off + static_cast<unsigned>(f) * 4u;
+      if (shared)
+        __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(v, dx_rsrc, off, 0, 0);
+      else
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v),
+                                              dx_rsrc, off, 0, 0);
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256)
+    stem_zero_fill_kernel(float4v* __restrict__ dst, size_t n_vec) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i < n_vec) dst[i] = float4v{0.f, 0.f, 0.f, 0.f};
+}
+
 }  // namespace
 
 bool conv2d_stem_supports(const snn_hip_conv2d_params& p) {
@@ -604,6 +798,43 @@ int launch_conv2d_stem_filter_backprop_f32(const float* x, const float* dy,
   const hipError_t err = hipGetLastError();
   temp_free_async(part, stream);
   if (err != hipSuccess) return report_hip_error(err, "stem filter backprop");
+  return SNN_HIP_OK;
+}
+
+// (From 16 images of 112 output rows: below that the general path measured
+// faster, 85 vs 92 us at batch 8.)
+bool conv2d_stem_input_backprop_supports(const snn_hip_conv2d_params& p) {
+  StemGeom g;
+  return make_geom(p, &g) &&
+         static_cast<long>(p.batch) * p.out_rows >= 8 * kMinOutputRows &&
+         (static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * kCh) % 4 == 0;
+}
+
+// dy, filter and dx 16-byte aligned.
+int launch_conv2d_stem_input_backprop_f32(const float* dy, const float* w,
+                                          float* dx,
+                                          const snn_hip_conv2d_params& p,
+                                          hipStream_t stream) {
+  StemGeom g;
+  if (!conv2d_stem_input_backprop_supports(p) || !make_geom(p, &g))
+    return SNN_HIP_INVALID_ALGORITHM;
+  const size_t n_vec =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * kCh / 4;
+  hipLaunchKernelGGL(stem_zero_fill_kernel,
+                     dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
+                     dim3(256), 0, stream, reinterpret_cast<float4v*>(dx),
+                     n_vec);
+  const size_t lds_bytes =
+      (static_cast<size_t>(g.lds_rows + 1) * g.row_floats + 64) * sizeof(float);
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(conv_stem_input_backprop_kernel),
+      hipFuncAttributeMaxDynamicSharedMemorySize,
+      static_cast<int>(kMaxLdsBytes));
+  (void)attr;
+  KernelTimer timer(stream);
+  hipLaunchKernelGGL(conv_stem_input_backprop_kernel,
+                     dim3(static_cast<unsigned>(p.batch * g.n_bands)),
+                     dim3(64 * kWaves), lds_bytes, stream, dy, w, dx, g);
   return SNN_HIP_OK;
 }
 

@@ -115,6 +115,11 @@ int launch_conv2d_stem_f32(const float* x, const float* w, float* y,
                            const snn_hip_conv2d_params& p, hipStream_t stream);
 // ... and its filter gradient (dw 16-byte aligned; partial filters in a
 // stream-ordered temporary).
+bool conv2d_stem_input_backprop_supports(const snn_hip_conv2d_params& p);
+int launch_conv2d_stem_input_backprop_f32(const float* dy, const float* w,
+                                          float* dx,
+                                          const snn_hip_conv2d_params& p,
+                                          hipStream_t stream);
 bool conv2d_stem_filter_backprop_supports(const snn_hip_conv2d_params& p);
 int launch_conv2d_stem_filter_backprop_f32(const float* x, const float* dy,
                                            float* dw,

@@ -138,6 +138,23 @@ def test_stem_rows_in_lds_kernel(batch, rows, cols, same):
               seed=360 + batch + rows)
 
 
+@pytest.mark.parametrize("batch,rows,cols,same", [
+    (60, 64, 64, True),     # bands of three steps, two-row last band
+    (40, 97, 61, True),     # 49 x 31 output: ragged pixel block, odd rows
+    (45, 85, 100, False),   # no padding
+    (17, 223, 221, True),   # odd image, padding 3
+    (16, 224, 224, True),   # the stem layer itself
+])
+def test_stem_input_backprop_rows_in_lds_kernel(batch, rows, cols, same):
+    """The 7x7 stride-2, 3 <- 64 channel input-gradient kernel that adds the
+    products into a band of input rows in LDS (used from 1792 output rows over
+    the batch upwards)."""
+    p = ops.conv_params(batch, rows, cols, 3, 64, 7, 2, same)
+    assert batch * p.out_rows >= 1792
+    conv_case(p, DIRECTION.INPUT_BACKPROP, [ALGO.IM2COL],
+              seed=370 + batch + rows)
+
+
 def test_config0_single_image_tiled():
     """Benchmark configuration 0: N=1, 56x56x64 -> 64, 3x3 s1 SAME, Tiled;
     also checked against the reference-loop-nest restatement in fp32."""

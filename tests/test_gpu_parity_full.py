@@ -126,11 +126,9 @@ def test_full_batch_backprop_3x3(size, ch, direction):
                                        DIRECTION.INPUT_BACKPROP,
                                        DIRECTION.FILTER_BACKPROP])
 def test_full_batch_stem_7x7_stride2(direction):
-    """[32,224,224,3] -> [32,112,112,64]: the rows-in-LDS forward kernel
-    (Im2col) beside the scalar gather forward (Direct), the
-    one-work-group-per-64-features filter gradient, and the input gradient as a
-    GEMM per output pixel + tap gather, whose temporary (112*112*147 floats
-    per image) makes it run in minibatches of 9 images."""
+    """[32,224,224,3] -> [32,112,112,64]: the rows-in-LDS kernels of the three
+    directions (Im2col) beside the scalar gather forward, the direct filter
+    gradient and the direct input gradient (Direct)."""
     p = ops.conv_params(32, 224, 224, 3, 64, 7, 2, True)
     assert (p.out_rows, p.pad_rows) == (112, 2)
     rng = np.random.default_rng(3100 + direction)
@@ -145,12 +143,18 @@ def test_full_batch_stem_7x7_stride2(direction):
         else:
             assert_close(got, ref, ("stem batch 32", algo, direction))
     if direction == DIRECTION.INPUT_BACKPROP:
-        # a caller workspace of 3.5 images: minibatches of 3, ragged last one
+        # The general path (GEMM per output pixel + tap gather, used below 16
+        # images) with a caller workspace of 3.5 images: minibatches of 3,
+        # ragged last one.
+        p8 = ops.conv_params(8, 224, 224, 3, 64, 7, 2, True)
+        n_a8, _, _ = ops.conv_sizes(p8, direction)
+        ref8 = ORACLE_FN[direction](a[:n_a8], b, oracle_params(p8, 64),
+                                    acc64=True)
         z = 112 * 112 * 147
         ws = torch.empty(int(3.5 * z), dtype=torch.float32, device="cuda")
-        got = ops.conv2d(da, db, p, direction, ALGO.IM2COL,
+        got = ops.conv2d(dev(a[:n_a8]), db, p8, direction, ALGO.IM2COL,
                          workspace=ws).cpu().numpy()
-        assert_close(got, ref, "stem input gradient, workspace minibatches")
+        assert_close(got, ref8, "stem input gradient, workspace minibatches")
 
 
 # ---- configuration 4 at its full size ---------------------------------------
