@@ -212,7 +212,9 @@ SNN_HIP_API int snn_hip_conv2d_filter_backprop_f16(
  * points above do not always: where a launch would otherwise fill only part
  * of the GPU they split a reduction across work-groups whose partial sums
  * meet through float atomics -- the implicit-GEMM filter gradient (Im2col /
- * Tiled / Direct-fallback tags) always, forward and input gradients of small
+ * Tiled / Direct-fallback tags) always, except for the 7x7 stride-2
+ * three-channel stem from 224 output rows over the batch upwards, whose
+ * partial filters are summed in a fixed order; forward and input gradients of small
  * problems (fewer than ~640 64x64 output tiles) and the fused Winograd
  * kernel below 128 work units -- and the order of those additions, hence the
  * last bits of the result, can change between runs.  The Winograd filter
