@@ -184,49 +184,76 @@ __global__ void __launch_bounds__(64 * kWaves)
   const unsigned lane_piece = lane & 7; // 16-byte position within the pixel
   const int n_chunks = g.y_px / kChunk;
 
+  // Every band has the same shape, so what a load instruction of this wave
+  // fetches is fixed relative to the band's first output row: its row (for
+  // the test against the image's top and bottom) and its byte offset are
+  // worked out once (a load then costs a handful of vector instructions
+  // instead of thirty, which nothing hides with one wave per SIMD).
+  constexpr int kMaxXLoads = 20, kMaxYLoads = 10;  // per wave: 78 KB buffers
+  const int x_loads = g.x_px / 8, y_loads = g.y_px / 8;
+  int x_row[kMaxXLoads], x_rel[kMaxXLoads], y_row[kMaxYLoads], y_rel[kMaxYLoads];
+#pragma unroll
+  for (int idx = 0; idx < kMaxXLoads; ++idx) {
+    const unsigned p = 8 * (wave + kWaves * idx) + lane_px;
+    const unsigned row = __umulhi(p, g.pitch_magic);
+    const int ix = static_cast<int>(p - row * g.pitch) - 1;
+    const bool ok = row < static_cast<unsigned>(g.band + 2) && ix >= 0 &&
+                    ix < g.cols;
+    // rows outside [-1, band] fail every test against the image
+    x_row[idx] = ok ? static_cast<int>(row) - 1 : -0x40000000;
+    x_rel[idx] = (((static_cast<int>(row) - 1) * g.cols + ix) * g.channels +
+                  ct * kTile) * 2 +
+                 static_cast<int>((lane_piece ^ swz(p)) << 4);
+  }
+#pragma unroll
+  for (int idx = 0; idx < kMaxYLoads; ++idx) {
+    const unsigned p = 8 * (wave + kWaves * idx) + lane_px;
+    const unsigned row = __umulhi(p, g.pitch_magic);
+    const int col = static_cast<int>(p - row * g.pitch);
+    const bool ok = row < static_cast<unsigned>(g.band) && col < g.cols;
+    y_row[idx] = ok ? static_cast<int>(row) : -0x40000000;
+    y_rel[idx] = ((static_cast<int>(row) * g.cols + col) * g.features +
+                  kt * kTile) * 2 +
+                 static_cast<int>((lane_piece ^ swz(p)) << 4);
+  }
+
   auto issue_task = [&](int task, char* buf) {
     for (int i = 0; i < g.group; ++i) {
       const int sb = task * g.group + i;
       const bool live = sb < g.n_subbands;
       const int n = sb / g.bands_per_image;
       const int oy0 = (sb - n * g.bands_per_image) * g.band;
+      // rows of the image, relative to oy0; none when the band is past the end
+      const int lo = live ? -oy0 : 1, hi = live ? g.rows - oy0 : 0;
+      const int x_base = (n * g.rows + oy0) * g.cols * g.channels * 2;
+      const int y_base = (n * g.rows + oy0) * g.cols * g.features * 2;
       char* base = buf + i * sb_px * kPixelBytes;
-      for (int l = wave; l < g.x_px / 8; l += kWaves) {
-        const unsigned p = 8 * l + lane_px;
-        const unsigned row = __umulhi(p, g.pitch_magic);
-        const int col = static_cast<int>(p - row * g.pitch);
-        const int iy = oy0 - 1 + static_cast<int>(row);
-        const int ix = col - 1;
-        const bool ok = live && row < static_cast<unsigned>(g.band + 2) &&
-                        iy >= 0 && iy < g.rows && ix >= 0 && ix < g.cols;
-        const unsigned off =
-            (static_cast<unsigned>((n * g.rows + iy) * g.cols + ix) *
-                 g.channels + ct * kTile) * 2u +
-            ((lane_piece ^ swz(p)) << 4);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            x_rsrc, (lds_ptr)(base + l * 1024), 16, ok ? off : kOobOffset, 0, 0,
-            0);
+#pragma unroll
+      for (int idx = 0; idx < kMaxXLoads; ++idx) {
+        const int l = wave + kWaves * idx;
+        if (l < x_loads) {
+          const bool ok = x_row[idx] >= lo && x_row[idx] < hi;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(
+              x_rsrc, (lds_ptr)(base + l * 1024), 16,
+              ok ? static_cast<unsigned>(x_base + x_rel[idx]) : kOobOffset, 0,
+              0, 0);
+        }
       }
       char* ybase = base + g.x_px * kPixelBytes;
-      for (int l = wave; l < g.y_px / 8; l += kWaves) {
-        const unsigned p = 8 * l + lane_px;
-        const unsigned row = __umulhi(p, g.pitch_magic);
-        const int col = static_cast<int>(p - row * g.pitch);
-        const int oy = oy0 + static_cast<int>(row);
-        const bool ok = live && row < static_cast<unsigned>(g.band) &&
-                        oy < g.rows && col < g.cols;
-        const unsigned off =
-            (static_cast<unsigned>((n * g.rows + oy) * g.cols + col) *
-                 g.features + kt * kTile) * 2u +
-            ((lane_piece ^ swz(p)) << 4);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            dy_rsrc, (lds_ptr)(ybase + l * 1024), 16, ok ? off : kOobOffset, 0,
-            0, 0);
+#pragma unroll
+      for (int idx = 0; idx < kMaxYLoads; ++idx) {
+        const int l = wave + kWaves * idx;
+        if (l < y_loads) {
+          const bool ok = y_row[idx] >= lo && y_row[idx] < hi;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(
+              dy_rsrc, (lds_ptr)(ybase + l * 1024), 16,
+              ok ? static_cast<unsigned>(y_base + y_rel[idx]) : kOobOffset, 0,
+              0, 0);
+        }
       }
     }
   };
 
-  // xw[r][h]: pixels 4 h ... 4 h + 3 of filter row r's 12, two halves a register
   auto fetch = [&](const char* at, half8& ya, uint2v (&xw)[3][3]) {
     ya = read_transposed(at + off_y[0], at + off_y[1]);
 #pragma unroll
