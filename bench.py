@@ -11,16 +11,22 @@ total algorithmic TFLOP/s (2*N*OH*OW*R*S*C*K per layer, whatever the
 algorithm).  The same JSON line carries
 
   roofline      the main kernel of the 3x3 convolutions against the fp32 MFMA
-                peak: algorithmic flops per launch over its average duration,
-                timed with HIP events on the launch stream; `traffic` is read
-                from the committed rocprofv3 summary named in `traffic_source`;
-                `hbm` lists the memory-bound half of the metric (depthwise and
-                pooling kernels against the HBM peak), `config0` the
-                single-image 56x56x64 layer through the Tiled algorithm,
+                peak: `achieved` = algorithmic flops per launch over its
+                average duration, timed with HIP events on the launch stream;
+                `frac_algorithmic` = achieved / peak, `frac` = the part of it
+                the matrix cores really execute (16/36 for Winograd) / peak;
+                `traffic` is read from the committed rocprofv3 summary named
+                in `traffic_source`.  The memory-bound half of the metric is
+                there as plain numbers: `hbm_<layer>_gbs` / `_frac` (of the
+                8 TB/s peak) / `_of_stream` (of what a ReLU stream of the same
+                byte count reaches in the same run: the ceiling a launch of
+                that size has on this GPU) for the depthwise and pooling
+                layers, `config0_*` for the single-image 56x56x64 layer,
   cpu_baseline  the reference's algorithms restated in C (oracle/), timed on
                 the host cores on bounded samples: the tiled convolution on
                 the same eight layers (`value`), the depthwise and pooling
-                loops (`memory_bound`) and the single-image layer (`config0`),
+                loops (`depthwise_gbs`, `maxpool_gbs`, `avgpool_gbs`) and the
+                single-image layer (`config0_tflops`),
   detail        per-layer / per-algorithm TFLOP/s, gradients, half precision.
 
 No executed fraction of a peak may exceed 1: `frac()` raises if one does.
@@ -190,6 +196,7 @@ def main():
     per_layer = []
     k3_flops = k3_kernel_ms = 0.0
     k3_kernels = 0
+    executed_flops_per_step = 0.0
     for w in work:
         def call(w=w):
             ops.conv2d(w["x"], w["w"], w["p"], DIRECTION.FORWARD, w["algo"],
@@ -207,6 +214,8 @@ def main():
                               tf, PEAK_FP32_MFMA_TFLOPS,
                               WINOGRAD_SHARE
                               if algo_names[w["algo"]] == "winograd" else 1.0)})
+        executed_flops_per_step += w["flops"] * (
+            WINOGRAD_SHARE if algo_names[w["algo"]] == "winograd" else 1.0)
         if w["name"].startswith("3x3"):
             k3_flops += w["flops"] * kt.kernels
             k3_kernel_ms += kt.total_ms
@@ -214,29 +223,36 @@ def main():
     achieved = k3_flops / k3_kernel_ms / 1e9
     k3_algos = sorted({algo_names[w["algo"]] for w in work
                        if w["name"].startswith("3x3")})
+    k3_share = WINOGRAD_SHARE if k3_algos == ["winograd"] else 1.0
     roofline = {
         "bound": "mfma",
         "kernel": "main kernel of the 3x3 s1 forward convolution (%s), the four "
                   "ResNet stages, one launch each per step" % "/".join(k3_algos),
+        # algorithmic flops (the direct convolution's count, as the metric is
+        # defined) per launch over the kernel's duration
         "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
         "unit": "TFLOP/s",
-        # algorithmic flops over the peak, as the metric is defined; above 1
-        # when the Winograd kernel outruns what the matrix cores could do on
-        # the direct algorithm (mfma_executed_frac is the pipe's own figure)
-        "frac": frac(achieved, PEAK_FP32_MFMA_TFLOPS,
-                     WINOGRAD_SHARE if k3_algos == ["winograd"] else 1.0),
+        # the matrix pipe's own figure: the multiplications really executed
+        # (16/36 of the algorithmic count for Winograd F(2x2,3x3)) over the peak
+        "frac": frac(achieved * k3_share, PEAK_FP32_MFMA_TFLOPS),
+        # algorithmic flops over the peak; above 1 when the Winograd kernel
+        # outruns what the matrix cores could do on the direct algorithm
+        "frac_algorithmic": frac(achieved, PEAK_FP32_MFMA_TFLOPS, k3_share),
+        "achieved_executed": round(achieved * k3_share, 2),
         "avg_kernel_ms": round(k3_kernel_ms / k3_kernels, 5),
         "algorithmic_gflop_per_launch": round(k3_flops / k3_kernels / 1e9, 4),
-        # Winograd F(2x2,3x3) executes 16/36 of the algorithmic flops on the
-        # matrix cores; this is the MFMA pipe's own utilisation
-        "mfma_executed_tflops": round(
-            achieved * (WINOGRAD_SHARE if k3_algos == ["winograd"] else 1.0), 2),
-        "mfma_executed_frac": frac(
-            achieved * (WINOGRAD_SHARE if k3_algos == ["winograd"] else 1.0),
+        # the whole step (Winograd layers at 16/36 of their flops, the 1x1
+        # GEMM layers at all of them) over the step time
+        "step_executed_tflops": round(
+            executed_flops_per_step / ms_per_step / 1e9, 2),
+        "step_executed_frac": frac(
+            executed_flops_per_step / ms_per_step / 1e9,
             PEAK_FP32_MFMA_TFLOPS),
+        # not measured in this run: FETCH_SIZE / WRITE_SIZE of the same kernel
+        # from the committed rocprofv3 summary
         "traffic": (profiled_traffic_bytes("wino_direct_kernel")
                     if k3_algos == ["winograd"] else None),
-        "traffic_source": TRAFFIC_PROFILE}
+        "traffic_source": "committed profile, not this run: " + TRAFFIC_PROFILE}
 
     # ---- memory-bound half of the metric: depthwise and pooling against HBM ----
     # Buffer sets rotate so that the 256 MB last-level cache cannot hold the
@@ -254,15 +270,47 @@ def main():
                 fn()
         return kt.total_ms / max(1, kt.kernels)
 
-    def mem_entry(name, nbytes, ms, kernel_ms):
+    from portdnn_amd.capi import POINTWISE_OP
+    stream_cache = {}
+
+    def stream_ms(nbytes):
+        """What a launch that moves `nbytes` can reach on this GPU: a ReLU
+        stream (snn_hip_pointwise_forward_f32: every element read once and
+        written once, 16 bytes per lane per access) of the same total byte
+        count, timed the same way as the kernels it is compared with."""
+        n = max(4, int(nbytes // 8) // 4 * 4)
+        if n not in stream_cache:
+            sets = rotate_sets(8 * n)
+            xs = [normal(n) for _ in range(sets)]
+            ys = [torch.empty(n, device="cuda") for _ in range(sets)]
+            state = {"i": 0}
+
+            def run():
+                i = state["i"] % sets
+                state["i"] += 1
+                ops.pointwise_forward(xs[i], POINTWISE_OP.RELU, out=ys[i])
+            stream_cache[n] = (
+                event_time_ms(run, reps=5 * sets, warm=sets, repeats=3),
+                device_ms(run, 5 * sets))
+            del xs, ys
+        return stream_cache[n]
+
+    def mem_entry(name, nbytes, ms, kernel_ms, with_stream=True):
         gbs = nbytes / ms / 1e6
         kgbs = nbytes / kernel_ms / 1e6
-        return {"op": name, "bytes": nbytes, "ms": round(ms, 5),
-                "gbs": round(gbs, 1),
-                "frac_hbm_peak": frac(gbs, PEAK_HBM_GBS),
-                "kernel_ms": round(kernel_ms, 5),
-                "kernel_gbs": round(kgbs, 1),
-                "kernel_frac_hbm_peak": frac(kgbs, PEAK_HBM_GBS)}
+        entry = {"op": name, "bytes": nbytes, "ms": round(ms, 5),
+                 "gbs": round(gbs, 1),
+                 "frac_hbm_peak": frac(gbs, PEAK_HBM_GBS),
+                 "kernel_ms": round(kernel_ms, 5),
+                 "kernel_gbs": round(kgbs, 1),
+                 "kernel_frac_hbm_peak": frac(kgbs, PEAK_HBM_GBS)}
+        if with_stream:
+            s_ms, s_kernel_ms = stream_ms(nbytes)
+            entry["stream_same_bytes_ms"] = round(s_ms, 5)
+            entry["stream_same_bytes_gbs"] = round(nbytes / s_ms / 1e6, 1)
+            entry["of_stream"] = round(s_ms / ms, 4)
+            entry["stream_same_bytes_kernel_ms"] = round(s_kernel_ms, 5)
+        return entry
 
     def depthwise_entry(size, ch, stride):
         p = ops.depthwise_params(BATCH, size, size, ch, 1, 3, stride, True)
@@ -311,13 +359,29 @@ def main():
     # the kernel's own duration, which rocprofv3 reports; the per-launch event
     # pairs behind `kernel_ms` in detail.memory_bound add 2-3 us to kernels
     # this short).
-    roofline["hbm"] = [
-        {"kernel": e["op"], "bytes_per_launch": e["bytes"],
-         "ms_per_launch": e["ms"], "achieved_gbs": e["gbs"],
-         "frac": e["frac_hbm_peak"]}
-        for e in mem if e["op"] in (
-            "depthwise3x3_112x112x64_s2", "depthwise3x3_56x56x128_s1",
-            "maxpool3x3_s2_112x112x64", "avgpool7x7_7x7x2048")]
+    # (plain numbers under flat keys: a reader that keeps only the scalar
+    # members of `roofline` still gets the memory-bound half of the metric)
+    short = {"depthwise3x3_112x112x32_s1": "dw_112x112x32_s1",
+             "depthwise3x3_112x112x64_s2": "dw_112x112x64_s2",
+             "depthwise3x3_56x56x128_s1": "dw_56x56x128_s1",
+             "depthwise3x3_28x28x256_s2": "dw_28x28x256_s2",
+             "depthwise3x3_14x14x512_s1": "dw_14x14x512_s1",
+             "depthwise3x3_7x7x1024_s1": "dw_7x7x1024_s1",
+             "maxpool3x3_s2_112x112x64": "maxpool",
+             "avgpool7x7_7x7x2048": "avgpool"}
+    roofline["hbm_peak_gbs"] = PEAK_HBM_GBS
+    for e in mem:
+        key = "hbm_" + short[e["op"]]
+        roofline[key + "_mb"] = round(e["bytes"] / 1e6, 2)
+        roofline[key + "_us"] = round(e["ms"] * 1e3, 2)
+        roofline[key + "_gbs"] = e["gbs"]
+        roofline[key + "_frac"] = e["frac_hbm_peak"]
+        roofline[key + "_of_stream"] = e["of_stream"]
+    # the ceiling itself: the ReLU stream at round sizes (read + write bytes)
+    for mb in (13, 26, 32, 103, 128, 256, 411):
+        s_ms, _ = stream_ms(mb * 1e6)
+        roofline["hbm_stream_%dmb_gbs" % mb] = round(mb / s_ms, 1)
+        roofline["hbm_stream_%dmb_frac" % mb] = frac(mb / s_ms, PEAK_HBM_GBS)
 
     # ---- configuration 0: one 56x56x64 image, 3x3 s1 SAME, Tiled -------------
     p0 = ops.conv_params(1, 56, 56, 64, 64, 3, 1, True)
@@ -332,12 +396,13 @@ def main():
             call0()
     kms0 = kt.total_ms / max(1, kt.kernels)
     fl0 = ops.conv_flops(p0, DIRECTION.FORWARD)
-    roofline["config0"] = {
-        "workload": "conv2d forward fp32 [1,56,56,64] x [3,3,64,64], s1 SAME, "
-                    "Tiled", "gflop": round(fl0 / 1e9, 4), "ms": round(ms0, 5),
-        "tflops": round(fl0 / ms0 / 1e9, 2), "kernel_ms": round(kms0, 5),
-        "kernel_tflops": round(fl0 / kms0 / 1e9, 2),
-        "kernel_frac_mfma_peak": frac(fl0 / kms0 / 1e9, PEAK_FP32_MFMA_TFLOPS)}
+    roofline["config0_workload"] = ("conv2d forward fp32 [1,56,56,64] x "
+                                    "[3,3,64,64], s1 SAME, Tiled")
+    roofline["config0_gflop"] = round(fl0 / 1e9, 4)
+    roofline["config0_ms"] = round(ms0, 5)
+    roofline["config0_tflops"] = round(fl0 / ms0 / 1e9, 2)
+    roofline["config0_frac"] = frac(fl0 / ms0 / 1e9, PEAK_FP32_MFMA_TFLOPS)
+    roofline["config0_kernel_ms"] = round(kms0, 5)
 
     detail = {"layers": per_layer, "memory_bound": mem}
     if not args.no_detail:
@@ -606,7 +671,7 @@ def main():
                 grads.append(mem_entry(
                     "depthwise3x3_%dx%dx%d_s%d_%s" % (size, size, ch, stride,
                                                       tag),
-                    nbytes, ms, device_ms(run, 5 * sets)))
+                    nbytes, ms, device_ms(run, 5 * sets), with_stream=False))
                 del a_s, b_s, o_s
         p = ops.pool_params(BATCH, 112, 112, 64, 3, 2, True)
         n_in = p.batch * p.in_rows * p.in_cols * p.channels
@@ -625,7 +690,8 @@ def main():
         ms = event_time_ms(run_max_grad, reps=3 * sets, warm=sets, repeats=3)
         grads.append(mem_entry("maxpool3x3_s2_112x112x64_grad",
                                4 * (2 * n_in + 2 * n_out), ms,
-                               device_ms(run_max_grad, 3 * sets)))
+                               device_ms(run_max_grad, 3 * sets),
+                               with_stream=False))
 
         def run_avg_grad():
             i = state["i"] % sets
@@ -634,7 +700,8 @@ def main():
         ms = event_time_ms(run_avg_grad, reps=3 * sets, warm=sets, repeats=3)
         grads.append(mem_entry("avgpool3x3_s2_112x112x64_grad",
                                4 * (n_in + n_out), ms,
-                               device_ms(run_avg_grad, 3 * sets)))
+                               device_ms(run_avg_grad, 3 * sets),
+                               with_stream=False))
         del xs, ys, dys, dxs
         detail["memory_bound_gradients"] = grads
 
@@ -711,11 +778,11 @@ def main():
         x = rng.uniform(-1, 1, 56 * 56 * 64).astype(np.float32)
         w = rng.uniform(-1, 1, 9 * 64 * 64).astype(np.float32)
         sec, runs = cpu_time(lambda: oracle.conv2d_tiled_forward(x, w, p), 2.0)
-        cpu["config0"] = {
-            "value": round(2.0 * 56 * 56 * 9 * 64 * 64 / sec / 1e12, 5),
-            "unit": "TFLOP/s", "ms": round(sec * 1e3, 3), "cores": cores,
-            "sample": "median of %d runs of the tiled restatement on "
-                      "[1,56,56,64] x [3,3,64,64]" % runs}
+        cpu["config0_tflops"] = round(
+            2.0 * 56 * 56 * 9 * 64 * 64 / sec / 1e12, 5)
+        cpu["config0_ms"] = round(sec * 1e3, 3)
+        cpu["config0_sample"] = ("median of %d runs of the tiled restatement "
+                                 "on [1,56,56,64] x [3,3,64,64]" % runs)
 
         # depthwise and pooling in the reference's loop order
         # (src/depthwise_conv2d/kernels.h:58-125, src/pooling/kernels.h:61-99:
@@ -749,6 +816,18 @@ def main():
                             "gbs": round(nbytes / sec / 1e9, 2), "runs": runs})
         cpu["memory_bound"] = mem_cpu
         cpu["memory_bound_unit"] = "GB/s"
+        cpu["memory_bound_sample"] = ("batch %d of each layer, reference loop "
+                                      "order, %d host threads" % (cb, cores))
+        for e in mem_cpu:
+            if e["op"].startswith("depthwise"):
+                cpu["depthwise_" + e["op"].split("_", 1)[1] + "_gbs"] = e["gbs"]
+            elif e["op"].startswith("maxpool"):
+                cpu["maxpool_gbs"] = e["gbs"]
+            else:
+                cpu["avgpool_gbs"] = e["gbs"]
+        dw = [e for e in mem_cpu if e["op"].startswith("depthwise")]
+        cpu["depthwise_gbs"] = round(
+            sum(e["bytes"] for e in dw) / sum(e["ms"] for e in dw) / 1e6, 2)
 
     line = {
         "metric": "conv2d fwd TFLOP/s + %MFMA peak; depthwise/pool GB/s + "

@@ -6,7 +6,10 @@
 // batch_matmul members of the backend concept
 // (include/portdnn/backend/backend_interface.h:93-118), here served by
 // libsnn_hip's MFMA GEMM.  Work is ordered on one HIP stream per backend
-// object; the library keeps no global mutable state.
+// object.  Launches from different backends do not share mutable state except
+// the library's per-device pool of stream-ordered temporaries (thread-safe)
+// and, for the one no-allocation depthwise entry point, its scratch array
+// (calls that overlap on one GPU race on it, as its declaration says).
 #ifndef PORTDNN_HIP_BACKEND_H_
 #define PORTDNN_HIP_BACKEND_H_
 

@@ -197,9 +197,25 @@ class MatmulSelector final : public internal::RuleSelector<Algorithm::Matmul> {
   char const* name() const override { return "MatmulSelector"; }
 };
 
-// What get_default_selector returns: the per-layer choice tuned for MI355X.
+namespace internal {
+template <typename T>
+struct DataType {
+  static_assert(sizeof(T) == 2, "supported data types: float and half");
+  static constexpr int value = SNN_HIP_DTYPE_F16;
+};
+template <>
+struct DataType<float> {
+  static constexpr int value = SNN_HIP_DTYPE_F32;
+};
+}  // namespace internal
+
+// What get_default_selector returns: the per-layer choice tuned for MI355X,
+// for float launches unless built for another element type
+// (get_default_selector_for<T>): the half-precision kernels are different
+// kernels, and half has no Winograd.
 class DefaultSelector final : public Selector {
  public:
+  explicit DefaultSelector(int dtype = SNN_HIP_DTYPE_F32) : dtype_(dtype) {}
   Algorithm select_forward(Conv2DParams const& p) override {
     return ask(p, SNN_HIP_FORWARD);
   }
@@ -212,11 +228,12 @@ class DefaultSelector final : public Selector {
   char const* name() const override { return "Default"; }
 
  private:
-  static Algorithm ask(Conv2DParams const& p, int direction) {
+  Algorithm ask(Conv2DParams const& p, int direction) const {
     const snn_hip_conv2d_params c = internal::to_c(p);
     return static_cast<Algorithm>(
-        snn_hip_conv2d_default_algorithm(&c, direction));
+        snn_hip_conv2d_default_algorithm_for(&c, direction, dtype_));
   }
+  int dtype_;
 };
 
 // portDNN takes a cl::sycl::device here; the HIP build takes the backend (or
@@ -227,6 +244,13 @@ inline std::unique_ptr<Selector> get_default_selector() {
 template <typename Backend>
 inline std::unique_ptr<Selector> get_default_selector(Backend const&) {
   return get_default_selector();
+}
+// Not in portDNN, whose selectors do not know the element type: the default
+// selector for launches of element type T.
+template <typename T>
+inline std::unique_ptr<Selector> get_default_selector_for() {
+  return std::unique_ptr<Selector>(
+      new DefaultSelector(internal::DataType<T>::value));
 }
 
 // ---- workspace ---------------------------------------------------------------
@@ -245,6 +269,21 @@ WorkspaceSize query_workspace_size(Conv2DParams const& params,
   (void)snn_hip_conv2d_workspace_size(&c, internal::Direction<ConvType>::value,
                                       static_cast<int>(algo),
                                       &ws.required_size, &ws.recommended_size);
+  return ws;
+}
+
+// Not in portDNN: the same query for launches of element type T, in elements
+// of T.  For half the answer differs from the type-blind one above (required
+// is 0, recommended is what the half kernels use).
+template <typename T, typename ConvType>
+WorkspaceSize query_workspace_size(Conv2DParams const& params,
+                                   Selector& selector) {
+  const snn_hip_conv2d_params c = internal::to_c(params);
+  const Algorithm algo = selector.select<ConvType>(params);
+  WorkspaceSize ws{0, 0};
+  (void)snn_hip_conv2d_workspace_size_for(
+      &c, internal::Direction<ConvType>::value, static_cast<int>(algo),
+      internal::DataType<T>::value, &ws.required_size, &ws.recommended_size);
   return ws;
 }
 

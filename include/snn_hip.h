@@ -161,6 +161,18 @@ SNN_HIP_API const char* snn_hip_last_error(void);
 SNN_HIP_API int snn_hip_kernel_timing_enable(int enable);
 SNN_HIP_API int snn_hip_kernel_timing_read(double* total_ms, int* kernels);
 
+/* Diagnostics for the stream-ordered temporaries some launches take when the
+ * caller passes no workspace (no counterpart in portDNN, whose temporaries
+ * come from backend.allocate): bytes currently reserved by, and the high-water
+ * mark of bytes in use in, the two pools such temporaries come from on the
+ * current device -- the library's own pool and the device's default pool.
+ * With reset_high != 0 the high-water marks are cleared after reading, so a
+ * caller can bracket a sequence of launches and see whether any of them took
+ * a temporary. */
+SNN_HIP_API int snn_hip_temporary_memory_stats(
+    unsigned long long* reserved_bytes, unsigned long long* used_high_bytes,
+    int reset_high);
+
 /* ---- dense convolution ---------------------------------------------------
  * Stand-ins for sycldnn::conv2d::internal::launch_{direct,tiled,matmul,
  * im2col,winograd} reached from sycldnn::conv2d::launch<T, ConvType>
@@ -194,10 +206,14 @@ SNN_HIP_API int snn_hip_conv2d_forward_f16(
     const snn_hip_conv2d_params* params, int algorithm, void* workspace,
     size_t workspace_elems, void* stream);
 /* The two gradients in half precision (fp32 accumulation), the reference's
- * launch<half, conv_type::InputBackprop / FilterBackprop>.  Stride-1 input
- * gradients with channel and feature counts in multiples of 64 run on the
- * matrix cores; everything else, and the filter gradient, on the direct
- * kernels. */
+ * launch<half, conv_type::InputBackprop / FilterBackprop>.  With channel
+ * counts in multiples of 64 they run on the matrix cores (3x3 stride-1 SAME
+ * and 1x1 filter gradients and stride-1 input gradients on binary16 matrix
+ * instructions, other shapes on fp32 matrix instructions fed binary16
+ * operands); shapes off those multiples run on the direct kernels.  No
+ * half-precision launch requires a workspace; one of the size
+ * snn_hip_conv2d_workspace_size_for reports saves a stream-ordered
+ * temporary. */
 SNN_HIP_API int snn_hip_conv2d_input_backprop_f16(
     const void* input, const void* filter, void* output,
     const snn_hip_conv2d_params* params, int algorithm, void* workspace,
@@ -239,6 +255,23 @@ SNN_HIP_API int snn_hip_conv2d_workspace_size(
     const snn_hip_conv2d_params* params, int direction, int algorithm,
     size_t* required_elems, size_t* recommended_elems);
 
+/* The same for a given element type (a snn_hip_dtype), in elements of that
+ * type.  portDNN's query does not know the element type
+ * (workspace_size.h:158-163 takes only the parameters and the selector); the
+ * half-precision kernels here are different kernels with different needs, so
+ * a caller that sizes its scratch from the fp32 answer would allocate the
+ * F(2x2,3x3) transform buffers for a launch that uses a filter-sized block.
+ * For SNN_HIP_DTYPE_F16 `required` is always 0 (a launch without scratch
+ * takes a stream-ordered temporary) and `recommended` is what the launch
+ * uses.  SNN_HIP_DTYPE_F32 answers as snn_hip_conv2d_workspace_size. */
+typedef enum snn_hip_dtype {
+  SNN_HIP_DTYPE_F32 = 0,
+  SNN_HIP_DTYPE_F16 = 1
+} snn_hip_dtype;
+SNN_HIP_API int snn_hip_conv2d_workspace_size_for(
+    const snn_hip_conv2d_params* params, int direction, int algorithm,
+    int dtype, size_t* required_elems, size_t* recommended_elems);
+
 /* Does `algorithm` support these parameters in this direction?  Mirrors the
  * concrete selectors (include/portdnn/conv2d/selector/{tiled,winograd,matmul}_
  * selector.h, constant_selector.h): returns `algorithm` if it does, else
@@ -251,6 +284,11 @@ SNN_HIP_API int snn_hip_conv2d_algorithm_supports(
  * MI355X. */
 SNN_HIP_API int snn_hip_conv2d_default_algorithm(
     const snn_hip_conv2d_params* params, int direction);
+/* The same for a given element type: half precision has no Winograd kernels,
+ * so its 3x3 layers get the Tiled (forward) / Im2col tag, whose kernels and
+ * workspace snn_hip_conv2d_workspace_size_for describes. */
+SNN_HIP_API int snn_hip_conv2d_default_algorithm_for(
+    const snn_hip_conv2d_params* params, int direction, int dtype);
 
 /* ---- depthwise convolution -----------------------------------------------
  * Stand-ins for sycldnn::depthwise_conv2d::internal::launch<ConvType>
@@ -278,7 +316,11 @@ SNN_HIP_API int snn_hip_depthwise_conv2d_filter_backprop_f32(
  * partial filters would not fit is rejected with SNN_HIP_INVALID_PARAMETER
  * and a message in snn_hip_last_error().  All calls on one GPU share that
  * array: calls that overlap on one GPU (different streams or threads) race;
- * stream-ordered calls are safe.  The stream's device must be current. */
+ * stream-ordered calls are safe.  The stream's device must be current.  The
+ * first call on each device looks the array's address up
+ * (hipGetSymbolAddress, which may load the library's device code): make one
+ * call per device before a stream capture begins; later calls only enqueue
+ * kernels. */
 SNN_HIP_API int snn_hip_depthwise_conv2d_filter_backprop_noalloc_f32(
     const float* input, const float* filter, float* output,
     const snn_hip_depthwise_params* params, void* stream);

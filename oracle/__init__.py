@@ -47,6 +47,10 @@ def lib():
                      "depthwise_input_backprop", "depthwise_filter_backprop"):
             getattr(L, "oracle_" + name).argtypes = [_FP, _FP, _FP, _PP,
                                                      ctypes.c_int]
+        L.oracle_conv2d_winograd_forward.argtypes = [_FP, _FP, _FP, _PP,
+                                                     ctypes.c_int,
+                                                     ctypes.c_int]
+        L.oracle_conv2d_winograd_forward.restype = ctypes.c_int
         L.oracle_conv2d_tiled_forward.argtypes = [_FP, _FP, _FP, _PP,
                                                   ctypes.c_int]
         L.oracle_conv2d_tiled_forward.restype = ctypes.c_int
@@ -119,6 +123,21 @@ def conv2d_input_backprop(dy, w, p, acc64=True):
 def conv2d_filter_backprop(x, dy, p, acc64=True):
     n = p.window_rows * p.window_cols * p.channels * p.features
     return _three("conv2d_filter_backprop", x, dy, n, p, acc64)
+
+
+def conv2d_winograd_forward(x, w, p, tile, acc64=False):
+    """Forward convolution by Winograd F(tile x tile, 3x3), tile 2 or 4, every
+    stage in float (or double): the fp32 behaviour of the algorithm."""
+    x, xp = _f(x)
+    w, wp = _f(w)
+    out = np.empty(p.batch * p.out_rows * p.out_cols * p.features,
+                   dtype=np.float32)
+    rc = lib().oracle_conv2d_winograd_forward(
+        xp, wp, out.ctypes.data_as(_FP), ctypes.byref(p), int(tile),
+        int(acc64))
+    if rc != 0:
+        raise ValueError("Winograd restatement: 3x3 stride 1, tile 2 or 4")
+    return out
 
 
 def conv2d_tiled_forward(x, w, p, threads=0):

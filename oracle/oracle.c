@@ -7,6 +7,7 @@
 #include <float.h>
 #include <math.h>
 #include <stddef.h>
+#include <stdlib.h>
 #ifdef _OPENMP
 #include <omp.h>
 #endif
@@ -90,6 +91,15 @@ void oracle_conv2d_input_backprop(const float* dy, const float* fil, float* dx,
 void oracle_conv2d_filter_backprop(const float* in, const float* dy, float* dw,
                                    const oracle_params* p, int acc64) {
   DISPATCH(conv2d_filter_backprop, in, dy, dw, p);
+}
+int oracle_conv2d_winograd_forward(const float* in, const float* fil,
+                                   float* out, const oracle_params* p,
+                                   int tile, int acc64) {
+  if ((tile != 2 && tile != 4) || p->window_rows != 3 || p->window_cols != 3 ||
+      p->stride_rows != 1 || p->stride_cols != 1)
+    return 1;
+  DISPATCH(conv2d_winograd_forward, in, fil, out, p, tile);
+  return 0;
 }
 void oracle_depthwise_forward(const float* in, const float* fil, float* out,
                               const oracle_params* p, int acc64) {

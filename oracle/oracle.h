@@ -21,7 +21,10 @@
  *     and is checked against the same goldens.
  *   matmul: textbook definition, checked against numpy float64 matmul for all
  *     transpose/beta combinations.
- *   Winograd transforms: algebraic identity against the direct convolution.
+ *   Winograd forward (F(2x2,3x3) and F(4x4,3x3), the reference's transform
+ *     matrices): with double accumulation it must equal the direct
+ *     convolution to ~1e-12 on random data and exactly on the integer goldens
+ *     (tests/test_oracle_golden.py); the float variant is the same code.
  *   pointwise (relu, tanh, log, floor, sqrt; forward and gradient) and
  *     binaryop (add, sub, mul, div with broadcasting): the reference's golden
  *     vectors of test/pointwise/ *.cc and test/binaryop/ *.cc
@@ -58,6 +61,14 @@ void oracle_calculate_padding(int input, int window, int stride, int same,
  * accumulates in float in the reference's loop order. */
 void oracle_conv2d_forward(const float* in, const float* fil, float* out,
                            const oracle_params* p, int acc64);
+/* The same result by the Winograd algorithm with tile x tile output blocks
+ * (2: Algorithm::Winograd, 4: Algorithm::WinogradLarge), 3x3 stride 1 only;
+ * every stage in float (acc64 == 0) or double.  Returns non-zero for other
+ * shapes.  include/portdnn/internal/conv2d/winograd/launch.h:63-264,
+ * src/conv2d/winograd/kernels/tiles_impl.h:70-198,774-1000. */
+int oracle_conv2d_winograd_forward(const float* in, const float* fil,
+                                   float* out, const oracle_params* p,
+                                   int tile, int acc64);
 void oracle_conv2d_input_backprop(const float* dy, const float* fil, float* dx,
                                   const oracle_params* p, int acc64);
 void oracle_conv2d_filter_backprop(const float* in, const float* dy, float* dw,

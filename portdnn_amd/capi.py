@@ -40,6 +40,11 @@ class DIRECTION:
     FILTER_BACKPROP = 2
 
 
+class DTYPE:
+    F32 = 0
+    F16 = 1
+
+
 class POOL_OP:
     MAX = 0
     MAX_WITH_NAN = 1
@@ -109,6 +114,9 @@ SIGNATURES = {
     "snn_hip_version": [],
     "snn_hip_status_string": [_I],
     "snn_hip_last_error": [],
+    "snn_hip_temporary_memory_stats": [
+        ctypes.POINTER(ctypes.c_ulonglong), ctypes.POINTER(ctypes.c_ulonglong),
+        _I],
     "snn_hip_kernel_timing_enable": [_I],
     "snn_hip_kernel_timing_read": [ctypes.POINTER(ctypes.c_double),
                                    ctypes.POINTER(ctypes.c_int)],
@@ -125,6 +133,9 @@ SIGNATURES = {
                                       ctypes.POINTER(_SZ)],
     "snn_hip_conv2d_algorithm_supports": [_P, _I, _I],
     "snn_hip_conv2d_default_algorithm": [_P, _I],
+    "snn_hip_conv2d_default_algorithm_for": [_P, _I, _I],
+    "snn_hip_conv2d_workspace_size_for": [_P, _I, _I, _I, ctypes.POINTER(_SZ),
+                                          ctypes.POINTER(_SZ)],
     "snn_hip_depthwise_conv2d_forward_f32": [_P, _P, _P, _P, _P],
     "snn_hip_depthwise_conv2d_input_backprop_f32": [_P, _P, _P, _P, _P],
     "snn_hip_depthwise_conv2d_filter_backprop_f32": [_P, _P, _P, _P, _P],

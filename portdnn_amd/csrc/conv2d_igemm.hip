@@ -2105,9 +2105,14 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
                             hipStream_t stream, float* workspace,
                             size_t workspace_elems,
                             const LaunchOptions* epilogue) {
+  if (direction == SNN_HIP_FORWARD && conv2d_small_supports(p) &&
+      SNN_TUNING_ENV("SNN_HIP_SMALL_OFF") == nullptr)
+    return launch_conv2d_small_f32(input, filter, output, p, stream, epilogue);
   if (direction == SNN_HIP_INPUT_BACKPROP &&
       conv2d_stem_input_backprop_supports(p) &&
       (reinterpret_cast<uintptr_t>(output) & 15u) == 0 &&
+      (epilogue == nullptr || !epilogue->deterministic ||
+       conv2d_stem_input_backprop_reproducible(p)) &&
       SNN_TUNING_ENV("SNN_HIP_STEM_OFF") == nullptr) {
     // three channels, 7x7 stride 2, 64 features: the kernel built for it
     return launch_conv2d_stem_input_backprop_f32(input, filter, output, p,

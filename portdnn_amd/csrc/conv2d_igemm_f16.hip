@@ -379,6 +379,32 @@ static bool as_forward_of_dy(const snn_hip_conv2d_params& p,
   return true;
 }
 
+// Halves of caller workspace the forward / input-gradient launchers below put
+// to use (the re-laid-out filter); 0 for the shapes that need none.
+size_t conv2d_f16_filter_pack_halves(int direction,
+                                     const snn_hip_conv2d_params& p) {
+  const size_t wgt_elems = static_cast<size_t>(p.window_rows) * p.window_cols *
+                           p.channels * p.features;
+  if (direction == SNN_HIP_FORWARD) {
+    if (!conv2d_igemm_f16_supports(p)) return 0;
+    const size_t pixels = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols;
+    if (p.window_rows == 1 && p.window_cols == 1 && p.stride_rows == 1 &&
+        p.stride_cols == 1 && p.pad_rows == 0 && p.pad_cols == 0 &&
+        p.out_rows == p.in_rows && p.out_cols == p.in_cols &&
+        pixels <= static_cast<size_t>(INT_MAX) &&
+        gemm_rows_f16_supports(static_cast<int>(pixels), p.channels,
+                               p.features))
+      return 0;
+    return wgt_elems;
+  }
+  if (direction == SNN_HIP_INPUT_BACKPROP) {
+    snn_hip_conv2d_params q;
+    if (!as_forward_of_dy(p, &q)) return 0;
+    return conv2d_rowtile_f16_supports(q) ? wgt_elems : 0;
+  }
+  return 0;
+}
+
 bool conv2d_input_backprop_f16_supports(const snn_hip_conv2d_params& p) {
   snn_hip_conv2d_params q;
   if (!as_forward_of_dy(p, &q)) return false;

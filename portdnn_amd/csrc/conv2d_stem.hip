@@ -810,6 +810,16 @@ bool conv2d_stem_input_backprop_supports(const snn_hip_conv2d_params& p) {
          (static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * kCh) % 4 == 0;
 }
 
+// Input rows that two neighbouring bands both touch receive their two parts
+// through float atomics into the zero-filled dX: two addends commute, so the
+// sum does not depend on their order.  With bands of two output rows (a pitch
+// of four input rows against a seven-row window) a row can belong to three
+// bands, and three addends do not.
+bool conv2d_stem_input_backprop_reproducible(const snn_hip_conv2d_params& p) {
+  StemGeom g;
+  return make_geom(p, &g) && (g.n_bands < 3 || kStride * g.band >= kWin - kStride);
+}
+
 // dy, filter and dx 16-byte aligned.
 int launch_conv2d_stem_input_backprop_f32(const float* dy, const float* w,
                                           float* dx,

@@ -128,7 +128,9 @@ __global__ void __launch_bounds__(256)
       for (int i = 0; i < VEC; ++i) op[i].accumulate(v[i]);
     }
   }
-  const int tally = (r1 - r0) * (c1 - c0);
+  // the number of elements accumulated (src/pooling/operators_impl.h:61-82
+  // counts them one by one): none when the window misses the image on an axis
+  const int tally = max(r1 - r0, 0) * max(c1 - c0, 0);
   float res[VEC];
 #pragma unroll
   for (int i = 0; i < VEC; ++i) res[i] = op[i].value(tally);
@@ -326,8 +328,10 @@ __global__ void __launch_bounds__(256)
   int c0 = ox * p.stride_cols - p.pad_cols;
   const int c1 = min(c0 + p.window_cols, p.in_cols);
   c0 = max(c0, 0);
-  const int width = c1 - c0;
-  const int n_taps = (r1 - r0) * width;
+  // a window wholly outside the image on an axis has no taps (both extents
+  // negative must not multiply to a positive count)
+  const int width = max(c1 - c0, 0);
+  const int n_taps = max(r1 - r0, 0) * width;
   Op acc[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) acc[i].init(lowest_of<T>());

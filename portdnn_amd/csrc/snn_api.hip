@@ -5,6 +5,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
@@ -16,8 +17,11 @@ namespace {
 thread_local std::string g_last_error;
 }
 
-// The opt-in kernel-timing record: the only process-wide state of the
-// library.  The switch is atomic and the list of event pairs is guarded by a
+// Process-wide state of the library: this opt-in kernel-timing record, the
+// per-device memory pool for stream-ordered temporaries below (created at
+// first use, kept until the process ends) and the scratch array of the
+// no-allocation depthwise entry point (depthwise.hip).
+// The timing switch is atomic and the list of event pairs is guarded by a
 // mutex, so launches from several threads may record concurrently; the list
 // stops growing at kMaxTimedKernels pairs until it is read.
 namespace {
@@ -307,10 +311,36 @@ void im2col_workspace(const snn_hip_conv2d_params& p, int direction,
 // no transformed tensors, only one partial filter per slice of the tile
 // range; shapes it does not take run on the implicit-GEMM kernel and need
 // nothing.
+//
+// Half precision: every algorithm tag runs on the binary16 matrix-core kernels
+// (or the direct kernel), none of which *requires* caller scratch -- without
+// it they take a stream-ordered temporary -- so `required` is 0 and
+// `recommended` is what the launch puts to use: the re-laid-out filter
+// (forward, stride-1 input gradient) or the fp32 partial tiles / accumulation
+// buffer of the filter gradient, counted in halves.
+size_t f16_workspace_halves(const snn_hip_conv2d_params& p, int direction) {
+  if (direction != SNN_HIP_FILTER_BACKPROP)
+    return conv2d_f16_filter_pack_halves(direction, p);
+  if (!conv2d_filter_backprop_f16_supports(p)) return 0;
+  if (conv2d_filter_backprop_3x3_f16_supports(p))
+    return 2 * conv2d_filter_backprop_3x3_f16_partial_floats(p);
+  if (conv2d_filter_backprop_1x1_f16_supports(p))
+    return 2 * conv2d_filter_backprop_1x1_f16_partial_floats(p);
+  return 2 * static_cast<size_t>(p.window_rows) * p.window_cols * p.channels *
+         p.features;
+}
+
 int workspace_size(const snn_hip_conv2d_params& p, int direction,
-                   int algorithm, size_t* required, size_t* recommended) {
+                   int algorithm, int dtype, size_t* required,
+                   size_t* recommended) {
   *required = 0;
   *recommended = 0;
+  if (dtype == SNN_HIP_DTYPE_F16) {
+    if (algorithm != SNN_HIP_ALGO_DIRECT &&
+        algorithm_supports(p, direction, algorithm) == algorithm)
+      *recommended = f16_workspace_halves(p, direction);
+    return SNN_HIP_OK;
+  }
   const bool filbk = direction == SNN_HIP_FILTER_BACKPROP;
   switch (algorithm) {
     case SNN_HIP_ALGO_WINOGRAD:
@@ -340,9 +370,17 @@ int workspace_size(const snn_hip_conv2d_params& p, int direction,
 // (src/conv2d/selector/default_selector.cc:49-128): 1x1 stride-1 unpadded
 // convolutions are one GEMM; everything else is the implicit-GEMM path, which
 // the Im2col tag names (Tiled where the reference's TiledSelector accepts it).
-int default_algorithm(const snn_hip_conv2d_params& p, int direction) {
+// Half precision has no Winograd kernels: its 3x3 layers run on the LDS-tile
+// kernel behind the Tiled / Im2col tags, so the policy never answers Winograd
+// for it (a Winograd tag would still run, on those same kernels).
+int default_algorithm(const snn_hip_conv2d_params& p, int direction,
+                      int dtype) {
   if (algorithm_supports(p, direction, SNN_HIP_ALGO_MATMUL))
     return SNN_HIP_ALGO_MATMUL;
+  if (dtype == SNN_HIP_DTYPE_F16)
+    return algorithm_supports(p, direction, SNN_HIP_ALGO_TILED)
+               ? SNN_HIP_ALGO_TILED
+               : SNN_HIP_ALGO_IM2COL;
   // 3x3 stride-1 layers whose channel counts fit the fused Winograd kernel:
   // measured 1.3-1.5x faster than the implicit GEMM on the batch-32 ResNet
   // shapes.  The caller sizes the workspace with query_workspace_size for
@@ -434,7 +472,8 @@ int launch_winograd_path(int direction, const T* input, const T* filter,
                          T* output, const snn_hip_conv2d_params& p,
                          T* workspace, size_t workspace_elems, hipStream_t s,
                          const LaunchOptions* epilogue = nullptr) {
-  return launch_gemm_path<T>(direction, input, filter, output, p, s);
+  return launch_gemm_path<T>(direction, input, filter, output, p, s, workspace,
+                             workspace_elems);
 }
 template <>
 int launch_winograd_path<float>(int direction, const float* input,
@@ -569,7 +608,10 @@ int conv2d_dispatch(int direction, const T* input, const T* filter, T* output,
       // internal/conv2d/winograd/launch.h:271-286: a Winograd launch without
       // the workspace its transforms need reports InsufficientWorkspace.
       size_t required = 0, recommended = 0;
-      workspace_size(p, direction, algorithm, &required, &recommended);
+      workspace_size(p, direction, algorithm,
+                     std::is_same<T, float>::value ? SNN_HIP_DTYPE_F32
+                                                   : SNN_HIP_DTYPE_F16,
+                     &required, &recommended);
       if (required > 0 && (workspace == nullptr || workspace_elems < required))
         return SNN_HIP_INSUFFICIENT_WORKSPACE;
       return launch_winograd_path<T>(direction, input, filter, output, p,
@@ -676,6 +718,44 @@ int snn_hip_kernel_timing_read(double* total_ms, int* kernels) {
   return status;
 }
 
+int snn_hip_temporary_memory_stats(unsigned long long* reserved_bytes,
+                                   unsigned long long* used_high_bytes,
+                                   int reset_high) {
+  if (reserved_bytes == nullptr || used_high_bytes == nullptr)
+    return SNN_HIP_INVALID_PARAMETER;
+  *reserved_bytes = 0;
+  *used_high_bytes = 0;
+  int device = 0;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return snn::report_hip_error(err, "hipGetDevice");
+  hipMemPool_t pools[2] = {nullptr, nullptr};
+  if (device >= 0 && device < snn::kMaxPoolDevices) {
+    std::lock_guard<std::mutex> lock(snn::g_pool_mutex);
+    pools[0] = snn::g_pools[device];
+  }
+  if (hipDeviceGetDefaultMemPool(&pools[1], device) != hipSuccess) {
+    (void)hipGetLastError();
+    pools[1] = nullptr;
+  }
+  for (hipMemPool_t pool : pools) {
+    if (pool == nullptr) continue;
+    uint64_t reserved = 0, high = 0;
+    err = hipMemPoolGetAttribute(pool, hipMemPoolAttrReservedMemCurrent,
+                                 &reserved);
+    if (err == hipSuccess)
+      err = hipMemPoolGetAttribute(pool, hipMemPoolAttrUsedMemHigh, &high);
+    if (err != hipSuccess)
+      return snn::report_hip_error(err, "hipMemPoolGetAttribute");
+    *reserved_bytes += reserved;
+    *used_high_bytes += high;
+    if (reset_high != 0) {
+      uint64_t zero = 0;
+      (void)hipMemPoolSetAttribute(pool, hipMemPoolAttrUsedMemHigh, &zero);
+    }
+  }
+  return SNN_HIP_OK;
+}
+
 int snn_hip_conv2d_forward_f32(const float* input, const float* filter,
                                float* output,
                                const snn_hip_conv2d_params* params,
@@ -764,7 +844,22 @@ int snn_hip_conv2d_workspace_size(const snn_hip_conv2d_params* params,
     return SNN_HIP_INVALID_PARAMETER;
   if (direction < SNN_HIP_FORWARD || direction > SNN_HIP_FILTER_BACKPROP)
     return SNN_HIP_INVALID_PARAMETER;
-  return workspace_size(*params, direction, algorithm, required_elems,
+  return workspace_size(*params, direction, algorithm, SNN_HIP_DTYPE_F32,
+                        required_elems, recommended_elems);
+}
+
+int snn_hip_conv2d_workspace_size_for(const snn_hip_conv2d_params* params,
+                                      int direction, int algorithm, int dtype,
+                                      size_t* required_elems,
+                                      size_t* recommended_elems) {
+  if (params == nullptr || required_elems == nullptr ||
+      recommended_elems == nullptr)
+    return SNN_HIP_INVALID_PARAMETER;
+  if (direction < SNN_HIP_FORWARD || direction > SNN_HIP_FILTER_BACKPROP)
+    return SNN_HIP_INVALID_PARAMETER;
+  if (dtype != SNN_HIP_DTYPE_F32 && dtype != SNN_HIP_DTYPE_F16)
+    return SNN_HIP_INVALID_PARAMETER;
+  return workspace_size(*params, direction, algorithm, dtype, required_elems,
                         recommended_elems);
 }
 
@@ -777,7 +872,15 @@ int snn_hip_conv2d_algorithm_supports(const snn_hip_conv2d_params* params,
 int snn_hip_conv2d_default_algorithm(const snn_hip_conv2d_params* params,
                                      int direction) {
   if (params == nullptr) return SNN_HIP_ALGO_NOT_SUPPORTED;
-  return default_algorithm(*params, direction);
+  return default_algorithm(*params, direction, SNN_HIP_DTYPE_F32);
+}
+
+int snn_hip_conv2d_default_algorithm_for(const snn_hip_conv2d_params* params,
+                                         int direction, int dtype) {
+  if (params == nullptr ||
+      (dtype != SNN_HIP_DTYPE_F32 && dtype != SNN_HIP_DTYPE_F16))
+    return SNN_HIP_ALGO_NOT_SUPPORTED;
+  return default_algorithm(*params, direction, dtype);
 }
 
 int snn_hip_depthwise_conv2d_forward_f32(

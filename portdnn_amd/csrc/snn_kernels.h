@@ -107,6 +107,14 @@ bool gemm_wreg_supports(int m, int k, int n);
 void launch_gemm_wreg(const float* x, const float* w, float* y, int m, int k,
                       int n, bool epilogue, const float* bias, bool relu,
                       hipStream_t stream);
+// Forward convolution of problems with few output tiles (one 56x56x64 image:
+// 49 tiles of 64x64) in one launch without atomics (conv2d_small.hip):
+// work-groups of 16 pixels x 64 features whose four waves split the
+// reduction.  Channels and features in multiples of 64; 16-byte aligned.
+bool conv2d_small_supports(const snn_hip_conv2d_params& p);
+int launch_conv2d_small_f32(const float* x, const float* w, float* y,
+                            const snn_hip_conv2d_params& p, hipStream_t stream,
+                            const LaunchOptions* epilogue = nullptr);
 // Forward convolution of a three-channel image with a 7x7 window, stride 2 and
 // 64 features (conv2d_stem.hip): input rows of a band of output rows in LDS,
 // the filter in registers.  Output 16-byte aligned, at most 128 output columns.
@@ -120,6 +128,9 @@ int launch_conv2d_stem_input_backprop_f32(const float* dy, const float* w,
                                           float* dx,
                                           const snn_hip_conv2d_params& p,
                                           hipStream_t stream);
+// (whether that launch adds at most two parts into any dX element, i.e. gives
+// the same bits every run)
+bool conv2d_stem_input_backprop_reproducible(const snn_hip_conv2d_params& p);
 bool conv2d_stem_filter_backprop_supports(const snn_hip_conv2d_params& p);
 int launch_conv2d_stem_filter_backprop_f32(const float* x, const float* dy,
                                            float* dw,
@@ -145,6 +156,10 @@ int launch_conv2d_igemm_f16(const _Float16* input, const _Float16* filter,
 bool gemm_rows_f16_supports(int m, int k, int n);
 int launch_gemm_rows_f16(const _Float16* x, const _Float16* w, _Float16* y,
                          int m, int k, int n, hipStream_t stream);
+// Halves of caller workspace the half-precision forward and input-gradient
+// launchers use for the re-laid-out filter (0: none needed).
+size_t conv2d_f16_filter_pack_halves(int direction,
+                                     const snn_hip_conv2d_params& p);
 // Stride-1 input gradient in half precision: the forward kernels above run on
 // dY with the filter's taps mirrored and its channel / feature roles swapped.
 // `supports` is false when neither kernel takes the shape.

@@ -85,12 +85,28 @@ def _ptr(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else None
 
 
-def workspace_size(p, direction, algorithm):
+def workspace_size(p, direction, algorithm, dtype=None):
+    """(required, recommended) elements; with a capi.DTYPE the element type's
+    own answer (snn_hip_conv2d_workspace_size_for)."""
     req, rec = ctypes.c_size_t(), ctypes.c_size_t()
-    capi.check(capi.lib().snn_hip_conv2d_workspace_size(
-        ctypes.byref(p), direction, algorithm, ctypes.byref(req),
-        ctypes.byref(rec)))
+    if dtype is None:
+        capi.check(capi.lib().snn_hip_conv2d_workspace_size(
+            ctypes.byref(p), direction, algorithm, ctypes.byref(req),
+            ctypes.byref(rec)))
+    else:
+        capi.check(capi.lib().snn_hip_conv2d_workspace_size_for(
+            ctypes.byref(p), direction, algorithm, dtype, ctypes.byref(req),
+            ctypes.byref(rec)))
     return req.value, rec.value
+
+
+def default_algorithm(p, direction, dtype=None):
+    """The library's default selector's choice (for a capi.DTYPE when given)."""
+    if dtype is None:
+        return capi.lib().snn_hip_conv2d_default_algorithm(ctypes.byref(p),
+                                                           direction)
+    return capi.lib().snn_hip_conv2d_default_algorithm_for(
+        ctypes.byref(p), direction, dtype)
 
 
 _CONV_FN = {
@@ -124,7 +140,8 @@ def conv2d(inp, fil, p, direction=DIRECTION.FORWARD, algorithm=ALGO.DIRECT,
     assert inp.is_contiguous() and fil.is_contiguous()
     if out is None:
         out = torch.empty(n_out, dtype=inp.dtype, device=inp.device)
-    if workspace is None and algorithm in (ALGO.WINOGRAD, ALGO.WINOGRAD_LARGE):
+    if (workspace is None and inp.dtype == torch.float32 and
+            algorithm in (ALGO.WINOGRAD, ALGO.WINOGRAD_LARGE)):
         _, rec = workspace_size(p, direction, algorithm)
         workspace = torch.empty(rec, dtype=inp.dtype, device=inp.device)
     capi.check(conv2d_raw(inp, fil, out, p, direction, algorithm, workspace))
@@ -300,6 +317,7 @@ __all__ = [
     "binaryop", "binaryop_raw", "calculate_padding", "conv2d",
     "conv2d_bias_act",
     "conv2d_raw", "conv_flops", "conv_params", "conv_sizes",
+    "default_algorithm",
     "depthwise_conv2d", "depthwise_params", "depthwise_sizes", "matmul",
     "pointwise_forward", "pointwise_grad", "pool_params", "pooling_avg_grad",
     "pooling_forward", "pooling_max_grad",

@@ -194,6 +194,50 @@ def test_default_algorithm_policy_on_benchmark_layers():
     assert default(odd, DIRECTION.FILTER_BACKPROP) == ALGO.IM2COL
 
 
+def test_default_algorithm_and_workspace_know_the_element_type():
+    """Half precision has no Winograd kernels: the typed default selector
+    never answers Winograd for it, and the typed workspace query reports what
+    the half kernels use (a filter-sized block or the filter gradient's
+    partial tiles), never the fp32 F(2x2,3x3) transform buffers.  The
+    type-blind entries keep answering for float."""
+    from portdnn_amd.capi import DTYPE
+    for size, ch in [(56, 64), (28, 128), (14, 256), (7, 512)]:
+        p3 = ops.conv_params(128, size, size, ch, ch, 3, 1, True)
+        p1 = ops.conv_params(128, size, size, ch, 4 * ch, 1, 1, False)
+        fil3, fil1 = 9 * ch * ch, 4 * ch * ch
+        for d in range(3):
+            a32 = ops.default_algorithm(p3, d, DTYPE.F32)
+            assert a32 == ops.default_algorithm(p3, d) == ALGO.WINOGRAD
+            assert ops.workspace_size(p3, d, a32, DTYPE.F32) == \
+                ops.workspace_size(p3, d, a32)
+            a16 = ops.default_algorithm(p3, d, DTYPE.F16)
+            assert a16 in (ALGO.TILED, ALGO.IM2COL)
+            assert capi.lib().snn_hip_conv2d_algorithm_supports(
+                ctypes.byref(p3), d, a16) == a16
+            assert ops.default_algorithm(p1, d, DTYPE.F16) == ALGO.MATMUL
+            # every tag, Winograd included, reports the half kernels' need
+            for algo in (a16, ALGO.IM2COL, ALGO.WINOGRAD, ALGO.WINOGRAD_LARGE):
+                req, rec = ops.workspace_size(p3, d, algo, DTYPE.F16)
+                assert req == 0
+                if d == DIRECTION.FILTER_BACKPROP:
+                    assert 0 < rec <= 2 * 256 * fil3  # <= 256 fp32 partials
+                else:
+                    assert rec == fil3
+            req, rec = ops.workspace_size(p1, d, ALGO.MATMUL, DTYPE.F16)
+            assert req == 0
+            if d == DIRECTION.FILTER_BACKPROP:
+                assert 0 < rec <= 2 * 256 * fil1
+            else:
+                assert rec == 0      # W[c][k] is read in place
+        assert ops.workspace_size(p3, 0, ALGO.DIRECT, DTYPE.F16) == (0, 0)
+    req, rec = ctypes.c_size_t(), ctypes.c_size_t()
+    assert capi.lib().snn_hip_conv2d_workspace_size_for(
+        ctypes.byref(p3), 0, ALGO.IM2COL, 7, ctypes.byref(req),
+        ctypes.byref(rec)) == STATUS.INVALID_PARAMETER
+    assert capi.lib().snn_hip_conv2d_default_algorithm_for(
+        ctypes.byref(p3), 0, 7) == ALGO.NOT_SUPPORTED
+
+
 def test_kernel_timing_argument_checks():
     L = capi.lib()
     assert L.snn_hip_kernel_timing_read(None, None) == STATUS.INVALID_PARAMETER

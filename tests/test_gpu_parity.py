@@ -171,6 +171,45 @@ def test_config0_single_image_tiled():
 
 
 @pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, window, stride, same
+    (1, 56, 56, 64, 64, 3, 1, True),      # configuration 0
+    (1, 50, 50, 64, 64, 3, 1, True),      # pixel count not a multiple of 16
+    (2, 27, 29, 128, 128, 3, 1, True),    # two channel groups, two feature blocks
+    (4, 56, 56, 64, 64, 3, 2, True),      # stride 2 (asymmetric padding)
+    (1, 58, 58, 64, 128, 3, 1, False),    # VALID
+    (1, 56, 56, 64, 64, 1, 1, False),     # 1x1: a single step
+    (1, 52, 52, 64, 64, 5, 1, True),      # 25 taps: beyond its step limit
+])
+def test_small_problem_kernel(shape):
+    """Few-tile forward convolutions (below 128 tiles of 64x64) run on the
+    kernel whose waves split the reduction inside a work-group -- one launch,
+    no atomics -- through the Tiled and Im2col tags; the same with bias and
+    ReLU folded in; and twice, bit for bit (its additions have a fixed
+    order).  The last shape has too long a reduction for it and must still be
+    right on the kernels that take it instead."""
+    batch, rows, cols, ch, feats, window, stride, same = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, window, stride, same)
+    rng = np.random.default_rng(1500 + rows + ch + window)
+    n_in, n_fil, _ = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x, w = uniform(rng, n_in), uniform(rng, n_fil)
+    bias = uniform(rng, feats)
+    ref = oracle.conv2d_forward(x, w, oracle_params(p, feats), acc64=True)
+    dx, dw = dev(x), dev(w)
+    for algo in (ALGO.TILED, ALGO.IM2COL):
+        if not supported(p, DIRECTION.FORWARD, algo):
+            continue
+        got = ops.conv2d(dx, dw, p, DIRECTION.FORWARD, algo)
+        assert_close(got.cpu().numpy(), ref, ("small", ALGO_NAME[algo], shape))
+        if window != 5:
+            again = ops.conv2d(dx, dw, p, DIRECTION.FORWARD, algo)
+            assert torch.equal(got.view(torch.int32), again.view(torch.int32))
+        fused = ops.conv2d_bias_act(dx, dw, dev(bias), p, algo, relu=True)
+        want = np.maximum(ref.reshape(-1, feats) + bias.astype(np.float64), 0)
+        assert_close(fused.cpu().numpy(), want.reshape(-1),
+                     ("small + bias + relu", ALGO_NAME[algo], shape))
+
+
+@pytest.mark.parametrize("shape", [
     # ragged / edge shapes: odd sizes, C and K not multiples of the tiles,
     # non-square windows and strides, VALID padding
     (3, 13, 17, 5, 7, 3, 3, 1, 1, True),
@@ -315,7 +354,8 @@ def sampled_forward_reference(x, w, p, samples):
 
 @pytest.mark.parametrize("size,ch,window", [(56, 64, 3), (28, 128, 3),
                                             (14, 256, 3), (7, 512, 3),
-                                            (56, 64, 1), (7, 512, 1)])
+                                            (56, 64, 1), (28, 128, 1),
+                                            (14, 256, 1), (7, 512, 1)])
 def test_full_batch_forward_sampled_and_linear(size, ch, window):
     feats = ch if window == 3 else 4 * ch
     p = ops.conv_params(32, size, size, ch, feats, window, 1, window == 3)
@@ -582,6 +622,34 @@ def test_pooling_ragged(shape):
                  ("max grad", shape))
     assert_close(ops.pooling_avg_grad(dev(dy), p).cpu().numpy(),
                  oracle.pool_avg_grad(dy, op), ("avg grad", shape))
+
+
+@pytest.mark.parametrize("channels", [8, 6])
+def test_pooling_window_wholly_outside_the_image(channels):
+    """Output sizes larger than the input implies are not rejected (nor are
+    they by the reference's validation, include/portdnn/pooling/launch.h:56-88),
+    so the last output row and column here own windows that lie outside the
+    image on both axes.  Such a window has no elements: the reference's
+    operators leave Max at lowest() and divide 0 by 0 for Average
+    (src/pooling/operators_impl.h:27-87).  Eight channels take the kernel that
+    deals window taps to lanes (16 taps), six the generic one."""
+    p = ops.pool_params(2, 7, 7, channels, 4, 4, False)
+    p.out_rows = p.out_cols = 3      # third window starts at row / column 8
+    op = oracle_params(p, 0)
+    rng = np.random.default_rng(77 + channels)
+    x = rng.standard_normal(2 * 7 * 7 * channels).astype(np.float32)
+    got = ops.pooling_forward(dev(x), p, POOL_OP.MAX).cpu().numpy()
+    ref = oracle.pool_max_forward(x, op)
+    assert np.array_equal(got, ref)
+    assert ref.reshape(2, 3, 3, channels)[0, 2, 2, 0] == \
+        np.finfo(np.float32).min
+    got = ops.pooling_forward(dev(x), p, POOL_OP.AVERAGE).cpu().numpy()
+    with np.errstate(invalid="ignore"):
+        ref = oracle.pool_avg_forward(x, op)
+    assert np.isnan(ref.reshape(2, 3, 3, channels)[:, 2, :, :]).all()
+    assert np.array_equal(np.isnan(got), np.isnan(ref))
+    ok = ~np.isnan(ref)
+    assert_close(got[ok], ref[ok], "avg outside")
 
 
 @pytest.mark.parametrize("shape", [

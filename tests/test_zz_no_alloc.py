@@ -54,9 +54,32 @@ CALLS = [(32, 56, 56, 256, 1), (32, 56, 56, 128, 1), (20, 55, 57, 128, 2),
          (24, 112, 112, 32, 1), (11, 111, 109, 64, 2), (4, 56, 56, 128, 2)]
 
 
+def temporary_memory(reset):
+    reserved, high = ctypes.c_ulonglong(), ctypes.c_ulonglong()
+    capi.check(capi.lib().snn_hip_temporary_memory_stats(
+        ctypes.byref(reserved), ctypes.byref(high), 1 if reset else 0))
+    return reserved.value, high.value
+
+
 def test_noalloc_filter_backprop_matches_allocating_entry():
     rng = np.random.default_rng(0x5EED + 77)
     pending = []
+    # Nothing may come out of the pools stream-ordered temporaries are taken
+    # from while the entry point runs: clear their high-water marks, and make
+    # sure the check can see a temporary at all (the allocating entry on the
+    # first shape takes one).
+    warm = ops.depthwise_params(*CALLS[0][:4], 1, 3, CALLS[0][4], True)
+    wx = torch.zeros(warm.batch * warm.in_rows * warm.in_cols * warm.channels,
+                     device="cuda")
+    wdy = torch.zeros(warm.batch * warm.out_rows * warm.out_cols *
+                      warm.channels, device="cuda")
+    ops.depthwise_conv2d(wx, wdy, warm, DIRECTION.FILTER_BACKPROP)
+    torch.cuda.synchronize()
+    assert temporary_memory(reset=True)[1] > 0
+    del wx, wdy
+    torch.cuda.synchronize()
+    temporary_memory(reset=True)
+    reserved_before, high_before = temporary_memory(reset=False)
     # every call is enqueued before any result is read, so the calls really
     # run in a row on the stream and share the scratch array
     for batch, rows, cols, ch, stride in CALLS:
@@ -68,6 +91,10 @@ def test_noalloc_filter_backprop_matches_allocating_entry():
         got = noalloc(dx, ddy, p)
         pending.append((p, x, dy, dx, ddy, got))
     torch.cuda.synchronize()
+    reserved_after, used_high = temporary_memory(reset=False)
+    assert used_high == high_before and reserved_after == reserved_before, (
+        "the no-allocation entry took a temporary", high_before, used_high,
+        reserved_before, reserved_after)
     for p, x, dy, dx, ddy, got in pending:
         want = ops.depthwise_conv2d(dx, ddy, p, DIRECTION.FILTER_BACKPROP)
         assert_close(got.cpu().numpy(), want.cpu().numpy(),
