@@ -376,6 +376,52 @@ SNNStatus launch_forward_bias_activation(
       stream);
 }
 
+// Not in portDNN, whose Winograd launch transforms the filter every time: a
+// launch in two calls for callers that run many launches with one filter.
+// prepare_filter writes what the selected algorithm derives from the filter
+// alone into the workspace (nothing, for most paths); launch_prepared is
+// launch<float, ConvType> trusting those contents.  The caller keeps the
+// workspace untouched in between and passes the same filter, parameters and
+// selector to both.
+template <typename T, typename ConvType, typename Backend>
+SNNStatus prepare_filter(
+    typename Backend::template pointer_type<T const> filter,
+    Conv2DParams const& params, Selector& selector, Backend& backend,
+    typename Backend::template pointer_type<T> workspace,
+    size_t workspace_size, const std::vector<hip::Event>& events = {}) {
+  static_assert(std::is_same<T, float>::value,
+                "prepare_filter is provided for float");
+  const snn_hip_conv2d_params c = internal::to_c(params);
+  const Algorithm algo = selector.select<ConvType>(params);
+  hipStream_t stream = backend.get_stream();
+  hip::detail::wait_for(stream, events);
+  return hip::detail::finish(
+      snn_hip_conv2d_prepare_filter_f32(
+          internal::Direction<ConvType>::value, filter, &c,
+          static_cast<int>(algo), workspace, workspace_size, stream),
+      stream);
+}
+template <typename T, typename ConvType, typename Backend>
+SNNStatus launch_prepared(
+    typename Backend::template pointer_type<T const> input,
+    typename Backend::template pointer_type<T const> filter,
+    typename Backend::template pointer_type<T> output,
+    Conv2DParams const& params, Selector& selector, Backend& backend,
+    typename Backend::template pointer_type<T> workspace,
+    size_t workspace_size, const std::vector<hip::Event>& events = {}) {
+  static_assert(std::is_same<T, float>::value,
+                "launch_prepared is provided for float");
+  const snn_hip_conv2d_params c = internal::to_c(params);
+  const Algorithm algo = selector.select<ConvType>(params);
+  hipStream_t stream = backend.get_stream();
+  hip::detail::wait_for(stream, events);
+  return hip::detail::finish(
+      snn_hip_conv2d_prepared_f32(internal::Direction<ConvType>::value, input,
+                                  filter, output, &c, static_cast<int>(algo),
+                                  workspace, workspace_size, stream),
+      stream);
+}
+
 // Not in portDNN, whose kernels always add in one fixed order: the same
 // convolution as launch<float, ConvType> with run-to-run bit-identical
 // results (no reduction split across work-groups, whose partial sums would

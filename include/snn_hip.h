@@ -248,6 +248,29 @@ SNN_HIP_API int snn_hip_conv2d_deterministic_f32(
     const snn_hip_conv2d_params* params, int algorithm, float* workspace,
     size_t workspace_elems, void* stream);
 
+/* A launch in two calls, for callers that run many launches with one filter
+ * (inference).  No counterpart in portDNN, whose Winograd launch transforms
+ * the filter every time (internal/conv2d/winograd/launch.h:212-235).
+ *
+ * snn_hip_conv2d_prepare_filter_f32 writes into `workspace` whatever a launch
+ * with these parameters, direction and algorithm derives from the filter
+ * alone -- today the transformed filter of the fused Winograd forward /
+ * input-gradient kernels; for every other path it does nothing and returns
+ * SNN_HIP_OK.  snn_hip_conv2d_prepared_f32 is then the same operation as the
+ * three fp32 entry points, except that it trusts those contents instead of
+ * recomputing them: the caller guarantees that `workspace` (same pointer,
+ * same size) still holds what a prepare call with the same filter values,
+ * parameters, direction and algorithm wrote, and that nothing else wrote to
+ * its first 16 * C * K elements since.  The one-call entry points never
+ * trust a workspace: they always transform the filter they are given. */
+SNN_HIP_API int snn_hip_conv2d_prepare_filter_f32(
+    int direction, const float* filter, const snn_hip_conv2d_params* params,
+    int algorithm, float* workspace, size_t workspace_elems, void* stream);
+SNN_HIP_API int snn_hip_conv2d_prepared_f32(
+    int direction, const float* input, const float* filter, float* output,
+    const snn_hip_conv2d_params* params, int algorithm, float* workspace,
+    size_t workspace_elems, void* stream);
+
 /* sycldnn::conv2d::query_workspace_size<ConvType>(params, selector)
  * (include/portdnn/conv2d/workspace_size.h:158-163) for an already selected
  * algorithm.  Sizes in elements. */

@@ -129,6 +129,8 @@ SIGNATURES = {
     "snn_hip_conv2d_forward_bias_act_f32": [_P, _P, _P, _P, _P, _I, _I, _P,
                                             _SZ, _P],
     "snn_hip_conv2d_deterministic_f32": [_I, _P, _P, _P, _P, _I, _P, _SZ, _P],
+    "snn_hip_conv2d_prepare_filter_f32": [_I, _P, _P, _I, _P, _SZ, _P],
+    "snn_hip_conv2d_prepared_f32": [_I, _P, _P, _P, _P, _I, _P, _SZ, _P],
     "snn_hip_conv2d_workspace_size": [_P, _I, _I, ctypes.POINTER(_SZ),
                                       ctypes.POINTER(_SZ)],
     "snn_hip_conv2d_algorithm_supports": [_P, _I, _I],

@@ -812,8 +812,9 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
                            g.tile_cols * (g.in_ch + g.out_ch);
   if (workspace == nullptr || workspace_elems < u_elems + per_image)
     return SNN_HIP_INSUFFICIENT_WORKSPACE;
-  if (!aligned16(workspace) || !aligned16(input) || !aligned16(output) ||
-      (backprop && !aligned16(filter)))
+  const bool prepare_only = epilogue != nullptr && epilogue->prepare_only;
+  if (!aligned16(workspace) || (backprop && !aligned16(filter)) ||
+      (!prepare_only && (!aligned16(input) || !aligned16(output))))
     return SNN_HIP_INVALID_PARAMETER;
   const size_t in_elems = static_cast<size_t>(p.batch) * g.in_rows *
                           g.in_cols * g.in_ch;
@@ -880,10 +881,20 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
   // even number of chunks; it wants U with the channels of a chunk dealt to
   // the lane halves eight at a time.
   const bool persistent = splits == 1 && n_chunks % 2 == 0;
-  hipLaunchKernelGGL(wino_filter_pack_kernel,
-                     dim3(ceil_div((g.in_ch / 4) * g.out_ch, 256)), dim3(256),
-                     0, stream, filter, workspace, p.channels, p.features,
-                     backprop, persistent);
+  // The transformed filter depends on the filter and on this launch plan
+  // only.  A caller that runs many launches with one filter may have it
+  // written once (prepare_only) and then launch with filter_prepared, which
+  // trusts what the workspace holds.
+  const bool prepared = epilogue != nullptr && epilogue->filter_prepared;
+  if (!prepared)
+    hipLaunchKernelGGL(wino_filter_pack_kernel,
+                       dim3(ceil_div((g.in_ch / 4) * g.out_ch, 256)),
+                       dim3(256), 0, stream, filter, workspace, p.channels,
+                       p.features, backprop, persistent);
+  if (epilogue != nullptr && epilogue->prepare_only) {
+    SNN_HIP_CHECK_LAUNCH();
+    return SNN_HIP_OK;
+  }
   if (splits > 1) {
     const size_t n_vec = out_elems / 4;  // out_ch % 32 == 0
     hipLaunchKernelGGL(wino_zero_fill_kernel,

@@ -835,6 +835,53 @@ int snn_hip_conv2d_deterministic_f32(int direction, const float* input,
                                 &options);
 }
 
+int snn_hip_conv2d_prepare_filter_f32(int direction, const float* filter,
+                                      const snn_hip_conv2d_params* params,
+                                      int algorithm, float* workspace,
+                                      size_t workspace_elems, void* stream) {
+  if (params == nullptr || filter == nullptr)
+    return SNN_HIP_INVALID_PARAMETER;
+  if (direction < SNN_HIP_FORWARD || direction > SNN_HIP_FILTER_BACKPROP)
+    return SNN_HIP_INVALID_PARAMETER;
+  const snn_hip_conv2d_params& p = *params;
+  const int v = validate(p);
+  if (v != SNN_HIP_OK) return v;
+  if (p.groups != 1 || p.filter_format == 2) return SNN_HIP_INVALID_ALGORITHM;
+  if (algorithm_supports(p, direction, algorithm) == SNN_HIP_ALGO_NOT_SUPPORTED)
+    return SNN_HIP_INVALID_ALGORITHM;
+  // Only the fused Winograd forward / input-gradient kernels keep anything
+  // derived from the filter alone; every other path has nothing to prepare.
+  if ((algorithm != SNN_HIP_ALGO_WINOGRAD &&
+       algorithm != SNN_HIP_ALGO_WINOGRAD_LARGE) ||
+      direction == SNN_HIP_FILTER_BACKPROP || p.input_format != 0 ||
+      !conv2d_winograd_fused_supports(direction, p))
+    return SNN_HIP_OK;
+  size_t required = 0, recommended = 0;
+  workspace_size(p, direction, algorithm, SNN_HIP_DTYPE_F32, &required,
+                 &recommended);
+  if (workspace == nullptr || workspace_elems < required)
+    return SNN_HIP_INSUFFICIENT_WORKSPACE;
+  LaunchOptions options;
+  options.prepare_only = true;
+  return launch_conv2d_winograd_fused_f32(direction, nullptr, filter, nullptr,
+                                          p, workspace, workspace_elems,
+                                          as_stream(stream), &options);
+}
+
+int snn_hip_conv2d_prepared_f32(int direction, const float* input,
+                                const float* filter, float* output,
+                                const snn_hip_conv2d_params* params,
+                                int algorithm, float* workspace,
+                                size_t workspace_elems, void* stream) {
+  if (direction < SNN_HIP_FORWARD || direction > SNN_HIP_FILTER_BACKPROP)
+    return SNN_HIP_INVALID_PARAMETER;
+  LaunchOptions options;
+  options.filter_prepared = true;
+  return conv2d_dispatch<float>(direction, input, filter, output, params,
+                                algorithm, workspace, workspace_elems, stream,
+                                &options);
+}
+
 int snn_hip_conv2d_workspace_size(const snn_hip_conv2d_params* params,
                                   int direction, int algorithm,
                                   size_t* required_elems,

@@ -25,6 +25,13 @@ struct LaunchOptions {
   bool relu = false;
   bool* applied = nullptr;
   bool deterministic = false;
+  //  * prepare_only: write whatever the launch derives from the filter alone
+  //    (the fused Winograd kernels' transformed filter) into the workspace
+  //    and launch nothing else; filter_prepared: the workspace already holds
+  //    it, from a prepare_only call with the same filter, parameters,
+  //    direction and algorithm.  Launchers with nothing to prepare ignore both.
+  bool prepare_only = false;
+  bool filter_prepared = false;
   bool wanted() const { return bias != nullptr || relu; }
 };
 

@@ -148,6 +148,27 @@ def conv2d(inp, fil, p, direction=DIRECTION.FORWARD, algorithm=ALGO.DIRECT,
     return out
 
 
+def conv2d_prepare_filter(fil, p, direction, algorithm, workspace):
+    """snn_hip_conv2d_prepare_filter_f32: what the launch derives from the
+    filter alone goes into `workspace`."""
+    capi.check(capi.lib().snn_hip_conv2d_prepare_filter_f32(
+        direction, _ptr(fil), ctypes.byref(p), algorithm, _ptr(workspace),
+        0 if workspace is None else workspace.numel(), _stream()))
+
+
+def conv2d_prepared(inp, fil, p, direction, algorithm, workspace, out=None):
+    """snn_hip_conv2d_prepared_f32: the launch that trusts a prepared
+    workspace."""
+    _, _, n_out = conv_sizes(p, direction)
+    if out is None:
+        out = torch.empty(n_out, dtype=inp.dtype, device=inp.device)
+    capi.check(capi.lib().snn_hip_conv2d_prepared_f32(
+        direction, _ptr(inp), _ptr(fil), _ptr(out), ctypes.byref(p), algorithm,
+        _ptr(workspace), 0 if workspace is None else workspace.numel(),
+        _stream()))
+    return out
+
+
 def conv2d_deterministic(inp, fil, p, direction, algorithm, workspace=None,
                          out=None):
     """snn_hip_conv2d_deterministic_f32: fixed order of additions."""
@@ -315,7 +336,7 @@ __all__ = [
     "ALGO", "BINARY_OP", "DIRECTION", "POINTWISE_OP", "POOL_OP", "STATUS",
     "ConvParams", "DepthwiseParams", "PoolParams", "add_padding_to",
     "binaryop", "binaryop_raw", "calculate_padding", "conv2d",
-    "conv2d_bias_act",
+    "conv2d_bias_act", "conv2d_prepare_filter", "conv2d_prepared",
     "conv2d_raw", "conv_flops", "conv_params", "conv_sizes",
     "default_algorithm",
     "depthwise_conv2d", "depthwise_params", "depthwise_sizes", "matmul",

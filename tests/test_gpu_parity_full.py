@@ -421,6 +421,56 @@ def test_f16_default_selector_with_exactly_the_queried_workspace(size, ch,
             del block
 
 
+@pytest.mark.parametrize("direction", [DIRECTION.FORWARD,
+                                       DIRECTION.INPUT_BACKPROP])
+@pytest.mark.parametrize("batch,size,ch", [(32, 14, 256), (4, 28, 128),
+                                           (2, 20, 24)])
+def test_prepared_filter_two_call_form(batch, size, ch, direction):
+    """prepare_filter + prepared launch equals the one-call launch bit for bit
+    (the same kernels run, minus the filter transform), for several inputs on
+    one prepared workspace; and the one-call form never trusts what a
+    workspace holds: after preparing filter A, a one-call launch with filter B
+    in the same workspace gives B's result.  (2, 20, 24) is off the fused
+    kernel's channel multiples: nothing is prepared and the prepared launch is
+    an ordinary one.)"""
+    p = ops.conv_params(batch, size, size, ch, ch, 3, 1, True)
+    rng = np.random.default_rng(4100 + size + direction)
+    n_a, n_b, n_out = ops.conv_sizes(p, direction)
+    wa, wb = dev(uniform(rng, n_b)), dev(uniform(rng, n_b))
+    _, rec = ops.workspace_size(p, direction, ALGO.WINOGRAD)
+    ws = torch.empty(rec, dtype=torch.float32, device="cuda")
+    ops.conv2d_prepare_filter(wa, p, direction, ALGO.WINOGRAD, ws)
+    for _ in range(3):
+        x = dev(uniform(rng, n_a))
+        got = ops.conv2d_prepared(x, wa, p, direction, ALGO.WINOGRAD, ws)
+        fresh = torch.empty(rec, dtype=torch.float32, device="cuda")
+        want = ops.conv2d(x, wa, p, direction, ALGO.WINOGRAD, workspace=fresh)
+        if batch * size * size >= 4096:   # no reduction split: same bits
+            assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+        else:
+            assert_close(got.cpu().numpy(), want.cpu().numpy().astype(
+                np.float64), "prepared vs one call")
+    # stale contents: the workspace holds U(A); the one-call form with B
+    x = uniform(rng, n_a)
+    got = ops.conv2d(dev(x), wb, p, direction, ALGO.WINOGRAD, workspace=ws)
+    ref = ORACLE_FN[direction](x, wb.cpu().numpy(), oracle_params(p, ch),
+                               acc64=True)
+    assert_close(got.cpu().numpy(), ref, "one call after a prepare of another "
+                 "filter")
+    # nothing to prepare for a filter gradient or another algorithm: no-ops
+    ops.conv2d_prepare_filter(wa, p, DIRECTION.FILTER_BACKPROP, ALGO.WINOGRAD,
+                              ws)
+    ops.conv2d_prepare_filter(wa, p, direction, ALGO.IM2COL, None)
+    got = ops.conv2d_prepared(dev(x), wb, p, direction, ALGO.IM2COL, None)
+    assert_close(got.cpu().numpy(), ref, "prepared launch, nothing prepared")
+    small = torch.empty(8, dtype=torch.float32, device="cuda")
+    if ch % 32 == 0:
+        assert capi.lib().snn_hip_conv2d_prepare_filter_f32(
+            direction, ctypes.c_void_p(wa.data_ptr()), ctypes.byref(p),
+            ALGO.WINOGRAD, ctypes.c_void_p(small.data_ptr()), 8, None) == \
+            STATUS.INSUFFICIENT_WORKSPACE
+
+
 # ---- reproducible launches ----------------------------------------------------
 
 @pytest.mark.parametrize("case", [
