@@ -186,6 +186,32 @@ def main():
     ms_per_step = elapsed * 1e3 / args.steps
     value = total_flops / (elapsed / args.steps) / 1e12
 
+    # The same step with the filters prepared once, outside the timed region
+    # (snn_hip_conv2d_prepare_filter_f32 + snn_hip_conv2d_prepared_f32: the
+    # inference case, one filter for many launches).  Reported beside `value`,
+    # which stays the one-call form that transforms the filter in every launch.
+    for w in work:
+        if w["ws"] is not None:
+            ops.conv2d_prepare_filter(w["w"], w["p"], DIRECTION.FORWARD,
+                                      w["algo"], w["ws"])
+
+    def step_prepared():
+        for w in work:
+            if w["ws"] is not None:
+                ops.conv2d_prepared(w["x"], w["w"], w["p"], DIRECTION.FORWARD,
+                                    w["algo"], w["ws"], out=w["y"])
+            else:
+                ops.conv2d(w["x"], w["w"], w["p"], DIRECTION.FORWARD,
+                           w["algo"], out=w["y"])
+    for _ in range(args.warmup):
+        step_prepared()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step_prepared()
+    torch.cuda.synchronize()
+    prepared_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
     # ---- roofline: the dominant kernel, HIP events on the launch stream -------
     # The library brackets the main kernel of each convolution launch (not the
     # filter preparation in front of it) with events on the stream it launches
@@ -248,6 +274,11 @@ def main():
         "step_executed_frac": frac(
             executed_flops_per_step / ms_per_step / 1e9,
             PEAK_FP32_MFMA_TFLOPS),
+        # the step with every filter transformed once beforehand (two-call
+        # form); `value` is the one-call form
+        "step_filter_prepared_ms": round(prepared_ms, 4),
+        "step_filter_prepared_tflops": round(
+            total_flops / prepared_ms / 1e9, 3),
         # not measured in this run: FETCH_SIZE / WRITE_SIZE of the same kernel
         # from the committed rocprofv3 summary
         "traffic": (profiled_traffic_bytes("wino_direct_kernel")

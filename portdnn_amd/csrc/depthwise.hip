@@ -10,6 +10,7 @@
 // contiguous 1 KiB (512 B for f16) run of the NHWC row -- fully coalesced --
 // and the window taps of neighbouring lanes/pixels are served from L1/L2.
 // Everything else goes through the scalar kernel.
+#include <cstdio>
 #include <cstdlib>
 #include <mutex>
 #include <string>
@@ -277,6 +278,180 @@ __global__ void __launch_bounds__(256)
               ? static_cast<unsigned>(out_base + (t * p.out_cols + u) * C) * kEsz
               : kOobOffset;
       BufVecN<T, V>::store(out_rsrc, off, acc[t][u]);
+    }
+  }
+}
+
+// Forward 3x3, multiplier == 1, fp32, C = 4 * CV with CV in {8, 16, 32}: tall
+// strips in which every input vector is loaded by exactly one lane.
+//
+// The strip kernel above re-loads the window columns its neighbours own (3.0
+// vector loads per output at 4 x 2) and leaves the cache to serve them.  Here
+// a wave is 64 / CV pixel lanes x CV channel vectors; a lane owns TW
+// consecutive output pixels, i.e. STRIDE * TW consecutive input columns (its
+// "own" columns: the window centres for stride 1, the first two window
+// columns for stride 2), loads only those, and takes the one column to the
+// left (stride 1) and to the right of its own range from the neighbouring
+// pixel lanes with a cross-lane read (ds_bpermute: the LDS crossbar, no LDS
+// memory).  Only the first and last pixel lane of a wave load a halo column
+// themselves.  A strip is TH output rows tall and walks down its input rows
+// with three (stride 1) or two (stride 2) rows of running sums, storing an
+// output row as soon as its third filter row has been added, so the rows that
+// two strips share are 2 in TH * STRIDE + 2.  The rows a strip owns are read
+// with streaming loads (nobody else reads them); its two halo rows and the
+// wave-edge halo columns, which other lanes own, with ordinary ones.
+// Work-groups are not remapped to XCDs: consecutive groups then stream
+// consecutive runs of the tensor on all XCDs together.  Per output the taps
+// are still accumulated in filter-row, filter-column order.
+template <int STRIDE, int TH, int TW, int CV, bool FLIP>
+__global__ void __launch_bounds__(256)
+    dw_forward_3x3_tall_kernel(const float* __restrict__ in,
+                               const float* __restrict__ fil,
+                               float* __restrict__ out,
+                               snn_hip_depthwise_params p, int n_strips,
+                               int n_wcols, unsigned n_waves) {
+  constexpr int PXW = 64 / CV;          // pixel lanes per wave
+  constexpr int OWN = STRIDE * TW;      // own input columns per lane
+  constexpr int A = STRIDE == 1 ? 1 : 0;  // own range starts A columns right of
+                                          // the first window column
+  constexpr int NR = (TH - 1) * STRIDE + 3;
+  constexpr int LIVE = STRIDE == 1 ? 3 : 2;  // output rows with open sums
+  constexpr int kNt = 2;                // streaming (nt) load
+  const unsigned w = blockIdx.x * 4u + (threadIdx.x >> 6);
+  if (w >= n_waves) return;  // whole waves only: the cross-lane reads below
+                             // need every lane of a live wave
+  const int lane = threadIdx.x & 63;
+  const int cvi = lane % CV, pl = lane / CV;
+  const int wcol = static_cast<int>(w % static_cast<unsigned>(n_wcols));
+  const unsigned rest = w / static_cast<unsigned>(n_wcols);
+  const int strip = static_cast<int>(rest % static_cast<unsigned>(n_strips));
+  const int n = static_cast<int>(rest / static_cast<unsigned>(n_strips));
+  const int C = p.channels, c = cvi * 4;
+  const size_t in_elems =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * C;
+  const size_t out_elems =
+      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * C;
+  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_elems * 4);
+  const __amdgpu_buffer_rsrc_t fil_rsrc =
+      make_rsrc(fil, static_cast<size_t>(9) * C * 4);
+  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_elems * 4);
+  float f[9][4];
+#pragma unroll
+  for (int t = 0; t < 9; ++t)
+    BufVec4<float>::load(fil_rsrc,
+                         static_cast<unsigned>((FLIP ? 8 - t : t) * C + c) * 4u,
+                         f[t]);
+  const int oy0 = strip * TH;
+  const int ox0 = (wcol * PXW + pl) * TW;  // first own output pixel
+  const int col0 = STRIDE * ox0 - p.pad_cols + A;  // first own input column
+  const int y0 = STRIDE * oy0 - p.pad_rows;        // first input row
+  // the wave's halo columns, loaded by its first / last pixel lane only
+  const int xl = STRIDE * (wcol * PXW * TW) - p.pad_cols + A - 1;
+  const int xr = STRIDE * ((wcol + 1) * PXW * TW) - p.pad_cols + A;
+  const bool first = pl == 0, last = pl == PXW - 1;
+  const bool l_ok = STRIDE == 1 && first &&
+                    static_cast<unsigned>(xl) < static_cast<unsigned>(p.in_cols);
+  const bool r_ok =
+      last && static_cast<unsigned>(xr) < static_cast<unsigned>(p.in_cols);
+  bool own_ok[OWN];
+#pragma unroll
+  for (int k = 0; k < OWN; ++k)
+    own_ok[k] = static_cast<unsigned>(col0 + k) <
+                static_cast<unsigned>(p.in_cols);
+  // element offset of (n, y0, column 0, c)
+  const int row0 = (n * p.in_rows + y0) * p.in_cols * C + c;
+  const int rstride = p.in_cols * C;
+  const int src_l = (lane - CV) * 4, src_r = (lane + CV) * 4;
+
+  float own[NR][OWN][4], hl[NR][4], hr[NR][4];
+#pragma unroll
+  for (int j = 0; j < NR; ++j) {
+    const bool row_ok =
+        static_cast<unsigned>(y0 + j) < static_cast<unsigned>(p.in_rows);
+    // rows A .. A + STRIDE * TH - 1 of the strip are read by this strip only
+    const bool mine = j >= A && j < A + STRIDE * TH;
+#pragma unroll
+    for (int k = 0; k < OWN; ++k) {
+      const unsigned off =
+          (row_ok && own_ok[k])
+              ? static_cast<unsigned>(row0 + j * rstride + (col0 + k) * C) * 4u
+              : kOobOffset;
+      const float4 t = __builtin_bit_cast(
+          float4, mine ? __builtin_amdgcn_raw_buffer_load_b128(in_rsrc, off, 0,
+                                                               kNt)
+                       : __builtin_amdgcn_raw_buffer_load_b128(in_rsrc, off, 0,
+                                                               0));
+      own[j][k][0] = t.x; own[j][k][1] = t.y;
+      own[j][k][2] = t.z; own[j][k][3] = t.w;
+    }
+    if (STRIDE == 1)
+      BufVec4<float>::load(
+          in_rsrc,
+          (row_ok && l_ok)
+              ? static_cast<unsigned>(row0 + j * rstride + xl * C) * 4u
+              : kOobOffset,
+          hl[j]);
+    BufVec4<float>::load(
+        in_rsrc,
+        (row_ok && r_ok)
+            ? static_cast<unsigned>(row0 + j * rstride + xr * C) * 4u
+            : kOobOffset,
+        hr[j]);
+  }
+
+  float acc[LIVE][TW][4];
+#pragma unroll
+  for (int j = 0; j < NR; ++j) {
+    // win[k + 1] is input column col0 + k, k = -1 .. OWN
+    float win[OWN + 2][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (STRIDE == 1) {
+        const float from_left = __builtin_bit_cast(
+            float, __builtin_amdgcn_ds_bpermute(
+                       src_l, __builtin_bit_cast(int, own[j][OWN - 1][i])));
+        win[0][i] = first ? hl[j][i] : from_left;
+      } else {
+        win[0][i] = 0.f;
+      }
+      const float from_right = __builtin_bit_cast(
+          float, __builtin_amdgcn_ds_bpermute(
+                     src_r, __builtin_bit_cast(int, own[j][0][i])));
+      win[OWN + 1][i] = last ? hr[j][i] : from_right;
+#pragma unroll
+      for (int k = 0; k < OWN; ++k) win[k + 1][i] = own[j][k][i];
+    }
+    // input row j is filter row r of output row t = (j - r) / STRIDE; the
+    // older output row first
+#pragma unroll
+    for (int r = 2; r >= 0; --r) {
+      if (j - r < 0 || (j - r) % STRIDE != 0) continue;
+      const int t = (j - r) / STRIDE;
+      if (t >= TH) continue;
+#pragma unroll
+      for (int u = 0; u < TW; ++u) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float a = r == 0 ? 0.f : acc[t % LIVE][u][i];
+#pragma unroll
+          for (int sx = 0; sx < 3; ++sx)
+            a = fmaf(win[STRIDE * u + sx - A + 1][i], f[r * 3 + sx][i], a);
+          acc[t % LIVE][u][i] = a;
+        }
+      }
+      if (r == 2) {
+#pragma unroll
+        for (int u = 0; u < TW; ++u) {
+          const bool ok = oy0 + t < p.out_rows && ox0 + u < p.out_cols;
+          BufVec4<float>::store(
+              out_rsrc,
+              ok ? static_cast<unsigned>(
+                       ((n * p.out_rows + oy0 + t) * p.out_cols + ox0 + u) * C +
+                       c) * 4u
+                 : kOobOffset,
+              acc[t % LIVE][u]);
+        }
+      }
     }
   }
 }
@@ -869,10 +1044,81 @@ __global__ void __launch_bounds__(kStrip* kSlices)
 //   stride 1: TW = 2 once a pixel's channel vectors fill a 128-byte line,
 //             TH = 4 for images of 28 rows and more, else 8 (4 with V = 8);
 //   stride 2: TW = 1, TH = 2 for outputs of 56 rows and more, else 8 (4).
+// The tall-strip kernel for the shapes it is built for: fp32, 32 / 64 / 128
+// channels, strips of 14 x 4 outputs per lane at stride 1 and 7 x 1 at stride
+// 2, enough waves to cover the GPU (smaller launches keep the short strips,
+// whose many lanes hide latency better).  Returns false when it does not take
+// the launch.
+template <bool FLIP>
+bool launch_dw_tall(const float* input, const float* filter, float* output,
+                    const snn_hip_depthwise_params& p, hipStream_t stream) {
+  const int cv = p.channels / 4;
+  if (cv != 8 && cv != 16 && cv != 32) return false;
+  if (p.pad_rows > 2 || p.pad_cols > 2) return false;
+  const int stride = p.stride_rows;
+  int th = stride == 1 ? 14 : 7, tw = stride == 1 ? 4 : 1;
+  // Developer overrides for tuning runs: SNN_HIP_DW_TALL=<th>x<tw> among the
+  // shapes instantiated below.
+  if (const char* tune = SNN_TUNING_ENV("SNN_HIP_DW_TALL")) {
+    int a = 0, b = 0;
+    if (sscanf(tune, "%dx%d", &a, &b) == 2) {
+      th = a;
+      tw = b;
+    }
+  }
+  if (p.out_rows < th) return false;
+  const int wpx = (64 / cv) * tw;
+  const int n_wcols = ceil_div(p.out_cols, wpx);
+  const int n_strips = ceil_div(p.out_rows, th);
+  const size_t waves = static_cast<size_t>(p.batch) * n_strips * n_wcols;
+  // ragged last wave column: at most a quarter of its lanes idle overall
+  if (static_cast<size_t>(n_wcols) * wpx * 4 > static_cast<size_t>(p.out_cols) * 5)
+    return false;
+  if (waves < 768 || waves > 0x3FFFFFFFu) return false;
+  const unsigned n_waves = static_cast<unsigned>(waves);
+  const dim3 grid(ceil_div(n_waves, 4u));
+#define SNN_DW_TALL(STRIDE, TH, TW, CV)                                       \
+  hipLaunchKernelGGL((dw_forward_3x3_tall_kernel<STRIDE, TH, TW, CV, FLIP>),  \
+                     grid, dim3(256), 0, stream, input, filter, output, p,    \
+                     n_strips, n_wcols, n_waves)
+#define SNN_DW_TALL_CV(STRIDE, TH, TW)               \
+  do {                                               \
+    if (cv == 8) SNN_DW_TALL(STRIDE, TH, TW, 8);     \
+    else if (cv == 16) SNN_DW_TALL(STRIDE, TH, TW, 16); \
+    else SNN_DW_TALL(STRIDE, TH, TW, 32);            \
+  } while (0)
+  if (stride == 1) {
+    if (th == 14 && tw == 4) SNN_DW_TALL_CV(1, 14, 4);
+#ifdef SNN_HIP_TUNING
+    else if (th == 14 && tw == 2) SNN_DW_TALL_CV(1, 14, 2);
+    else if (th == 7 && tw == 4) SNN_DW_TALL_CV(1, 7, 4);
+    else if (th == 8 && tw == 4) SNN_DW_TALL_CV(1, 8, 4);
+#endif
+    else return false;
+  } else {
+    if (th == 7 && tw == 1) SNN_DW_TALL_CV(2, 7, 1);
+#ifdef SNN_HIP_TUNING
+    else if (th == 7 && tw == 2) SNN_DW_TALL_CV(2, 7, 2);
+    else if (th == 4 && tw == 2) SNN_DW_TALL_CV(2, 4, 2);
+    else if (th == 4 && tw == 1) SNN_DW_TALL_CV(2, 4, 1);
+    else if (th == 14 && tw == 1) SNN_DW_TALL_CV(2, 14, 1);
+#endif
+    else return false;
+  }
+#undef SNN_DW_TALL_CV
+#undef SNN_DW_TALL
+  return true;
+}
+
 template <typename T, int V, bool FLIP>
 void launch_dw_strip(const T* input, const T* filter, T* output,
                      const snn_hip_depthwise_params& p, hipStream_t stream) {
   constexpr int kBlock = 256;
+  if constexpr (std::is_same<T, float>::value && V == 4) {
+    if (SNN_TUNING_ENV("SNN_HIP_DW_TALL_OFF") == nullptr &&
+        launch_dw_tall<FLIP>(input, filter, output, p, stream))
+      return;
+  }
   const int cv = p.channels / V;
   const int th_max = V == 8 ? 4 : 8;  // 8 rows x 8 channels: ~250 registers
   int th, tw;

@@ -295,6 +295,151 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// ---- 3x3 stride-2 forward, fp32, tall strips --------------------------------
+// C = 4 * CV with CV in {8, 16, 32}.  A wave is 64 / CV pixel lanes x CV
+// channel vectors; a lane owns one output pixel, i.e. the first two columns of
+// its window, loads only those, and takes the third column -- the first
+// column of the pixel lane to its right -- with a cross-lane read
+// (ds_bpermute: the LDS crossbar, no LDS memory).  Only the last pixel lane of
+// a wave loads that column itself.  A strip is TH output rows tall: it walks
+// down 2 TH + 1 input rows with two rows of open windows and stores an output
+// row as soon as its third window row has been folded in, so two strips share
+// one input row in 2 TH + 1.  Rows the strip owns are read with streaming
+// loads, the shared row and the wave-edge column with ordinary ones;
+// work-groups are not remapped to XCDs, so consecutive groups stream
+// consecutive runs of the tensor on all XCDs together.  Taps outside the
+// image never enter a maximum (they are replaced by lowest()) and read as
+// zero for the average, whose divisor is the in-image element count; the
+// window is scanned row-major as in src/pooling/kernels.h:61-99.
+template <typename Op, int TH, int CV>
+__global__ void __launch_bounds__(256)
+    pool_forward_3x3_s2_tall_kernel(const float* __restrict__ in,
+                                    float* __restrict__ out,
+                                    snn_hip_pooling_params p, int n_strips,
+                                    int n_wcols, unsigned n_waves) {
+  constexpr int PXW = 64 / CV;
+  constexpr int NR = 2 * TH + 1;
+  constexpr bool kAvg = IsAverage<Op>::value;
+  constexpr int kNt = 2;  // streaming (nt) load
+  const unsigned w = blockIdx.x * 4u + (threadIdx.x >> 6);
+  if (w >= n_waves) return;  // whole waves only (cross-lane reads below)
+  const int lane = threadIdx.x & 63;
+  const int cvi = lane % CV, pl = lane / CV;
+  const int wcol = static_cast<int>(w % static_cast<unsigned>(n_wcols));
+  const unsigned rest = w / static_cast<unsigned>(n_wcols);
+  const int strip = static_cast<int>(rest % static_cast<unsigned>(n_strips));
+  const int n = static_cast<int>(rest / static_cast<unsigned>(n_strips));
+  const int C = p.channels, c = cvi * 4;
+  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(
+      in, static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * C * 4);
+  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(
+      out, static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * C * 4);
+  const float ident = kAvg ? 0.f : lowest_of<float>();
+  const int oy0 = strip * TH;
+  const int ox = wcol * PXW + pl;
+  const int col0 = 2 * ox - p.pad_cols;   // first window column
+  const int y0 = 2 * oy0 - p.pad_rows;    // first input row of the strip
+  const int xr = 2 * (wcol + 1) * PXW - p.pad_cols;  // the wave's halo column
+  const bool last = pl == PXW - 1;
+  const bool c0_ok =
+      static_cast<unsigned>(col0) < static_cast<unsigned>(p.in_cols);
+  const bool c1_ok =
+      static_cast<unsigned>(col0 + 1) < static_cast<unsigned>(p.in_cols);
+  const bool r_ok =
+      last && static_cast<unsigned>(xr) < static_cast<unsigned>(p.in_cols);
+  const int row0 = (n * p.in_rows + y0) * p.in_cols * C + c;
+  const int rstride = p.in_cols * C;
+  const int src_r = (lane + CV) * 4;
+
+  float own[NR][2][4], hr[NR][4];
+#pragma unroll
+  for (int j = 0; j < NR; ++j) {
+    const bool row_ok =
+        static_cast<unsigned>(y0 + j) < static_cast<unsigned>(p.in_rows);
+    const bool mine = j < 2 * TH;  // the last row also opens the next strip
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const bool ok = row_ok && (k == 0 ? c0_ok : c1_ok);
+      const unsigned off =
+          ok ? static_cast<unsigned>(row0 + j * rstride + (col0 + k) * C) * 4u
+             : kOobOffset;
+      const float4 t = __builtin_bit_cast(
+          float4, mine ? __builtin_amdgcn_raw_buffer_load_b128(in_rsrc, off, 0,
+                                                               kNt)
+                       : __builtin_amdgcn_raw_buffer_load_b128(in_rsrc, off, 0,
+                                                               0));
+      own[j][k][0] = ok ? t.x : ident; own[j][k][1] = ok ? t.y : ident;
+      own[j][k][2] = ok ? t.z : ident; own[j][k][3] = ok ? t.w : ident;
+    }
+    const bool ok = row_ok && r_ok;
+    const float4 t = __builtin_bit_cast(
+        float4,
+        __builtin_amdgcn_raw_buffer_load_b128(
+            in_rsrc,
+            ok ? static_cast<unsigned>(row0 + j * rstride + xr * C) * 4u
+               : kOobOffset,
+            0, 0));
+    hr[j][0] = ok ? t.x : ident; hr[j][1] = ok ? t.y : ident;
+    hr[j][2] = ok ? t.z : ident; hr[j][3] = ok ? t.w : ident;
+  }
+
+  const int c_lo = max(col0, 0), c_hi = min(col0 + 3, p.in_cols);
+  Op acc[2][4];
+#pragma unroll
+  for (int j = 0; j < NR; ++j) {
+    float third[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float from_right = __builtin_bit_cast(
+          float, __builtin_amdgcn_ds_bpermute(
+                     src_r, __builtin_bit_cast(int, own[j][0][i])));
+      third[i] = last ? hr[j][i] : from_right;
+    }
+    // input row j is window row r of output row t = (j - r) / 2; the older
+    // output row first
+#pragma unroll
+    for (int r = 2; r >= 0; r -= 2) {
+      if (j - r < 0 || ((j - r) & 1) != 0) continue;
+      const int t = (j - r) / 2;
+      if (t >= TH) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (r == 0) acc[t & 1][i].init(lowest_of<float>());
+        acc[t & 1][i].accumulate(own[j][0][i]);
+        acc[t & 1][i].accumulate(own[j][1][i]);
+        acc[t & 1][i].accumulate(third[i]);
+      }
+      if (r == 2) {
+        const int ry = y0 + 2 * t;
+        const int tally = max(min(ry + 3, p.in_rows) - max(ry, 0), 0) *
+                          max(c_hi - c_lo, 0);
+        float res[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) res[i] = acc[t & 1][i].value(tally);
+        const bool ok = oy0 + t < p.out_rows && ox < p.out_cols;
+        BufVec4<float>::store(
+            out_rsrc,
+            ok ? static_cast<unsigned>(
+                     ((n * p.out_rows + oy0 + t) * p.out_cols + ox) * C + c) * 4u
+               : kOobOffset,
+            res);
+      }
+    }
+    // odd input rows are window row 1 of one output row only
+    if ((j & 1) != 0) {
+      const int t = (j - 1) / 2;
+      if (t < TH) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          acc[t & 1][i].accumulate(own[j][0][i]);
+          acc[t & 1][i].accumulate(own[j][1][i]);
+          acc[t & 1][i].accumulate(third[i]);
+        }
+      }
+    }
+  }
+}
+
 // ---- windows covering most of a small image (global pooling) ---------------
 // One work-group per (image, output pixel, group of 16 channel vectors).  The
 // window taps are dealt to 16 tap slices -- four per wave, lane = slice * 16 +
@@ -758,8 +903,41 @@ int launch_forward_op(const T* input, T* output,
       p.pad_rows < 3 && p.pad_cols < 3 &&
       (p.out_rows - 1) * p.stride_rows - p.pad_rows < p.in_rows &&
       (p.out_cols - 1) * p.stride_cols - p.pad_cols < p.in_cols;
-  if (p.channels % 4 == 0 && is3x3 && overlaps && in_bytes < 0x7FFFFFF0u &&
-      n_out * sizeof(T) < 0x7FFFFFF0u) {
+  // fp32, stride 2, 32 / 64 / 128 channels and enough waves to cover the GPU:
+  // the tall-strip kernel
+  bool tall = false;
+  if constexpr (std::is_same<T, float>::value) {
+    const int cv = p.channels / 4;
+    constexpr int kTallRows = 7;
+    const int pxw = cv > 0 ? 64 / cv : 0;
+    if (p.channels % 4 == 0 && is3x3 && p.stride_rows == 2 &&
+        (cv == 8 || cv == 16 || cv == 32) && p.out_rows >= kTallRows &&
+        in_bytes < 0x7FFFFFF0u && n_out * sizeof(T) < 0x7FFFFFF0u &&
+        SNN_TUNING_ENV("SNN_HIP_POOL_TALL_OFF") == nullptr) {
+      const int n_wcols = ceil_div(p.out_cols, pxw);
+      const int n_strips = ceil_div(p.out_rows, kTallRows);
+      const size_t waves = static_cast<size_t>(p.batch) * n_strips * n_wcols;
+      if (waves >= 768 && waves < 0x3FFFFFFFu &&
+          static_cast<size_t>(n_wcols) * pxw * 4 <=
+              static_cast<size_t>(p.out_cols) * 5) {
+        const unsigned n_waves = static_cast<unsigned>(waves);
+        const dim3 grid(ceil_div(n_waves, 4u));
+#define SNN_POOL_TALL(CV)                                                      \
+  hipLaunchKernelGGL((pool_forward_3x3_s2_tall_kernel<Op, kTallRows, CV>),    \
+                     grid, dim3(kBlock), 0, stream, input, output, p,          \
+                     n_strips, n_wcols, n_waves)
+        if (cv == 8) SNN_POOL_TALL(8);
+        else if (cv == 16) SNN_POOL_TALL(16);
+        else SNN_POOL_TALL(32);
+#undef SNN_POOL_TALL
+        tall = true;
+      }
+    }
+  }
+  if (tall) {
+    // launched above
+  } else if (p.channels % 4 == 0 && is3x3 && overlaps &&
+             in_bytes < 0x7FFFFFF0u && n_out * sizeof(T) < 0x7FFFFFF0u) {
     const size_t per_row =
         static_cast<size_t>(p.batch) * p.out_cols * (p.channels / 4);
     // Two output rows per lane: measured on MI355X with the XCD-contiguous

@@ -503,6 +503,39 @@ def test_depthwise_input_backprop_stride2_blocks(shape):
                  ("dw inbk s2", shape))
 
 
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, stride, same
+    (64, 50, 45, 64, 1, True),     # ragged last strip, ragged last wave column
+    (64, 50, 45, 64, 1, False),    # VALID: window starts at its own column
+    (40, 44, 64, 32, 1, True),     # two full wave columns of 32 pixels
+    (72, 30, 28, 128, 1, True),    # two pixel lanes per wave
+    (48, 61, 59, 32, 2, True),     # stride 2, odd size: padding 1
+    (48, 60, 58, 128, 2, False),   # stride 2, VALID
+    (32, 57, 57, 64, 2, True),
+])
+def test_depthwise_tall_strip_kernel(shape):
+    """Shapes that reach the tall-strip forward kernel (every input vector
+    loaded by one lane, window columns of the neighbours read across lanes):
+    ragged strips and wave columns, both strides, every padding, and its
+    mirrored-tap form as the stride-1 input gradient."""
+    n, h, w_, c, st, same = shape
+    p = ops.depthwise_params(n, h, w_, c, 1, 3, st, same)
+    op = oracle_params(p, 1)
+    rng = np.random.default_rng(sum(shape[:5]) + 5)
+    x = rng.standard_normal(n * h * w_ * c).astype(np.float32)
+    w = rng.standard_normal(9 * c).astype(np.float32)
+    got = ops.depthwise_conv2d(dev(x), dev(w), p).cpu().numpy()
+    assert_close(got, oracle.depthwise_forward(x, w, op),
+                 ("dw tall fwd", shape))
+    if st == 1:
+        dy = rng.standard_normal(n * p.out_rows * p.out_cols * c).astype(
+            np.float32)
+        got = ops.depthwise_conv2d(dev(dy), dev(w), p,
+                                   DIRECTION.INPUT_BACKPROP).cpu().numpy()
+        assert_close(got, oracle.depthwise_input_backprop(dy, w, op),
+                     ("dw tall inbk", shape))
+
+
 @pytest.mark.parametrize("size,ch,stride", MOBILENET)
 def test_depthwise_full_batch_matches_oracle(size, ch, stride):
     """Batch 32: the depthwise oracle is cheap enough to run in full."""
@@ -650,6 +683,37 @@ def test_pooling_window_wholly_outside_the_image(channels):
     assert np.array_equal(np.isnan(got), np.isnan(ref))
     ok = ~np.isnan(ref)
     assert_close(got[ok], ref[ok], "avg outside")
+
+
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, same
+    (48, 61, 59, 32, True),     # odd size: padding 1, ragged strip and wave column
+    (40, 60, 58, 128, False),   # VALID, two pixel lanes per wave
+    (32, 57, 57, 64, True),
+    (32, 112, 112, 64, True),   # the benchmark layer
+])
+def test_pooling_3x3_stride2_tall_strip_kernel(shape):
+    """Shapes that reach the tall-strip 3x3 stride-2 forward kernel (a lane
+    loads two window columns and reads the third from the next pixel lane):
+    maxima bit-exact with and without NaNs in the data under both NaN rules,
+    the average against the oracle."""
+    n, h, w_, c, same = shape
+    p = ops.pool_params(n, h, w_, c, 3, 2, same)
+    op = oracle_params(p, 0)
+    rng = np.random.default_rng(sum(shape[:4]) + 9)
+    x = rng.standard_normal(n * h * w_ * c).astype(np.float32)
+    got = ops.pooling_forward(dev(x), p, POOL_OP.MAX).cpu().numpy()
+    assert np.array_equal(got, oracle.pool_max_forward(x, op)), shape
+    assert_close(ops.pooling_forward(dev(x), p, POOL_OP.AVERAGE).cpu().numpy(),
+                 oracle.pool_avg_forward(x, op), ("avg tall", shape))
+    if n * h * w_ * c < 30_000_000:
+        x[rng.integers(0, x.size, x.size // 50)] = np.nan
+        for pool_op, nan_mode in ((POOL_OP.MAX, False),
+                                  (POOL_OP.MAX_WITH_NAN, True)):
+            got = ops.pooling_forward(dev(x), p, pool_op).cpu().numpy()
+            ref = oracle.pool_max_forward(x, op, nan_mode=nan_mode)
+            assert np.array_equal(got, ref, equal_nan=True), (shape, nan_mode)
+            assert np.isnan(ref).any() == nan_mode
 
 
 @pytest.mark.parametrize("shape", [
