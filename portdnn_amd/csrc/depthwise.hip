@@ -302,21 +302,68 @@ __global__ void __launch_bounds__(256)
 // wave-edge halo columns, which other lanes own, with ordinary ones.
 // Work-groups are not remapped to XCDs: consecutive groups then stream
 // consecutive runs of the tensor on all XCDs together.  Per output the taps
-// are still accumulated in filter-row, filter-column order.
-template <int STRIDE, int TH, int TW, int CV, bool FLIP>
+// are still accumulated in filter-row, filter-column order.  T is float (four
+// channels per lane) or half (eight).
+//
+// 16 bytes of T as raw words, and as floats.
+// A loaded vector is split into scalar words through the struct type (the
+// whole result bit-cast to uint4): element access on the builtin's own vector
+// type has produced wrong code with this compiler.
+__device__ inline void load_words(__amdgpu_buffer_rsrc_t r, unsigned off,
+                                  unsigned (&v)[4], bool streaming) {
+  const uint4 t = __builtin_bit_cast(
+      uint4, streaming ? __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 2)
+                       : __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0));
+  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+template <typename T>
+struct Raw16;
+template <>
+struct Raw16<float> {
+  static constexpr int kElems = 4;
+  __device__ static void to_float(const unsigned (&r)[4], float (&v)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __builtin_bit_cast(float, r[i]);
+  }
+  __device__ static uint4v from_float(const float (&v)[4]) {
+    return __builtin_bit_cast(uint4v, make_float4(v[0], v[1], v[2], v[3]));
+  }
+};
+template <>
+struct Raw16<_Float16> {
+  static constexpr int kElems = 8;
+  typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+  __device__ static void to_float(const unsigned (&r)[4], float (&v)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const half2v h = __builtin_bit_cast(half2v, r[i]);
+      v[2 * i] = static_cast<float>(h.x);
+      v[2 * i + 1] = static_cast<float>(h.y);
+    }
+  }
+  __device__ static uint4v from_float(const float (&v)[8]) {
+    typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+    half8 t;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t[i] = static_cast<_Float16>(v[i]);
+    return __builtin_bit_cast(uint4v, t);
+  }
+};
+
+template <typename T, int STRIDE, int TH, int TW, int CV, bool FLIP>
 __global__ void __launch_bounds__(256)
-    dw_forward_3x3_tall_kernel(const float* __restrict__ in,
-                               const float* __restrict__ fil,
-                               float* __restrict__ out,
+    dw_forward_3x3_tall_kernel(const T* __restrict__ in,
+                               const T* __restrict__ fil, T* __restrict__ out,
                                snn_hip_depthwise_params p, int n_strips,
                                int n_wcols, unsigned n_waves) {
+  constexpr int V = Raw16<T>::kElems;   // channels per lane: 16 bytes
+  constexpr unsigned kEsz = sizeof(T);
   constexpr int PXW = 64 / CV;          // pixel lanes per wave
   constexpr int OWN = STRIDE * TW;      // own input columns per lane
   constexpr int A = STRIDE == 1 ? 1 : 0;  // own range starts A columns right of
                                           // the first window column
   constexpr int NR = (TH - 1) * STRIDE + 3;
   constexpr int LIVE = STRIDE == 1 ? 3 : 2;  // output rows with open sums
-  constexpr int kNt = 2;                // streaming (nt) load
   const unsigned w = blockIdx.x * 4u + (threadIdx.x >> 6);
   if (w >= n_waves) return;  // whole waves only: the cross-lane reads below
                              // need every lane of a live wave
@@ -326,21 +373,24 @@ __global__ void __launch_bounds__(256)
   const unsigned rest = w / static_cast<unsigned>(n_wcols);
   const int strip = static_cast<int>(rest % static_cast<unsigned>(n_strips));
   const int n = static_cast<int>(rest / static_cast<unsigned>(n_strips));
-  const int C = p.channels, c = cvi * 4;
+  const int C = p.channels, c = cvi * V;
   const size_t in_elems =
       static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * C;
   const size_t out_elems =
       static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * C;
-  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_elems * 4);
+  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_elems * kEsz);
   const __amdgpu_buffer_rsrc_t fil_rsrc =
-      make_rsrc(fil, static_cast<size_t>(9) * C * 4);
-  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_elems * 4);
-  float f[9][4];
+      make_rsrc(fil, static_cast<size_t>(9) * C * kEsz);
+  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_elems * kEsz);
+  float f[9][V];
 #pragma unroll
-  for (int t = 0; t < 9; ++t)
-    BufVec4<float>::load(fil_rsrc,
-                         static_cast<unsigned>((FLIP ? 8 - t : t) * C + c) * 4u,
-                         f[t]);
+  for (int t = 0; t < 9; ++t) {
+    unsigned words[4];
+    load_words(fil_rsrc,
+               static_cast<unsigned>((FLIP ? 8 - t : t) * C + c) * kEsz, words,
+               false);
+    Raw16<T>::to_float(words, f[t]);
+  }
   const int oy0 = strip * TH;
   const int ox0 = (wcol * PXW + pl) * TW;  // first own output pixel
   const int col0 = STRIDE * ox0 - p.pad_cols + A;  // first own input column
@@ -363,7 +413,7 @@ __global__ void __launch_bounds__(256)
   const int rstride = p.in_cols * C;
   const int src_l = (lane - CV) * 4, src_r = (lane + CV) * 4;
 
-  float own[NR][OWN][4], hl[NR][4], hr[NR][4];
+  unsigned own[NR][OWN][4], hl[NR][4], hr[NR][4];
 #pragma unroll
   for (int j = 0; j < NR; ++j) {
     const bool row_ok =
@@ -371,55 +421,54 @@ __global__ void __launch_bounds__(256)
     // rows A .. A + STRIDE * TH - 1 of the strip are read by this strip only
     const bool mine = j >= A && j < A + STRIDE * TH;
 #pragma unroll
-    for (int k = 0; k < OWN; ++k) {
-      const unsigned off =
-          (row_ok && own_ok[k])
-              ? static_cast<unsigned>(row0 + j * rstride + (col0 + k) * C) * 4u
-              : kOobOffset;
-      const float4 t = __builtin_bit_cast(
-          float4, mine ? __builtin_amdgcn_raw_buffer_load_b128(in_rsrc, off, 0,
-                                                               kNt)
-                       : __builtin_amdgcn_raw_buffer_load_b128(in_rsrc, off, 0,
-                                                               0));
-      own[j][k][0] = t.x; own[j][k][1] = t.y;
-      own[j][k][2] = t.z; own[j][k][3] = t.w;
-    }
-    if (STRIDE == 1)
-      BufVec4<float>::load(
+    for (int k = 0; k < OWN; ++k)
+      load_words(
           in_rsrc,
-          (row_ok && l_ok)
-              ? static_cast<unsigned>(row0 + j * rstride + xl * C) * 4u
+          (row_ok && own_ok[k])
+              ? static_cast<unsigned>(row0 + j * rstride + (col0 + k) * C) * kEsz
               : kOobOffset,
-          hl[j]);
-    BufVec4<float>::load(
-        in_rsrc,
-        (row_ok && r_ok)
-            ? static_cast<unsigned>(row0 + j * rstride + xr * C) * 4u
-            : kOobOffset,
-        hr[j]);
+          own[j][k], mine);
+    if (STRIDE == 1)
+      load_words(in_rsrc,
+                 (row_ok && l_ok)
+                     ? static_cast<unsigned>(row0 + j * rstride + xl * C) * kEsz
+                     : kOobOffset,
+                 hl[j], false);
+    load_words(in_rsrc,
+               (row_ok && r_ok)
+                   ? static_cast<unsigned>(row0 + j * rstride + xr * C) * kEsz
+                   : kOobOffset,
+               hr[j], false);
   }
 
-  float acc[LIVE][TW][4];
+  float acc[LIVE][TW][V];
 #pragma unroll
   for (int j = 0; j < NR; ++j) {
-    // win[k + 1] is input column col0 + k, k = -1 .. OWN
-    float win[OWN + 2][4];
+    // win[k + 1] is input column col0 + k, k = -1 .. OWN.  The neighbours'
+    // columns cross the lanes as raw words (half as many exchanges for T =
+    // half as exchanging the converted values would take).
+    float win[OWN + 2][V];
+    {
+      unsigned left[4], right[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (STRIDE == 1) {
-        const float from_left = __builtin_bit_cast(
-            float, __builtin_amdgcn_ds_bpermute(
-                       src_l, __builtin_bit_cast(int, own[j][OWN - 1][i])));
-        win[0][i] = first ? hl[j][i] : from_left;
-      } else {
-        win[0][i] = 0.f;
+      for (int i = 0; i < 4; ++i) {
+        if (STRIDE == 1) {
+          const unsigned from_left =
+              static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(
+                  src_l, static_cast<int>(own[j][OWN - 1][i])));
+          left[i] = first ? hl[j][i] : from_left;
+        } else {
+          left[i] = 0u;
+        }
+        const unsigned from_right =
+            static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(
+                src_r, static_cast<int>(own[j][0][i])));
+        right[i] = last ? hr[j][i] : from_right;
       }
-      const float from_right = __builtin_bit_cast(
-          float, __builtin_amdgcn_ds_bpermute(
-                     src_r, __builtin_bit_cast(int, own[j][0][i])));
-      win[OWN + 1][i] = last ? hr[j][i] : from_right;
+      Raw16<T>::to_float(left, win[0]);
+      Raw16<T>::to_float(right, win[OWN + 1]);
 #pragma unroll
-      for (int k = 0; k < OWN; ++k) win[k + 1][i] = own[j][k][i];
+      for (int k = 0; k < OWN; ++k) Raw16<T>::to_float(own[j][k], win[k + 1]);
     }
     // input row j is filter row r of output row t = (j - r) / STRIDE; the
     // older output row first
@@ -431,7 +480,7 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
       for (int u = 0; u < TW; ++u) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < V; ++i) {
           float a = r == 0 ? 0.f : acc[t % LIVE][u][i];
 #pragma unroll
           for (int sx = 0; sx < 3; ++sx)
@@ -443,13 +492,13 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
         for (int u = 0; u < TW; ++u) {
           const bool ok = oy0 + t < p.out_rows && ox0 + u < p.out_cols;
-          BufVec4<float>::store(
-              out_rsrc,
+          __builtin_amdgcn_raw_buffer_store_b128(
+              Raw16<T>::from_float(acc[t % LIVE][u]), out_rsrc,
               ok ? static_cast<unsigned>(
                        ((n * p.out_rows + oy0 + t) * p.out_cols + ox0 + u) * C +
-                       c) * 4u
+                       c) * kEsz
                  : kOobOffset,
-              acc[t % LIVE][u]);
+              0, kStoreAux);
         }
       }
     }
@@ -1049,14 +1098,26 @@ __global__ void __launch_bounds__(kStrip* kSlices)
 // 2, enough waves to cover the GPU (smaller launches keep the short strips,
 // whose many lanes hide latency better).  Returns false when it does not take
 // the launch.
-template <bool FLIP>
-bool launch_dw_tall(const float* input, const float* filter, float* output,
+template <typename T, bool FLIP>
+bool launch_dw_tall(const T* input, const T* filter, T* output,
                     const snn_hip_depthwise_params& p, hipStream_t stream) {
-  const int cv = p.channels / 4;
-  if (cv != 8 && cv != 16 && cv != 32) return false;
+  constexpr int kV = 16 / sizeof(T);  // channels per lane
+  constexpr bool kHalf = sizeof(T) == 2;
+  if (p.channels % kV != 0) return false;
+  const int cv = p.channels / kV;
+  if (cv != 4 && cv != 8 && cv != 16 && cv != 32) return false;
+  if (cv == 4 && !kHalf) return false;   // fp32: 32 / 64 / 128 channels
+  if (cv == 32 && kHalf) return false;   // half: 32 / 64 / 128 channels
   if (p.pad_rows > 2 || p.pad_cols > 2) return false;
   const int stride = p.stride_rows;
-  int th = stride == 1 ? 14 : 7, tw = stride == 1 ? 4 : 1;
+  // Half precision at stride 1 stays on the short strips: measured at batch
+  // 128, 112x112x32 runs 44.8 us there against 61 us here (14 x 2 per lane;
+  // 57 us at 7 x 4) and 56x56x128 43.6 against 50 us, while the stride-2
+  // layer gains (112x112x64: 47.2 -> 44.0 us, 0.73 of the HBM peak).
+  if (kHalf && stride == 1 && SNN_TUNING_ENV("SNN_HIP_DW_TALL") == nullptr)
+    return false;
+  // half keeps eight channels per lane: half the columns for the same bytes
+  int th = stride == 1 ? 14 : 7, tw = stride == 1 ? (kHalf ? 2 : 4) : 1;
   // Developer overrides for tuning runs: SNN_HIP_DW_TALL=<th>x<tw> among the
   // shapes instantiated below.
   if (const char* tune = SNN_TUNING_ENV("SNN_HIP_DW_TALL")) {
@@ -1071,35 +1132,49 @@ bool launch_dw_tall(const float* input, const float* filter, float* output,
   const int n_wcols = ceil_div(p.out_cols, wpx);
   const int n_strips = ceil_div(p.out_rows, th);
   const size_t waves = static_cast<size_t>(p.batch) * n_strips * n_wcols;
-  // ragged last wave column: at most a quarter of its lanes idle overall
+  // ragged last wave column: at most a fifth of the lanes idle overall
   if (static_cast<size_t>(n_wcols) * wpx * 4 > static_cast<size_t>(p.out_cols) * 5)
     return false;
   if (waves < 768 || waves > 0x3FFFFFFFu) return false;
   const unsigned n_waves = static_cast<unsigned>(waves);
   const dim3 grid(ceil_div(n_waves, 4u));
-#define SNN_DW_TALL(STRIDE, TH, TW, CV)                                       \
-  hipLaunchKernelGGL((dw_forward_3x3_tall_kernel<STRIDE, TH, TW, CV, FLIP>),  \
-                     grid, dim3(256), 0, stream, input, filter, output, p,    \
+#define SNN_DW_TALL(STRIDE, TH, TW, CV)                                         \
+  hipLaunchKernelGGL((dw_forward_3x3_tall_kernel<T, STRIDE, TH, TW, CV, FLIP>), \
+                     grid, dim3(256), 0, stream, input, filter, output, p,      \
                      n_strips, n_wcols, n_waves)
-#define SNN_DW_TALL_CV(STRIDE, TH, TW)               \
-  do {                                               \
-    if (cv == 8) SNN_DW_TALL(STRIDE, TH, TW, 8);     \
-    else if (cv == 16) SNN_DW_TALL(STRIDE, TH, TW, 16); \
-    else SNN_DW_TALL(STRIDE, TH, TW, 32);            \
+#define SNN_DW_TALL_CV(STRIDE, TH, TW)                                \
+  do {                                                                \
+    if constexpr (kHalf) {                                            \
+      if (cv == 4) SNN_DW_TALL(STRIDE, TH, TW, 4);                    \
+      else if (cv == 8) SNN_DW_TALL(STRIDE, TH, TW, 8);               \
+      else SNN_DW_TALL(STRIDE, TH, TW, 16);                           \
+    } else {                                                          \
+      if (cv == 8) SNN_DW_TALL(STRIDE, TH, TW, 8);                    \
+      else if (cv == 16) SNN_DW_TALL(STRIDE, TH, TW, 16);             \
+      else SNN_DW_TALL(STRIDE, TH, TW, 32);                           \
+    }                                                                 \
   } while (0)
   if (stride == 1) {
-    if (th == 14 && tw == 4) SNN_DW_TALL_CV(1, 14, 4);
+    if constexpr (kHalf) {
 #ifdef SNN_HIP_TUNING
-    else if (th == 14 && tw == 2) SNN_DW_TALL_CV(1, 14, 2);
-    else if (th == 7 && tw == 4) SNN_DW_TALL_CV(1, 7, 4);
-    else if (th == 8 && tw == 4) SNN_DW_TALL_CV(1, 8, 4);
+      if (th == 14 && tw == 2) SNN_DW_TALL_CV(1, 14, 2);
+      else if (th == 7 && tw == 4) SNN_DW_TALL_CV(1, 7, 4);
+      else if (th == 7 && tw == 2) SNN_DW_TALL_CV(1, 7, 2);
+      else if (th == 14 && tw == 1) SNN_DW_TALL_CV(1, 14, 1);
+      else
 #endif
-    else return false;
+        return false;
+    } else {
+      if (th == 14 && tw == 4) SNN_DW_TALL_CV(1, 14, 4);
+#ifdef SNN_HIP_TUNING
+      else if (th == 14 && tw == 2) SNN_DW_TALL_CV(1, 14, 2);
+      else if (th == 7 && tw == 4) SNN_DW_TALL_CV(1, 7, 4);
+#endif
+      else return false;
+    }
   } else {
     if (th == 7 && tw == 1) SNN_DW_TALL_CV(2, 7, 1);
 #ifdef SNN_HIP_TUNING
-    else if (th == 7 && tw == 2) SNN_DW_TALL_CV(2, 7, 2);
-    else if (th == 4 && tw == 2) SNN_DW_TALL_CV(2, 4, 2);
     else if (th == 4 && tw == 1) SNN_DW_TALL_CV(2, 4, 1);
     else if (th == 14 && tw == 1) SNN_DW_TALL_CV(2, 14, 1);
 #endif
@@ -1114,9 +1189,9 @@ template <typename T, int V, bool FLIP>
 void launch_dw_strip(const T* input, const T* filter, T* output,
                      const snn_hip_depthwise_params& p, hipStream_t stream) {
   constexpr int kBlock = 256;
-  if constexpr (std::is_same<T, float>::value && V == 4) {
+  if constexpr (V * sizeof(T) == 16) {
     if (SNN_TUNING_ENV("SNN_HIP_DW_TALL_OFF") == nullptr &&
-        launch_dw_tall<FLIP>(input, filter, output, p, stream))
+        launch_dw_tall<T, FLIP>(input, filter, output, p, stream))
       return;
   }
   const int cv = p.channels / V;

@@ -513,27 +513,36 @@ def test_depthwise_input_backprop_stride2_blocks(shape):
     (48, 60, 58, 128, 2, False),   # stride 2, VALID
     (32, 57, 57, 64, 2, True),
 ])
-def test_depthwise_tall_strip_kernel(shape):
+@pytest.mark.parametrize("half", [False, True])
+def test_depthwise_tall_strip_kernel(shape, half):
     """Shapes that reach the tall-strip forward kernel (every input vector
     loaded by one lane, window columns of the neighbours read across lanes):
     ragged strips and wave columns, both strides, every padding, and its
-    mirrored-tap form as the stride-1 input gradient."""
+    mirrored-tap form as the stride-1 input gradient; fp32 and half (eight
+    channels per lane, twice the pixel lanes per wave)."""
     n, h, w_, c, st, same = shape
     p = ops.depthwise_params(n, h, w_, c, 1, 3, st, same)
     op = oracle_params(p, 1)
     rng = np.random.default_rng(sum(shape[:5]) + 5)
     x = rng.standard_normal(n * h * w_ * c).astype(np.float32)
     w = rng.standard_normal(9 * c).astype(np.float32)
-    got = ops.depthwise_conv2d(dev(x), dev(w), p).cpu().numpy()
-    assert_close(got, oracle.depthwise_forward(x, w, op),
-                 ("dw tall fwd", shape))
+    dy = rng.standard_normal(n * p.out_rows * p.out_cols * c).astype(
+        np.float32)
+    if half:
+        x, w, dy = (a.astype(np.float16).astype(np.float32)
+                    for a in (x, w, dy))
+        dtype, check = torch.float16, assert_close_f16
+    else:
+        dtype, check = torch.float32, assert_close
+    got = ops.depthwise_conv2d(dev(x, dtype), dev(w, dtype), p)
+    check(got.float().cpu().numpy(), oracle.depthwise_forward(x, w, op),
+          ("dw tall fwd", shape, half))
     if st == 1:
-        dy = rng.standard_normal(n * p.out_rows * p.out_cols * c).astype(
-            np.float32)
-        got = ops.depthwise_conv2d(dev(dy), dev(w), p,
-                                   DIRECTION.INPUT_BACKPROP).cpu().numpy()
-        assert_close(got, oracle.depthwise_input_backprop(dy, w, op),
-                     ("dw tall inbk", shape))
+        got = ops.depthwise_conv2d(dev(dy, dtype), dev(w, dtype), p,
+                                   DIRECTION.INPUT_BACKPROP)
+        check(got.float().cpu().numpy(),
+              oracle.depthwise_input_backprop(dy, w, op),
+              ("dw tall inbk", shape, half))
 
 
 @pytest.mark.parametrize("size,ch,stride", MOBILENET)
