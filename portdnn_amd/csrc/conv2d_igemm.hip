@@ -2108,6 +2108,31 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
   if (direction == SNN_HIP_FORWARD && conv2d_small_supports(p) &&
       SNN_TUNING_ENV("SNN_HIP_SMALL_OFF") == nullptr)
     return launch_conv2d_small_f32(input, filter, output, p, stream, epilogue);
+  const bool aligned16 =
+      ((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(filter) |
+        reinterpret_cast<uintptr_t>(output)) & 15u) == 0;
+  if (direction == SNN_HIP_FORWARD && aligned16 &&
+      conv2d_rowtile_supports(p) &&
+      SNN_TUNING_ENV("SNN_HIP_ROWTILE_OFF") == nullptr)
+    return launch_conv2d_rowtile_f32(input, filter, output, p, stream, false,
+                                     epilogue);
+  if (direction == SNN_HIP_INPUT_BACKPROP && aligned16 &&
+      p.stride_rows == 1 && p.stride_cols == 1 &&
+      p.window_rows - 1 - p.pad_rows >= 0 &&
+      p.window_cols - 1 - p.pad_cols >= 0 &&
+      SNN_TUNING_ENV("SNN_HIP_ROWTILE_OFF") == nullptr) {
+    // dX = dY convolved with the mirrored filter, channels and features
+    // exchanged, padding window - 1 - pad
+    snn_hip_conv2d_params q = p;
+    q.in_rows = p.out_rows;   q.in_cols = p.out_cols;
+    q.out_rows = p.in_rows;   q.out_cols = p.in_cols;
+    q.channels = p.features;  q.features = p.channels;
+    q.pad_rows = p.window_rows - 1 - p.pad_rows;
+    q.pad_cols = p.window_cols - 1 - p.pad_cols;
+    if (conv2d_rowtile_supports(q))
+      return launch_conv2d_rowtile_f32(input, filter, output, q, stream, true,
+                                       nullptr);
+  }
   if (direction == SNN_HIP_INPUT_BACKPROP &&
       conv2d_stem_input_backprop_supports(p) &&
       (reinterpret_cast<uintptr_t>(output) & 15u) == 0 &&

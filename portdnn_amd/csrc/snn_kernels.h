@@ -122,6 +122,19 @@ bool conv2d_small_supports(const snn_hip_conv2d_params& p);
 int launch_conv2d_small_f32(const float* x, const float* w, float* y,
                             const snn_hip_conv2d_params& p, hipStream_t stream,
                             const LaunchOptions* epilogue = nullptr);
+// Stride-1 convolution with windows larger than 1x1 on MFMA with the input
+// rows of a run of output pixels resident in LDS (conv2d_rowtile.hip): each
+// input element reaches a compute unit once per 64 features instead of once
+// per filter tap.  Channels in multiples of 16, features of 64; tensors
+// 16-byte aligned.  `transposed_filter`: `filter` is the HWCF tensor of the
+// convolution whose input gradient this is (`p` then describes the forward
+// convolution over dY: channels and features exchanged, padding window - 1 -
+// pad); taps are mirrored and the channel index is the reduction index.
+bool conv2d_rowtile_supports(const snn_hip_conv2d_params& p);
+int launch_conv2d_rowtile_f32(const float* input, const float* filter,
+                              float* output, const snn_hip_conv2d_params& p,
+                              hipStream_t stream, bool transposed_filter,
+                              const LaunchOptions* epilogue = nullptr);
 // Forward convolution of a three-channel image with a 7x7 window, stride 2 and
 // 64 features (conv2d_stem.hip): input rows of a band of output rows in LDS,
 // the filter in registers.  Output 16-byte aligned, at most 128 output columns.

@@ -210,6 +210,55 @@ def test_small_problem_kernel(shape):
 
 
 @pytest.mark.parametrize("shape", [
+    (16, 56, 56, 16, 128, 3, 3, True),   # one channel block, 13 pixel blocks a wave
+    (32, 28, 28, 32, 128, 3, 3, True),   # two channel blocks, 7 pixel blocks
+    (24, 40, 40, 48, 128, 3, 3, True),   # 10 pixel blocks
+    (16, 56, 56, 64, 64, 3, 3, True),    # the input gradient qualifies as well
+    (16, 56, 56, 16, 128, 5, 5, True),   # 25 taps: the loop over any window
+    (16, 58, 58, 32, 128, 3, 3, False),  # VALID
+    (8, 100, 250, 16, 64, 3, 3, True),   # tiles longer than a row, across images
+    (16, 56, 56, 32, 128, 1, 3, True),   # fewer taps than filter loads in flight
+])
+def test_input_rows_in_lds_kernel(shape):
+    """Large stride-1 convolutions through the Tiled and Im2col tags run on the
+    kernel that keeps the input rows of a run of output pixels in LDS (16
+    channels at a time) and reads the filter straight from the HWCF tensor:
+    forward, and the input gradient as a forward convolution over dY with
+    mirrored taps (the kernel takes it when the channel count is a multiple of
+    64, other shapes fall to the gather kernel and must be right all the
+    same); bias and ReLU folded into the store; twice, bit for bit."""
+    batch, rows, cols, ch, feats, wr, wc, same = shape
+    p = ops.ConvParams(channels=ch, features=feats, batch=batch, in_rows=rows,
+                       in_cols=cols, window_rows=wr, window_cols=wc,
+                       stride_rows=1, stride_cols=1)
+    ops.add_padding_to(p, same)
+    rng = np.random.default_rng(2600 + rows + ch + wr)
+    for direction in (DIRECTION.FORWARD, DIRECTION.INPUT_BACKPROP):
+        n_in, n_fil, _ = ops.conv_sizes(p, direction)
+        a, w = uniform(rng, n_in), uniform(rng, n_fil)
+        ref = ORACLE_FN[direction](a, w, oracle_params(p, feats), acc64=True)
+        da, dw = dev(a), dev(w)
+        for algo in (ALGO.TILED, ALGO.IM2COL):
+            if not supported(p, direction, algo):
+                continue
+            got = ops.conv2d(da, dw, p, direction, algo)
+            assert_close(got.cpu().numpy(), ref,
+                         ("rows in LDS", ALGO_NAME[algo], direction, shape))
+            if direction == DIRECTION.FORWARD or ch % 64 == 0:
+                again = ops.conv2d(da, dw, p, direction, algo)
+                assert torch.equal(got.view(torch.int32),
+                                   again.view(torch.int32)), (direction, shape)
+        if direction == DIRECTION.FORWARD:
+            bias = uniform(rng, feats)
+            fused = ops.conv2d_bias_act(da, dw, dev(bias), p, ALGO.IM2COL,
+                                        relu=True)
+            want = np.maximum(ref.reshape(-1, feats) + bias.astype(np.float64),
+                              0)
+            assert_close(fused.cpu().numpy(), want.reshape(-1),
+                         ("rows in LDS + bias + relu", shape))
+
+
+@pytest.mark.parametrize("shape", [
     # ragged / edge shapes: odd sizes, C and K not multiples of the tiles,
     # non-square windows and strides, VALID padding
     (3, 13, 17, 5, 7, 3, 3, 1, 1, True),
