@@ -453,6 +453,11 @@ def main():
                                    "algorithm": algo_names[algo],
                                    "ms": round(ms, 4),
                                    "tflops": round(w["flops"] / ms / 1e9, 2)})
+                if algo in (ALGO.TILED, ALGO.IM2COL, ALGO.WINOGRAD):
+                    # scalar copy for readers that keep only flat members:
+                    # algorithmic fraction of the fp32 MFMA peak, whole call
+                    roofline["%s_%s_frac" % (algo_names[algo], w["name"])] = \
+                        round(w["flops"] / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)
                 del ws
         detail["algorithms"] = algo_table
 

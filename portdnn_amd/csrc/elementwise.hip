@@ -135,6 +135,7 @@ int launch_pointwise_op(const T* in, const T* err, T* out, size_t n,
                         hipStream_t stream) {
   constexpr int L = Vec16<T>::kLanes;
   const bool vec = aligned16(in) && aligned16(out) && (!GRAD || aligned16(err));
+  KernelTimer timer(stream);
   if (vec) {
     const size_t n_vec = n / L;
     const size_t groups =
