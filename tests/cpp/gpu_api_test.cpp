@@ -478,6 +478,56 @@ static void test_bias_activation(backend::HIPBackend& backend) {
   CHECK(close(d_fused.host(), d_three.host(), true));
 }
 
+// The two-call form: prepare_filter once, launch_prepared many times; the
+// one-call launch in between must not depend on what the workspace holds.
+static void test_prepared_filter(backend::HIPBackend& backend) {
+  Conv2DParams p{};
+  p.channels = 64; p.features = 64; p.batch = 3;
+  p.in_rows = p.in_cols = 14;
+  p.window_rows = p.window_cols = 3;
+  p.stride_rows = p.stride_cols = 1;
+  p = helpers::add_padding_to(p, PaddingMode::SAME);
+  const auto sizes = conv2d::get_sizes<ct::Forward>(p);
+  const auto x = uniform_data(sizes.input_size, 31);
+  const auto w = uniform_data(sizes.filter_size, 32);
+  DeviceBuffer d_x(backend, x), d_w(backend, w);
+  DeviceBuffer d_one(backend, sizes.output_size),
+      d_two(backend, sizes.output_size);
+  std::unique_ptr<conv2d::Selector> def(new conv2d::WinogradSelector());
+  const auto ws = conv2d::query_workspace_size<float, ct::Forward>(p, *def);
+  CHECK(ws.recommended_size >= ws.required_size && ws.required_size > 0);
+  DeviceBuffer d_ws(backend, ws.recommended_size);
+  auto st = conv2d::launch<float, ct::Forward>(d_x.ptr, d_w.ptr, d_one.ptr, p,
+                                               *def, backend, d_ws.ptr,
+                                               ws.recommended_size);
+  CHECK(st.status == StatusCode::OK);
+  st.event.wait_and_throw();
+  // garbage in the workspace, then prepare + two prepared launches
+  (void)hipMemset(d_ws.ptr, 0xff, ws.recommended_size * sizeof(float));
+  st = conv2d::prepare_filter<float, ct::Forward>(
+      d_w.ptr, p, *def, backend, d_ws.ptr, ws.recommended_size);
+  CHECK(st.status == StatusCode::OK);
+  for (int rep = 0; rep < 2; ++rep) {
+    st = conv2d::launch_prepared<float, ct::Forward>(
+        d_x.ptr, d_w.ptr, d_two.ptr, p, *def, backend, d_ws.ptr,
+        ws.recommended_size);
+    CHECK(st.status == StatusCode::OK);
+  }
+  st.event.wait_and_throw();
+  CHECK(close(d_two.host(), d_one.host(), true));
+  // an algorithm with nothing to prepare takes both calls as well
+  conv2d::Im2colSelector im2col;
+  st = conv2d::prepare_filter<float, ct::Forward>(d_w.ptr, p, im2col, backend,
+                                                  d_ws.ptr, ws.recommended_size);
+  CHECK(st.status == StatusCode::OK);
+  st = conv2d::launch_prepared<float, ct::Forward>(
+      d_x.ptr, d_w.ptr, d_two.ptr, p, im2col, backend, d_ws.ptr,
+      ws.recommended_size);
+  CHECK(st.status == StatusCode::OK);
+  st.event.wait_and_throw();
+  CHECK(close(d_two.host(), d_one.host(), false));
+}
+
 static void test_compat(hipStream_t stream) {
   using namespace compat;
   using A = conv2d::Algorithm;
@@ -606,6 +656,7 @@ int main() {
     test_matmul(backend);
     test_elementwise(backend);
     test_bias_activation(backend);
+    test_prepared_filter(backend);
   }
   test_compat(stream);
   (void)hipStreamDestroy(stream);

@@ -166,6 +166,36 @@ static void test_workspace() {
   CHECK(w.required_size <= w.recommended_size);
 }
 
+// The element type as a template argument: half never gets Winograd and
+// needs no workspace (not in portDNN, whose queries do not know the type).
+static void test_typed_selector_and_workspace() {
+  // (a host compiler need not know _Float16: the headers take any two-byte
+  // element type for binary16)
+  using half_t = unsigned short;
+  auto p33 = make(3, 1, 56, 64, 64, 128, PaddingMode::SAME);
+  auto p11 = make(1, 1, 56, 64, 256, 128, PaddingMode::VALID);
+  auto for_float = conv2d::get_default_selector_for<float>();
+  auto for_half = conv2d::get_default_selector_for<half_t>();
+  CHECK(for_float->select<ct::Forward>(p33) == Algorithm::Winograd);
+  CHECK(for_half->select<ct::Forward>(p33) != Algorithm::Winograd);
+  CHECK(for_half->select<ct::Forward>(p33) != Algorithm::NotSupported);
+  CHECK(for_half->select<ct::InputBackprop>(p33) != Algorithm::Winograd);
+  CHECK(for_half->select<ct::FilterBackprop>(p33) != Algorithm::Winograd);
+  CHECK(for_half->select<ct::Forward>(p11) == Algorithm::Matmul);
+  auto f = conv2d::query_workspace_size<float, ct::Forward>(p33, *for_float);
+  auto untyped = conv2d::query_workspace_size<ct::Forward>(p33, *for_float);
+  CHECK_EQ(f.required_size, untyped.required_size);
+  CHECK_EQ(f.recommended_size, untyped.recommended_size);
+  CHECK(f.required_size > 0);
+  auto h = conv2d::query_workspace_size<half_t, ct::Forward>(p33, *for_half);
+  CHECK_EQ(h.required_size, 0);
+  CHECK(h.recommended_size >= 9u * 64u * 64u);  // the re-laid-out filter
+  conv2d::WinogradSelector wino;  // the tag on half data: no fp32 buffers
+  h = conv2d::query_workspace_size<half_t, ct::Forward>(p33, wino);
+  CHECK_EQ(h.required_size, 0);
+  CHECK(h.recommended_size < f.required_size);
+}
+
 static void test_status_codes() {
   // No GPU work is enqueued by any of these: every launch fails validation.
   backend::HIPBackend backend;
@@ -233,6 +263,7 @@ int main() {
   test_sizes();
   test_selectors();
   test_workspace();
+  test_typed_selector_and_workspace();
   test_status_codes();
   return report("host_api_test");
 }

@@ -256,6 +256,15 @@ def test_input_rows_in_lds_kernel(shape):
                               0)
             assert_close(fused.cpu().numpy(), want.reshape(-1),
                          ("rows in LDS + bias + relu", shape))
+            # operands that are not 16-byte aligned go to the kernels that
+            # load word by word, with the same result
+            pad_a = torch.empty(a.size + 1, device="cuda")
+            pad_w = torch.empty(w.size + 3, device="cuda")
+            pad_a[1:].copy_(da)
+            pad_w[3:].copy_(dw)
+            got = ops.conv2d(pad_a[1:], pad_w[3:], p, direction, ALGO.IM2COL)
+            assert_close(got.cpu().numpy(), ref,
+                         ("rows in LDS, unaligned operands", shape))
 
 
 @pytest.mark.parametrize("shape", [
