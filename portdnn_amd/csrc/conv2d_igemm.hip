@@ -1594,9 +1594,33 @@ void launch_auto(const float* src, const float* wgt, float* dst,
                             g.step_rows == 1 && g.step_cols == 1 &&
                             g.off_rows == 0 && g.off_cols == 0 &&
                             g.src_rows == g.p_rows && g.src_cols == g.p_cols;
-    if (plain_rows && gemm_rows_wanted(g.m_total, g.k_total, g.n_total, 1)) {
+    // (64-feature filters are too narrow for the plain-rows tiles, not for
+    // the filter-in-registers kernel it hands short reductions to)
+    if (plain_rows &&
+        (gemm_rows_wanted(g.m_total, g.k_total, g.n_total, 1) ||
+         (gemm_wreg_supports(g.m_total, g.k_total, g.n_total) &&
+          SNN_TUNING_ENV("SNN_HIP_GEMM_WREG_OFF") == nullptr))) {
       launch_gemm_rows(src, wgt, dst, g.m_total, g.k_total, g.n_total, 1, 0, 0,
                        0, stream, epilogue);
+      return;
+    }
+  }
+  if constexpr (B_K_INNER && !STRIDED) {
+    // The input gradient of a 1x1 stride-1 unpadded convolution is the plain
+    // product dX[m][c] = sum_k dY[m][k] W[c][k]: with few enough features
+    // (the reduction) the kernel that keeps the filter in registers takes it,
+    // reading W as it is stored.
+    const bool plain_rows = g.win_rows == 1 && g.win_cols == 1 &&
+                            g.step_rows == 1 && g.step_cols == 1 &&
+                            g.off_rows == 0 && g.off_cols == 0 &&
+                            g.src_rows == g.p_rows && g.src_cols == g.p_cols &&
+                            g.div_rows == 1 && g.div_cols == 1;
+    if (plain_rows &&
+        gemm_wreg_supports(g.m_total, g.k_total, g.n_total, true) &&
+        SNN_TUNING_ENV("SNN_HIP_GEMM_WREG_OFF") == nullptr) {
+      KernelTimer timer(stream);
+      launch_gemm_wreg(src, wgt, dst, g.m_total, g.k_total, g.n_total, false,
+                       nullptr, false, stream, true);
       return;
     }
   }

@@ -60,14 +60,22 @@ constexpr int vmcnt_imm(int n) {
 
 // (The kernels proper are the plain functions below: the compiler drops the
 // host side of a kernel *template* whose body names the LDS-direct load.)
-template <int KSTEPS, int PB, int FB, bool EPI>
+//
+// NS = 2: slices of 64 * FB features for filters with too few features for
+// eight waves (n = 64): waves 0-3 and 4-7 hold the same four feature blocks
+// and take the lower and the upper half of a tile of 32 * PB pixels.
+// TRANSW: W is stored n x k (k contiguous) -- the 1x1 input gradient
+// dX[m][c] = sum_k dY[m][k] * W[c][k] with the HWCF filter as it is; only the
+// one-off filter load differs.
+template <int KSTEPS, int PB, int FB, bool EPI, int NS, bool TRANSW>
 __device__ __forceinline__ void gemm_wreg_body(
     const float* __restrict__ x, const float* __restrict__ w,
     float* __restrict__ y, int m, int n, int n_cols, int m_tiles,
     int cols_by_xcd, int stream_stores, const float* __restrict__ bias,
     int relu) {
   constexpr int K = 4 * KSTEPS;
-  constexpr int TP = 16 * PB;                     // pixels per tile
+  constexpr int TP = 16 * PB * NS;                // pixels per tile
+  constexpr int FW = kWaves / NS;                 // waves along the features
   constexpr int TILE_FLOATS = TP * K;
   constexpr int TILE_BYTES = TILE_FLOATS * 4;
   constexpr int ROUNDS = TILE_BYTES / (1024 * kWaves);  // loads per wave and tile
@@ -102,7 +110,8 @@ __device__ __forceinline__ void gemm_wreg_body(
     col = j % n_cols;
     tile = (j / n_cols) * 8 + xcd;
   }
-  const int n0 = (col * kWaves + wave) * 16 * FB;
+  const int wf = wave % FW, wp = wave / FW;
+  const int n0 = (col * FW + wf) * 16 * FB;
 
   const __amdgpu_buffer_rsrc_t x_rsrc =
       make_rsrc(x, static_cast<size_t>(m) * K * 4);
@@ -118,7 +127,11 @@ __device__ __forceinline__ void gemm_wreg_body(
 #pragma unroll
       for (int s = 0; s < 4; ++s)
         wreg[fb][4 * g + s] =
-            w[static_cast<size_t>(16 * g + 4 * q + s) * n + n0 + 16 * fb + l16];
+            TRANSW
+                ? w[static_cast<size_t>(n0 + 16 * fb + l16) * K + 16 * g +
+                    4 * q + s]
+                : w[static_cast<size_t>(16 * g + 4 * q + s) * n + n0 +
+                    16 * fb + l16];
   float4v bias4[FB];
   if (EPI) {
 #pragma unroll
@@ -154,10 +167,10 @@ __device__ __forceinline__ void gemm_wreg_body(
   unsigned read_off[PB];
 #pragma unroll
   for (int pb = 0; pb < PB; ++pb)
-    read_off[pb] = static_cast<unsigned>((16 * pb + l16) * K) * 4u;
+    read_off[pb] = static_cast<unsigned>((16 * (wp * PB + pb) + l16) * K) * 4u;
   const unsigned swz = static_cast<unsigned>(l16 & 7);
   const unsigned out_lane =
-      static_cast<unsigned>(l16 * n + n0 + 4 * q) * 4u;
+      static_cast<unsigned>((16 * wp * PB + l16) * n + n0 + 4 * q) * 4u;
   const unsigned out_tile_bytes = static_cast<unsigned>(TP * n) * 4u;
 
   auto compute = [&](const float* stage, int t) {
@@ -244,52 +257,60 @@ __device__ __forceinline__ void gemm_wreg_body(
 }
 
 struct Plan {
-  int pb, fb, n_cols, m_tiles;
+  int pb, fb, ns, n_cols, m_tiles;
 };
 
 // The tiling whose work-group tiles divide most evenly over the 256 groups.
-bool make_plan(int m, int k, int n, Plan* plan) {
+bool make_plan(int m, int k, int n, Plan* plan, bool one_block = false) {
   if (k != 64 && k != 128 && k != 256 && k != 512) return false;
   double best = 0.0;
   bool found = false;
-  for (int fb = 2; fb >= 1; --fb) {
-    const int slice = 16 * kWaves * fb;
-    if (n % slice != 0) continue;
-    const int n_cols = n / slice;
-    if (n_cols > kGroups / 8 || (n_cols & (n_cols - 1)) != 0) continue;
-    for (int pb = 2; pb >= 1; --pb) {
-      const int tile_bytes = 16 * pb * k * 4;
-      if (tile_bytes % (1024 * kWaves) != 0) continue;
-      if (3 * tile_bytes > 96 * 1024) continue;  // three tiles in LDS
-      if (fb * (k / 4) > 128) continue;          // filter registers per lane
-      const int m_tiles = ceil_div(m, 16 * pb);
-      const int workers = kGroups / n_cols;
-      const int rounds = ceil_div(m_tiles, workers);
-      if (rounds < 4) continue;  // too little work to amortise the filter load
-      const double eff =
-          static_cast<double>(m) / (static_cast<double>(rounds) * workers * 16 * pb);
-      if (eff > best + 1e-9) {
-        best = eff;
-        *plan = Plan{pb, fb, n_cols, m_tiles};
-        found = true;
+  for (int ns = 1; ns <= 2; ++ns) {
+    for (int fb = one_block ? 1 : 2; fb >= 1; --fb) {
+      const int slice = 16 * (kWaves / ns) * fb;
+      if (n % slice != 0) continue;
+      if (ns == 2 && fb != 1) continue;  // (built: one feature block per wave)
+      const int n_cols = n / slice;
+      if (n_cols > kGroups / 8 || (n_cols & (n_cols - 1)) != 0) continue;
+      for (int pb = 2; pb >= 1; --pb) {
+        if (ns == 2 && pb != 1) continue;
+        const int tile_bytes = 16 * pb * ns * k * 4;
+        if (tile_bytes % (1024 * kWaves) != 0) continue;
+        if (3 * tile_bytes > 96 * 1024) continue;  // three tiles in LDS
+        if (fb * (k / 4) > 128) continue;          // filter registers per lane
+        const int m_tiles = ceil_div(m, 16 * pb * ns);
+        const int workers = kGroups / n_cols;
+        const int rounds = ceil_div(m_tiles, workers);
+        if (rounds < 4) continue;  // too little work to amortise the filter load
+        const double eff = static_cast<double>(m) /
+                           (static_cast<double>(rounds) * workers * 16 * pb * ns);
+        if (eff > best + 1e-9) {
+          best = eff;
+          *plan = Plan{pb, fb, ns, n_cols, m_tiles};
+          found = true;
+        }
       }
     }
+    // eight feature waves whenever the feature count allows them
+    if (found) break;
   }
   return found;
 }
 
-#define SNN_WREG_KERNEL(KSTEPS, PB, FB, E)                                      \
+#define SNN_WREG_KERNEL_AS(KSTEPS, PB, FB, E, NS, TRANSW, NAME)                 \
   __global__ void __launch_bounds__(64 * kWaves)                               \
       __attribute__((amdgpu_waves_per_eu(2, 2)))                               \
-      gemm_wreg_k##KSTEPS##_p##PB##_f##FB##_e##E(                              \
-          const float* __restrict__ x, const float* __restrict__ w,            \
-          float* __restrict__ y, int m, int n, int n_cols, int m_tiles,        \
-          int cols_by_xcd, int stream_stores, const float* __restrict__ bias,  \
-          int relu) {                                                          \
-    gemm_wreg_body<KSTEPS, PB, FB, E != 0>(x, w, y, m, n, n_cols, m_tiles,     \
-                                           cols_by_xcd, stream_stores, bias,   \
-                                           relu);                              \
+      NAME(const float* __restrict__ x, const float* __restrict__ w,           \
+           float* __restrict__ y, int m, int n, int n_cols, int m_tiles,       \
+           int cols_by_xcd, int stream_stores, const float* __restrict__ bias, \
+           int relu) {                                                         \
+    gemm_wreg_body<KSTEPS, PB, FB, E != 0, NS, TRANSW>(                        \
+        x, w, y, m, n, n_cols, m_tiles, cols_by_xcd, stream_stores, bias,      \
+        relu);                                                                 \
   }
+#define SNN_WREG_KERNEL(KSTEPS, PB, FB, E)      \
+  SNN_WREG_KERNEL_AS(KSTEPS, PB, FB, E, 1, false, \
+                     gemm_wreg_k##KSTEPS##_p##PB##_f##FB##_e##E)
 #define SNN_WREG_KERNELS(KSTEPS, PB, FB) \
   SNN_WREG_KERNEL(KSTEPS, PB, FB, 0)     \
   SNN_WREG_KERNEL(KSTEPS, PB, FB, 1)
@@ -302,13 +323,54 @@ SNN_WREG_KERNELS(32, 1, 2) SNN_WREG_KERNELS(32, 1, 1)
 SNN_WREG_KERNELS(64, 2, 2) SNN_WREG_KERNELS(64, 2, 1)
 SNN_WREG_KERNELS(64, 1, 2) SNN_WREG_KERNELS(64, 1, 1)
 SNN_WREG_KERNELS(128, 1, 1)
+// 64-feature slices (four feature waves x two pixel halves)
+SNN_WREG_KERNEL_AS(16, 1, 1, 0, 2, false, gemm_wreg_half_k16_e0)
+SNN_WREG_KERNEL_AS(16, 1, 1, 1, 2, false, gemm_wreg_half_k16_e1)
+SNN_WREG_KERNEL_AS(32, 1, 1, 0, 2, false, gemm_wreg_half_k32_e0)
+SNN_WREG_KERNEL_AS(32, 1, 1, 1, 2, false, gemm_wreg_half_k32_e1)
+SNN_WREG_KERNEL_AS(64, 1, 1, 0, 2, false, gemm_wreg_half_k64_e0)
+SNN_WREG_KERNEL_AS(64, 1, 1, 1, 2, false, gemm_wreg_half_k64_e1)
+// W stored n x k (the 1x1 input gradient): one feature block per wave
+SNN_WREG_KERNEL_AS(16, 2, 1, 0, 1, true, gemm_wreg_t_k16_p2)
+SNN_WREG_KERNEL_AS(32, 2, 1, 0, 1, true, gemm_wreg_t_k32_p2)
+SNN_WREG_KERNEL_AS(32, 1, 1, 0, 1, true, gemm_wreg_t_k32_p1)
+SNN_WREG_KERNEL_AS(64, 2, 1, 0, 1, true, gemm_wreg_t_k64_p2)
+SNN_WREG_KERNEL_AS(64, 1, 1, 0, 1, true, gemm_wreg_t_k64_p1)
+SNN_WREG_KERNEL_AS(16, 1, 1, 0, 2, true, gemm_wreg_t_half_k16)
+SNN_WREG_KERNEL_AS(32, 1, 1, 0, 2, true, gemm_wreg_t_half_k32)
+SNN_WREG_KERNEL_AS(64, 1, 1, 0, 2, true, gemm_wreg_t_half_k64)
 #undef SNN_WREG_KERNELS
 #undef SNN_WREG_KERNEL
+#undef SNN_WREG_KERNEL_AS
 
 using WregKernel = void (*)(const float*, const float*, float*, int, int, int,
                             int, int, int, const float*, int);
 
-WregKernel pick_kernel(int k, const Plan& plan, bool epilogue) {
+WregKernel pick_kernel(int k, const Plan& plan, bool epilogue,
+                       bool transpose_w) {
+  if (transpose_w) {
+    // (k = 512 measured 3 % slower than the general kernel on the input
+    // gradient of 28x28x128 -> 512 at batch 32; k <= 256 8 - 22 % faster)
+    if (epilogue || plan.fb != 1 || k > 256) return nullptr;
+    if (plan.ns == 2) {
+      if (plan.pb != 1) return nullptr;
+      return k == 64 ? gemm_wreg_t_half_k16
+             : k == 128 ? gemm_wreg_t_half_k32
+             : k == 256 ? gemm_wreg_t_half_k64
+                        : nullptr;
+    }
+    if (k == 64 && plan.pb == 2) return gemm_wreg_t_k16_p2;
+    if (k == 128) return plan.pb == 2 ? gemm_wreg_t_k32_p2 : gemm_wreg_t_k32_p1;
+    if (k == 256) return plan.pb == 2 ? gemm_wreg_t_k64_p2 : gemm_wreg_t_k64_p1;
+    return nullptr;
+  }
+  if (plan.ns == 2) {
+    if (plan.pb != 1 || plan.fb != 1) return nullptr;
+    if (k == 64) return epilogue ? gemm_wreg_half_k16_e1 : gemm_wreg_half_k16_e0;
+    if (k == 128) return epilogue ? gemm_wreg_half_k32_e1 : gemm_wreg_half_k32_e0;
+    if (k == 256) return epilogue ? gemm_wreg_half_k64_e1 : gemm_wreg_half_k64_e0;
+    return nullptr;
+  }
 #define SNN_WREG_PICK(KSTEPS, PB, FB)                     \
   if (k == 4 * KSTEPS && plan.pb == PB && plan.fb == FB)  \
     return epilogue ? gemm_wreg_k##KSTEPS##_p##PB##_f##FB##_e1 \
@@ -325,20 +387,21 @@ WregKernel pick_kernel(int k, const Plan& plan, bool epilogue) {
 
 }  // namespace
 
-bool gemm_wreg_supports(int m, int k, int n) {
+bool gemm_wreg_supports(int m, int k, int n, bool transpose_w) {
   Plan plan;
   return static_cast<size_t>(m) * max(k, n) * sizeof(float) <= kMaxBufferBytes &&
-         make_plan(m, k, n, &plan) && pick_kernel(k, plan, false) != nullptr;
+         make_plan(m, k, n, &plan, transpose_w) &&
+         pick_kernel(k, plan, false, transpose_w) != nullptr;
 }
 
 // bias (one value per column, may be null) and relu are applied when
 // `epilogue` is true.  Operands 16-byte aligned.
 void launch_gemm_wreg(const float* x, const float* w, float* y, int m, int k,
                       int n, bool epilogue, const float* bias, bool relu,
-                      hipStream_t stream) {
+                      hipStream_t stream, bool transpose_w) {
   Plan plan;
-  if (!make_plan(m, k, n, &plan)) return;
-  const WregKernel kernel = pick_kernel(k, plan, epilogue);
+  if (!make_plan(m, k, n, &plan, transpose_w)) return;
+  const WregKernel kernel = pick_kernel(k, plan, epilogue, transpose_w);
   if (kernel == nullptr) return;
   hipLaunchKernelGGL(kernel, dim3(kGroups), dim3(64 * kWaves), 0, stream, x, w,
                      y, m, n, plan.n_cols, plan.m_tiles,

@@ -106,14 +106,16 @@ int launch_conv2d_winograd_filter_backprop_f32(
     float* workspace, size_t workspace_elems, hipStream_t stream);
 
 // Row-major fp32 GEMM Y = X (m x k) * W (k x n) with the filter in registers
-// (gemm_wreg.hip): k = 64, 128 or 256, n in whole feature slices, enough rows
-// to keep 256 persistent work-groups busy.  Operands 16-byte aligned.  With
-// `epilogue`, bias (one value per column, may be null) is added and relu
-// applied on the way out.
-bool gemm_wreg_supports(int m, int k, int n);
+// (gemm_wreg.hip): k = 64, 128, 256 or 512, n in whole feature slices (128 or
+// 256 features, or 64 for k <= 256), enough rows to keep 256 persistent
+// work-groups busy.  Operands 16-byte aligned.  With `epilogue`, bias (one
+// value per column, may be null) is added and relu applied on the way out.
+// `transpose_w`: W is stored n x k (the 1x1 input gradient, whose filter
+// operand is the HWCF tensor read with the feature index as the reduction).
+bool gemm_wreg_supports(int m, int k, int n, bool transpose_w = false);
 void launch_gemm_wreg(const float* x, const float* w, float* y, int m, int k,
                       int n, bool epilogue, const float* bias, bool relu,
-                      hipStream_t stream);
+                      hipStream_t stream, bool transpose_w = false);
 // Forward convolution of problems with few output tiles (one 56x56x64 image:
 // 49 tiles of 64x64) in one launch without atomics (conv2d_small.hip):
 // work-groups of 16 pixels x 64 features whose four waves split the

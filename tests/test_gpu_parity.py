@@ -929,6 +929,40 @@ def test_matmul_filter_in_registers_kernel(shape):
     assert torch.all(out[m * n:] == 7.0)
 
 
+@pytest.mark.parametrize("shape", [
+    (12, 56, 56, 256, 64),   # 64 features: four feature waves x two pixel halves
+    (12, 55, 57, 64, 64),    # ... with a row count that ends inside a tile
+    (13, 56, 56, 128, 64),
+    (32, 28, 28, 512, 128),  # its input gradient: reduction 128, 512 columns
+    (16, 56, 56, 64, 256),   # input gradient: reduction 256, 64 columns
+])
+def test_conv1x1_narrow_filters_and_input_gradient_in_registers(shape):
+    """1x1 convolutions with 64 features, and the input gradient of 1x1
+    convolutions with up to 256 features (dX = dY * W^T, the filter read with
+    its feature index as the reduction), run on the filter-in-registers kernel
+    too: against the oracle, forward also with bias and ReLU folded in."""
+    batch, rows, cols, ch, feats = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, 1, 1, False)
+    rng = np.random.default_rng(6262 + ch + feats)
+    for direction in (DIRECTION.FORWARD, DIRECTION.INPUT_BACKPROP):
+        n_in, n_fil, _ = ops.conv_sizes(p, direction)
+        a, w = uniform(rng, n_in), uniform(rng, n_fil)
+        ref = ORACLE_FN[direction](a, w, oracle_params(p, feats), acc64=True)
+        da, dw = dev(a), dev(w)
+        for algo in (ALGO.MATMUL, ALGO.IM2COL):
+            got = ops.conv2d(da, dw, p, direction, algo)
+            assert_close(got.cpu().numpy(), ref,
+                         ("1x1", ALGO_NAME[algo], direction, shape))
+        if direction == DIRECTION.FORWARD:
+            bias = uniform(rng, feats) * 4
+            got = ops.conv2d_bias_act(da, dw, dev(bias), p, ALGO.MATMUL,
+                                      relu=True)
+            want = np.maximum(ref.reshape(-1, feats) + bias.astype(np.float64),
+                              0)
+            assert_close(got.cpu().numpy(), want.reshape(-1),
+                         ("1x1 + bias + relu", shape))
+
+
 @pytest.mark.parametrize("shape", [(4, 56, 56, 64, 256), (6, 28, 28, 128, 512),
                                    (12, 14, 14, 256, 1024),
                                    (32, 7, 7, 512, 2048)])
