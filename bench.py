@@ -170,10 +170,15 @@ def main():
             flops=ops.conv_flops(p, DIRECTION.FORWARD)))
     total_flops = sum(w["flops"] for w in work)
 
+    # (calls bound once: each is then one C ABI call per launch, without the
+    # Python wrapper's per-call argument conversions)
+    step_calls = [ops.conv2d_bound(w["x"], w["w"], w["y"], w["p"],
+                                   DIRECTION.FORWARD, w["algo"], w["ws"])
+                  for w in work]
+
     def step():
-        for w in work:
-            ops.conv2d(w["x"], w["w"], w["p"], DIRECTION.FORWARD, w["algo"],
-                       workspace=w["ws"], out=w["y"])
+        for call in step_calls:
+            call()
 
     for _ in range(args.warmup):
         step()
@@ -195,14 +200,17 @@ def main():
             ops.conv2d_prepare_filter(w["w"], w["p"], DIRECTION.FORWARD,
                                       w["algo"], w["ws"])
 
+    prepared_calls = [
+        ops.conv2d_prepared_bound(w["x"], w["w"], w["y"], w["p"],
+                                  DIRECTION.FORWARD, w["algo"], w["ws"])
+        if w["ws"] is not None else
+        ops.conv2d_bound(w["x"], w["w"], w["y"], w["p"], DIRECTION.FORWARD,
+                         w["algo"])
+        for w in work]
+
     def step_prepared():
-        for w in work:
-            if w["ws"] is not None:
-                ops.conv2d_prepared(w["x"], w["w"], w["p"], DIRECTION.FORWARD,
-                                    w["algo"], w["ws"], out=w["y"])
-            else:
-                ops.conv2d(w["x"], w["w"], w["p"], DIRECTION.FORWARD,
-                           w["algo"], out=w["y"])
+        for call in prepared_calls:
+            call()
     for _ in range(args.warmup):
         step_prepared()
     torch.cuda.synchronize()
@@ -316,10 +324,14 @@ def main():
             ys = [torch.empty(n, device="cuda") for _ in range(sets)]
             state = {"i": 0}
 
+            calls = [ops.pointwise_forward_bound(xs[i], ys[i],
+                                                 POINTWISE_OP.RELU)
+                     for i in range(sets)]
+
             def run():
                 i = state["i"] % sets
                 state["i"] += 1
-                ops.pointwise_forward(xs[i], POINTWISE_OP.RELU, out=ys[i])
+                calls[i]()
             stream_cache[n] = (
                 event_time_ms(run, reps=5 * sets, warm=sets, repeats=3),
                 device_ms(run, 5 * sets))
@@ -353,10 +365,13 @@ def main():
         f = normal(n_fil)
         state = {"i": 0}
 
+        calls = [ops.depthwise_conv2d_bound(xs[i], f, ys[i], p)
+                 for i in range(sets)]
+
         def run():
             i = state["i"] % sets
             state["i"] += 1
-            ops.depthwise_conv2d(xs[i], f, p, out=ys[i])
+            calls[i]()
         ms = event_time_ms(run, reps=5 * sets, warm=sets, repeats=3)
         return mem_entry("depthwise3x3_%dx%dx%d_s%d" % (size, size, ch, stride),
                          nbytes, ms, device_ms(run, 5 * sets))
@@ -370,10 +385,13 @@ def main():
         ys = [torch.empty(n_out, device="cuda") for _ in range(sets)]
         state = {"i": 0}
 
+        calls = [ops.pooling_forward_bound(xs[i], ys[i], p, op)
+                 for i in range(sets)]
+
         def run():
             i = state["i"] % sets
             state["i"] += 1
-            ops.pooling_forward(xs[i], p, op, out=ys[i])
+            calls[i]()
         ms = event_time_ms(run, reps=5 * sets, warm=sets, repeats=3)
         return mem_entry(name, nbytes, ms, device_ms(run, 5 * sets))
 
@@ -419,8 +437,7 @@ def main():
     x0, w0 = uniform(56 * 56 * 64), uniform(9 * 64 * 64)
     y0 = torch.empty(56 * 56 * 64, device="cuda")
 
-    def call0():
-        ops.conv2d(x0, w0, p0, DIRECTION.FORWARD, ALGO.TILED, out=y0)
+    call0 = ops.conv2d_bound(x0, w0, y0, p0, DIRECTION.FORWARD, ALGO.TILED)
     ms0 = event_time_ms(call0, reps=50)
     with ops.kernel_timing() as kt:
         for _ in range(50):

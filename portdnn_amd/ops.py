@@ -148,6 +148,39 @@ def conv2d(inp, fil, p, direction=DIRECTION.FORWARD, algorithm=ALGO.DIRECT,
     return out
 
 
+def _bind(fn, *cargs):
+    """A zero-argument callable that makes one C ABI call with arguments
+    converted once: timing loops over kernels of a few microseconds would
+    otherwise measure the per-call conversions of the wrappers above (6-7 us
+    against 2 for the call itself).  The stream is the one current now."""
+    def call():
+        code = fn(*cargs)
+        if code:
+            capi.check(code)
+    return call
+
+
+def conv2d_bound(inp, fil, out, p, direction, algorithm, workspace=None):
+    """conv2d with everything fixed: returns the callable that launches it."""
+    n_in, n_fil, n_out = conv_sizes(p, direction)
+    assert (inp.numel(), fil.numel(), out.numel()) == (n_in, n_fil, n_out)
+    assert inp.is_contiguous() and fil.is_contiguous() and out.is_contiguous()
+    fn = getattr(capi.lib(), _CONV_FN[(direction, inp.dtype)])
+    return _bind(fn, _ptr(inp), _ptr(fil), _ptr(out), ctypes.byref(p),
+                 algorithm, _ptr(workspace),
+                 0 if workspace is None else workspace.numel(),
+                 ctypes.c_void_p(_stream()))
+
+
+def conv2d_prepared_bound(inp, fil, out, p, direction, algorithm, workspace):
+    """conv2d_prepared with everything fixed."""
+    return _bind(capi.lib().snn_hip_conv2d_prepared_f32, direction, _ptr(inp),
+                 _ptr(fil), _ptr(out), ctypes.byref(p), algorithm,
+                 _ptr(workspace),
+                 0 if workspace is None else workspace.numel(),
+                 ctypes.c_void_p(_stream()))
+
+
 def conv2d_prepare_filter(fil, p, direction, algorithm, workspace):
     """snn_hip_conv2d_prepare_filter_f32: what the launch derives from the
     filter alone goes into `workspace`."""
@@ -238,6 +271,25 @@ def depthwise_conv2d(inp, fil, p, direction=DIRECTION.FORWARD, out=None):
     return out
 
 
+def depthwise_conv2d_bound(inp, fil, out, p, direction=DIRECTION.FORWARD):
+    """depthwise_conv2d with everything fixed (see _bind)."""
+    n_in, n_fil, n_out = depthwise_sizes(p, direction)
+    assert (inp.numel(), fil.numel(), out.numel()) == (n_in, n_fil, n_out)
+    fn = getattr(capi.lib(), _DW_FN[(direction, inp.dtype)])
+    return _bind(fn, _ptr(inp), _ptr(fil), _ptr(out), ctypes.byref(p),
+                 ctypes.c_void_p(_stream()))
+
+
+def pooling_forward_bound(inp, out, p, op):
+    """pooling_forward with everything fixed (see _bind)."""
+    assert inp.numel() == p.batch * p.in_rows * p.in_cols * p.channels
+    assert out.numel() == p.batch * p.out_rows * p.out_cols * p.channels
+    name = ("snn_hip_pooling_forward_f32" if inp.dtype == torch.float32 else
+            "snn_hip_pooling_forward_f16")
+    return _bind(getattr(capi.lib(), name), _ptr(inp), _ptr(out),
+                 ctypes.byref(p), op, ctypes.c_void_p(_stream()))
+
+
 def pooling_forward(inp, p, op, out=None):
     assert inp.numel() == p.batch * p.in_rows * p.in_cols * p.channels
     if out is None:
@@ -296,6 +348,14 @@ def pointwise_forward(x, op, out=None):
     fn = getattr(capi.lib(), "snn_hip_pointwise_forward" + _suffix(x))
     capi.check(fn(_ptr(x), _ptr(out), x.numel(), op, _stream()))
     return out
+
+
+def pointwise_forward_bound(x, out, op):
+    """pointwise_forward with everything fixed (see _bind)."""
+    assert out.numel() == x.numel()
+    fn = getattr(capi.lib(), "snn_hip_pointwise_forward" + _suffix(x))
+    return _bind(fn, _ptr(x), _ptr(out), x.numel(), op,
+                 ctypes.c_void_p(_stream()))
 
 
 def pointwise_grad(val, err, op, out=None):
