@@ -2140,6 +2140,11 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
       SNN_TUNING_ENV("SNN_HIP_ROWTILE_OFF") == nullptr)
     return launch_conv2d_rowtile_f32(input, filter, output, p, stream, false,
                                      epilogue);
+  if (direction == SNN_HIP_FORWARD && aligned16 &&
+      conv2d_rowsplit_supports(p) &&
+      SNN_TUNING_ENV("SNN_HIP_ROWSPLIT_OFF") == nullptr)
+    return launch_conv2d_rowsplit_f32(input, filter, output, p, stream, false,
+                                      epilogue);
   if (direction == SNN_HIP_INPUT_BACKPROP && aligned16 &&
       p.stride_rows == 1 && p.stride_cols == 1 &&
       p.window_rows - 1 - p.pad_rows >= 0 &&
@@ -2156,6 +2161,10 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
     if (conv2d_rowtile_supports(q))
       return launch_conv2d_rowtile_f32(input, filter, output, q, stream, true,
                                        nullptr);
+    if (conv2d_rowsplit_supports(q) &&
+        SNN_TUNING_ENV("SNN_HIP_ROWSPLIT_OFF") == nullptr)
+      return launch_conv2d_rowsplit_f32(input, filter, output, q, stream, true,
+                                        nullptr);
   }
   if (direction == SNN_HIP_INPUT_BACKPROP &&
       conv2d_stem_input_backprop_supports(p) &&

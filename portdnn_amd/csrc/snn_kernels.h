@@ -137,6 +137,16 @@ int launch_conv2d_rowtile_f32(const float* input, const float* filter,
                               float* output, const snn_hip_conv2d_params& p,
                               hipStream_t stream, bool transposed_filter,
                               const LaunchOptions* epilogue = nullptr);
+// The same for deep, small layers (conv2d_rowsplit.hip): every wave of a
+// work-group holds all of the tile's 16 x 16 output blocks and one eighth of
+// the channels, with its own LDS tile and no barrier in the reduction; the
+// eight partial results are added in LDS in a fixed order.  Channels in
+// multiples of 128, features of 32; arguments as above.
+bool conv2d_rowsplit_supports(const snn_hip_conv2d_params& p);
+int launch_conv2d_rowsplit_f32(const float* input, const float* filter,
+                               float* output, const snn_hip_conv2d_params& p,
+                               hipStream_t stream, bool transposed_filter,
+                               const LaunchOptions* epilogue = nullptr);
 // Forward convolution of a three-channel image with a 7x7 window, stride 2 and
 // 64 features (conv2d_stem.hip): input rows of a band of output rows in LDS,
 // the filter in registers.  Output 16-byte aligned, at most 128 output columns.

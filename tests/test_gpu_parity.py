@@ -268,6 +268,56 @@ def test_input_rows_in_lds_kernel(shape):
 
 
 @pytest.mark.parametrize("shape", [
+    (32, 14, 14, 256, 256, 3, 3, True),  # 4 feature blocks a wave, 2 channel
+                                         # blocks a wave
+    (32, 7, 7, 512, 512, 3, 3, True),    # 2 feature blocks a wave, tiles that
+                                         # span images, 4 channel blocks a wave
+    (40, 14, 14, 128, 96, 3, 3, True),   # 96 features: three slices of 32
+    (64, 14, 14, 128, 128, 5, 5, True),  # 25 taps, tiles of whole rows
+    (64, 16, 16, 128, 128, 3, 3, False), # VALID
+])
+def test_reduction_split_over_waves_kernel(shape):
+    """Deep stride-1 layers with few pixels (channels a multiple of 128) run on
+    the kernel whose eight waves each hold the whole output tile and split the
+    channel blocks among themselves, meeting in LDS at the end: forward and
+    the input gradient (a forward convolution over dY with mirrored taps),
+    against the oracle over the whole tensor; bias and ReLU folded into the
+    store; no atomics, so twice gives the same bits."""
+    batch, rows, cols, ch, feats, wr, wc, same = shape
+    p = ops.ConvParams(channels=ch, features=feats, batch=batch, in_rows=rows,
+                       in_cols=cols, window_rows=wr, window_cols=wc,
+                       stride_rows=1, stride_cols=1)
+    ops.add_padding_to(p, same)
+    rng = np.random.default_rng(2700 + rows + ch + wr)
+    for direction in (DIRECTION.FORWARD, DIRECTION.INPUT_BACKPROP):
+        n_in, n_fil, _ = ops.conv_sizes(p, direction)
+        a, w = uniform(rng, n_in), uniform(rng, n_fil)
+        ref = ORACLE_FN[direction](a, w, oracle_params(p, feats), acc64=True)
+        da, dw = dev(a), dev(w)
+        for algo in (ALGO.TILED, ALGO.IM2COL):
+            if not supported(p, direction, algo):
+                continue
+            got = ops.conv2d(da, dw, p, direction, algo)
+            assert_close(got.cpu().numpy(), ref,
+                         ("reduction split over waves", ALGO_NAME[algo],
+                          direction, shape))
+            # (the gradient of the 96-feature and of the VALID shape falls to
+            # kernels that add partial sums atomically)
+            if direction == DIRECTION.FORWARD or (same and feats % 128 == 0):
+                again = ops.conv2d(da, dw, p, direction, algo)
+                assert torch.equal(got.view(torch.int32),
+                                   again.view(torch.int32)), (direction, shape)
+        if direction == DIRECTION.FORWARD:
+            bias = uniform(rng, feats)
+            fused = ops.conv2d_bias_act(da, dw, dev(bias), p, ALGO.IM2COL,
+                                        relu=True)
+            want = np.maximum(ref.reshape(-1, feats) + bias.astype(np.float64),
+                              0)
+            assert_close(fused.cpu().numpy(), want.reshape(-1),
+                         ("reduction split over waves + bias + relu", shape))
+
+
+@pytest.mark.parametrize("shape", [
     # ragged / edge shapes: odd sizes, C and K not multiples of the tiles,
     # non-square windows and strides, VALID padding
     (3, 13, 17, 5, 7, 3, 3, 1, 1, True),
