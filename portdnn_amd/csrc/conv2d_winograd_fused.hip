@@ -43,6 +43,7 @@ constexpr unsigned kOob = 0x7FFFFFF0u;
 constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
 
 typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+typedef float float4v __attribute__((ext_vector_type(4)));
 
 // The (tile block, feature block) units of a launch and how they are dealt
 // to the 8 XCDs: xcd_m x xcd_f = 8.
@@ -79,14 +80,16 @@ __device__ inline float4 operator-(float4 a, float4 b) {
 }
 
 // U = G g Gt for four consecutive input channels of one output channel,
-// written in B-operand order:
-//   u[xi][co / 32][ci / 8][lane = co % 32 + 32 * ((ci % 8) / 4)][ci % 4].
+// written in B-operand order, 1 KiB per (xi, 32 features, group):
+//   u[xi][co / 32][group][lane][ci % 4]
+// with (group, lane) as the main kernel's matrix instruction wants them (see
+// `order` below).
 // For the input gradient g[r][s] = W[2-r][2-s][co][ci] (mirrored taps, channel
 // and feature roles swapped).
 __global__ void __launch_bounds__(256)
     wino_filter_pack_kernel(const float* __restrict__ w, float* __restrict__ u,
                             int channels, int features, bool backprop,
-                            bool halves) {
+                            int order) {
   const int cin = backprop ? features : channels;
   const int cout = backprop ? channels : features;
   const int idx = blockIdx.x * 256 + threadIdx.x;
@@ -137,14 +140,17 @@ __global__ void __launch_bounds__(256)
   }
   const int fblocks = cout / kFeat;
   const int cgroups = cin / 8;
-  // Channel quad cq = ci / 4 goes to (channel group, lane half).  Default:
-  // group cq / 2, half cq % 2 (a group is 8 consecutive channels).  `halves`
-  // (cin % 16 == 0): within 16 channels the lower lane half takes channels
-  // 0 - 7 and the upper 8 - 15, so quad cq = 4 c16 + 2 half + q is group
-  // 2 c16 + q.
-  const int half = halves ? (cq >> 1) & 1 : cq & 1;
-  const int group = halves ? 2 * (cq >> 2) + (cq & 1) : cq >> 1;
-  const int lane = co % kFeat + 32 * half;
+  // Order 0 (32x32x2 instruction): channel quad cq = ci / 4 is lane half
+  // cq % 2 of group cq / 2 (a group is 8 consecutive channels), lane co % 32
+  // within the half.  Order 1 (16x16x4 instruction, cin % 16 == 0): quad
+  // cq = 4 c16 + q of feature co = 32 fb + 16 F + n is lane n + 16 q of group
+  // 2 c16 + F (a group is 16 channels x 16 features).
+  int group = cq >> 1;
+  int lane = co % kFeat + 32 * (cq & 1);
+  if (order == 1) {
+    group = 2 * (cq >> 2) + ((co % kFeat) >> 4);
+    lane = (co & 15) + 16 * (cq & 3);
+  }
   const size_t base =
       ((static_cast<size_t>(co / kFeat) * cgroups + group) * 64 + lane) * 4;
   const size_t xi_stride = static_cast<size_t>(fblocks) * cgroups * 256;
@@ -449,9 +455,14 @@ __global__ void __launch_bounds__(512)
 //   raw[p][T][piece][t] is 16 bytes: pixel p of the 4x4 patch, tile 16 T + t,
 //   channels 4 piece .. 4 piece + 3.  Each wave reads the two patch rows its
 //   xi row combines (Bt d: d0 - d2, d1 + d2, d2 - d1, d1 - d3), applies the
-//   column transform in registers and feeds the results to the matrix
-//   instructions as the A operand: lane (tile, half) covers channels
-//   8 half .. 8 half + 7 of the chunk (the filter pack orders U to match).
+//   column transform in registers and feeds the results to
+//   v_mfma_f32_16x16x4_f32 as the A operand: lane (t, piece) holds tiles t and
+//   16 + t, channels 4 piece .. 4 piece + 3 -- the order the gather's lanes
+//   wrote the raw buffer in, so every lane reads back its own 16 bytes -- and
+//   instruction e of a chunk reduces channels 4 q + e over the lane quarters q
+//   (the filter pack orders U to match).  A unit is 2 x 2 blocks of 16 tiles x
+//   16 features per xi plane (the 32x32x2 form of this kernel measured 1-2 %
+//   slower on three of the four batch-32 ResNet layers, the same on the last).
 //   The transformed input never exists in memory.  One barrier per chunk; at
 //   the end of a unit At m A goes through the raw buffer that was multiplied
 //   last (two more barriers).
@@ -561,8 +572,7 @@ __global__ void __launch_bounds__(256)
         soff, 0, 0);
   };
 
-  // ---- multiply: lane (tile, half) ---------------------------------------
-  const int tile_r = lane & 31, half = lane >> 5;
+  // ---- multiply: lane (tile % 16, channel quad) --------------------------
   const unsigned n_fblocks = static_cast<unsigned>(ug.n_fblocks);
   const unsigned u_lane = static_cast<unsigned>(lane) * 16u;
   const unsigned cgroups = static_cast<unsigned>(g.in_ch) / 8u;
@@ -586,19 +596,20 @@ __global__ void __launch_bounds__(256)
   const int ra = wave == 0 ? 0 : (wave == 2 ? 2 : 1);
   const int rb = wave == 0 ? 2 : (wave == 1 ? 2 : (wave == 2 ? 1 : 3));
   const float sgn = wave == 1 ? 1.f : -1.f;
-  // 16-byte piece (row r, column 0, this lane's tile, channel quad 2 half)
-  // of a raw buffer; columns are 128 pieces apart, the second quad 16.
-  const int piece_t = ((tile_r >> 4) * 4 + 2 * half) * 16 + (tile_r & 15);
-  const int raw_a = (ra * 4 * 128 + piece_t) * 4;
-  const int raw_b = (rb * 4 * 128 + piece_t) * 4;
-  auto read_rows = [&](const float* raw, int q, float4 (&da)[4],
+  // Block (patch row r, column pc, tile half T) of a raw buffer is 1 KiB in
+  // the order the gather's lanes wrote it -- tile 16 T + lane % 16, channel
+  // quad lane / 16 -- which is the matrix instruction's operand order: every
+  // lane reads its own 16 bytes.
+  const int raw_a = ra * 8 * 256 + lane * 4;
+  const int raw_b = rb * 8 * 256 + lane * 4;
+  auto read_rows = [&](const float* raw, int T, float4 (&da)[4],
                        float4 (&db)[4]) {
 #pragma unroll
     for (int pc = 0; pc < 4; ++pc) {
       da[pc] = *reinterpret_cast<const float4*>(raw + raw_a +
-                                                (pc * 128 + q * 16) * 4);
+                                                (pc * 2 + T) * 256);
       db[pc] = *reinterpret_cast<const float4*>(raw + raw_b +
-                                                (pc * 128 + q * 16) * 4);
+                                                (pc * 2 + T) * 256);
     }
   };
   auto fma4 = [&](const float4& x, const float4& y) {
@@ -615,28 +626,31 @@ __global__ void __launch_bounds__(256)
     a[2] = t2 - t1;
     a[3] = t1 - t3;
   };
-  float16v acc[4];
-  // Four matrix instructions: reduction step e of the four xi planes.
-  auto mma_group = [&](const float4 (&a)[4], const float4 (&b)[4], int e) {
+  // acc[xi plane][tile half T][feature half F]: tiles 16 T + 4 (lane / 16)
+  // + r, feature 16 F + lane % 16.
+  float4v acc[4][2][2];
+  // Four matrix instructions: reduction step e (channels 4 q + e over the
+  // lane quarters q) of the four xi planes, one 16 x 16 block each.
+  auto mma_group = [&](const float4 (&a)[4], const float4 (&b)[4], int e,
+                       int T, int F) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(comp(a[j], e),
-                                                    comp(b[j], e), acc[j], 0,
-                                                    0, 0);
+      acc[j][T][F] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+          comp(a[j], e), comp(b[j], e), acc[j][T][F], 0, 0, 0);
   };
-  // B operand: b0 for the first channel quad of a chunk, b1x / b1y in turn
+  // B operand: b0 for the first 16 features of the block, b1x / b1y in turn
   // for the second.
   float4 b0[4], b1x[4], b1y[4];
-  // One chunk from `raw`.  Every vector-memory instruction sits behind a
-  // group of four matrix instructions (256 cycles of matrix work), so the
-  // texture path takes them one at a time and the wave never stands at a
-  // full queue: the eight gather loads of the next chunk of the stream
-  // (chunk g_chunk of the unit the offsets are set for; into the other raw
-  // buffer, which every wave finished reading before the barrier) behind
-  // the groups of the first quad, and behind those of the second quad the
-  // refills of b0 (used up by then) and of the idle b1 for the chunk after
-  // (nb_base, nb_cg).  The fences keep the compiler from collecting the
-  // loads in one place.
+  // One chunk from `raw`: the first feature half against both tile halves,
+  // then the second.  Every vector-memory instruction sits behind a group of
+  // four matrix instructions (128 cycles of matrix work), so the texture
+  // path takes them one at a time and the wave never stands at a full queue:
+  // the eight gather loads of the next chunk of the stream (chunk g_chunk of
+  // the unit the offsets are set for; into the other raw buffer, which every
+  // wave finished reading before the barrier) behind the groups of the first
+  // feature half, and behind those of the second the refills of b0 (used up
+  // by then) and of the idle b1 for the chunk after (nb_base, nb_cg).  The
+  // fences keep the compiler from collecting the loads in one place.
   auto step = [&](const float* raw, float* raw_next, int g_chunk,
                   float4 (&b1)[4], float4 (&b1_idle)[4], unsigned nb_base,
                   int nb_cg) {
@@ -649,19 +663,31 @@ __global__ void __launch_bounds__(256)
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      mma_group(a0, b0, e);
+      mma_group(a0, b0, e, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
-      gather(raw_next, g_chunk, 2 * e);
-      gather(raw_next, g_chunk, 2 * e + 1);
+      gather(raw_next, g_chunk, e);
       __builtin_amdgcn_sched_barrier(0);
     }
     transform(da, db, a1);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      mma_group(a1, b1, e);
+      mma_group(a1, b0, e, 1, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      gather(raw_next, g_chunk, 4 + e);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      mma_group(a0, b1, e, 0, 1);
       __builtin_amdgcn_sched_barrier(0);
       b0[e] = load_b(nb_base, nb_cg, e);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      mma_group(a1, b1, e, 1, 1);
+      __builtin_amdgcn_sched_barrier(0);
       b1_idle[e] = load_b(nb_base, nb_cg + 1, e);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -693,7 +719,10 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+      for (int T = 0; T < 2; ++T)
+#pragma unroll
+        for (int F = 0; F < 2; ++F)
+          acc[j][T][F] = float4v{0.f, 0.f, 0.f, 0.f};
     const int next_unit = unit + stride < n_local ? unit + stride : unit;
     const unsigned u_next = u_base_of(next_unit);
     // The unit's bias is fetched now: a load issued at the end of the unit
@@ -713,19 +742,29 @@ __global__ void __launch_bounds__(256)
     }
     // At m A: along xi's column index inside the lane, into raw buffer 1
     // (every wave is past its reads of it; buffer 0 is being filled) ...
+    // as s[xi row][output column ob][tile][feature], 32 floats per tile with
+    // the two feature halves swapped for every other group of four tiles (so
+    // that the lane quarters, four tiles apart, write different banks).
     {
-      float* const s_base = lds_raw1 + (wave * 2 * 16) * 64 + lane;
+      const int swz = 16 * ((lane >> 4) & 1);
+      float* const s_base = lds_raw1 + wave * 2 * 1024 + (lane >> 4) * 4 * 32;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        s_base[v * 64] = acc[0][v] + acc[1][v] + acc[2][v];
-        s_base[(16 + v) * 64] = acc[1][v] - acc[2][v] - acc[3][v];
-      }
+      for (int T = 0; T < 2; ++T)
+#pragma unroll
+        for (int F = 0; F < 2; ++F)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int at = (16 * T + r) * 32 + ((16 * F + (lane & 15)) ^ swz);
+            s_base[at] = acc[0][T][F][r] + acc[1][T][F][r] + acc[2][T][F][r];
+            s_base[1024 + at] =
+                acc[1][T][F][r] - acc[2][T][F][r] - acc[3][T][F][r];
+          }
     }
     __syncthreads();
-    // ... then along its row index across the waves.
-    const int q = tid & 15;
-    const int v = (tid >> 4) & 15;
-    const int m = 8 * (v >> 2) + 4 * (q >> 3) + (v & 3);
+    // ... then along its row index across the waves: thread (tile m, feature
+    // quad tid % 8).
+    const int m = tid >> 3;
+    const int fq4 = (4 * (tid & 7)) ^ (16 * ((m >> 2) & 1));
     const int tile_off = lds_tile_off[count & 1][m];
     const int flags = lds_tile_flags[count & 1][m];
 #pragma unroll
@@ -734,7 +773,7 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         s[i] = *reinterpret_cast<const float4*>(
-            lds_raw1 + ((i * 2 + ob) * 16 + v) * 64 + 4 * q);
+            lds_raw1 + ((i * 2 + ob) * 32 + m) * 32 + fq4);
       float4 y0 = s[0] + s[1] + s[2];
       float4 y1 = s[1] - s[2] - s[3];
       if (bias != nullptr) {
@@ -878,9 +917,9 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
   const unsigned u_bytes = static_cast<unsigned>(u_elems * 4);
   const unsigned out_bytes = static_cast<unsigned>(out_elems * 4);
   // The persistent kernel takes every launch that is not split and has an
-  // even number of chunks; it wants U with the channels of a chunk dealt to
-  // the lane halves eight at a time.
+  // even number of chunks; it wants U in the 16x16x4 instruction's order.
   const bool persistent = splits == 1 && n_chunks % 2 == 0;
+  const int pack_order = persistent ? 1 : 0;
   // The transformed filter depends on the filter and on this launch plan
   // only.  A caller that runs many launches with one filter may have it
   // written once (prepare_only) and then launch with filter_prepared, which
@@ -890,7 +929,7 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
     hipLaunchKernelGGL(wino_filter_pack_kernel,
                        dim3(ceil_div((g.in_ch / 4) * g.out_ch, 256)),
                        dim3(256), 0, stream, filter, workspace, p.channels,
-                       p.features, backprop, persistent);
+                       p.features, backprop, pack_order);
   if (epilogue != nullptr && epilogue->prepare_only) {
     SNN_HIP_CHECK_LAUNCH();
     return SNN_HIP_OK;
