@@ -468,7 +468,15 @@ bool conv2d_rowsplit_supports(const snn_hip_conv2d_params& p) {
                    p.channels * p.features;
   if (p.stride_rows != 1 || p.stride_cols != 1) return false;
   if (p.channels % (kKC * kWaves) != 0 || p.features % 32 != 0) return false;
-  if (p.window_rows * p.window_cols == 1) return false;
+  // 1x1 windows: only long reductions (at 512 channels a wave has four
+  // channel blocks and the general kernels measured faster, at 1024 this one
+  // is 15 % ahead)
+  if (p.window_rows * p.window_cols == 1) {
+    int min_channels = 1024;
+    if (const char* tune = SNN_TUNING_ENV("SNN_HIP_ROWSPLIT_1X1"))
+      min_channels = std::atoi(tune);
+    if (p.channels < min_channels) return false;
+  }
   if (std::max(std::max(x, y), w) * 4 > kMaxBufferBytes) return false;
   const SplitPlan plan = make_plan(p);
   if (plan.lds_bytes == 0) return false;
