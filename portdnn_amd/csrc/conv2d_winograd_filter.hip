@@ -354,6 +354,23 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// The same sum for a few splits: one float4 element per lane, the splits added
+// in order (with two splits the kernel above leaves 14 of its 16 lane groups
+// idle).
+__global__ void __launch_bounds__(256)
+    wino_filter_reduce_few_kernel(const float4* __restrict__ part,
+                                  float4* __restrict__ dw, unsigned n_vec,
+                                  int n_splits) {
+  const unsigned i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= n_vec) return;
+  float4 a = part[i];
+  for (int s = 1; s < n_splits; ++s) {
+    const float4 b = part[static_cast<size_t>(s) * n_vec + i];
+    a = make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
+  }
+  dw[i] = a;
+}
+
 struct FilterPlan {
   FilterGeom g;
   int splits;
@@ -431,10 +448,16 @@ int launch_conv2d_winograd_filter_backprop_f32(
                      static_cast<unsigned>(dy_elems * 4), n_groups, dw_elems);
   if (two_pass) {
     const unsigned n_vec = static_cast<unsigned>(dw_elems / 4);
-    hipLaunchKernelGGL(wino_filter_reduce_kernel, dim3(ceil_div(n_vec, 16u)),
-                       dim3(256), 0, stream,
-                       reinterpret_cast<const float4*>(workspace),
-                       reinterpret_cast<float4*>(dw), n_vec, plan.splits);
+    if (plan.splits <= 8)
+      hipLaunchKernelGGL(wino_filter_reduce_few_kernel,
+                         dim3(ceil_div(n_vec, 256u)), dim3(256), 0, stream,
+                         reinterpret_cast<const float4*>(workspace),
+                         reinterpret_cast<float4*>(dw), n_vec, plan.splits);
+    else
+      hipLaunchKernelGGL(wino_filter_reduce_kernel, dim3(ceil_div(n_vec, 16u)),
+                         dim3(256), 0, stream,
+                         reinterpret_cast<const float4*>(workspace),
+                         reinterpret_cast<float4*>(dw), n_vec, plan.splits);
   }
   SNN_HIP_CHECK_LAUNCH();
   return SNN_HIP_OK;
