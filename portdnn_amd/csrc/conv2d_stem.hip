@@ -515,22 +515,34 @@ __global__ void __launch_bounds__(64 * kWaves)
       }
 }
 
-// dW = sum of the work-groups' partial filters: 16 consecutive float4 x 16
-// groups of partials per work-group.
+// dW = sum of the work-groups' partial filters: 4 consecutive float4 x 64
+// groups of partials per work-group (588 work-groups for the 147 x 64 filter,
+// four partials per lane at 256 of them), the groups meeting through LDS in a
+// fixed order.
 __global__ void __launch_bounds__(256)
     stem_filter_backprop_reduce_kernel(const float4v* __restrict__ part,
                                        float4v* __restrict__ dw, int n_parts) {
-  __shared__ float4v sums[16][16];
-  const int o16 = threadIdx.x & 15, group = threadIdx.x >> 4;
-  const int o = blockIdx.x * 16 + o16;
+  __shared__ float4v sums[64][4];
+  const int o4 = threadIdx.x & 3, group = threadIdx.x >> 2;
+  const int o = blockIdx.x * 4 + o4;
   float4v sum = {0.f, 0.f, 0.f, 0.f};
-  for (int sp = group; sp < n_parts; sp += 16)
+  for (int sp = group; sp < n_parts; sp += 64)
     sum += part[static_cast<size_t>(sp) * (kPartFloats / 4) + o];
-  sums[group][o16] = sum;
+  sums[group][o4] = sum;
+  __syncthreads();
+  // eight lanes per element add eight groups each, then one adds the eight
+  __shared__ float4v sums8[8][4];
+  if (group < 8) {
+    sum = sums[8 * group][o4];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) sum += sums[8 * group + i][o4];
+    sums8[group][o4] = sum;
+  }
   __syncthreads();
   if (group != 0) return;
+  sum = sums8[0][o4];
 #pragma unroll
-  for (int i = 1; i < 16; ++i) sum += sums[i][o16];
+  for (int i = 1; i < 8; ++i) sum += sums8[i][o4];
   dw[o] = sum;
 }
 
@@ -790,9 +802,9 @@ int launch_conv2d_stem_filter_backprop_f32(const float* x, const float* dy,
     hipLaunchKernelGGL(conv_stem_filter_backprop_kernel, dim3(n_groups),
                        dim3(64 * kWaves), lds_bytes, stream, x, dy, part, g);
   }
-  static_assert(kPartFloats % 64 == 0, "whole groups of 16 float4");
+  static_assert(kPartFloats % 16 == 0, "whole groups of 4 float4");
   hipLaunchKernelGGL(stem_filter_backprop_reduce_kernel,
-                     dim3(kPartFloats / 64), dim3(256), 0, stream,
+                     dim3(kPartFloats / 16), dim3(256), 0, stream,
                      reinterpret_cast<const float4v*>(part),
                      reinterpret_cast<float4v*>(dw), static_cast<int>(n_groups));
   const hipError_t err = hipGetLastError();
