@@ -1249,6 +1249,18 @@ __global__ void __launch_bounds__(256)
       for (int e = 0; e < 4; ++e) rows[0][j][e] = rows[2][j][e];
   }
 
+  // The four dX pixels of a block row are stored after the next block row's
+  // loads have been issued: vector-memory operations retire in order, so
+  // stores issued before those loads would have to be acknowledged before
+  // the loads' data could be used.
+  float ee[4], eo[4], oe[4], oo[4];
+  unsigned st_off[4];
+  auto store_block_row = [&]() {
+    BufVec4<float>::store(dx_rsrc, st_off[0], ee);
+    BufVec4<float>::store(dx_rsrc, st_off[1], eo);
+    BufVec4<float>::store(dx_rsrc, st_off[2], oe);
+    BufVec4<float>::store(dx_rsrc, st_off[3], oo);
+  };
 #pragma unroll
   for (int i = 0; i < TH; ++i) {
     const int br = br0 + i;
@@ -1258,6 +1270,9 @@ __global__ void __launch_bounds__(256)
     load_out_pair(dy_rsrc, br, g);
     load_in_row(y + 1, rows[1]);
     load_in_row(y + 2, rows[2]);
+    __builtin_amdgcn_sched_barrier(0);
+    if (i > 0) store_block_row();
+    __builtin_amdgcn_sched_barrier(0);
     bool y_ok[3];
 #pragma unroll
     for (int r = 0; r < 3; ++r)
@@ -1302,7 +1317,6 @@ __global__ void __launch_bounds__(256)
         }
     }
     // the four dX pixels; windows in (output row, output column) order
-    float ee[4], eo[4], oe[4], oo[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       float v = 0.f;
@@ -1324,16 +1338,11 @@ __global__ void __launch_bounds__(256)
     const unsigned base = in_image + static_cast<unsigned>(y) * in_row_bytes +
                           in_col0 + static_cast<unsigned>(2 * C) * 4u;
     const unsigned col_bytes = static_cast<unsigned>(C) * 4u;
-    BufVec4<float>::store(dx_rsrc, (y_ok[0] && x_ok[2]) ? base : kOobOffset,
-                          ee);
-    BufVec4<float>::store(
-        dx_rsrc, (y_ok[0] && x_ok[3]) ? base + col_bytes : kOobOffset, eo);
-    BufVec4<float>::store(
-        dx_rsrc, (y_ok[1] && x_ok[2]) ? base + in_row_bytes : kOobOffset, oe);
-    BufVec4<float>::store(
-        dx_rsrc,
-        (y_ok[1] && x_ok[3]) ? base + in_row_bytes + col_bytes : kOobOffset,
-        oo);
+    st_off[0] = (y_ok[0] && x_ok[2]) ? base : kOobOffset;
+    st_off[1] = (y_ok[0] && x_ok[3]) ? base + col_bytes : kOobOffset;
+    st_off[2] = (y_ok[1] && x_ok[2]) ? base + in_row_bytes : kOobOffset;
+    st_off[3] =
+        (y_ok[1] && x_ok[3]) ? base + in_row_bytes + col_bytes : kOobOffset;
 #pragma unroll
     for (int w = 0; w < 2; ++w)
 #pragma unroll
@@ -1346,6 +1355,7 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
       for (int e = 0; e < 4; ++e) rows[0][j][e] = rows[2][j][e];
   }
+  store_block_row();
 }
 
 template <int WIN, int STRIDE>
@@ -1424,7 +1434,18 @@ int launch_pooling_max_grad(const float* input_data, const float* output_data,
     const int n_bcols = (p.in_cols + p.pad_cols - 1) / 2 - p.pad_cols / 2 + 1;
     const size_t per_row =
         static_cast<size_t>(p.batch) * n_bcols * (p.channels / 4);
-    const int th = per_row * ceil_div(n_brows, 4) >= 150000 ? 4 : 2;
+    // Block rows per lane: a strip re-reads the three input rows and the
+    // output / dY row of the block row above it, so the longest strip that
+    // still leaves about six waves per CU (112x112x64 at batch 32: 14 block
+    // rows, 1.1 x the input read instead of 1.4 x, 60 -> 56 us; 28 leave 3.5
+    // waves per CU: 76 us).
+    int th = per_row * ceil_div(n_brows, 14) >= 100000
+                 ? 14
+                 : per_row * ceil_div(n_brows, 4) >= 150000 ? 4 : 2;
+    if (const char* tune = SNN_TUNING_ENV("SNN_HIP_POOL_GRAD_TH")) {
+      const int v = std::atoi(tune);
+      if (v == 2 || v == 4 || v == 14) th = v;
+    }
     const int n_strips = ceil_div(n_brows, th);
     const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
     const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
@@ -1433,7 +1454,12 @@ int launch_pooling_max_grad(const float* input_data, const float* output_data,
                          output_data, input_backprop, output_backprop, p,
                          n_bcols, n_strips, n_items);
     };
-    if (th == 4) {
+    if (th == 14) {
+      if (nan_mode)
+        launch(pool_max_grad_3x3_s2_kernel<14, true>);
+      else
+        launch(pool_max_grad_3x3_s2_kernel<14, false>);
+    } else if (th == 4) {
       if (nan_mode)
         launch(pool_max_grad_3x3_s2_kernel<4, true>);
       else

@@ -847,6 +847,8 @@ def test_pooling_3x3_stride2_tall_strip_kernel(shape):
     (2, 30, 18, 20, 2, 2, False),    # disjoint windows
     (1, 16, 16, 4, 3, 2, True),      # exactly one tile
     (32, 90, 75, 64, 3, 2, True),    # 3x3 s2 with four block rows per lane
+    (64, 90, 90, 64, 3, 2, False),   # ... with fourteen, VALID
+    (16, 91, 78, 128, 3, 2, True),   # ... odd rows, ragged last strip
     (3, 21, 20, 16, 3, 2, False),    # 3x3 s2 VALID, unused last column
 ])
 @pytest.mark.parametrize("nan_mode", [False, True])
