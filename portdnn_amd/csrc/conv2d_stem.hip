@@ -39,7 +39,6 @@ constexpr int kWin = 7, kCh = 3, kStride = 2, kFeatures = 64;
 constexpr int kRowK = kWin * kCh;                 // 21 reduction values per filter row
 constexpr int kK = kWin * kRowK;                  // 147
 constexpr int kSteps = (kK + 3) / 4;              // 37 matrix instructions per block
-constexpr int kFb = kFeatures / 16;               // 4 feature blocks
 constexpr unsigned kOobOffset = 0x7FFFFFF0u;
 constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
 constexpr size_t kMaxLdsBytes = 150 * 1024;

@@ -1261,7 +1261,10 @@ __global__ void __launch_bounds__(256)
     BufVec4<float>::store(dx_rsrc, st_off[2], oe);
     BufVec4<float>::store(dx_rsrc, st_off[3], oo);
   };
-#pragma unroll
+  // (short strips unrolled in full; nothing in the body is indexed by i, so the
+  // 14-row strip runs as a loop of two block rows a turn -- one a turn
+  // measured 62 us, two or seven 57)
+#pragma unroll TH <= 4 ? TH : 2
   for (int i = 0; i < TH; ++i) {
     const int br = br0 + i;
     const int y = 2 * br - p.pad_rows;  // image row of padded row 2 * br
