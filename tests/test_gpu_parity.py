@@ -1824,3 +1824,70 @@ def test_scale_blend():
     assert np.array_equal(d.cpu().numpy(), np.zeros(16, dtype=np.float32))
     assert L.snn_hip_scale_blend_f32(d.data_ptr(), None, 1.0, 1.0, 16,
                                      None) == STATUS.INVALID_PARAMETER
+
+
+@pytest.mark.gpu
+def test_forward_chain_in_a_hip_graph_replays_like_eager():
+    """Callers that capture their launch-bound loops (serving) record library
+    calls into a HIP graph: a chain 3x3 conv (Winograd with the caller's
+    workspace) -> ReLU -> 1x1 conv -> 3x3 conv (Tiled) -> depthwise 3x3 ->
+    max pool 3x3 s2 is captured once and replayed three times, with eager
+    work of the program's own and synchronisations in between; every replay
+    must give the eager result bit for bit (these paths allocate nothing, clear
+    nothing with memset nodes and add nothing atomically)."""
+    batch, size, ch = 16, 56, 64
+    rng = np.random.default_rng(4100)
+    p3 = ops.conv_params(batch, size, size, ch, ch, 3, 1, True)
+    p1 = ops.conv_params(batch, size, size, ch, 4 * ch, 1, 1, False)
+    p3b = ops.conv_params(batch, size, size, 4 * ch, ch, 3, 1, True)
+    pd = ops.depthwise_params(batch, size, size, ch, 1, 3, 1, True)
+    pp = ops.pool_params(batch, size, size, ch, 3, 2, True)
+    x = dev(uniform(rng, ops.conv_sizes(p3, DIRECTION.FORWARD)[0]))
+    w3 = dev(uniform(rng, ops.conv_sizes(p3, DIRECTION.FORWARD)[1]))
+    w1 = dev(uniform(rng, ops.conv_sizes(p1, DIRECTION.FORWARD)[1]))
+    w3b = dev(uniform(rng, ops.conv_sizes(p3b, DIRECTION.FORWARD)[1]))
+    wd = dev(uniform(rng, ops.depthwise_sizes(pd, DIRECTION.FORWARD)[1]))
+    _, ws_elems = ops.workspace_size(p3, DIRECTION.FORWARD, ALGO.WINOGRAD)
+    ws = torch.empty(ws_elems, device="cuda")
+    n3 = ops.conv_sizes(p3, DIRECTION.FORWARD)[2]
+    n1 = ops.conv_sizes(p1, DIRECTION.FORWARD)[2]
+    bufs = [torch.empty(n3, device="cuda"), torch.empty(n3, device="cuda"),
+            torch.empty(n1, device="cuda"), torch.empty(n3, device="cuda"),
+            torch.empty(n3, device="cuda"),
+            torch.empty(batch * 28 * 28 * ch, device="cuda")]
+
+    def chain():
+        ops.conv2d(x, w3, p3, DIRECTION.FORWARD, ALGO.WINOGRAD, workspace=ws,
+                   out=bufs[0])
+        ops.pointwise_forward(bufs[0], POINTWISE_OP.RELU, out=bufs[1])
+        ops.conv2d(bufs[1], w1, p1, DIRECTION.FORWARD, ALGO.MATMUL,
+                   out=bufs[2])
+        ops.conv2d(bufs[2], w3b, p3b, DIRECTION.FORWARD, ALGO.TILED,
+                   out=bufs[3])
+        ops.depthwise_conv2d(bufs[3], wd, pd, DIRECTION.FORWARD, out=bufs[4])
+        ops.pooling_forward(bufs[4], pp, POOL_OP.MAX, out=bufs[5])
+
+    chain()
+    torch.cuda.synchronize()
+    eager = [b.clone() for b in bufs]
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        chain()  # first calls (function attributes, plan caches) outside capture
+        with torch.cuda.graph(graph, stream=side):
+            chain()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    scratch = torch.empty(1 << 20, device="cuda")
+    for replay in range(3):
+        for b in bufs:
+            b.fill_(float("nan"))
+        ws.fill_(float("nan"))
+        scratch.normal_()  # the program's own eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for i, (b, e) in enumerate(zip(bufs, eager)):
+            assert torch.equal(b.view(torch.int32), e.view(torch.int32)), (
+                "replay", replay, "buffer", i)
