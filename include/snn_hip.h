@@ -231,7 +231,10 @@ SNN_HIP_API int snn_hip_conv2d_filter_backprop_f16(
  * Tiled / Direct-fallback tags) always, except for the 7x7 stride-2
  * three-channel stem from 224 output rows over the batch upwards, whose
  * partial filters are summed in a fixed order; forward and input gradients of small
- * problems (fewer than ~640 64x64 output tiles) and the fused Winograd
+ * problems (fewer than ~640 64x64 output tiles, unless one of the kernels
+ * that sum their parts in a fixed order takes the launch: stride-1 layers
+ * with channels in multiples of 128, forward problems of fewer than 128
+ * tiles) and the fused Winograd
  * kernel below 128 work units -- and the order of those additions, hence the
  * last bits of the result, can change between runs.  The Winograd filter
  * gradient and every launch without such a split are reproducible.
