@@ -23,7 +23,7 @@
 //     w[tap][c0 + 4 q + t][f0 + f] for the four instructions t = 0..3 of a
 //     16-channel step, four 4-byte loads from the HWCF tensor (one 16-byte
 //     load for the input gradient, whose reduction index is contiguous), all
-//     L2 hits, issued two steps ahead;
+//     L2 hits, six fragment buffers in rotation, five steps ahead;
 //   * the pixel operand of those four instructions is one ds_read_b128 of
 //     channels c0 + 4 q .. + 3 of the lane's pixel slot (l % 16); a slot is
 //     five 16-byte pieces, so 16 consecutive slots fall into different banks;
@@ -36,7 +36,8 @@
 // The tile length is chosen on the host so that the work-groups come out as
 // a whole number of rounds over the 256 compute units with as few idle pixel
 // blocks as possible (batch-32 ResNet: 392 pixels x 64 features for 56x56x64,
-// 196 for 28x28x128, 98 for 14x14x256: one work-group per compute unit each).
+// 196 for 28x28x128: one work-group per compute unit each; the deeper layers
+// have too few pixels for this shape and run on conv2d_rowsplit.hip).
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
