@@ -892,19 +892,27 @@ __global__ void __launch_bounds__(kDwFilbkThreads)
           static_cast<unsigned>(n * p.in_rows * p.in_cols * C) * 4u;
       const unsigned row_bytes = static_cast<unsigned>(p.in_cols * C) * 4u;
       float win[RING][NC][4];
+      // (Offsets of rows and columns outside the image are made out of range
+      // with mask arithmetic, not with a conditional: the compiler turns a
+      // per-lane condition around these loads into two branches that load
+      // into the same registers, and has to wait for every load in flight
+      // between them -- which undid the row of loads issued ahead.)
       auto load_row = [&](int rel, float (&dst)[NC][4]) {
         const int y = y0 + rel;
-        const bool ok =
-            static_cast<unsigned>(y) < static_cast<unsigned>(p.in_rows);
+        const unsigned bad_row =
+            0u - static_cast<unsigned>(static_cast<unsigned>(y) >=
+                                       static_cast<unsigned>(p.in_rows));
         const unsigned base =
             image_off + static_cast<unsigned>(y) * row_bytes;
 #pragma unroll
-        for (int sc = 0; sc < NC; ++sc)
+        for (int sc = 0; sc < NC; ++sc) {
+          const unsigned bad =
+              bad_row |
+              (0u - static_cast<unsigned>(col_off[sc] == kOobOffset));
           BufVec4<float>::load(
-              in_rsrc,
-              (ok && col_off[sc] != kOobOffset) ? base + col_off[sc]
-                                                : kOobOffset,
+              in_rsrc, ((base + col_off[sc]) & ~bad) | (kOobOffset & bad),
               dst[sc]);
+        }
       };
       const unsigned dy_off0 =
           static_cast<unsigned>(((n * p.out_rows + oy0) * p.out_cols + ox) * C +
@@ -917,14 +925,17 @@ __global__ void __launch_bounds__(kDwFilbkThreads)
         for (int rel = 3 - STRIDE; rel < 3; ++rel)
           load_row(i * STRIDE + rel, win[(i * STRIDE + rel) % RING]);
 #pragma unroll
-        for (int tw = 0; tw < TW; ++tw)
+        for (int tw = 0; tw < TW; ++tw) {
+          const unsigned bad =
+              0u - static_cast<unsigned>(oy0 + i >= p.out_rows ||
+                                         ox + tw >= p.out_cols);
           BufVec4<float>::load(
               dy_rsrc,
-              (oy0 + i < p.out_rows && ox + tw < p.out_cols)
-                  ? dy_off0 + static_cast<unsigned>(i) * dy_row_bytes +
-                        static_cast<unsigned>(tw * C) * 4u
-                  : kOobOffset,
+              ((dy_off0 + static_cast<unsigned>(i) * dy_row_bytes +
+                static_cast<unsigned>(tw * C) * 4u) & ~bad) |
+                  (kOobOffset & bad),
               g[i % GRING][tw]);
+        }
       };
 #pragma unroll
       for (int rel = 0; rel < 3 - STRIDE; ++rel) load_row(rel, win[rel % RING]);
@@ -1353,18 +1364,14 @@ static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
     hipLaunchKernelGGL(kernel, grid, dim3(kDwFilbkThreads), 0, stream, x, dy,
                        dw, part, p, cvw, spg, n_strips, n_rb, n_cb);
   };
-  // Loads one output row ahead of the arithmetic pay everywhere except in
-  // the large stride-2 launches, whose five-column rows then cost occupancy.
+  // Loads two output rows ahead of the arithmetic at stride 1, one at stride 2
+  // (measured at batch 32: 112x112x32 30.1 / 27.5 / 26.5 / 26.4 us for 0 / 1 /
+  // 2 / 3 rows, 112x112x64 stride 2 32.6 / 30.1 / 31.1 / 32.6 us).
   if (p.stride_rows == 1) {
     if (th == 8)
-      launch(dw_filter_backprop_3x3_strip_kernel<1, 8, tw, 1>);
+      launch(dw_filter_backprop_3x3_strip_kernel<1, 8, tw, 2>);
     else
       launch(dw_filter_backprop_3x3_strip_kernel<1, 4, tw, 1>);
-  } else if (in_bytes >= kLargeInputBytes) {
-    if (th == 8)
-      launch(dw_filter_backprop_3x3_strip_kernel<2, 8, tw, 0>);
-    else
-      launch(dw_filter_backprop_3x3_strip_kernel<2, 4, tw, 0>);
   } else {
     if (th == 8)
       launch(dw_filter_backprop_3x3_strip_kernel<2, 8, tw, 1>);
