@@ -1167,31 +1167,47 @@ __global__ void __launch_bounds__(256)
   const unsigned in_row_bytes = static_cast<unsigned>(p.in_cols * C) * 4u;
   const unsigned in_image = static_cast<unsigned>(n * p.in_rows) * in_row_bytes;
   const unsigned in_col0 = static_cast<unsigned>(x0 * C + ch) * 4u;
+  // (Offsets outside the image are made out of range with mask arithmetic,
+  // not with a conditional: the compiler turns a per-lane condition around
+  // these loads into two branches that load into the same registers and waits
+  // for every load in flight between them.)
+  unsigned x_bad[5];
+#pragma unroll
+  for (int j = 0; j < 5; ++j) x_bad[j] = 0u - static_cast<unsigned>(!x_ok[j]);
   auto load_in_row = [&](int y, float (&v)[5][4]) {
-    const bool ok = static_cast<unsigned>(y) < static_cast<unsigned>(p.in_rows);
+    const unsigned y_bad = 0u - static_cast<unsigned>(
+                                    static_cast<unsigned>(y) >=
+                                    static_cast<unsigned>(p.in_rows));
     const unsigned base =
         in_image + static_cast<unsigned>(y) * in_row_bytes + in_col0;
 #pragma unroll
-    for (int j = 0; j < 5; ++j)
+    for (int j = 0; j < 5; ++j) {
+      const unsigned bad = y_bad | x_bad[j];
       BufVec4<float>::load(
           in_rsrc,
-          (ok && x_ok[j]) ? base + static_cast<unsigned>(j * C) * 4u
-                          : kOobOffset,
+          ((base + static_cast<unsigned>(j * C) * 4u) & ~bad) |
+              (kOobOffset & bad),
           v[j]);
+    }
   };
+  const unsigned w_bad[2] = {0u - static_cast<unsigned>(!w_ok[0]),
+                             0u - static_cast<unsigned>(!w_ok[1])};
   auto load_out_pair = [&](__amdgpu_buffer_rsrc_t rsrc, int oy,
                            float (&v)[2][4]) {
-    const bool ok =
-        static_cast<unsigned>(oy) < static_cast<unsigned>(p.out_rows);
+    const unsigned oy_bad = 0u - static_cast<unsigned>(
+                                     static_cast<unsigned>(oy) >=
+                                     static_cast<unsigned>(p.out_rows));
     const unsigned base = static_cast<unsigned>(
         ((n * p.out_rows + oy) * p.out_cols + bc - 1) * C + ch) * 4u;
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < 2; ++j) {
+      const unsigned bad = oy_bad | w_bad[j];
       BufVec4<float>::load(
           rsrc,
-          (ok && w_ok[j]) ? base + static_cast<unsigned>(j * C) * 4u
-                          : kOobOffset,
+          ((base + static_cast<unsigned>(j * C) * 4u) & ~bad) |
+              (kOobOffset & bad),
           v[j]);
+    }
   };
 
   // windows of the block row above: first-maximum position (9: none) and dY
