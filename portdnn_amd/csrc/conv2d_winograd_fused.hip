@@ -86,20 +86,26 @@ __device__ inline float4 operator-(float4 a, float4 b) {
 // `order` below).
 // For the input gradient g[r][s] = W[2-r][2-s][co][ci] (mirrored taps, channel
 // and feature roles swapped).
+// (The direction is a template parameter and each form loads all of its taps
+// in one straight run before the arithmetic: with a run-time `backprop` the
+// compiler put every tap's load in a branch of its own and let at most eight
+// be in flight, five round trips to memory for a kernel that is nothing but
+// latency on the small filters.)
+template <bool BACKPROP>
 __global__ void __launch_bounds__(256)
     wino_filter_pack_kernel(const float* __restrict__ w, float* __restrict__ u,
-                            int channels, int features, bool backprop,
-                            int order) {
-  const int cin = backprop ? features : channels;
-  const int cout = backprop ? channels : features;
+                            int channels, int features, int order) {
+  const int cin = BACKPROP ? features : channels;
+  const int cout = BACKPROP ? channels : features;
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= (cin / 4) * cout) return;
   const int co = idx % cout, cq = idx / cout;
-  float uu[16][4];
-  // The four channels of the quad are contiguous in W for the input gradient
-  // (W[2-r][2-s][co][ci]): one 16-byte load per tap.
-  float4 gq[3][3];
-  if (backprop) {
+  // g[t][r][s]: tap (r, s) of input channel 4 cq + t.  The four channels of
+  // the quad are contiguous in W for the input gradient (W[2-r][2-s][co][ci]):
+  // one 16-byte load per tap; forward they are a row of W apart.
+  float g[4][3][3];
+  if (BACKPROP) {
+    float4 gq[3][3];
 #pragma unroll
     for (int r = 0; r < 3; ++r)
 #pragma unroll
@@ -107,28 +113,34 @@ __global__ void __launch_bounds__(256)
         gq[r][s] = *reinterpret_cast<const float4*>(
             w + ((static_cast<size_t>(2 - r) * 3 + (2 - s)) * channels + co) *
                     features + 4 * cq);
+    __builtin_amdgcn_sched_barrier(0);  // every load before the first use
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int s = 0; s < 3; ++s) g[t][r][s] = comp(gq[r][s], t);
+  } else {
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int s = 0; s < 3; ++s)
+          g[t][r][s] = w[((static_cast<size_t>(r) * 3 + s) * channels + 4 * cq +
+                          t) * features + co];
+    __builtin_amdgcn_sched_barrier(0);
   }
+  float uu[16][4];
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
-    const int ci = 4 * cq + t;
-    float g[3][3];
-#pragma unroll
-    for (int r = 0; r < 3; ++r)
-#pragma unroll
-      for (int s = 0; s < 3; ++s) {
-        g[r][s] =
-            backprop
-                ? comp(gq[r][s], t)
-                : w[((static_cast<size_t>(r) * 3 + s) * channels + ci) *
-                        features + co];
-      }
     float h[4][3];  // G g
 #pragma unroll
     for (int s = 0; s < 3; ++s) {
-      h[0][s] = g[0][s];
-      h[1][s] = 0.5f * (g[0][s] + g[1][s] + g[2][s]);
-      h[2][s] = 0.5f * (g[0][s] - g[1][s] + g[2][s]);
-      h[3][s] = g[2][s];
+      h[0][s] = g[t][0][s];
+      h[1][s] = 0.5f * (g[t][0][s] + g[t][1][s] + g[t][2][s]);
+      h[2][s] = 0.5f * (g[t][0][s] - g[t][1][s] + g[t][2][s]);
+      h[3][s] = g[t][2][s];
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -926,10 +938,11 @@ int launch_conv2d_winograd_fused_f32(int direction, const float* input,
   // trusts what the workspace holds.
   const bool prepared = epilogue != nullptr && epilogue->filter_prepared;
   if (!prepared)
-    hipLaunchKernelGGL(wino_filter_pack_kernel,
+    hipLaunchKernelGGL(backprop ? wino_filter_pack_kernel<true>
+                                : wino_filter_pack_kernel<false>,
                        dim3(ceil_div((g.in_ch / 4) * g.out_ch, 256)),
                        dim3(256), 0, stream, filter, workspace, p.channels,
-                       p.features, backprop, pack_order);
+                       p.features, pack_order);
   if (epilogue != nullptr && epilogue->prepare_only) {
     SNN_HIP_CHECK_LAUNCH();
     return SNN_HIP_OK;

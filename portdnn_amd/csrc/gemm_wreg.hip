@@ -118,20 +118,40 @@ __device__ __forceinline__ void gemm_wreg_body(
   const __amdgpu_buffer_rsrc_t y_rsrc =
       make_rsrc(y, static_cast<size_t>(m) * n * 4);
 
-  // the filter slice of this wave, in matrix-operand order
+  // The filter slice of this wave, in matrix-operand order: buffer loads
+  // whose lane part is one register and whose step part is a scalar offset
+  // (a pointer per load would be 2 K / 4 address registers: the compiler
+  // spilled them and waited on the way).  W stored n x k gives the four steps
+  // of a group with one 16-byte load.
+  const __amdgpu_buffer_rsrc_t w_rsrc =
+      make_rsrc(w, static_cast<size_t>(K) * n * 4);
   float wreg[FB][KSTEPS];
 #pragma unroll
-  for (int fb = 0; fb < FB; ++fb)
+  for (int fb = 0; fb < FB; ++fb) {
+    if (TRANSW) {
+      const unsigned voff =
+          static_cast<unsigned>((n0 + 16 * fb + l16) * K + 4 * q) * 4u;
 #pragma unroll
-    for (int g = 0; g < KSTEPS / 4; ++g)
+      for (int g = 0; g < KSTEPS / 4; ++g) {
+        const float4v v = __builtin_bit_cast(
+            float4v, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, voff,
+                                                           64 * g, 0));
 #pragma unroll
-      for (int s = 0; s < 4; ++s)
-        wreg[fb][4 * g + s] =
-            TRANSW
-                ? w[static_cast<size_t>(n0 + 16 * fb + l16) * K + 16 * g +
-                    4 * q + s]
-                : w[static_cast<size_t>(16 * g + 4 * q + s) * n + n0 +
-                    16 * fb + l16];
+        for (int s = 0; s < 4; ++s) wreg[fb][4 * g + s] = v[s];
+      }
+    } else {
+      const unsigned voff =
+          static_cast<unsigned>(4 * q * n + n0 + 16 * fb + l16) * 4u;
+#pragma unroll
+      for (int g = 0; g < KSTEPS / 4; ++g)
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+          wreg[fb][4 * g + s] = __builtin_bit_cast(
+              float, __builtin_amdgcn_raw_buffer_load_b32(
+                         w_rsrc, voff,
+                         static_cast<unsigned>((16 * g + s) * n) * 4u, 0));
+    }
+  }
   float4v bias4[FB];
   if (EPI) {
 #pragma unroll
@@ -242,9 +262,16 @@ __device__ __forceinline__ void gemm_wreg_body(
     compute(cur, tile);                                  \
     tile += workers;                                     \
   }
-  __builtin_amdgcn_sched_barrier(0);  // (the filter loads above go first)
   issue(s0, tile);
   issue(s1, tile + workers);
+  // The filter registers are pinned here so that their loads are in flight
+  // together with the first two tiles (left alone, the compiler sinks the
+  // loads below the wait, to their first use: two round trips to memory in a
+  // row before the first matrix instruction).
+#pragma unroll
+  for (int fb = 0; fb < FB; ++fb)
+#pragma unroll
+    for (int i = 0; i < KSTEPS; ++i) asm volatile("" : "+v"(wreg[fb][i]));
   __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
   for (;;) {
     SNN_WREG_STEP(s0, s2)
