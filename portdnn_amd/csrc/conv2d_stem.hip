@@ -643,21 +643,27 @@ __global__ void __launch_bounds__(64 * kWaves)
                                                       acc[b], 0, 0, 0);
     // A float one lane updates for pixel 4 q + v is another lane's for pixel
     // 4 q + v + 1 (two taps to the left), so the four v must stay in program
-    // order: volatile, and the LDS serves a wave's accesses in order.  The
-    // five row blocks of one v never meet (their rho differ by less than the
-    // 24 floats between lane groups, or sit in different LDS rows) and go as
-    // one batch of reads and one of writes.
-    volatile float* base = lds + kStride * row * kRowFloats + 96 * pb;
+    // order (the LDS serves a wave's accesses in order): a compiler barrier
+    // between the batches keeps them there.  (Not `volatile`: every volatile
+    // access waits for all vector-memory loads in flight as well, the next
+    // block's dY among them -- a round trip to memory per block.)  The five
+    // row blocks of one v never meet (their rho differ by less than the 24
+    // floats between lane groups, or sit in different LDS rows) and go as one
+    // batch of reads and one of writes.
+    float* base = lds + kStride * row * kRowFloats + 96 * pb;
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       float old[kRhoBlocks];
+      asm volatile("" ::: "memory");
 #pragma unroll
       for (int b = 0; b < kRhoBlocks; ++b)
         old[b] = base[(z_off[b] >= 0 ? z_off[b] : 0) + 6 * v];
+      asm volatile("" ::: "memory");
 #pragma unroll
       for (int b = 0; b < kRhoBlocks; ++b)
         if (z_off[b] >= 0) base[z_off[b] + 6 * v] = old[b] + acc[b][v];
     }
+    asm volatile("" ::: "memory");
   };
 
   // A block (output row, pixel block) touches LDS rows 2 row ... 2 row + 6 and
@@ -733,10 +739,30 @@ __global__ void __launch_bounds__(64 * kWaves)
   }
 }
 
+// Zeroes the rows of dX that the band kernel does not store: the kWin - kStride
+// rows that two neighbouring bands share (both add into them with atomics)
+// and the rows below the last band's reach (no window touches them).  Block
+// (image x band, r): band b < n_bands - 1 clears shared row r of its lower
+// edge, the last band every fifth row from its reach + r on.
 __global__ void __launch_bounds__(256)
-    stem_zero_fill_kernel(float4v* __restrict__ dst, size_t n_vec) {
-  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (i < n_vec) dst[i] = float4v{0.f, 0.f, 0.f, 0.f};
+    stem_zero_rows_kernel(float* __restrict__ dx, StemGeom g) {
+  const int n = blockIdx.x / g.n_bands;
+  const int band = blockIdx.x % g.n_bands;
+  const int row_floats = g.in_cols * kCh;
+  const int first = kStride * (band + 1) * g.band - g.pad_rows;
+  if (band + 1 < g.n_bands) {
+    const int y = first + static_cast<int>(blockIdx.y);
+    if (y < 0 || y >= g.in_rows) return;
+    float* row = dx + (static_cast<size_t>(n) * g.in_rows + y) * row_floats;
+    for (int i = threadIdx.x; i < row_floats; i += 256) row[i] = 0.f;
+  } else {
+    for (int y = first + (kWin - kStride) + static_cast<int>(blockIdx.y);
+         y < g.in_rows; y += kWin - kStride) {
+      if (y < 0) continue;
+      float* row = dx + (static_cast<size_t>(n) * g.in_rows + y) * row_floats;
+      for (int i = threadIdx.x; i < row_floats; i += 256) row[i] = 0.f;
+    }
+  }
 }
 
 }  // namespace
@@ -839,12 +865,10 @@ int launch_conv2d_stem_input_backprop_f32(const float* dy, const float* w,
   StemGeom g;
   if (!conv2d_stem_input_backprop_supports(p) || !make_geom(p, &g))
     return SNN_HIP_INVALID_ALGORITHM;
-  const size_t n_vec =
-      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * kCh / 4;
-  hipLaunchKernelGGL(stem_zero_fill_kernel,
-                     dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
-                     dim3(256), 0, stream, reinterpret_cast<float4v*>(dx),
-                     n_vec);
+  hipLaunchKernelGGL(stem_zero_rows_kernel,
+                     dim3(static_cast<unsigned>(p.batch * g.n_bands),
+                          kWin - kStride),
+                     dim3(256), 0, stream, dx, g);
   const size_t lds_bytes =
       (static_cast<size_t>(g.lds_rows + 1) * g.row_floats + 64) * sizeof(float);
   static const hipError_t attr = hipFuncSetAttribute(

@@ -142,6 +142,7 @@ def test_stem_rows_in_lds_kernel(batch, rows, cols, same):
     (60, 64, 64, True),     # bands of three steps, two-row last band
     (40, 97, 61, True),     # 49 x 31 output: ragged pixel block, odd rows
     (45, 85, 100, False),   # no padding
+    (46, 86, 100, False),   # ... and a last input row that no window reads
     (17, 223, 221, True),   # odd image, padding 3
     (16, 224, 224, True),   # the stem layer itself
 ])
@@ -153,6 +154,17 @@ def test_stem_input_backprop_rows_in_lds_kernel(batch, rows, cols, same):
     assert batch * p.out_rows >= 1792
     conv_case(p, DIRECTION.INPUT_BACKPROP, [ALGO.IM2COL],
               seed=370 + batch + rows)
+    # The kernel stores most rows, adds into the rows two bands share and
+    # writes nothing where no window reaches: whatever dX held before must be
+    # gone everywhere.
+    rng = np.random.default_rng(371 + batch + rows)
+    n_dy, n_fil, n_dx = ops.conv_sizes(p, DIRECTION.INPUT_BACKPROP)
+    dy, w = uniform(rng, n_dy), uniform(rng, n_fil)
+    ref = oracle.conv2d_input_backprop(dy, w, oracle_params(p, 64), acc64=True)
+    out = torch.full((n_dx,), float("nan"), device="cuda")
+    ops.conv2d(dev(dy), dev(w), p, DIRECTION.INPUT_BACKPROP, ALGO.IM2COL,
+               out=out)
+    assert_close(out.cpu().numpy(), ref, ("stem input gradient over NaN", p))
 
 
 def test_config0_single_image_tiled():
