@@ -1774,7 +1774,9 @@ static int launch_input_backprop_col2im(const float* dy, const float* filter,
 }
 
 static int launch_filter_backprop(const float* x, const float* dy, float* dw,
-                           const snn_hip_conv2d_params& p, hipStream_t stream) {
+                                  const snn_hip_conv2d_params& p,
+                                  float* workspace, size_t workspace_elems,
+                                  hipStream_t stream) {
   FilterBackpropGeom g;
   g.batch = p.batch; g.in_rows = p.in_rows; g.in_cols = p.in_cols;
   g.channels = p.channels; g.out_rows = p.out_rows; g.out_cols = p.out_cols;
@@ -1792,6 +1794,32 @@ static int launch_filter_backprop(const float* x, const float* dy, float* dw,
       (reinterpret_cast<uintptr_t>(dw) & 15u) == 0 &&
       SNN_TUNING_ENV("SNN_HIP_STEM_OFF") == nullptr)
     return launch_conv2d_stem_filter_backprop_f32(x, dy, dw, p, stream);
+  if (conv2d_filter_backprop_1x1_f32_supports(p) &&
+      SNN_TUNING_ENV("SNN_HIP_FB1X1_OFF") == nullptr) {
+    // partial filters go to the workspace when it holds them, else to a
+    // stream-ordered temporary
+    const size_t part_floats = conv2d_filter_backprop_1x1_f32_partial_floats(p);
+    float* part = workspace;
+    const bool own =
+        part_floats != 0 &&
+        (workspace == nullptr ||
+         (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0 ||
+         workspace_elems < part_floats);
+    if (own) {
+      void* ptr = nullptr;
+      if (temp_malloc_async(&ptr, part_floats * sizeof(float), stream) !=
+          hipSuccess)
+        return SNN_HIP_ALLOCATION_PROBLEM;
+      part = static_cast<float*>(ptr);
+    }
+    const int status =
+        launch_conv2d_filter_backprop_1x1_f32(x, dy, dw, part, p, stream);
+    const hipError_t err = hipGetLastError();
+    if (own) temp_free_async(part, stream);
+    if (status != SNN_HIP_OK) return status;
+    if (err != hipSuccess) return report_hip_error(err, "1x1 filter backprop");
+    return SNN_HIP_OK;
+  }
   if (p.channels % 64 != 0) {
     // few (tap, channel) pairs: one work-group column per 64 features, the
     // pixel range split over about two work-groups per CU
@@ -2183,7 +2211,8 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
     return launch_input_backprop_col2im(input, filter, output, p, workspace,
                                         workspace_elems, stream);
   if (direction == SNN_HIP_FILTER_BACKPROP) {
-    const int rc = launch_filter_backprop(input, filter, output, p, stream);
+    const int rc = launch_filter_backprop(input, filter, output, p, workspace,
+                                          workspace_elems, stream);
     SNN_HIP_CHECK_LAUNCH();
     return rc;
   }

@@ -367,10 +367,16 @@ __global__ void __launch_bounds__(64 * WF * WP)
         for (int j = 0; j < PB; ++j) rb[j] = rb_next[j];
       }
       if constexpr (MULTI) {
-        // End of the channel block.  Vector-memory loads complete in order,
-        // so the next tile, issued at the block's start, has landed once the
-        // filter loads of the block's later units have been waited for.
-        __syncthreads();
+        // End of the channel block.  Vector-memory loads complete in order:
+        // the next tile was issued at the block's start, so it has landed
+        // once only the filter loads of the last two units (2 * kFA each)
+        // can still be outstanding.  No fence: this tile's pixel fragments
+        // have all been read into registers, and the barrier alone makes
+        // every wave's part of the next tile visible.
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (4 * kFA));
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
         const int t = cur_off;
         cur_off = nxt_off;
         nxt_off = t;
@@ -432,16 +438,19 @@ __global__ void __launch_bounds__(64 * WF * WP)
           // End of the channel block.  Vector-memory loads complete in order:
           // the next tile was issued before the filter loads of all units but
           // the first, so it has landed once only the last two units' filter
-          // loads (four each) can still be outstanding.  (The compiler adds
-          // its own, stricter wait before a barrier that follows LDS-direct
-          // loads.)
+          // loads (four each) can still be outstanding.  No fence: this
+          // tile's pixel fragments have all been read into registers, and
+          // the barrier alone makes every wave's part of the next tile
+          // visible.
           if (units_per_chunk >= 3)
             __builtin_amdgcn_s_waitcnt(kWaitVm8);
           else if (units_per_chunk == 2)
             __builtin_amdgcn_s_waitcnt(kWaitVm4);
           else
             __builtin_amdgcn_s_waitcnt(kWaitVm0);
-          __syncthreads();
+          __builtin_amdgcn_sched_barrier(0);
+          __builtin_amdgcn_s_barrier();
+          __builtin_amdgcn_sched_barrier(0);
           unsigned char* const t = const_cast<unsigned char*>(cur);
           cur = nxt;
           nxt = t;

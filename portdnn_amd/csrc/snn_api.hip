@@ -363,6 +363,16 @@ int workspace_size(const snn_hip_conv2d_params& p, int direction,
     default:
       break;
   }
+  // The 1x1 filter gradient behind the Tiled / Im2col / Matmul tags puts
+  // partial filters there when it is given the room (else it takes a
+  // stream-ordered temporary).
+  if (filbk &&
+      (algorithm == SNN_HIP_ALGO_TILED || algorithm == SNN_HIP_ALGO_IM2COL ||
+       algorithm == SNN_HIP_ALGO_MATMUL) &&
+      algorithm_supports(p, direction, algorithm) == algorithm &&
+      conv2d_filter_backprop_1x1_f32_supports(p))
+    *recommended = std::max(
+        *recommended, conv2d_filter_backprop_1x1_f32_partial_floats(p));
   return SNN_HIP_OK;
 }
 
@@ -447,11 +457,13 @@ int launch_gemm_path<float>(int direction, const float* input,
                             const snn_hip_conv2d_params& p, hipStream_t s,
                             float* workspace, size_t workspace_elems,
                             const LaunchOptions* epilogue) {
-  // The implicit-GEMM filter gradient always meets its partial tiles through
-  // float atomics; a launch that must be reproducible takes the direct kernel
-  // (one lane per filter element, fixed order) instead.
+  // The implicit-GEMM filter gradient meets its partial tiles through float
+  // atomics; a launch that must be reproducible takes the direct kernel (one
+  // lane per filter element, fixed order) instead.  The 1x1 kernel adds in a
+  // fixed order and serves both.
   const bool atomics_only = direction == SNN_HIP_FILTER_BACKPROP &&
-                            epilogue != nullptr && epilogue->deterministic;
+                            epilogue != nullptr && epilogue->deterministic &&
+                            !conv2d_filter_backprop_1x1_f32_supports(p);
   if (conv2d_igemm_supports(direction, p) && aligned16(input) &&
       aligned16(filter) && aligned16(output) && !atomics_only)
     return launch_conv2d_igemm_f32(direction, input, filter, output, p, s,

@@ -336,6 +336,59 @@ def test_reduction_split_over_waves_kernel(shape):
 
 
 @pytest.mark.parametrize("shape", [
+    (32, 7, 7, 512, 2048),   # one work-group per tile: written once
+    (32, 14, 14, 256, 1024), # four work-groups per tile
+    (5, 9, 11, 64, 128),     # pixel count not a multiple of 4
+    (3, 20, 20, 192, 64),    # 3 tiles, waves past the end with no pixels
+    (2, 12, 12, 64, 64),     # one tile, 9 steps a wave
+    (8, 28, 28, 128, 512),
+])
+def test_filter_gradient_of_1x1_layers_from_registers(shape):
+    """The filter gradient of 1x1 stride-1 unpadded layers (channels and
+    features multiples of 64) runs on the kernel that feeds both NHWC operands
+    straight into the matrix instruction, the pixel range split over the waves
+    of a work-group and, for few tiles, over work-groups whose partial filters
+    a second kernel adds: against the oracle over the whole tensor, through
+    every tag that reaches it; partial filters in a temporary, in a workspace
+    of the size the query recommends and past one too small or misaligned;
+    everything is added in a fixed order, so every call gives the same bits,
+    the reproducible entry point included."""
+    batch, rows, cols, ch, feats = shape
+    p = ops.ConvParams(channels=ch, features=feats, batch=batch, in_rows=rows,
+                       in_cols=cols, window_rows=1, window_cols=1,
+                       stride_rows=1, stride_cols=1)
+    ops.add_padding_to(p, False)
+    rng = np.random.default_rng(3100 + rows + ch)
+    direction = DIRECTION.FILTER_BACKPROP
+    n_in, n_fil, _ = ops.conv_sizes(p, direction)
+    a, w = uniform(rng, n_in), uniform(rng, n_fil)
+    ref = ORACLE_FN[direction](a, w, oracle_params(p, feats), acc64=True)
+    da, dw = dev(a), dev(w)
+    first = None
+    for algo in (ALGO.MATMUL, ALGO.TILED, ALGO.IM2COL):
+        if not supported(p, direction, algo):
+            continue
+        got = ops.conv2d(da, dw, p, direction, algo)
+        assert_close(got.cpu().numpy(), ref,
+                     ("1x1 filter gradient", ALGO_NAME[algo], shape))
+        if first is None:
+            first = got
+        assert torch.equal(got.view(torch.int32), first.view(torch.int32))
+    _, rec = ops.workspace_size(p, direction, ALGO.MATMUL)
+    # (one work-group per tile -- as many tiles as compute units, or too few
+    # steps of 4 pixels to split further than over the 8 waves -- needs none)
+    tiles = (ch // 64) * (feats // 64)
+    steps = (batch * rows * cols + 3) // 4
+    assert (rec == 0) == (max(1, min(256 // tiles, steps // 64)) == 1), rec
+    room = torch.full((rec + 8,), float("nan"), device="cuda")
+    for ws in (room[:rec], room[1:rec + 1], room[:max(rec - 4, 0)]):
+        got = ops.conv2d(da, dw, p, direction, ALGO.MATMUL, workspace=ws)
+        assert torch.equal(got.view(torch.int32), first.view(torch.int32))
+    got = ops.conv2d_deterministic(da, dw, p, direction, ALGO.MATMUL)
+    assert torch.equal(got.view(torch.int32), first.view(torch.int32))
+
+
+@pytest.mark.parametrize("shape", [
     # ragged / edge shapes: odd sizes, C and K not multiples of the tiles,
     # non-square windows and strides, VALID padding
     (3, 13, 17, 5, 7, 3, 3, 1, 1, True),
