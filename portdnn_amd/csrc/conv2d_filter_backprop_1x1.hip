@@ -40,6 +40,7 @@ constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
 constexpr int kWaves = 8;         // shares of a work-group's pixel range
 constexpr int kTile = 64;         // channels and features per tile
 constexpr int kDepth = 4;         // steps of 4 pixels in flight per wave
+                                  // (3 and 6 measured the same)
 constexpr int kComputeUnits = 256;
 constexpr int kMinStepsPerWave = 8;
 constexpr size_t kLdsBytes = kWaves * kTile * kTile * sizeof(float);
@@ -58,18 +59,21 @@ __device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* p,
                                            0x00020000);
 }
 
-// dW = sum of the partial filters, in split order: 64 float4 columns x 4
-// groups of splits per work-group, the groups meeting in LDS.
+// dW = sum of the partial filters, in a fixed order: COLS float4 columns x
+// 256 / COLS groups of splits per work-group (group g adds splits g, g +
+// groups, ...), the groups meeting in LDS.
+template <int COLS>
 __global__ void __launch_bounds__(256)
     filter_backprop_1x1_reduce_kernel(const float4* __restrict__ part,
                                       float4* __restrict__ dw, unsigned n_vec,
                                       int splits) {
-  __shared__ float4 sums[4][64];
-  const int col_l = threadIdx.x & 63, sg = threadIdx.x >> 6;
-  const unsigned col = blockIdx.x * 64 + col_l;  // n_vec % 64 == 0
+  constexpr int kGroups = 256 / COLS;
+  __shared__ float4 sums[kGroups][COLS];
+  const int col_l = threadIdx.x % COLS, sg = threadIdx.x / COLS;
+  const unsigned col = blockIdx.x * COLS + col_l;  // n_vec % 64 == 0
   float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll 4
-  for (int s = sg; s < splits; s += 4) {
+  for (int s = sg; s < splits; s += kGroups) {
     const float4 v = part[static_cast<size_t>(s) * n_vec + col];
     sum.x += v.x;
     sum.y += v.y;
@@ -80,7 +84,7 @@ __global__ void __launch_bounds__(256)
   __syncthreads();
   if (sg == 0) {
 #pragma unroll
-    for (int t = 1; t < 4; ++t) {
+    for (int t = 1; t < kGroups; ++t) {
       const float4 v = sums[t][col_l];
       sum.x += v.x;
       sum.y += v.y;
@@ -283,10 +287,17 @@ int launch_conv2d_filter_backprop_1x1_f32(const float* x, const float* dy,
                        static_cast<unsigned>(plan.splits * dw_elems * 4),
                        static_cast<unsigned>(dw_elems * 4), n_groups);
     const unsigned n_vec = static_cast<unsigned>(dw_elems / 4);
-    hipLaunchKernelGGL(filter_backprop_1x1_reduce_kernel, dim3(n_vec / 64),
-                       dim3(256), 0, stream,
-                       reinterpret_cast<const float4*>(partial),
-                       reinterpret_cast<float4*>(dw), n_vec, plan.splits);
+    // (few columns and many splits: narrower work-groups, more of them)
+    if (n_vec / 64 >= 128 || plan.splits <= 4)
+      hipLaunchKernelGGL(filter_backprop_1x1_reduce_kernel<64>,
+                         dim3(n_vec / 64), dim3(256), 0, stream,
+                         reinterpret_cast<const float4*>(partial),
+                         reinterpret_cast<float4*>(dw), n_vec, plan.splits);
+    else
+      hipLaunchKernelGGL(filter_backprop_1x1_reduce_kernel<16>,
+                         dim3(n_vec / 16), dim3(256), 0, stream,
+                         reinterpret_cast<const float4*>(partial),
+                         reinterpret_cast<float4*>(dw), n_vec, plan.splits);
   } else {
     hipLaunchKernelGGL(filter_backprop_1x1_f32_kernel, dim3(n_groups),
                        dim3(64 * kWaves), kLdsBytes, stream, x, dy, dw, plan.g,

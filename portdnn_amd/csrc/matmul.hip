@@ -124,6 +124,39 @@ int launch_matmul_f32(const float* lhs, const float* rhs, float* output,
     return launch_batched_gemm_mfma_f32(lhs, rhs, output, batches, m, k, n,
                                         stream, transpose_rhs, accumulate);
   }
+  // A^T B with both operands stored [k x .]: the filter gradient of a 1x1
+  // convolution over k pixels with m channels and n features, on its kernel
+  // (partial results, if any, in a stream-ordered temporary).
+  if (transpose_lhs && !transpose_rhs && batches == 1 && beta == 0.f &&
+      ((reinterpret_cast<uintptr_t>(lhs) | reinterpret_cast<uintptr_t>(rhs) |
+        reinterpret_cast<uintptr_t>(output)) & 15u) == 0) {
+    snn_hip_conv2d_params p = {};
+    p.batch = 1;
+    p.in_rows = p.out_rows = 1;
+    p.in_cols = p.out_cols = k;
+    p.window_rows = p.window_cols = 1;
+    p.stride_rows = p.stride_cols = 1;
+    p.dilation_rows = p.dilation_cols = 1;
+    p.groups = 1;
+    p.channels = m;
+    p.features = n;
+    if (conv2d_filter_backprop_1x1_f32_supports(p)) {
+      const size_t part_floats =
+          conv2d_filter_backprop_1x1_f32_partial_floats(p);
+      void* part = nullptr;
+      if (part_floats != 0 &&
+          temp_malloc_async(&part, part_floats * sizeof(float), stream) !=
+              hipSuccess)
+        return SNN_HIP_ALLOCATION_PROBLEM;
+      const int status = launch_conv2d_filter_backprop_1x1_f32(
+          lhs, rhs, output, static_cast<float*>(part), p, stream);
+      const hipError_t err = hipGetLastError();
+      if (part != nullptr) temp_free_async(part, stream);
+      if (status != SNN_HIP_OK) return status;
+      SNN_HIP_TRY(err);
+      return SNN_HIP_OK;
+    }
+  }
   const dim3 grid(static_cast<unsigned>(ceil_div(m, kTile)),
                   static_cast<unsigned>(ceil_div(n, kTile)),
                   static_cast<unsigned>(batches));

@@ -1004,6 +1004,30 @@ def test_matmul(trans_a, trans_b, shape):
 
 
 @pytest.mark.parametrize("shape", [
+    # m, k, n of A^T B with A stored [k x m]
+    (64, 25088, 256),    # one row of tiles, the reduction split 64 ways
+    (128, 1001, 192),    # k not a multiple of 4
+    (64, 263, 64),       # a single tile
+    (1024, 2048, 1024),  # more tiles than compute units
+])
+def test_matmul_transposed_lhs_on_the_filter_gradient_kernel(shape):
+    """A^T * B with m and n multiples of 64 is the filter gradient of a 1x1
+    convolution over k pixels and runs on its matrix-core kernel; nothing is
+    written past the result."""
+    m, k, n = shape
+    rng = np.random.default_rng(sum(shape) + 23)
+    a, b = uniform(rng, k * m), uniform(rng, k * n)
+    ref = oracle.matmul(a, b, 1, m, k, n, True, False, 0.0)
+    out = torch.full((m * n + 64,), 7.0, device="cuda")
+    got = ops.matmul(dev(a), dev(b), 1, m, k, n, True, False, 0.0,
+                     out=out[:m * n])
+    assert_close(got.cpu().numpy(), ref, ("matmul A^T B", shape))
+    assert torch.all(out[m * n:] == 7.0)
+    again = ops.matmul(dev(a), dev(b), 1, m, k, n, True, False, 0.0)
+    assert torch.equal(got.view(torch.int32), again.view(torch.int32))
+
+
+@pytest.mark.parametrize("shape", [
     # batches, m, k, n: shapes that take the plain-rows kernel
     (1, 6390, 256, 1000),   # 112-row tiles: 57 full + 6 rows, 24 columns short
     (1, 16390, 64, 252),    # 64-row tiles, ragged last row tile and column tile
