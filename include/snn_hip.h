@@ -230,9 +230,9 @@ SNN_HIP_API int snn_hip_conv2d_filter_backprop_f16(
  * meet through float atomics -- the implicit-GEMM filter gradient (Im2col /
  * Tiled / Direct-fallback tags) always, except for the 7x7 stride-2
  * three-channel stem from 224 output rows over the batch upwards and for
- * 1x1 stride-1 unpadded layers with channels and features in multiples of
- * 64 (16-byte aligned operands, at least 256 pixels), whose partial filters
- * are summed in a fixed order; forward and input gradients of small
+ * layers with channels and features in multiples of 64 (16-byte aligned
+ * operands, at least 256 output pixels), whose partial filters are summed in
+ * a fixed order; forward and input gradients of small
  * problems (fewer than ~640 64x64 output tiles, unless one of the kernels
  * that sum their parts in a fixed order takes the launch: stride-1 layers
  * with channels in multiples of 128, forward problems of fewer than 128
@@ -245,7 +245,7 @@ SNN_HIP_API int snn_hip_conv2d_filter_backprop_f16(
  * entry points (`direction` is a snn_hip_direction) with a fixed order of
  * additions: no reduction splits (small problems run on fewer work-groups),
  * and a filter gradient outside the Winograd algorithm runs on the direct
- * kernel, one lane per filter element (the 1x1 layers named above keep their
+ * kernel, one lane per filter element (the layers named above keep their
  * kernel).  Two calls with the same arguments
  * return bit-identical results.  Workspace sizes are those of
  * snn_hip_conv2d_workspace_size. */

@@ -1,0 +1,399 @@
+// fp32 filter gradient on MFMA (gfx950) with both operands loaded from memory
+// straight into the matrix instruction's registers:
+//   dW[r][s][c][k] = sum over output pixels m of X[m shifted by (r, s)][c] * dY[m][k]
+// (portDNN: a matmul with the left operand transposed for 1x1 windows,
+// src/conv2d/matmul, and the im2col / tiled filter-gradient kernels otherwise,
+// include/portdnn/conv2d/launch.h:59-118 with conv_type::FilterBackprop).
+//
+// The reduction index (the pixel) is the slow dimension of both NHWC operands,
+// which is exactly how v_mfma_f32_16x16x4_f32 wants them: lane l supplies
+// A[row l % 16][k = l / 16] and B[k = l / 16][column l % 16], i.e. for both
+// operands element [pixel m0 + l / 16][16 consecutive positions].  Letting row
+// i of accumulator block e stand for channel c0 + 4 i + e (and column j of
+// block f for feature k0 + 4 j + f) turns one 16-byte load per lane -- 4
+// pixels x 64 consecutive channels per wave, 256 contiguous bytes per pixel --
+// into the A operands of four blocks, and the same for dY.  So a wave owns a
+// 64 x 64 tile of one filter tap of dW (4 x 4 blocks, 64 accumulators) and per
+// step of 4 pixels issues two loads and 16 matrix instructions: no LDS, no
+// barrier and no transposition anywhere in the reduction loop, and the
+// operands stream from L2 into a rotation of register buffers a few steps
+// ahead.  With a window the input pixel of a lane is the output pixel moved by
+// the tap; taps that fall into the padding load zeros (offset out of range).
+//
+// The pixel range of a (tap, tile) unit is split over the 8 waves of a
+// work-group, whose partial tiles meet in LDS and are added in wave order, and
+// -- where there are fewer units than compute units -- over several
+// work-groups, which write their sums as partial filters [split][R S C][K]
+// (float atomics on dW measured 14 us per call for the million additions of a
+// batch-32 layer) for a second kernel to add in a fixed order.  Either way the
+// result is reproducible.
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+
+#include "gemm_tile.h"
+#include "snn_kernels.h"
+
+namespace snn {
+namespace {
+
+using gemm::xcd_remap;
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
+constexpr unsigned kOob = 0x7FFFFFF0u;
+constexpr int kWaves = 8;         // shares of a work-group's pixel range
+constexpr int kTile = 64;         // channels and features per tile
+constexpr int kDepth = 4;         // steps of 4 pixels in flight per wave
+                                  // (3 and 6 measured the same)
+constexpr int kComputeUnits = 256;
+constexpr int kMinStepsPerWave = 8;
+constexpr size_t kLdsBytes = kWaves * kTile * kTile * sizeof(float);
+constexpr double kMaxPartialBytes = 256.0 * 1024 * 1024;
+
+struct XtDy {
+  int m_total;         // output pixels: batch * out_rows * out_cols
+  int channels, features;
+  int c_tiles;         // channels / 64
+  int n_units;         // taps * c_tiles * features / 64
+  int steps_per_wave;  // steps of 4 pixels per wave
+  // windows only
+  int taps, win_cols;
+  int in_rows, in_cols, out_rows, out_cols;
+  int stride_rows, stride_cols, pad_rows, pad_cols;
+};
+
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* p,
+                                                   unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes,
+                                           0x00020000);
+}
+
+// dW = sum of the partial filters, in a fixed order: COLS float4 columns x
+// 256 / COLS groups of splits per work-group (group g adds splits g, g +
+// groups, ...), the groups meeting in LDS.
+template <int COLS>
+__global__ void __launch_bounds__(256)
+    filter_backprop_direct_reduce_kernel(const float4* __restrict__ part,
+                                      float4* __restrict__ dw, unsigned n_vec,
+                                      int splits) {
+  constexpr int kGroups = 256 / COLS;
+  __shared__ float4 sums[kGroups][COLS];
+  const int col_l = threadIdx.x % COLS, sg = threadIdx.x / COLS;
+  const unsigned col = blockIdx.x * COLS + col_l;  // n_vec % 64 == 0
+  float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 4
+  for (int s = sg; s < splits; s += kGroups) {
+    const float4 v = part[static_cast<size_t>(s) * n_vec + col];
+    sum.x += v.x;
+    sum.y += v.y;
+    sum.z += v.z;
+    sum.w += v.w;
+  }
+  sums[sg][col_l] = sum;
+  __syncthreads();
+  if (sg == 0) {
+#pragma unroll
+    for (int t = 1; t < kGroups; ++t) {
+      const float4 v = sums[t][col_l];
+      sum.x += v.x;
+      sum.y += v.y;
+      sum.z += v.z;
+      sum.w += v.w;
+    }
+    dw[col] = sum;
+  }
+}
+
+// `out`: dW, or the partial filters when a unit's pixels are split over
+// work-groups (`split_bytes` apart, else 0).  WINDOW: any window, stride and
+// padding; otherwise 1x1, stride 1, unpadded, where X is one flat matrix.
+template <bool WINDOW>
+__global__ void __launch_bounds__(64 * kWaves)
+    filter_backprop_direct_f32_kernel(const float* __restrict__ x,
+                                      const float* __restrict__ dy,
+                                      float* __restrict__ out, XtDy g,
+                                      unsigned x_bytes, unsigned out_bytes,
+                                      unsigned split_bytes, unsigned n_groups) {
+  extern __shared__ __align__(16) float lds[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // Units vary fastest (taps first): the work-groups an XCD runs side by side
+  // share pixel ranges (and with them operand rows in its L2).
+  const unsigned group = xcd_remap(blockIdx.x, n_groups);
+  const int split = static_cast<int>(group / g.n_units);
+  const int unit = static_cast<int>(group % g.n_units);
+  const int tap = WINDOW ? unit % g.taps : 0;
+  const int tile = WINDOW ? unit / g.taps : unit;
+  const int c0 = (tile % g.c_tiles) * kTile;
+  const int k0 = (tile / g.c_tiles) * kTile;
+
+  const int share = split * kWaves + wave;
+  const int m_begin = min(g.m_total, share * g.steps_per_wave * 4);
+  const int m_end = min(g.m_total, m_begin + g.steps_per_wave * 4);
+  const int n_steps = (m_end - m_begin + 3) >> 2;
+
+  // Loads of dY past this wave's last pixel fall out of the buffer's range
+  // and return zeros: the range ends where the wave's share ends (which also
+  // cancels whatever X holds there).
+  const unsigned x_row = static_cast<unsigned>(g.channels) * 4u;
+  const unsigned y_row = static_cast<unsigned>(g.features) * 4u;
+  const __amdgpu_buffer_rsrc_t x_rsrc =
+      make_rsrc(x, WINDOW ? x_bytes : static_cast<unsigned>(m_end) * x_row);
+  const __amdgpu_buffer_rsrc_t y_rsrc =
+      make_rsrc(dy, static_cast<unsigned>(m_end) * y_row);
+  const int l16 = lane & 15, quad = lane >> 4;
+  const unsigned x_col = static_cast<unsigned>(c0 + 4 * l16) * 4u;
+  unsigned vx = static_cast<unsigned>(m_begin + quad) * x_row + x_col;
+  unsigned vy = static_cast<unsigned>(m_begin + quad) * y_row +
+                static_cast<unsigned>(k0 + 4 * l16) * 4u;
+  // windows: the output pixel this lane loads next, as (image, row, column),
+  // and the tap's displacement
+  int px_n = 0, px_y = 0, px_x = 0, tap_y = 0, tap_x = 0;
+  if constexpr (WINDOW) {
+    const int m = m_begin + quad;
+    px_x = m % g.out_cols;
+    const int t = m / g.out_cols;
+    px_y = t % g.out_rows;
+    px_n = t / g.out_rows;
+    tap_y = tap / g.win_cols - g.pad_rows;
+    tap_x = tap % g.win_cols - g.pad_cols;
+  }
+
+  float4v xa[kDepth], yb[kDepth];
+  auto issue = [&](int d) {
+    if constexpr (WINDOW) {
+      const int iy = px_y * g.stride_rows + tap_y;
+      const int ix = px_x * g.stride_cols + tap_x;
+      // all ones where the tap falls outside the image (mask arithmetic: a
+      // per-lane condition around the load would become a branch)
+      const unsigned bad =
+          0u - static_cast<unsigned>(
+                   (static_cast<unsigned>(iy) >= static_cast<unsigned>(g.in_rows)) |
+                   (static_cast<unsigned>(ix) >= static_cast<unsigned>(g.in_cols)));
+      const unsigned off =
+          static_cast<unsigned>((px_n * g.in_rows + iy) * g.in_cols + ix) * x_row +
+          x_col;
+      vx = (off & ~bad) | (kOob & bad);
+      px_x += 4;
+      while (px_x >= g.out_cols) {
+        px_x -= g.out_cols;
+        if (++px_y == g.out_rows) {
+          px_y = 0;
+          ++px_n;
+        }
+      }
+    }
+    xa[d] = __builtin_bit_cast(
+        float4v, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, vx, 0, 0));
+    yb[d] = __builtin_bit_cast(
+        float4v, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, vy, 0, 0));
+    if constexpr (!WINDOW) vx += 4u * x_row;
+    vy += 4u * y_row;
+  };
+  float4v acc[4][4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+#pragma unroll
+    for (int f = 0; f < 4; ++f)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[e][f][v] = 0.f;
+  auto multiply = [&](int d) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int f = 0; f < 4; ++f)
+        acc[e][f] = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[d][e], yb[d][f],
+                                                         acc[e][f], 0, 0, 0);
+  };
+
+  // (the scheduling barriers keep the loads in the order the loop's waits
+  // count on: the oldest pair outstanding is the one multiplied next)
+#pragma unroll
+  for (int d = 0; d < kDepth; ++d) {
+    issue(d);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  int s = 0;
+  for (; s + kDepth <= n_steps; s += kDepth) {
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) {
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(d);
+      __builtin_amdgcn_sched_barrier(0);
+      issue(d);  // step s + d + kDepth (zeros past the end)
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  const int rest = n_steps - s;
+#pragma unroll
+  for (int d = 0; d < kDepth - 1; ++d)
+    if (d < rest) multiply(d);
+
+  // The 8 partial tiles meet in LDS: [wave][64 channels][64 features].
+  float* const mine = lds + wave * (kTile * kTile);
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int row = 16 * quad + 4 * v + e;
+      *reinterpret_cast<float4*>(mine + row * kTile + 4 * l16) =
+          make_float4(acc[e][0][v], acc[e][1][v], acc[e][2][v], acc[e][3][v]);
+    }
+  __syncthreads();
+  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_bytes);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int idx = tid + 64 * kWaves * i;  // float4 of the tile
+    float4 sum = *reinterpret_cast<const float4*>(lds + 4 * idx);
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) {
+      const float4 part =
+          *reinterpret_cast<const float4*>(lds + w * (kTile * kTile) + 4 * idx);
+      sum.x += part.x;
+      sum.y += part.y;
+      sum.z += part.z;
+      sum.w += part.w;
+    }
+    const int row = idx >> 4, col = (idx & 15) * 4;
+    const unsigned off =
+        static_cast<unsigned>(split) * split_bytes +
+        (static_cast<unsigned>(tap * g.channels + c0 + row) *
+             static_cast<unsigned>(g.features) +
+         static_cast<unsigned>(k0 + col)) * 4u;
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, sum),
+                                           out_rsrc, off, 0, 0);
+  }
+}
+
+struct Plan {
+  XtDy g;
+  int splits;   // work-groups per (tap, tile) unit
+  bool window;  // anything but 1x1, stride 1, unpadded
+};
+
+Plan make_plan(const snn_hip_conv2d_params& p) {
+  Plan plan;
+  XtDy& g = plan.g;
+  g.m_total = p.batch * p.out_rows * p.out_cols;
+  g.channels = p.channels;
+  g.features = p.features;
+  g.c_tiles = p.channels / kTile;
+  g.taps = p.window_rows * p.window_cols;
+  g.win_cols = p.window_cols;
+  g.in_rows = p.in_rows;   g.in_cols = p.in_cols;
+  g.out_rows = p.out_rows; g.out_cols = p.out_cols;
+  g.stride_rows = p.stride_rows; g.stride_cols = p.stride_cols;
+  g.pad_rows = p.pad_rows; g.pad_cols = p.pad_cols;
+  g.n_units = g.taps * g.c_tiles * (p.features / kTile);
+  plan.window = g.taps != 1 || p.stride_rows != 1 || p.stride_cols != 1 ||
+                p.pad_rows != 0 || p.pad_cols != 0 ||
+                p.in_rows != p.out_rows || p.in_cols != p.out_cols;
+  const int total_steps = ceil_div(g.m_total, 4);
+  // Work-groups per unit: the count with the least estimated time.  A compute
+  // unit holds one work-group (128 KB of LDS), so the launch runs in rounds of
+  // 256; a wave's step is 16 matrix instructions of 32 cycles sharing a SIMD
+  // with another wave (0.49 us), a round costs about 4 us of first loads and
+  // LDS reduction on top, and partial filters are written and read back at
+  // about 4 MB per us plus the second launch.
+  const double dw_bytes = 4.0 * g.taps * p.channels * p.features;
+  const int max_splits = std::max(
+      1, std::min({kComputeUnits, total_steps / (kWaves * kMinStepsPerWave),
+                   static_cast<int>(kMaxPartialBytes / dw_bytes)}));
+  int splits = 1;
+  double best = -1;
+  for (int sp = 1; sp <= max_splits; ++sp) {
+    const int rounds = ceil_div(g.n_units * sp, kComputeUnits);
+    const int steps = ceil_div(total_steps, sp * kWaves);
+    double t = rounds * (steps * 0.49 + 4.0);
+    if (sp > 1) t += 2.0 * sp * dw_bytes / 4e6 + 3.0;
+    if (best < 0 || t < best) {
+      best = t;
+      splits = sp;
+    }
+  }
+  g.steps_per_wave = ceil_div(total_steps, splits * kWaves);
+  plan.splits = ceil_div(total_steps, g.steps_per_wave * kWaves);
+  return plan;
+}
+
+}  // namespace
+
+bool conv2d_filter_backprop_direct_f32_supports(
+    const snn_hip_conv2d_params& p) {
+  if (p.channels % kTile != 0 || p.features % kTile != 0) return false;
+  const size_t m = static_cast<size_t>(p.batch) * p.out_rows * p.out_cols;
+  if (m < 4 * kWaves * kMinStepsPerWave) return false;
+  // every byte offset a lane forms, prefetch past the end included
+  const size_t rows = m + 4 * (kDepth + 1);
+  if (rows * p.features * sizeof(float) > kMaxBufferBytes) return false;
+  const size_t in_rows = static_cast<size_t>(p.batch + 1) * p.in_rows *
+                             p.in_cols + 4 * (kDepth + 1);
+  if (in_rows * p.channels * sizeof(float) > kMaxBufferBytes) return false;
+  return static_cast<size_t>(p.window_rows) * p.window_cols * p.channels *
+             p.features * sizeof(float) <= kMaxBufferBytes;
+}
+
+size_t conv2d_filter_backprop_direct_f32_partial_floats(
+    const snn_hip_conv2d_params& p) {
+  const Plan plan = make_plan(p);
+  if (plan.splits == 1) return 0;
+  return static_cast<size_t>(plan.splits) * plan.g.taps * p.channels *
+         p.features;
+}
+
+int launch_conv2d_filter_backprop_direct_f32(const float* x, const float* dy,
+                                             float* dw, float* partial,
+                                             const snn_hip_conv2d_params& p,
+                                             hipStream_t stream) {
+  const Plan plan = make_plan(p);
+  const size_t dw_elems =
+      static_cast<size_t>(plan.g.taps) * p.channels * p.features;
+  const size_t x_bytes = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                         p.channels * sizeof(float);
+  const unsigned n_groups = static_cast<unsigned>(plan.g.n_units) *
+                            static_cast<unsigned>(plan.splits);
+  static const hipError_t attr_flat = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(filter_backprop_direct_f32_kernel<false>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  static const hipError_t attr_window = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(filter_backprop_direct_f32_kernel<true>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  if (attr_flat != hipSuccess || attr_window != hipSuccess)
+    return SNN_HIP_DEVICE_ERROR;
+  if (plan.splits > 1 && partial == nullptr) return SNN_HIP_INVALID_PARAMETER;
+  float* const out = plan.splits > 1 ? partial : dw;
+  const unsigned out_bytes = static_cast<unsigned>(plan.splits * dw_elems * 4);
+  const unsigned split_bytes =
+      plan.splits > 1 ? static_cast<unsigned>(dw_elems * 4) : 0u;
+  KernelTimer timer(stream);
+  if (plan.window)
+    hipLaunchKernelGGL(filter_backprop_direct_f32_kernel<true>, dim3(n_groups),
+                       dim3(64 * kWaves), kLdsBytes, stream, x, dy, out, plan.g,
+                       static_cast<unsigned>(x_bytes), out_bytes, split_bytes,
+                       n_groups);
+  else
+    hipLaunchKernelGGL(filter_backprop_direct_f32_kernel<false>, dim3(n_groups),
+                       dim3(64 * kWaves), kLdsBytes, stream, x, dy, out, plan.g,
+                       static_cast<unsigned>(x_bytes), out_bytes, split_bytes,
+                       n_groups);
+  if (plan.splits > 1) {
+    const unsigned n_vec = static_cast<unsigned>(dw_elems / 4);
+    // (few columns and many splits: narrower work-groups, more of them)
+    if (n_vec / 64 >= 128 || plan.splits <= 4)
+      hipLaunchKernelGGL(filter_backprop_direct_reduce_kernel<64>,
+                         dim3(n_vec / 64), dim3(256), 0, stream,
+                         reinterpret_cast<const float4*>(partial),
+                         reinterpret_cast<float4*>(dw), n_vec, plan.splits);
+    else
+      hipLaunchKernelGGL(filter_backprop_direct_reduce_kernel<16>,
+                         dim3(n_vec / 16), dim3(256), 0, stream,
+                         reinterpret_cast<const float4*>(partial),
+                         reinterpret_cast<float4*>(dw), n_vec, plan.splits);
+  }
+  return SNN_HIP_OK;
+}
+
+}  // namespace snn

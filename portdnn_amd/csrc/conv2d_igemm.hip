@@ -1794,11 +1794,11 @@ static int launch_filter_backprop(const float* x, const float* dy, float* dw,
       (reinterpret_cast<uintptr_t>(dw) & 15u) == 0 &&
       SNN_TUNING_ENV("SNN_HIP_STEM_OFF") == nullptr)
     return launch_conv2d_stem_filter_backprop_f32(x, dy, dw, p, stream);
-  if (conv2d_filter_backprop_1x1_f32_supports(p) &&
-      SNN_TUNING_ENV("SNN_HIP_FB1X1_OFF") == nullptr) {
+  if (conv2d_filter_backprop_direct_f32_supports(p) &&
+      SNN_TUNING_ENV("SNN_HIP_FBDIRECT_OFF") == nullptr) {
     // partial filters go to the workspace when it holds them, else to a
     // stream-ordered temporary
-    const size_t part_floats = conv2d_filter_backprop_1x1_f32_partial_floats(p);
+    const size_t part_floats = conv2d_filter_backprop_direct_f32_partial_floats(p);
     float* part = workspace;
     const bool own =
         part_floats != 0 &&
@@ -1813,11 +1813,11 @@ static int launch_filter_backprop(const float* x, const float* dy, float* dw,
       part = static_cast<float*>(ptr);
     }
     const int status =
-        launch_conv2d_filter_backprop_1x1_f32(x, dy, dw, part, p, stream);
+        launch_conv2d_filter_backprop_direct_f32(x, dy, dw, part, p, stream);
     const hipError_t err = hipGetLastError();
     if (own) temp_free_async(part, stream);
     if (status != SNN_HIP_OK) return status;
-    if (err != hipSuccess) return report_hip_error(err, "1x1 filter backprop");
+    if (err != hipSuccess) return report_hip_error(err, "filter backprop");
     return SNN_HIP_OK;
   }
   if (p.channels % 64 != 0) {

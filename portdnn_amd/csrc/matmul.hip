@@ -140,15 +140,15 @@ int launch_matmul_f32(const float* lhs, const float* rhs, float* output,
     p.groups = 1;
     p.channels = m;
     p.features = n;
-    if (conv2d_filter_backprop_1x1_f32_supports(p)) {
+    if (conv2d_filter_backprop_direct_f32_supports(p)) {
       const size_t part_floats =
-          conv2d_filter_backprop_1x1_f32_partial_floats(p);
+          conv2d_filter_backprop_direct_f32_partial_floats(p);
       void* part = nullptr;
       if (part_floats != 0 &&
           temp_malloc_async(&part, part_floats * sizeof(float), stream) !=
               hipSuccess)
         return SNN_HIP_ALLOCATION_PROBLEM;
-      const int status = launch_conv2d_filter_backprop_1x1_f32(
+      const int status = launch_conv2d_filter_backprop_direct_f32(
           lhs, rhs, output, static_cast<float*>(part), p, stream);
       const hipError_t err = hipGetLastError();
       if (part != nullptr) temp_free_async(part, stream);

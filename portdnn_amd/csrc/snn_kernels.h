@@ -147,18 +147,18 @@ int launch_conv2d_rowsplit_f32(const float* input, const float* filter,
                                float* output, const snn_hip_conv2d_params& p,
                                hipStream_t stream, bool transposed_filter,
                                const LaunchOptions* epilogue = nullptr);
-// Filter gradient of 1x1 stride-1 unpadded convolutions
-// (conv2d_filter_backprop_1x1.hip): both operands straight from NHWC memory
-// into the matrix instruction's registers, a 64 x 64 tile of dW per wave, the
-// pixel range split over the waves of a work-group (added in LDS) and, for
-// few tiles, over work-groups, whose partial filters (`partial`,
-// ..._partial_floats(p) floats, 16-byte aligned; may be null when that is 0)
-// a second kernel adds in a fixed order.  Channels and features in multiples
-// of 64, all pointers 16-byte aligned.
-bool conv2d_filter_backprop_1x1_f32_supports(const snn_hip_conv2d_params& p);
-size_t conv2d_filter_backprop_1x1_f32_partial_floats(
+// fp32 filter gradient with both operands straight from NHWC memory into the
+// matrix instruction's registers (conv2d_filter_backprop_direct.hip): a 64 x
+// 64 tile of one filter tap of dW per wave, the pixel range split over the
+// waves of a work-group (added in LDS) and, for few (tap, tile) units, over
+// work-groups, whose partial filters (`partial`, ..._partial_floats(p) floats,
+// 16-byte aligned; may be null when that is 0) a second kernel adds in a fixed
+// order.  Any window, stride and padding; channels and features in multiples
+// of 64, at least 256 output pixels, all pointers 16-byte aligned.
+bool conv2d_filter_backprop_direct_f32_supports(const snn_hip_conv2d_params& p);
+size_t conv2d_filter_backprop_direct_f32_partial_floats(
     const snn_hip_conv2d_params& p);
-int launch_conv2d_filter_backprop_1x1_f32(const float* input,
+int launch_conv2d_filter_backprop_direct_f32(const float* input,
                                           const float* output_gradient,
                                           float* filter_gradient,
                                           float* partial,

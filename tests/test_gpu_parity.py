@@ -336,55 +336,65 @@ def test_reduction_split_over_waves_kernel(shape):
 
 
 @pytest.mark.parametrize("shape", [
-    (32, 7, 7, 512, 2048),   # one work-group per tile: written once
-    (32, 14, 14, 256, 1024), # four work-groups per tile
-    (5, 9, 11, 64, 128),     # pixel count not a multiple of 4
-    (3, 20, 20, 192, 64),    # 3 tiles, waves past the end with no pixels
-    (2, 12, 12, 64, 64),     # one tile, 9 steps a wave
-    (8, 28, 28, 128, 512),
+    # batch, rows, cols, channels, features, window, stride, SAME
+    (32, 7, 7, 512, 2048, 1, 1, 1, 1, False),   # one work-group per tile
+    (32, 14, 14, 256, 1024, 1, 1, 1, 1, False), # four work-groups per tile
+    (5, 9, 11, 64, 128, 1, 1, 1, 1, False),     # pixel count not a multiple of 4
+    (3, 20, 20, 192, 64, 1, 1, 1, 1, False),    # waves past the end, no pixels
+    (2, 12, 12, 64, 64, 1, 1, 1, 1, False),     # one tile, 9 steps a wave
+    (8, 28, 28, 128, 512, 1, 1, 1, 1, False),
+    (8, 14, 14, 128, 64, 3, 3, 1, 1, True),     # 3x3 SAME: 9 taps, padding
+    (4, 28, 28, 64, 128, 3, 3, 2, 2, True),     # 3x3 stride 2
+    (4, 28, 28, 128, 256, 1, 1, 2, 2, False),   # 1x1 stride 2
+    (6, 20, 18, 64, 64, 5, 3, 1, 2, False),     # VALID, 5x3 window, strides 1x2
+    (40, 7, 3, 64, 64, 3, 3, 1, 1, True),       # rows shorter than a step
+    (8, 7, 7, 256, 128, 3, 3, 1, 1, True),
 ])
-def test_filter_gradient_of_1x1_layers_from_registers(shape):
-    """The filter gradient of 1x1 stride-1 unpadded layers (channels and
-    features multiples of 64) runs on the kernel that feeds both NHWC operands
-    straight into the matrix instruction, the pixel range split over the waves
-    of a work-group and, for few tiles, over work-groups whose partial filters
-    a second kernel adds: against the oracle over the whole tensor, through
-    every tag that reaches it; partial filters in a temporary, in a workspace
-    of the size the query recommends and past one too small or misaligned;
-    everything is added in a fixed order, so every call gives the same bits,
-    the reproducible entry point included."""
-    batch, rows, cols, ch, feats = shape
+def test_filter_gradient_from_registers(shape):
+    """The filter gradient of layers with channels and features in multiples
+    of 64 (behind the Tiled / Im2col / Matmul tags) runs on the kernel that
+    feeds both NHWC operands straight into the matrix instruction -- one (tap,
+    64 x 64 tile) unit per work-group, the pixel range split over its waves
+    and, for few units, over work-groups whose partial filters a second kernel
+    adds: against the oracle over the whole tensor, through every tag that
+    reaches it; partial filters in a temporary, in a workspace of the size the
+    query recommends and past one too small or misaligned; everything is added
+    in a fixed order, so every call gives the same bits, the reproducible
+    entry point included."""
+    batch, rows, cols, ch, feats, wr, wc, sr, sc, same = shape
     p = ops.ConvParams(channels=ch, features=feats, batch=batch, in_rows=rows,
-                       in_cols=cols, window_rows=1, window_cols=1,
-                       stride_rows=1, stride_cols=1)
-    ops.add_padding_to(p, False)
-    rng = np.random.default_rng(3100 + rows + ch)
+                       in_cols=cols, window_rows=wr, window_cols=wc,
+                       stride_rows=sr, stride_cols=sc)
+    ops.add_padding_to(p, same)
+    rng = np.random.default_rng(3100 + rows + ch + wr)
     direction = DIRECTION.FILTER_BACKPROP
     n_in, n_fil, _ = ops.conv_sizes(p, direction)
     a, w = uniform(rng, n_in), uniform(rng, n_fil)
     ref = ORACLE_FN[direction](a, w, oracle_params(p, feats), acc64=True)
     da, dw = dev(a), dev(w)
-    first = None
+    first, tag = None, None
     for algo in (ALGO.MATMUL, ALGO.TILED, ALGO.IM2COL):
         if not supported(p, direction, algo):
             continue
         got = ops.conv2d(da, dw, p, direction, algo)
         assert_close(got.cpu().numpy(), ref,
-                     ("1x1 filter gradient", ALGO_NAME[algo], shape))
+                     ("filter gradient", ALGO_NAME[algo], shape))
         if first is None:
-            first = got
+            first, tag = got, algo
         assert torch.equal(got.view(torch.int32), first.view(torch.int32))
-    _, rec = ops.workspace_size(p, direction, ALGO.MATMUL)
-    # (one work-group per tile -- as many tiles as compute units, or too few
+    assert first is not None
+    _, rec = ops.workspace_size(p, direction, tag)
+    # (one work-group per unit -- as many units as compute units, or too few
     # steps of 4 pixels to split further than over the 8 waves -- needs none)
-    tiles = (ch // 64) * (feats // 64)
-    steps = (batch * rows * cols + 3) // 4
-    assert (rec == 0) == (max(1, min(256 // tiles, steps // 64)) == 1), rec
+    units = wr * wc * (ch // 64) * (feats // 64)
+    steps = (batch * p.out_rows * p.out_cols + 3) // 4
+    if max(1, min(256 // units, steps // 64)) > 1:
+        assert rec >= 2 * wr * wc * ch * feats, rec
     room = torch.full((rec + 8,), float("nan"), device="cuda")
-    for ws in (room[:rec], room[1:rec + 1], room[:max(rec - 4, 0)]):
-        got = ops.conv2d(da, dw, p, direction, ALGO.MATMUL, workspace=ws)
+    for ws in (room[:rec], room[1:rec + 1], room[:max(rec // 2 - 4, 0)]):
+        got = ops.conv2d(da, dw, p, direction, tag, workspace=ws)
         assert torch.equal(got.view(torch.int32), first.view(torch.int32))
-    got = ops.conv2d_deterministic(da, dw, p, direction, ALGO.MATMUL)
+    got = ops.conv2d_deterministic(da, dw, p, direction, tag)
     assert torch.equal(got.view(torch.int32), first.view(torch.int32))
 
 
