@@ -55,8 +55,8 @@ constexpr double kMaxPartialBytes = 256.0 * 1024 * 1024;
 struct XtDy {
   int m_total;         // output pixels: batch * out_rows * out_cols
   int channels, features;
-  int c_tiles;         // channels / 64
-  int n_units;         // taps * c_tiles * features / 64
+  int c_tiles;         // ceil(channels / 64)
+  int n_units;         // taps * c_tiles * ceil(features / 64)
   int steps_per_wave;  // steps of 4 pixels per wave
   // windows only
   int taps, win_cols;
@@ -81,10 +81,11 @@ __global__ void __launch_bounds__(256)
   constexpr int kGroups = 256 / COLS;
   __shared__ float4 sums[kGroups][COLS];
   const int col_l = threadIdx.x % COLS, sg = threadIdx.x / COLS;
-  const unsigned col = blockIdx.x * COLS + col_l;  // n_vec % 64 == 0
+  const unsigned col = blockIdx.x * COLS + col_l;
+  const int mine = col < n_vec ? splits : 0;  // past the end: nothing to add
   float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll 4
-  for (int s = sg; s < splits; s += kGroups) {
+  for (int s = sg; s < mine; s += kGroups) {
     const float4 v = part[static_cast<size_t>(s) * n_vec + col];
     sum.x += v.x;
     sum.y += v.y;
@@ -102,7 +103,7 @@ __global__ void __launch_bounds__(256)
       sum.z += v.z;
       sum.w += v.w;
     }
-    dw[col] = sum;
+    if (col < n_vec) dw[col] = sum;
   }
 }
 
@@ -146,9 +147,19 @@ __global__ void __launch_bounds__(64 * kWaves)
       make_rsrc(dy, static_cast<unsigned>(m_end) * y_row);
   const int l16 = lane & 15, quad = lane >> 4;
   const unsigned x_col = static_cast<unsigned>(c0 + 4 * l16) * 4u;
-  unsigned vx = static_cast<unsigned>(m_begin + quad) * x_row + x_col;
-  unsigned vy = static_cast<unsigned>(m_begin + quad) * y_row +
-                static_cast<unsigned>(k0 + 4 * l16) * 4u;
+  // Channels / features past the end (counts that are not multiples of 64):
+  // those lanes load zeros from out of range, and stay there.
+  const bool x_live = c0 + 4 * l16 < g.channels;
+  const bool y_live = k0 + 4 * l16 < g.features;
+  unsigned vx = x_live
+                    ? static_cast<unsigned>(m_begin + quad) * x_row + x_col
+                    : kOob;
+  unsigned vy = y_live ? static_cast<unsigned>(m_begin + quad) * y_row +
+                             static_cast<unsigned>(k0 + 4 * l16) * 4u
+                       : kOob;
+  const unsigned x_step = x_live ? 4u * x_row : 0u;
+  const unsigned y_step = y_live ? 4u * y_row : 0u;
+  const unsigned x_dead = x_live ? 0u : ~0u;
   // windows: the output pixel this lane loads next, as (image, row, column),
   // and the tap's displacement
   int px_n = 0, px_y = 0, px_x = 0, tap_y = 0, tap_x = 0;
@@ -170,9 +181,10 @@ __global__ void __launch_bounds__(64 * kWaves)
       // all ones where the tap falls outside the image (mask arithmetic: a
       // per-lane condition around the load would become a branch)
       const unsigned bad =
-          0u - static_cast<unsigned>(
-                   (static_cast<unsigned>(iy) >= static_cast<unsigned>(g.in_rows)) |
-                   (static_cast<unsigned>(ix) >= static_cast<unsigned>(g.in_cols)));
+          x_dead |
+          (0u - static_cast<unsigned>(
+                    (static_cast<unsigned>(iy) >= static_cast<unsigned>(g.in_rows)) |
+                    (static_cast<unsigned>(ix) >= static_cast<unsigned>(g.in_cols))));
       const unsigned off =
           static_cast<unsigned>((px_n * g.in_rows + iy) * g.in_cols + ix) * x_row +
           x_col;
@@ -190,8 +202,8 @@ __global__ void __launch_bounds__(64 * kWaves)
         float4v, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, vx, 0, 0));
     yb[d] = __builtin_bit_cast(
         float4v, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, vy, 0, 0));
-    if constexpr (!WINDOW) vx += 4u * x_row;
-    vy += 4u * y_row;
+    if constexpr (!WINDOW) vx += x_step;
+    vy += y_step;
   };
   float4v acc[4][4];
 #pragma unroll
@@ -263,8 +275,10 @@ __global__ void __launch_bounds__(64 * kWaves)
         (static_cast<unsigned>(tap * g.channels + c0 + row) *
              static_cast<unsigned>(g.features) +
          static_cast<unsigned>(k0 + col)) * 4u;
+    // (rows and columns past the end of a ragged tile: dropped, out of range)
+    const bool live = c0 + row < g.channels && k0 + col < g.features;
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, sum),
-                                           out_rsrc, off, 0, 0);
+                                           out_rsrc, live ? off : kOob, 0, 0);
   }
 }
 
@@ -280,14 +294,14 @@ Plan make_plan(const snn_hip_conv2d_params& p) {
   g.m_total = p.batch * p.out_rows * p.out_cols;
   g.channels = p.channels;
   g.features = p.features;
-  g.c_tiles = p.channels / kTile;
+  g.c_tiles = ceil_div(p.channels, kTile);
   g.taps = p.window_rows * p.window_cols;
   g.win_cols = p.window_cols;
   g.in_rows = p.in_rows;   g.in_cols = p.in_cols;
   g.out_rows = p.out_rows; g.out_cols = p.out_cols;
   g.stride_rows = p.stride_rows; g.stride_cols = p.stride_cols;
   g.pad_rows = p.pad_rows; g.pad_cols = p.pad_cols;
-  g.n_units = g.taps * g.c_tiles * (p.features / kTile);
+  g.n_units = g.taps * g.c_tiles * ceil_div(p.features, kTile);
   plan.window = g.taps != 1 || p.stride_rows != 1 || p.stride_cols != 1 ||
                 p.pad_rows != 0 || p.pad_cols != 0 ||
                 p.in_rows != p.out_rows || p.in_cols != p.out_cols;
@@ -321,9 +335,11 @@ Plan make_plan(const snn_hip_conv2d_params& p) {
 
 }  // namespace
 
-bool conv2d_filter_backprop_direct_f32_supports(
-    const snn_hip_conv2d_params& p) {
-  if (p.channels % kTile != 0 || p.features % kTile != 0) return false;
+bool conv2d_filter_backprop_direct_f32_supports(const snn_hip_conv2d_params& p,
+                                                bool ragged) {
+  // whole tiles, or (ragged) lanes that load 16 bytes inside one pixel
+  const int unit = ragged ? 4 : kTile;
+  if (p.channels % unit != 0 || p.features % unit != 0) return false;
   const size_t m = static_cast<size_t>(p.batch) * p.out_rows * p.out_cols;
   if (m < 4 * kWaves * kMinStepsPerWave) return false;
   // every byte offset a lane forms, prefetch past the end included
@@ -384,12 +400,12 @@ int launch_conv2d_filter_backprop_direct_f32(const float* x, const float* dy,
     // (few columns and many splits: narrower work-groups, more of them)
     if (n_vec / 64 >= 128 || plan.splits <= 4)
       hipLaunchKernelGGL(filter_backprop_direct_reduce_kernel<64>,
-                         dim3(n_vec / 64), dim3(256), 0, stream,
+                         dim3(ceil_div(n_vec, 64u)), dim3(256), 0, stream,
                          reinterpret_cast<const float4*>(partial),
                          reinterpret_cast<float4*>(dw), n_vec, plan.splits);
     else
       hipLaunchKernelGGL(filter_backprop_direct_reduce_kernel<16>,
-                         dim3(n_vec / 16), dim3(256), 0, stream,
+                         dim3(ceil_div(n_vec, 16u)), dim3(256), 0, stream,
                          reinterpret_cast<const float4*>(partial),
                          reinterpret_cast<float4*>(dw), n_vec, plan.splits);
   }

@@ -1773,6 +1773,17 @@ static int launch_input_backprop_col2im(const float* dy, const float* filter,
   return SNN_HIP_OK;
 }
 
+// Whole 64 x 64 tiles; channel counts that are neither multiples of 64 nor
+// few enough for the one-work-group kernel also take it, with ragged tiles
+// (no other matrix-core kernel fits them).
+bool conv2d_filter_backprop_direct_f32_wanted(const snn_hip_conv2d_params& p) {
+  const bool ragged_only =
+      p.channels % 64 != 0 &&
+      p.window_rows * p.window_cols * p.channels > kSmallQMax;
+  return conv2d_filter_backprop_direct_f32_supports(p, ragged_only) &&
+         (ragged_only || SNN_TUNING_ENV("SNN_HIP_FBDIRECT_OFF") == nullptr);
+}
+
 static int launch_filter_backprop(const float* x, const float* dy, float* dw,
                                   const snn_hip_conv2d_params& p,
                                   float* workspace, size_t workspace_elems,
@@ -1794,8 +1805,7 @@ static int launch_filter_backprop(const float* x, const float* dy, float* dw,
       (reinterpret_cast<uintptr_t>(dw) & 15u) == 0 &&
       SNN_TUNING_ENV("SNN_HIP_STEM_OFF") == nullptr)
     return launch_conv2d_stem_filter_backprop_f32(x, dy, dw, p, stream);
-  if (conv2d_filter_backprop_direct_f32_supports(p) &&
-      SNN_TUNING_ENV("SNN_HIP_FBDIRECT_OFF") == nullptr) {
+  if (conv2d_filter_backprop_direct_f32_wanted(p)) {
     // partial filters go to the workspace when it holds them, else to a
     // stream-ordered temporary
     const size_t part_floats = conv2d_filter_backprop_direct_f32_partial_floats(p);
@@ -2083,7 +2093,8 @@ bool conv2d_igemm_supports(int direction, const snn_hip_conv2d_params& p) {
   // tap, or the whole (tap, channel) range must fit one work-group
   return p.features % 4 == 0 &&
          (p.channels % 64 == 0 ||
-          p.window_rows * p.window_cols * p.channels <= kSmallQMax);
+          p.window_rows * p.window_cols * p.channels <= kSmallQMax ||
+          conv2d_filter_backprop_direct_f32_supports(p, true));
 }
 
 bool batched_gemm_mfma_supports(int m, int k, int n, const void* a,

@@ -364,13 +364,14 @@ int workspace_size(const snn_hip_conv2d_params& p, int direction,
       break;
   }
   // The filter gradient kernel behind the Tiled / Im2col / Matmul tags
-  // (channels and features in multiples of 64) puts partial filters there
-  // when it is given the room (else it takes a stream-ordered temporary).
+  // (channels and features in multiples of 64, or ragged shapes no other
+  // matrix-core kernel fits) puts partial filters there when it is given the
+  // room (else it takes a stream-ordered temporary).
   if (filbk &&
       (algorithm == SNN_HIP_ALGO_TILED || algorithm == SNN_HIP_ALGO_IM2COL ||
        algorithm == SNN_HIP_ALGO_MATMUL) &&
       algorithm_supports(p, direction, algorithm) == algorithm &&
-      conv2d_filter_backprop_direct_f32_supports(p))
+      conv2d_filter_backprop_direct_f32_wanted(p))
     *recommended = std::max(
         *recommended, conv2d_filter_backprop_direct_f32_partial_floats(p));
   return SNN_HIP_OK;
@@ -463,7 +464,7 @@ int launch_gemm_path<float>(int direction, const float* input,
   // and features in multiples of 64 adds in a fixed order and serves both.
   const bool atomics_only = direction == SNN_HIP_FILTER_BACKPROP &&
                             epilogue != nullptr && epilogue->deterministic &&
-                            !conv2d_filter_backprop_direct_f32_supports(p);
+                            !conv2d_filter_backprop_direct_f32_wanted(p);
   if (conv2d_igemm_supports(direction, p) && aligned16(input) &&
       aligned16(filter) && aligned16(output) && !atomics_only)
     return launch_conv2d_igemm_f32(direction, input, filter, output, p, s,

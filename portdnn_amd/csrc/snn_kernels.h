@@ -154,8 +154,13 @@ int launch_conv2d_rowsplit_f32(const float* input, const float* filter,
 // work-groups, whose partial filters (`partial`, ..._partial_floats(p) floats,
 // 16-byte aligned; may be null when that is 0) a second kernel adds in a fixed
 // order.  Any window, stride and padding; channels and features in multiples
-// of 64, at least 256 output pixels, all pointers 16-byte aligned.
-bool conv2d_filter_backprop_direct_f32_supports(const snn_hip_conv2d_params& p);
+// of 64 (`ragged`: of 4, the tiles that stick out padded with zeros), at
+// least 256 output pixels, all pointers 16-byte aligned.
+bool conv2d_filter_backprop_direct_f32_supports(const snn_hip_conv2d_params& p,
+                                                bool ragged = false);
+// Whether the implicit-GEMM launcher sends this filter gradient to that kernel
+// (conv2d_igemm.hip).
+bool conv2d_filter_backprop_direct_f32_wanted(const snn_hip_conv2d_params& p);
 size_t conv2d_filter_backprop_direct_f32_partial_floats(
     const snn_hip_conv2d_params& p);
 int launch_conv2d_filter_backprop_direct_f32(const float* input,

@@ -349,6 +349,11 @@ def test_reduction_split_over_waves_kernel(shape):
     (6, 20, 18, 64, 64, 5, 3, 1, 2, False),     # VALID, 5x3 window, strides 1x2
     (40, 7, 3, 64, 64, 3, 3, 1, 1, True),       # rows shorter than a step
     (8, 7, 7, 256, 128, 3, 3, 1, 1, True),
+    # channel counts that are neither multiples of 64 nor few enough for the
+    # one-work-group kernel: ragged tiles
+    (4, 14, 14, 96, 80, 3, 3, 1, 1, True),
+    (6, 10, 10, 36, 100, 3, 3, 2, 2, True),
+    (8, 12, 12, 200, 72, 1, 1, 1, 1, False),
 ])
 def test_filter_gradient_from_registers(shape):
     """The filter gradient of layers with channels and features in multiples
@@ -386,7 +391,7 @@ def test_filter_gradient_from_registers(shape):
     _, rec = ops.workspace_size(p, direction, tag)
     # (one work-group per unit -- as many units as compute units, or too few
     # steps of 4 pixels to split further than over the 8 waves -- needs none)
-    units = wr * wc * (ch // 64) * (feats // 64)
+    units = wr * wc * ((ch + 63) // 64) * ((feats + 63) // 64)
     steps = (batch * p.out_rows * p.out_cols + 3) // 4
     if max(1, min(256 // units, steps // 64)) > 1:
         assert rec >= 2 * wr * wc * ch * feats, rec
