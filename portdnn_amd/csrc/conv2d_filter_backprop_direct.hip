@@ -1,5 +1,6 @@
-// fp32 filter gradient on MFMA (gfx950) with both operands loaded from memory
-// straight into the matrix instruction's registers:
+// Filter gradient on the fp32 MFMA (gfx950) with both operands loaded from
+// memory straight into the matrix instruction's registers (fp32 tensors, or
+// binary16 tensors converted on the way in and accumulated in fp32):
 //   dW[r][s][c][k] = sum over output pixels m of X[m shifted by (r, s)][c] * dY[m][k]
 // (portDNN: a matmul with the left operand transposed for 1x1 windows,
 // src/conv2d/matmul, and the im2col / tiled filter-gradient kernels otherwise,
@@ -27,6 +28,12 @@
 // (float atomics on dW measured 14 us per call for the million additions of a
 // batch-32 layer) for a second kernel to add in a fixed order.  Either way the
 // result is reproducible.
+//
+// Channel and feature counts that are not multiples of 64 leave the lanes of
+// a tile that stick out loading zeros from out of range and their stores
+// dropped; counts that are not multiples of 4 load and store element by
+// element (VEC == 1) -- a slow way to feed the matrix cores, but the only
+// alternative for such shapes is one lane per filter element.
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
@@ -40,7 +47,9 @@ namespace {
 using gemm::xcd_remap;
 
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
 constexpr size_t kMaxBufferBytes = 0x7FFFFFF0u;
 constexpr unsigned kOob = 0x7FFFFFF0u;
 constexpr int kWaves = 8;         // shares of a work-group's pixel range
@@ -70,54 +79,103 @@ __device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* p,
                                            0x00020000);
 }
 
-// dW = sum of the partial filters, in a fixed order: COLS float4 columns x
-// 256 / COLS groups of splits per work-group (group g adds splits g, g +
-// groups, ...), the groups meeting in LDS.
-template <int COLS>
+// Four consecutive elements of T at byte offset `off` as floats.  VEC == 4:
+// one load; VEC == 1: four, element e from out of range (zero) where dead[e]
+// is all ones.
+template <typename T, int VEC>
+__device__ inline float4v load_four(__amdgpu_buffer_rsrc_t rsrc, unsigned off,
+                                    const unsigned (&dead)[4]) {
+  float4v r;
+  if constexpr (VEC == 4) {
+    if constexpr (sizeof(T) == 4) {
+      r = __builtin_bit_cast(
+          float4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0));
+    } else {
+      const half4v h = __builtin_bit_cast(
+          half4v, __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, 0, 0));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[e] = static_cast<float>(h[e]);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const unsigned o = (off + e * static_cast<unsigned>(sizeof(T))) | dead[e];
+      if constexpr (sizeof(T) == 4) {
+        r[e] = __builtin_bit_cast(
+            float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, o, 0, 0));
+      } else {
+        r[e] = static_cast<float>(__builtin_bit_cast(
+            _Float16, __builtin_amdgcn_raw_buffer_load_b16(rsrc, o, 0, 0)));
+      }
+    }
+  }
+  return r;
+}
+
+// out = sum of the partial filters, in a fixed order, as T: COLS columns (of
+// VEC floats) x 256 / COLS groups of splits per work-group (group g adds
+// splits g, g + groups, ...), the groups meeting in LDS.
+template <typename T, int VEC, int COLS>
 __global__ void __launch_bounds__(256)
-    filter_backprop_direct_reduce_kernel(const float4* __restrict__ part,
-                                      float4* __restrict__ dw, unsigned n_vec,
-                                      int splits) {
+    filter_backprop_direct_reduce_kernel(const float* __restrict__ part,
+                                         T* __restrict__ dw, unsigned n_cols,
+                                         int splits) {
   constexpr int kGroups = 256 / COLS;
-  __shared__ float4 sums[kGroups][COLS];
+  __shared__ __align__(16) float sums[kGroups][COLS][VEC];
   const int col_l = threadIdx.x % COLS, sg = threadIdx.x / COLS;
   const unsigned col = blockIdx.x * COLS + col_l;
-  const int mine = col < n_vec ? splits : 0;  // past the end: nothing to add
-  float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+  const int mine = col < n_cols ? splits : 0;  // past the end: nothing to add
+  float sum[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) sum[e] = 0.f;
 #pragma unroll 4
   for (int s = sg; s < mine; s += kGroups) {
-    const float4 v = part[static_cast<size_t>(s) * n_vec + col];
-    sum.x += v.x;
-    sum.y += v.y;
-    sum.z += v.z;
-    sum.w += v.w;
-  }
-  sums[sg][col_l] = sum;
-  __syncthreads();
-  if (sg == 0) {
-#pragma unroll
-    for (int t = 1; t < kGroups; ++t) {
-      const float4 v = sums[t][col_l];
-      sum.x += v.x;
-      sum.y += v.y;
-      sum.z += v.z;
-      sum.w += v.w;
+    const float* const src = part + (static_cast<size_t>(s) * n_cols + col) * VEC;
+    if constexpr (VEC == 4) {
+      const float4 v = *reinterpret_cast<const float4*>(src);
+      sum[0] += v.x;
+      sum[1] += v.y;
+      sum[2] += v.z;
+      sum[3] += v.w;
+    } else {
+      sum[0] += *src;
     }
-    if (col < n_vec) dw[col] = sum;
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) sums[sg][col_l][e] = sum[e];
+  __syncthreads();
+  if (sg != 0 || col >= n_cols) return;
+#pragma unroll
+  for (int t = 1; t < kGroups; ++t)
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) sum[e] += sums[t][col_l][e];
+  T* const dst = dw + static_cast<size_t>(col) * VEC;
+  if constexpr (VEC == 1) {
+    *dst = static_cast<T>(sum[0]);
+  } else if constexpr (sizeof(T) == 4) {
+    *reinterpret_cast<float4*>(dst) = make_float4(sum[0], sum[1], sum[2], sum[3]);
+  } else {
+    half4v h;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(sum[e]);
+    *reinterpret_cast<half4v*>(dst) = h;
   }
 }
 
-// `out`: dW, or the partial filters when a unit's pixels are split over
-// work-groups (`split_bytes` apart, else 0).  WINDOW: any window, stride and
-// padding; otherwise 1x1, stride 1, unpadded, where X is one flat matrix.
-template <bool WINDOW>
+// `out` (fp32): dW, or the partial filters when a unit's pixels are split
+// over work-groups or the tensors are binary16 (`split_bytes` apart, else 0).
+// WINDOW: any window, stride and padding; otherwise 1x1, stride 1, unpadded,
+// where X is one flat matrix.  VEC: 4 = channel and feature counts in
+// multiples of 4 (vector loads and stores), 1 = any.
+template <bool WINDOW, typename T, int VEC>
 __global__ void __launch_bounds__(64 * kWaves)
-    filter_backprop_direct_f32_kernel(const float* __restrict__ x,
-                                      const float* __restrict__ dy,
-                                      float* __restrict__ out, XtDy g,
-                                      unsigned x_bytes, unsigned out_bytes,
-                                      unsigned split_bytes, unsigned n_groups) {
+    filter_backprop_direct_kernel(const T* __restrict__ x,
+                                  const T* __restrict__ dy,
+                                  float* __restrict__ out, XtDy g,
+                                  unsigned x_bytes, unsigned out_bytes,
+                                  unsigned split_bytes, unsigned n_groups) {
   extern __shared__ __align__(16) float lds[];
+  constexpr unsigned kElem = sizeof(T);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -139,23 +197,30 @@ __global__ void __launch_bounds__(64 * kWaves)
   // Loads of dY past this wave's last pixel fall out of the buffer's range
   // and return zeros: the range ends where the wave's share ends (which also
   // cancels whatever X holds there).
-  const unsigned x_row = static_cast<unsigned>(g.channels) * 4u;
-  const unsigned y_row = static_cast<unsigned>(g.features) * 4u;
+  const unsigned x_row = static_cast<unsigned>(g.channels) * kElem;
+  const unsigned y_row = static_cast<unsigned>(g.features) * kElem;
   const __amdgpu_buffer_rsrc_t x_rsrc =
       make_rsrc(x, WINDOW ? x_bytes : static_cast<unsigned>(m_end) * x_row);
   const __amdgpu_buffer_rsrc_t y_rsrc =
       make_rsrc(dy, static_cast<unsigned>(m_end) * y_row);
   const int l16 = lane & 15, quad = lane >> 4;
-  const unsigned x_col = static_cast<unsigned>(c0 + 4 * l16) * 4u;
+  const unsigned x_col = static_cast<unsigned>(c0 + 4 * l16) * kElem;
   // Channels / features past the end (counts that are not multiples of 64):
-  // those lanes load zeros from out of range, and stay there.
+  // those lanes -- with VEC == 1 those elements -- load zeros from out of
+  // range, and stay there.
   const bool x_live = c0 + 4 * l16 < g.channels;
   const bool y_live = k0 + 4 * l16 < g.features;
+  unsigned x_dead_e[4], y_dead_e[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    x_dead_e[e] = c0 + 4 * l16 + e < g.channels ? 0u : ~0u;
+    y_dead_e[e] = k0 + 4 * l16 + e < g.features ? 0u : ~0u;
+  }
   unsigned vx = x_live
                     ? static_cast<unsigned>(m_begin + quad) * x_row + x_col
                     : kOob;
   unsigned vy = y_live ? static_cast<unsigned>(m_begin + quad) * y_row +
-                             static_cast<unsigned>(k0 + 4 * l16) * 4u
+                             static_cast<unsigned>(k0 + 4 * l16) * kElem
                        : kOob;
   const unsigned x_step = x_live ? 4u * x_row : 0u;
   const unsigned y_step = y_live ? 4u * y_row : 0u;
@@ -198,10 +263,8 @@ __global__ void __launch_bounds__(64 * kWaves)
         }
       }
     }
-    xa[d] = __builtin_bit_cast(
-        float4v, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, vx, 0, 0));
-    yb[d] = __builtin_bit_cast(
-        float4v, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, vy, 0, 0));
+    xa[d] = load_four<T, VEC>(x_rsrc, vx, x_dead_e);
+    yb[d] = load_four<T, VEC>(y_rsrc, vy, y_dead_e);
     if constexpr (!WINDOW) vx += x_step;
     vy += y_step;
   };
@@ -276,9 +339,21 @@ __global__ void __launch_bounds__(64 * kWaves)
              static_cast<unsigned>(g.features) +
          static_cast<unsigned>(k0 + col)) * 4u;
     // (rows and columns past the end of a ragged tile: dropped, out of range)
-    const bool live = c0 + row < g.channels && k0 + col < g.features;
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, sum),
-                                           out_rsrc, live ? off : kOob, 0, 0);
+    const bool row_live = c0 + row < g.channels;
+    if constexpr (VEC == 4) {
+      const bool live = row_live && k0 + col < g.features;
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, sum),
+                                             out_rsrc, live ? off : kOob, 0, 0);
+    } else {
+      const float vals[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool live = row_live && k0 + col + e < g.features;
+        __builtin_amdgcn_raw_buffer_store_b32(
+            __builtin_bit_cast(unsigned, vals[e]), out_rsrc,
+            live ? off + 4u * e : kOob, 0, 0);
+      }
+    }
   }
 }
 
@@ -286,6 +361,7 @@ struct Plan {
   XtDy g;
   int splits;   // work-groups per (tap, tile) unit
   bool window;  // anything but 1x1, stride 1, unpadded
+  bool vec4;    // channels and features in multiples of 4
 };
 
 Plan make_plan(const snn_hip_conv2d_params& p) {
@@ -305,6 +381,7 @@ Plan make_plan(const snn_hip_conv2d_params& p) {
   plan.window = g.taps != 1 || p.stride_rows != 1 || p.stride_cols != 1 ||
                 p.pad_rows != 0 || p.pad_cols != 0 ||
                 p.in_rows != p.out_rows || p.in_cols != p.out_cols;
+  plan.vec4 = p.channels % 4 == 0 && p.features % 4 == 0;
   const int total_steps = ceil_div(g.m_total, 4);
   // Work-groups per unit: the count with the least estimated time.  A compute
   // unit holds one work-group (128 KB of LDS), so the launch runs in rounds of
@@ -333,23 +410,106 @@ Plan make_plan(const snn_hip_conv2d_params& p) {
   return plan;
 }
 
-}  // namespace
-
-bool conv2d_filter_backprop_direct_f32_supports(const snn_hip_conv2d_params& p,
-                                                bool ragged) {
-  // whole tiles, or (ragged) lanes that load 16 bytes inside one pixel
-  const int unit = ragged ? 4 : kTile;
-  if (p.channels % unit != 0 || p.features % unit != 0) return false;
+bool supports(const snn_hip_conv2d_params& p, bool ragged, size_t elem) {
+  // whole tiles, or (ragged) any counts
+  if (!ragged && (p.channels % kTile != 0 || p.features % kTile != 0))
+    return false;
   const size_t m = static_cast<size_t>(p.batch) * p.out_rows * p.out_cols;
   if (m < 4 * kWaves * kMinStepsPerWave) return false;
   // every byte offset a lane forms, prefetch past the end included
   const size_t rows = m + 4 * (kDepth + 1);
-  if (rows * p.features * sizeof(float) > kMaxBufferBytes) return false;
+  if (rows * p.features * elem > kMaxBufferBytes) return false;
   const size_t in_rows = static_cast<size_t>(p.batch + 1) * p.in_rows *
                              p.in_cols + 4 * (kDepth + 1);
-  if (in_rows * p.channels * sizeof(float) > kMaxBufferBytes) return false;
+  if (in_rows * p.channels * elem > kMaxBufferBytes) return false;
   return static_cast<size_t>(p.window_rows) * p.window_cols * p.channels *
              p.features * sizeof(float) <= kMaxBufferBytes;
+}
+
+template <bool WINDOW, typename T, int VEC>
+hipError_t launch_main(const T* x, const T* dy, float* out, const Plan& plan,
+                       size_t x_bytes, unsigned out_bytes, unsigned split_bytes,
+                       unsigned n_groups, hipStream_t stream) {
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(filter_backprop_direct_kernel<WINDOW, T, VEC>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  if (attr != hipSuccess) return attr;
+  hipLaunchKernelGGL((filter_backprop_direct_kernel<WINDOW, T, VEC>),
+                     dim3(n_groups), dim3(64 * kWaves), kLdsBytes, stream, x, dy,
+                     out, plan.g, static_cast<unsigned>(x_bytes), out_bytes,
+                     split_bytes, n_groups);
+  return hipSuccess;
+}
+
+template <typename T, int VEC>
+void launch_reduce(const float* partial, T* dw, size_t dw_elems, int splits,
+                   hipStream_t stream) {
+  const unsigned n_cols = static_cast<unsigned>(dw_elems / VEC);
+  // (few columns and many splits: narrower work-groups, more of them)
+  if (n_cols / 64 >= 128 || splits <= 4)
+    hipLaunchKernelGGL((filter_backprop_direct_reduce_kernel<T, VEC, 64>),
+                       dim3(ceil_div(n_cols, 64u)), dim3(256), 0, stream,
+                       partial, dw, n_cols, splits);
+  else
+    hipLaunchKernelGGL((filter_backprop_direct_reduce_kernel<T, VEC, 16>),
+                       dim3(ceil_div(n_cols, 16u)), dim3(256), 0, stream,
+                       partial, dw, n_cols, splits);
+}
+
+// T == float: dW written by the main kernel when one work-group owns a unit;
+// otherwise partial filters and the reduce kernel (which also rounds to T).
+template <typename T>
+int launch(const T* x, const T* dy, T* dw, float* partial,
+           const snn_hip_conv2d_params& p, hipStream_t stream) {
+  const Plan plan = make_plan(p);
+  const size_t dw_elems =
+      static_cast<size_t>(plan.g.taps) * p.channels * p.features;
+  const size_t x_bytes = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                         p.channels * sizeof(T);
+  const unsigned n_groups = static_cast<unsigned>(plan.g.n_units) *
+                            static_cast<unsigned>(plan.splits);
+  const bool direct = sizeof(T) == 4 && plan.splits == 1;
+  if (!direct && partial == nullptr) return SNN_HIP_INVALID_PARAMETER;
+  float* const out = direct ? reinterpret_cast<float*>(dw) : partial;
+  const unsigned out_bytes = static_cast<unsigned>(plan.splits * dw_elems * 4);
+  const unsigned split_bytes =
+      plan.splits > 1 ? static_cast<unsigned>(dw_elems * 4) : 0u;
+  KernelTimer timer(stream);
+  hipError_t err;
+  if (plan.window)
+    err = plan.vec4 ? launch_main<true, T, 4>(x, dy, out, plan, x_bytes,
+                                              out_bytes, split_bytes, n_groups,
+                                              stream)
+                    : launch_main<true, T, 1>(x, dy, out, plan, x_bytes,
+                                              out_bytes, split_bytes, n_groups,
+                                              stream);
+  else
+    err = plan.vec4 ? launch_main<false, T, 4>(x, dy, out, plan, x_bytes,
+                                               out_bytes, split_bytes, n_groups,
+                                               stream)
+                    : launch_main<false, T, 1>(x, dy, out, plan, x_bytes,
+                                               out_bytes, split_bytes, n_groups,
+                                               stream);
+  if (err != hipSuccess) return SNN_HIP_DEVICE_ERROR;
+  if (!direct) {
+    if (plan.vec4)
+      launch_reduce<T, 4>(partial, dw, dw_elems, plan.splits, stream);
+    else
+      launch_reduce<T, 1>(partial, dw, dw_elems, plan.splits, stream);
+  }
+  return SNN_HIP_OK;
+}
+
+}  // namespace
+
+bool conv2d_filter_backprop_direct_f32_supports(const snn_hip_conv2d_params& p,
+                                                bool ragged) {
+  return supports(p, ragged, sizeof(float));
+}
+
+bool conv2d_filter_backprop_direct_f16_supports(
+    const snn_hip_conv2d_params& p) {
+  return supports(p, true, sizeof(_Float16));
 }
 
 size_t conv2d_filter_backprop_direct_f32_partial_floats(
@@ -360,56 +520,26 @@ size_t conv2d_filter_backprop_direct_f32_partial_floats(
          p.features;
 }
 
+size_t conv2d_filter_backprop_direct_f16_partial_floats(
+    const snn_hip_conv2d_params& p) {
+  const Plan plan = make_plan(p);
+  return static_cast<size_t>(plan.splits) * plan.g.taps * p.channels *
+         p.features;
+}
+
 int launch_conv2d_filter_backprop_direct_f32(const float* x, const float* dy,
                                              float* dw, float* partial,
                                              const snn_hip_conv2d_params& p,
                                              hipStream_t stream) {
-  const Plan plan = make_plan(p);
-  const size_t dw_elems =
-      static_cast<size_t>(plan.g.taps) * p.channels * p.features;
-  const size_t x_bytes = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
-                         p.channels * sizeof(float);
-  const unsigned n_groups = static_cast<unsigned>(plan.g.n_units) *
-                            static_cast<unsigned>(plan.splits);
-  static const hipError_t attr_flat = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(filter_backprop_direct_f32_kernel<false>),
-      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  static const hipError_t attr_window = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(filter_backprop_direct_f32_kernel<true>),
-      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  if (attr_flat != hipSuccess || attr_window != hipSuccess)
-    return SNN_HIP_DEVICE_ERROR;
-  if (plan.splits > 1 && partial == nullptr) return SNN_HIP_INVALID_PARAMETER;
-  float* const out = plan.splits > 1 ? partial : dw;
-  const unsigned out_bytes = static_cast<unsigned>(plan.splits * dw_elems * 4);
-  const unsigned split_bytes =
-      plan.splits > 1 ? static_cast<unsigned>(dw_elems * 4) : 0u;
-  KernelTimer timer(stream);
-  if (plan.window)
-    hipLaunchKernelGGL(filter_backprop_direct_f32_kernel<true>, dim3(n_groups),
-                       dim3(64 * kWaves), kLdsBytes, stream, x, dy, out, plan.g,
-                       static_cast<unsigned>(x_bytes), out_bytes, split_bytes,
-                       n_groups);
-  else
-    hipLaunchKernelGGL(filter_backprop_direct_f32_kernel<false>, dim3(n_groups),
-                       dim3(64 * kWaves), kLdsBytes, stream, x, dy, out, plan.g,
-                       static_cast<unsigned>(x_bytes), out_bytes, split_bytes,
-                       n_groups);
-  if (plan.splits > 1) {
-    const unsigned n_vec = static_cast<unsigned>(dw_elems / 4);
-    // (few columns and many splits: narrower work-groups, more of them)
-    if (n_vec / 64 >= 128 || plan.splits <= 4)
-      hipLaunchKernelGGL(filter_backprop_direct_reduce_kernel<64>,
-                         dim3(ceil_div(n_vec, 64u)), dim3(256), 0, stream,
-                         reinterpret_cast<const float4*>(partial),
-                         reinterpret_cast<float4*>(dw), n_vec, plan.splits);
-    else
-      hipLaunchKernelGGL(filter_backprop_direct_reduce_kernel<16>,
-                         dim3(ceil_div(n_vec, 16u)), dim3(256), 0, stream,
-                         reinterpret_cast<const float4*>(partial),
-                         reinterpret_cast<float4*>(dw), n_vec, plan.splits);
-  }
-  return SNN_HIP_OK;
+  return launch<float>(x, dy, dw, partial, p, stream);
+}
+
+int launch_conv2d_filter_backprop_direct_f16(const _Float16* x,
+                                             const _Float16* dy, _Float16* dw,
+                                             float* partial,
+                                             const snn_hip_conv2d_params& p,
+                                             hipStream_t stream) {
+  return launch<_Float16>(x, dy, dw, partial, p, stream);
 }
 
 }  // namespace snn

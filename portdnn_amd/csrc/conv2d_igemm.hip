@@ -1773,15 +1773,16 @@ static int launch_input_backprop_col2im(const float* dy, const float* filter,
   return SNN_HIP_OK;
 }
 
-// Whole 64 x 64 tiles; channel counts that are neither multiples of 64 nor
-// few enough for the one-work-group kernel also take it, with ragged tiles
-// (no other matrix-core kernel fits them).
+// Every shape it supports except those the one-work-group kernel takes (few
+// (tap, channel) pairs, e.g. a three-channel stem).
 bool conv2d_filter_backprop_direct_f32_wanted(const snn_hip_conv2d_params& p) {
-  const bool ragged_only =
-      p.channels % 64 != 0 &&
-      p.window_rows * p.window_cols * p.channels > kSmallQMax;
-  return conv2d_filter_backprop_direct_f32_supports(p, ragged_only) &&
-         (ragged_only || SNN_TUNING_ENV("SNN_HIP_FBDIRECT_OFF") == nullptr);
+  const bool whole = p.channels % 64 == 0 && p.features % 64 == 0;
+  const bool small_q =
+      p.channels % 64 != 0 && p.features % 4 == 0 &&
+      p.window_rows * p.window_cols * p.channels <= kSmallQMax;
+  if (small_q || !conv2d_filter_backprop_direct_f32_supports(p, true))
+    return false;
+  return !whole || SNN_TUNING_ENV("SNN_HIP_FBDIRECT_OFF") == nullptr;
 }
 
 static int launch_filter_backprop(const float* x, const float* dy, float* dw,
@@ -1932,10 +1933,11 @@ bool conv2d_filter_backprop_f16_supports(const snn_hip_conv2d_params& p) {
                    p.channels;
   const size_t y = static_cast<size_t>(p.batch) * p.out_rows * p.out_cols *
                    p.features;
-  return p.channels % 64 == 0 && p.features % 4 == 0 &&
-         max(x, y) * sizeof(_Float16) <= kMaxBufferBytes &&
-         static_cast<size_t>(p.window_rows) * p.window_cols * p.channels *
-                 p.features * sizeof(float) <= kMaxBufferBytes;
+  return (p.channels % 64 == 0 && p.features % 4 == 0 &&
+          max(x, y) * sizeof(_Float16) <= kMaxBufferBytes &&
+          static_cast<size_t>(p.window_rows) * p.window_cols * p.channels *
+                  p.features * sizeof(float) <= kMaxBufferBytes) ||
+         conv2d_filter_backprop_direct_f16_supports(p);
 }
 
 int launch_conv2d_filter_backprop_f16(const _Float16* x, const _Float16* dy,
@@ -1981,6 +1983,28 @@ int launch_conv2d_filter_backprop_f16(const _Float16* x, const _Float16* dy,
         is_3x3
             ? launch_conv2d_filter_backprop_3x3_f16(x, dy, dw, part, p, stream)
             : launch_conv2d_filter_backprop_1x1_f16(x, dy, dw, part, p, stream);
+    const hipError_t err = hipGetLastError();
+    if (own) temp_free_async(part, stream);
+    if (status != SNN_HIP_OK) return status;
+    if (err != hipSuccess) return report_hip_error(err, "f16 filter backprop");
+    return SNN_HIP_OK;
+  }
+  if (conv2d_filter_backprop_direct_f16_supports(p)) {
+    // every other shape with at least 256 output pixels: binary16 operands
+    // converted on the way into the fp32 matrix instruction's registers, fp32
+    // partial filters (workspace or temporary), one pass that adds and rounds
+    const size_t part_floats = conv2d_filter_backprop_direct_f16_partial_floats(p);
+    float* part = reinterpret_cast<float*>(workspace);
+    const bool own = !ws_aligned || workspace_elems < 2 * part_floats;
+    if (own) {
+      void* ptr = nullptr;
+      if (temp_malloc_async(&ptr, part_floats * sizeof(float), stream) !=
+          hipSuccess)
+        return SNN_HIP_ALLOCATION_PROBLEM;
+      part = static_cast<float*>(ptr);
+    }
+    const int status =
+        launch_conv2d_filter_backprop_direct_f16(x, dy, dw, part, p, stream);
     const hipError_t err = hipGetLastError();
     if (own) temp_free_async(part, stream);
     if (status != SNN_HIP_OK) return status;
@@ -2091,10 +2115,10 @@ bool conv2d_igemm_supports(int direction, const snn_hip_conv2d_params& p) {
     return p.features % 4 == 0;
   // filter backprop: a 64-wide tile of (tap, channel) must lie inside one
   // tap, or the whole (tap, channel) range must fit one work-group
-  return p.features % 4 == 0 &&
-         (p.channels % 64 == 0 ||
-          p.window_rows * p.window_cols * p.channels <= kSmallQMax ||
-          conv2d_filter_backprop_direct_f32_supports(p, true));
+  return (p.features % 4 == 0 &&
+          (p.channels % 64 == 0 ||
+           p.window_rows * p.window_cols * p.channels <= kSmallQMax)) ||
+         conv2d_filter_backprop_direct_f32_supports(p, true);
 }
 
 bool batched_gemm_mfma_supports(int m, int k, int n, const void* a,

@@ -326,6 +326,8 @@ size_t f16_workspace_halves(const snn_hip_conv2d_params& p, int direction) {
     return 2 * conv2d_filter_backprop_3x3_f16_partial_floats(p);
   if (conv2d_filter_backprop_1x1_f16_supports(p))
     return 2 * conv2d_filter_backprop_1x1_f16_partial_floats(p);
+  if (conv2d_filter_backprop_direct_f16_supports(p))
+    return 2 * conv2d_filter_backprop_direct_f16_partial_floats(p);
   return 2 * static_cast<size_t>(p.window_rows) * p.window_cols * p.channels *
          p.features;
 }

@@ -147,28 +147,40 @@ int launch_conv2d_rowsplit_f32(const float* input, const float* filter,
                                float* output, const snn_hip_conv2d_params& p,
                                hipStream_t stream, bool transposed_filter,
                                const LaunchOptions* epilogue = nullptr);
-// fp32 filter gradient with both operands straight from NHWC memory into the
+// Filter gradient with both operands straight from NHWC memory into the fp32
 // matrix instruction's registers (conv2d_filter_backprop_direct.hip): a 64 x
 // 64 tile of one filter tap of dW per wave, the pixel range split over the
 // waves of a work-group (added in LDS) and, for few (tap, tile) units, over
 // work-groups, whose partial filters (`partial`, ..._partial_floats(p) floats,
 // 16-byte aligned; may be null when that is 0) a second kernel adds in a fixed
-// order.  Any window, stride and padding; channels and features in multiples
-// of 64 (`ragged`: of 4, the tiles that stick out padded with zeros), at
-// least 256 output pixels, all pointers 16-byte aligned.
+// order.  Any window, stride and padding, at least 256 output pixels, all
+// pointers 16-byte aligned; channels and features in multiples of 64, or
+// (`ragged`) any counts: the tiles that stick out are padded with zeros, and
+// counts that are not multiples of 4 are loaded element by element.  The f16
+// form reads and writes binary16 tensors, accumulates in fp32 and always goes
+// through partial filters (at least one), which the second kernel rounds.
 bool conv2d_filter_backprop_direct_f32_supports(const snn_hip_conv2d_params& p,
                                                 bool ragged = false);
-// Whether the implicit-GEMM launcher sends this filter gradient to that kernel
-// (conv2d_igemm.hip).
+bool conv2d_filter_backprop_direct_f16_supports(const snn_hip_conv2d_params& p);
+// Whether the implicit-GEMM launcher sends this fp32 filter gradient to that
+// kernel (conv2d_igemm.hip).
 bool conv2d_filter_backprop_direct_f32_wanted(const snn_hip_conv2d_params& p);
 size_t conv2d_filter_backprop_direct_f32_partial_floats(
     const snn_hip_conv2d_params& p);
+size_t conv2d_filter_backprop_direct_f16_partial_floats(
+    const snn_hip_conv2d_params& p);
 int launch_conv2d_filter_backprop_direct_f32(const float* input,
-                                          const float* output_gradient,
-                                          float* filter_gradient,
-                                          float* partial,
-                                          const snn_hip_conv2d_params& p,
-                                          hipStream_t stream);
+                                             const float* output_gradient,
+                                             float* filter_gradient,
+                                             float* partial,
+                                             const snn_hip_conv2d_params& p,
+                                             hipStream_t stream);
+int launch_conv2d_filter_backprop_direct_f16(const _Float16* input,
+                                             const _Float16* output_gradient,
+                                             _Float16* filter_gradient,
+                                             float* partial,
+                                             const snn_hip_conv2d_params& p,
+                                             hipStream_t stream);
 // Forward convolution of a three-channel image with a 7x7 window, stride 2 and
 // 64 features (conv2d_stem.hip): input rows of a band of output rows in LDS,
 // the filter in registers.  Output 16-byte aligned, at most 128 output columns.

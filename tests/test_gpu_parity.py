@@ -1545,6 +1545,65 @@ def test_f16_filter_backprop_1x1_transposing_reads(shape):
         assert_close_f16(got, ref, ("f16 filbk 1x1", shape, ws is None))
 
 
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, window, stride, SAME
+    (8, 32, 32, 16, 16, 3, 1, True),     # ragged tiles, vector loads
+    (8, 32, 32, 24, 24, 3, 1, True),
+    (8, 32, 32, 40, 72, 1, 1, False),
+    (4, 28, 28, 144, 144, 3, 1, True),
+    (4, 28, 28, 100, 100, 5, 1, True),
+    (4, 56, 56, 12, 20, 3, 2, True),
+    (8, 28, 28, 128, 256, 1, 2, False),  # whole tiles, stride 2
+    (8, 32, 32, 3, 64, 3, 1, True),      # channels not a multiple of 4:
+    (8, 32, 32, 64, 66, 3, 1, True),     # element by element
+    (8, 32, 32, 66, 10, 1, 1, False),
+    (8, 32, 32, 64, 3, 3, 1, True),
+])
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_filter_gradient_from_registers_ragged_and_half(shape, dtype):
+    """Shapes that used to have no matrix-core filter gradient -- channel or
+    feature counts that are not multiples of 64 (binary16: any but the 3x3 and
+    1x1 stride-1 layers with whole tiles) or of 4 -- run on the kernel that
+    loads both operands straight into the fp32 matrix instruction, binary16
+    operands converted on the way, against the oracle in double precision on
+    the same operands; with and without a workspace for the partial filters;
+    twice gives the same bits."""
+    batch, rows, cols, ch, feats, window, stride, same = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, window, stride, same)
+    rng = np.random.default_rng(790 + rows + ch + feats)
+    direction = DIRECTION.FILTER_BACKPROP
+    n_x, n_dy, n_dw = ops.conv_sizes(p, direction)
+    half = dtype == "f16"
+    x, dy = uniform(rng, n_x), uniform(rng, n_dy)
+    if half:
+        x, dy = x.astype(np.float16), dy.astype(np.float16)
+    ref = oracle.conv2d_filter_backprop(x.astype(np.float32),
+                                        dy.astype(np.float32),
+                                        oracle_params(p, feats), acc64=True)
+    tdt = torch.float16 if half else torch.float32
+    dx_, ddy = dev(x, tdt), dev(dy, tdt)
+    _, rec = ops.workspace_size(p, direction, ALGO.IM2COL, dtype=(
+        capi.DTYPE.F16 if half else capi.DTYPE.F32))
+    first = None
+    for ws in (None, torch.empty(rec + 8, dtype=tdt, device="cuda")):
+        got = ops.conv2d(dx_, ddy, p, direction, ALGO.IM2COL, workspace=ws)
+        if half:
+            assert_close_f16(got.float().cpu().numpy(), ref,
+                             ("f16 filter gradient", shape, ws is None))
+        else:
+            assert_close(got.cpu().numpy(), ref,
+                         ("filter gradient", shape, ws is None))
+        if first is None:
+            first = got
+        # (fp32 layers with few (tap, channel) pairs keep the one-work-group
+        # kernel, whose partial sums meet through float atomics)
+        if (not half and ch % 64 != 0 and feats % 4 == 0 and
+                window * window * ch <= 192):
+            continue
+        assert torch.equal(got.view(torch.int16 if half else torch.int32),
+                           first.view(torch.int16 if half else torch.int32))
+
+
 def test_f16_conv_filter_backprop():
     p = ops.conv_params(3, 10, 9, 16, 24, 3, 1, True)
     rng = np.random.default_rng(781)
