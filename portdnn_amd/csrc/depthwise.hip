@@ -1096,6 +1096,74 @@ __global__ void __launch_bounds__(kStrip* kSlices)
   }
 }
 
+// The same with the output pixels also split over work-groups (blockIdx.z:
+// `per_chunk` consecutive pixels each), for launches whose (tap, strip) pairs
+// alone would leave most of the GPU idle: a slice walks its run of pixels
+// with (image, row, column) advanced incrementally, and the work-groups' sums
+// meet in the zero-filled fp32 buffer `acc` through float atomics.
+template <typename T>
+__global__ void __launch_bounds__(kStrip* kSlices)
+    dw_filter_backprop_split_kernel(const T* __restrict__ in,
+                                    const T* __restrict__ dy,
+                                    float* __restrict__ acc,
+                                    snn_hip_depthwise_params p, int per_chunk) {
+  __shared__ float partial[kSlices][kStrip];
+  const int C = p.channels, M = p.channel_multiplier;
+  const int CM = C * M;
+  const int lane = threadIdx.x % kStrip;
+  const int slice = threadIdx.x / kStrip;
+  const int cm = blockIdx.y * kStrip + lane;
+  const int s = blockIdx.x % p.window_cols;
+  const int r = blockIdx.x / p.window_cols;
+  const int c = cm / M;
+  const int n_pix = p.batch * p.out_rows * p.out_cols;
+  const int begin = blockIdx.z * per_chunk;
+  const int end = min(n_pix, begin + per_chunk);
+  const int per_slice = (end - begin + kSlices - 1) / kSlices;
+  const int first = begin + slice * per_slice;
+  const int last = min(end, first + per_slice);
+  float sum = 0.f;
+  if (cm < CM && first < last) {
+    int ox = first % p.out_cols;
+    const int t = first / p.out_cols;
+    int oy = t % p.out_rows;
+    int n = t / p.out_rows;
+#pragma unroll 4
+    for (int pix = first; pix < last; ++pix) {
+      const int y = oy * p.stride_rows - p.pad_rows + r;
+      const int x = ox * p.stride_cols - p.pad_cols + s;
+      if (y >= 0 && y < p.in_rows && x >= 0 && x < p.in_cols) {
+        const float xv = Elem<T>::load(
+            in + ((static_cast<size_t>(n) * p.in_rows + y) * p.in_cols + x) * C +
+            c);
+        const float gv = Elem<T>::load(dy + static_cast<size_t>(pix) * CM + cm);
+        sum = fmaf(xv, gv, sum);
+      }
+      if (++ox == p.out_cols) {
+        ox = 0;
+        if (++oy == p.out_rows) {
+          oy = 0;
+          ++n;
+        }
+      }
+    }
+  }
+  partial[slice][lane] = sum;
+  __syncthreads();
+  if (slice == 0 && cm < CM) {
+    sum = partial[0][lane];
+    for (int i = 1; i < kSlices; ++i) sum += partial[i][lane];
+    atomicAdd(acc + static_cast<size_t>(blockIdx.x) * CM + cm, sum);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+    dw_round_kernel(const float* __restrict__ acc, T* __restrict__ out, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = Elem<T>::from_float(acc[i]);
+}
+
 // Launches the 3x3 strip kernel with V channels per lane and a TH x TW block
 // of outputs per lane.  A lane loads (TH + 2)(TW + 2) input vectors for
 // TH * TW outputs (stride 1), so larger blocks cut the L1 traffic, but fewer
@@ -1527,11 +1595,52 @@ int launch_depthwise(int direction, const T* input, const T* filter, T* output,
       }
     }
     if (!done) {
-      const dim3 grid(static_cast<unsigned>(p.window_rows * p.window_cols),
-                      static_cast<unsigned>(ceil_div(CM, size_t{kStrip})));
-      hipLaunchKernelGGL(dw_filter_backprop_kernel<T>, grid,
-                         dim3(kStrip * kSlices), 0, stream, input, filter,
-                         output, p);
+      const int taps = p.window_rows * p.window_cols;
+      const int strips = static_cast<int>(ceil_div(CM, size_t{kStrip}));
+      // about 2048 work-groups, each slice with at least 16 pixels
+      const int chunks =
+          n_pix_sz > 0x7FFFFFFFu
+              ? 1
+              : max(1, min(2048 / (taps * strips),
+                           static_cast<int>(n_pix_sz) / (kSlices * 16)));
+      if (chunks == 1) {
+        // (one work-group per (tap, strip) walks every pixel: no atomics)
+        hipLaunchKernelGGL(dw_filter_backprop_kernel<T>,
+                           dim3(static_cast<unsigned>(taps),
+                                static_cast<unsigned>(strips)),
+                           dim3(kStrip * kSlices), 0, stream, input, filter,
+                           output, p);
+      } else {
+        // fp32 accumulation: the result itself, or for binary16 a temporary
+        // that one more pass rounds
+        const int dw_elems = taps * static_cast<int>(CM);
+        float* acc = reinterpret_cast<float*>(output);
+        if constexpr (!std::is_same<T, float>::value) {
+          void* ptr = nullptr;
+          if (temp_malloc_async(&ptr, dw_elems * sizeof(float), stream) !=
+              hipSuccess)
+            return SNN_HIP_ALLOCATION_PROBLEM;
+          acc = static_cast<float*>(ptr);
+        }
+        const int per_chunk = ceil_div(static_cast<int>(n_pix_sz), chunks);
+        hipLaunchKernelGGL(dw_zero_kernel, dim3(ceil_div(dw_elems, 256)),
+                           dim3(256), 0, stream, acc, dw_elems);
+        hipLaunchKernelGGL(
+            dw_filter_backprop_split_kernel<T>,
+            dim3(static_cast<unsigned>(taps), static_cast<unsigned>(strips),
+                 static_cast<unsigned>(
+                     ceil_div(static_cast<int>(n_pix_sz), per_chunk))),
+            dim3(kStrip * kSlices), 0, stream, input, filter, acc, p,
+            per_chunk);
+        if constexpr (!std::is_same<T, float>::value) {
+          hipLaunchKernelGGL(dw_round_kernel<T>, dim3(ceil_div(dw_elems, 256)),
+                             dim3(256), 0, stream, acc, output, dw_elems);
+          const hipError_t err = hipGetLastError();
+          temp_free_async(acc, stream);
+          if (err != hipSuccess)
+            return report_hip_error(err, "depthwise filter backprop");
+        }
+      }
     }
   }
   SNN_HIP_CHECK_LAUNCH();

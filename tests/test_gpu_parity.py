@@ -1644,6 +1644,49 @@ def test_f16_depthwise_backprops(shape):
                      ("f16 dw filbk", shape))
 
 
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, multiplier, window, stride
+    (8, 28, 28, 66, 1, 3, 1),    # channels not a multiple of 4
+    (8, 28, 28, 30, 1, 3, 2),
+    (4, 28, 28, 64, 2, 3, 1),    # channel multiplier 2
+    (4, 28, 28, 96, 1, 5, 1),    # 5x5
+    (4, 14, 14, 480, 1, 7, 1),   # 7x7
+    (4, 56, 56, 3, 8, 3, 2),     # three channels, multiplier 8
+    (8, 28, 28, 128, 1, 1, 1),   # 1x1 window
+    (4, 56, 56, 64, 1, 3, 1),    # (binary16: the MobileNet shape itself)
+])
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_depthwise_filter_gradient_general_shapes_split_over_work_groups(
+        shape, dtype):
+    """Depthwise filter gradients outside the fp32 3x3 kernels (other windows,
+    channel multipliers, channel counts that are not multiples of 4, every
+    binary16 shape) split the output pixels over work-groups whose sums meet
+    through float atomics in an fp32 buffer: against the oracle in double
+    precision on the same operands."""
+    n, h, w_, c, mult, window, stride = shape
+    p = ops.depthwise_params(n, h, w_, c, mult, window, stride, True)
+    op = oracle_params(p, mult)
+    rng = np.random.default_rng(795 + h + c + window)
+    half = dtype == "f16"
+    x = uniform(rng, n * h * w_ * c)
+    dy = uniform(rng, n * p.out_rows * p.out_cols * c * mult)
+    if half:
+        x, dy = x.astype(np.float16), dy.astype(np.float16)
+    ref = oracle.depthwise_filter_backprop(x.astype(np.float32),
+                                           dy.astype(np.float32), op)
+    tdt = torch.float16 if half else torch.float32
+    out = torch.full((window * window * c * mult + 16,), 7.0, dtype=tdt,
+                     device="cuda")
+    got = ops.depthwise_conv2d(dev(x, tdt), dev(dy, tdt), p,
+                               DIRECTION.FILTER_BACKPROP,
+                               out=out[:window * window * c * mult])
+    if half:
+        assert_close_f16(got.float().cpu().numpy(), ref, ("f16 dw filbk", shape))
+    else:
+        assert_close(got.cpu().numpy(), ref, ("dw filbk", shape))
+    assert torch.all(out[window * window * c * mult:] == 7.0)
+
+
 @pytest.mark.parametrize("size,ch,stride", MOBILENET)
 def test_f16_depthwise_forward(size, ch, stride):
     p = ops.depthwise_params(2, size, size, ch, 1, 3, stride, True)
