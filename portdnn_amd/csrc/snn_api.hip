@@ -427,12 +427,105 @@ int launch_gemm_path(int direction, const T* input, const T* filter, T* output,
                      const snn_hip_conv2d_params& p, hipStream_t s,
                      T* workspace = nullptr, size_t workspace_elems = 0,
                      const LaunchOptions* epilogue = nullptr);
+
+// out[r][j] = j < valid ? in[r][j] : 0 for j < out_cols: widens (zeros in the
+// new columns) or narrows the last dimension of a row-major matrix.
+template <typename T>
+__global__ void __launch_bounds__(256)
+    copy_columns_kernel(const T* __restrict__ in, int in_cols,
+                        T* __restrict__ out, int out_cols, int valid,
+                        size_t total) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= total) return;
+  const size_t r = i / out_cols;
+  const int j = static_cast<int>(i - r * out_cols);
+  out[i] = j < valid ? in[r * in_cols + j] : static_cast<T>(0);
+}
+
+template <typename T>
+void copy_columns(const T* in, int in_cols, T* out, int out_cols, int valid,
+                  size_t rows, hipStream_t s) {
+  const size_t total = rows * out_cols;
+  hipLaunchKernelGGL(copy_columns_kernel<T>,
+                     dim3(static_cast<unsigned>(ceil_div(total, size_t{256}))),
+                     dim3(256), 0, s, in, in_cols, out, out_cols, valid, total);
+}
+
+// Feature counts that are not multiples of 4 (an RGB output layer, 21
+// classes): the matrix-core kernels load and store features four at a time,
+// so for a forward convolution or an input gradient the tensors that carry
+// the feature dimension are copied into stream-ordered temporaries with the
+// count rounded up (zeros in the new columns), the launch runs on the padded
+// problem -- when `padded_ok` says a matrix-core kernel takes it -- and a
+// forward result is copied back without the padding.  The copies move a
+// fraction of what the one-lane-per-output kernel would otherwise read.
+// Returns -1 when it does not apply.
+template <typename T, typename Supports>
+int launch_gemm_path_padded(int direction, const T* input, const T* filter,
+                            T* output, const snn_hip_conv2d_params& p,
+                            hipStream_t s, const LaunchOptions* epilogue,
+                            Supports padded_ok) {
+  if (direction == SNN_HIP_FILTER_BACKPROP || p.features % 4 == 0) return -1;
+  if (epilogue != nullptr && epilogue->wanted()) return -1;  // bias has K entries
+  // (an input gradient over three features or fewer is a short loop per
+  // output: the direct kernel measured faster, 80 against 99 us)
+  if (direction == SNN_HIP_INPUT_BACKPROP && p.features < 4) return -1;
+  snn_hip_conv2d_params q = p;
+  q.features = (p.features + 3) / 4 * 4;
+  if (!padded_ok(q)) return -1;
+  const size_t pixels = static_cast<size_t>(p.batch) * p.out_rows * p.out_cols;
+  const size_t filter_rows =
+      static_cast<size_t>(p.window_rows) * p.window_cols * p.channels;
+  // (small problems stay where they were: three more launches and two
+  // temporaries cost more than the direct kernel's whole run)
+  if (pixels * filter_rows * p.features < (size_t{1} << 24)) return -1;
+  void *wide_filter = nullptr, *wide_pixels = nullptr;
+  if (temp_malloc_async(&wide_filter, filter_rows * q.features * sizeof(T), s) !=
+      hipSuccess)
+    return SNN_HIP_ALLOCATION_PROBLEM;
+  if (temp_malloc_async(&wide_pixels, pixels * q.features * sizeof(T), s) !=
+      hipSuccess) {
+    temp_free_async(wide_filter, s);
+    return SNN_HIP_ALLOCATION_PROBLEM;
+  }
+  copy_columns(filter, p.features, static_cast<T*>(wide_filter), q.features,
+               p.features, filter_rows, s);
+  int status;
+  if (direction == SNN_HIP_FORWARD) {
+    status = launch_gemm_path<T>(direction, input, static_cast<T*>(wide_filter),
+                                 static_cast<T*>(wide_pixels), q, s, nullptr, 0,
+                                 epilogue);
+    copy_columns(static_cast<const T*>(wide_pixels), q.features, output,
+                 p.features, p.features, pixels, s);
+  } else {
+    copy_columns(input, p.features, static_cast<T*>(wide_pixels), q.features,
+                 p.features, pixels, s);
+    status = launch_gemm_path<T>(direction, static_cast<T*>(wide_pixels),
+                                 static_cast<T*>(wide_filter), output, q, s,
+                                 nullptr, 0, epilogue);
+  }
+  const hipError_t err = hipGetLastError();
+  temp_free_async(wide_pixels, s);
+  temp_free_async(wide_filter, s);
+  if (status != SNN_HIP_OK) return status;
+  if (err != hipSuccess) return report_hip_error(err, "padded features");
+  return SNN_HIP_OK;
+}
 template <>
 int launch_gemm_path<_Float16>(int direction, const _Float16* input,
                                const _Float16* filter, _Float16* output,
                                const snn_hip_conv2d_params& p, hipStream_t s,
                                _Float16* workspace, size_t workspace_elems,
                                const LaunchOptions*) {
+  if (direction == SNN_HIP_INPUT_BACKPROP && aligned16(output)) {
+    const int padded = launch_gemm_path_padded<_Float16>(
+        direction, input, filter, output, p, s, nullptr,
+        [](const snn_hip_conv2d_params& q) {
+          return conv2d_input_backprop_f16_supports(q) ||
+                 conv2d_input_backprop_general_f16_supports(q);
+        });
+    if (padded >= 0) return padded;
+  }
   if (direction == SNN_HIP_FORWARD && conv2d_igemm_f16_supports(p) &&
       aligned16(input) && aligned16(filter) && aligned16(output))
     return launch_conv2d_igemm_f16(input, filter, output, p, workspace,
@@ -467,6 +560,15 @@ int launch_gemm_path<float>(int direction, const float* input,
   const bool atomics_only = direction == SNN_HIP_FILTER_BACKPROP &&
                             epilogue != nullptr && epilogue->deterministic &&
                             !conv2d_filter_backprop_direct_f32_wanted(p);
+  if ((direction == SNN_HIP_FORWARD && aligned16(input)) ||
+      (direction == SNN_HIP_INPUT_BACKPROP && aligned16(output))) {
+    const int padded = launch_gemm_path_padded<float>(
+        direction, input, filter, output, p, s, epilogue,
+        [direction](const snn_hip_conv2d_params& q) {
+          return conv2d_igemm_supports(direction, q);
+        });
+    if (padded >= 0) return padded;
+  }
   if (conv2d_igemm_supports(direction, p) && aligned16(input) &&
       aligned16(filter) && aligned16(output) && !atomics_only)
     return launch_conv2d_igemm_f32(direction, input, filter, output, p, s,

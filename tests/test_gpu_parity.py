@@ -1604,6 +1604,54 @@ def test_filter_gradient_from_registers_ragged_and_half(shape, dtype):
                            first.view(torch.int16 if half else torch.int32))
 
 
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, window, stride, SAME
+    (8, 32, 32, 64, 66, 3, 1, True),
+    (8, 64, 64, 64, 3, 3, 1, True),      # an RGB output layer
+    (8, 32, 32, 128, 21, 1, 1, False),   # 21 classes
+    (4, 33, 31, 48, 1, 3, 2, True),      # one feature, stride 2
+])
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_feature_counts_that_are_not_multiples_of_four_run_padded(shape, dtype):
+    """Forward convolutions (fp32) and input gradients (fp32, binary16) whose
+    feature count is not a multiple of 4 run on the matrix-core kernels over
+    copies of the filter and of the tensor that carries the features, widened
+    with zeros, instead of one lane per output: against the oracle in double
+    precision, nothing written past the result."""
+    batch, rows, cols, ch, feats, window, stride, same = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, window, stride, same)
+    rng = np.random.default_rng(805 + rows + ch + feats)
+    half = dtype == "f16"
+    tdt = torch.float16 if half else torch.float32
+    for direction in (DIRECTION.FORWARD, DIRECTION.INPUT_BACKPROP):
+        n_a, n_b, n_o = ops.conv_sizes(p, direction)
+        a, b = uniform(rng, n_a), uniform(rng, n_b)
+        if half:
+            a, b = a.astype(np.float16), b.astype(np.float16)
+        ref = ORACLE_FN[direction](a.astype(np.float32), b.astype(np.float32),
+                                   oracle_params(p, feats), acc64=True)
+        out = torch.full((n_o + 16,), 7.0, dtype=tdt, device="cuda")
+        got = ops.conv2d(dev(a, tdt), dev(b, tdt), p, direction, ALGO.IM2COL,
+                         out=out[:n_o])
+        if half:
+            assert_close_f16(got.float().cpu().numpy(), ref,
+                             ("f16 padded features", direction, shape))
+        else:
+            assert_close(got.cpu().numpy(), ref,
+                         ("padded features", direction, shape))
+        assert torch.all(out[n_o:] == 7.0)
+    if not half:
+        # bias and ReLU are indexed by the feature: that launch is not padded
+        n_in, n_fil, _ = ops.conv_sizes(p, DIRECTION.FORWARD)
+        x, w, bias = uniform(rng, n_in), uniform(rng, n_fil), uniform(rng, feats)
+        ref = oracle.conv2d_forward(x, w, oracle_params(p, feats), acc64=True)
+        want = np.maximum(ref.reshape(-1, feats) + bias.astype(np.float64), 0)
+        got = ops.conv2d_bias_act(dev(x), dev(w), dev(bias), p, ALGO.IM2COL,
+                                  relu=True)
+        assert_close(got.cpu().numpy(), want.reshape(-1),
+                     ("bias + relu, ragged features", shape))
+
+
 def test_f16_conv_filter_backprop():
     p = ops.conv_params(3, 10, 9, 16, 24, 3, 1, True)
     rng = np.random.default_rng(781)
