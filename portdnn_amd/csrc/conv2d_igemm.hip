@@ -2101,6 +2101,47 @@ int launch_conv2d_input_backprop_general_f16(const _Float16* dy,
   return SNN_HIP_OK;
 }
 
+// Half-precision forward convolution for the shapes the binary16 kernels do
+// not take (channel counts that are not multiples of 64, windows of more than
+// 32 taps): the same general kernel, gathering X four channels at a time.
+bool conv2d_forward_general_f16_supports(const snn_hip_conv2d_params& p) {
+  const size_t x = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *
+                   p.channels;
+  const size_t y = static_cast<size_t>(p.batch) * p.out_rows * p.out_cols *
+                   p.features;
+  const size_t w = static_cast<size_t>(p.window_rows) * p.window_cols *
+                   p.channels * p.features;
+  return p.channels % 4 == 0 && p.features % 4 == 0 &&
+         max(max(x, y), w) * sizeof(_Float16) <= kMaxBufferBytes;
+}
+
+int launch_conv2d_forward_general_f16(const _Float16* x, const _Float16* filter,
+                                      _Float16* y,
+                                      const snn_hip_conv2d_params& p,
+                                      hipStream_t stream) {
+  Gather g;
+  fill_gather(p, SNN_HIP_FORWARD, &g);
+  constexpr int BM = 64, BN = 64;
+  const unsigned tiles_m = static_cast<unsigned>(ceil_div(g.m_total, BM));
+  const unsigned tiles_n = static_cast<unsigned>(ceil_div(g.n_total, BN));
+  const unsigned n_tiles = tiles_m * tiles_n;
+  const int n_chunks = ceil_div(g.k_total, kBK);
+  constexpr size_t kLdsBytes =
+      2 * sizeof(float) * (k_inner_floats(BM) + row_inner_floats(BN));
+  const unsigned src_bytes = static_cast<unsigned>(
+      static_cast<size_t>(g.batch) * g.src_rows * g.src_cols * g.src_ch * 2);
+  const unsigned wgt_bytes = static_cast<unsigned>(
+      static_cast<size_t>(p.window_rows) * p.window_cols * p.channels *
+      p.features * 2);
+  KernelTimer timer(stream);
+  hipLaunchKernelGGL(
+      (conv_igemm_kernel<BM, BN, 2, 2, false, false, false, false, _Float16>),
+      dim3(n_tiles, 1), dim3(kThreads), kLdsBytes, stream, x, filter, y, g,
+      src_bytes, wgt_bytes, tiles_n, n_tiles, n_chunks);
+  SNN_HIP_CHECK_LAUNCH();
+  return SNN_HIP_OK;
+}
+
 bool conv2d_igemm_supports(int direction, const snn_hip_conv2d_params& p) {
   // buffer descriptors address at most kMaxBufferBytes
   const size_t x = static_cast<size_t>(p.batch) * p.in_rows * p.in_cols *

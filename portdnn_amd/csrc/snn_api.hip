@@ -530,6 +530,10 @@ int launch_gemm_path<_Float16>(int direction, const _Float16* input,
       aligned16(input) && aligned16(filter) && aligned16(output))
     return launch_conv2d_igemm_f16(input, filter, output, p, workspace,
                                    workspace_elems, s);
+  if (direction == SNN_HIP_FORWARD &&
+      conv2d_forward_general_f16_supports(p) && aligned16(input) &&
+      aligned16(filter) && aligned16(output))
+    return launch_conv2d_forward_general_f16(input, filter, output, p, s);
   if (direction == SNN_HIP_INPUT_BACKPROP &&
       conv2d_input_backprop_f16_supports(p) && aligned16(input) &&
       aligned16(filter) && aligned16(output))

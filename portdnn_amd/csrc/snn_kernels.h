@@ -237,6 +237,15 @@ int launch_conv2d_input_backprop_f16(const _Float16* dy,
                                      size_t workspace_elems,
                                      hipStream_t stream);
 
+// Half-precision forward convolution for the shapes the binary16 kernels do
+// not take (conv2d_igemm.hip): the general implicit-GEMM kernel reading
+// binary16 operands.  Channels and features in multiples of 4.
+bool conv2d_forward_general_f16_supports(const snn_hip_conv2d_params& p);
+int launch_conv2d_forward_general_f16(const _Float16* input,
+                                      const _Float16* filter, _Float16* output,
+                                      const snn_hip_conv2d_params& p,
+                                      hipStream_t stream);
+
 // Half-precision gradients on the fp32 matrix instructions
 // (conv2d_igemm.hip): the filter gradient for channel counts in multiples of
 // 64 (fp32 accumulation buffer in the workspace when it holds twice the

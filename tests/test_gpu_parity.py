@@ -1385,6 +1385,41 @@ def test_f16_conv_forward_lds_tile_kernel(shape):
     assert_close_f16(got, ref, ("f16 lds tile", shape))
 
 
+@pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, window, stride, SAME
+    (8, 28, 28, 144, 144, 3, 1, True),   # channels not a multiple of 64
+    (4, 28, 28, 100, 100, 5, 1, True),
+    (8, 32, 32, 16, 16, 3, 1, True),
+    (8, 56, 56, 12, 20, 3, 2, True),
+    (2, 56, 56, 64, 64, 7, 1, True),     # 49 taps
+    (8, 17, 19, 40, 72, 1, 1, False),
+])
+def test_f16_conv_forward_general_kernel(shape):
+    """Half-precision forward convolutions outside the binary16 kernels'
+    shapes (channel counts that are not multiples of 64, more than 32 taps)
+    run on the general implicit-GEMM kernel reading binary16 operands with
+    fp32 accumulation, not one lane per output: against the oracle in double
+    precision on the same half-rounded operands; nothing written past the
+    result."""
+    batch, rows, cols, ch, feats, window, stride, same = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, window, stride, same)
+    rng = np.random.default_rng(770 + rows + ch + window)
+    n_in, n_fil, n_out = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x = uniform(rng, n_in).astype(np.float16)
+    w = uniform(rng, n_fil).astype(np.float16)
+    ref = oracle.conv2d_forward(x.astype(np.float32), w.astype(np.float32),
+                                oracle_params(p, feats), acc64=True)
+    out = torch.full((n_out + 16,), 7.0, dtype=torch.float16, device="cuda")
+    for algo in (ALGO.IM2COL, ALGO.TILED):
+        if not supported(p, DIRECTION.FORWARD, algo):
+            continue
+        got = ops.conv2d(dev(x, torch.float16), dev(w, torch.float16), p,
+                         DIRECTION.FORWARD, algo, out=out[:n_out])
+        assert_close_f16(got.float().cpu().numpy(), ref,
+                         ("f16 general forward", ALGO_NAME[algo], shape))
+        assert torch.all(out[n_out:] == 7.0)
+
+
 @pytest.mark.parametrize("size,ch,feats,window", [
     (28, 128, 128, 3),   # LDS-tile kernel, four channel blocks
     (56, 64, 64, 3),     # LDS-tile kernel, one channel block
