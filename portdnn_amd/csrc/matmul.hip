@@ -102,6 +102,96 @@ __global__ void __launch_bounds__(256)
   if (i < n) c[i] *= beta;
 }
 
+// out[r][c] (rows2 x cols2, row-major) = in[r * row_stride + c * col_stride]
+// for r < rows and c < cols, else 0: copies a matrix, transposing and / or
+// widening it with zeros.
+__global__ void __launch_bounds__(256)
+    repack_matrix_kernel(const float* __restrict__ in, float* __restrict__ out,
+                         int rows, int cols, size_t row_stride,
+                         size_t col_stride, int cols2, size_t total) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= total) return;
+  const size_t r = i / cols2;
+  const int c = static_cast<int>(i - r * cols2);
+  out[i] = (r < static_cast<size_t>(rows) && c < cols)
+               ? in[r * row_stride + c * col_stride]
+               : 0.f;
+}
+
+void repack_matrix(const float* in, float* out, int rows, int cols,
+                   size_t row_stride, size_t col_stride, int rows2, int cols2,
+                   hipStream_t stream) {
+  const size_t total = static_cast<size_t>(rows2) * cols2;
+  hipLaunchKernelGGL(repack_matrix_kernel,
+                     dim3(static_cast<unsigned>(ceil_div(total, size_t{256}))),
+                     dim3(256), 0, stream, in, out, rows, cols, row_stride,
+                     col_stride, cols2, total);
+}
+
+// One large product the matrix-core kernel does not take as it stands (A
+// transposed, k not a multiple of 32, n not a multiple of 4): the operands
+// that do not fit are rewritten into stream-ordered temporaries -- A as m x
+// k', B as k' x n', zeros in the new rows and columns -- the kernel runs on
+// those, and a widened result is copied back.  The copies move O(mk + kn +
+// mn) floats against the O(mkn) of the product.  Returns -1 when it does not
+// apply.
+int launch_matmul_repacked_f32(const float* lhs, const float* rhs,
+                               float* output, int m, int k, int n,
+                               bool transpose_lhs, bool transpose_rhs,
+                               hipStream_t stream) {
+  if (m < 32 || static_cast<double>(m) * k * n < double(1 << 24)) return -1;
+  const int k2 = (k + 31) / 32 * 32;
+  // (B stored n x k is taken with any n)
+  const bool keep_bt = transpose_rhs && k2 == k;
+  const int n2 = keep_bt ? n : (n + 3) / 4 * 4;
+  const bool new_a = transpose_lhs || k2 != k;
+  const bool new_b = !keep_bt && (transpose_rhs || k2 != k || n2 != n);
+  const bool new_c = n2 != n;
+  if ((reinterpret_cast<uintptr_t>(lhs) | reinterpret_cast<uintptr_t>(rhs) |
+       reinterpret_cast<uintptr_t>(output)) & 15u)
+    return -1;
+  float *a2 = nullptr, *b2 = nullptr, *c2 = nullptr;
+  auto release = [&]() {
+    if (c2 != nullptr) temp_free_async(c2, stream);
+    if (b2 != nullptr) temp_free_async(b2, stream);
+    if (a2 != nullptr) temp_free_async(a2, stream);
+  };
+  auto grab = [&](float** ptr, size_t elems) {
+    void* raw = nullptr;
+    if (temp_malloc_async(&raw, elems * sizeof(float), stream) != hipSuccess)
+      return false;
+    *ptr = static_cast<float*>(raw);
+    return true;
+  };
+  if ((new_a && !grab(&a2, static_cast<size_t>(m) * k2)) ||
+      (new_b && !grab(&b2, static_cast<size_t>(k2) * n2)) ||
+      (new_c && !grab(&c2, static_cast<size_t>(m) * n2))) {
+    release();
+    return SNN_HIP_ALLOCATION_PROBLEM;
+  }
+  const float* a = new_a ? a2 : lhs;
+  const float* b = new_b ? b2 : rhs;
+  float* c = new_c ? c2 : output;
+  if (!batched_gemm_mfma_supports(m, k2, n2, a, b, c, keep_bt)) {
+    release();
+    return -1;
+  }
+  if (new_a)  // A[i][j]: stored m x k, or (transposed) k x m
+    repack_matrix(lhs, a2, m, k, transpose_lhs ? 1 : k, transpose_lhs ? m : 1,
+                  m, k2, stream);
+  if (new_b)  // B[i][j]: stored k x n, or (transposed) n x k
+    repack_matrix(rhs, b2, k, n, transpose_rhs ? 1 : n, transpose_rhs ? k : 1,
+                  k2, n2, stream);
+  const int status = launch_batched_gemm_mfma_f32(a, b, c, 1, m, k2, n2, stream,
+                                                  keep_bt, false);
+  if (new_c) repack_matrix(c2, output, m, n, n2, 1, m, n, stream);
+  const hipError_t err = hipGetLastError();
+  release();
+  if (status != SNN_HIP_OK) return status;
+  if (err != hipSuccess) return report_hip_error(err, "repacked matmul");
+  return SNN_HIP_OK;
+}
+
 }  // namespace
 
 int launch_matmul_f32(const float* lhs, const float* rhs, float* output,
@@ -156,6 +246,11 @@ int launch_matmul_f32(const float* lhs, const float* rhs, float* output,
       SNN_HIP_TRY(err);
       return SNN_HIP_OK;
     }
+  }
+  if (batches == 1 && beta == 0.f) {
+    const int repacked = launch_matmul_repacked_f32(
+        lhs, rhs, output, m, k, n, transpose_lhs, transpose_rhs, stream);
+    if (repacked >= 0) return repacked;
   }
   const dim3 grid(static_cast<unsigned>(ceil_div(m, kTile)),
                   static_cast<unsigned>(ceil_div(n, kTile)),

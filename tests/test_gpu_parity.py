@@ -1005,7 +1005,11 @@ def test_f16_pooling_gradients(shape):
 @pytest.mark.parametrize("shape", [(1, 64, 64, 64), (3, 37, 29, 53),
                                    (1, 1568, 512, 2048), (2, 130, 7, 258),
                                    (16, 200, 64, 64), (3, 100, 96, 50),
-                                   (1, 4096, 1024, 1024), (2, 33, 32, 3)])
+                                   (1, 4096, 1024, 1024), (2, 33, 32, 3),
+                                   # large and odd: repacked for the
+                                   # matrix-core kernel (k -> 32s, n -> 4s)
+                                   (1, 2047, 1023, 1001), (1, 512, 4096, 30),
+                                   (1, 4096, 512, 10)])
 def test_matmul(trans_a, trans_b, shape):
     b_, m, k, n = shape
     rng = np.random.default_rng(sum(shape))
