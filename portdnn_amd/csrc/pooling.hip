@@ -1386,6 +1386,15 @@ void launch_max_grad_tile(const float* in, const float* out, const float* dy,
   while (cv_per_group > 1 && cv_per_group / 2 >= cv) cv_per_group /= 2;
   const int tiles_x = ceil_div(p.in_cols, kGradTile);
   const int tiles_y = ceil_div(p.in_rows, kGradTile);
+  // A work-group's lanes walk the tile's windows and pixels in turns of 256 /
+  // cv_per_group: with few tiles, fewer channels per work-group give more
+  // work-groups and shorter turns (56x56x64 at batch 16: 256 work-groups of
+  // 20 + 16 turns took 143 us, 1024 of 5 + 4 turns 54 us; going on to 4096
+  // work-groups or 32 contiguous bytes per pixel measured slower).
+  while (cv_per_group > 4 &&
+         static_cast<long>(p.batch) * tiles_y * tiles_x *
+                 ceil_div(cv, cv_per_group) < 2048)
+    cv_per_group /= 2;
   const dim3 grid(static_cast<unsigned>(p.batch * tiles_y * tiles_x),
                   static_cast<unsigned>(ceil_div(cv, cv_per_group)));
   hipLaunchKernelGGL((pool_max_grad_tile_kernel<WIN, STRIDE>), grid, dim3(256),
