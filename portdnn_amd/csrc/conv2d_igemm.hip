@@ -1885,6 +1885,32 @@ static int launch_filter_backprop(const float* x, const float* dy, float* dw,
 
 namespace {
 
+// dX of a strided 1x1 unpadded convolution from the dense gradient of its
+// output pixels: dx[n][y][x][.] = t[n][y / sr][x / sc][.] where both
+// coordinates are multiples of the strides (and the quotient is an output
+// pixel), zero elsewhere.  One float4 per lane; every element of dX written.
+__global__ void __launch_bounds__(256)
+    scatter_strided_pixels_kernel(const float4* __restrict__ t,
+                                  float4* __restrict__ dx, int in_rows,
+                                  int in_cols, int out_rows, int out_cols,
+                                  int stride_rows, int stride_cols, int cv,
+                                  size_t n_vec) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= n_vec) return;
+  const int c = static_cast<int>(i % cv);
+  size_t pix = i / cv;
+  const int x = static_cast<int>(pix % in_cols);
+  pix /= in_cols;
+  const int y = static_cast<int>(pix % in_rows);
+  const size_t n = pix / in_rows;
+  const int oy = y / stride_rows, ox = x / stride_cols;
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (oy * stride_rows == y && ox * stride_cols == x && oy < out_rows &&
+      ox < out_cols)
+    v = t[((n * out_rows + oy) * out_cols + ox) * cv + c];
+  dx[i] = v;
+}
+
 __global__ void __launch_bounds__(256)
     f32_to_f16_kernel(const float* __restrict__ in, _Float16* __restrict__ out,
                       size_t n) {
@@ -2249,6 +2275,46 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
       SNN_TUNING_ENV("SNN_HIP_ROWSPLIT_OFF") == nullptr)
     return launch_conv2d_rowsplit_f32(input, filter, output, p, stream, false,
                                       epilogue);
+  if (direction == SNN_HIP_INPUT_BACKPROP && aligned16 &&
+      p.window_rows == 1 && p.window_cols == 1 && p.pad_rows == 0 &&
+      p.pad_cols == 0 && (p.stride_rows > 1 || p.stride_cols > 1) &&
+      p.channels % 4 == 0 && p.features % 4 == 0 &&
+      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols >= 1024 &&
+      SNN_TUNING_ENV("SNN_HIP_STRIDED_1X1_OFF") == nullptr) {
+    // A strided 1x1 layer (a ResNet shortcut): only the input pixels at
+    // multiples of the stride receive a gradient, and theirs is the stride-1
+    // input gradient over the output pixels.  That product runs dense into a
+    // stream-ordered temporary on the stride-1 kernels, and one pass writes
+    // dX from it, zeros included (the general strided kernel multiplied the
+    // zeros too: 56x56x256 -> 512 at batch 32 288 us).
+    snn_hip_conv2d_params q = p;
+    q.in_rows = p.out_rows;
+    q.in_cols = p.out_cols;
+    q.stride_rows = q.stride_cols = 1;
+    const size_t t_elems =
+        static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * p.channels;
+    void* t = nullptr;
+    if (temp_malloc_async(&t, t_elems * sizeof(float), stream) != hipSuccess)
+      return SNN_HIP_ALLOCATION_PROBLEM;
+    const int status = launch_conv2d_igemm_f32(
+        direction, input, filter, static_cast<float*>(t), q, stream, workspace,
+        workspace_elems, epilogue);
+    if (status == SNN_HIP_OK) {
+      const size_t n_vec = static_cast<size_t>(p.batch) * p.in_rows *
+                           p.in_cols * p.channels / 4;
+      hipLaunchKernelGGL(
+          scatter_strided_pixels_kernel,
+          dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))), dim3(256),
+          0, stream, static_cast<const float4*>(t),
+          reinterpret_cast<float4*>(output), p.in_rows, p.in_cols, p.out_rows,
+          p.out_cols, p.stride_rows, p.stride_cols, p.channels / 4, n_vec);
+    }
+    const hipError_t err = hipGetLastError();
+    temp_free_async(t, stream);
+    if (status != SNN_HIP_OK) return status;
+    if (err != hipSuccess) return report_hip_error(err, "strided 1x1 input backprop");
+    return SNN_HIP_OK;
+  }
   if (direction == SNN_HIP_INPUT_BACKPROP && aligned16 &&
       p.stride_rows == 1 && p.stride_cols == 1 &&
       p.window_rows - 1 - p.pad_rows >= 0 &&

@@ -404,6 +404,38 @@ def test_filter_gradient_from_registers(shape):
 
 
 @pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, stride
+    (8, 56, 56, 256, 512, 2),    # a ResNet shortcut
+    (4, 28, 28, 512, 1024, 2),
+    (3, 57, 55, 64, 128, 2),     # odd image: the last row and column count
+    (6, 40, 40, 32, 64, 3),      # stride 3
+])
+def test_input_gradient_of_strided_1x1_layers(shape):
+    """The input gradient of a strided 1x1 unpadded layer is the stride-1
+    gradient over the output pixels, written to the input pixels at multiples
+    of the stride, zeros elsewhere: computed dense on the stride-1 kernels and
+    scattered in one pass; against the oracle over the whole tensor, every
+    element of dX written (the output starts as NaN)."""
+    batch, rows, cols, ch, feats, stride = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, 1, stride, False)
+    rng = np.random.default_rng(2900 + rows + ch)
+    direction = DIRECTION.INPUT_BACKPROP
+    n_dy, n_fil, n_dx = ops.conv_sizes(p, direction)
+    dy, w = uniform(rng, n_dy), uniform(rng, n_fil)
+    ref = ORACLE_FN[direction](dy, w, oracle_params(p, feats), acc64=True)
+    out = torch.full((n_dx + 16,), float("nan"), device="cuda")
+    out[n_dx:] = 7.0
+    for algo in (ALGO.MATMUL, ALGO.IM2COL, ALGO.TILED):
+        if not supported(p, direction, algo):
+            continue
+        out[:n_dx] = float("nan")
+        got = ops.conv2d(dev(dy), dev(w), p, direction, algo, out=out[:n_dx])
+        assert_close(got.cpu().numpy(), ref,
+                     ("strided 1x1 input gradient", ALGO_NAME[algo], shape))
+        assert torch.all(out[n_dx:] == 7.0)
+
+
+@pytest.mark.parametrize("shape", [
     # ragged / edge shapes: odd sizes, C and K not multiples of the tiles,
     # non-square windows and strides, VALID padding
     (3, 13, 17, 5, 7, 3, 3, 1, 1, True),
