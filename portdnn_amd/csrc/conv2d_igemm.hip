@@ -1911,6 +1911,77 @@ __global__ void __launch_bounds__(256)
   dx[i] = v;
 }
 
+// Strided input gradient by stride classes.  The input pixels whose
+// coordinates are (py, px) modulo the strides receive gradient only through
+// the taps r = rho_r + sr u, s = rho_s + sc v with rho = (p + pad) mod stride,
+// and for them the gradient is a stride-1 convolution of dY with that
+// sub-filter, channels and features exchanged:
+//   dX[n][sr y' + py][sc x' + px][c] =
+//       sum_{u', v', k} dY[n][y' - pad'_r + u'][x' - pad'_c + v'][k] G[u'][v'][k][c]
+// with G[u'][v'][k][c] = W[rho_r + sr (Rc - 1 - u')][rho_s + sc (Sc - 1 - v')][c][k]
+// and pad' = Rc - 1 - (p + pad - rho) / stride.
+constexpr int kMaxStrideClasses = 16;
+struct StrideClasses {
+  int stride_rows, stride_cols, pad_rows, pad_cols;
+  int win_rows, win_cols, channels, features;
+  // per class (py * stride_cols + px): first element of its sub-filter and
+  // of its dense result, its size in pixels
+  unsigned filter_base[kMaxStrideClasses];
+  size_t pixel_base[kMaxStrideClasses];  // in units of pixels (x channels)
+  int rows[kMaxStrideClasses], cols[kMaxStrideClasses];
+  int taps_r[kMaxStrideClasses], taps_c[kMaxStrideClasses];
+};
+
+// Every filter element to its place in the sub-filter of its class.
+__global__ void __launch_bounds__(256)
+    stride_class_filters_kernel(const float* __restrict__ w,
+                                float* __restrict__ g, StrideClasses sc,
+                                unsigned total) {
+  const unsigned i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int k = i % sc.features;
+  unsigned t = i / sc.features;
+  const int c = t % sc.channels;
+  t /= sc.channels;
+  const int s = t % sc.win_cols;
+  const int r = t / sc.win_cols;
+  const int py = ((r - sc.pad_rows) % sc.stride_rows + sc.stride_rows) %
+                 sc.stride_rows;
+  const int px = ((s - sc.pad_cols) % sc.stride_cols + sc.stride_cols) %
+                 sc.stride_cols;
+  const int cls = py * sc.stride_cols + px;
+  if (sc.taps_r[cls] == 0) return;  // a class without pixels keeps no filter
+  const int u = sc.taps_r[cls] - 1 - r / sc.stride_rows;  // r = rho + sr u
+  const int v = sc.taps_c[cls] - 1 - s / sc.stride_cols;
+  g[sc.filter_base[cls] +
+    ((static_cast<unsigned>(u) * sc.taps_c[cls] + v) * sc.features + k) *
+        sc.channels +
+    c] = w[i];
+}
+
+// dX from the dense results of the classes (zeros for a class no tap reaches).
+__global__ void __launch_bounds__(256)
+    interleave_stride_classes_kernel(const float4* __restrict__ t,
+                                     float4* __restrict__ dx, StrideClasses sc,
+                                     int in_rows, int in_cols, int cv,
+                                     size_t n_vec) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= n_vec) return;
+  const int c = static_cast<int>(i % cv);
+  size_t pix = i / cv;
+  const int x = static_cast<int>(pix % in_cols);
+  pix /= in_cols;
+  const int y = static_cast<int>(pix % in_rows);
+  const size_t n = pix / in_rows;
+  const int cls = (y % sc.stride_rows) * sc.stride_cols + x % sc.stride_cols;
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (sc.taps_r[cls] > 0 && sc.taps_c[cls] > 0)
+    v = t[(sc.pixel_base[cls] +
+           (n * sc.rows[cls] + y / sc.stride_rows) * sc.cols[cls] +
+           x / sc.stride_cols) * cv + c];
+  dx[i] = v;
+}
+
 __global__ void __launch_bounds__(256)
     f32_to_f16_kernel(const float* __restrict__ in, _Float16* __restrict__ out,
                       size_t n) {
@@ -2314,6 +2385,105 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
     if (status != SNN_HIP_OK) return status;
     if (err != hipSuccess) return report_hip_error(err, "strided 1x1 input backprop");
     return SNN_HIP_OK;
+  }
+  if (direction == SNN_HIP_INPUT_BACKPROP && aligned16 &&
+      (p.stride_rows > 1 || p.stride_cols > 1) &&
+      p.stride_rows * p.stride_cols <= kMaxStrideClasses &&
+      p.channels % 4 == 0 && p.features % 4 == 0 &&
+      // (from 2^30 multiply-adds: below that the extra launches cost more
+      // than the multiplied zeros, 73 against 56 us at batch 4)
+      static_cast<double>(p.batch) * p.out_rows * p.out_cols * p.window_rows *
+              p.window_cols * p.channels * p.features >= double(1 << 30) &&
+      SNN_TUNING_ENV("SNN_HIP_STRIDE_CLASSES_OFF") == nullptr) {
+    // The general strided kernel walks every tap for every input pixel and
+    // multiplies zeros for those that do not reach it (3/4 of them at stride
+    // 2: 56x56x128 -> 128, 3x3, at batch 32 343 us against 90 forward).  By
+    // stride classes every class is a dense stride-1 forward convolution of
+    // dY on the fast kernels.
+    StrideClasses sc;
+    sc.stride_rows = p.stride_rows; sc.stride_cols = p.stride_cols;
+    sc.pad_rows = p.pad_rows;       sc.pad_cols = p.pad_cols;
+    sc.win_rows = p.window_rows;    sc.win_cols = p.window_cols;
+    sc.channels = p.channels;       sc.features = p.features;
+    bool ok = true;
+    unsigned filter_elems = 0;
+    size_t pixels = 0;
+    int pad_r[kMaxStrideClasses], pad_c[kMaxStrideClasses];
+    for (int py = 0; py < p.stride_rows; ++py)
+      for (int px = 0; px < p.stride_cols; ++px) {
+        const int cls = py * p.stride_cols + px;
+        const int rho_r = (py + p.pad_rows) % p.stride_rows;
+        const int rho_c = (px + p.pad_cols) % p.stride_cols;
+        sc.taps_r[cls] =
+            max(0, (p.window_rows - rho_r + p.stride_rows - 1) / p.stride_rows);
+        sc.taps_c[cls] =
+            max(0, (p.window_cols - rho_c + p.stride_cols - 1) / p.stride_cols);
+        sc.rows[cls] = max(0, (p.in_rows - py + p.stride_rows - 1) / p.stride_rows);
+        sc.cols[cls] = max(0, (p.in_cols - px + p.stride_cols - 1) / p.stride_cols);
+        pad_r[cls] = sc.taps_r[cls] - 1 - (py + p.pad_rows - rho_r) / p.stride_rows;
+        pad_c[cls] = sc.taps_c[cls] - 1 - (px + p.pad_cols - rho_c) / p.stride_cols;
+        sc.filter_base[cls] = filter_elems;
+        sc.pixel_base[cls] = pixels;
+        const bool empty = sc.taps_r[cls] == 0 || sc.taps_c[cls] == 0 ||
+                           sc.rows[cls] == 0 || sc.cols[cls] == 0;
+        if (!empty) {
+          ok = ok && pad_r[cls] >= 0 && pad_c[cls] >= 0;
+          pixels += static_cast<size_t>(p.batch) * sc.rows[cls] * sc.cols[cls];
+        } else {
+          sc.taps_r[cls] = sc.taps_c[cls] = 0;
+        }
+        filter_elems += static_cast<unsigned>(sc.taps_r[cls]) * sc.taps_c[cls] *
+                        p.channels * p.features;
+      }
+    if (ok) {
+      void *g = nullptr, *t = nullptr;
+      const unsigned w_elems = static_cast<unsigned>(p.window_rows) *
+                               p.window_cols * p.channels * p.features;
+      if (temp_malloc_async(&g, max(filter_elems, 4u) * sizeof(float), stream) !=
+          hipSuccess)
+        return SNN_HIP_ALLOCATION_PROBLEM;
+      if (temp_malloc_async(&t, max(pixels, size_t{1}) * p.channels * sizeof(float),
+                            stream) != hipSuccess) {
+        temp_free_async(g, stream);
+        return SNN_HIP_ALLOCATION_PROBLEM;
+      }
+      hipLaunchKernelGGL(stride_class_filters_kernel,
+                         dim3(ceil_div(w_elems, 256u)), dim3(256), 0, stream,
+                         filter, static_cast<float*>(g), sc, w_elems);
+      int status = SNN_HIP_OK;
+      for (int cls = 0; cls < p.stride_rows * p.stride_cols; ++cls) {
+        if (sc.taps_r[cls] == 0 || status != SNN_HIP_OK) continue;
+        snn_hip_conv2d_params q = p;
+        q.in_rows = p.out_rows;   q.in_cols = p.out_cols;
+        q.out_rows = sc.rows[cls]; q.out_cols = sc.cols[cls];
+        q.channels = p.features;  q.features = p.channels;
+        q.window_rows = sc.taps_r[cls]; q.window_cols = sc.taps_c[cls];
+        q.stride_rows = q.stride_cols = 1;
+        q.pad_rows = pad_r[cls];  q.pad_cols = pad_c[cls];
+        status = launch_conv2d_igemm_f32(
+            SNN_HIP_FORWARD, input,
+            static_cast<const float*>(g) + sc.filter_base[cls],
+            static_cast<float*>(t) + sc.pixel_base[cls] * p.channels, q, stream,
+            nullptr, 0, nullptr);
+      }
+      if (status == SNN_HIP_OK) {
+        const size_t n_vec = static_cast<size_t>(p.batch) * p.in_rows *
+                             p.in_cols * p.channels / 4;
+        hipLaunchKernelGGL(
+            interleave_stride_classes_kernel,
+            dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
+            dim3(256), 0, stream, static_cast<const float4*>(t),
+            reinterpret_cast<float4*>(output), sc, p.in_rows, p.in_cols,
+            p.channels / 4, n_vec);
+      }
+      const hipError_t err = hipGetLastError();
+      temp_free_async(t, stream);
+      temp_free_async(g, stream);
+      if (status != SNN_HIP_OK) return status;
+      if (err != hipSuccess)
+        return report_hip_error(err, "strided input backprop");
+      return SNN_HIP_OK;
+    }
   }
   if (direction == SNN_HIP_INPUT_BACKPROP && aligned16 &&
       p.stride_rows == 1 && p.stride_cols == 1 &&

@@ -404,6 +404,43 @@ def test_filter_gradient_from_registers(shape):
 
 
 @pytest.mark.parametrize("shape", [
+    # batch, rows, cols, channels, features, window, stride, SAME
+    # (from 2^30 multiply-adds on; smaller launches keep the general kernel)
+    (16, 56, 56, 128, 128, 3, 2, True),  # a ResNet 3x3 stride-2 layer
+    (16, 57, 55, 128, 128, 3, 2, True),  # odd image
+    (16, 57, 55, 128, 144, 3, 2, False), # VALID
+    (8, 40, 40, 128, 128, 5, 2, True),   # 5x5: classes of 3x3, 3x2, 2x3, 2x2 taps
+    (18, 45, 45, 128, 256, 3, 3, True),  # stride 3: one tap per class
+    (4, 64, 64, 64, 96, 7, 2, True),     # 7x7 stride 2 over 64 channels
+    (48, 40, 40, 128, 256, 2, 3, False), # stride above the window: empty classes
+    (4, 28, 28, 256, 256, 3, 2, True),   # below the threshold: general kernel
+])
+def test_strided_input_gradient_by_stride_classes(shape):
+    """A strided input gradient is computed class by class of input pixels
+    modulo the strides -- each a dense stride-1 forward convolution of dY with
+    the sub-filter of the taps that reach the class, on the stride-1 kernels
+    -- and interleaved into dX in one pass: against the oracle over the whole
+    tensor, every element of dX written (the output starts as NaN)."""
+    batch, rows, cols, ch, feats, window, stride, same = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, window, stride, same)
+    rng = np.random.default_rng(2950 + rows + ch + window)
+    direction = DIRECTION.INPUT_BACKPROP
+    n_dy, n_fil, n_dx = ops.conv_sizes(p, direction)
+    dy, w = uniform(rng, n_dy), uniform(rng, n_fil)
+    ref = ORACLE_FN[direction](dy, w, oracle_params(p, feats), acc64=True)
+    out = torch.full((n_dx + 16,), float("nan"), device="cuda")
+    out[n_dx:] = 7.0
+    for algo in (ALGO.IM2COL, ALGO.TILED):
+        if not supported(p, direction, algo):
+            continue
+        out[:n_dx] = float("nan")
+        got = ops.conv2d(dev(dy), dev(w), p, direction, algo, out=out[:n_dx])
+        assert_close(got.cpu().numpy(), ref,
+                     ("strided input gradient", ALGO_NAME[algo], shape))
+        assert torch.all(out[n_dx:] == 7.0)
+
+
+@pytest.mark.parametrize("shape", [
     # batch, rows, cols, channels, features, stride
     (8, 56, 56, 256, 512, 2),    # a ResNet shortcut
     (4, 28, 28, 512, 1024, 2),
