@@ -1932,19 +1932,16 @@ struct StrideClasses {
   int taps_r[kMaxStrideClasses], taps_c[kMaxStrideClasses];
 };
 
-// Every filter element to its place in the sub-filter of its class.
+// Every filter element to its place in the sub-filter of its class: per tap
+// a C x K matrix becomes K x C, 32 x 32 tiles through LDS so that reads and
+// writes are both contiguous.  Grid: (K tiles, C tiles, taps), 32 x 8 lanes.
 __global__ void __launch_bounds__(256)
     stride_class_filters_kernel(const float* __restrict__ w,
-                                float* __restrict__ g, StrideClasses sc,
-                                unsigned total) {
-  const unsigned i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= total) return;
-  const int k = i % sc.features;
-  unsigned t = i / sc.features;
-  const int c = t % sc.channels;
-  t /= sc.channels;
-  const int s = t % sc.win_cols;
-  const int r = t / sc.win_cols;
+                                float* __restrict__ g, StrideClasses sc) {
+  __shared__ float tile[32][33];
+  const int tap = blockIdx.z;
+  const int s = tap % sc.win_cols;
+  const int r = tap / sc.win_cols;
   const int py = ((r - sc.pad_rows) % sc.stride_rows + sc.stride_rows) %
                  sc.stride_rows;
   const int px = ((s - sc.pad_cols) % sc.stride_cols + sc.stride_cols) %
@@ -1953,10 +1950,27 @@ __global__ void __launch_bounds__(256)
   if (sc.taps_r[cls] == 0) return;  // a class without pixels keeps no filter
   const int u = sc.taps_r[cls] - 1 - r / sc.stride_rows;  // r = rho + sr u
   const int v = sc.taps_c[cls] - 1 - s / sc.stride_cols;
-  g[sc.filter_base[cls] +
-    ((static_cast<unsigned>(u) * sc.taps_c[cls] + v) * sc.features + k) *
-        sc.channels +
-    c] = w[i];
+  const int k0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const float* const src =
+      w + static_cast<size_t>(tap) * sc.channels * sc.features;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = c0 + ty + 8 * i, k = k0 + tx;
+    tile[ty + 8 * i][tx] = (c < sc.channels && k < sc.features)
+                               ? src[static_cast<size_t>(c) * sc.features + k]
+                               : 0.f;
+  }
+  __syncthreads();
+  float* const dst =
+      g + sc.filter_base[cls] +
+      static_cast<size_t>(u * sc.taps_c[cls] + v) * sc.features * sc.channels;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int k = k0 + ty + 8 * i, c = c0 + tx;
+    if (k < sc.features && c < sc.channels)
+      dst[static_cast<size_t>(k) * sc.channels + c] = tile[tx][ty + 8 * i];
+  }
 }
 
 // dX from the dense results of the classes (zeros for a class no tap reaches).
@@ -2437,8 +2451,6 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
       }
     if (ok) {
       void *g = nullptr, *t = nullptr;
-      const unsigned w_elems = static_cast<unsigned>(p.window_rows) *
-                               p.window_cols * p.channels * p.features;
       if (temp_malloc_async(&g, max(filter_elems, 4u) * sizeof(float), stream) !=
           hipSuccess)
         return SNN_HIP_ALLOCATION_PROBLEM;
@@ -2447,9 +2459,12 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
         temp_free_async(g, stream);
         return SNN_HIP_ALLOCATION_PROBLEM;
       }
-      hipLaunchKernelGGL(stride_class_filters_kernel,
-                         dim3(ceil_div(w_elems, 256u)), dim3(256), 0, stream,
-                         filter, static_cast<float*>(g), sc, w_elems);
+      hipLaunchKernelGGL(
+          stride_class_filters_kernel,
+          dim3(static_cast<unsigned>(ceil_div(p.features, 32)),
+               static_cast<unsigned>(ceil_div(p.channels, 32)),
+               static_cast<unsigned>(p.window_rows * p.window_cols)),
+          dim3(256), 0, stream, filter, static_cast<float*>(g), sc);
       int status = SNN_HIP_OK;
       for (int cls = 0; cls < p.stride_rows * p.stride_cols; ++cls) {
         if (sc.taps_r[cls] == 0 || status != SNN_HIP_OK) continue;
