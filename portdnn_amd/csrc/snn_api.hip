@@ -512,6 +512,68 @@ int launch_gemm_path_padded(int direction, const T* input, const T* filter,
   return SNN_HIP_OK;
 }
 template <>
+int launch_gemm_path<float>(int direction, const float* input,
+                            const float* filter, float* output,
+                            const snn_hip_conv2d_params& p, hipStream_t s,
+                            float* workspace, size_t workspace_elems,
+                            const LaunchOptions* epilogue);
+
+template <typename From, typename To>
+__global__ void __launch_bounds__(256)
+    convert_kernel(const From* __restrict__ in, To* __restrict__ out, size_t n) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i < n) out[i] = static_cast<To>(in[i]);
+}
+
+template <typename From, typename To>
+void convert(const From* in, To* out, size_t n, hipStream_t s) {
+  hipLaunchKernelGGL((convert_kernel<From, To>),
+                     dim3(static_cast<unsigned>(ceil_div(n, size_t{256}))),
+                     dim3(256), 0, s, in, out, n);
+}
+
+// A binary16 launch that no binary16 matrix-core kernel takes (three input
+// channels, channel or feature counts that are not multiples of 4, strided
+// input gradients) through the fp32 kernels: operands widened into
+// stream-ordered temporaries, the fp32 launch -- every path it has -- and the
+// result rounded back.  Products and sums are then fp32 on binary16-rounded
+// operands, as in the binary16 kernels.  From 2^24 multiply-adds; returns -1
+// when it does not apply.
+int launch_f16_through_fp32(int direction, const _Float16* input,
+                            const _Float16* filter, _Float16* output,
+                            const snn_hip_conv2d_params& p, hipStream_t s) {
+  const double macs = static_cast<double>(p.batch) * p.out_rows * p.out_cols *
+                      p.window_rows * p.window_cols * p.channels * p.features;
+  if (macs < double(1 << 24)) return -1;
+  const ConvSizes sz = conv_sizes(p, direction);
+  void *in32 = nullptr, *fil32 = nullptr, *out32 = nullptr;
+  auto release = [&]() {
+    if (out32 != nullptr) temp_free_async(out32, s);
+    if (fil32 != nullptr) temp_free_async(fil32, s);
+    if (in32 != nullptr) temp_free_async(in32, s);
+  };
+  if (temp_malloc_async(&in32, sz.input * sizeof(float), s) != hipSuccess ||
+      temp_malloc_async(&fil32, sz.filter * sizeof(float), s) != hipSuccess ||
+      temp_malloc_async(&out32, sz.output * sizeof(float), s) != hipSuccess) {
+    release();
+    return SNN_HIP_ALLOCATION_PROBLEM;
+  }
+  convert(input, static_cast<float*>(in32), sz.input, s);
+  convert(filter, static_cast<float*>(fil32), sz.filter, s);
+  const int status = launch_gemm_path<float>(
+      direction, static_cast<const float*>(in32),
+      static_cast<const float*>(fil32), static_cast<float*>(out32), p, s,
+      nullptr, 0, nullptr);
+  if (status == SNN_HIP_OK)
+    convert(static_cast<const float*>(out32), output, sz.output, s);
+  const hipError_t err = hipGetLastError();
+  release();
+  if (status != SNN_HIP_OK) return status;
+  if (err != hipSuccess) return report_hip_error(err, "binary16 through fp32");
+  return SNN_HIP_OK;
+}
+
+template <>
 int launch_gemm_path<_Float16>(int direction, const _Float16* input,
                                const _Float16* filter, _Float16* output,
                                const snn_hip_conv2d_params& p, hipStream_t s,
@@ -539,16 +601,38 @@ int launch_gemm_path<_Float16>(int direction, const _Float16* input,
       aligned16(filter) && aligned16(output))
     return launch_conv2d_input_backprop_f16(input, filter, output, p,
                                             workspace, workspace_elems, s);
+  // (a strided input gradient from 2^30 multiply-adds: the fp32 launch splits
+  // it into stride classes, the general binary16 kernel multiplies the zeros
+  // of the taps that do not reach a pixel -- 1.39 ms against 67 us forward for
+  // 56x56x128 -> 128, 3x3 stride 2, at batch 128)
+  if (direction == SNN_HIP_INPUT_BACKPROP &&
+      (p.stride_rows > 1 || p.stride_cols > 1) &&
+      static_cast<double>(p.batch) * p.out_rows * p.out_cols * p.window_rows *
+              p.window_cols * p.channels * p.features >= double(1 << 30)) {
+    const int rc = launch_f16_through_fp32(direction, input, filter, output, p, s);
+    if (rc >= 0) return rc;
+  }
   if (direction == SNN_HIP_INPUT_BACKPROP &&
       conv2d_input_backprop_general_f16_supports(p) && aligned16(input) &&
       aligned16(filter))
     return launch_conv2d_input_backprop_general_f16(input, filter, output, p,
                                                     s);
+  // (few (tap, channel) pairs -- a three-channel stem: fp32 has kernels built
+  // for that; 64-channel tiles would be nearly empty)
+  if (direction == SNN_HIP_FILTER_BACKPROP && p.channels <= 8 &&
+      p.window_rows * p.window_cols * p.channels <= 192) {
+    const int rc = launch_f16_through_fp32(direction, input, filter, output, p, s);
+    if (rc >= 0) return rc;
+  }
   if (direction == SNN_HIP_FILTER_BACKPROP &&
       conv2d_filter_backprop_f16_supports(p) && aligned16(input) &&
       aligned16(filter))
     return launch_conv2d_filter_backprop_f16(input, filter, output, p,
                                              workspace, workspace_elems, s);
+  {
+    const int rc = launch_f16_through_fp32(direction, input, filter, output, p, s);
+    if (rc >= 0) return rc;
+  }
   return launch_conv2d_direct<_Float16>(direction, input, filter, output, p, s);
 }
 template <>

@@ -1705,7 +1705,9 @@ def test_filter_gradient_from_registers_ragged_and_half(shape, dtype):
             first = got
         # (fp32 layers with few (tap, channel) pairs keep the one-work-group
         # kernel, whose partial sums meet through float atomics)
-        if (not half and ch % 64 != 0 and feats % 4 == 0 and
+        # (binary16 layers with at most 8 channels go the same way, through
+        # fp32 copies)
+        if ((not half or ch <= 8) and ch % 64 != 0 and feats % 4 == 0 and
                 window * window * ch <= 192):
             continue
         assert torch.equal(got.view(torch.int16 if half else torch.int32),
