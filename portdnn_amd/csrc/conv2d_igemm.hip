@@ -1935,10 +1935,11 @@ struct StrideClasses {
 // Every filter element to its place in the sub-filter of its class: per tap
 // a C x K matrix becomes K x C, 32 x 32 tiles through LDS so that reads and
 // writes are both contiguous.  Grid: (K tiles, C tiles, taps), 32 x 8 lanes.
+template <typename T>
 __global__ void __launch_bounds__(256)
-    stride_class_filters_kernel(const float* __restrict__ w,
-                                float* __restrict__ g, StrideClasses sc) {
-  __shared__ float tile[32][33];
+    stride_class_filters_kernel(const T* __restrict__ w, T* __restrict__ g,
+                                StrideClasses sc) {
+  __shared__ T tile[32][33];
   const int tap = blockIdx.z;
   const int s = tap % sc.win_cols;
   const int r = tap / sc.win_cols;
@@ -1952,17 +1953,17 @@ __global__ void __launch_bounds__(256)
   const int v = sc.taps_c[cls] - 1 - s / sc.stride_cols;
   const int k0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
   const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-  const float* const src =
+  const T* const src =
       w + static_cast<size_t>(tap) * sc.channels * sc.features;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int c = c0 + ty + 8 * i, k = k0 + tx;
     tile[ty + 8 * i][tx] = (c < sc.channels && k < sc.features)
                                ? src[static_cast<size_t>(c) * sc.features + k]
-                               : 0.f;
+                               : static_cast<T>(0);
   }
   __syncthreads();
-  float* const dst =
+  T* const dst =
       g + sc.filter_base[cls] +
       static_cast<size_t>(u * sc.taps_c[cls] + v) * sc.features * sc.channels;
 #pragma unroll
@@ -1974,9 +1975,10 @@ __global__ void __launch_bounds__(256)
 }
 
 // dX from the dense results of the classes (zeros for a class no tap reaches).
+template <typename V>  // four elements: float4, or 8 bytes of binary16
 __global__ void __launch_bounds__(256)
-    interleave_stride_classes_kernel(const float4* __restrict__ t,
-                                     float4* __restrict__ dx, StrideClasses sc,
+    interleave_stride_classes_kernel(const V* __restrict__ t,
+                                     V* __restrict__ dx, StrideClasses sc,
                                      int in_rows, int in_cols, int cv,
                                      size_t n_vec) {
   const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
@@ -1988,7 +1990,7 @@ __global__ void __launch_bounds__(256)
   const int y = static_cast<int>(pix % in_rows);
   const size_t n = pix / in_rows;
   const int cls = (y % sc.stride_rows) * sc.stride_cols + x % sc.stride_cols;
-  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  V v = {};
   if (sc.taps_r[cls] > 0 && sc.taps_c[cls] > 0)
     v = t[(sc.pixel_base[cls] +
            (n * sc.rows[cls] + y / sc.stride_rows) * sc.cols[cls] +
@@ -2338,6 +2340,128 @@ int launch_batched_gemm_mfma_f32(const float* a, const float* b, float* c,
   return SNN_HIP_OK;
 }
 
+// The stride classes of an input gradient, each through `forward` (a
+// stride-1 forward convolution of T tensors: parameters, input, filter,
+// output), then interleaved.  Returns -1 when a class would need negative
+// padding (the caller then takes another path).
+template <typename T, typename V, typename Forward>
+int strided_input_backprop_by_classes(const T* input, const T* filter,
+                                      T* output,
+                                      const snn_hip_conv2d_params& p,
+                                      hipStream_t stream, Forward forward) {
+  StrideClasses sc;
+  sc.stride_rows = p.stride_rows; sc.stride_cols = p.stride_cols;
+  sc.pad_rows = p.pad_rows;       sc.pad_cols = p.pad_cols;
+  sc.win_rows = p.window_rows;    sc.win_cols = p.window_cols;
+  sc.channels = p.channels;       sc.features = p.features;
+  bool ok = true;
+  unsigned filter_elems = 0;
+  size_t pixels = 0;
+  int pad_r[kMaxStrideClasses], pad_c[kMaxStrideClasses];
+  for (int py = 0; py < p.stride_rows; ++py)
+    for (int px = 0; px < p.stride_cols; ++px) {
+      const int cls = py * p.stride_cols + px;
+      const int rho_r = (py + p.pad_rows) % p.stride_rows;
+      const int rho_c = (px + p.pad_cols) % p.stride_cols;
+      sc.taps_r[cls] =
+          max(0, (p.window_rows - rho_r + p.stride_rows - 1) / p.stride_rows);
+      sc.taps_c[cls] =
+          max(0, (p.window_cols - rho_c + p.stride_cols - 1) / p.stride_cols);
+      sc.rows[cls] = max(0, (p.in_rows - py + p.stride_rows - 1) / p.stride_rows);
+      sc.cols[cls] = max(0, (p.in_cols - px + p.stride_cols - 1) / p.stride_cols);
+      pad_r[cls] = sc.taps_r[cls] - 1 - (py + p.pad_rows - rho_r) / p.stride_rows;
+      pad_c[cls] = sc.taps_c[cls] - 1 - (px + p.pad_cols - rho_c) / p.stride_cols;
+      sc.filter_base[cls] = filter_elems;
+      sc.pixel_base[cls] = pixels;
+      const bool empty = sc.taps_r[cls] == 0 || sc.taps_c[cls] == 0 ||
+                         sc.rows[cls] == 0 || sc.cols[cls] == 0;
+      if (!empty) {
+        ok = ok && pad_r[cls] >= 0 && pad_c[cls] >= 0;
+        pixels += static_cast<size_t>(p.batch) * sc.rows[cls] * sc.cols[cls];
+      } else {
+        sc.taps_r[cls] = sc.taps_c[cls] = 0;
+      }
+      filter_elems += static_cast<unsigned>(sc.taps_r[cls]) * sc.taps_c[cls] *
+                      p.channels * p.features;
+    }
+  if (ok) {
+    void *g = nullptr, *t = nullptr;
+    if (temp_malloc_async(&g, max(filter_elems, 4u) * sizeof(T), stream) !=
+        hipSuccess)
+      return SNN_HIP_ALLOCATION_PROBLEM;
+    if (temp_malloc_async(&t, max(pixels, size_t{1}) * p.channels * sizeof(T),
+                          stream) != hipSuccess) {
+      temp_free_async(g, stream);
+      return SNN_HIP_ALLOCATION_PROBLEM;
+    }
+    hipLaunchKernelGGL(
+        stride_class_filters_kernel<T>,
+        dim3(static_cast<unsigned>(ceil_div(p.features, 32)),
+             static_cast<unsigned>(ceil_div(p.channels, 32)),
+             static_cast<unsigned>(p.window_rows * p.window_cols)),
+        dim3(256), 0, stream, filter, static_cast<T*>(g), sc);
+    int status = SNN_HIP_OK;
+    for (int cls = 0; cls < p.stride_rows * p.stride_cols; ++cls) {
+      if (sc.taps_r[cls] == 0 || status != SNN_HIP_OK) continue;
+      snn_hip_conv2d_params q = p;
+      q.in_rows = p.out_rows;   q.in_cols = p.out_cols;
+      q.out_rows = sc.rows[cls]; q.out_cols = sc.cols[cls];
+      q.channels = p.features;  q.features = p.channels;
+      q.window_rows = sc.taps_r[cls]; q.window_cols = sc.taps_c[cls];
+      q.stride_rows = q.stride_cols = 1;
+      q.pad_rows = pad_r[cls];  q.pad_cols = pad_c[cls];
+      status = forward(q, input, static_cast<const T*>(g) + sc.filter_base[cls],
+                       static_cast<T*>(t) + sc.pixel_base[cls] * p.channels);
+    }
+    if (status == SNN_HIP_OK) {
+      const size_t n_vec = static_cast<size_t>(p.batch) * p.in_rows *
+                           p.in_cols * p.channels / 4;
+      hipLaunchKernelGGL(
+          interleave_stride_classes_kernel<V>,
+          dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
+          dim3(256), 0, stream, static_cast<const V*>(t),
+          reinterpret_cast<V*>(output), sc, p.in_rows, p.in_cols,
+          p.channels / 4, n_vec);
+    }
+    const hipError_t err = hipGetLastError();
+    temp_free_async(t, stream);
+    temp_free_async(g, stream);
+    if (status != SNN_HIP_OK) return status;
+    if (err != hipSuccess)
+      return report_hip_error(err, "strided input backprop");
+    return SNN_HIP_OK;
+  }
+  return -1;
+}
+
+bool conv2d_strided_input_backprop_f16_supports(
+    const snn_hip_conv2d_params& p) {
+  return (p.stride_rows > 1 || p.stride_cols > 1) &&
+         p.stride_rows * p.stride_cols <= kMaxStrideClasses &&
+         p.channels % 4 == 0 && p.features % 64 == 0 &&
+         static_cast<double>(p.batch) * p.out_rows * p.out_cols *
+                 p.window_rows * p.window_cols * p.channels * p.features >=
+             double(1 << 30);
+}
+
+// Binary16: the classes run on the binary16 forward kernels (dY's feature
+// count, the classes' channel count, in multiples of 64).  -1: not taken.
+int launch_conv2d_strided_input_backprop_f16(const _Float16* dy,
+                                             const _Float16* filter,
+                                             _Float16* dx,
+                                             const snn_hip_conv2d_params& p,
+                                             hipStream_t stream) {
+  typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+  return strided_input_backprop_by_classes<_Float16, half4v>(
+      dy, filter, dx, p, stream,
+      [&](const snn_hip_conv2d_params& q, const _Float16* in,
+          const _Float16* fil, _Float16* out) {
+        if (conv2d_igemm_f16_supports(q))
+          return launch_conv2d_igemm_f16(in, fil, out, q, nullptr, 0, stream);
+        return launch_conv2d_forward_general_f16(in, fil, out, q, stream);
+      });
+}
+
 int launch_conv2d_igemm_f32(int direction, const float* input,
                             const float* filter, float* output,
                             const snn_hip_conv2d_params& p,
@@ -2414,91 +2538,14 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
     // 2: 56x56x128 -> 128, 3x3, at batch 32 343 us against 90 forward).  By
     // stride classes every class is a dense stride-1 forward convolution of
     // dY on the fast kernels.
-    StrideClasses sc;
-    sc.stride_rows = p.stride_rows; sc.stride_cols = p.stride_cols;
-    sc.pad_rows = p.pad_rows;       sc.pad_cols = p.pad_cols;
-    sc.win_rows = p.window_rows;    sc.win_cols = p.window_cols;
-    sc.channels = p.channels;       sc.features = p.features;
-    bool ok = true;
-    unsigned filter_elems = 0;
-    size_t pixels = 0;
-    int pad_r[kMaxStrideClasses], pad_c[kMaxStrideClasses];
-    for (int py = 0; py < p.stride_rows; ++py)
-      for (int px = 0; px < p.stride_cols; ++px) {
-        const int cls = py * p.stride_cols + px;
-        const int rho_r = (py + p.pad_rows) % p.stride_rows;
-        const int rho_c = (px + p.pad_cols) % p.stride_cols;
-        sc.taps_r[cls] =
-            max(0, (p.window_rows - rho_r + p.stride_rows - 1) / p.stride_rows);
-        sc.taps_c[cls] =
-            max(0, (p.window_cols - rho_c + p.stride_cols - 1) / p.stride_cols);
-        sc.rows[cls] = max(0, (p.in_rows - py + p.stride_rows - 1) / p.stride_rows);
-        sc.cols[cls] = max(0, (p.in_cols - px + p.stride_cols - 1) / p.stride_cols);
-        pad_r[cls] = sc.taps_r[cls] - 1 - (py + p.pad_rows - rho_r) / p.stride_rows;
-        pad_c[cls] = sc.taps_c[cls] - 1 - (px + p.pad_cols - rho_c) / p.stride_cols;
-        sc.filter_base[cls] = filter_elems;
-        sc.pixel_base[cls] = pixels;
-        const bool empty = sc.taps_r[cls] == 0 || sc.taps_c[cls] == 0 ||
-                           sc.rows[cls] == 0 || sc.cols[cls] == 0;
-        if (!empty) {
-          ok = ok && pad_r[cls] >= 0 && pad_c[cls] >= 0;
-          pixels += static_cast<size_t>(p.batch) * sc.rows[cls] * sc.cols[cls];
-        } else {
-          sc.taps_r[cls] = sc.taps_c[cls] = 0;
-        }
-        filter_elems += static_cast<unsigned>(sc.taps_r[cls]) * sc.taps_c[cls] *
-                        p.channels * p.features;
-      }
-    if (ok) {
-      void *g = nullptr, *t = nullptr;
-      if (temp_malloc_async(&g, max(filter_elems, 4u) * sizeof(float), stream) !=
-          hipSuccess)
-        return SNN_HIP_ALLOCATION_PROBLEM;
-      if (temp_malloc_async(&t, max(pixels, size_t{1}) * p.channels * sizeof(float),
-                            stream) != hipSuccess) {
-        temp_free_async(g, stream);
-        return SNN_HIP_ALLOCATION_PROBLEM;
-      }
-      hipLaunchKernelGGL(
-          stride_class_filters_kernel,
-          dim3(static_cast<unsigned>(ceil_div(p.features, 32)),
-               static_cast<unsigned>(ceil_div(p.channels, 32)),
-               static_cast<unsigned>(p.window_rows * p.window_cols)),
-          dim3(256), 0, stream, filter, static_cast<float*>(g), sc);
-      int status = SNN_HIP_OK;
-      for (int cls = 0; cls < p.stride_rows * p.stride_cols; ++cls) {
-        if (sc.taps_r[cls] == 0 || status != SNN_HIP_OK) continue;
-        snn_hip_conv2d_params q = p;
-        q.in_rows = p.out_rows;   q.in_cols = p.out_cols;
-        q.out_rows = sc.rows[cls]; q.out_cols = sc.cols[cls];
-        q.channels = p.features;  q.features = p.channels;
-        q.window_rows = sc.taps_r[cls]; q.window_cols = sc.taps_c[cls];
-        q.stride_rows = q.stride_cols = 1;
-        q.pad_rows = pad_r[cls];  q.pad_cols = pad_c[cls];
-        status = launch_conv2d_igemm_f32(
-            SNN_HIP_FORWARD, input,
-            static_cast<const float*>(g) + sc.filter_base[cls],
-            static_cast<float*>(t) + sc.pixel_base[cls] * p.channels, q, stream,
-            nullptr, 0, nullptr);
-      }
-      if (status == SNN_HIP_OK) {
-        const size_t n_vec = static_cast<size_t>(p.batch) * p.in_rows *
-                             p.in_cols * p.channels / 4;
-        hipLaunchKernelGGL(
-            interleave_stride_classes_kernel,
-            dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
-            dim3(256), 0, stream, static_cast<const float4*>(t),
-            reinterpret_cast<float4*>(output), sc, p.in_rows, p.in_cols,
-            p.channels / 4, n_vec);
-      }
-      const hipError_t err = hipGetLastError();
-      temp_free_async(t, stream);
-      temp_free_async(g, stream);
-      if (status != SNN_HIP_OK) return status;
-      if (err != hipSuccess)
-        return report_hip_error(err, "strided input backprop");
-      return SNN_HIP_OK;
-    }
+    const int rc = strided_input_backprop_by_classes<float, float4>(
+        input, filter, output, p, stream,
+        [&](const snn_hip_conv2d_params& q, const float* in, const float* fil,
+            float* out) {
+          return launch_conv2d_igemm_f32(SNN_HIP_FORWARD, in, fil, out, q, stream,
+                                         nullptr, 0, nullptr);
+        });
+    if (rc >= 0) return rc;
   }
   if (direction == SNN_HIP_INPUT_BACKPROP && aligned16 &&
       p.stride_rows == 1 && p.stride_cols == 1 &&

@@ -606,6 +606,13 @@ int launch_gemm_path<_Float16>(int direction, const _Float16* input,
   // of the taps that do not reach a pixel -- 1.39 ms against 67 us forward for
   // 56x56x128 -> 128, 3x3 stride 2, at batch 128)
   if (direction == SNN_HIP_INPUT_BACKPROP &&
+      conv2d_strided_input_backprop_f16_supports(p) && aligned16(input) &&
+      aligned16(filter) && aligned16(output)) {
+    const int rc =
+        launch_conv2d_strided_input_backprop_f16(input, filter, output, p, s);
+    if (rc >= 0) return rc;
+  }
+  if (direction == SNN_HIP_INPUT_BACKPROP &&
       (p.stride_rows > 1 || p.stride_cols > 1) &&
       static_cast<double>(p.batch) * p.out_rows * p.out_cols * p.window_rows *
               p.window_cols * p.channels * p.features >= double(1 << 30)) {

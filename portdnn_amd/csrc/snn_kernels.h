@@ -237,6 +237,18 @@ int launch_conv2d_input_backprop_f16(const _Float16* dy,
                                      size_t workspace_elems,
                                      hipStream_t stream);
 
+// Half-precision strided input gradient by stride classes (conv2d_igemm.hip):
+// every class of input pixels modulo the strides is a dense stride-1 forward
+// convolution of dY on the binary16 kernels.  Features in multiples of 64,
+// channels of 4, from 2^30 multiply-adds; the launch returns -1 when the
+// geometry does not fit (then nothing was launched).
+bool conv2d_strided_input_backprop_f16_supports(const snn_hip_conv2d_params& p);
+int launch_conv2d_strided_input_backprop_f16(const _Float16* output_gradient,
+                                             const _Float16* filter,
+                                             _Float16* input_gradient,
+                                             const snn_hip_conv2d_params& p,
+                                             hipStream_t stream);
+
 // Half-precision forward convolution for the shapes the binary16 kernels do
 // not take (conv2d_igemm.hip): the general implicit-GEMM kernel reading
 // binary16 operands.  Channels and features in multiples of 4.

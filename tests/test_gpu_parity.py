@@ -415,28 +415,41 @@ def test_filter_gradient_from_registers(shape):
     (48, 40, 40, 128, 256, 2, 3, False), # stride above the window: empty classes
     (4, 28, 28, 256, 256, 3, 2, True),   # below the threshold: general kernel
 ])
-def test_strided_input_gradient_by_stride_classes(shape):
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_strided_input_gradient_by_stride_classes(shape, dtype):
     """A strided input gradient is computed class by class of input pixels
     modulo the strides -- each a dense stride-1 forward convolution of dY with
     the sub-filter of the taps that reach the class, on the stride-1 kernels
-    -- and interleaved into dX in one pass: against the oracle over the whole
-    tensor, every element of dX written (the output starts as NaN)."""
+    (binary16: on the binary16 ones when the feature count is a multiple of
+    64, else through fp32 copies) -- and interleaved into dX in one pass:
+    against the oracle over the whole tensor, every element of dX written (the
+    output starts as NaN)."""
     batch, rows, cols, ch, feats, window, stride, same = shape
     p = ops.conv_params(batch, rows, cols, ch, feats, window, stride, same)
     rng = np.random.default_rng(2950 + rows + ch + window)
     direction = DIRECTION.INPUT_BACKPROP
     n_dy, n_fil, n_dx = ops.conv_sizes(p, direction)
+    half = dtype == "f16"
+    tdt = torch.float16 if half else torch.float32
     dy, w = uniform(rng, n_dy), uniform(rng, n_fil)
-    ref = ORACLE_FN[direction](dy, w, oracle_params(p, feats), acc64=True)
-    out = torch.full((n_dx + 16,), float("nan"), device="cuda")
+    if half:
+        dy, w = dy.astype(np.float16), w.astype(np.float16)
+    ref = ORACLE_FN[direction](dy.astype(np.float32), w.astype(np.float32),
+                               oracle_params(p, feats), acc64=True)
+    out = torch.full((n_dx + 16,), float("nan"), dtype=tdt, device="cuda")
     out[n_dx:] = 7.0
     for algo in (ALGO.IM2COL, ALGO.TILED):
         if not supported(p, direction, algo):
             continue
         out[:n_dx] = float("nan")
-        got = ops.conv2d(dev(dy), dev(w), p, direction, algo, out=out[:n_dx])
-        assert_close(got.cpu().numpy(), ref,
-                     ("strided input gradient", ALGO_NAME[algo], shape))
+        got = ops.conv2d(dev(dy, tdt), dev(w, tdt), p, direction, algo,
+                         out=out[:n_dx])
+        if half:
+            assert_close_f16(got.float().cpu().numpy(), ref,
+                             ("f16 strided input gradient", shape))
+        else:
+            assert_close(got.cpu().numpy(), ref,
+                         ("strided input gradient", ALGO_NAME[algo], shape))
         assert torch.all(out[n_dx:] == 7.0)
 
 
