@@ -1460,6 +1460,80 @@ static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
   return SNN_HIP_OK;
 }
 
+// Four elements per lane (element counts here are multiples of 4).
+template <typename From, typename To>
+__global__ void __launch_bounds__(256)
+    dw_convert_kernel(const From* __restrict__ in, To* __restrict__ out,
+                      size_t n_vec) {
+  typedef From from4 __attribute__((ext_vector_type(4)));
+  typedef To to4 __attribute__((ext_vector_type(4)));
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= n_vec) return;
+  const from4 v = reinterpret_cast<const from4*>(in)[i];
+  to4 r;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) r[e] = static_cast<To>(v[e]);
+  reinterpret_cast<to4*>(out)[i] = r;
+}
+
+template <typename T>
+int launch_depthwise(int direction, const T* input, const T* filter, T* output,
+                     const snn_hip_depthwise_params& p, hipStream_t stream,
+                     float* static_scratch);
+
+// The binary16 3x3 filter gradient of a large layer through the fp32 strip
+// kernel: both operands widened into stream-ordered temporaries, the fp32
+// launch, the small result rounded (the general binary16 kernel, one
+// channel per lane and a tap per work-group, took 1.07 ms where fp32 takes
+// 77 us: 112x112x32 at batch 128).  -1: does not apply.
+int launch_depthwise_filter_backprop_f16_through_fp32(
+    const _Float16* input, const _Float16* dy, _Float16* dw,
+    const snn_hip_depthwise_params& p, hipStream_t stream) {
+  const size_t n_x =
+      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
+  const size_t n_dy =
+      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * p.channels;
+  if (p.channel_multiplier != 1 || p.channels % 4 != 0 || p.window_rows != 3 ||
+      p.window_cols != 3 || p.stride_rows != p.stride_cols ||
+      (p.stride_rows != 1 && p.stride_rows != 2) || n_dy < (size_t{1} << 21) ||
+      n_x * sizeof(float) >= 0x7FFFFFF0u)
+    return -1;
+  const size_t n_dw = static_cast<size_t>(9) * p.channels;
+  void *x32 = nullptr, *dy32 = nullptr, *dw32 = nullptr;
+  auto release = [&]() {
+    if (dw32 != nullptr) temp_free_async(dw32, stream);
+    if (dy32 != nullptr) temp_free_async(dy32, stream);
+    if (x32 != nullptr) temp_free_async(x32, stream);
+  };
+  if (temp_malloc_async(&x32, n_x * sizeof(float), stream) != hipSuccess ||
+      temp_malloc_async(&dy32, n_dy * sizeof(float), stream) != hipSuccess ||
+      temp_malloc_async(&dw32, n_dw * sizeof(float), stream) != hipSuccess) {
+    release();
+    return SNN_HIP_ALLOCATION_PROBLEM;
+  }
+  auto convert = [&](auto* in, auto* out, size_t n) {
+    hipLaunchKernelGGL(
+        (dw_convert_kernel<std::remove_cv_t<std::remove_pointer_t<decltype(in)>>,
+                           std::remove_pointer_t<decltype(out)>>),
+        dim3(static_cast<unsigned>(ceil_div(n / 4, size_t{256}))), dim3(256), 0,
+        stream, in, out, n / 4);
+  };
+  convert(input, static_cast<float*>(x32), n_x);
+  convert(dy, static_cast<float*>(dy32), n_dy);
+  const int status = launch_depthwise<float>(
+      SNN_HIP_FILTER_BACKPROP, static_cast<const float*>(x32),
+      static_cast<const float*>(dy32), static_cast<float*>(dw32), p, stream,
+      nullptr);
+  if (status == SNN_HIP_OK)
+    convert(static_cast<const float*>(dw32), dw, n_dw);
+  const hipError_t err = hipGetLastError();
+  release();
+  if (status != SNN_HIP_OK) return status;
+  if (err != hipSuccess)
+    return report_hip_error(err, "binary16 depthwise filter backprop");
+  return SNN_HIP_OK;
+}
+
 template <typename T>
 int launch_depthwise(int direction, const T* input, const T* filter, T* output,
                      const snn_hip_depthwise_params& p, hipStream_t stream,
@@ -1556,6 +1630,11 @@ int launch_depthwise(int direction, const T* input, const T* filter, T* output,
     const size_t n_pix_sz =
         static_cast<size_t>(p.batch) * p.out_rows * p.out_cols;
     bool done = false;
+    if constexpr (std::is_same<T, _Float16>::value) {
+      const int rc = launch_depthwise_filter_backprop_f16_through_fp32(
+          input, filter, output, p, stream);
+      if (rc >= 0) return rc;
+    }
     if constexpr (std::is_same<T, float>::value) {
       if (p.channel_multiplier == 1 && p.channels % 4 == 0 &&
           p.window_rows == 3 && p.window_cols == 3 &&

@@ -1825,6 +1825,8 @@ def test_f16_depthwise_backprops(shape):
     (4, 56, 56, 3, 8, 3, 2),     # three channels, multiplier 8
     (8, 28, 28, 128, 1, 1, 1),   # 1x1 window
     (4, 56, 56, 64, 1, 3, 1),    # (binary16: the MobileNet shape itself)
+    (16, 56, 56, 64, 1, 3, 1),   # (binary16, large: through the fp32 kernel)
+    (16, 112, 112, 32, 1, 3, 2),
 ])
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
 def test_depthwise_filter_gradient_general_shapes_split_over_work_groups(
