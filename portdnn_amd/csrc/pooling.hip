@@ -1127,12 +1127,12 @@ __global__ void __launch_bounds__(256)
 // (src/pooling/kernels.h:197-239) -- and carries those two positions and dY
 // values down as the "windows above" of the next block row.  Each dX pixel
 // adds its windows in output-row, output-column order.
-template <int TH, bool NAN_MODE>
+template <int TH, bool NAN_MODE, typename T = float>
 __global__ void __launch_bounds__(256)
-    pool_max_grad_3x3_s2_kernel(const float* __restrict__ in,
-                                const float* __restrict__ out,
-                                const float* __restrict__ dy,
-                                float* __restrict__ dx, snn_hip_pooling_params p,
+    pool_max_grad_3x3_s2_kernel(const T* __restrict__ in,
+                                const T* __restrict__ out,
+                                const T* __restrict__ dy,
+                                T* __restrict__ dx, snn_hip_pooling_params p,
                                 int n_bcols, int n_strips, unsigned n_items) {
   constexpr bool nan_mode = NAN_MODE;
   const unsigned idx = blockIdx.x * 256u + threadIdx.x;
@@ -1147,14 +1147,15 @@ __global__ void __launch_bounds__(256)
   const int br0 = static_cast<int>(t % static_cast<unsigned>(n_strips)) * TH +
                   p.pad_rows / 2;
   const int n = static_cast<int>(t / static_cast<unsigned>(n_strips));
+  constexpr unsigned kEsz = sizeof(T);
   const size_t in_elems =
       static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * C;
   const size_t out_elems =
       static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * C;
-  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_elems * 4);
-  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_elems * 4);
-  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, out_elems * 4);
-  const __amdgpu_buffer_rsrc_t dx_rsrc = make_rsrc(dx, in_elems * 4);
+  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_elems * kEsz);
+  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_elems * kEsz);
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, out_elems * kEsz);
+  const __amdgpu_buffer_rsrc_t dx_rsrc = make_rsrc(dx, in_elems * kEsz);
 
   // input columns 2 * bc - 2 .. 2 * bc + 2 (padded), image column x0 + j
   const int x0 = 2 * bc - 2 - p.pad_cols;
@@ -1164,9 +1165,9 @@ __global__ void __launch_bounds__(256)
     x_ok[j] = static_cast<unsigned>(x0 + j) < static_cast<unsigned>(p.in_cols);
   // windows bc - 1 and bc
   const bool w_ok[2] = {bc >= 1 && bc - 1 < p.out_cols, bc < p.out_cols};
-  const unsigned in_row_bytes = static_cast<unsigned>(p.in_cols * C) * 4u;
+  const unsigned in_row_bytes = static_cast<unsigned>(p.in_cols * C) * kEsz;
   const unsigned in_image = static_cast<unsigned>(n * p.in_rows) * in_row_bytes;
-  const unsigned in_col0 = static_cast<unsigned>(x0 * C + ch) * 4u;
+  const unsigned in_col0 = static_cast<unsigned>(x0 * C + ch) * kEsz;
   // (Offsets outside the image are made out of range with mask arithmetic,
   // not with a conditional: the compiler turns a per-lane condition around
   // these loads into two branches that load into the same registers and waits
@@ -1183,9 +1184,9 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
     for (int j = 0; j < 5; ++j) {
       const unsigned bad = y_bad | x_bad[j];
-      BufVec4<float>::load(
+      BufVec4<T>::load(
           in_rsrc,
-          ((base + static_cast<unsigned>(j * C) * 4u) & ~bad) |
+          ((base + static_cast<unsigned>(j * C) * kEsz) & ~bad) |
               (kOobOffset & bad),
           v[j]);
     }
@@ -1198,13 +1199,13 @@ __global__ void __launch_bounds__(256)
                                      static_cast<unsigned>(oy) >=
                                      static_cast<unsigned>(p.out_rows));
     const unsigned base = static_cast<unsigned>(
-        ((n * p.out_rows + oy) * p.out_cols + bc - 1) * C + ch) * 4u;
+        ((n * p.out_rows + oy) * p.out_cols + bc - 1) * C + ch) * kEsz;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const unsigned bad = oy_bad | w_bad[j];
-      BufVec4<float>::load(
+      BufVec4<T>::load(
           rsrc,
-          ((base + static_cast<unsigned>(j * C) * 4u) & ~bad) |
+          ((base + static_cast<unsigned>(j * C) * kEsz) & ~bad) |
               (kOobOffset & bad),
           v[j]);
     }
@@ -1272,10 +1273,10 @@ __global__ void __launch_bounds__(256)
   float ee[4], eo[4], oe[4], oo[4];
   unsigned st_off[4];
   auto store_block_row = [&]() {
-    BufVec4<float>::store(dx_rsrc, st_off[0], ee);
-    BufVec4<float>::store(dx_rsrc, st_off[1], eo);
-    BufVec4<float>::store(dx_rsrc, st_off[2], oe);
-    BufVec4<float>::store(dx_rsrc, st_off[3], oo);
+    BufVec4<T>::store(dx_rsrc, st_off[0], ee);
+    BufVec4<T>::store(dx_rsrc, st_off[1], eo);
+    BufVec4<T>::store(dx_rsrc, st_off[2], oe);
+    BufVec4<T>::store(dx_rsrc, st_off[3], oo);
   };
   // (short strips unrolled in full; nothing in the body is indexed by i, so the
   // 14-row strip runs as a loop of two block rows a turn -- one a turn
@@ -1355,8 +1356,8 @@ __global__ void __launch_bounds__(256)
       oo[e] = pos[1][e] == 4 ? 0.f + g[1][e] : 0.f;
     }
     const unsigned base = in_image + static_cast<unsigned>(y) * in_row_bytes +
-                          in_col0 + static_cast<unsigned>(2 * C) * 4u;
-    const unsigned col_bytes = static_cast<unsigned>(C) * 4u;
+                          in_col0 + static_cast<unsigned>(2 * C) * kEsz;
+    const unsigned col_bytes = static_cast<unsigned>(C) * kEsz;
     st_off[0] = (y_ok[0] && x_ok[2]) ? base : kOobOffset;
     st_off[1] = (y_ok[0] && x_ok[3]) ? base + col_bytes : kOobOffset;
     st_off[2] = (y_ok[1] && x_ok[2]) ? base + in_row_bytes : kOobOffset;
@@ -1400,6 +1401,57 @@ void launch_max_grad_tile(const float* in, const float* out, const float* dy,
   hipLaunchKernelGGL((pool_max_grad_tile_kernel<WIN, STRIDE>), grid, dim3(256),
                      0, stream, in, out, dy, dx, p, nan_mode, tiles_x, tiles_y,
                      cv_per_group);
+}
+
+// The 3x3 stride-2 max gradient without LDS (pool_max_grad_3x3_s2_kernel),
+// fp32 or binary16 tensors.
+template <typename T>
+void launch_max_grad_3x3_s2(const T* input_data, const T* output_data,
+                            const T* input_backprop, T* output_backprop,
+                            const snn_hip_pooling_params& p, bool nan_mode,
+                            hipStream_t stream) {
+  constexpr int kBlock = 256;
+  // block rows / columns: padded coordinates pad .. in + pad - 1, halved
+  const int n_brows = (p.in_rows + p.pad_rows - 1) / 2 - p.pad_rows / 2 + 1;
+  const int n_bcols = (p.in_cols + p.pad_cols - 1) / 2 - p.pad_cols / 2 + 1;
+  const size_t per_row =
+      static_cast<size_t>(p.batch) * n_bcols * (p.channels / 4);
+  // Block rows per lane: a strip re-reads the three input rows and the
+  // output / dY row of the block row above it, so the longest strip that
+  // still leaves about six waves per CU (112x112x64 at batch 32: 14 block
+  // rows, 1.1 x the input read instead of 1.4 x, 60 -> 56 us; 28 leave 3.5
+  // waves per CU: 76 us).
+  int th = per_row * ceil_div(n_brows, 14) >= 100000
+               ? 14
+               : per_row * ceil_div(n_brows, 4) >= 150000 ? 4 : 2;
+  if (const char* tune = SNN_TUNING_ENV("SNN_HIP_POOL_GRAD_TH")) {
+    const int v = std::atoi(tune);
+    if (v == 2 || v == 4 || v == 14) th = v;
+  }
+  const int n_strips = ceil_div(n_brows, th);
+  const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
+  const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(kBlock), 0, stream, input_data,
+                       output_data, input_backprop, output_backprop, p,
+                       n_bcols, n_strips, n_items);
+  };
+  if (th == 14) {
+    if (nan_mode)
+      launch(pool_max_grad_3x3_s2_kernel<14, true, T>);
+    else
+      launch(pool_max_grad_3x3_s2_kernel<14, false, T>);
+  } else if (th == 4) {
+    if (nan_mode)
+      launch(pool_max_grad_3x3_s2_kernel<4, true, T>);
+    else
+      launch(pool_max_grad_3x3_s2_kernel<4, false, T>);
+  } else {
+    if (nan_mode)
+      launch(pool_max_grad_3x3_s2_kernel<2, true, T>);
+    else
+      launch(pool_max_grad_3x3_s2_kernel<2, false, T>);
+  }
 }
 
 }  // namespace
@@ -1457,47 +1509,8 @@ int launch_pooling_max_grad(const float* input_data, const float* output_data,
   static const bool use_tiles = SNN_TUNING_ENV("SNN_HIP_POOL_GRAD_TILES") != nullptr;
   if (vec4 && square && p.window_rows == 3 && p.stride_rows == 2 &&
       !use_tiles && n_in * 4 < 0x7FFFFFF0u && n_out * 4 < 0x7FFFFFF0u) {
-    // block rows / columns: padded coordinates pad .. in + pad - 1, halved
-    const int n_brows = (p.in_rows + p.pad_rows - 1) / 2 - p.pad_rows / 2 + 1;
-    const int n_bcols = (p.in_cols + p.pad_cols - 1) / 2 - p.pad_cols / 2 + 1;
-    const size_t per_row =
-        static_cast<size_t>(p.batch) * n_bcols * (p.channels / 4);
-    // Block rows per lane: a strip re-reads the three input rows and the
-    // output / dY row of the block row above it, so the longest strip that
-    // still leaves about six waves per CU (112x112x64 at batch 32: 14 block
-    // rows, 1.1 x the input read instead of 1.4 x, 60 -> 56 us; 28 leave 3.5
-    // waves per CU: 76 us).
-    int th = per_row * ceil_div(n_brows, 14) >= 100000
-                 ? 14
-                 : per_row * ceil_div(n_brows, 4) >= 150000 ? 4 : 2;
-    if (const char* tune = SNN_TUNING_ENV("SNN_HIP_POOL_GRAD_TH")) {
-      const int v = std::atoi(tune);
-      if (v == 2 || v == 4 || v == 14) th = v;
-    }
-    const int n_strips = ceil_div(n_brows, th);
-    const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
-    const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
-    auto launch = [&](auto kernel) {
-      hipLaunchKernelGGL(kernel, grid, dim3(kBlock), 0, stream, input_data,
-                         output_data, input_backprop, output_backprop, p,
-                         n_bcols, n_strips, n_items);
-    };
-    if (th == 14) {
-      if (nan_mode)
-        launch(pool_max_grad_3x3_s2_kernel<14, true>);
-      else
-        launch(pool_max_grad_3x3_s2_kernel<14, false>);
-    } else if (th == 4) {
-      if (nan_mode)
-        launch(pool_max_grad_3x3_s2_kernel<4, true>);
-      else
-        launch(pool_max_grad_3x3_s2_kernel<4, false>);
-    } else {
-      if (nan_mode)
-        launch(pool_max_grad_3x3_s2_kernel<2, true>);
-      else
-        launch(pool_max_grad_3x3_s2_kernel<2, false>);
-    }
+    launch_max_grad_3x3_s2<float>(input_data, output_data, input_backprop,
+                                  output_backprop, p, nan_mode, stream);
   } else if (vec4 && square && p.window_rows == 3 && p.stride_rows == 2) {
     launch_max_grad_tile<3, 2>(input_data, output_data, input_backprop,
                                output_backprop, p, nan_mode, stream);
@@ -1611,7 +1624,17 @@ int launch_pooling_max_grad_f16(const _Float16* input_data,
   const size_t n_in =
       static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
   const bool nan_mode = op == SNN_HIP_POOL_MAX_WITH_NAN;
+  const size_t n_out =
+      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * p.channels;
   if (p.channels % 4 == 0 && grad_aligned8(input_data) &&
+      grad_aligned8(output_data) && grad_aligned8(input_backprop) &&
+      grad_aligned8(output_backprop) && p.window_rows == 3 &&
+      p.window_cols == 3 && p.stride_rows == 2 && p.stride_cols == 2 &&
+      n_in * 2 < 0x7FFFFFF0u && n_out * 2 < 0x7FFFFFF0u) {
+    // the fp32 kernel for this window, reading and writing binary16
+    launch_max_grad_3x3_s2<_Float16>(input_data, output_data, input_backprop,
+                                     output_backprop, p, nan_mode, stream);
+  } else if (p.channels % 4 == 0 && grad_aligned8(input_data) &&
       grad_aligned8(output_data) && grad_aligned8(input_backprop) &&
       grad_aligned8(output_backprop)) {
     const size_t n_vec = n_in / 4;
