@@ -782,10 +782,10 @@ __global__ void __launch_bounds__(256)
 // order (window row, then window column, starting from zero;
 // src/pooling/kernels.h:291-375); a window that does not exist contributes
 // +0, which leaves every sum as it is.
-template <int TH>
+template <int TH, typename T = float>
 __global__ void __launch_bounds__(256)
-    pool_avg_grad_3x3_s2_kernel(const float* __restrict__ dy,
-                                float* __restrict__ dx,
+    pool_avg_grad_3x3_s2_kernel(const T* __restrict__ dy,
+                                T* __restrict__ dx,
                                 snn_hip_pooling_params p, int n_bcols,
                                 int n_strips, unsigned n_items) {
   const unsigned idx = blockIdx.x * 256u + threadIdx.x;
@@ -800,12 +800,13 @@ __global__ void __launch_bounds__(256)
   const int br0 = static_cast<int>(t % static_cast<unsigned>(n_strips)) * TH +
                   p.pad_rows / 2;
   const int n = static_cast<int>(t / static_cast<unsigned>(n_strips));
+  constexpr unsigned kEsz = sizeof(T);
   const size_t in_elems =
       static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * C;
   const size_t out_elems =
       static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * C;
-  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, out_elems * 4);
-  const __amdgpu_buffer_rsrc_t dx_rsrc = make_rsrc(dx, in_elems * 4);
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, out_elems * kEsz);
+  const __amdgpu_buffer_rsrc_t dx_rsrc = make_rsrc(dx, in_elems * kEsz);
 
   // windows bc - 1 and bc: present, and their number of in-image columns
   bool w_ok[2];
@@ -823,12 +824,12 @@ __global__ void __launch_bounds__(256)
         static_cast<unsigned>(oy) < static_cast<unsigned>(p.out_rows);
     const unsigned base =
         static_cast<unsigned>(((n * p.out_rows + oy) * p.out_cols + bc - 1) *
-                                  C + ch) * 4u;
+                                  C + ch) * kEsz;
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-      BufVec4<float>::load(dy_rsrc,
+      BufVec4<T>::load(dy_rsrc,
                            (row_ok && w_ok[j])
-                               ? base + static_cast<unsigned>(j * C) * 4u
+                               ? base + static_cast<unsigned>(j * C) * kEsz
                                : kOobOffset,
                            g[j]);
   };
@@ -846,8 +847,8 @@ __global__ void __launch_bounds__(256)
   const bool x_ok[2] = {
       static_cast<unsigned>(x0) < static_cast<unsigned>(p.in_cols),
       static_cast<unsigned>(x0 + 1) < static_cast<unsigned>(p.in_cols)};
-  const unsigned row_bytes = static_cast<unsigned>(p.in_cols * C) * 4u;
-  const unsigned col_bytes = static_cast<unsigned>(C) * 4u;
+  const unsigned row_bytes = static_cast<unsigned>(p.in_cols * C) * kEsz;
+  const unsigned col_bytes = static_cast<unsigned>(C) * kEsz;
 
   float rows[TH + 1][2][4];
 #pragma unroll
@@ -873,14 +874,14 @@ __global__ void __launch_bounds__(256)
         static_cast<unsigned>(y0 + 1) < static_cast<unsigned>(p.in_rows)};
     const unsigned base =
         static_cast<unsigned>(((n * p.in_rows + y0) * p.in_cols + x0) * C + ch) *
-        4u;
-    BufVec4<float>::store(dx_rsrc, (y_ok[0] && x_ok[0]) ? base : kOobOffset,
+        kEsz;
+    BufVec4<T>::store(dx_rsrc, (y_ok[0] && x_ok[0]) ? base : kOobOffset,
                           ee);
-    BufVec4<float>::store(
+    BufVec4<T>::store(
         dx_rsrc, (y_ok[0] && x_ok[1]) ? base + col_bytes : kOobOffset, eo);
-    BufVec4<float>::store(
+    BufVec4<T>::store(
         dx_rsrc, (y_ok[1] && x_ok[0]) ? base + row_bytes : kOobOffset, oe);
-    BufVec4<float>::store(
+    BufVec4<T>::store(
         dx_rsrc,
         (y_ok[1] && x_ok[1]) ? base + row_bytes + col_bytes : kOobOffset, oo);
   }
@@ -1454,6 +1455,32 @@ void launch_max_grad_3x3_s2(const T* input_data, const T* output_data,
   }
 }
 
+// The 3x3 stride-2 average gradient (pool_avg_grad_3x3_s2_kernel), fp32 or
+// binary16 tensors.
+template <typename T>
+void launch_avg_grad_3x3_s2(const T* input_backprop, T* output_backprop,
+                            const snn_hip_pooling_params& p,
+                            hipStream_t stream) {
+  constexpr int kBlock = 256;
+  // block rows / columns: padded coordinates pad .. in + pad - 1, halved
+  const int n_brows = (p.in_rows + p.pad_rows - 1) / 2 - p.pad_rows / 2 + 1;
+  const int n_bcols = (p.in_cols + p.pad_cols - 1) / 2 - p.pad_cols / 2 + 1;
+  const size_t per_row =
+      static_cast<size_t>(p.batch) * n_bcols * (p.channels / 4);
+  const int th = per_row * ceil_div(n_brows, 4) >= 150000 ? 4 : 2;
+  const int n_strips = ceil_div(n_brows, th);
+  const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
+  const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
+  if (th == 4)
+    hipLaunchKernelGGL((pool_avg_grad_3x3_s2_kernel<4, T>), grid, dim3(kBlock), 0,
+                       stream, input_backprop, output_backprop, p, n_bcols,
+                       n_strips, n_items);
+  else
+    hipLaunchKernelGGL((pool_avg_grad_3x3_s2_kernel<2, T>), grid, dim3(kBlock), 0,
+                       stream, input_backprop, output_backprop, p, n_bcols,
+                       n_strips, n_items);
+}
+
 }  // namespace
 
 template <typename T>
@@ -1551,23 +1578,7 @@ int launch_pooling_avg_grad(const float* input_backprop,
       grad_aligned16(output_backprop) && p.window_rows == 3 &&
       p.window_cols == 3 && p.stride_rows == 2 && p.stride_cols == 2 &&
       n_in * 4 < 0x7FFFFFF0u && n_out * 4 < 0x7FFFFFF0u && !no_s2) {
-    // block rows / columns: padded coordinates pad .. in + pad - 1, halved
-    const int n_brows = (p.in_rows + p.pad_rows - 1) / 2 - p.pad_rows / 2 + 1;
-    const int n_bcols = (p.in_cols + p.pad_cols - 1) / 2 - p.pad_cols / 2 + 1;
-    const size_t per_row =
-        static_cast<size_t>(p.batch) * n_bcols * (p.channels / 4);
-    const int th = per_row * ceil_div(n_brows, 4) >= 150000 ? 4 : 2;
-    const int n_strips = ceil_div(n_brows, th);
-    const unsigned n_items = static_cast<unsigned>(per_row * n_strips);
-    const dim3 grid(ceil_div(n_items, static_cast<unsigned>(kBlock)));
-    if (th == 4)
-      hipLaunchKernelGGL(pool_avg_grad_3x3_s2_kernel<4>, grid, dim3(kBlock), 0,
-                         stream, input_backprop, output_backprop, p, n_bcols,
-                         n_strips, n_items);
-    else
-      hipLaunchKernelGGL(pool_avg_grad_3x3_s2_kernel<2>, grid, dim3(kBlock), 0,
-                         stream, input_backprop, output_backprop, p, n_bcols,
-                         n_strips, n_items);
+    launch_avg_grad_3x3_s2<float>(input_backprop, output_backprop, p, stream);
   } else if (p.channels % 4 == 0 && grad_aligned16(input_backprop) &&
              grad_aligned16(output_backprop)) {
     const size_t n_vec = n_in / 4;
@@ -1660,7 +1671,16 @@ int launch_pooling_avg_grad_f16(const _Float16* input_backprop,
   constexpr int kBlock = 256;
   const size_t n_in =
       static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
+  const size_t n_out =
+      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * p.channels;
   if (p.channels % 4 == 0 && grad_aligned8(input_backprop) &&
+      grad_aligned8(output_backprop) && p.window_rows == 3 &&
+      p.window_cols == 3 && p.stride_rows == 2 && p.stride_cols == 2 &&
+      n_in * 2 < 0x7FFFFFF0u && n_out * 2 < 0x7FFFFFF0u) {
+    // the fp32 kernel for this window, reading and writing binary16
+    launch_avg_grad_3x3_s2<_Float16>(input_backprop, output_backprop, p,
+                                     stream);
+  } else if (p.channels % 4 == 0 && grad_aligned8(input_backprop) &&
       grad_aligned8(output_backprop)) {
     const size_t n_vec = n_in / 4;
     hipLaunchKernelGGL((pool_avg_grad_kernel<4, _Float16>),
