@@ -465,7 +465,9 @@ def test_input_gradient_of_strided_1x1_layers(shape):
     gradient over the output pixels, written to the input pixels at multiples
     of the stride, zeros elsewhere: computed dense on the stride-1 kernels and
     scattered in one pass; against the oracle over the whole tensor, every
-    element of dX written (the output starts as NaN)."""
+    element of dX written (the output starts as NaN).  The forward layer
+    gathers the pixels it reads and runs on the stride-1 kernels too, bias
+    and ReLU included."""
     batch, rows, cols, ch, feats, stride = shape
     p = ops.conv_params(batch, rows, cols, ch, feats, 1, stride, False)
     rng = np.random.default_rng(2900 + rows + ch)
@@ -483,6 +485,20 @@ def test_input_gradient_of_strided_1x1_layers(shape):
         assert_close(got.cpu().numpy(), ref,
                      ("strided 1x1 input gradient", ALGO_NAME[algo], shape))
         assert torch.all(out[n_dx:] == 7.0)
+    n_x, n_w, n_y = ops.conv_sizes(p, DIRECTION.FORWARD)
+    x, bias = uniform(rng, n_x), uniform(rng, feats)
+    ref = oracle.conv2d_forward(x, w, oracle_params(p, feats), acc64=True)
+    for algo in (ALGO.MATMUL, ALGO.IM2COL, ALGO.TILED):
+        if not supported(p, DIRECTION.FORWARD, algo):
+            continue
+        got = ops.conv2d(dev(x), dev(w), p, DIRECTION.FORWARD, algo)
+        assert_close(got.cpu().numpy(), ref,
+                     ("strided 1x1 forward", ALGO_NAME[algo], shape))
+    fused = ops.conv2d_bias_act(dev(x), dev(w), dev(bias), p, ALGO.IM2COL,
+                                relu=True)
+    want = np.maximum(ref.reshape(-1, feats) + bias.astype(np.float64), 0)
+    assert_close(fused.cpu().numpy(), want.reshape(-1),
+                 ("strided 1x1 forward + bias + relu", shape))
 
 
 @pytest.mark.parametrize("shape", [
