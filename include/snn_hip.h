@@ -230,10 +230,10 @@ SNN_HIP_API int snn_hip_conv2d_filter_backprop_f16(
  * meet through float atomics -- the implicit-GEMM filter gradient (Im2col /
  * Tiled / Direct-fallback tags) always, except for the 7x7 stride-2
  * three-channel stem from 224 output rows over the batch upwards and for
- * layers with channels and features in multiples of 64 -- or of 4, when
- * window size x channels exceeds 192 and the channel count is not a multiple
- * of 64 -- (16-byte aligned operands, at least 256 output pixels), whose
- * partial filters are summed in a fixed order; forward and input gradients of small
+ * every other layer with at least 32 channels, or with window size x channels
+ * above 192, or with a feature count that is not a multiple of 4 (16-byte
+ * aligned operands, at least 256 output pixels), whose partial filters are
+ * summed in a fixed order; forward and input gradients of small
  * problems (fewer than ~640 64x64 output tiles, unless one of the kernels
  * that sum their parts in a fixed order takes the launch: stride-1 layers
  * with channels in multiples of 128, forward problems of fewer than 128
