@@ -835,15 +835,16 @@ __global__ void __launch_bounds__(kDwFilbkThreads)
 // that order; rows and columns past the end of the image read zeros through
 // the buffer range check and add nothing.  The pixel lanes of a wave are added
 // up across lanes, the four waves through LDS.
-template <int STRIDE, int TH, int TW, int AHEAD>
+template <int STRIDE, int TH, int TW, int AHEAD, typename T = float>
 __global__ void __launch_bounds__(kDwFilbkThreads)
-    dw_filter_backprop_3x3_strip_kernel(const float* __restrict__ in,
-                                        const float* __restrict__ dy,
+    dw_filter_backprop_3x3_strip_kernel(const T* __restrict__ in,
+                                        const T* __restrict__ dy,
                                         float* __restrict__ dw,
                                         float* __restrict__ part,
                                         snn_hip_depthwise_params p, int cvw,
                                         int strips_per_group, int n_strips,
                                         int n_row_blocks, int n_col_blocks) {
+  constexpr unsigned kEsz = sizeof(T);
   // A strip is TH output rows of TW adjacent output columns, so an input row
   // costs NC column loads for TW outputs.  The loads of output row i + AHEAD
   // are issued before the products of row i.
@@ -863,8 +864,8 @@ __global__ void __launch_bounds__(kDwFilbkThreads)
       static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * C;
   const size_t dy_elems =
       static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * C;
-  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_elems * 4);
-  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, dy_elems * 4);
+  const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, in_elems * kEsz);
+  const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(dy, dy_elems * kEsz);
   float acc[9][4];
 #pragma unroll
   for (int t = 0; t < 9; ++t)
@@ -886,11 +887,11 @@ __global__ void __launch_bounds__(kDwFilbkThreads)
       for (int sc = 0; sc < NC; ++sc)
         col_off[sc] = static_cast<unsigned>(x0 + sc) <
                               static_cast<unsigned>(p.in_cols)
-                          ? static_cast<unsigned>((x0 + sc) * C + c) * 4u
+                          ? static_cast<unsigned>((x0 + sc) * C + c) * kEsz
                           : kOobOffset;
       const unsigned image_off =
-          static_cast<unsigned>(n * p.in_rows * p.in_cols * C) * 4u;
-      const unsigned row_bytes = static_cast<unsigned>(p.in_cols * C) * 4u;
+          static_cast<unsigned>(n * p.in_rows * p.in_cols * C) * kEsz;
+      const unsigned row_bytes = static_cast<unsigned>(p.in_cols * C) * kEsz;
       float win[RING][NC][4];
       // (Offsets of rows and columns outside the image are made out of range
       // with mask arithmetic, not with a conditional: the compiler turns a
@@ -909,15 +910,15 @@ __global__ void __launch_bounds__(kDwFilbkThreads)
           const unsigned bad =
               bad_row |
               (0u - static_cast<unsigned>(col_off[sc] == kOobOffset));
-          BufVec4<float>::load(
+          BufVec4<T>::load(
               in_rsrc, ((base + col_off[sc]) & ~bad) | (kOobOffset & bad),
               dst[sc]);
         }
       };
       const unsigned dy_off0 =
           static_cast<unsigned>(((n * p.out_rows + oy0) * p.out_cols + ox) * C +
-                                c) * 4u;
-      const unsigned dy_row_bytes = static_cast<unsigned>(p.out_cols * C) * 4u;
+                                c) * kEsz;
+      const unsigned dy_row_bytes = static_cast<unsigned>(p.out_cols * C) * kEsz;
       float g[GRING][TW][4];
       // the input rows output row i adds that row i - 1 lacked, and its dY
       auto load_out_row = [&](int i) {
@@ -929,10 +930,10 @@ __global__ void __launch_bounds__(kDwFilbkThreads)
           const unsigned bad =
               0u - static_cast<unsigned>(oy0 + i >= p.out_rows ||
                                          ox + tw >= p.out_cols);
-          BufVec4<float>::load(
+          BufVec4<T>::load(
               dy_rsrc,
               ((dy_off0 + static_cast<unsigned>(i) * dy_row_bytes +
-                static_cast<unsigned>(tw * C) * 4u) & ~bad) |
+                static_cast<unsigned>(tw * C) * kEsz) & ~bad) |
                   (kOobOffset & bad),
               g[i % GRING][tw]);
         }
@@ -1371,7 +1372,8 @@ int dw_scratch_on_current_device(float** out) {
 // when the caller brings it (kDwScratchElems floats), else to a stream-ordered
 // temporary, and a second kernel adds them up (also the fallback when the
 // allocation fails).
-static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
+template <typename T>
+static int launch_dw_filbk_strip(const T* x, const T* dy, float* dw,
                                  const snn_hip_depthwise_params& p, int cvw,
                                  int grid_y, hipStream_t stream,
                                  float* static_scratch) {
@@ -1389,7 +1391,7 @@ static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
     return ceil_div(n_strips, *spg);
   };
   const size_t in_bytes = static_cast<size_t>(p.batch) * p.in_rows *
-                          p.in_cols * p.channels * sizeof(float);
+                          p.in_cols * p.channels * sizeof(T);
   // Large inputs: about 448 work-groups, every lane two or more strips (more,
   // shorter work-groups lose to their own start and end).  Small ones: up to
   // 1024, for the sake of parallelism.
@@ -1437,14 +1439,14 @@ static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
   // 2 / 3 rows, 112x112x64 stride 2 32.6 / 30.1 / 31.1 / 32.6 us).
   if (p.stride_rows == 1) {
     if (th == 8)
-      launch(dw_filter_backprop_3x3_strip_kernel<1, 8, tw, 2>);
+      launch((dw_filter_backprop_3x3_strip_kernel<1, 8, tw, 2, T>));
     else
-      launch(dw_filter_backprop_3x3_strip_kernel<1, 4, tw, 1>);
+      launch((dw_filter_backprop_3x3_strip_kernel<1, 4, tw, 1, T>));
   } else {
     if (th == 8)
-      launch(dw_filter_backprop_3x3_strip_kernel<2, 8, tw, 1>);
+      launch((dw_filter_backprop_3x3_strip_kernel<2, 8, tw, 1, T>));
     else
-      launch(dw_filter_backprop_3x3_strip_kernel<2, 4, tw, 1>);
+      launch((dw_filter_backprop_3x3_strip_kernel<2, 4, tw, 1, T>));
   }
   if (part != nullptr) {
     const int n_vec = dw_elems / 4;
@@ -1457,80 +1459,6 @@ static int launch_dw_filbk_strip(const float* x, const float* dy, float* dw,
         grid_x);
     if (temporary) temp_free_async(part, stream);
   }
-  return SNN_HIP_OK;
-}
-
-// Four elements per lane (element counts here are multiples of 4).
-template <typename From, typename To>
-__global__ void __launch_bounds__(256)
-    dw_convert_kernel(const From* __restrict__ in, To* __restrict__ out,
-                      size_t n_vec) {
-  typedef From from4 __attribute__((ext_vector_type(4)));
-  typedef To to4 __attribute__((ext_vector_type(4)));
-  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (i >= n_vec) return;
-  const from4 v = reinterpret_cast<const from4*>(in)[i];
-  to4 r;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) r[e] = static_cast<To>(v[e]);
-  reinterpret_cast<to4*>(out)[i] = r;
-}
-
-template <typename T>
-int launch_depthwise(int direction, const T* input, const T* filter, T* output,
-                     const snn_hip_depthwise_params& p, hipStream_t stream,
-                     float* static_scratch);
-
-// The binary16 3x3 filter gradient of a large layer through the fp32 strip
-// kernel: both operands widened into stream-ordered temporaries, the fp32
-// launch, the small result rounded (the general binary16 kernel, one
-// channel per lane and a tap per work-group, took 1.07 ms where fp32 takes
-// 77 us: 112x112x32 at batch 128).  -1: does not apply.
-int launch_depthwise_filter_backprop_f16_through_fp32(
-    const _Float16* input, const _Float16* dy, _Float16* dw,
-    const snn_hip_depthwise_params& p, hipStream_t stream) {
-  const size_t n_x =
-      static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels;
-  const size_t n_dy =
-      static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * p.channels;
-  if (p.channel_multiplier != 1 || p.channels % 4 != 0 || p.window_rows != 3 ||
-      p.window_cols != 3 || p.stride_rows != p.stride_cols ||
-      (p.stride_rows != 1 && p.stride_rows != 2) || n_dy < (size_t{1} << 21) ||
-      n_x * sizeof(float) >= 0x7FFFFFF0u)
-    return -1;
-  const size_t n_dw = static_cast<size_t>(9) * p.channels;
-  void *x32 = nullptr, *dy32 = nullptr, *dw32 = nullptr;
-  auto release = [&]() {
-    if (dw32 != nullptr) temp_free_async(dw32, stream);
-    if (dy32 != nullptr) temp_free_async(dy32, stream);
-    if (x32 != nullptr) temp_free_async(x32, stream);
-  };
-  if (temp_malloc_async(&x32, n_x * sizeof(float), stream) != hipSuccess ||
-      temp_malloc_async(&dy32, n_dy * sizeof(float), stream) != hipSuccess ||
-      temp_malloc_async(&dw32, n_dw * sizeof(float), stream) != hipSuccess) {
-    release();
-    return SNN_HIP_ALLOCATION_PROBLEM;
-  }
-  auto convert = [&](auto* in, auto* out, size_t n) {
-    hipLaunchKernelGGL(
-        (dw_convert_kernel<std::remove_cv_t<std::remove_pointer_t<decltype(in)>>,
-                           std::remove_pointer_t<decltype(out)>>),
-        dim3(static_cast<unsigned>(ceil_div(n / 4, size_t{256}))), dim3(256), 0,
-        stream, in, out, n / 4);
-  };
-  convert(input, static_cast<float*>(x32), n_x);
-  convert(dy, static_cast<float*>(dy32), n_dy);
-  const int status = launch_depthwise<float>(
-      SNN_HIP_FILTER_BACKPROP, static_cast<const float*>(x32),
-      static_cast<const float*>(dy32), static_cast<float*>(dw32), p, stream,
-      nullptr);
-  if (status == SNN_HIP_OK)
-    convert(static_cast<const float*>(dw32), dw, n_dw);
-  const hipError_t err = hipGetLastError();
-  release();
-  if (status != SNN_HIP_OK) return status;
-  if (err != hipSuccess)
-    return report_hip_error(err, "binary16 depthwise filter backprop");
   return SNN_HIP_OK;
 }
 
@@ -1631,9 +1559,41 @@ int launch_depthwise(int direction, const T* input, const T* filter, T* output,
         static_cast<size_t>(p.batch) * p.out_rows * p.out_cols;
     bool done = false;
     if constexpr (std::is_same<T, _Float16>::value) {
-      const int rc = launch_depthwise_filter_backprop_f16_through_fp32(
-          input, filter, output, p, stream);
-      if (rc >= 0) return rc;
+      // binary16, 3x3, stride 1 or 2: the fp32 strip kernel reading binary16,
+      // its sums in an fp32 temporary of the filter's size that one more pass
+      // rounds (the general kernel below took 1.07 ms where this takes about
+      // what fp32 does: 112x112x32 at batch 128)
+      if (p.channel_multiplier == 1 && p.channels % 4 == 0 &&
+          p.window_rows == 3 && p.window_cols == 3 &&
+          p.stride_rows == p.stride_cols &&
+          (p.stride_rows == 1 || p.stride_rows == 2) &&
+          n_pix_sz * p.channels * sizeof(T) < 0x7FFFFFF0u &&
+          static_cast<size_t>(p.batch) * p.in_rows * p.in_cols * p.channels *
+                  sizeof(T) < 0x7FFFFFF0u &&
+          n_pix_sz * p.channels >= (size_t{1} << 18)) {
+        const int cv = p.channels / 4;
+        int cvw = 1;
+        while (cvw * 2 <= cv && cvw < 32) cvw *= 2;  // >= 8 pixel lanes
+        const int grid_y = ceil_div(cv, cvw);
+        const int dw_elems = 9 * p.channels;
+        void* acc = nullptr;
+        if (temp_malloc_async(&acc, dw_elems * sizeof(float), stream) !=
+            hipSuccess)
+          return SNN_HIP_ALLOCATION_PROBLEM;
+        const int status = launch_dw_filbk_strip<T>(
+            input, filter, static_cast<float*>(acc), p, cvw, grid_y, stream,
+            nullptr);
+        if (status == SNN_HIP_OK)
+          hipLaunchKernelGGL(dw_round_kernel<T>, dim3(ceil_div(dw_elems, 256)),
+                             dim3(256), 0, stream,
+                             static_cast<const float*>(acc), output, dw_elems);
+        const hipError_t err = hipGetLastError();
+        temp_free_async(acc, stream);
+        if (status != SNN_HIP_OK) return status;
+        if (err != hipSuccess)
+          return report_hip_error(err, "binary16 depthwise filter backprop");
+        return SNN_HIP_OK;
+      }
     }
     if constexpr (std::is_same<T, float>::value) {
       if (p.channel_multiplier == 1 && p.channels % 4 == 0 &&
@@ -1658,7 +1618,7 @@ int launch_depthwise(int direction, const T* input, const T* filter, T* output,
             (p.stride_rows == 1 || p.stride_rows == 2) &&
             SNN_TUNING_ENV("SNN_HIP_DW_FILBK_PIXEL") == nullptr;
         if (strip_ok) {
-          const int status = launch_dw_filbk_strip(
+          const int status = launch_dw_filbk_strip<float>(
               input, filter, output, p, cvw, grid_y, stream, static_scratch);
           if (status != SNN_HIP_OK) return status;
         } else {
