@@ -525,11 +525,35 @@ __global__ void __launch_bounds__(256)
   if (i < n) out[i] = static_cast<To>(in[i]);
 }
 
+// Four elements per lane.
+template <typename From, typename To>
+__global__ void __launch_bounds__(256)
+    convert4_kernel(const From* __restrict__ in, To* __restrict__ out,
+                    size_t n_vec) {
+  typedef From from4 __attribute__((ext_vector_type(4)));
+  typedef To to4 __attribute__((ext_vector_type(4)));
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= n_vec) return;
+  const from4 v = reinterpret_cast<const from4*>(in)[i];
+  to4 r;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) r[e] = static_cast<To>(v[e]);
+  reinterpret_cast<to4*>(out)[i] = r;
+}
+
 template <typename From, typename To>
 void convert(const From* in, To* out, size_t n, hipStream_t s) {
-  hipLaunchKernelGGL((convert_kernel<From, To>),
-                     dim3(static_cast<unsigned>(ceil_div(n, size_t{256}))),
-                     dim3(256), 0, s, in, out, n);
+  const bool vec = n % 4 == 0 &&
+                   (reinterpret_cast<uintptr_t>(in) % (4 * sizeof(From))) == 0 &&
+                   (reinterpret_cast<uintptr_t>(out) % (4 * sizeof(To))) == 0;
+  if (vec)
+    hipLaunchKernelGGL((convert4_kernel<From, To>),
+                       dim3(static_cast<unsigned>(ceil_div(n / 4, size_t{256}))),
+                       dim3(256), 0, s, in, out, n / 4);
+  else
+    hipLaunchKernelGGL((convert_kernel<From, To>),
+                       dim3(static_cast<unsigned>(ceil_div(n, size_t{256}))),
+                       dim3(256), 0, s, in, out, n);
 }
 
 // A binary16 launch that no binary16 matrix-core kernel takes (three input
