@@ -2388,13 +2388,17 @@ int strided_input_backprop_by_classes(const T* input, const T* filter,
     }
   if (ok) {
     void *g = nullptr, *t = nullptr;
+    // (no room for the temporaries: the caller takes another path)
     if (temp_malloc_async(&g, max(filter_elems, 4u) * sizeof(T), stream) !=
-        hipSuccess)
-      return SNN_HIP_ALLOCATION_PROBLEM;
+        hipSuccess) {
+      (void)hipGetLastError();
+      return -1;
+    }
     if (temp_malloc_async(&t, max(pixels, size_t{1}) * p.channels * sizeof(T),
                           stream) != hipSuccess) {
+      (void)hipGetLastError();
       temp_free_async(g, stream);
-      return SNN_HIP_ALLOCATION_PROBLEM;
+      return -1;
     }
     hipLaunchKernelGGL(
         stride_class_filters_kernel<T>,
@@ -2505,26 +2509,29 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
     const size_t t_elems =
         static_cast<size_t>(p.batch) * p.out_rows * p.out_cols * p.channels;
     void* t = nullptr;
-    if (temp_malloc_async(&t, t_elems * sizeof(float), stream) != hipSuccess)
-      return SNN_HIP_ALLOCATION_PROBLEM;
-    const int status = launch_conv2d_igemm_f32(
-        direction, input, filter, static_cast<float*>(t), q, stream, workspace,
-        workspace_elems, epilogue);
-    if (status == SNN_HIP_OK) {
-      const size_t n_vec = static_cast<size_t>(p.batch) * p.in_rows *
-                           p.in_cols * p.channels / 4;
-      hipLaunchKernelGGL(
-          scatter_strided_pixels_kernel,
-          dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))), dim3(256),
-          0, stream, static_cast<const float4*>(t),
-          reinterpret_cast<float4*>(output), p.in_rows, p.in_cols, p.out_rows,
-          p.out_cols, p.stride_rows, p.stride_cols, p.channels / 4, n_vec);
+    if (temp_malloc_async(&t, t_elems * sizeof(float), stream) == hipSuccess) {
+      const int status = launch_conv2d_igemm_f32(
+          direction, input, filter, static_cast<float*>(t), q, stream,
+          workspace, workspace_elems, epilogue);
+      if (status == SNN_HIP_OK) {
+        const size_t n_vec = static_cast<size_t>(p.batch) * p.in_rows *
+                             p.in_cols * p.channels / 4;
+        hipLaunchKernelGGL(
+            scatter_strided_pixels_kernel,
+            dim3(static_cast<unsigned>(ceil_div(n_vec, size_t{256}))),
+            dim3(256), 0, stream, static_cast<const float4*>(t),
+            reinterpret_cast<float4*>(output), p.in_rows, p.in_cols,
+            p.out_rows, p.out_cols, p.stride_rows, p.stride_cols,
+            p.channels / 4, n_vec);
+      }
+      const hipError_t err = hipGetLastError();
+      temp_free_async(t, stream);
+      if (status != SNN_HIP_OK) return status;
+      if (err != hipSuccess)
+        return report_hip_error(err, "strided 1x1 input backprop");
+      return SNN_HIP_OK;
     }
-    const hipError_t err = hipGetLastError();
-    temp_free_async(t, stream);
-    if (status != SNN_HIP_OK) return status;
-    if (err != hipSuccess) return report_hip_error(err, "strided 1x1 input backprop");
-    return SNN_HIP_OK;
+    (void)hipGetLastError();  // no room: the general strided kernel below
   }
   if (direction == SNN_HIP_INPUT_BACKPROP && aligned16 &&
       (p.stride_rows > 1 || p.stride_cols > 1) &&

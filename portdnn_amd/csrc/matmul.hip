@@ -166,8 +166,10 @@ int launch_matmul_repacked_f32(const float* lhs, const float* rhs,
   if ((new_a && !grab(&a2, static_cast<size_t>(m) * k2)) ||
       (new_b && !grab(&b2, static_cast<size_t>(k2) * n2)) ||
       (new_c && !grab(&c2, static_cast<size_t>(m) * n2))) {
+    // (no room for the copies: the general kernel takes the product)
+    (void)hipGetLastError();
     release();
-    return SNN_HIP_ALLOCATION_PROBLEM;
+    return -1;
   }
   const float* a = new_a ? a2 : lhs;
   const float* b = new_b ? b2 : rhs;

@@ -480,13 +480,17 @@ int launch_gemm_path_padded(int direction, const T* input, const T* filter,
   // temporaries cost more than the direct kernel's whole run)
   if (pixels * filter_rows * p.features < (size_t{1} << 24)) return -1;
   void *wide_filter = nullptr, *wide_pixels = nullptr;
+  // (no room for the copies: the launch stays on the path it had)
   if (temp_malloc_async(&wide_filter, filter_rows * q.features * sizeof(T), s) !=
-      hipSuccess)
-    return SNN_HIP_ALLOCATION_PROBLEM;
+      hipSuccess) {
+    (void)hipGetLastError();
+    return -1;
+  }
   if (temp_malloc_async(&wide_pixels, pixels * q.features * sizeof(T), s) !=
       hipSuccess) {
+    (void)hipGetLastError();
     temp_free_async(wide_filter, s);
-    return SNN_HIP_ALLOCATION_PROBLEM;
+    return -1;
   }
   copy_columns(filter, p.features, static_cast<T*>(wide_filter), q.features,
                p.features, filter_rows, s);
@@ -579,8 +583,10 @@ int launch_f16_through_fp32(int direction, const _Float16* input,
   if (temp_malloc_async(&in32, sz.input * sizeof(float), s) != hipSuccess ||
       temp_malloc_async(&fil32, sz.filter * sizeof(float), s) != hipSuccess ||
       temp_malloc_async(&out32, sz.output * sizeof(float), s) != hipSuccess) {
+    // (no room for the copies: the launch stays on the path it had)
+    (void)hipGetLastError();
     release();
-    return SNN_HIP_ALLOCATION_PROBLEM;
+    return -1;
   }
   convert(input, static_cast<float*>(in32), sz.input, s);
   convert(filter, static_cast<float*>(fil32), sz.filter, s);
