@@ -1095,8 +1095,13 @@ __global__ void __launch_bounds__(kThreads)
 // rows are 193 floats apart so that lanes that differ in the pixel hit
 // different banks.  The up to 6 x 2 accumulator blocks are dealt to the four
 // waves round-robin.  Partial sums meet in dW through float atomics.
+// Layers with at most eight channels and a longer (tap, channel) range (an
+// 11x11x3 stem: 363) run as up to kSmallQParts parts of 192 in blockIdx.z,
+// each part an independent launch of the same scheme over its rows of dW.
 constexpr int kSmallQMax = 192;
 constexpr int kSmallQStride = kSmallQMax + 1;
+constexpr int kSmallQParts = 4;
+constexpr int kSmallQPartsMaxChannels = 8;
 
 __global__ void __launch_bounds__(kThreads)
     conv_filter_backprop_smallq_kernel(const float* __restrict__ x,
@@ -1114,7 +1119,10 @@ __global__ void __launch_bounds__(kThreads)
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n0 = blockIdx.x * BN;
-  const int q_total = g.win_rows * g.win_cols * g.channels;
+  // this part's rows of dW: q_begin .. q_begin + q_total - 1
+  const int q_begin = blockIdx.z * kSmallQMax;
+  const int q_total =
+      min(kSmallQMax, g.win_rows * g.win_cols * g.channels - q_begin);
   const int n_mblocks = (q_total + 31) / 32;
   const int n_blocks = 2 * n_mblocks;
 
@@ -1150,8 +1158,8 @@ __global__ void __launch_bounds__(kThreads)
   // (tap row, tap col, channel) of a_q0
   int q_r, q_s, q_c;
   {
-    const int tap = a_q0 / g.channels;
-    q_c = a_q0 - tap * g.channels;
+    const int tap = (q_begin + a_q0) / g.channels;
+    q_c = q_begin + a_q0 - tap * g.channels;
     q_r = tap / g.win_cols;
     q_s = tap - q_r * g.win_cols;
   }
@@ -1277,7 +1285,7 @@ __global__ void __launch_bounds__(kThreads)
       const int q = q_base + 8 * (v >> 2) + (v & 3);
       const unsigned off =
           (col < g.features && q < q_total)
-              ? static_cast<unsigned>(q) * row_bytes +
+              ? static_cast<unsigned>(q_begin + q) * row_bytes +
                     static_cast<unsigned>(col) * 4u
               : kOob;
       __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(acc[i][v], dw_rsrc, off,
@@ -1775,13 +1783,20 @@ static int launch_input_backprop_col2im(const float* dy, const float* filter,
 
 // Every shape it supports except those the one-work-group kernel takes (few
 // (tap, channel) pairs, e.g. a three-channel stem).
-bool conv2d_filter_backprop_direct_f32_wanted(const snn_hip_conv2d_params& p) {
+bool conv2d_filter_backprop_direct_f32_wanted(const snn_hip_conv2d_params& p,
+                                              bool reproducible) {
   const bool whole = p.channels % 64 == 0 && p.features % 64 == 0;
   // (from 32 channels on the 64-channel tiles are at least half full and
-  // measured faster: 112x112x32 -> 64, 1x1, at batch 32 89.6 us there)
+  // measured faster: 112x112x32 -> 64, 1x1, at batch 32 89.6 us there; with
+  // at most eight channels they are so empty that the one-work-group kernel
+  // in parts wins -- 11x11x3 -> 96 stride 4 at batch 16: 1000 us here -- but
+  // it sums through atomics, so a reproducible launch stays here)
+  const int q = p.window_rows * p.window_cols * p.channels;
   const bool small_q =
-      p.channels < 32 && p.features % 4 == 0 &&
-      p.window_rows * p.window_cols * p.channels <= kSmallQMax;
+      p.features % 4 == 0 &&
+      ((p.channels < 32 && q <= kSmallQMax) ||
+       (!reproducible && p.channels <= kSmallQPartsMaxChannels &&
+        q <= kSmallQParts * kSmallQMax));
   if (small_q || !conv2d_filter_backprop_direct_f32_supports(p, true))
     return false;
   return !whole || SNN_TUNING_ENV("SNN_HIP_FBDIRECT_OFF") == nullptr;
@@ -1790,7 +1805,7 @@ bool conv2d_filter_backprop_direct_f32_wanted(const snn_hip_conv2d_params& p) {
 static int launch_filter_backprop(const float* x, const float* dy, float* dw,
                                   const snn_hip_conv2d_params& p,
                                   float* workspace, size_t workspace_elems,
-                                  hipStream_t stream) {
+                                  hipStream_t stream, bool reproducible) {
   FilterBackpropGeom g;
   g.batch = p.batch; g.in_rows = p.in_rows; g.in_cols = p.in_cols;
   g.channels = p.channels; g.out_rows = p.out_rows; g.out_cols = p.out_cols;
@@ -1808,7 +1823,7 @@ static int launch_filter_backprop(const float* x, const float* dy, float* dw,
       (reinterpret_cast<uintptr_t>(dw) & 15u) == 0 &&
       SNN_TUNING_ENV("SNN_HIP_STEM_OFF") == nullptr)
     return launch_conv2d_stem_filter_backprop_f32(x, dy, dw, p, stream);
-  if (conv2d_filter_backprop_direct_f32_wanted(p)) {
+  if (conv2d_filter_backprop_direct_f32_wanted(p, reproducible)) {
     // partial filters go to the workspace when it holds them, else to a
     // stream-ordered temporary
     const size_t part_floats = conv2d_filter_backprop_direct_f32_partial_floats(p);
@@ -1837,8 +1852,11 @@ static int launch_filter_backprop(const float* x, const float* dy, float* dw,
     // few (tap, channel) pairs: one work-group column per 64 features, the
     // pixel range split over about two work-groups per CU
     const int n_chunks = ceil_div(g.m_total, kBK);
+    const int q_parts =
+        ceil_div(p.window_rows * p.window_cols * p.channels, kSmallQMax);
     const int col_groups = ceil_div(p.features, 64);
-    int splits = max(1, min(ceil_div(512, col_groups), n_chunks / 4));
+    int splits =
+        max(1, min(ceil_div(512, col_groups * q_parts), n_chunks / 4));
     const int per_split = ceil_div(n_chunks, splits);
     splits = ceil_div(n_chunks, per_split);
     const size_t n_vec = dw_elems / 4;  // features % 4 == 0
@@ -1854,9 +1872,8 @@ static int launch_filter_backprop(const float* x, const float* dy, float* dw,
     (void)attr;
     KernelTimer timer(stream);
     hipLaunchKernelGGL(conv_filter_backprop_smallq_kernel,
-                       dim3(col_groups, splits), dim3(kThreads), kLdsBytes,
-                       stream, x,
-                       dy, dw, g, static_cast<unsigned>(x_elems * 4),
+                       dim3(col_groups, splits, q_parts), dim3(kThreads),
+                       kLdsBytes, stream, x, dy, dw, g, static_cast<unsigned>(x_elems * 4),
                        static_cast<unsigned>(dy_elems * 4),
                        static_cast<unsigned>(dw_elems * 4), per_split);
     return SNN_HIP_OK;
@@ -2594,8 +2611,9 @@ int launch_conv2d_igemm_f32(int direction, const float* input,
     return launch_input_backprop_col2im(input, filter, output, p, workspace,
                                         workspace_elems, stream);
   if (direction == SNN_HIP_FILTER_BACKPROP) {
-    const int rc = launch_filter_backprop(input, filter, output, p, workspace,
-                                          workspace_elems, stream);
+    const int rc = launch_filter_backprop(
+        input, filter, output, p, workspace, workspace_elems, stream,
+        epilogue != nullptr && epilogue->deterministic);
     SNN_HIP_CHECK_LAUNCH();
     return rc;
   }

@@ -479,19 +479,18 @@ int launch_gemm_path_padded(int direction, const T* input, const T* filter,
   // (small problems stay where they were: three more launches and two
   // temporaries cost more than the direct kernel's whole run)
   if (pixels * filter_rows * p.features < (size_t{1} << 24)) return -1;
-  void *wide_filter = nullptr, *wide_pixels = nullptr;
+  // one temporary holds both copies (the filter's rounded up to 256 bytes)
+  const size_t filter_elems =
+      (filter_rows * q.features + 127) / 128 * 128;
+  void* wide_filter = nullptr;
   // (no room for the copies: the launch stays on the path it had)
-  if (temp_malloc_async(&wide_filter, filter_rows * q.features * sizeof(T), s) !=
-      hipSuccess) {
+  if (temp_malloc_async(&wide_filter,
+                        (filter_elems + pixels * q.features) * sizeof(T),
+                        s) != hipSuccess) {
     (void)hipGetLastError();
     return -1;
   }
-  if (temp_malloc_async(&wide_pixels, pixels * q.features * sizeof(T), s) !=
-      hipSuccess) {
-    (void)hipGetLastError();
-    temp_free_async(wide_filter, s);
-    return -1;
-  }
+  void* const wide_pixels = static_cast<T*>(wide_filter) + filter_elems;
   copy_columns(filter, p.features, static_cast<T*>(wide_filter), q.features,
                p.features, filter_rows, s);
   int status;
@@ -509,7 +508,6 @@ int launch_gemm_path_padded(int direction, const T* input, const T* filter,
                                  nullptr, 0, epilogue);
   }
   const hipError_t err = hipGetLastError();
-  temp_free_async(wide_pixels, s);
   temp_free_async(wide_filter, s);
   if (status != SNN_HIP_OK) return status;
   if (err != hipSuccess) return report_hip_error(err, "padded features");
@@ -574,30 +572,34 @@ int launch_f16_through_fp32(int direction, const _Float16* input,
                       p.window_rows * p.window_cols * p.channels * p.features;
   if (macs < double(1 << 24)) return -1;
   const ConvSizes sz = conv_sizes(p, direction);
-  void *in32 = nullptr, *fil32 = nullptr, *out32 = nullptr;
-  auto release = [&]() {
-    if (out32 != nullptr) temp_free_async(out32, s);
-    if (fil32 != nullptr) temp_free_async(fil32, s);
-    if (in32 != nullptr) temp_free_async(in32, s);
-  };
-  if (temp_malloc_async(&in32, sz.input * sizeof(float), s) != hipSuccess ||
-      temp_malloc_async(&fil32, sz.filter * sizeof(float), s) != hipSuccess ||
-      temp_malloc_async(&out32, sz.output * sizeof(float), s) != hipSuccess) {
+  // One stream-ordered temporary for the three widened tensors and the
+  // workspace the fp32 launch would otherwise allocate for itself (every
+  // allocation costs tens of microseconds of host time).
+  auto padded = [](size_t floats) { return (floats + 63) / 64 * 64; };
+  size_t ws_required = 0, ws_floats = 0;
+  (void)workspace_size(p, direction, SNN_HIP_ALGO_IM2COL, SNN_HIP_DTYPE_F32,
+                       &ws_required, &ws_floats);
+  if (ws_floats > (size_t{256} << 20) / sizeof(float)) ws_floats = 0;
+  const size_t total = padded(sz.input) + padded(sz.filter) +
+                       padded(sz.output) + padded(ws_floats);
+  void* block = nullptr;
+  if (temp_malloc_async(&block, total * sizeof(float), s) != hipSuccess) {
     // (no room for the copies: the launch stays on the path it had)
     (void)hipGetLastError();
-    release();
     return -1;
   }
-  convert(input, static_cast<float*>(in32), sz.input, s);
-  convert(filter, static_cast<float*>(fil32), sz.filter, s);
-  const int status = launch_gemm_path<float>(
-      direction, static_cast<const float*>(in32),
-      static_cast<const float*>(fil32), static_cast<float*>(out32), p, s,
-      nullptr, 0, nullptr);
+  float* const in32 = static_cast<float*>(block);
+  float* const fil32 = in32 + padded(sz.input);
+  float* const out32 = fil32 + padded(sz.filter);
+  float* const ws32 = ws_floats != 0 ? out32 + padded(sz.output) : nullptr;
+  convert(input, in32, sz.input, s);
+  convert(filter, fil32, sz.filter, s);
+  const int status = launch_gemm_path<float>(direction, in32, fil32, out32, p,
+                                             s, ws32, ws_floats, nullptr);
   if (status == SNN_HIP_OK)
     convert(static_cast<const float*>(out32), output, sz.output, s);
   const hipError_t err = hipGetLastError();
-  release();
+  temp_free_async(block, s);
   if (status != SNN_HIP_OK) return status;
   if (err != hipSuccess) return report_hip_error(err, "binary16 through fp32");
   return SNN_HIP_OK;
@@ -609,6 +611,14 @@ int launch_gemm_path<_Float16>(int direction, const _Float16* input,
                                const snn_hip_conv2d_params& p, hipStream_t s,
                                _Float16* workspace, size_t workspace_elems,
                                const LaunchOptions*) {
+  // (a gradient of at most eight channels: the binary16 kernels' 64-channel
+  // tiles would be nearly empty, fp32 has kernels for such layers -- 224x224
+  // 3 <- 64, 3x3, at batch 8: 286 us on the general binary16 kernel over a
+  // copy widened to four channels, 69 us in fp32)
+  if (direction == SNN_HIP_INPUT_BACKPROP && p.channels <= 8) {
+    const int rc = launch_f16_through_fp32(direction, input, filter, output, p, s);
+    if (rc >= 0) return rc;
+  }
   if (direction == SNN_HIP_INPUT_BACKPROP && aligned16(output)) {
     const int padded = launch_gemm_path_padded<_Float16>(
         direction, input, filter, output, p, s, nullptr,
@@ -657,7 +667,7 @@ int launch_gemm_path<_Float16>(int direction, const _Float16* input,
   // (few (tap, channel) pairs -- a three-channel stem: fp32 has kernels built
   // for that; 64-channel tiles would be nearly empty)
   if (direction == SNN_HIP_FILTER_BACKPROP && p.channels <= 8 &&
-      p.window_rows * p.window_cols * p.channels <= 192) {
+      p.window_rows * p.window_cols * p.channels <= 768) {
     const int rc = launch_f16_through_fp32(direction, input, filter, output, p, s);
     if (rc >= 0) return rc;
   }
@@ -684,7 +694,7 @@ int launch_gemm_path<float>(int direction, const float* input,
   // and features in multiples of 64 adds in a fixed order and serves both.
   const bool atomics_only = direction == SNN_HIP_FILTER_BACKPROP &&
                             epilogue != nullptr && epilogue->deterministic &&
-                            !conv2d_filter_backprop_direct_f32_wanted(p);
+                            !conv2d_filter_backprop_direct_f32_wanted(p, true);
   if ((direction == SNN_HIP_FORWARD && aligned16(input)) ||
       (direction == SNN_HIP_INPUT_BACKPROP && aligned16(output))) {
     const int padded = launch_gemm_path_padded<float>(

@@ -163,8 +163,10 @@ bool conv2d_filter_backprop_direct_f32_supports(const snn_hip_conv2d_params& p,
                                                 bool ragged = false);
 bool conv2d_filter_backprop_direct_f16_supports(const snn_hip_conv2d_params& p);
 // Whether the implicit-GEMM launcher sends this fp32 filter gradient to that
-// kernel (conv2d_igemm.hip).
-bool conv2d_filter_backprop_direct_f32_wanted(const snn_hip_conv2d_params& p);
+// kernel (conv2d_igemm.hip); `reproducible` keeps shapes here whose faster
+// kernel sums through atomics.
+bool conv2d_filter_backprop_direct_f32_wanted(const snn_hip_conv2d_params& p,
+                                              bool reproducible = false);
 size_t conv2d_filter_backprop_direct_f32_partial_floats(
     const snn_hip_conv2d_params& p);
 size_t conv2d_filter_backprop_direct_f16_partial_floats(

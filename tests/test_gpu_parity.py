@@ -1791,6 +1791,43 @@ def test_feature_counts_that_are_not_multiples_of_four_run_padded(shape, dtype):
                      ("bias + relu, ragged features", shape))
 
 
+@pytest.mark.parametrize("shape", [
+    (3, 67, 67, 3, 96, 11, 4, False),   # 363 (tap, channel) pairs: two parts
+    (4, 40, 40, 4, 32, 11, 2, True),    # 484: three parts
+    (1, 30, 30, 8, 64, 9, 1, True),     # 648: four parts
+])
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_few_channel_layers_with_large_windows(shape, dtype):
+    """Layers of at most eight channels whose (tap, channel) range is longer
+    than the one-work-group filter gradient kernel holds (an 11x11x3 stem) run
+    that kernel in parts of 192 rows of dW; their binary16 input gradient and
+    filter gradient run through the fp32 kernels.  All three directions
+    against the oracle in double precision."""
+    batch, rows, cols, ch, feats, window, stride, same = shape
+    p = ops.conv_params(batch, rows, cols, ch, feats, window, stride, same)
+    rng = np.random.default_rng(911 + rows + ch + feats)
+    half = dtype == "f16"
+    tdt = torch.float16 if half else torch.float32
+    for direction in (DIRECTION.FORWARD, DIRECTION.INPUT_BACKPROP,
+                      DIRECTION.FILTER_BACKPROP):
+        n_a, n_b, n_o = ops.conv_sizes(p, direction)
+        a, b = uniform(rng, n_a), uniform(rng, n_b)
+        if half:
+            a, b = a.astype(np.float16), b.astype(np.float16)
+        ref = ORACLE_FN[direction](a.astype(np.float32), b.astype(np.float32),
+                                   oracle_params(p, feats), acc64=True)
+        out = torch.full((n_o + 16,), 7.0, dtype=tdt, device="cuda")
+        got = ops.conv2d(dev(a, tdt), dev(b, tdt), p, direction, ALGO.IM2COL,
+                         out=out[:n_o])
+        if half:
+            assert_close_f16(got.float().cpu().numpy(), ref,
+                             ("f16 few channels", direction, shape))
+        else:
+            assert_close(got.cpu().numpy(), ref,
+                         ("few channels", direction, shape))
+        assert torch.all(out[n_o:] == 7.0)
+
+
 def test_f16_conv_filter_backprop():
     p = ops.conv_params(3, 10, 9, 16, 24, 3, 1, True)
     rng = np.random.default_rng(781)
