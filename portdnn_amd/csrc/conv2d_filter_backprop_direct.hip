@@ -1,6 +1,8 @@
-// Filter gradient on the fp32 MFMA (gfx950) with both operands loaded from
-// memory straight into the matrix instruction's registers (fp32 tensors, or
-// binary16 tensors converted on the way in and accumulated in fp32):
+// Filter gradient on the matrix cores (gfx950) with both operands loaded from
+// memory straight into the matrix instruction's registers (fp32 tensors on the
+// fp32 instruction; binary16 tensors on the binary16 instruction, see
+// filter_backprop_direct_h16_kernel, or -- channel / feature counts that are
+// not multiples of 4 -- converted on the way into the fp32 one; fp32 sums):
 //   dW[r][s][c][k] = sum over output pixels m of X[m shifted by (r, s)][c] * dY[m][k]
 // (portDNN: a matmul with the left operand transposed for 1x1 windows,
 // src/conv2d/matmul, and the im2col / tiled filter-gradient kernels otherwise,
@@ -162,6 +164,67 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// The 8 waves' partial tiles (acc[e][f][v]: channel c0 + 16 quad + 4 v + e,
+// feature k0 + 4 l16 + f) meet in LDS and are added in wave order; the sum
+// goes to `out` at this split's partial filter.
+template <int VEC>
+__device__ inline void reduce_and_store(const float4v (&acc)[4][4], float* lds,
+                                        int wave, int tid, float* out,
+                                        unsigned out_bytes, int split,
+                                        unsigned split_bytes, int tap, int c0,
+                                        int k0, const XtDy& g) {
+  const int lane = tid & 63;
+  const int l16 = lane & 15, quad = lane >> 4;
+  // The 8 partial tiles meet in LDS: [wave][64 channels][64 features].
+  float* const mine = lds + wave * (kTile * kTile);
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int row = 16 * quad + 4 * v + e;
+      *reinterpret_cast<float4*>(mine + row * kTile + 4 * l16) =
+          make_float4(acc[e][0][v], acc[e][1][v], acc[e][2][v], acc[e][3][v]);
+    }
+  __syncthreads();
+  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_bytes);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int idx = tid + 64 * kWaves * i;  // float4 of the tile
+    float4 sum = *reinterpret_cast<const float4*>(lds + 4 * idx);
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) {
+      const float4 part =
+          *reinterpret_cast<const float4*>(lds + w * (kTile * kTile) + 4 * idx);
+      sum.x += part.x;
+      sum.y += part.y;
+      sum.z += part.z;
+      sum.w += part.w;
+    }
+    const int row = idx >> 4, col = (idx & 15) * 4;
+    const unsigned off =
+        static_cast<unsigned>(split) * split_bytes +
+        (static_cast<unsigned>(tap * g.channels + c0 + row) *
+             static_cast<unsigned>(g.features) +
+         static_cast<unsigned>(k0 + col)) * 4u;
+    // (rows and columns past the end of a ragged tile: dropped, out of range)
+    const bool row_live = c0 + row < g.channels;
+    if constexpr (VEC == 4) {
+      const bool live = row_live && k0 + col < g.features;
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, sum),
+                                             out_rsrc, live ? off : kOob, 0, 0);
+    } else {
+      const float vals[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool live = row_live && k0 + col + e < g.features;
+        __builtin_amdgcn_raw_buffer_store_b32(
+            __builtin_bit_cast(unsigned, vals[e]), out_rsrc,
+            live ? off + 4u * e : kOob, 0, 0);
+      }
+    }
+  }
+}
+
 // `out` (fp32): dW, or the partial filters when a unit's pixels are split
 // over work-groups or the tensors are binary16 (`split_bytes` apart, else 0).
 // WINDOW: any window, stride and padding; otherwise 1x1, stride 1, unpadded,
@@ -307,54 +370,181 @@ __global__ void __launch_bounds__(64 * kWaves)
   for (int d = 0; d < kDepth - 1; ++d)
     if (d < rest) multiply(d);
 
-  // The 8 partial tiles meet in LDS: [wave][64 channels][64 features].
-  float* const mine = lds + wave * (kTile * kTile);
+  reduce_and_store<VEC>(acc, lds, wave, tid, out, out_bytes, split,
+                        split_bytes, tap, c0, k0, g);
+}
+
+// Binary16 tensors with channel and feature counts in multiples of 4 on the
+// binary16 matrix instruction: v_mfma_f32_16x16x16_f16 takes from lane l four
+// consecutive reduction indices, A[row l % 16][4 (l / 16) .. + 3], so a step is
+// 16 pixels and a lane loads, for each of ITS four pixels 4 (l / 16) + j, the
+// 8 bytes of its four channels (features) and regroups the 4 x 4 halves in
+// registers into one operand per accumulator block: eight loads, sixteen
+// two-half packs and 16 matrix instructions per 16 pixels, against 64 matrix
+// instructions of the fp32 form (whose products are the same: binary16 times
+// binary16 is exact in fp32, and the sums are fp32 in both).  Tile, units,
+// splits, partial filters and the reduction are those of the kernel above.
+constexpr int kDepthH = 3;  // steps of 16 pixels in flight per wave
+
+template <bool WINDOW>
+__global__ void __launch_bounds__(64 * kWaves)
+    filter_backprop_direct_h16_kernel(const _Float16* __restrict__ x,
+                                      const _Float16* __restrict__ dy,
+                                      float* __restrict__ out, XtDy g,
+                                      unsigned x_bytes, unsigned out_bytes,
+                                      unsigned split_bytes, unsigned n_groups) {
+  extern __shared__ __align__(16) float lds[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const unsigned group = xcd_remap(blockIdx.x, n_groups);
+  const int split = static_cast<int>(group / g.n_units);
+  const int unit = static_cast<int>(group % g.n_units);
+  const int tap = WINDOW ? unit % g.taps : 0;
+  const int tile = WINDOW ? unit / g.taps : unit;
+  const int c0 = (tile % g.c_tiles) * kTile;
+  const int k0 = (tile / g.c_tiles) * kTile;
+
+  const int share = split * kWaves + wave;
+  const int m_begin = min(g.m_total, share * g.steps_per_wave * 4);
+  const int m_end = min(g.m_total, m_begin + g.steps_per_wave * 4);
+  const int n_steps = (m_end - m_begin + 15) >> 4;
+
+  // dY (and X without a window) past this wave's last pixel is out of the
+  // buffer's range and loads zeros; with a window X's offsets are masked.
+  const unsigned x_row = static_cast<unsigned>(g.channels) * 2u;
+  const unsigned y_row = static_cast<unsigned>(g.features) * 2u;
+  const __amdgpu_buffer_rsrc_t x_rsrc =
+      make_rsrc(x, WINDOW ? x_bytes : static_cast<unsigned>(m_end) * x_row);
+  const __amdgpu_buffer_rsrc_t y_rsrc =
+      make_rsrc(dy, static_cast<unsigned>(m_end) * y_row);
+  const int l16 = lane & 15, quad = lane >> 4;
+  const unsigned x_col = static_cast<unsigned>(c0 + 4 * l16) * 2u;
+  const bool x_live = c0 + 4 * l16 < g.channels;
+  const bool y_live = k0 + 4 * l16 < g.features;
+  int m_lane = m_begin + 4 * quad;  // the first of this lane's four pixels
+  unsigned vx = x_live ? static_cast<unsigned>(m_lane) * x_row + x_col : kOob;
+  unsigned vy = y_live ? static_cast<unsigned>(m_lane) * y_row +
+                             static_cast<unsigned>(k0 + 4 * l16) * 2u
+                       : kOob;
+  const unsigned x_step = x_live ? 16u * x_row : 0u;
+  const unsigned y_step = y_live ? 16u * y_row : 0u;
+  const unsigned x_dead = x_live ? 0u : ~0u;
+  int px_n = 0, px_y = 0, px_x = 0, tap_y = 0, tap_x = 0;
+  if constexpr (WINDOW) {
+    px_x = m_lane % g.out_cols;
+    const int t = m_lane / g.out_cols;
+    px_y = t % g.out_rows;
+    px_n = t / g.out_rows;
+    tap_y = tap / g.win_cols - g.pad_rows;
+    tap_x = tap % g.win_cols - g.pad_cols;
+  }
+
+  uint2v hx[kDepthH][4], hy[kDepthH][4];
+  auto issue = [&](int d) {
+    unsigned ox[4];
+    if constexpr (WINDOW) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int iy = px_y * g.stride_rows + tap_y;
+        const int ix = px_x * g.stride_cols + tap_x;
+        // all ones where the tap falls outside the image or the pixel is
+        // past this wave's share (mask arithmetic, no branch around a load)
+        const unsigned bad =
+            x_dead |
+            (0u - static_cast<unsigned>(
+                      (static_cast<unsigned>(iy) >= static_cast<unsigned>(g.in_rows)) |
+                      (static_cast<unsigned>(ix) >= static_cast<unsigned>(g.in_cols)) |
+                      (m_lane + j >= m_end)));
+        const unsigned off =
+            static_cast<unsigned>((px_n * g.in_rows + iy) * g.in_cols + ix) *
+                x_row + x_col;
+        ox[j] = (off & ~bad) | (kOob & bad);
+        // the next pixel
+        const bool row_end = px_x + 1 == g.out_cols;
+        const bool img_end = row_end & (px_y + 1 == g.out_rows);
+        px_x = row_end ? 0 : px_x + 1;
+        px_y = img_end ? 0 : px_y + (row_end ? 1 : 0);
+        px_n += img_end ? 1 : 0;
+      }
+      // the other lanes' twelve pixels
+      px_x += 12;
+      while (px_x >= g.out_cols) {
+        px_x -= g.out_cols;
+        if (++px_y == g.out_rows) {
+          px_y = 0;
+          ++px_n;
+        }
+      }
+      m_lane += 16;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ox[j] = vx + static_cast<unsigned>(j) * x_row;
+      vx += x_step;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      hx[d][j] = __builtin_bit_cast(
+          uint2v, __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, ox[j], 0, 0));
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      hy[d][j] = __builtin_bit_cast(
+          uint2v, __builtin_amdgcn_raw_buffer_load_b64(
+                      y_rsrc, vy + static_cast<unsigned>(j) * y_row, 0, 0));
+    vy += y_step;
+  };
+  float4v acc[4][4];
 #pragma unroll
   for (int e = 0; e < 4; ++e)
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const int row = 16 * quad + 4 * v + e;
-      *reinterpret_cast<float4*>(mine + row * kTile + 4 * l16) =
-          make_float4(acc[e][0][v], acc[e][1][v], acc[e][2][v], acc[e][3][v]);
+    for (int f = 0; f < 4; ++f)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[e][f][v] = 0.f;
+  // element e of the four pixels' vectors, as one operand
+  auto gather = [](const uint2v (&h)[4], int e) {
+    half4v r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = __builtin_bit_cast(half4v, h[j])[e];
+    return r;
+  };
+  auto multiply = [&](int d) {
+    half4v a[4], b[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      a[e] = gather(hx[d], e);
+      b[e] = gather(hy[d], e);
     }
-  __syncthreads();
-  const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out, out_bytes);
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int idx = tid + 64 * kWaves * i;  // float4 of the tile
-    float4 sum = *reinterpret_cast<const float4*>(lds + 4 * idx);
+    for (int e = 0; e < 4; ++e)
 #pragma unroll
-    for (int w = 1; w < kWaves; ++w) {
-      const float4 part =
-          *reinterpret_cast<const float4*>(lds + w * (kTile * kTile) + 4 * idx);
-      sum.x += part.x;
-      sum.y += part.y;
-      sum.z += part.z;
-      sum.w += part.w;
-    }
-    const int row = idx >> 4, col = (idx & 15) * 4;
-    const unsigned off =
-        static_cast<unsigned>(split) * split_bytes +
-        (static_cast<unsigned>(tap * g.channels + c0 + row) *
-             static_cast<unsigned>(g.features) +
-         static_cast<unsigned>(k0 + col)) * 4u;
-    // (rows and columns past the end of a ragged tile: dropped, out of range)
-    const bool row_live = c0 + row < g.channels;
-    if constexpr (VEC == 4) {
-      const bool live = row_live && k0 + col < g.features;
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, sum),
-                                             out_rsrc, live ? off : kOob, 0, 0);
-    } else {
-      const float vals[4] = {sum.x, sum.y, sum.z, sum.w};
+      for (int f = 0; f < 4; ++f)
+        acc[e][f] = __builtin_amdgcn_mfma_f32_16x16x16f16(a[e], b[f], acc[e][f],
+                                                          0, 0, 0);
+  };
+
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const bool live = row_live && k0 + col + e < g.features;
-        __builtin_amdgcn_raw_buffer_store_b32(
-            __builtin_bit_cast(unsigned, vals[e]), out_rsrc,
-            live ? off + 4u * e : kOob, 0, 0);
-      }
+  for (int d = 0; d < kDepthH; ++d) {
+    issue(d);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  int s = 0;
+  for (; s + kDepthH <= n_steps; s += kDepthH) {
+#pragma unroll
+    for (int d = 0; d < kDepthH; ++d) {
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(d);
+      __builtin_amdgcn_sched_barrier(0);
+      issue(d);  // step s + d + kDepthH (zeros past the end)
     }
   }
+  __builtin_amdgcn_sched_barrier(0);
+  const int rest = n_steps - s;
+#pragma unroll
+  for (int d = 0; d < kDepthH - 1; ++d)
+    if (d < rest) multiply(d);
+
+  reduce_and_store<4>(acc, lds, wave, tid, out, out_bytes, split, split_bytes,
+                      tap, c0, k0, g);
 }
 
 struct Plan {
@@ -388,7 +578,9 @@ Plan make_plan(const snn_hip_conv2d_params& p) {
   // 256; a wave's step is 16 matrix instructions of 32 cycles sharing a SIMD
   // with another wave (0.49 us), a round costs about 4 us of first loads and
   // LDS reduction on top, and partial filters are written and read back at
-  // about 4 MB per us plus the second launch.
+  // about 4 MB per us plus the second launch.  (The binary16 kernel's step
+  // is about a third of that; a model with 0.17 us chose splits that measured
+  // the same or up to 5 % slower on nine layers, so both share this one.)
   const double dw_bytes = 4.0 * g.taps * p.channels * p.features;
   const int max_splits = std::max(
       1, std::min({kComputeUnits, total_steps / (kWaves * kMinStepsPerWave),
@@ -417,10 +609,10 @@ bool supports(const snn_hip_conv2d_params& p, bool ragged, size_t elem) {
   const size_t m = static_cast<size_t>(p.batch) * p.out_rows * p.out_cols;
   if (m < 4 * kWaves * kMinStepsPerWave) return false;
   // every byte offset a lane forms, prefetch past the end included
-  const size_t rows = m + 4 * (kDepth + 1);
+  const size_t rows = m + 16 * (kDepthH + 2);
   if (rows * p.features * elem > kMaxBufferBytes) return false;
   const size_t in_rows = static_cast<size_t>(p.batch + 1) * p.in_rows *
-                             p.in_cols + 4 * (kDepth + 1);
+                             p.in_cols + 16 * (kDepthH + 2);
   if (in_rows * p.channels * elem > kMaxBufferBytes) return false;
   return static_cast<size_t>(p.window_rows) * p.window_cols * p.channels *
              p.features * sizeof(float) <= kMaxBufferBytes;
@@ -438,6 +630,22 @@ hipError_t launch_main(const T* x, const T* dy, float* out, const Plan& plan,
                      dim3(n_groups), dim3(64 * kWaves), kLdsBytes, stream, x, dy,
                      out, plan.g, static_cast<unsigned>(x_bytes), out_bytes,
                      split_bytes, n_groups);
+  return hipSuccess;
+}
+
+template <bool WINDOW>
+hipError_t launch_main_h16(const _Float16* x, const _Float16* dy, float* out,
+                           const Plan& plan, size_t x_bytes, unsigned out_bytes,
+                           unsigned split_bytes, unsigned n_groups,
+                           hipStream_t stream) {
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(filter_backprop_direct_h16_kernel<WINDOW>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  if (attr != hipSuccess) return attr;
+  hipLaunchKernelGGL((filter_backprop_direct_h16_kernel<WINDOW>), dim3(n_groups),
+                     dim3(64 * kWaves), kLdsBytes, stream, x, dy, out, plan.g,
+                     static_cast<unsigned>(x_bytes), out_bytes, split_bytes,
+                     n_groups);
   return hipSuccess;
 }
 
@@ -476,6 +684,18 @@ int launch(const T* x, const T* dy, T* dw, float* partial,
       plan.splits > 1 ? static_cast<unsigned>(dw_elems * 4) : 0u;
   KernelTimer timer(stream);
   hipError_t err;
+  if constexpr (sizeof(T) == 2) {
+    if (plan.vec4 && SNN_TUNING_ENV("SNN_HIP_FBDIRECT_H16_OFF") == nullptr) {
+      err = plan.window
+                ? launch_main_h16<true>(x, dy, out, plan, x_bytes, out_bytes,
+                                        split_bytes, n_groups, stream)
+                : launch_main_h16<false>(x, dy, out, plan, x_bytes, out_bytes,
+                                         split_bytes, n_groups, stream);
+      if (err != hipSuccess) return SNN_HIP_DEVICE_ERROR;
+      launch_reduce<T, 4>(partial, dw, dw_elems, plan.splits, stream);
+      return SNN_HIP_OK;
+    }
+  }
   if (plan.window)
     err = plan.vec4 ? launch_main<true, T, 4>(x, dy, out, plan, x_bytes,
                                               out_bytes, split_bytes, n_groups,

@@ -1695,14 +1695,18 @@ def test_f16_filter_backprop_1x1_transposing_reads(shape):
     (8, 32, 32, 64, 66, 3, 1, True),     # element by element
     (8, 32, 32, 66, 10, 1, 1, False),
     (8, 32, 32, 64, 3, 3, 1, True),
+    (3, 13, 11, 96, 64, 3, 1, True),     # 429 pixels: shares that end inside
+    (5, 9, 7, 48, 80, 1, 1, False),      # a step of 4 (fp32) or 16 (binary16)
 ])
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
 def test_filter_gradient_from_registers_ragged_and_half(shape, dtype):
     """Shapes that used to have no matrix-core filter gradient -- channel or
     feature counts that are not multiples of 64 (binary16: any but the 3x3 and
     1x1 stride-1 layers with whole tiles) or of 4 -- run on the kernel that
-    loads both operands straight into the fp32 matrix instruction, binary16
-    operands converted on the way, against the oracle in double precision on
+    loads both operands straight into the matrix instruction's registers
+    (binary16 with counts in multiples of 4: the binary16 instruction, four
+    pixels per lane regrouped in registers; other binary16 counts converted on
+    the way into the fp32 instruction), against the oracle in double precision on
     the same operands; with and without a workspace for the partial filters;
     twice gives the same bits."""
     batch, rows, cols, ch, feats, window, stride, same = shape
