@@ -107,10 +107,13 @@ constexpr int kStraddles = count_straddles();
 // w % 4 every time -- it keeps that quarter of the filter (37 registers) -- and
 // the four SIMDs the same work (with one output row per step and one pixel
 // block per wave the eighth wave idled).
+// TY: the output's element type (fp32, or binary16 rounded on the store for
+// the binary16 launch, whose 64-feature tensor is the large one).
+template <typename TY>
 __global__ void __launch_bounds__(64 * kWaves)
     __attribute__((amdgpu_waves_per_eu(2, 2)))
     conv_stem_7x7s2_kernel(const float* __restrict__ x,
-                           const float* __restrict__ w, float* __restrict__ y,
+                           const float* __restrict__ w, TY* __restrict__ y,
                            StemGeom g) {
   extern __shared__ __align__(16) float lds[];
   // one word past the rows that always holds zero
@@ -130,7 +133,8 @@ __global__ void __launch_bounds__(64 * kWaves)
   const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(
       x, static_cast<size_t>(g.batch) * g.in_rows * g.in_cols * kCh * 4);
   const __amdgpu_buffer_rsrc_t y_rsrc = make_rsrc(
-      y, static_cast<size_t>(g.batch) * g.out_rows * g.out_cols * kFeatures * 4);
+      y, static_cast<size_t>(g.batch) * g.out_rows * g.out_cols * kFeatures *
+             sizeof(TY));
 
   if (threadIdx.x == 0) lds[zero_word] = 0.f;
 
@@ -271,9 +275,21 @@ __global__ void __launch_bounds__(64 * kWaves)
               ? static_cast<unsigned>(((n * g.out_rows + oy) * g.out_cols + ox) *
                                           kFeatures +
                                       16 * fb + 4 * q) *
-                    4u
+                    static_cast<unsigned>(sizeof(TY))
               : kOobOffset;
-      __builtin_amdgcn_raw_buffer_store_b128(acc[i], y_rsrc, off, 0, kStoreAux);
+      if constexpr (sizeof(TY) == 4) {
+        __builtin_amdgcn_raw_buffer_store_b128(acc[i], y_rsrc, off, 0,
+                                               kStoreAux);
+      } else {
+        typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+        typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
+        const float4v r = __builtin_bit_cast(float4v, acc[i]);
+        half4v h;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(r[e]);
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2v, h),
+                                              y_rsrc, off, 0, kStoreAux);
+      }
     }
   }
   __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
@@ -772,24 +788,40 @@ bool conv2d_stem_supports(const snn_hip_conv2d_params& p) {
   return make_geom(p, &g);
 }
 
-// The output must be 16-byte aligned (the loads need nothing beyond 4).
-int launch_conv2d_stem_f32(const float* x, const float* w, float* y,
-                           const snn_hip_conv2d_params& p,
-                           hipStream_t stream) {
+namespace {
+template <typename TY>
+int launch_stem_forward(const float* x, const float* w, TY* y,
+                        const snn_hip_conv2d_params& p, hipStream_t stream) {
   StemGeom g;
   if (!make_geom(p, &g)) return SNN_HIP_INVALID_ALGORITHM;
   const size_t lds_bytes =
       (static_cast<size_t>(g.lds_rows + 1) * g.row_floats + 64) * sizeof(float);
   static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(conv_stem_7x7s2_kernel),
+      reinterpret_cast<const void*>(conv_stem_7x7s2_kernel<TY>),
       hipFuncAttributeMaxDynamicSharedMemorySize,
       static_cast<int>(kMaxLdsBytes));
   (void)attr;
   KernelTimer timer(stream);
-  hipLaunchKernelGGL(conv_stem_7x7s2_kernel,
+  hipLaunchKernelGGL(conv_stem_7x7s2_kernel<TY>,
                      dim3(static_cast<unsigned>(p.batch * g.n_bands)),
                      dim3(64 * kWaves), lds_bytes, stream, x, w, y, g);
   return SNN_HIP_OK;
+}
+}  // namespace
+
+// The output must be 16-byte aligned (the loads need nothing beyond 4).
+int launch_conv2d_stem_f32(const float* x, const float* w, float* y,
+                           const snn_hip_conv2d_params& p,
+                           hipStream_t stream) {
+  return launch_stem_forward<float>(x, w, y, p, stream);
+}
+
+// fp32 input and filter, the output rounded to binary16 on the store (8-byte
+// aligned).
+int launch_conv2d_stem_f32_to_f16(const float* x, const float* w, _Float16* y,
+                                  const snn_hip_conv2d_params& p,
+                                  hipStream_t stream) {
+  return launch_stem_forward<_Float16>(x, w, y, p, stream);
 }
 
 bool conv2d_stem_filter_backprop_supports(const snn_hip_conv2d_params& p) {

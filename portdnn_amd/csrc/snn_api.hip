@@ -572,6 +572,33 @@ int launch_f16_through_fp32(int direction, const _Float16* input,
                       p.window_rows * p.window_cols * p.channels * p.features;
   if (macs < double(1 << 24)) return -1;
   const ConvSizes sz = conv_sizes(p, direction);
+  // The 7x7 stride-2 three-channel stem, forward: the fp32 kernel rounds its
+  // output -- the large tensor -- to binary16 on the store, so only the image
+  // and the filter are widened (430 -> 328 us at batch 128).  (The filter
+  // gradient reading dY as binary16, one 2-byte load per lane where the fp32
+  // kernel has a 4-byte one, measured slower than the widening pass it saves:
+  // 623 against 444 us.)
+  if (direction == SNN_HIP_FORWARD && conv2d_stem_supports(p) &&
+      (reinterpret_cast<uintptr_t>(output) & 7u) == 0) {
+    auto padded = [](size_t floats) { return (floats + 63) / 64 * 64; };
+    void* block = nullptr;
+    if (temp_malloc_async(&block,
+                          (padded(sz.input) + padded(sz.filter)) * sizeof(float),
+                          s) == hipSuccess) {
+      float* const in32 = static_cast<float*>(block);
+      float* const fil32 = in32 + padded(sz.input);
+      convert(input, in32, sz.input, s);
+      convert(filter, fil32, sz.filter, s);
+      const int status =
+          launch_conv2d_stem_f32_to_f16(in32, fil32, output, p, s);
+      const hipError_t err = hipGetLastError();
+      temp_free_async(block, s);
+      if (status != SNN_HIP_OK) return status;
+      if (err != hipSuccess) return report_hip_error(err, "binary16 stem");
+      return SNN_HIP_OK;
+    }
+    (void)hipGetLastError();
+  }
   // One stream-ordered temporary for the three widened tensors and the
   // workspace the fp32 launch would otherwise allocate for itself (every
   // allocation costs tens of microseconds of host time).

@@ -204,6 +204,12 @@ int launch_conv2d_stem_filter_backprop_f32(const float* x, const float* dy,
                                            float* dw,
                                            const snn_hip_conv2d_params& p,
                                            hipStream_t stream);
+// The forward stem kernel with its output -- the large tensor -- rounded to
+// binary16 on the store and everything else fp32: what a binary16 stem launch
+// runs after widening its image and filter.
+int launch_conv2d_stem_f32_to_f16(const float* x, const float* w, _Float16* y,
+                                  const snn_hip_conv2d_params& p,
+                                  hipStream_t stream);
 
 // The same in half precision with fp32 accumulation (gemm_wreg_f16.hip):
 // k = 64, 128, 256 or 512.

@@ -120,6 +120,34 @@ def test_stem_7x7_stride2(direction):
 
 
 @pytest.mark.parametrize("batch,rows,cols,same", [
+    (5, 97, 61, True),      # ragged pixel block, odd rows
+    (6, 85, 100, False),    # no padding
+    (2, 224, 224, True),    # the stem layer itself
+])
+def test_stem_in_half_precision(batch, rows, cols, same):
+    """A binary16 launch of the 7x7 stride-2 three-channel stem runs the fp32
+    stem kernels: forward, the image and the filter widened into a temporary
+    and the output rounded to binary16 by the kernel's own store; the
+    gradients through fp32 copies.  Against the oracle in double precision on the same
+    binary16-rounded operands; nothing written past the result."""
+    p = ops.conv_params(batch, rows, cols, 3, 64, 7, 2, same)
+    rng = np.random.default_rng(331 + rows + cols)
+    for direction in (DIRECTION.FORWARD, DIRECTION.INPUT_BACKPROP,
+                      DIRECTION.FILTER_BACKPROP):
+        n_a, n_b, n_o = ops.conv_sizes(p, direction)
+        a = uniform(rng, n_a).astype(np.float16)
+        b = uniform(rng, n_b).astype(np.float16)
+        ref = ORACLE_FN[direction](a.astype(np.float32), b.astype(np.float32),
+                                   oracle_params(p, 64), acc64=True)
+        out = torch.full((n_o + 16,), 7.0, dtype=torch.float16, device="cuda")
+        got = ops.conv2d(dev(a, torch.float16), dev(b, torch.float16), p,
+                         direction, ALGO.IM2COL, out=out[:n_o])
+        assert_close_f16(got.float().cpu().numpy(), ref,
+                         ("f16 stem", direction, batch, rows, cols))
+        assert torch.all(out[n_o:] == 7.0)
+
+
+@pytest.mark.parametrize("batch,rows,cols,same", [
     (40, 64, 64, True),     # bands of three steps, two-row last band
     (5, 97, 61, True),      # 49 x 31 output: ragged pixel block, odd rows
     (6, 85, 100, False),    # no padding
